@@ -1,0 +1,30 @@
+"""MI355X-native RG-LRU: the reference's RG_LRU / RecurrentBlock interface over hand-written
+gfx950 HIP kernels (``scan_mode="hip"``)."""
+
+from .hip_scan import (
+    PreparedParams,
+    hip_rglru,
+    hip_rglru_scan,
+    hip_rglru_step,
+    hip_scan_available,
+    hip_scan_is_usable,
+)
+from .modules import (
+    BlockDiagonalLinear,
+    RG_LRU,
+    RecurrentBlock,
+    RecurrentBlockCache,
+)
+
+__all__ = [
+    "BlockDiagonalLinear",
+    "PreparedParams",
+    "RG_LRU",
+    "RecurrentBlock",
+    "RecurrentBlockCache",
+    "hip_rglru",
+    "hip_rglru_scan",
+    "hip_rglru_step",
+    "hip_scan_available",
+    "hip_scan_is_usable",
+]

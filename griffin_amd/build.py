@@ -1,0 +1,58 @@
+"""Build librglru_hip.so (hand-written gfx950 kernels + the C ABI) in-tree with hipcc.
+
+    python -m griffin_amd.build            # compile griffin_amd/librglru_hip.so
+
+hipcc cross-compiles without a GPU present, so this runs on a CPU-only machine.
+"""
+
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB_NAME = "librglru_hip.so"
+LIB_PATH = os.path.join(HERE, LIB_NAME)
+SOURCES = ["rglru_scan.hip", "rglru_fused.hip"]
+ARCH = "gfx950"
+
+
+def hipcc_path() -> str:
+    found = shutil.which("hipcc")
+    if found:
+        return found
+    candidate = os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "bin", "hipcc")
+    if os.path.exists(candidate):
+        return candidate
+    raise RuntimeError("hipcc not found: the RG-LRU HIP library cannot be built")
+
+
+def build(verbose: bool = False) -> str:
+    """Compile every kernel for gfx950 and link the shared library; returns its path."""
+    cmd = [
+        hipcc_path(), "-O3", "-std=c++17", "-fPIC", "-shared", f"--offload-arch={ARCH}",
+        "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+        "-Wno-unused-command-line-argument", "-ffp-contract=off",
+        "-I", os.path.join(os.path.dirname(HERE), "include"),
+    ]
+    cmd += [os.path.join(CSRC, s) for s in SOURCES]
+    tmp = LIB_PATH + ".tmp"
+    cmd += ["-o", tmp]
+    if verbose:
+        print(" ".join(cmd))
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    log = "\n".join(line for line in (proc.stdout + proc.stderr).splitlines() if noise not in line)
+    if proc.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + log)
+    if verbose and log.strip():
+        print(log)
+    os.replace(tmp, LIB_PATH)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build(verbose="-v" in sys.argv))

@@ -1,0 +1,721 @@
+// Fused RG-LRU kernels for gfx950: parameter preparation, forward, backward, decode step.
+//
+// Work decomposition.  The gates are block diagonal (griffin/griffin.py:129-154), so a tile of
+// TR = 32 * MT tokens of one sequence and one gate block depends on nothing but the same tokens
+// of that block.  A workgroup of four waves stages that x tile once in LDS; each wave owns one
+// 32-channel slab of the block:
+//   - the two gate pre-activations of its slab come from MFMA (rows = time, columns = channels,
+//     K = the block's input channels), weights kept in registers when the block is <= 128 wide;
+//   - the row permutation tile_row() makes every lane own a run of consecutive time steps of one
+//     channel, so the gate math (griffin/griffin.py:237-255) and the recurrence
+//     h_t = a_t h_{t-1} + z_t (griffin/griffin.py:279-284) run in registers, in time order;
+//   - carries between tiles travel through the publish / look-back protocol of rglru_device.h.
+// Workgroups are persistent: each is bound to one weight set ("unit" = gate block x group of four
+// slabs) and pulls (chunk, sequence) tiles of that unit from a ticket counter, in chain order.
+
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+
+#include "rglru_device.h"
+#include "rglru_host.h"
+#include "rglru_layout.h"
+
+namespace rglru {
+
+// ------------------------------------------------------------------------------------------
+// Parameter preparation
+// ------------------------------------------------------------------------------------------
+struct PrepArgs {
+  const void* w_a; const void* w_x; const float* b_a; const float* b_x; const float* lambda;
+  void* wg; float* bias; float* sp; float* cs;
+  int W, nb, bw, bwp, Wp;
+  float c;
+};
+
+RGLRU_DEVICE float log_sigmoid(float v) {
+  return v >= 0.f ? -log1pf(expf(-v)) : v - log1pf(expf(v));
+}
+
+template <typename IO>
+__global__ void prepare_kernel(PrepArgs p) {
+  const long long per_gate = (long long)p.nb * p.bwp * p.bwp;
+  const long long n_w = 2 * per_gate;
+  const long long total = n_w + p.Wp;
+  long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x;
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  for (; i < total; i += stride) {
+    if (i < n_w) {
+      int gate = (int)(i / per_gate);
+      long long rem = i - gate * per_gate;
+      int k = (int)(rem / ((long long)p.bwp * p.bwp));
+      int oj = (int)(rem - (long long)k * p.bwp * p.bwp);
+      int o = oj / p.bwp, j = oj - o * p.bwp;
+      float v = 0.f;
+      if (o < p.bw && j < p.bw) {
+        const IO* src = (const IO*)(gate ? p.w_x : p.w_a);
+        v = (float)src[((long long)k * p.bw + o) * p.bw + j];
+      }
+      ((IO*)p.wg)[i] = (IO)v;
+    } else {
+      int kp = (int)(i - n_w);
+      int k = kp / p.bwp, o = kp - k * p.bwp;
+      float ba = 0.f, bx = 0.f, sp = 0.f, cs = 0.f;
+      if (o < p.bw) {
+        int ch = k * p.bw + o;
+        ba = p.b_a[ch]; bx = p.b_x[ch];
+        float ls = log_sigmoid(p.lambda[ch]);
+        cs = p.c * ls;
+        sp = cs * kLog2e;
+      }
+      p.bias[kp] = ba; p.bias[p.Wp + kp] = bx; p.sp[kp] = sp; p.cs[kp] = cs;
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// Arguments common to the fused kernels
+// ------------------------------------------------------------------------------------------
+struct FusedArgs {
+  // tensors
+  const void* x; const void* wg; const float* bias; const float* sp; const float* cs;
+  const float* h0; const uint8_t* flags;
+  void* y; float* h_last;                                 // forward
+  const void* dy; const float* dh_last;                   // backward in
+  void* dx; void* du_a; void* du_x; float* dh0;           // backward out
+  float* h_state;                                         // decode step (in place)
+  // workspace
+  float* ckpt; float* agg_a; float* agg_h; float* incl; unsigned* status; unsigned* ticket;
+  unsigned* fail; float* partial;
+  // geometry
+  int B, T, W, nb, bw, bwp, S, Wp, groups, units;
+  int nC, nCf, ckpt_nC, slabs, wg_per_unit, aligned;
+  long long tiles_per_unit, limit;
+};
+
+// ------------------------------------------------------------------------------------------
+// Gate pre-activations of one tile.
+//   rows: `TR` consecutive rows starting at `row0` of a [rows_total, W] matrix (rows beyond
+//   rows_total read as zero); columns: gate block k.  On return ua/ux hold W x + b for the wave's
+//   slab (register v of tile mt <-> local row hf*16*MT + 16*mt + v) and xv the matching x values.
+// Every thread of the workgroup must call this (it contains barriers).
+// ------------------------------------------------------------------------------------------
+template <typename IO, int MT, int NKG>
+RGLRU_DEVICE void gate_tile(const FusedArgs& p, const IO* xmat, long long row0, long long rows_total,
+                            int k, int slab, bool slab_ok, const IO* w_a_row, const IO* w_x_row,
+                            const typename Io<IO>::Frag (&held_a)[NKG > 0 ? NKG : 1],
+                            const typename Io<IO>::Frag (&held_x)[NKG > 0 ? NKG : 1],
+                            float bias_a, float bias_x, IO* lds,
+                            f32x16 (&ua)[MT], f32x16 (&ux)[MT], float (&xv)[16 * MT]) {
+  typedef Io<IO> Tr;
+  typedef typename Tr::Frag Frag;
+  constexpr int TR = 32 * MT;
+  constexpr int KG = Tr::KG, HW = Tr::HW, KCMAX = Tr::KCMAX;
+  constexpr int LDSROW = KCMAX + HW;
+  const int tid = threadIdx.x, lane = tid & 63, r = lane & 31, hf = lane >> 5;
+
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) { ua[mt][v] = bias_a; ux[mt][v] = bias_x; }
+#pragma unroll
+  for (int e = 0; e < 16 * MT; ++e) xv[e] = 0.f;
+
+  for (int kc0 = 0; kc0 < p.bwp; kc0 += KCMAX) {
+    const int kcw = (p.bwp - kc0) < KCMAX ? (p.bwp - kc0) : KCMAX;
+    const int vecs = kcw / HW;
+    for (int idx = tid; idx < TR * vecs; idx += kThreads) {
+      const int row = idx / vecs, cv = idx - row * vecs;
+      const int col = kc0 + cv * HW;                      // column inside the gate block
+      Frag v = Tr::zero();
+      const long long grow = row0 + row;
+      if (grow < rows_total) {
+        const IO* src = xmat + grow * (long long)p.W + (long long)k * p.bw + col;
+        if (p.aligned && col + HW <= p.bw) {
+          v = *reinterpret_cast<const Frag*>(src);
+        } else {
+#pragma unroll
+          for (int e = 0; e < HW; ++e) if (col + e < p.bw) v[e] = src[e];
+        }
+      }
+      *reinterpret_cast<Frag*>(lds + row * LDSROW + cv * HW) = v;
+    }
+    __syncthreads();
+    if (slab_ok) {
+      if constexpr (NKG > 0) {
+#pragma unroll
+        for (int kg = 0; kg < NKG; ++kg) {
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            Frag xa = *reinterpret_cast<const Frag*>(lds + tile_row<MT>(mt, r) * LDSROW + kg * KG + hf * HW);
+            Tr::mma(ua[mt], xa, held_a[kg]);
+            Tr::mma(ux[mt], xa, held_x[kg]);
+          }
+        }
+      } else {
+        for (int kk = 0; kk < kcw; kk += KG) {
+          Frag fa = *reinterpret_cast<const Frag*>(w_a_row + kc0 + kk);
+          Frag fx = *reinterpret_cast<const Frag*>(w_x_row + kc0 + kk);
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            Frag xa = *reinterpret_cast<const Frag*>(lds + tile_row<MT>(mt, r) * LDSROW + kk + hf * HW);
+            Tr::mma(ua[mt], xa, fa);
+            Tr::mma(ux[mt], xa, fx);
+          }
+        }
+      }
+      const int own = slab * 32 - kc0;                    // first column of this wave's slab in the slice
+      if (own >= 0 && own < kcw) {
+#pragma unroll
+        for (int e = 0; e < 16 * MT; ++e) xv[e] = (float)lds[(hf * 16 * MT + e) * LDSROW + own + r];
+      }
+    }
+    __syncthreads();
+  }
+}
+
+template <typename IO, int NKG>
+RGLRU_DEVICE void load_held(const IO* w_a_row, const IO* w_x_row,
+                            typename Io<IO>::Frag (&held_a)[NKG > 0 ? NKG : 1],
+                            typename Io<IO>::Frag (&held_x)[NKG > 0 ? NKG : 1]) {
+  typedef Io<IO> Tr;
+  if constexpr (NKG > 0) {
+#pragma unroll
+    for (int kg = 0; kg < NKG; ++kg) {
+      held_a[kg] = *reinterpret_cast<const typename Tr::Frag*>(w_a_row + kg * Tr::KG);
+      held_x[kg] = *reinterpret_cast<const typename Tr::Frag*>(w_x_row + kg * Tr::KG);
+    }
+  } else {
+    held_a[0] = Tr::zero(); held_x[0] = Tr::zero();
+  }
+}
+
+// Identity of the wave inside its unit; shared by the kernels below.
+struct WaveId {
+  int lane, r, hf, wave, unit, wg_in_unit, k, slab, o, ch, kp;
+  bool slab_ok, ch_ok;
+};
+
+RGLRU_DEVICE WaveId wave_identity(const FusedArgs& p, int block) {
+  WaveId w;
+  w.lane = threadIdx.x & 63; w.r = w.lane & 31; w.hf = w.lane >> 5; w.wave = threadIdx.x >> 6;
+  w.unit = block % p.units; w.wg_in_unit = block / p.units;
+  w.k = w.unit / p.groups;
+  w.slab = (w.unit % p.groups) * kWaves + w.wave;
+  w.slab_ok = w.slab < p.S;
+  w.o = w.slab * 32 + w.r;
+  w.ch_ok = w.slab_ok && w.o < p.bw;
+  w.ch = w.k * p.bw + w.o;
+  w.kp = w.k * p.bwp + (w.slab_ok ? w.o : 0);
+  return w;
+}
+
+RGLRU_DEVICE unsigned token_flags(const FusedArgs& p, long long token_row, long long rows_total) {
+  if (token_row >= rows_total) return RGLRU_FLAG_INACTIVE;
+  return p.flags ? (unsigned)p.flags[token_row] : 0u;
+}
+
+// ------------------------------------------------------------------------------------------
+// Forward
+// ------------------------------------------------------------------------------------------
+template <typename IO, int NKG>
+__global__ __launch_bounds__(kThreads) void fwd_kernel(FusedArgs p) {
+  constexpr int MT = 2, TR = 32 * MT, EL = 16 * MT;
+  typedef Io<IO> Tr;
+  typedef typename Tr::Frag Frag;
+  __shared__ __attribute__((aligned(16))) IO lds[TR * (Tr::KCMAX + Tr::HW)];
+  __shared__ unsigned s_ticket;
+
+  const WaveId w = wave_identity(p, blockIdx.x);
+  const int hf = w.hf;
+  const IO* wg = (const IO*)p.wg;
+  const IO* w_a_row = wg + ((long long)(0 * p.nb + w.k) * p.bwp + (w.slab_ok ? w.o : 0)) * p.bwp + hf * Tr::HW;
+  const IO* w_x_row = wg + ((long long)(1 * p.nb + w.k) * p.bwp + (w.slab_ok ? w.o : 0)) * p.bwp + hf * Tr::HW;
+  Frag held_a[NKG > 0 ? NKG : 1], held_x[NKG > 0 ? NKG : 1];
+  load_held<IO, NKG>(w_a_row, w_x_row, held_a, held_x);
+  const float bias_a = p.bias[w.kp], bias_x = p.bias[p.Wp + w.kp];
+  const float sp = w.ch_ok ? p.sp[w.kp] : 0.f;
+  const IO* x = (const IO*)p.x;
+  IO* y = (IO*)p.y;
+  const long long W = p.W;
+
+  for (;;) {
+    if (threadIdx.x == 0) s_ticket = atomicAdd(p.ticket + w.unit, 1u);
+    __syncthreads();
+    const long long tk = s_ticket;
+    if (tk >= p.tiles_per_unit) break;
+    const int c = (int)(tk / p.B), b = (int)(tk - (long long)c * p.B);
+    const int t0 = c * TR;
+
+    f32x16 ua[MT], ux[MT];
+    float xv[EL];
+    gate_tile<IO, MT, NKG>(p, x + (long long)b * p.T * W, t0, p.T, w.k, w.slab, w.slab_ok, w_a_row, w_x_row,
+                           held_a, held_x, bias_a, bias_x, lds, ua, ux, xv);
+    if (!w.slab_ok) continue;                             // no barrier is skipped: gate_tile ended on one
+
+    // gate math, in time order for this lane: local step e <-> t0 + hf * EL + e
+    float a[EL], z[EL];
+    const long long trow = (long long)b * p.T + t0 + hf * EL;
+#pragma unroll
+    for (int e = 0; e < EL; ++e) {
+      unsigned fl = (t0 + hf * EL + e < p.T) ? (p.flags ? (unsigned)p.flags[trow + e] : 0u) : RGLRU_FLAG_INACTIVE;
+      GateOut go = gate_forward(ua[e >> 4][e & 15], ux[e >> 4][e & 15], xv[e], sp, fl);
+      a[e] = go.a; z[e] = go.z;
+    }
+    // affine map of this lane's run, then of the whole tile
+    float A = 1.f, H = 0.f;
+#pragma unroll
+    for (int e = 0; e < EL; ++e) { H = fmaf(a[e], H, z[e]); A *= a[e]; }
+    const float A_o = xhalf(A, hf), H_o = xhalf(H, hf);
+    const float A_lo = hf ? A_o : A, H_lo = hf ? H_o : H;
+    const float A_hi = hf ? A : A_o, H_hi = hf ? H : H_o;
+    const float A_t = A_hi * A_lo, H_t = fmaf(A_hi, H_lo, H_hi);
+
+    CarryChain chain;
+    const long long seq_f = (long long)b * p.nCf * W + w.ch;
+    chain.agg_a = p.agg_a + seq_f; chain.agg_h = p.agg_h + seq_f; chain.stride = W;
+    chain.incl = p.ckpt + ((long long)b * p.ckpt_nC + 1) * W + w.ch;        // state after tile p is checkpoint 2p+1
+    chain.incl_stride = 2 * W;
+    chain.status = p.status + (long long)b * p.nCf * p.slabs + (w.k * p.S + w.slab);
+    chain.status_stride = p.slabs;
+
+    float h_in;
+    if (c == 0) {
+      h_in = (w.ch_ok && p.h0) ? p.h0[(long long)b * W + w.ch] : 0.f;
+    } else {
+      if (w.ch_ok && hf == 0) { st_coherent(chain.agg_a + c * W, A_t); st_coherent(chain.agg_h + c * W, H_t); }
+      carry_publish(chain.status + (long long)c * chain.status_stride, 1u);
+      h_in = carry_lookback(chain, c, -1, -1, 0.f, w.ch_ok, p.limit, p.fail);
+    }
+    const float h_end = fmaf(A_t, h_in, H_t);
+    const float h_mid = fmaf(A_lo, h_in, H_lo);
+    if (w.ch_ok) {
+      if (hf == 0) st_coherent(chain.incl + c * chain.incl_stride, h_end);
+      else p.ckpt[((long long)b * p.ckpt_nC + 2 * c) * W + w.ch] = h_mid;
+    }
+    carry_publish(chain.status + (long long)c * chain.status_stride, 2u);
+    if (c == p.nCf - 1 && p.h_last && w.ch_ok && hf == 0) p.h_last[(long long)b * W + w.ch] = h_end;
+
+    float h = hf ? h_mid : h_in;
+    IO* yrow = y + trow * W + w.ch;
+#pragma unroll
+    for (int e = 0; e < EL; ++e) {
+      h = fmaf(a[e], h, z[e]);
+      if (w.ch_ok && (t0 + hf * EL + e < p.T)) yrow[e * W] = (IO)h;
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// Backward (gate recomputation + reverse scan).  Chunks of 32 tokens, walked from the last to the
+// first.  Emits the direct input gradient, the gradients at both gate pre-activations and
+// per-workgroup partial sums for the bias and Lambda gradients.
+// ------------------------------------------------------------------------------------------
+template <typename IO, int NKG>
+__global__ __launch_bounds__(kThreads) void bwd_kernel(FusedArgs p) {
+  constexpr int MT = 1, TR = 32, EL = 16;
+  typedef Io<IO> Tr;
+  typedef typename Tr::Frag Frag;
+  __shared__ __attribute__((aligned(16))) IO lds[TR * (Tr::KCMAX + Tr::HW)];
+  __shared__ unsigned s_ticket;
+
+  const WaveId w = wave_identity(p, blockIdx.x);
+  const int hf = w.hf;
+  const IO* wg = (const IO*)p.wg;
+  const IO* w_a_row = wg + ((long long)(0 * p.nb + w.k) * p.bwp + (w.slab_ok ? w.o : 0)) * p.bwp + hf * Tr::HW;
+  const IO* w_x_row = wg + ((long long)(1 * p.nb + w.k) * p.bwp + (w.slab_ok ? w.o : 0)) * p.bwp + hf * Tr::HW;
+  Frag held_a[NKG > 0 ? NKG : 1], held_x[NKG > 0 ? NKG : 1];
+  load_held<IO, NKG>(w_a_row, w_x_row, held_a, held_x);
+  const float bias_a = p.bias[w.kp], bias_x = p.bias[p.Wp + w.kp];
+  const float sp = w.ch_ok ? p.sp[w.kp] : 0.f;
+  const float cs = w.ch_ok ? p.cs[w.kp] : 0.f;
+  const IO* x = (const IO*)p.x;
+  const IO* dy = (const IO*)p.dy;
+  IO* dx = (IO*)p.dx; IO* dua = (IO*)p.du_a; IO* dux = (IO*)p.du_x;
+  const long long W = p.W;
+  float sum_ba = 0.f, sum_bx = 0.f, sum_l = 0.f;
+
+  for (;;) {
+    if (threadIdx.x == 0) s_ticket = atomicAdd(p.ticket + w.unit, 1u);
+    __syncthreads();
+    const long long tk = s_ticket;
+    if (tk >= p.tiles_per_unit) break;
+    const int cr = (int)(tk / p.B), b = (int)(tk - (long long)cr * p.B);
+    const int c = p.nC - 1 - cr;
+    const int t0 = c * TR;
+
+    f32x16 ua[MT], ux[MT];
+    float xv[EL];
+    gate_tile<IO, MT, NKG>(p, x + (long long)b * p.T * W, t0, p.T, w.k, w.slab, w.slab_ok, w_a_row, w_x_row,
+                           held_a, held_x, bias_a, bias_x, lds, ua, ux, xv);
+    if (!w.slab_ok) continue;
+
+    const long long trow = (long long)b * p.T + t0 + hf * EL;
+    float r[EL], gi[EL], a[EL], g[EL], g2[EL], z[EL], gy[EL];
+    unsigned flv[EL];
+#pragma unroll
+    for (int e = 0; e < EL; ++e) {
+      const bool in = t0 + hf * EL + e < p.T;
+      unsigned fl = in ? (p.flags ? (unsigned)p.flags[trow + e] : 0u) : RGLRU_FLAG_INACTIVE;
+      flv[e] = fl;
+      GateOut go = gate_forward(ua[0][e], ux[0][e], xv[e], sp, fl);
+      r[e] = go.r; gi[e] = go.i; a[e] = go.a; g[e] = go.g; g2[e] = go.g2; z[e] = go.z;
+      gy[e] = (in && w.ch_ok) ? (float)dy[(trow + e) * W + w.ch] : 0.f;
+    }
+    // forward recomputation of h_{t-1} from the chunk checkpoint
+    float A = 1.f, H = 0.f;
+#pragma unroll
+    for (int e = 0; e < EL; ++e) { H = fmaf(a[e], H, z[e]); A *= a[e]; }
+    const float A_o = xhalf(A, hf), H_o = xhalf(H, hf);
+    const float A_lo = hf ? A_o : A, H_lo = hf ? H_o : H;
+    const float A_hi = hf ? A : A_o;
+    float h_start = 0.f;
+    if (w.ch_ok) {
+      if (c == 0) h_start = p.h0 ? p.h0[(long long)b * W + w.ch] : 0.f;
+      else h_start = p.ckpt[((long long)b * p.ckpt_nC + (c - 1)) * W + w.ch];
+    }
+    float h = hf ? fmaf(A_lo, h_start, H_lo) : h_start;
+    float hp[EL];
+#pragma unroll
+    for (int e = 0; e < EL; ++e) { hp[e] = h; h = fmaf(a[e], h, z[e]); }
+
+    // reverse affine map of this lane's run and of the chunk
+    float carry = 0.f;
+#pragma unroll
+    for (int e = EL - 1; e >= 0; --e) { float d = gy[e] + carry; carry = a[e] * d; }
+    const float D = carry, D_o = xhalf(D, hf);
+    const float D_lo = hf ? D_o : D, D_hi = hf ? D : D_o;
+    const float A_t = A_lo * A_hi, D_t = fmaf(A_lo, D_hi, D_lo);
+
+    CarryChain chain;
+    const long long seq = (long long)b * p.nC * W + w.ch;
+    chain.agg_a = p.agg_a + seq; chain.agg_h = p.agg_h + seq; chain.incl = p.incl + seq;
+    chain.stride = W; chain.incl_stride = W;
+    chain.status = p.status + (long long)b * p.nC * p.slabs + (w.k * p.S + w.slab);
+    chain.status_stride = p.slabs;
+
+    float d_in;
+    if (c == p.nC - 1) {
+      d_in = (w.ch_ok && p.dh_last) ? p.dh_last[(long long)b * W + w.ch] : 0.f;
+    } else {
+      if (w.ch_ok && hf == 0) { st_coherent(chain.agg_a + c * W, A_t); st_coherent(chain.agg_h + c * W, D_t); }
+      carry_publish(chain.status + (long long)c * chain.status_stride, 1u);
+      d_in = carry_lookback(chain, c, +1, p.nC, 0.f, w.ch_ok, p.limit, p.fail);
+    }
+    const float d_out = fmaf(A_t, d_in, D_t);
+    if (w.ch_ok && hf == 0) st_coherent(chain.incl + c * W, d_out);
+    carry_publish(chain.status + (long long)c * chain.status_stride, 2u);
+    if (c == 0 && p.dh0 && w.ch_ok && hf == 0) p.dh0[(long long)b * W + w.ch] = d_out;
+
+    carry = hf ? d_in : fmaf(A_hi, d_in, D_hi);
+#pragma unroll
+    for (int e = EL - 1; e >= 0; --e) {
+      const float d = gy[e] + carry;
+      carry = a[e] * d;
+      const unsigned fl = flv[e];
+      const bool rst = fl & 1u, ina = fl & 2u;
+      const float xe = xv[e];
+      // z = g * i * x
+      float dg = d * gi[e] * xe;
+      float di = d * g[e] * xe;
+      float dxd = d * g[e] * gi[e];
+      // g = sqrt(g2) with the bounded derivative; a = exp(l), g2 = 1 - exp(2l)
+      float dg2 = dg * __builtin_amdgcn_rsqf(fmaxf(4.0f * g2[e], 1e-6f));
+      float dl = fmaf(d * hp[e], a[e], -2.0f * (a[e] * a[e]) * dg2);
+      if (rst) dl = 0.f;
+      float dr = dl * cs;
+      float va = dr * r[e] * (1.0f - r[e]);
+      float vx = di * gi[e] * (1.0f - gi[e]);
+      if (ina) { dl = 0.f; va = 0.f; vx = 0.f; dxd = 0.f; }
+      sum_l = fmaf(dl, r[e], sum_l);
+      sum_ba += va; sum_bx += vx;
+      if (w.ch_ok && (t0 + hf * EL + e < p.T)) {
+        const long long at = (trow + e) * W + w.ch;
+        dx[at] = (IO)dxd; dua[at] = (IO)va; dux[at] = (IO)vx;
+      }
+    }
+  }
+  // per-workgroup partial sums (every slot is written, so the buffer needs no clearing)
+  if (w.slab_ok) {
+    sum_ba += xhalf(sum_ba, hf); sum_bx += xhalf(sum_bx, hf); sum_l += xhalf(sum_l, hf);
+    if (hf == 0) {
+      float* part = p.partial + (long long)w.wg_in_unit * 3 * p.Wp + w.k * p.bwp + w.o;
+      part[0] = sum_ba; part[p.Wp] = sum_bx; part[2 * p.Wp] = sum_l;
+    }
+  }
+}
+
+struct ReduceArgs {
+  const float* partial; const float* lambda; float* db_a; float* db_x; float* dlambda;
+  int W, bw, bwp, Wp, wg_per_unit; float c;
+};
+
+__global__ void reduce_kernel(ReduceArgs p) {
+  int ch = blockIdx.x * blockDim.x + threadIdx.x;
+  if (ch >= p.W) return;
+  int k = ch / p.bw, o = ch - k * p.bw;
+  int kp = k * p.bwp + o;
+  float sa = 0.f, sx = 0.f, sl = 0.f;
+  for (int g = 0; g < p.wg_per_unit; ++g) {
+    const float* part = p.partial + (long long)g * 3 * p.Wp + kp;
+    sa += part[0]; sx += part[p.Wp]; sl += part[2 * p.Wp];
+  }
+  p.db_a[ch] = sa; p.db_x[ch] = sx;
+  float lam = p.lambda[ch];
+  float sig_neg = 1.0f / (1.0f + expf(lam));           // d/dLambda log sigmoid(Lambda) = sigmoid(-Lambda)
+  p.dlambda[ch] = p.c * sl * sig_neg;
+}
+
+// ------------------------------------------------------------------------------------------
+// Decode step: rows are sequences, no scan; h is updated in place.
+// ------------------------------------------------------------------------------------------
+template <typename IO, int NKG>
+__global__ __launch_bounds__(kThreads) void step_kernel(FusedArgs p) {
+  constexpr int MT = 1, TR = 32, EL = 16;
+  typedef Io<IO> Tr;
+  typedef typename Tr::Frag Frag;
+  __shared__ __attribute__((aligned(16))) IO lds[TR * (Tr::KCMAX + Tr::HW)];
+
+  const WaveId w = wave_identity(p, blockIdx.x);
+  const int hf = w.hf;
+  const IO* wg = (const IO*)p.wg;
+  const IO* w_a_row = wg + ((long long)(0 * p.nb + w.k) * p.bwp + (w.slab_ok ? w.o : 0)) * p.bwp + hf * Tr::HW;
+  const IO* w_x_row = wg + ((long long)(1 * p.nb + w.k) * p.bwp + (w.slab_ok ? w.o : 0)) * p.bwp + hf * Tr::HW;
+  Frag held_a[NKG > 0 ? NKG : 1], held_x[NKG > 0 ? NKG : 1];
+  load_held<IO, NKG>(w_a_row, w_x_row, held_a, held_x);
+  const float bias_a = p.bias[w.kp], bias_x = p.bias[p.Wp + w.kp];
+  const float sp = w.ch_ok ? p.sp[w.kp] : 0.f;
+  const long long W = p.W;
+  const long long row0 = (long long)w.wg_in_unit * TR;
+
+  f32x16 ua[MT], ux[MT];
+  float xv[EL];
+  gate_tile<IO, MT, NKG>(p, (const IO*)p.x, row0, p.B, w.k, w.slab, w.slab_ok, w_a_row, w_x_row,
+                         held_a, held_x, bias_a, bias_x, lds, ua, ux, xv);
+  if (!w.ch_ok) return;
+  IO* y = (IO*)p.y;
+#pragma unroll
+  for (int e = 0; e < EL; ++e) {
+    const long long row = row0 + hf * EL + e;
+    if (row >= p.B) break;
+    unsigned fl = p.flags ? (unsigned)p.flags[row] : 0u;
+    GateOut go = gate_forward(ua[0][e], ux[0][e], xv[e], sp, fl);
+    const long long at = row * W + w.ch;
+    float h = fmaf(go.a, p.h_state[at], go.z);
+    p.h_state[at] = h;
+    y[at] = (IO)h;
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// Host side
+// ------------------------------------------------------------------------------------------
+static int check_geometry(const char* who, int64_t W, int64_t nb, int dtype) {
+  if (dtype != RGLRU_F32 && dtype != RGLRU_BF16) return fail(RGLRU_E_ARG, "%s: dtype must be RGLRU_F32 or RGLRU_BF16, got %d", who, dtype);
+  if (W <= 0 || nb <= 0 || W % nb != 0) return fail(RGLRU_E_ARG, "%s: width %lld is not divisible into %lld gate blocks", who, (long long)W, (long long)nb);
+  if (W / nb > 512) return fail(RGLRU_E_UNSUPPORTED, "%s: gate block width %lld exceeds the supported maximum of 512", who, (long long)(W / nb));
+  if (W >= (1 << 24)) return fail(RGLRU_E_UNSUPPORTED, "%s: width too large", who);
+  return RGLRU_OK;
+}
+
+static size_t elem_size(int dtype) { return dtype == RGLRU_BF16 ? 2 : 4; }
+
+static void fill_common(FusedArgs& a, const Geometry& g, const void* prep, int dtype) {
+  PrepLayout pl = make_prep_layout(g, elem_size(dtype));
+  const char* pb = (const char*)prep;
+  a.wg = pb + pl.wg; a.bias = (const float*)(pb + pl.bias); a.sp = (const float*)(pb + pl.sp); a.cs = (const float*)(pb + pl.cs);
+  a.W = (int)g.W; a.nb = (int)g.nb; a.bw = (int)g.bw; a.bwp = (int)g.bwp; a.S = (int)g.S; a.Wp = (int)g.Wp;
+  a.groups = (int)g.groups; a.units = (int)g.units;
+  a.limit = spin_limit();
+}
+
+static int is_aligned(const void* ptr, int64_t W, int64_t bw, size_t es) {
+  return ((uintptr_t)ptr % 16 == 0) && ((W * (int64_t)es) % 16 == 0) && ((bw * (int64_t)es) % 16 == 0);
+}
+
+// number of register-held K groups for this block width, or 0 for the streaming variant
+static int held_groups(const Geometry& g, int dtype) {
+  if (dtype == RGLRU_BF16) {
+    if (g.bwp == 128) return 8;
+    if (g.bwp == 64) return 4;
+    if (g.bwp == 32) return 2;
+  }
+  return 0;
+}
+
+#define RGLRU_DISPATCH(KERNEL, grid, stream, args, dtype, nkg)                                         \
+  do {                                                                                                 \
+    if ((dtype) == RGLRU_BF16) {                                                                       \
+      if ((nkg) == 8) hipLaunchKernelGGL((KERNEL<__bf16, 8>), grid, dim3(kThreads), 0, stream, args);  \
+      else if ((nkg) == 4) hipLaunchKernelGGL((KERNEL<__bf16, 4>), grid, dim3(kThreads), 0, stream, args); \
+      else if ((nkg) == 2) hipLaunchKernelGGL((KERNEL<__bf16, 2>), grid, dim3(kThreads), 0, stream, args); \
+      else hipLaunchKernelGGL((KERNEL<__bf16, 0>), grid, dim3(kThreads), 0, stream, args);             \
+    } else {                                                                                           \
+      hipLaunchKernelGGL((KERNEL<float, 0>), grid, dim3(kThreads), 0, stream, args);                   \
+    }                                                                                                  \
+  } while (0)
+
+static int launch_clear(char* base, size_t begin, size_t end, hipStream_t s) {
+  long long words = (long long)(end - begin) / 4;
+  int cb = (int)((words + 255) / 256); if (cb > 1024) cb = 1024; if (cb < 1) cb = 1;
+  hipLaunchKernelGGL(clear_words_kernel, dim3(cb), dim3(256), 0, s, (unsigned*)(base + begin), words);
+  return check_launch("workspace clear");
+}
+
+static int pick_wg_per_unit(const Geometry& g, long long tiles_per_unit, int per_cu, long long cap) {
+  long long target = (long long)num_compute_units() * per_cu;
+  long long n = (target + g.units - 1) / g.units;
+  if (n > tiles_per_unit) n = tiles_per_unit;
+  if (n > cap) n = cap;
+  if (n < 1) n = 1;
+  return (int)n;
+}
+
+}  // namespace rglru
+
+using namespace rglru;
+
+extern "C" {
+
+int rglru_hip_max_block_width(void) { return 512; }
+
+size_t rglru_hip_prep_bytes(int64_t W, int64_t nb, int dtype) {
+  if (check_geometry("prep_bytes", W, nb, dtype)) return 0;
+  return make_prep_layout(make_geometry(W, nb), elem_size(dtype)).total;
+}
+
+int rglru_hip_prepare(const void* w_a, const float* b_a, const void* w_x, const float* b_x,
+                      const float* lambda, float c, int64_t W, int64_t nb, int dtype,
+                      void* prep, void* stream) {
+  int rc = check_geometry("prepare", W, nb, dtype);
+  if (rc) return rc;
+  if (!w_a || !b_a || !w_x || !b_x || !lambda || !prep) return fail(RGLRU_E_ARG, "prepare: null pointer");
+  Geometry g = make_geometry(W, nb);
+  PrepLayout pl = make_prep_layout(g, elem_size(dtype));
+  char* pb = (char*)prep;
+  PrepArgs a;
+  a.w_a = w_a; a.w_x = w_x; a.b_a = b_a; a.b_x = b_x; a.lambda = lambda;
+  a.wg = pb + pl.wg; a.bias = (float*)(pb + pl.bias); a.sp = (float*)(pb + pl.sp); a.cs = (float*)(pb + pl.cs);
+  a.W = (int)W; a.nb = (int)nb; a.bw = (int)g.bw; a.bwp = (int)g.bwp; a.Wp = (int)g.Wp; a.c = c;
+  long long total = 2 * g.nb * g.bwp * g.bwp + g.Wp;
+  int blocks = (int)((total + 255) / 256); if (blocks > 2048) blocks = 2048;
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == RGLRU_BF16) hipLaunchKernelGGL(prepare_kernel<__bf16>, dim3(blocks), dim3(256), 0, s, a);
+  else hipLaunchKernelGGL(prepare_kernel<float>, dim3(blocks), dim3(256), 0, s, a);
+  return check_launch("prepare");
+}
+
+size_t rglru_hip_workspace_bytes(int64_t B, int64_t T, int64_t W, int64_t nb) {
+  if (B <= 0 || T <= 0 || W <= 0 || nb <= 0 || W % nb) return 0;
+  return make_work_layout(B, T, make_geometry(W, nb)).total;
+}
+
+int rglru_hip_fwd(const void* x, const void* prep, const float* h0, const uint8_t* flags,
+                  void* y, float* h_last, void* ws,
+                  int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, void* stream) {
+  int rc = check_geometry("fwd", W, nb, dtype);
+  if (rc) return rc;
+  if (B <= 0 || T <= 0) return fail(RGLRU_E_ARG, "fwd: B and T must be positive (got %lld, %lld)", (long long)B, (long long)T);
+  if (!x || !prep || !y || !ws) return fail(RGLRU_E_ARG, "fwd: null pointer");
+  if (B * T * W >= (1ll << 40) || B * T >= (1ll << 31)) return fail(RGLRU_E_UNSUPPORTED, "fwd: tensor too large");
+  Geometry g = make_geometry(W, nb);
+  WorkLayout L = make_work_layout(B, T, g);
+  hipStream_t s = (hipStream_t)stream;
+  char* wb = (char*)ws;
+  rc = launch_clear(wb, L.clear_begin, L.clear_end, s);
+  if (rc) return rc;
+  FusedArgs a;
+  memset(&a, 0, sizeof(a));
+  fill_common(a, g, prep, dtype);
+  a.x = x; a.h0 = h0; a.flags = flags; a.y = y; a.h_last = h_last;
+  a.ckpt = (float*)(wb + L.ckpt); a.agg_a = (float*)(wb + L.f_agg_a); a.agg_h = (float*)(wb + L.f_agg_h);
+  a.status = (unsigned*)(wb + L.f_status); a.ticket = (unsigned*)(wb + L.f_ticket); a.fail = (unsigned*)(wb + L.fail);
+  a.B = (int)B; a.T = (int)T; a.nC = (int)L.nC; a.ckpt_nC = (int)L.nC; a.nCf = (int)L.nCf; a.slabs = (int)L.slabs;
+  a.aligned = is_aligned(x, W, g.bw, elem_size(dtype));
+  a.tiles_per_unit = B * L.nCf;
+  a.wg_per_unit = pick_wg_per_unit(g, a.tiles_per_unit, 2, 1 << 20);
+  dim3 grid((unsigned)(a.wg_per_unit * g.units));
+  RGLRU_DISPATCH(fwd_kernel, grid, s, a, dtype, held_groups(g, dtype));
+  return check_launch("fwd");
+}
+
+int rglru_hip_bwd(const void* x, const void* prep, const float* lambda, const float* h0,
+                  const uint8_t* flags, const void* dy, const float* dh_last, void* ws,
+                  void* dx, void* du_a, void* du_x, float* db_a, float* db_x, float* dlambda,
+                  float* dh0, int64_t B, int64_t T, int64_t W, int64_t nb, float c, int dtype,
+                  void* stream) {
+  int rc = check_geometry("bwd", W, nb, dtype);
+  if (rc) return rc;
+  if (B <= 0 || T <= 0) return fail(RGLRU_E_ARG, "bwd: B and T must be positive (got %lld, %lld)", (long long)B, (long long)T);
+  if (!x || !prep || !lambda || !dy || !ws || !dx || !du_a || !du_x || !db_a || !db_x || !dlambda)
+    return fail(RGLRU_E_ARG, "bwd: null pointer");
+  if (B * T * W >= (1ll << 40) || B * T >= (1ll << 31)) return fail(RGLRU_E_UNSUPPORTED, "bwd: tensor too large");
+  Geometry g = make_geometry(W, nb);
+  WorkLayout L = make_work_layout(B, T, g);
+  hipStream_t s = (hipStream_t)stream;
+  char* wb = (char*)ws;
+  rc = launch_clear(wb, L.b_status, L.clear_end, s);      // backward status words, tickets, failure word
+  if (rc) return rc;
+  FusedArgs a;
+  memset(&a, 0, sizeof(a));
+  fill_common(a, g, prep, dtype);
+  a.x = x; a.h0 = h0; a.flags = flags; a.dy = dy; a.dh_last = dh_last;
+  a.dx = dx; a.du_a = du_a; a.du_x = du_x; a.dh0 = dh0;
+  a.ckpt = (float*)(wb + L.ckpt); a.agg_a = (float*)(wb + L.b_agg_a); a.agg_h = (float*)(wb + L.b_agg_h);
+  a.incl = (float*)(wb + L.b_incl);
+  a.status = (unsigned*)(wb + L.b_status); a.ticket = (unsigned*)(wb + L.b_ticket); a.fail = (unsigned*)(wb + L.fail);
+  a.partial = (float*)(wb + L.partial);
+  a.B = (int)B; a.T = (int)T; a.nC = (int)((T + kChunk - 1) / kChunk); a.ckpt_nC = (int)L.nC; a.nCf = (int)L.nCf; a.slabs = (int)L.slabs;
+  a.aligned = is_aligned(x, W, g.bw, elem_size(dtype));
+  a.tiles_per_unit = B * (long long)a.nC;
+  a.wg_per_unit = pick_wg_per_unit(g, a.tiles_per_unit, 2, L.max_wg);
+  dim3 grid((unsigned)(a.wg_per_unit * g.units));
+  RGLRU_DISPATCH(bwd_kernel, grid, s, a, dtype, held_groups(g, dtype));
+  rc = check_launch("bwd");
+  if (rc) return rc;
+  ReduceArgs r;
+  r.partial = a.partial; r.lambda = lambda; r.db_a = db_a; r.db_x = db_x; r.dlambda = dlambda;
+  r.W = (int)W; r.bw = (int)g.bw; r.bwp = (int)g.bwp; r.Wp = (int)g.Wp; r.wg_per_unit = a.wg_per_unit; r.c = c;
+  hipLaunchKernelGGL(reduce_kernel, dim3((unsigned)((W + 255) / 256)), dim3(256), 0, s, r);
+  return check_launch("bwd reduce");
+}
+
+int rglru_hip_step(const void* x, const void* prep, float* h, const uint8_t* flags, void* y,
+                   int64_t B, int64_t W, int64_t nb, int dtype, void* stream) {
+  int rc = check_geometry("step", W, nb, dtype);
+  if (rc) return rc;
+  if (B <= 0) return fail(RGLRU_E_ARG, "step: B must be positive (got %lld)", (long long)B);
+  if (!x || !prep || !h || !y) return fail(RGLRU_E_ARG, "step: null pointer");
+  if (B * W >= (1ll << 40)) return fail(RGLRU_E_UNSUPPORTED, "step: tensor too large");
+  Geometry g = make_geometry(W, nb);
+  FusedArgs a;
+  memset(&a, 0, sizeof(a));
+  fill_common(a, g, prep, dtype);
+  a.x = x; a.flags = flags; a.y = y; a.h_state = h;
+  a.B = (int)B; a.T = 1;
+  a.aligned = is_aligned(x, W, g.bw, elem_size(dtype));
+  long long row_tiles = (B + 31) / 32;
+  dim3 grid((unsigned)(row_tiles * g.units));
+  hipStream_t s = (hipStream_t)stream;
+  RGLRU_DISPATCH(step_kernel, grid, s, a, dtype, held_groups(g, dtype));
+  return check_launch("step");
+}
+
+int rglru_hip_workspace_status(const void* ws, int64_t B, int64_t T, int64_t W, int64_t nb,
+                               int scan_only, void* stream, int* status) {
+  if (!ws || !status) return fail(RGLRU_E_ARG, "workspace_status: null pointer");
+  size_t off;
+  if (scan_only) off = make_scan_layout(B, T, W).fail;
+  else {
+    if (nb <= 0 || W % nb) return fail(RGLRU_E_ARG, "workspace_status: bad geometry");
+    off = make_work_layout(B, T, make_geometry(W, nb)).fail;
+  }
+  unsigned word = 0;
+  hipError_t e = hipMemcpyAsync(&word, (const char*)ws + off, 4, hipMemcpyDeviceToHost, (hipStream_t)stream);
+  if (e == hipSuccess) e = hipStreamSynchronize((hipStream_t)stream);
+  if (e != hipSuccess) return fail(RGLRU_E_LAUNCH, "workspace_status: %s", hipGetErrorString(e));
+  *status = (int)word;
+  return RGLRU_OK;
+}
+
+}  // extern "C"

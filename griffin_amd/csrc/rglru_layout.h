@@ -1,0 +1,116 @@
+// Byte layouts of the two opaque buffers of the C ABI, computed identically on host and device.
+#pragma once
+
+#include <stddef.h>
+#include <stdint.h>
+
+namespace rglru {
+
+inline int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
+
+// Geometry derived from (W, nb): block width, padded block width, 32-channel slabs.
+struct Geometry {
+  int64_t W, nb, bw, bwp, S, Wp;      // Wp = nb * bwp padded channels; S slabs per block
+  int64_t groups;                      // workgroups needed to cover one block (4 slabs each)
+  int64_t units;                       // nb * groups: independent weight sets
+};
+
+inline Geometry make_geometry(int64_t W, int64_t nb) {
+  Geometry g;
+  g.W = W; g.nb = nb; g.bw = W / nb;
+  g.bwp = round_up(g.bw, 32);
+  g.S = g.bwp / 32;
+  g.Wp = nb * g.bwp;
+  g.groups = (g.S + 3) / 4;
+  g.units = nb * g.groups;
+  return g;
+}
+
+// Prepared parameter image.
+//   wg    [2][nb][bwp][bwp]  storage type, zero padded: gate weights, row = output channel
+//   bias  [2][Wp]            fp32
+//   sp    [Wp]               fp32   c * log2(sigmoid(Lambda))
+//   cs    [Wp]               fp32   c * log(sigmoid(Lambda))
+struct PrepLayout {
+  size_t wg, bias, sp, cs, total;
+};
+
+inline PrepLayout make_prep_layout(const Geometry& g, size_t elem) {
+  PrepLayout p;
+  size_t off = 0;
+  p.wg = off;   off += (size_t)round_up(2 * g.nb * g.bwp * g.bwp * (int64_t)elem, 256);
+  p.bias = off; off += (size_t)round_up(2 * g.Wp * 4, 256);
+  p.sp = off;   off += (size_t)round_up(g.Wp * 4, 256);
+  p.cs = off;   off += (size_t)round_up(g.Wp * 4, 256);
+  p.total = off;
+  return p;
+}
+
+// Workspace of one forward/backward pair.  nC = chunks of 32 tokens (rounded up to even),
+// nCf = forward tiles of 64 tokens, slabs = nb * S status words per (sequence, chunk).
+//   ckpt        [B][nC][W]   fp32 state after each chunk (kept for backward)
+//   f_agg_a/h   [B][nCf][W]  forward carry records
+//   b_agg_a/h, b_incl [B][nC][W]  backward carry records
+//   partial     [maxWg][3][Wp]  per-workgroup sums for db_a, db_x, dLambda
+//   --- cleared before each pass ---
+//   f_status    [B][nCf][slabs]   b_status [B][nC][slabs]
+//   f_ticket    [units]           b_ticket [units]
+//   fail        [1]
+struct WorkLayout {
+  int64_t nC, nCf, slabs, max_wg;
+  size_t ckpt, f_agg_a, f_agg_h, b_agg_a, b_agg_h, b_incl, partial;
+  size_t clear_begin, f_status, b_status, f_ticket, b_ticket, fail, clear_end, total;
+};
+
+inline WorkLayout make_work_layout(int64_t B, int64_t T, const Geometry& g) {
+  WorkLayout w;
+  w.nCf = (T + 63) / 64;
+  w.nC = 2 * w.nCf;
+  w.slabs = g.nb * g.S;
+  w.max_wg = 256;                      // most workgroups one unit may use in backward
+  size_t off = 0;
+  auto take = [&](int64_t bytes) { size_t at = off; off += (size_t)round_up(bytes, 256); return at; };
+  w.ckpt = take(B * w.nC * g.W * 4);
+  w.f_agg_a = take(B * w.nCf * g.W * 4);
+  w.f_agg_h = take(B * w.nCf * g.W * 4);
+  w.b_agg_a = take(B * w.nC * g.W * 4);
+  w.b_agg_h = take(B * w.nC * g.W * 4);
+  w.b_incl = take(B * w.nC * g.W * 4);
+  w.partial = take(w.max_wg * 3 * g.Wp * 4);
+  w.clear_begin = off;
+  w.f_status = take(B * w.nCf * w.slabs * 4);
+  w.b_status = take(B * w.nC * w.slabs * 4);
+  w.f_ticket = take(g.units * 4);
+  w.b_ticket = take(g.units * 4);
+  w.fail = take(4);
+  w.clear_end = off;
+  w.total = off;
+  return w;
+}
+
+// Scan-only workspace: chunks of 32 tokens, groups of 64 channels.
+//   agg_a, agg_h, incl [B][nC][W]; then (cleared) status [B][nC][groups], ticket, fail.
+struct ScanLayout {
+  int64_t nC, groups;
+  size_t agg_a, agg_h, incl, clear_begin, status, ticket, fail, clear_end, total;
+};
+
+inline ScanLayout make_scan_layout(int64_t B, int64_t T, int64_t W) {
+  ScanLayout s;
+  s.nC = (T + 31) / 32;
+  s.groups = (W + 63) / 64;
+  size_t off = 0;
+  auto take = [&](int64_t bytes) { size_t at = off; off += (size_t)round_up(bytes, 256); return at; };
+  s.agg_a = take(B * s.nC * W * 4);
+  s.agg_h = take(B * s.nC * W * 4);
+  s.incl = take(B * s.nC * W * 4);
+  s.clear_begin = off;
+  s.status = take(B * s.nC * s.groups * 4);
+  s.ticket = take(4);
+  s.fail = take(4);
+  s.clear_end = off;
+  s.total = off;
+  return s;
+}
+
+}  // namespace rglru

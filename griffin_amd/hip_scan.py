@@ -1,0 +1,363 @@
+"""PyTorch operators over the C ABI of librglru_hip.so, and the one-time device self-test.
+
+Mirrors the reference's operator module (griffin/triton_scan.py): ``hip_rglru_scan`` has the
+contract of ``fused_rglru_scan`` (:274-276), ``hip_scan_available`` / ``hip_scan_is_usable`` those of
+``triton_scan_available`` / ``triton_scan_is_usable`` (:125-127, :180-204).  ``hip_rglru`` is one
+fusion level higher: it takes x and the RG-LRU parameters and runs gates + scan in one kernel.
+
+There is no CPU fallback in this file: every operator raises when the library or a GPU is missing.
+"""
+
+from __future__ import annotations
+
+import threading
+import warnings
+
+import torch
+from torch import Tensor
+from torch.autograd.function import once_differentiable
+
+from . import _lib
+
+_VALIDATION_LOCK = threading.Lock()
+_VALIDATED: dict[int, bool] = {}
+
+SUPPORTED_DTYPES = (torch.float32, torch.bfloat16)
+
+
+def hip_scan_available() -> bool:
+    """Whether the HIP library is built and loads (reference: triton_scan_available)."""
+    return _lib.available()
+
+
+def _stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _ptr(t: Tensor | None) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+def _require_gpu(name: str, *tensors: Tensor) -> None:
+    _lib.load()  # raises RuntimeError when the extension is missing
+    if not torch.cuda.is_available():
+        raise RuntimeError(f"{name} requires a CUDA/HIP device, none is available")
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError(f"{name} requires CUDA/HIP tensors, got a {t.device.type} tensor")
+
+
+# ----------------------------------------------------------------------------------------------
+# scan-only operator: h_t = a_t h_{t-1} + z_t
+# ----------------------------------------------------------------------------------------------
+class _HipScan(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, decay: Tensor, current_input: Tensor, initial_state: Tensor) -> Tensor:
+        _require_gpu("hip_rglru_scan", decay, current_input, initial_state)
+        if decay.dim() != 3 or decay.shape != current_input.shape:
+            raise ValueError("decay and current_input must share shape [batch, sequence, width]")
+        if initial_state.shape != (decay.size(0), decay.size(2)):
+            raise ValueError("initial_state must have shape [batch, width]")
+        if decay.dtype != torch.float32 or current_input.dtype != torch.float32:
+            raise TypeError("hip_rglru_scan expects fp32 decay and normalized input")
+        if initial_state.dtype != torch.float32:
+            raise TypeError("hip_rglru_scan expects fp32 recurrent state")
+        lib = _lib.load()
+        decay = decay.contiguous()
+        current_input = current_input.contiguous()
+        initial_state = initial_state.contiguous()
+        B, T, W = decay.shape
+        out = torch.empty_like(current_input)
+        if out.numel() == 0:
+            ctx.save_for_backward(decay, initial_state, out)
+            return out
+        with torch.cuda.device(decay.device):
+            ws = torch.empty(lib.rglru_hip_scan_workspace_bytes(B, T, W), dtype=torch.uint8, device=decay.device)
+            _lib.check(lib.rglru_hip_scan_fwd(decay.data_ptr(), current_input.data_ptr(), initial_state.data_ptr(),
+                                              out.data_ptr(), ws.data_ptr(), B, T, W, _stream_ptr(decay.device)),
+                       "rglru_hip_scan_fwd")
+        ctx.save_for_backward(decay, initial_state, out)
+        return out
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, grad_out: Tensor):
+        decay, initial_state, out = ctx.saved_tensors
+        lib = _lib.load()
+        grad_out = grad_out.contiguous()
+        B, T, W = decay.shape
+        d_decay = torch.empty_like(decay)
+        d_input = torch.empty_like(decay)
+        d_state = torch.empty_like(initial_state)
+        if decay.numel() == 0:
+            return d_decay, d_input, d_state.zero_()
+        with torch.cuda.device(decay.device):
+            ws = torch.empty(lib.rglru_hip_scan_workspace_bytes(B, T, W), dtype=torch.uint8, device=decay.device)
+            _lib.check(lib.rglru_hip_scan_bwd(decay.data_ptr(), initial_state.data_ptr(), out.data_ptr(),
+                                              grad_out.data_ptr(), d_decay.data_ptr(), d_input.data_ptr(),
+                                              d_state.data_ptr(), ws.data_ptr(), B, T, W, _stream_ptr(decay.device)),
+                       "rglru_hip_scan_bwd")
+        return d_decay, d_input, d_state
+
+
+def hip_rglru_scan(decay: Tensor, current_input: Tensor, initial_state: Tensor) -> Tensor:
+    """Differentiable linear recurrence on the GPU (contract of griffin/triton_scan.py:274-276)."""
+    return _HipScan.apply(decay, current_input, initial_state)
+
+
+# ----------------------------------------------------------------------------------------------
+# fused operator: gates + scan
+# ----------------------------------------------------------------------------------------------
+def _dtype_code(dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return _lib.RGLRU_F32
+    if dtype == torch.bfloat16:
+        return _lib.RGLRU_BF16
+    raise TypeError(f"hip RG-LRU supports float32 and bfloat16 activations, got {dtype}")
+
+
+def pack_flags(reset_mask: Tensor | None, active_mask: Tensor | None) -> Tensor | None:
+    """One byte per token: bit 0 = reset, bit 1 = inactive.  None when no token is flagged."""
+    flags = None
+    if reset_mask is not None:
+        flags = reset_mask.to(torch.uint8)
+    if active_mask is not None:
+        idle = (~active_mask.to(torch.bool)).to(torch.uint8) * 2
+        flags = idle if flags is None else flags + idle
+    return None if flags is None else flags.contiguous()
+
+
+class PreparedParams:
+    """Kernel-side image of the RG-LRU parameters (see rglru_hip_prepare)."""
+
+    def __init__(self, w_a: Tensor, b_a: Tensor, w_x: Tensor, b_x: Tensor, lam: Tensor, c: float, dtype: torch.dtype):
+        lib = _lib.load()
+        nb, bw, _ = w_a.shape
+        self.width = nb * bw
+        self.blocks = nb
+        self.dtype = dtype
+        self.c = float(c)
+        code = _dtype_code(dtype)
+        size = lib.rglru_hip_prep_bytes(self.width, nb, code)
+        if size == 0:
+            _lib.check(2, "rglru_hip_prep_bytes")
+        device = w_a.device
+        self.lam32 = lam.detach().to(torch.float32).contiguous()
+        w_a_c = w_a.detach().to(dtype).contiguous()
+        w_x_c = w_x.detach().to(dtype).contiguous()
+        b_a_c = b_a.detach().to(torch.float32).contiguous()
+        b_x_c = b_x.detach().to(torch.float32).contiguous()
+        with torch.cuda.device(device):
+            self.image = torch.empty(size, dtype=torch.uint8, device=device)
+            _lib.check(lib.rglru_hip_prepare(w_a_c.data_ptr(), b_a_c.data_ptr(), w_x_c.data_ptr(), b_x_c.data_ptr(),
+                                             self.lam32.data_ptr(), self.c, self.width, nb, code,
+                                             self.image.data_ptr(), _stream_ptr(device)), "rglru_hip_prepare")
+
+
+def _check_fused_inputs(x: Tensor, w_a: Tensor, h0: Tensor | None, flags: Tensor | None) -> None:
+    if x.dim() != 3:
+        raise ValueError(f"hip RG-LRU expects [batch, sequence, width], got {tuple(x.shape)}")
+    B, T, W = x.shape
+    nb, bw, bw2 = w_a.shape
+    if bw != bw2 or nb * bw != W:
+        raise ValueError(f"gate weights {tuple(w_a.shape)} do not match width {W}")
+    if h0 is not None and h0.shape != (B, W):
+        raise ValueError(f"initial state must have shape ({B}, {W}), got {tuple(h0.shape)}")
+    if flags is not None and flags.shape != (B, T):
+        raise ValueError(f"token flags must have shape ({B}, {T}), got {tuple(flags.shape)}")
+    if T == 0 or B == 0:
+        raise ValueError("hip RG-LRU does not accept empty batches or sequences")
+    _dtype_code(x.dtype)
+
+
+class _HipRGLRU(torch.autograd.Function):
+    """y, h_T = RG-LRU(x; W_a, b_a, W_x, b_x, Lambda) with a recomputing backward."""
+
+    @staticmethod
+    def forward(ctx, x, w_a, b_a, w_x, b_x, lam, h0, flags, c):
+        _require_gpu("hip RG-LRU", x, w_a, b_a, w_x, b_x, lam, h0, flags)
+        _check_fused_inputs(x, w_a, h0, flags)
+        lib = _lib.load()
+        x = x.contiguous()
+        B, T, W = x.shape
+        nb = w_a.shape[0]
+        code = _dtype_code(x.dtype)
+        prep = PreparedParams(w_a, b_a, w_x, b_x, lam, c, x.dtype)
+        h0c = None if h0 is None else h0.detach().to(torch.float32).contiguous()
+        device = x.device
+        with torch.cuda.device(device):
+            y = torch.empty_like(x)
+            h_last = torch.empty(B, W, dtype=torch.float32, device=device)
+            ws = torch.empty(lib.rglru_hip_workspace_bytes(B, T, W, nb), dtype=torch.uint8, device=device)
+            _lib.check(lib.rglru_hip_fwd(x.data_ptr(), prep.image.data_ptr(), _ptr(h0c), _ptr(flags), y.data_ptr(),
+                                         h_last.data_ptr(), ws.data_ptr(), B, T, W, nb, code, _stream_ptr(device)),
+                       "rglru_hip_fwd")
+        ctx.save_for_backward(x, w_a, w_x, h0c, flags, ws, prep.image, prep.lam32)
+        ctx.c = float(c)
+        ctx.param_dtypes = (w_a.dtype, b_a.dtype, w_x.dtype, b_x.dtype, lam.dtype)
+        ctx.h0_dtype = None if h0 is None else h0.dtype
+        return y, h_last
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, dy, dh_last):
+        x, w_a, w_x, h0c, flags, ws, image, lam32 = ctx.saved_tensors
+        lib = _lib.load()
+        B, T, W = x.shape
+        nb, bw, _ = w_a.shape
+        code = _dtype_code(x.dtype)
+        device = x.device
+        dy = torch.zeros_like(x) if dy is None else dy.to(x.dtype).contiguous()
+        dhl = None if dh_last is None else dh_last.to(torch.float32).contiguous()
+        with torch.cuda.device(device):
+            dx = torch.empty_like(x)
+            du_a = torch.empty_like(x)
+            du_x = torch.empty_like(x)
+            db_a = torch.empty(W, dtype=torch.float32, device=device)
+            db_x = torch.empty(W, dtype=torch.float32, device=device)
+            dlam = torch.empty(W, dtype=torch.float32, device=device)
+            dh0 = torch.empty(B, W, dtype=torch.float32, device=device) if ctx.needs_input_grad[6] else None
+            _lib.check(lib.rglru_hip_bwd(x.data_ptr(), image.data_ptr(), lam32.data_ptr(), _ptr(h0c), _ptr(flags),
+                                         dy.data_ptr(), _ptr(dhl), ws.data_ptr(), dx.data_ptr(), du_a.data_ptr(),
+                                         du_x.data_ptr(), db_a.data_ptr(), db_x.data_ptr(), dlam.data_ptr(),
+                                         _ptr(dh0), B, T, W, nb, ctx.c, code, _stream_ptr(device)), "rglru_hip_bwd")
+            # block-diagonal GEMMs: dW[k] = du[:, k]^T x[:, k];  dx[:, k] += du[:, k] W[k]
+            n = B * T
+            xk = x.view(n, nb, bw).transpose(0, 1)               # [nb, n, bw] (strided view)
+            ua = du_a.view(n, nb, bw).transpose(0, 1)
+            ux = du_x.view(n, nb, bw).transpose(0, 1)
+            wa = w_a.detach().to(x.dtype)
+            wx = w_x.detach().to(x.dtype)
+            dw_a = torch.bmm(ua.transpose(1, 2), xk)
+            dw_x = torch.bmm(ux.transpose(1, 2), xk)
+            dxg = torch.bmm(ua, wa)
+            dxg = torch.baddbmm(dxg, ux, wx)
+            dx = (dx.view(n, nb, bw).float() + dxg.transpose(0, 1).float()).to(x.dtype).view(B, T, W)
+        pd = ctx.param_dtypes
+        grads = (dx, dw_a.to(pd[0]), db_a.view(nb, bw).to(pd[1]), dw_x.to(pd[2]), db_x.view(nb, bw).to(pd[3]),
+                 dlam.to(pd[4]), None if dh0 is None else dh0.to(ctx.h0_dtype), None, None)
+        return grads
+
+
+def hip_rglru(x: Tensor, w_a: Tensor, b_a: Tensor, w_x: Tensor, b_x: Tensor, lam: Tensor, c: float = 8.0,
+              h0: Tensor | None = None, reset_mask: Tensor | None = None,
+              active_mask: Tensor | None = None) -> tuple[Tensor, Tensor]:
+    """Fused RG-LRU on the GPU: returns (y in x.dtype, final state in fp32).  Differentiable in
+    x, the five parameters and h0 (first order)."""
+    flags = pack_flags(reset_mask, active_mask)
+    return _HipRGLRU.apply(x, w_a, b_a, w_x, b_x, lam, h0, flags, c)
+
+
+def hip_rglru_step(x: Tensor, prep: PreparedParams, state: Tensor, flags: Tensor | None = None) -> Tensor:
+    """One decode step: ``state`` [B, W] fp32 is updated in place; returns y [B, W] in x.dtype."""
+    _require_gpu("hip RG-LRU step", x, state, flags)
+    if x.dim() != 2 or x.shape[1] != prep.width:
+        raise ValueError(f"step expects x of shape [batch, {prep.width}], got {tuple(x.shape)}")
+    if state.shape != x.shape or state.dtype != torch.float32 or not state.is_contiguous():
+        raise ValueError("step expects a contiguous fp32 state of the same shape as x")
+    if x.dtype != prep.dtype:
+        raise TypeError(f"parameters were prepared for {prep.dtype}, got activations in {x.dtype}")
+    lib = _lib.load()
+    x = x.contiguous()
+    with torch.cuda.device(x.device):
+        y = torch.empty_like(x)
+        _lib.check(lib.rglru_hip_step(x.data_ptr(), prep.image.data_ptr(), state.data_ptr(), _ptr(flags),
+                                      y.data_ptr(), x.shape[0], prep.width, prep.blocks, _dtype_code(x.dtype),
+                                      _stream_ptr(x.device)), "rglru_hip_step")
+    return y
+
+
+# ----------------------------------------------------------------------------------------------
+# one-time self-test (reference: griffin/triton_scan.py:130-204)
+# ----------------------------------------------------------------------------------------------
+def _loop_scan(decay: Tensor, current_input: Tensor, state: Tensor) -> Tensor:
+    rows = []
+    for t in range(decay.size(1)):
+        state = decay[:, t] * state + current_input[:, t]
+        rows.append(state)
+    return torch.stack(rows, dim=1)
+
+
+def _validate_hip_scan(device: torch.device) -> None:
+    """Forward/backward parity of both operators against autograd through a plain loop, on the
+    seed-free inputs of the reference self-test (width 257 = one partial tile, 7 steps) and on a
+    second case long enough to cross chunk boundaries."""
+    from . import portable
+
+    for width, steps in ((257, 7), (96, 75)):
+        k = torch.arange(width * steps, device=device, dtype=torch.float32)
+        decay = (0.9 + 0.05 * torch.sin(k / 97.0)).reshape(1, steps, width)
+        inp = (0.1 * torch.cos(k / 53.0)).reshape(1, steps, width)
+        state = torch.sin(torch.arange(width, device=device) / 31.0)[None]
+        upstream = torch.cos(k / 71.0).reshape(1, steps, width)
+        ref_in = [t.detach().clone().requires_grad_(True) for t in (decay, inp, state)]
+        hip_in = [t.detach().clone().requires_grad_(True) for t in (decay, inp, state)]
+        ref_out = _loop_scan(*ref_in)
+        hip_out = hip_rglru_scan(*hip_in)
+        ref_g = torch.autograd.grad(ref_out, ref_in, upstream)
+        hip_g = torch.autograd.grad(hip_out, hip_in, upstream)
+        torch.cuda.synchronize(device)
+        torch.testing.assert_close(hip_out, ref_out, atol=2e-5, rtol=2e-5)
+        for got, want in zip(hip_g, ref_g):
+            torch.testing.assert_close(got, want, atol=3e-5, rtol=3e-5)
+
+    # fused operator on a small closed-form module: W = 48 in 3 blocks, 70 steps, reset + padding
+    B, T, W, nb = 2, 70, 48, 3
+    bw = W // nb
+    k = torch.arange(B * T * W, device=device, dtype=torch.float32)
+    x = torch.sin(k / 37.0).reshape(B, T, W)
+    kw = torch.arange(nb * bw * bw, device=device, dtype=torch.float32)
+    w_a = (0.3 * torch.cos(kw / 11.0)).reshape(nb, bw, bw)
+    w_x = (0.3 * torch.sin(kw / 13.0)).reshape(nb, bw, bw)
+    kb = torch.arange(W, device=device, dtype=torch.float32)
+    b_a = (0.1 * torch.sin(kb / 5.0)).reshape(nb, bw)
+    b_x = (0.1 * torch.cos(kb / 7.0)).reshape(nb, bw)
+    lam = 4.0 + 3.0 * torch.sin(kb / 9.0) ** 2
+    h0 = torch.cos(torch.arange(B * W, device=device, dtype=torch.float32) / 17.0).reshape(B, W)
+    reset = torch.zeros(B, T, dtype=torch.bool, device=device)
+    reset[:, 40] = True
+    active = torch.ones(B, T, dtype=torch.bool, device=device)
+    active[1, -5:] = False
+    upstream = torch.cos(k / 29.0).reshape(B, T, W)
+
+    def run(use_hip):
+        leaves = [t.detach().clone().requires_grad_(True) for t in (x, w_a, b_a, w_x, b_x, lam, h0)]
+        if use_hip:
+            y, _ = hip_rglru(*leaves[:6], 8.0, leaves[6], reset, active)
+        else:
+            a, z = portable.decay_and_input(*leaves[:6], 8.0, reset, active, torch.float32)
+            y = _loop_scan(a, z, leaves[6])
+        return y, torch.autograd.grad(y, leaves, upstream)
+
+    ref_y, ref_g = run(False)
+    hip_y, hip_g = run(True)
+    torch.cuda.synchronize(device)
+    torch.testing.assert_close(hip_y, ref_y, atol=2e-5, rtol=2e-5)
+    for got, want in zip(hip_g, ref_g):
+        scale = max(1.0, float(want.abs().max()))
+        torch.testing.assert_close(got, want, atol=3e-5 * scale, rtol=3e-5)
+
+
+def hip_scan_is_usable(device: torch.device | str) -> bool:
+    """Validate the HIP kernels once per device before ``scan_mode="auto"`` may use them."""
+    resolved = torch.device(device)
+    if resolved.type != "cuda" or not torch.cuda.is_available() or not hip_scan_available():
+        return False
+    index = torch.cuda.current_device() if resolved.index is None else resolved.index
+    with _VALIDATION_LOCK:
+        if index in _VALIDATED:
+            return _VALIDATED[index]
+        try:
+            with torch.enable_grad(), torch.cuda.device(index):
+                _validate_hip_scan(torch.device("cuda", index))
+        except Exception as error:  # launch failures and numerical mismatches both fall back
+            _VALIDATED[index] = False
+            warnings.warn(
+                "HIP RG-LRU scan failed its CUDA/HIP self-test; using the portable scan instead. "
+                f"Original error: {error}",
+                RuntimeWarning,
+                stacklevel=2,
+            )
+        else:
+            _VALIDATED[index] = True
+        return _VALIDATED[index]

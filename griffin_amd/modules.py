@@ -1,0 +1,309 @@
+"""Host-side mirror of the reference's RG-LRU module interface with a ``scan_mode="hip"`` backend.
+
+Constructor signatures, parameter names and shapes, argument validation, error types and the
+dispatch rules follow griffin/griffin.py:119-306 (RG_LRU, BlockDiagonalLinear) and :309-529
+(RecurrentBlock and its cache), so that callers, state_dicts and tests of the reference carry
+over.  What differs is the accelerator path: ``"hip"`` (explicit, fails loudly) and ``"auto"`` on
+GPU tensors (after a one-time parity self-test, with a warning and the portable scan as fallback)
+run the hand-written gfx950 kernels; the Triton backend is gone and ``"fused"`` is kept as an
+alias of ``"hip"``.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+import math
+from typing import Literal
+
+import torch
+from torch import Tensor
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import hip_scan, portable
+
+ScanMode = Literal["auto", "sequential", "associative", "hip", "fused"]
+SCAN_MODES = ("auto", "sequential", "associative", "hip", "fused")
+
+
+@dataclass
+class RecurrentBlockCache:
+    """State that lets a recurrent block continue on a later chunk (griffin/griffin.py:26-32)."""
+
+    rnn_state: Tensor
+    conv_state: Tensor
+    segment_position: Tensor
+
+
+def _compatible_block_count(width: int, requested_blocks: int) -> int:
+    """Largest block count <= requested that divides width (griffin/griffin.py:119-126)."""
+    if width <= 0 or requested_blocks <= 0:
+        raise ValueError("width and requested_blocks must be positive")
+    count = min(width, requested_blocks)
+    while width % count:
+        count -= 1
+    return count
+
+
+class BlockDiagonalLinear(nn.Module):
+    """Block-diagonal projection: weight [blocks, out, in], bias [blocks, out] (griffin/griffin.py:129-154)."""
+
+    def __init__(self, width: int, num_blocks: int = 16):
+        super().__init__()
+        self.width = width
+        self.num_blocks = _compatible_block_count(width, num_blocks)
+        self.block_width = width // self.num_blocks
+        self.weight = nn.Parameter(torch.empty(self.num_blocks, self.block_width, self.block_width))
+        self.bias = nn.Parameter(torch.empty(self.num_blocks, self.block_width))
+        self.reset_parameters()
+
+    def reset_parameters(self) -> None:
+        nn.init.normal_(self.weight, mean=0.0, std=math.sqrt(1.0 / self.block_width))
+        nn.init.zeros_(self.bias)
+
+    def forward(self, x: Tensor) -> Tensor:
+        return portable.block_diagonal_project(x, self.weight, self.bias)
+
+
+class RG_LRU(nn.Module):
+    """Real-Gated Linear Recurrent Unit (griffin/griffin.py:157-306) with a HIP scan backend."""
+
+    def __init__(self, rnn_width: int, c: float = 8.0, gate_blocks: int = 16, scan_mode: ScanMode = "auto"):
+        super().__init__()
+        self.rnn_width = rnn_width
+        self.c = c
+        if scan_mode not in SCAN_MODES:
+            raise ValueError(f"Unknown RG-LRU scan mode: {scan_mode}")
+        self.scan_mode = scan_mode
+        self.recurrence_gate = BlockDiagonalLinear(rnn_width, gate_blocks)
+        self.input_gate = BlockDiagonalLinear(rnn_width, gate_blocks)
+        self.Lambda = nn.Parameter(torch.empty(rnn_width))
+        self.reset_parameters()
+
+    def reset_parameters(self) -> None:
+        self.recurrence_gate.reset_parameters()
+        self.input_gate.reset_parameters()
+        with torch.no_grad():
+            decay_to_the_c = torch.empty_like(self.Lambda).uniform_(0.9, 0.999)
+            self.Lambda.copy_(torch.logit(decay_to_the_c.pow(1.0 / self.c)))
+
+    # -- dispatch ---------------------------------------------------------------------------
+    def _hip_covers(self, xt: Tensor) -> bool:
+        return (
+            xt.dtype in hip_scan.SUPPORTED_DTYPES
+            and self.recurrence_gate.block_width <= 512
+            and xt.numel() > 0
+        )
+
+    def forward(
+        self,
+        xt: Tensor,
+        ht_minus_1: Tensor | None = None,
+        *,
+        reset_mask: Tensor | None = None,
+        active_mask: Tensor | None = None,
+        return_state: bool = False,
+    ):
+        if xt.dim() != 3:
+            raise ValueError(f"RG_LRU expects [batch, sequence, width], got {tuple(xt.shape)}")
+        batch, steps, width = xt.shape
+        if width != self.rnn_width:
+            raise ValueError(f"Expected width {self.rnn_width}, got {width}")
+        for name, mask in (("reset_mask", reset_mask), ("active_mask", active_mask)):
+            if mask is not None and mask.shape != (batch, steps):
+                raise ValueError(f"{name} must have shape ({batch}, {steps}), got {tuple(mask.shape)}")
+        if ht_minus_1 is not None and ht_minus_1.shape != (batch, width):
+            raise ValueError(f"ht_minus_1 must have shape ({batch}, {width}), got {tuple(ht_minus_1.shape)}")
+        state_dtype = torch.float32 if xt.dtype in (torch.float16, torch.bfloat16) else xt.dtype
+        if reset_mask is not None:
+            reset_mask = reset_mask.to(device=xt.device, dtype=torch.bool)
+        if active_mask is not None:
+            active_mask = active_mask.to(device=xt.device, dtype=torch.bool)
+        if ht_minus_1 is not None:
+            ht_minus_1 = ht_minus_1.to(device=xt.device, dtype=state_dtype)
+
+        mode = self.scan_mode
+        if mode not in SCAN_MODES:
+            raise ValueError(f"Unknown RG-LRU scan mode: {mode}")
+        explicit_hip = mode in ("hip", "fused")
+        auto_hip = (
+            mode == "auto"
+            and xt.is_cuda
+            and self._hip_covers(xt)
+            and hip_scan.hip_scan_is_usable(xt.device)
+        )
+        if explicit_hip or auto_hip:
+            if explicit_hip and not xt.is_cuda:
+                raise RuntimeError(
+                    f'scan_mode="{mode}" requires CUDA/HIP tensors and the RG-LRU HIP library; '
+                    f"got a {xt.device.type} tensor"
+                )
+            y, state = hip_scan.hip_rglru(
+                xt, self.recurrence_gate.weight, self.recurrence_gate.bias, self.input_gate.weight,
+                self.input_gate.bias, self.Lambda, self.c, ht_minus_1, reset_mask, active_mask,
+            )
+            return (y, state) if return_state else y
+
+        if reset_mask is None:
+            reset_mask = torch.zeros(batch, steps, device=xt.device, dtype=torch.bool)
+        if active_mask is None:
+            active_mask = torch.ones(batch, steps, device=xt.device, dtype=torch.bool)
+        state = (
+            torch.zeros(batch, width, device=xt.device, dtype=state_dtype) if ht_minus_1 is None else ht_minus_1
+        )
+        a, z = portable.decay_and_input(
+            xt, self.recurrence_gate.weight, self.recurrence_gate.bias, self.input_gate.weight,
+            self.input_gate.bias, self.Lambda, self.c, reset_mask, active_mask, state_dtype,
+        )
+        use_associative = mode == "associative" or (mode == "auto" and xt.is_cuda and steps > 1)
+        if use_associative:
+            states = portable.associative_scan(a, z, state)
+        else:
+            states = portable.sequential_scan(a, z, state)
+        y = states.to(xt.dtype)
+        return (y, states[:, -1]) if return_state else y
+
+    _associative_scan = staticmethod(portable.associative_scan)
+
+
+def _resolve_segment_positions(x, segment_pos, previous_position=None, active_mask=None) -> Tensor:
+    """Explicit positions, or previous + running count of active tokens (griffin/griffin.py:309-338)."""
+    batch, steps = x.shape[:2]
+    if steps == 0:
+        raise ValueError("Empty token sequences are not supported")
+    if segment_pos is not None:
+        if segment_pos.shape != (batch, steps):
+            raise ValueError(f"segment_pos must have shape ({batch}, {steps}), got {tuple(segment_pos.shape)}")
+        return segment_pos.to(device=x.device, dtype=torch.long)
+    if previous_position is None:
+        start = torch.full((batch,), -1, device=x.device, dtype=torch.long)
+    else:
+        if previous_position.shape != (batch,):
+            raise ValueError("Cached segment positions have an incompatible shape")
+        start = previous_position.to(device=x.device, dtype=torch.long)
+    if active_mask is None:
+        counts = torch.arange(1, steps + 1, device=x.device, dtype=torch.long).expand(batch, steps)
+    else:
+        counts = active_mask.to(torch.long).cumsum(dim=1)
+    return start[:, None] + counts
+
+
+def _last_active_position(segment_pos: Tensor, active_mask: Tensor, previous_position: Tensor | None) -> Tensor:
+    """Position of each row's last active token, or the previous one when the row is all padding
+    (griffin/griffin.py:341-358), computed without a per-row host loop."""
+    batch, steps = segment_pos.shape
+    if previous_position is None:
+        fallback = torch.full((batch,), -1, device=segment_pos.device, dtype=torch.long)
+    else:
+        fallback = previous_position.to(device=segment_pos.device, dtype=torch.long)
+    index = torch.arange(steps, device=segment_pos.device).expand(batch, steps)
+    last = torch.where(active_mask, index, torch.full_like(index, -1)).max(dim=1).values
+    picked = segment_pos.gather(1, last.clamp_min(0)[:, None])[:, 0]
+    return torch.where(last >= 0, picked, fallback)
+
+
+class RecurrentBlock(nn.Module):
+    """Linear -> causal depthwise conv -> RG-LRU, gated by GeLU(Linear), then Linear out
+    (griffin/griffin.py:361-529).  The RG-LRU inside honours ``scan_mode`` unchanged."""
+
+    def __init__(self, input_dim: int, rnn_width: int, conv_kernel_size: int = 4, gate_blocks: int = 16,
+                 final_w_init_variance_scale: float = 1.0, scan_mode: ScanMode = "auto"):
+        super().__init__()
+        if conv_kernel_size <= 0:
+            raise ValueError("conv_kernel_size must be positive")
+        self.rnn_width = rnn_width
+        self.conv_kernel_size = conv_kernel_size
+        self.linear_x = nn.Linear(input_dim, rnn_width)
+        self.linear_y = nn.Linear(input_dim, rnn_width)
+        self.temporal_conv = nn.Conv1d(rnn_width, rnn_width, kernel_size=conv_kernel_size, padding=0,
+                                       groups=rnn_width)
+        self.rg_lru = RG_LRU(rnn_width, gate_blocks=gate_blocks, scan_mode=scan_mode)
+        self.linear_out = nn.Linear(rnn_width, input_dim)
+        self.final_w_init_variance_scale = final_w_init_variance_scale
+        self.reset_parameters()
+
+    def reset_parameters(self) -> None:
+        nn.init.normal_(self.linear_x.weight, std=math.sqrt(1.0 / self.linear_x.in_features))
+        nn.init.normal_(self.linear_y.weight, std=math.sqrt(1.0 / self.linear_y.in_features))
+        nn.init.normal_(self.linear_out.weight,
+                        std=math.sqrt(self.final_w_init_variance_scale / self.linear_out.in_features))
+        nn.init.normal_(self.temporal_conv.weight, std=math.sqrt(0.01 / self.conv_kernel_size))
+        for layer in (self.linear_x, self.linear_y, self.linear_out, self.temporal_conv):
+            nn.init.zeros_(layer.bias)
+
+    def _empty_conv_state(self, x: Tensor) -> Tensor:
+        return x.new_zeros(x.size(0), self.conv_kernel_size - 1, self.rnn_width)
+
+    def _dense_conv(self, projected: Tensor, conv_state: Tensor, segment_pos: Tensor):
+        """All-tokens-active path (griffin/griffin.py:476-487): taps are masked per document."""
+        taps = self.temporal_conv.weight[:, 0, :]
+        history = self.conv_kernel_size - 1
+        steps = projected.size(1)
+        padded = torch.cat((conv_state.to(projected), projected), dim=1)
+        out = projected.new_zeros(projected.shape) + self.temporal_conv.bias
+        for lag in range(self.conv_kernel_size):
+            window = padded[:, history - lag: history - lag + steps]
+            same_document = (segment_pos >= lag).to(window.dtype).unsqueeze(-1)
+            out = out + window * same_document * taps[:, history - lag]
+        return out, (padded[:, padded.size(1) - history:] if history else padded[:, :0])
+
+    def _padded_conv(self, projected: Tensor, conv_state: Tensor, segment_pos: Tensor, active_mask: Tensor):
+        """Right-padded batches (griffin/griffin.py:488-510): padding never enters the history."""
+        taps = self.temporal_conv.weight[:, 0, :]
+        history = self.conv_kernel_size - 1
+        window = conv_state.to(projected)
+        rows = []
+        for t in range(projected.size(1)):
+            live = active_mask[:, t, None]
+            fresh = (segment_pos[:, t] == 0)[:, None, None] & live[:, :, None]
+            window = window.masked_fill(fresh, 0.0)
+            now = projected[:, t]
+            value = now * taps[:, -1] + self.temporal_conv.bias
+            if history:
+                value = value + (window * taps[:, :history].T).sum(dim=1)
+            rows.append(value.masked_fill(~live, 0.0))
+            if history:
+                advanced = torch.cat((window[:, 1:], now[:, None]), dim=1)
+                window = torch.where(live[:, :, None], advanced, window)
+        return torch.stack(rows, dim=1), window
+
+    def forward(self, x: Tensor, cache: RecurrentBlockCache | None = None, segment_pos: Tensor | None = None,
+                *, active_mask: Tensor | None = None, return_cache: bool = False):
+        if x.dim() != 3:
+            raise ValueError(f"RecurrentBlock expects [batch, sequence, width], got {tuple(x.shape)}")
+        batch, steps = x.shape[:2]
+        everything_active = active_mask is None
+        if active_mask is None:
+            active_mask = torch.ones(batch, steps, device=x.device, dtype=torch.bool)
+        elif active_mask.shape != (batch, steps):
+            raise ValueError("active_mask must match the input [batch, sequence] dimensions")
+        else:
+            active_mask = active_mask.to(device=x.device, dtype=torch.bool)
+        previous_position = None if cache is None else cache.segment_position
+        segment_pos = _resolve_segment_positions(
+            x, segment_pos, previous_position, None if everything_active else active_mask)
+
+        gate_branch = F.gelu(self.linear_y(x), approximate="tanh")
+        projected = self.linear_x(x)
+        conv_state = self._empty_conv_state(projected) if cache is None else cache.conv_state
+        if conv_state.shape != (batch, self.conv_kernel_size - 1, self.rnn_width):
+            raise ValueError("Recurrent convolution cache has an incompatible shape")
+        if everything_active or bool(active_mask.all()):
+            recurrent_in, new_conv_state = self._dense_conv(projected, conv_state, segment_pos)
+        else:
+            recurrent_in, new_conv_state = self._padded_conv(projected, conv_state, segment_pos, active_mask)
+
+        recurrent_out, new_rnn_state = self.rg_lru(
+            recurrent_in,
+            None if cache is None else cache.rnn_state,
+            reset_mask=segment_pos == 0,
+            active_mask=None if everything_active else active_mask,
+            return_state=True,
+        )
+        output = self.linear_out(recurrent_out * gate_branch)
+        if not everything_active:
+            output = output.masked_fill(~active_mask.unsqueeze(-1), 0.0)
+        if return_cache:
+            return output, RecurrentBlockCache(
+                new_rnn_state, new_conv_state, _last_active_position(segment_pos, active_mask, previous_position))
+        return output

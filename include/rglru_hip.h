@@ -1,0 +1,122 @@
+/*
+ * C ABI of the MI355X (gfx950) RG-LRU library, librglru_hip.so.
+ *
+ * This is the boundary a host binds instead of the reference's Triton operator and the
+ * PyTorch gate chain that feeds it:
+ *
+ *   reference interface replaced                         entry point here
+ *   ---------------------------------------------------  -------------------------------
+ *   griffin/triton_scan.py:207-244  _FusedRGLRUScan.forward   rglru_hip_scan_fwd
+ *   griffin/triton_scan.py:246-271  _FusedRGLRUScan.backward  rglru_hip_scan_bwd
+ *   griffin/griffin.py:237-289      RG_LRU.forward (gates + scan, T > 1)   rglru_hip_prepare + rglru_hip_fwd
+ *   autograd of griffin/griffin.py:237-289                                   rglru_hip_bwd
+ *   griffin/griffin.py:279-284 with T == 1 (decode step, carried state)     rglru_hip_step
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer owned by the caller; tensors are row-major with the
+ *     width axis contiguous; nothing here allocates, frees or synchronises;
+ *   - work is enqueued on `stream` (a hipStream_t passed as void*; NULL = the null stream);
+ *   - every function returns 0 on success or a non-zero code (RGLRU_E_*); the text of the
+ *     last failure on the calling thread is returned by rglru_hip_last_error();
+ *   - the library keeps no per-call state: forward and backward may be issued from different
+ *     host threads (PyTorch runs backward on its autograd thread);
+ *   - `dtype` selects the storage type of x / y / dy / dx and of the gate weights:
+ *     RGLRU_F32 or RGLRU_BF16.  State, biases, Lambda and every parameter gradient are fp32.
+ *   - `flags` is one byte per token, [B, T]: bit 0 = reset (griffin/griffin.py:248-249: a <- 0,
+ *     g <- 1), bit 1 = inactive / padding (griffin/griffin.py:252-255: a <- 1, z <- 0).
+ *     NULL means no reset and all tokens active.
+ */
+#ifndef RGLRU_HIP_H
+#define RGLRU_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RGLRU_ABI_VERSION 1
+
+enum { RGLRU_F32 = 0, RGLRU_BF16 = 1 };
+
+enum {
+  RGLRU_OK = 0,
+  RGLRU_E_ARG = 1,      /* bad shape / null pointer / unsupported dtype */
+  RGLRU_E_UNSUPPORTED = 2, /* shape outside what the kernels cover (e.g. gate block wider than 512) */
+  RGLRU_E_LAUNCH = 3    /* the HIP runtime refused a launch; see rglru_hip_last_error() */
+};
+
+#define RGLRU_FLAG_RESET 1u
+#define RGLRU_FLAG_INACTIVE 2u
+
+/* Time steps per checkpoint: forward stores the fp32 state after every RGLRU_CHUNK tokens and
+ * backward restarts its recomputation from those. */
+#define RGLRU_CHUNK 32
+
+int rglru_hip_abi_version(void);
+const char* rglru_hip_last_error(void);
+
+/* Largest gate-block width (W / nb) the fused kernels accept. */
+int rglru_hip_max_block_width(void);
+
+/* ---- scan-only contract: h_t = a_t * h_{t-1} + z_t, all fp32 ------------------------------
+ * Replaces griffin/triton_scan.py:31-60 and :63-122.  a, z, h, dh, da, dz are [B, T, W];
+ * h0, dh0 are [B, W].  `ws` is scratch of rglru_hip_scan_workspace_bytes(B, T, W) bytes; its
+ * contents on entry do not matter and a forward and a backward call may not share it
+ * concurrently. */
+size_t rglru_hip_scan_workspace_bytes(int64_t B, int64_t T, int64_t W);
+int rglru_hip_scan_fwd(const float* a, const float* z, const float* h0, float* h, void* ws,
+                       int64_t B, int64_t T, int64_t W, void* stream);
+int rglru_hip_scan_bwd(const float* a, const float* h0, const float* h, const float* dh,
+                       float* da, float* dz, float* dh0, void* ws,
+                       int64_t B, int64_t T, int64_t W, void* stream);
+
+/* ---- fused RG-LRU ---------------------------------------------------------------------------
+ * Parameters follow griffin/griffin.py:138-141, 174-176: w_a, w_x are [nb, bw, bw] (out, in) in
+ * `param_dtype`; b_a, b_x are [nb, bw] and lambda is [W], fp32.  rglru_hip_prepare converts them
+ * once into the padded, kernel-friendly image `prep` (rglru_hip_prep_bytes bytes) that fwd, bwd
+ * and step consume; it must be re-run after the parameters change. */
+size_t rglru_hip_prep_bytes(int64_t W, int64_t nb, int dtype);
+int rglru_hip_prepare(const void* w_a, const float* b_a, const void* w_x, const float* b_x,
+                      const float* lambda, float c, int64_t W, int64_t nb, int dtype,
+                      void* prep, void* stream);
+
+/* Workspace shared by one forward call and its backward call.  Forward fills it (chunk
+ * checkpoints of the fp32 state, carry records); backward reads the checkpoints and uses the
+ * rest as scratch.  Contents on entry to forward do not matter. */
+size_t rglru_hip_workspace_bytes(int64_t B, int64_t T, int64_t W, int64_t nb);
+
+/* y[B,T,W] (dtype) and h_last[B,W] (fp32, may be NULL) from x[B,T,W], h0[B,W] (fp32, NULL = 0). */
+int rglru_hip_fwd(const void* x, const void* prep, const float* h0, const uint8_t* flags,
+                  void* y, float* h_last, void* ws,
+                  int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, void* stream);
+
+/* Backward of rglru_hip_fwd.  Recomputes the gates and the decay from x (nothing but the chunk
+ * checkpoints in `ws` is kept from forward).  dy[B,T,W] (dtype); dh_last[B,W] fp32 or NULL.
+ * Outputs: dx[B,T,W] (dtype) receives only the direct path dL/dz * g * i; du_a, du_x [B,T,W]
+ * (dtype) receive the gradients at the two gate pre-activations, from which the caller forms
+ * dW = du^T x, and dx += du W with two library GEMMs; db_a, db_x [nb*bw], dlambda [W] and
+ * dh0 [B,W] (may be NULL) are fp32 and complete. */
+int rglru_hip_bwd(const void* x, const void* prep, const float* lambda, const float* h0,
+                  const uint8_t* flags, const void* dy, const float* dh_last, void* ws,
+                  void* dx, void* du_a, void* du_x, float* db_a, float* db_x, float* dlambda,
+                  float* dh0, int64_t B, int64_t T, int64_t W, int64_t nb, float c, int dtype,
+                  void* stream);
+
+/* One decode step (T == 1): h[B,W] fp32 is updated in place, y[B,W] (dtype) = h as stored. */
+int rglru_hip_step(const void* x, const void* prep, float* h, const uint8_t* flags, void* y,
+                   int64_t B, int64_t W, int64_t nb, int dtype, void* stream);
+
+/* Test hook: number of polls a wave may spend waiting for a neighbouring chunk's carry before it
+ * gives up, records the failure in the workspace and finishes with unspecified results.  The
+ * default is large enough never to trigger in normal operation.  Returns the previous value. */
+int64_t rglru_hip_set_spin_limit(int64_t polls);
+/* Synchronising debug helper: copies the failure word of a workspace to the host (0 = clean). */
+int rglru_hip_workspace_status(const void* ws, int64_t B, int64_t T, int64_t W, int64_t nb,
+                               int scan_only, void* stream, int* status);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RGLRU_HIP_H */

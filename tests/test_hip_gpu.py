@@ -1,0 +1,170 @@
+"""GPU parity tests: the HIP kernels, called through the C ABI, against the CPU oracle."""
+
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import rglru_oracle as orc
+from tests.helpers import PARAMS, hip_run, oracle_run, rel_err
+
+pytestmark = pytest.mark.gpu
+
+FP32_TOL = 1e-5     # norm-wise relative, fp32 storage (h and every gradient)
+BF16_TOL = 2e-2     # bf16 storage, fp32 state, against the fp32 oracle on the rounded inputs
+
+
+def _say(*args):
+    print(*args, flush=True)
+
+
+# ------------------------------------------------------------------ scan-only operator
+@pytest.mark.parametrize("shape", [(2, 37, 65), (1, 7, 257), (3, 300, 130), (2, 1, 64), (1, 1025, 32)])
+def test_scan_op_matches_loop(shape):
+    from griffin_amd import hip_rglru_scan
+
+    B, T, W = shape
+    gen = torch.Generator().manual_seed(0)
+    a = torch.sigmoid(torch.randn(B, T, W, generator=gen) + 2.0)
+    z = torch.randn(B, T, W, generator=gen)
+    h0 = torch.randn(B, W, generator=gen)
+    dh = torch.randn(B, T, W, generator=gen)
+    _say("scan case", shape)
+    want = orc.scan_autograd(a, z, h0, dh)
+    leaves = [t.cuda().requires_grad_(True) for t in (a, z, h0)]
+    h = hip_rglru_scan(*leaves)
+    grads = torch.autograd.grad(h, leaves, dh.cuda())
+    torch.cuda.synchronize()
+    errs = [rel_err(h, want[0])] + [rel_err(g, w) for g, w in zip(grads, want[1:])]
+    _say("  rel errors h, da, dz, dh0:", ["%.2e" % e for e in errs])
+    torch.testing.assert_close(h.cpu(), want[0], atol=2e-5, rtol=2e-5)
+    for g, w in zip(grads, want[1:]):
+        torch.testing.assert_close(g.cpu(), w, atol=3e-5, rtol=3e-5)
+    assert max(errs) < FP32_TOL
+
+
+def test_scan_op_selftest_inputs():
+    from griffin_amd import hip_rglru_scan
+
+    a, z, h0, up = orc.selftest_inputs()
+    want = orc.scan_autograd(a, z, h0, up)
+    leaves = [t.cuda().requires_grad_(True) for t in (a, z, h0)]
+    h = hip_rglru_scan(*leaves)
+    grads = torch.autograd.grad(h, leaves, up.cuda())
+    torch.testing.assert_close(h.cpu(), want[0], atol=2e-5, rtol=2e-5)
+    for g, w in zip(grads, want[1:]):
+        torch.testing.assert_close(g.cpu(), w, atol=3e-5, rtol=3e-5)
+
+
+# ------------------------------------------------------------------ fused operator, fp32
+FP32_CASES = [
+    # B, T, W, nb, masks, h0
+    (2, 29, 32, 4, True, True),      # reference GPU test shape (tests/test_rglru.py:170-204)
+    (2, 5, 6, 6, False, False),      # block width 1
+    (1, 70, 257, 1, True, True),     # prime width: one 257-wide block, partial slab
+    (2, 100, 128, 1, False, True),   # one 128-wide block
+    (2, 130, 640, 2, True, False),   # 320-wide blocks (two LDS slices in fp32)
+    (2, 256, 256, 8, False, False),  # the reference-runnable benchmark configuration
+    (3, 1, 64, 2, True, True),       # single step through the sequence kernels
+]
+
+
+def _masks(B, T, enabled):
+    if not enabled:
+        return None, None
+    reset = torch.zeros(B, T, dtype=torch.bool)
+    reset[:, T // 2] = True
+    reset[0, 0] = True
+    active = torch.ones(B, T, dtype=torch.bool)
+    if T > 4:
+        active[B - 1, T - 4:] = False
+    return reset, active
+
+
+@pytest.mark.parametrize("cfg", FP32_CASES)
+def test_fused_fp32_matches_oracle(cfg):
+    B, T, W, nb, masks, with_h0 = cfg
+    _say("fused fp32 case", cfg)
+    case = orc.make_case(B, T, W, nb, seed=1, h0_std=0.5 if with_h0 else 0.0)
+    case["b_a"] = case["b_a"] + 0.1
+    case["b_x"] = case["b_x"] - 0.2
+    reset, active = _masks(B, T, masks)
+    dh_last = torch.randn(B, W, generator=torch.Generator().manual_seed(5)) if with_h0 else None
+    y, h_last, grads = hip_run(case, torch.float32, reset, active, dh_last)
+    ry, rh, rgrads = oracle_run(case, torch.float32, reset, active, dh_last)
+    # arbitrate against fp64: the fp32 CPU path has summation noise of its own
+    _, _, g64 = oracle_run(case, torch.float64, reset, active, None if dh_last is None else dh_last.double())
+    errs = {"y": rel_err(y, ry), "h_last": rel_err(h_last, rh)}
+    for name in grads:
+        errs[name] = min(rel_err(grads[name], rgrads[name]), rel_err(grads[name], g64[name]))
+    _say("  rel errors:", {k: "%.2e" % v for k, v in errs.items()})
+    for name, err in errs.items():
+        assert err < FP32_TOL, (name, err)
+
+
+# ------------------------------------------------------------------ fused operator, bf16
+BF16_CASES = [
+    (2, 200, 256, 2, True, True),    # 128-wide blocks: register-held weights
+    (2, 96, 128, 2, False, False),   # 64-wide blocks
+    (2, 64, 64, 2, True, False),     # 32-wide blocks
+    (1, 150, 640, 2, True, True),    # 320-wide blocks: streamed weights, two LDS slices
+    (2, 33, 24, 3, True, True),      # unaligned rows (width 24 -> 48-byte rows, 8-wide blocks)
+]
+
+
+@pytest.mark.parametrize("cfg", BF16_CASES)
+def test_fused_bf16_matches_fp32_oracle(cfg):
+    B, T, W, nb, masks, with_h0 = cfg
+    _say("fused bf16 case", cfg)
+    case = orc.make_case(B, T, W, nb, seed=2, h0_std=0.5 if with_h0 else 0.0)
+    reset, active = _masks(B, T, masks)
+    dh_last = torch.randn(B, W, generator=torch.Generator().manual_seed(6)) if with_h0 else None
+    y, h_last, grads = hip_run(case, torch.bfloat16, reset, active, dh_last)
+    ry, rh, rgrads = oracle_run(case, torch.bfloat16, reset, active, dh_last)
+    assert y.dtype == torch.bfloat16 and h_last.dtype == torch.float32
+    errs = {"y": rel_err(y.float(), ry), "h_last": rel_err(h_last, rh)}
+    for name in grads:
+        errs[name] = rel_err(grads[name].float(), rgrads[name])
+    _say("  rel errors:", {k: "%.2e" % v for k, v in errs.items()})
+    for name, err in errs.items():
+        assert err < BF16_TOL, (name, err)
+
+
+# ------------------------------------------------------------------ golden vectors of the reference
+@pytest.mark.parametrize("name", ["rglru_plain_b2_t16_w32", "rglru_masks_b2_t16_w32", "rglru_odd_b3_t37_w65"])
+def test_fused_matches_reference_golden_vectors(golden_dir, name):
+    data = np.load(os.path.join(golden_dir, name + ".npz"))
+    d = {k: torch.from_numpy(data[k]) for k in data.files}
+    case = {k: d[k] for k in PARAMS}
+    case["dy"] = d["dy"]
+    case["h0"] = d.get("h0")
+    y, h_last, grads = hip_run(case, torch.float32, d["reset"], d["active"], d.get("dh"))
+    errs = {"y": rel_err(y, d["y"]), "h_last": rel_err(h_last, d["h_last"])}
+    for key in PARAMS:
+        errs[key] = rel_err(grads[key], d["g_" + key])
+    if "g_h0" in d:
+        errs["h0"] = rel_err(grads["h0"], d["g_h0"])
+    _say(name, {k: "%.2e" % v for k, v in errs.items()})
+    for key, err in errs.items():
+        assert err < FP32_TOL, (key, err)
+
+
+# ------------------------------------------------------------------ decode step
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, FP32_TOL), (torch.bfloat16, BF16_TOL)])
+def test_step_kernel_matches_oracle(dtype, tol):
+    from griffin_amd import PreparedParams, hip_rglru_step
+
+    B, W, nb, steps = 5, 96, 3, 6
+    case = orc.make_case(B, steps, W, nb, seed=3, h0_std=0.5)
+    p = [case[k].to(dtype) for k in PARAMS]
+    prep = PreparedParams(*[t.cuda() for t in p[1:]], 8.0, dtype)
+    state = case["h0"].float().cuda().clone()
+    ys = []
+    for t in range(steps):
+        ys.append(hip_rglru_step(p[0][:, t].cuda().contiguous(), prep, state))
+    torch.cuda.synchronize()
+    ry, rh = orc.rglru_forward(*[t.float() for t in p], h0=case["h0"].float())
+    got = torch.stack(ys, dim=1).float()
+    _say("step", dtype, "y err %.2e state err %.2e" % (rel_err(got, ry), rel_err(state, rh)))
+    assert rel_err(got, ry) < tol and rel_err(state, rh) < tol
