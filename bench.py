@@ -1,0 +1,170 @@
+"""Benchmark of the fused RG-LRU forward + backward on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-graph]
+
+One step = one forward + one backward of the RG-LRU (gates + scan, recomputing backward) over one
+batch of synthetic input, B=8, T=2048, W=1024, 8 gate blocks, bf16 storage with fp32 state: the
+configuration the headline metric is quoted on.  Inputs are resident in HBM before the timed region.
+Prints ONE JSON line.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+# HBM bytes per launch of the backward kernel at the benchmark workload, from rocprofv3 --pmc
+# FETCH_SIZE / WRITE_SIZE runs scaled by a copy kernel of known size (see profiles/).  None until
+# measured.
+MEASURED_TRAFFIC_BYTES = {"bwd_kernel": None, "fwd_kernel": None}
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph replay")
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--seq", type=int, default=2048)
+    ap.add_argument("--width", type=int, default=1024)
+    ap.add_argument("--blocks", type=int, default=8)
+    return ap.parse_args()
+
+
+def cpu_baseline(case, budget_s=20.0):
+    """The oracle (port of the reference's CPU sequential path, fp32) on the host cores: forward +
+    autograd backward on the same workload, bf16-rounded inputs upcast to fp32."""
+    from tests.helpers import oracle_run
+
+    threads = os.cpu_count() or 1
+    torch.set_num_threads(threads)
+    B, T, _ = case["x"].shape
+    t0 = time.perf_counter()
+    oracle_run(case, torch.bfloat16)            # warm-up
+    first = time.perf_counter() - t0
+    times = []
+    while (not times) or (sum(times) + first < budget_s and len(times) < 5):
+        t0 = time.perf_counter()
+        oracle_run(case, torch.bfloat16)
+        times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return {
+        "value": B * T / med, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+        "sample": f"{len(times)} fwd+bwd iterations of the full workload after 1 warm-up, median {med:.3f} s",
+    }
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only; --gpus must be 1", file=sys.stderr)
+        sys.exit(2)
+    from griffin_amd import _lib, hip_rglru
+    from oracle import rglru_oracle as orc
+
+    lib = _lib.load()
+    if not torch.cuda.is_available():
+        raise RuntimeError("bench.py needs a GPU")
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    B, T, W, nb = args.batch, args.seq, args.width, args.blocks
+    case = orc.make_case(B, T, W, nb, seed=0)
+    dt = torch.bfloat16
+    x = case["x"].to(dt).to(dev).requires_grad_(True)
+    params = [case[k].to(dt).to(dev).requires_grad_(True) for k in ("w_a", "b_a", "w_x", "b_x", "lam")]
+    dy = case["dy"].to(dt).to(dev)
+    leaves = [x] + params
+
+    def step():
+        y, _ = hip_rglru(x, *params, 8.0)
+        return torch.autograd.grad(y, leaves, dy)
+
+    for _ in range(max(args.warmup, 3)):
+        step()
+    torch.cuda.synchronize()
+
+    graph = None
+    if not args.no_graph:
+        try:
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                step()
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                captured = step()
+            for _ in range(3):
+                graph.replay()
+            torch.cuda.synchronize()
+        except Exception as error:  # fall back to eager timing, and say so
+            print(f"bench.py: graph capture failed ({error}); timing eager launches", file=sys.stderr)
+            graph = None
+
+    run = graph.replay if graph is not None else step
+    for _ in range(args.warmup):
+        run()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        run()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+
+    # per-kernel durations, HIP events on the launch stream (library measurement hook), eager launches
+    lib.rglru_hip_set_timing(1)
+    fwd_ms, bwd_ms = [], []
+    for _ in range(20):
+        step()
+        fwd_ms.append(lib.rglru_hip_kernel_ms(0))
+        bwd_ms.append(lib.rglru_hip_kernel_ms(1))
+    lib.rglru_hip_set_timing(0)
+    if min(fwd_ms) <= 0 or min(bwd_ms) <= 0:
+        raise RuntimeError(f"kernel timing hook returned no measurement: fwd {fwd_ms[:3]} bwd {bwd_ms[:3]}")
+    fwd_avg = sum(fwd_ms) / len(fwd_ms)
+    bwd_avg = sum(bwd_ms) / len(bwd_ms)
+
+    n = B * T * W
+    elem = 2
+    bytes_fwd, bytes_bwd = 2 * elem * n, 3 * elem * n
+    dominant = "bwd_kernel" if bwd_avg >= fwd_avg else "fwd_kernel"
+    dom_bytes, dom_ms = (bytes_bwd, bwd_avg) if dominant == "bwd_kernel" else (bytes_fwd, fwd_avg)
+    achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
+    out = {
+        "metric": "RG-LRU fwd+bwd tokens/s", "value": B * T / (ms_per_step * 1e-3), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16 storage, f32 state",
+        "data": "synthetic",
+        "config": {"workload": f"RG-LRU fwd+bwd B{B} T{T} W{W} nb{nb} bf16", "batch": B, "seq_len": T,
+                   "width": W, "gate_blocks": nb, "launch": "hip graph replay" if graph is not None else "eager"},
+        "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES[dominant],
+                     "algorithmic_bytes": dom_bytes, "kernel_ms": dom_ms},
+        "kernels": {"fwd_kernel_ms": fwd_avg, "bwd_kernel_ms": bwd_avg,
+                    "fwd_GBps": bytes_fwd / (fwd_avg * 1e-3) / 1e9, "bwd_GBps": bytes_bwd / (bwd_avg * 1e-3) / 1e9,
+                    "fwd_bwd_GBps_whole_step": 5 * elem * n / (ms_per_step * 1e-3) / 1e9,
+                    "fwd_bwd_frac_of_peak_whole_step": 5 * elem * n / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS},
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(case)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -57,6 +57,78 @@ template <> struct Io<float> {
   static RGLRU_DEVICE Frag zero() { Frag f = {0.f, 0.f, 0.f, 0.f}; return f; }
 };
 
+// ------------------------------------------------------------------------------------------
+// Buffer addressing.  Tiles are read and written through raw buffer descriptors whose base is the
+// first row of the tile and whose extent covers only the rows that exist: 32-bit lane offsets, a
+// scalar row offset, and accesses past the extent are dropped by the hardware (loads return 0),
+// which removes every bounds branch from the streaming code.  Only the per-lane offset takes part
+// in the range check, so code that relies on it puts the row term into the lane offset.
+// ------------------------------------------------------------------------------------------
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+constexpr unsigned kOutOfRange = 0x7fffffffu;
+
+RGLRU_DEVICE rsrc_t make_rsrc(const void* base, unsigned bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+
+template <typename IO> struct BufIo;
+template <> struct BufIo<__bf16> {
+  static RGLRU_DEVICE void store(__bf16 v, rsrc_t r, unsigned voff, unsigned soff) {
+    __builtin_amdgcn_raw_buffer_store_b16(__builtin_bit_cast(short, v), r, voff, soff, 0);
+  }
+  static RGLRU_DEVICE float load(rsrc_t r, unsigned voff, unsigned soff) {
+    return (float)__builtin_bit_cast(__bf16, (short)__builtin_amdgcn_raw_buffer_load_b16(r, voff, soff, 0));
+  }
+};
+template <> struct BufIo<float> {
+  static RGLRU_DEVICE void store(float v, rsrc_t r, unsigned voff, unsigned soff) {
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, v), r, voff, soff, 0);
+  }
+  static RGLRU_DEVICE float load(rsrc_t r, unsigned voff, unsigned soff) {
+    return __builtin_bit_cast(float, (int)__builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
+  }
+};
+RGLRU_DEVICE void buf_store_b128(i32x4 v, rsrc_t r, unsigned voff) {
+  __builtin_amdgcn_raw_buffer_store_b128(v, r, voff, 0, 0);
+}
+template <typename Frag> RGLRU_DEVICE Frag buf_load_frag(rsrc_t r, unsigned voff) {
+  return __builtin_bit_cast(Frag, __builtin_amdgcn_raw_buffer_load_b128(r, voff, 0, 0));
+}
+
+// ------------------------------------------------------------------------------------------
+// Per-wave output staging.  After the scan a lane holds consecutive time steps of ONE channel,
+// while memory wants consecutive channels of one time step.  Two-byte stores straight from that
+// layout cost one address per lane and element; instead each wave transposes its ROWS x 32 tile of
+// 16-bit values through a private LDS area (two-byte LDS writes, 16-byte LDS reads) and writes
+// 64-byte row segments with 16-byte stores.  The upper half-wave's rows are skewed by 64 bytes so
+// that the two halves use different banks.
+// ------------------------------------------------------------------------------------------
+template <int ROWS> struct WaveStage {
+  static constexpr int kRowBytes = 64;
+  static constexpr int kBytes = ROWS * kRowBytes + 128;
+  static RGLRU_DEVICE unsigned row_offset(int row) { return (unsigned)row * kRowBytes + (row >= ROWS / 2 ? 64u : 0u); }
+};
+
+RGLRU_DEVICE void wave_lds_fence() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Store a staged ROWS x 32 tile of 16-bit values: `r` covers the tile's rows (row stride
+// row_bytes), col_bytes is the byte offset of the wave's first channel inside a row.
+template <int ROWS>
+RGLRU_DEVICE void stage_flush(const unsigned char* stage, rsrc_t r, unsigned row_bytes, unsigned col_bytes, int lane) {
+#pragma unroll
+  for (int i = 0; i < ROWS / 16; ++i) {
+    const int row = 16 * i + (lane >> 2);
+    const unsigned seg = (unsigned)(lane & 3) * 16u;
+    i32x4 v = *reinterpret_cast<const i32x4*>(stage + WaveStage<ROWS>::row_offset(row) + seg);
+    buf_store_b128(v, r, (unsigned)row * row_bytes + col_bytes + seg);
+  }
+}
+
 // Row m (0..31) of accumulator tile mt holds local time step tile_row(mt, m).  With this map,
 // register v of tile mt in lane half hf is local time hf * 16 * MT + 16 * mt + v: each lane
 // owns 16 * MT consecutive steps, the lower half-wave the first half of the tile.
@@ -73,77 +145,96 @@ RGLRU_DEVICE float xhalf(float v, int hf) {
 
 // ------------------------------------------------------------------------------------------
 // Chunk carry protocol.  A scan over time is cut into chunks that are processed by different
-// waves.  Each (sequence, chunk, 32-channel slab) owns one status word and three fp32 records
-// per channel: the chunk's affine map (A, H) with carry_out = A * carry_in + H, and, once its
-// own carry_in is known, the carry it hands on ("inclusive").  Status: 0 = nothing yet,
-// 1 = (A, H) valid, 2 = inclusive valid.  A wave that needs its carry_in walks towards the
-// start of the chain, composing (A, H) records until it meets an inclusive one or the boundary.
-// Chunks are handed out through a ticket counter in chain order, so every record a wave waits
-// for belongs to a wave that is already running.
+// waves.  Each (sequence, chunk, channel) owns two 64-bit records {fp32 value, 32-bit version}
+// that describe the chunk as an affine map of the carry: carry_out = A * carry_in + H.
+//   version 0            nothing published yet (records start out cleared)
+//   version kVerLocal    (A, H) is the chunk's own map: the reader must go on to the chunk before
+//   version kVerFinal    the chunk knows its carry_in: A = 0 and H = carry_out, the walk ends here
+// Value and version travel in one naturally aligned 8-byte access issued at device scope (sc1), so
+// a reader sees a record entirely or not at all and no fence is needed on either side; a reader
+// that catches the two records of a chunk at different versions simply polls again.  A wave that
+// needs its carry_in loads the records of the kDepth chunks before it in one round trip and
+// composes them in chain order until the accumulated A becomes 0 or the boundary is reached.
+// Chunks are handed out through ticket counters in chain order, so every record a wave waits for
+// belongs to a wave that is already running.
 // ------------------------------------------------------------------------------------------
-RGLRU_DEVICE void st_coherent(float* p, float v) {
-  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-RGLRU_DEVICE float ld_coherent(const float* p) {
-  return __hip_atomic_load(const_cast<float*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
+typedef unsigned long long rec_t;
+constexpr unsigned kVerLocal = 1u, kVerFinal = 2u;
+constexpr int kDepth = 4;
 
-RGLRU_DEVICE void carry_publish(unsigned* status, unsigned value) {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-  if ((threadIdx.x & 63) == 0)
-    __hip_atomic_store(status, value, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+RGLRU_DEVICE void rec_store(rec_t* p, float v, unsigned ver) {
+  __hip_atomic_store(p, ((rec_t)ver << 32) | (rec_t)__float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-
-// Poll one status word until it is non-zero (wave-uniform).  Returns 0 after `limit` polls and
-// records the failure, so that every wave still reaches the end of the kernel.
-RGLRU_DEVICE unsigned carry_wait(unsigned* status, long long limit, unsigned* fail_word) {
-  unsigned v = __hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  v = __builtin_amdgcn_readfirstlane(v);
-  long long polls = 0;
-  while (v == 0) {
-    if (++polls > limit) {
-      if ((threadIdx.x & 63) == 0) atomicOr(fail_word, 1u);
-      return 0;
-    }
-    __builtin_amdgcn_s_sleep(2);
-    v = __hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    v = __builtin_amdgcn_readfirstlane(v);
-  }
-  return v;
+RGLRU_DEVICE rec_t rec_load(const rec_t* p) {
+  return __hip_atomic_load(const_cast<rec_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+RGLRU_DEVICE unsigned rec_ver(rec_t r) { return (unsigned)(r >> 32); }
+RGLRU_DEVICE float rec_val(rec_t r) { return __uint_as_float((unsigned)r); }
 
 struct CarryChain {
-  float* agg_a;       // per-lane pointers, already offset to (sequence, channel); chunk c at + c * stride
-  float* agg_h;
-  float* incl;
-  unsigned* status;   // wave-uniform pointer, chunk c at + c * status_stride
+  rec_t* rec_a;       // per-lane pointers, already offset to (sequence, channel); chunk c at + c * stride
+  rec_t* rec_h;
   long long stride;
-  long long incl_stride;
-  long long status_stride;
 };
 
-// carry_in of chunk c.  `step` is -1 when the chain runs forward in time (the predecessor of c is
+RGLRU_DEVICE void carry_publish(const CarryChain& ch, int c, float a, float h, unsigned ver) {
+  rec_store(ch.rec_a + c * ch.stride, a, ver);
+  rec_store(ch.rec_h + c * ch.stride, h, ver);
+}
+
+// carry_in of chunk c.  `step` is -1 when the chain runs forward in time (the chunk before c is
 // c - 1) and +1 when it runs backward; `end` is the index one past the first chunk of the chain
-// (-1 or the chunk count), where `boundary` is the carry.
+// (-1 or the chunk count), where `boundary` is the carry.  After `limit` fruitless polls the wave
+// records the failure and returns an unspecified value, so every wave still reaches the end of the
+// kernel.
 RGLRU_DEVICE float carry_lookback(const CarryChain& ch, int c, int step, int end, float boundary,
                                   bool lane_ok, long long limit, unsigned* fail_word) {
   float acc_a = 1.f, acc_h = 0.f;
+  bool done = !lane_ok;
   int p = c + step;
+  long long polls = 0;
   for (;;) {
-    if (p == end) return acc_a * boundary + acc_h;
-    unsigned s = carry_wait(ch.status + p * ch.status_stride, limit, fail_word);
-    if (s == 0) return acc_h;
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-    if (s == 2) {
-      float v = lane_ok ? ld_coherent(ch.incl + p * ch.incl_stride) : 0.f;
-      return acc_a * v + acc_h;
+    rec_t ra[kDepth], rh[kDepth];
+#pragma unroll
+    for (int d = 0; d < kDepth; ++d) {
+      const int q = p + d * step;
+      const bool inside = (step < 0) ? (q > end) : (q < end);
+      ra[d] = 0; rh[d] = 0;
+      if (inside && !done) {
+        ra[d] = rec_load(ch.rec_a + q * ch.stride);
+        rh[d] = rec_load(ch.rec_h + q * ch.stride);
+      }
     }
-    float pa = lane_ok ? ld_coherent(ch.agg_a + p * ch.stride) : 1.f;
-    float ph = lane_ok ? ld_coherent(ch.agg_h + p * ch.stride) : 0.f;
-    acc_h = acc_a * ph + acc_h;
-    acc_a *= pa;
-    p += step;
+    bool stalled = false;
+#pragma unroll
+    for (int d = 0; d < kDepth; ++d) {
+      if (stalled) break;
+      const int q = p + d * step;
+      if (q == end) {                                    // wave-uniform
+        if (!done) { acc_h = fmaf(acc_a, boundary, acc_h); acc_a = 0.f; done = true; }
+        break;
+      }
+      const unsigned va = rec_ver(ra[d]), vh = rec_ver(rh[d]);
+      const bool ready = done || (va == vh && va != 0u);
+      if (!__all(ready)) { stalled = true; p = q; break; }
+      if (!done) {
+        acc_h = fmaf(acc_a, rec_val(rh[d]), acc_h);
+        acc_a *= rec_val(ra[d]);
+        if (va == kVerFinal) { acc_a = 0.f; done = true; }
+      }
+    }
+    if (__all(done)) break;
+    if (stalled) {
+      if (++polls > limit) {
+        if ((threadIdx.x & 63) == 0) atomicOr(fail_word, 1u);
+        break;
+      }
+      __builtin_amdgcn_s_sleep(1);
+    } else {
+      p += kDepth * step;
+    }
   }
+  return acc_h;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -161,34 +252,48 @@ RGLRU_DEVICE float sigmoid_fast(float u) {
 }
 
 // 1 - exp(y) for y <= 0 without cancellation: Taylor series near zero, direct form elsewhere.
-RGLRU_DEVICE float one_minus_exp(float y, float a_squared) {
-  float q = 1.0f / 5040.0f;
-  q = fmaf(q, y, 1.0f / 720.0f);
-  q = fmaf(q, y, 1.0f / 120.0f);
-  q = fmaf(q, y, 1.0f / 24.0f);
-  q = fmaf(q, y, 1.0f / 6.0f);
-  q = fmaf(q, y, 0.5f);
-  q = fmaf(q, y, 1.0f);
-  float series = -y * q;
-  float direct = 1.0f - a_squared;
-  return y > -0.25f ? series : direct;
+// PRECISE (fp32 storage): degree-7 series below |y| = 0.25, relative error < 1e-7 everywhere.
+// Otherwise (bf16 storage): two-term series below |y| = 2^-7, relative error < 2e-5.
+template <bool PRECISE>
+RGLRU_DEVICE float one_minus_exp(float y, float a) {
+  const float direct = fmaf(-a, a, 1.0f);
+  if constexpr (PRECISE) {
+    float q = 1.0f / 5040.0f;
+    q = fmaf(q, y, 1.0f / 720.0f);
+    q = fmaf(q, y, 1.0f / 120.0f);
+    q = fmaf(q, y, 1.0f / 24.0f);
+    q = fmaf(q, y, 1.0f / 6.0f);
+    q = fmaf(q, y, 0.5f);
+    q = fmaf(q, y, 1.0f);
+    return y > -0.25f ? -y * q : direct;
+  } else {
+    const float series = -y * fmaf(y, 0.5f, 1.0f);
+    return y > -0.0078125f ? series : direct;
+  }
 }
 
+// MASKED = false: the token is known to be an ordinary one (no reset, active), fl is ignored.
+template <bool PRECISE, bool MASKED>
 RGLRU_DEVICE GateOut gate_forward(float ua, float ux, float x, float sp, unsigned fl) {
   GateOut o;
+#ifdef RGLRU_EXP_NOGATES
+  o.r = ua; o.i = ux; o.a = 0.9f; o.g = 0.4f; o.g2 = 0.16f; o.z = x * ux; return o;
+#endif
   o.r = sigmoid_fast(ua);
   o.i = sigmoid_fast(ux);
   float l2 = o.r * sp;                         // log2(a) <= 0
   float a = __builtin_amdgcn_exp2f(l2);
-  float g2 = one_minus_exp(l2 * (2.0f * kLn2), a * a);
-  g2 = fmaxf(g2, 0.0f);
+  float g2 = fmaxf(one_minus_exp<PRECISE>(l2 * (2.0f * kLn2), a), 0.0f);
   float g = __builtin_amdgcn_sqrtf(g2);
   o.g2 = g2;
-  if (fl & 1u) { a = 0.f; g = 1.f; }
+  if constexpr (MASKED) { if (fl & 1u) { a = 0.f; g = 1.f; } }
   float z = g * o.i * x;
-  if (fl & 2u) { a = 1.f; z = 0.f; }
+  if constexpr (MASKED) { if (fl & 2u) { a = 1.f; z = 0.f; } }
   o.a = a; o.g = g; o.z = z;
   return o;
 }
+
+template <typename IO> struct Precise { static constexpr bool value = true; };
+template <> struct Precise<__bf16> { static constexpr bool value = false; };
 
 }  // namespace rglru

@@ -73,6 +73,15 @@ __global__ void prepare_kernel(PrepArgs p) {
   }
 }
 
+#ifdef RGLRU_TRACE
+// Development aid (not part of the shipped library): per-wave phase timestamps.
+#define RGLRU_STAMP(p, slot) do { if ((p).trace && (threadIdx.x & 63) == 0) { \
+    long long* t_ = (p).trace + ((((long long)blockIdx.x * 4 + (threadIdx.x >> 6)) * 8 + trace_iter) * 12 + (slot)); \
+    if (trace_iter < 8) *t_ = (long long)__builtin_readcyclecounter(); } } while (0)
+#else
+#define RGLRU_STAMP(p, slot) do { } while (0)
+#endif
+
 // ------------------------------------------------------------------------------------------
 // Arguments common to the fused kernels
 // ------------------------------------------------------------------------------------------
@@ -85,109 +94,31 @@ struct FusedArgs {
   void* dx; void* du_a; void* du_x; float* dh0;           // backward out
   float* h_state;                                         // decode step (in place)
   // workspace
-  float* ckpt; float* agg_a; float* agg_h; float* incl; unsigned* status; unsigned* ticket;
+  float* ckpt; rec_t* rec_a; rec_t* rec_h; unsigned* ticket;
   unsigned* fail; float* partial;
   // geometry
   int B, T, W, nb, bw, bwp, S, Wp, groups, units;
-  int nC, nCf, ckpt_nC, slabs, wg_per_unit, aligned;
-  long long tiles_per_unit, limit;
+  int nC, nCf, ckpt_nC, wg_per_unit, aligned, full_slabs, queues;
+  long long limit;
+#ifdef RGLRU_TRACE
+  long long* trace;
+#endif
 };
 
-// ------------------------------------------------------------------------------------------
-// Gate pre-activations of one tile.
-//   rows: `TR` consecutive rows starting at `row0` of a [rows_total, W] matrix (rows beyond
-//   rows_total read as zero); columns: gate block k.  On return ua/ux hold W x + b for the wave's
-//   slab (register v of tile mt <-> local row hf*16*MT + 16*mt + v) and xv the matching x values.
-// Every thread of the workgroup must call this (it contains barriers).
-// ------------------------------------------------------------------------------------------
-template <typename IO, int MT, int NKG>
-RGLRU_DEVICE void gate_tile(const FusedArgs& p, const IO* xmat, long long row0, long long rows_total,
-                            int k, int slab, bool slab_ok, const IO* w_a_row, const IO* w_x_row,
-                            const typename Io<IO>::Frag (&held_a)[NKG > 0 ? NKG : 1],
-                            const typename Io<IO>::Frag (&held_x)[NKG > 0 ? NKG : 1],
-                            float bias_a, float bias_x, IO* lds,
-                            f32x16 (&ua)[MT], f32x16 (&ux)[MT], float (&xv)[16 * MT]) {
-  typedef Io<IO> Tr;
-  typedef typename Tr::Frag Frag;
-  constexpr int TR = 32 * MT;
-  constexpr int KG = Tr::KG, HW = Tr::HW, KCMAX = Tr::KCMAX;
-  constexpr int LDSROW = KCMAX + HW;
-  const int tid = threadIdx.x, lane = tid & 63, r = lane & 31, hf = lane >> 5;
-
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-    for (int v = 0; v < 16; ++v) { ua[mt][v] = bias_a; ux[mt][v] = bias_x; }
-#pragma unroll
-  for (int e = 0; e < 16 * MT; ++e) xv[e] = 0.f;
-
-  for (int kc0 = 0; kc0 < p.bwp; kc0 += KCMAX) {
-    const int kcw = (p.bwp - kc0) < KCMAX ? (p.bwp - kc0) : KCMAX;
-    const int vecs = kcw / HW;
-    for (int idx = tid; idx < TR * vecs; idx += kThreads) {
-      const int row = idx / vecs, cv = idx - row * vecs;
-      const int col = kc0 + cv * HW;                      // column inside the gate block
-      Frag v = Tr::zero();
-      const long long grow = row0 + row;
-      if (grow < rows_total) {
-        const IO* src = xmat + grow * (long long)p.W + (long long)k * p.bw + col;
-        if (p.aligned && col + HW <= p.bw) {
-          v = *reinterpret_cast<const Frag*>(src);
-        } else {
-#pragma unroll
-          for (int e = 0; e < HW; ++e) if (col + e < p.bw) v[e] = src[e];
-        }
-      }
-      *reinterpret_cast<Frag*>(lds + row * LDSROW + cv * HW) = v;
-    }
-    __syncthreads();
-    if (slab_ok) {
-      if constexpr (NKG > 0) {
-#pragma unroll
-        for (int kg = 0; kg < NKG; ++kg) {
-#pragma unroll
-          for (int mt = 0; mt < MT; ++mt) {
-            Frag xa = *reinterpret_cast<const Frag*>(lds + tile_row<MT>(mt, r) * LDSROW + kg * KG + hf * HW);
-            Tr::mma(ua[mt], xa, held_a[kg]);
-            Tr::mma(ux[mt], xa, held_x[kg]);
-          }
-        }
-      } else {
-        for (int kk = 0; kk < kcw; kk += KG) {
-          Frag fa = *reinterpret_cast<const Frag*>(w_a_row + kc0 + kk);
-          Frag fx = *reinterpret_cast<const Frag*>(w_x_row + kc0 + kk);
-#pragma unroll
-          for (int mt = 0; mt < MT; ++mt) {
-            Frag xa = *reinterpret_cast<const Frag*>(lds + tile_row<MT>(mt, r) * LDSROW + kk + hf * HW);
-            Tr::mma(ua[mt], xa, fa);
-            Tr::mma(ux[mt], xa, fx);
-          }
-        }
-      }
-      const int own = slab * 32 - kc0;                    // first column of this wave's slab in the slice
-      if (own >= 0 && own < kcw) {
-#pragma unroll
-        for (int e = 0; e < 16 * MT; ++e) xv[e] = (float)lds[(hf * 16 * MT + e) * LDSROW + own + r];
-      }
-    }
-    __syncthreads();
-  }
-}
-
-template <typename IO, int NKG>
-RGLRU_DEVICE void load_held(const IO* w_a_row, const IO* w_x_row,
-                            typename Io<IO>::Frag (&held_a)[NKG > 0 ? NKG : 1],
-                            typename Io<IO>::Frag (&held_x)[NKG > 0 ? NKG : 1]) {
-  typedef Io<IO> Tr;
-  if constexpr (NKG > 0) {
-#pragma unroll
-    for (int kg = 0; kg < NKG; ++kg) {
-      held_a[kg] = *reinterpret_cast<const typename Tr::Frag*>(w_a_row + kg * Tr::KG);
-      held_x[kg] = *reinterpret_cast<const typename Tr::Frag*>(w_x_row + kg * Tr::KG);
-    }
-  } else {
-    held_a[0] = Tr::zero(); held_x[0] = Tr::zero();
-  }
+// Ticket queues.  A unit's (chunk, sequence) tiles are dealt to `queues` counters: queue j owns the
+// sequences b = j, j + queues, ...; its tickets enumerate them chunk-major, i.e. in chain order.  A
+// workgroup serves queue wg_in_unit % queues.  Spreading the tickets keeps same-address atomics rare.
+struct Queue {
+  unsigned* counter; int first_b, n_b; long long tiles;
+};
+RGLRU_DEVICE Queue make_queue(const FusedArgs& p, int unit, int wg_in_unit, int chunks) {
+  Queue q;
+  const int j = wg_in_unit % p.queues;
+  q.counter = p.ticket + unit * kMaxQueues + j;
+  q.first_b = j;
+  q.n_b = (p.B - j + p.queues - 1) / p.queues;
+  q.tiles = (long long)q.n_b * chunks;
+  return q;
 }
 
 // Identity of the wave inside its unit; shared by the kernels below.
@@ -205,103 +136,344 @@ RGLRU_DEVICE WaveId wave_identity(const FusedArgs& p, int block) {
   w.slab_ok = w.slab < p.S;
   w.o = w.slab * 32 + w.r;
   w.ch_ok = w.slab_ok && w.o < p.bw;
-  w.ch = w.k * p.bw + w.o;
+  w.ch = w.k * p.bw + (w.ch_ok ? w.o : 0);
   w.kp = w.k * p.bwp + (w.slab_ok ? w.o : 0);
   return w;
 }
 
-RGLRU_DEVICE unsigned token_flags(const FusedArgs& p, long long token_row, long long rows_total) {
-  if (token_row >= rows_total) return RGLRU_FLAG_INACTIVE;
+// ------------------------------------------------------------------------------------------
+// x tile staging.  A tile is TR consecutive rows (tokens, or sequences for the decode step) of one
+// gate block, kept in LDS with row stride KS + HW elements.
+// ------------------------------------------------------------------------------------------
+template <typename IO>
+RGLRU_DEVICE typename Io<IO>::Frag load_x_frag(const FusedArgs& p, const IO* xmat, long long grow,
+                                               long long rows_total, int k, int col) {
+  typedef Io<IO> Tr;
+  typename Tr::Frag v = Tr::zero();
+  if (grow < rows_total) {
+    const IO* src = xmat + grow * (long long)p.W + (long long)k * p.bw + col;
+    if (p.aligned && col + Tr::HW <= p.bw) {
+      v = *reinterpret_cast<const typename Tr::Frag*>(src);
+    } else {
+#pragma unroll
+      for (int e = 0; e < Tr::HW; ++e) if (col + e < p.bw) v[e] = src[e];
+    }
+  }
+  return v;
+}
+
+// Gate pre-activations of one tile, generic variant (any block width, weights streamed from
+// memory, K staged through LDS in slices of KCMAX).  On return ua/ux hold W x + b for the wave's
+// slab (register v of tile mt <-> local row hf*16*MT + 16*mt + v) and xv the matching x values.
+// Every thread of the workgroup must call this (it contains barriers).
+template <typename IO, int MT>
+RGLRU_DEVICE void gate_tile_generic(const FusedArgs& p, const IO* xmat, long long row0, long long rows_total,
+                                    int k, int slab, bool slab_ok, const IO* w_a_row, const IO* w_x_row,
+                                    float bias_a, float bias_x, IO* lds,
+                                    f32x16 (&ua)[MT], f32x16 (&ux)[MT], float (&xv)[16 * MT]) {
+  typedef Io<IO> Tr;
+  typedef typename Tr::Frag Frag;
+  constexpr int TR = 32 * MT;
+  constexpr int KG = Tr::KG, HW = Tr::HW, KCMAX = Tr::KCMAX;
+  constexpr int LDSROW = KCMAX + HW;
+  const int tid = threadIdx.x, lane = tid & 63, r = lane & 31, hf = lane >> 5;
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) { ua[mt][v] = bias_a; ux[mt][v] = bias_x; }
+#pragma unroll
+  for (int e = 0; e < 16 * MT; ++e) xv[e] = 0.f;
+
+  for (int kc0 = 0; kc0 < p.bwp; kc0 += KCMAX) {
+    const int kcw = (p.bwp - kc0) < KCMAX ? (p.bwp - kc0) : KCMAX;
+    const int vecs = kcw / HW;
+    for (int idx = tid; idx < TR * vecs; idx += kThreads) {
+      const int row = idx / vecs, cv = idx - row * vecs;
+      Frag v = load_x_frag<IO>(p, xmat, row0 + row, rows_total, k, kc0 + cv * HW);
+      *reinterpret_cast<Frag*>(lds + row * LDSROW + cv * HW) = v;
+    }
+    __syncthreads();
+    if (slab_ok) {
+      for (int kk = 0; kk < kcw; kk += KG) {
+        Frag fa = *reinterpret_cast<const Frag*>(w_a_row + kc0 + kk);
+        Frag fx = *reinterpret_cast<const Frag*>(w_x_row + kc0 + kk);
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          Frag xa = *reinterpret_cast<const Frag*>(lds + tile_row<MT>(mt, r) * LDSROW + kk + hf * HW);
+          Tr::mma(ua[mt], xa, fa);
+          Tr::mma(ux[mt], xa, fx);
+        }
+      }
+      const int own = slab * 32 - kc0;                    // first column of this wave's slab in the slice
+      if (own >= 0 && own < kcw) {
+#pragma unroll
+        for (int e = 0; e < 16 * MT; ++e) xv[e] = (float)lds[(hf * 16 * MT + e) * LDSROW + own + r];
+      }
+    }
+    __syncthreads();
+  }
+}
+
+// Register-resident weights: the wave's 32 rows of both gate matrices, NKG K groups each.
+template <typename IO, int NKG>
+struct HeldWeights {
+  typename Io<IO>::Frag a[NKG > 0 ? NKG : 1], x[NKG > 0 ? NKG : 1];
+  RGLRU_DEVICE void load(const IO* w_a_row, const IO* w_x_row) {
+    if constexpr (NKG > 0) {
+#pragma unroll
+      for (int kg = 0; kg < NKG; ++kg) {
+        a[kg] = *reinterpret_cast<const typename Io<IO>::Frag*>(w_a_row + kg * Io<IO>::KG);
+        x[kg] = *reinterpret_cast<const typename Io<IO>::Frag*>(w_x_row + kg * Io<IO>::KG);
+      }
+    }
+  }
+};
+
+// MFMA phase for register-held weights, one accumulator tile: the whole block width (NKG * KG
+// columns) is in LDS with row stride NKG * KG + HW.  Also returns the 16 x values of the tile in
+// accumulator layout.
+template <typename IO, int MT, int NKG>
+RGLRU_DEVICE void gate_mfma_held(const IO* lds, const HeldWeights<IO, NKG>& hw, int mt, int slab, int r, int hf,
+                                 float bias_a, float bias_x, f32x16& ua, f32x16& ux, float (&xv)[16]) {
+  typedef Io<IO> Tr;
+  typedef typename Tr::Frag Frag;
+  constexpr int KG = Tr::KG, HW = Tr::HW;
+  constexpr int LDSROW = NKG * KG + HW;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) { ua[v] = bias_a; ux[v] = bias_x; }
+  const IO* row = lds + tile_row<MT>(mt, r) * LDSROW + hf * HW;
+#pragma unroll
+  for (int kg = 0; kg < NKG; ++kg) {
+    Frag xa = *reinterpret_cast<const Frag*>(row + kg * KG);
+    Tr::mma(ua, xa, hw.a[kg]);
+    Tr::mma(ux, xa, hw.x[kg]);
+  }
+#pragma unroll
+  for (int e = 0; e < 16; ++e) xv[e] = (float)lds[(hf * 16 * MT + 16 * mt + e) * LDSROW + slab * 32 + r];
+}
+
+RGLRU_DEVICE unsigned token_flag(const FusedArgs& p, long long token_row, bool inside) {
+  if (!inside) return RGLRU_FLAG_INACTIVE;
   return p.flags ? (unsigned)p.flags[token_row] : 0u;
 }
 
 // ------------------------------------------------------------------------------------------
 // Forward
 // ------------------------------------------------------------------------------------------
-template <typename IO, int NKG>
-__global__ __launch_bounds__(kThreads) void fwd_kernel(FusedArgs p) {
-  constexpr int MT = 2, TR = 32 * MT, EL = 16 * MT;
-  typedef Io<IO> Tr;
-  typedef typename Tr::Frag Frag;
-  __shared__ __attribute__((aligned(16))) IO lds[TR * (Tr::KCMAX + Tr::HW)];
-  __shared__ unsigned s_ticket;
+// Gate math of 16 consecutive local steps (first = index of the first one in this lane's run).
+// MASKED = false is the common case: no flags, the tile lies inside the sequence.
+template <typename IO, bool MASKED>
+RGLRU_DEVICE void fwd_gates(const FusedArgs& p, long long trow, int t_first, const f32x16& ua, const f32x16& ux,
+                            const float (&xv)[16], float sp, float* a, float* z) {
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    unsigned fl = 0u;
+    if constexpr (MASKED) fl = token_flag(p, trow + v, t_first + v < p.T);
+    GateOut go = gate_forward<Precise<IO>::value, MASKED>(ua[v], ux[v], xv[v], sp, fl);
+    a[v] = go.a; z[v] = go.z;
+  }
+}
 
-  const WaveId w = wave_identity(p, blockIdx.x);
+// Local scan, carry exchange, final scan and stores of one wave's 64-token tile.
+// Local scan, carry exchange, final scan and stores of one wave's tile of 32 * MT tokens.
+// `prefetch` is called once the tile's own map has been published, i.e. right before the wave
+// starts waiting for its carry.
+template <typename IO, int MT, bool MASKED, bool STAGED, typename Prefetch>
+RGLRU_DEVICE void fwd_scan_store(const FusedArgs& p, const WaveId& w, int b, int c, const float (&a)[16 * MT],
+                                 const float (&z)[16 * MT], unsigned char* stage, Prefetch prefetch,
+                                 int trace_iter = 0) {
+  constexpr int EL = 16 * MT, TR = 32 * MT;
   const int hf = w.hf;
-  const IO* wg = (const IO*)p.wg;
-  const IO* w_a_row = wg + ((long long)(0 * p.nb + w.k) * p.bwp + (w.slab_ok ? w.o : 0)) * p.bwp + hf * Tr::HW;
-  const IO* w_x_row = wg + ((long long)(1 * p.nb + w.k) * p.bwp + (w.slab_ok ? w.o : 0)) * p.bwp + hf * Tr::HW;
-  Frag held_a[NKG > 0 ? NKG : 1], held_x[NKG > 0 ? NKG : 1];
-  load_held<IO, NKG>(w_a_row, w_x_row, held_a, held_x);
-  const float bias_a = p.bias[w.kp], bias_x = p.bias[p.Wp + w.kp];
-  const float sp = w.ch_ok ? p.sp[w.kp] : 0.f;
-  const IO* x = (const IO*)p.x;
-  IO* y = (IO*)p.y;
   const long long W = p.W;
-
-  for (;;) {
-    if (threadIdx.x == 0) s_ticket = atomicAdd(p.ticket + w.unit, 1u);
-    __syncthreads();
-    const long long tk = s_ticket;
-    if (tk >= p.tiles_per_unit) break;
-    const int c = (int)(tk / p.B), b = (int)(tk - (long long)c * p.B);
-    const int t0 = c * TR;
-
-    f32x16 ua[MT], ux[MT];
-    float xv[EL];
-    gate_tile<IO, MT, NKG>(p, x + (long long)b * p.T * W, t0, p.T, w.k, w.slab, w.slab_ok, w_a_row, w_x_row,
-                           held_a, held_x, bias_a, bias_x, lds, ua, ux, xv);
-    if (!w.slab_ok) continue;                             // no barrier is skipped: gate_tile ended on one
-
-    // gate math, in time order for this lane: local step e <-> t0 + hf * EL + e
-    float a[EL], z[EL];
-    const long long trow = (long long)b * p.T + t0 + hf * EL;
+  const int t0 = c * TR;
+  const bool ch_ok = MASKED ? w.ch_ok : true;
+  // affine map of this lane's run, then of the whole tile
+  float A = 1.f, H = 0.f;
 #pragma unroll
-    for (int e = 0; e < EL; ++e) {
-      unsigned fl = (t0 + hf * EL + e < p.T) ? (p.flags ? (unsigned)p.flags[trow + e] : 0u) : RGLRU_FLAG_INACTIVE;
-      GateOut go = gate_forward(ua[e >> 4][e & 15], ux[e >> 4][e & 15], xv[e], sp, fl);
-      a[e] = go.a; z[e] = go.z;
-    }
-    // affine map of this lane's run, then of the whole tile
-    float A = 1.f, H = 0.f;
-#pragma unroll
-    for (int e = 0; e < EL; ++e) { H = fmaf(a[e], H, z[e]); A *= a[e]; }
-    const float A_o = xhalf(A, hf), H_o = xhalf(H, hf);
-    const float A_lo = hf ? A_o : A, H_lo = hf ? H_o : H;
-    const float A_hi = hf ? A : A_o, H_hi = hf ? H : H_o;
-    const float A_t = A_hi * A_lo, H_t = fmaf(A_hi, H_lo, H_hi);
+  for (int e = 0; e < EL; ++e) { H = fmaf(a[e], H, z[e]); A *= a[e]; }
+  const float A_o = xhalf(A, hf), H_o = xhalf(H, hf);
+  const float A_lo = hf ? A_o : A, H_lo = hf ? H_o : H;
+  const float A_hi = hf ? A : A_o, H_hi = hf ? H : H_o;
+  const float A_t = A_hi * A_lo, H_t = fmaf(A_hi, H_lo, H_hi);
 
-    CarryChain chain;
-    const long long seq_f = (long long)b * p.nCf * W + w.ch;
-    chain.agg_a = p.agg_a + seq_f; chain.agg_h = p.agg_h + seq_f; chain.stride = W;
-    chain.incl = p.ckpt + ((long long)b * p.ckpt_nC + 1) * W + w.ch;        // state after tile p is checkpoint 2p+1
-    chain.incl_stride = 2 * W;
-    chain.status = p.status + (long long)b * p.nCf * p.slabs + (w.k * p.S + w.slab);
-    chain.status_stride = p.slabs;
+  CarryChain chain;
+  const long long seq = (long long)b * p.nCf * W + w.ch;
+  chain.rec_a = p.rec_a + seq; chain.rec_h = p.rec_h + seq; chain.stride = W;
 
-    float h_in;
-    if (c == 0) {
-      h_in = (w.ch_ok && p.h0) ? p.h0[(long long)b * W + w.ch] : 0.f;
-    } else {
-      if (w.ch_ok && hf == 0) { st_coherent(chain.agg_a + c * W, A_t); st_coherent(chain.agg_h + c * W, H_t); }
-      carry_publish(chain.status + (long long)c * chain.status_stride, 1u);
-      h_in = carry_lookback(chain, c, -1, -1, 0.f, w.ch_ok, p.limit, p.fail);
+  float h_in;
+  if (c == 0) {
+    h_in = (ch_ok && p.h0) ? p.h0[(long long)b * W + w.ch] : 0.f;
+    prefetch();
+  } else {
+    if (ch_ok && hf == 0) carry_publish(chain, c, A_t, H_t, kVerLocal);
+    prefetch();
+    RGLRU_STAMP(p, 5);
+#ifdef RGLRU_EXP_NOLOOKBACK
+    h_in = 0.f;
+#else
+    h_in = carry_lookback(chain, c, -1, -1, 0.f, ch_ok, p.limit, p.fail);
+#endif
+    RGLRU_STAMP(p, 6);
+  }
+  const float h_end = fmaf(A_t, h_in, H_t);
+  const float h_mid = fmaf(A_lo, h_in, H_lo);
+  if (ch_ok) {
+    if (hf == 0) {
+      carry_publish(chain, c, 0.f, h_end, kVerFinal);
+      p.ckpt[((long long)b * p.ckpt_nC + c * MT + (MT - 1)) * W + w.ch] = h_end;
+      if (c == p.nCf - 1 && p.h_last) p.h_last[(long long)b * W + w.ch] = h_end;
+    } else if (MT == 2) {
+      p.ckpt[((long long)b * p.ckpt_nC + c * MT) * W + w.ch] = h_mid;
     }
-    const float h_end = fmaf(A_t, h_in, H_t);
-    const float h_mid = fmaf(A_lo, h_in, H_lo);
-    if (w.ch_ok) {
-      if (hf == 0) st_coherent(chain.incl + c * chain.incl_stride, h_end);
-      else p.ckpt[((long long)b * p.ckpt_nC + 2 * c) * W + w.ch] = h_mid;
-    }
-    carry_publish(chain.status + (long long)c * chain.status_stride, 2u);
-    if (c == p.nCf - 1 && p.h_last && w.ch_ok && hf == 0) p.h_last[(long long)b * W + w.ch] = h_end;
+  }
 
-    float h = hf ? h_mid : h_in;
-    IO* yrow = y + trow * W + w.ch;
+  float h = hf ? h_mid : h_in;
+  // y tile through a buffer descriptor: rows past the end of the sequence are dropped
+  const int rows = (p.T - t0) < TR ? (p.T - t0) : TR;
+  const unsigned row_bytes = (unsigned)p.W * (unsigned)sizeof(IO);
+  const rsrc_t ry = make_rsrc((const IO*)p.y + ((long long)b * p.T + t0) * W, (unsigned)rows * row_bytes);
+  if constexpr (STAGED) {
+    // 16-bit outputs: transpose through the wave's staging area, then 16-byte stores
+    unsigned char* my = stage + WaveStage<TR>::row_offset(hf * EL) + w.r * 2;
 #pragma unroll
     for (int e = 0; e < EL; ++e) {
       h = fmaf(a[e], h, z[e]);
-      if (w.ch_ok && (t0 + hf * EL + e < p.T)) yrow[e * W] = (IO)h;
+      *reinterpret_cast<IO*>(my + e * WaveStage<TR>::kRowBytes) = (IO)h;
+    }
+    wave_lds_fence();
+#ifndef RGLRU_EXP_NOSTORE
+    stage_flush<TR>(stage, ry, row_bytes, (unsigned)(w.k * p.bw + w.slab * 32) * 2u, w.lane);
+#endif
+    wave_lds_fence();
+  } else {
+    unsigned voff = ch_ok ? (unsigned)(hf * EL) * row_bytes + (unsigned)w.ch * (unsigned)sizeof(IO) : kOutOfRange;
+#pragma unroll
+    for (int e = 0; e < EL; ++e) {
+      h = fmaf(a[e], h, z[e]);
+      BufIo<IO>::store((IO)h, ry, voff + (unsigned)e * row_bytes, 0u);
+    }
+  }
+}
+
+constexpr int kFwdMT = 1;               // forward tile = 32 * kFwdMT tokens
+
+template <typename IO, int NKG, bool MASKED>
+__global__ __launch_bounds__(kThreads, 2) void fwd_kernel(FusedArgs p) {
+  constexpr int MT = kFwdMT, TR = 32 * MT, EL = 16 * MT;
+  typedef Io<IO> Tr;
+  typedef typename Tr::Frag Frag;
+  constexpr int KC = NKG > 0 ? NKG * Tr::KG : Tr::KCMAX;           // LDS tile width in elements
+  constexpr int LDSROW = KC + Tr::HW;
+  __shared__ __attribute__((aligned(16))) IO lds[TR * LDSROW];
+  __shared__ __attribute__((aligned(16))) unsigned char stage_all[kWaves * WaveStage<TR>::kBytes];
+  __shared__ unsigned s_ticket[2];
+
+  const WaveId w = wave_identity(p, blockIdx.x);
+  const int hf = w.hf, tid = threadIdx.x;
+  unsigned char* stage = stage_all + w.wave * WaveStage<TR>::kBytes;
+  const IO* wg = (const IO*)p.wg;
+  const IO* w_a_row = wg + ((long long)(0 * p.nb + w.k) * p.bwp + (w.slab_ok ? w.o : 0)) * p.bwp + hf * Tr::HW;
+  const IO* w_x_row = wg + ((long long)(1 * p.nb + w.k) * p.bwp + (w.slab_ok ? w.o : 0)) * p.bwp + hf * Tr::HW;
+  const float bias_a = p.bias[w.kp], bias_x = p.bias[p.Wp + w.kp];
+  const float sp = w.ch_ok ? p.sp[w.kp] : 0.f;
+  const IO* x = (const IO*)p.x;
+  const long long W = p.W;
+  const Queue q = make_queue(p, w.unit, w.wg_in_unit, p.nCf);
+
+  if constexpr (NKG > 0) {
+    // software-pipelined loop: the next ticket is taken while the current tile's MFMAs run and the
+    // next x tile is requested right before the wave starts waiting for its carry
+    HeldWeights<IO, NKG> hw;
+    hw.load(w_a_row, w_x_row);
+    constexpr int VPR = KC / Tr::HW;                     // 16-byte vectors per tile row
+    constexpr int NV = (TR * VPR + kThreads - 1) / kThreads;
+    Frag pre[NV];
+    const unsigned row_bytes = (unsigned)p.W * (unsigned)sizeof(IO);
+    unsigned pre_off[NV];                                // lane offsets inside a tile (fixed)
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int idx = tid + i * kThreads;
+      const int row = idx / VPR, cv = idx - row * VPR;
+      pre_off[i] = (idx < TR * VPR) ? (unsigned)row * row_bytes + (unsigned)(w.k * p.bw + cv * Tr::HW) * (unsigned)sizeof(IO)
+                                    : kOutOfRange;
+    }
+    auto issue = [&](long long tk) {
+      if (tk >= q.tiles) return;
+      const int c = (int)(tk / q.n_b), b = q.first_b + (int)(tk - (long long)c * q.n_b) * p.queues;
+      const int rows = (p.T - c * TR) < TR ? (p.T - c * TR) : TR;
+      const rsrc_t rx = make_rsrc(x + ((long long)b * p.T + (long long)c * TR) * W, (unsigned)rows * row_bytes);
+#pragma unroll
+      for (int i = 0; i < NV; ++i) pre[i] = buf_load_frag<Frag>(rx, pre_off[i]);
+    };
+    if (tid == 0) s_ticket[0] = atomicAdd(q.counter, 1u);
+    __syncthreads();
+    long long tk = s_ticket[0];
+    int par = 0;
+    issue(tk);
+    int trace_iter = 0; (void)trace_iter;
+    while (tk < q.tiles) {
+      RGLRU_STAMP(p, 0);
+      const int c = (int)(tk / q.n_b), b = q.first_b + (int)(tk - (long long)c * q.n_b) * p.queues;
+      const long long trow = (long long)b * p.T + c * TR + hf * EL;
+      unsigned next_raw = 0;
+      if (tid == 0) next_raw = atomicAdd(q.counter, 1u);
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        const int idx = tid + i * kThreads;
+        const int row = idx / VPR, cv = idx - row * VPR;
+        if (idx < TR * VPR) *reinterpret_cast<Frag*>(lds + row * LDSROW + cv * Tr::HW) = pre[i];
+      }
+      __syncthreads();
+      RGLRU_STAMP(p, 1);
+      float a[EL], z[EL];
+      if (w.slab_ok) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          f32x16 ua, ux;
+          float xv[16];
+          gate_mfma_held<IO, MT, NKG>(lds, hw, mt, w.slab, w.r, hf, bias_a, bias_x, ua, ux, xv);
+          fwd_gates<IO, MASKED>(p, trow + 16 * mt, c * TR + hf * EL + 16 * mt, ua, ux, xv, sp, a + 16 * mt, z + 16 * mt);
+        }
+      }
+      RGLRU_STAMP(p, 2);
+      if (tid == 0) s_ticket[par ^ 1] = next_raw;
+      __syncthreads();
+      RGLRU_STAMP(p, 3);
+      par ^= 1;
+      const long long tk_next = s_ticket[par];
+      if (w.slab_ok) {
+        RGLRU_STAMP(p, 4);
+        fwd_scan_store<IO, MT, MASKED, sizeof(IO) == 2>(p, w, b, c, a, z, stage, [&]() { issue(tk_next); }, trace_iter);
+      } else {
+        issue(tk_next);
+      }
+      RGLRU_STAMP(p, 7);
+      ++trace_iter;
+      tk = tk_next;
+    }
+  } else {
+    for (;;) {
+      if (tid == 0) s_ticket[0] = atomicAdd(q.counter, 1u);
+      __syncthreads();
+      const long long tk = s_ticket[0];
+      if (tk >= q.tiles) break;
+      const int c = (int)(tk / q.n_b), b = q.first_b + (int)(tk - (long long)c * q.n_b) * p.queues;
+      f32x16 ua[MT], ux[MT];
+      float xv[EL];
+      gate_tile_generic<IO, MT>(p, x + (long long)b * p.T * W, (long long)c * TR, p.T, w.k, w.slab, w.slab_ok,
+                                w_a_row, w_x_row, bias_a, bias_x, lds, ua, ux, xv);
+      if (w.slab_ok) {
+        const long long trow = (long long)b * p.T + c * TR + hf * EL;
+        float a[EL], z[EL];
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+          float xpart[16];
+#pragma unroll
+          for (int e = 0; e < 16; ++e) xpart[e] = xv[16 * mt + e];
+          fwd_gates<IO, true>(p, trow + 16 * mt, c * TR + hf * EL + 16 * mt, ua[mt], ux[mt], xpart, sp, a + 16 * mt, z + 16 * mt);
+        }
+        fwd_scan_store<IO, MT, true, false>(p, w, b, c, a, z, stage, []() {});
+      }
     }
   }
 }
@@ -316,16 +488,18 @@ __global__ __launch_bounds__(kThreads) void bwd_kernel(FusedArgs p) {
   constexpr int MT = 1, TR = 32, EL = 16;
   typedef Io<IO> Tr;
   typedef typename Tr::Frag Frag;
-  __shared__ __attribute__((aligned(16))) IO lds[TR * (Tr::KCMAX + Tr::HW)];
+  constexpr int KC = NKG > 0 ? NKG * Tr::KG : Tr::KCMAX;
+  constexpr int LDSROW = KC + Tr::HW;
+  __shared__ __attribute__((aligned(16))) IO lds[TR * LDSROW];
   __shared__ unsigned s_ticket;
 
   const WaveId w = wave_identity(p, blockIdx.x);
-  const int hf = w.hf;
+  const int hf = w.hf, tid = threadIdx.x;
   const IO* wg = (const IO*)p.wg;
   const IO* w_a_row = wg + ((long long)(0 * p.nb + w.k) * p.bwp + (w.slab_ok ? w.o : 0)) * p.bwp + hf * Tr::HW;
   const IO* w_x_row = wg + ((long long)(1 * p.nb + w.k) * p.bwp + (w.slab_ok ? w.o : 0)) * p.bwp + hf * Tr::HW;
-  Frag held_a[NKG > 0 ? NKG : 1], held_x[NKG > 0 ? NKG : 1];
-  load_held<IO, NKG>(w_a_row, w_x_row, held_a, held_x);
+  HeldWeights<IO, NKG> hw;
+  hw.load(w_a_row, w_x_row);
   const float bias_a = p.bias[w.kp], bias_x = p.bias[p.Wp + w.kp];
   const float sp = w.ch_ok ? p.sp[w.kp] : 0.f;
   const float cs = w.ch_ok ? p.cs[w.kp] : 0.f;
@@ -334,20 +508,33 @@ __global__ __launch_bounds__(kThreads) void bwd_kernel(FusedArgs p) {
   IO* dx = (IO*)p.dx; IO* dua = (IO*)p.du_a; IO* dux = (IO*)p.du_x;
   const long long W = p.W;
   float sum_ba = 0.f, sum_bx = 0.f, sum_l = 0.f;
+  const Queue q = make_queue(p, w.unit, w.wg_in_unit, p.nC);
 
   for (;;) {
-    if (threadIdx.x == 0) s_ticket = atomicAdd(p.ticket + w.unit, 1u);
+    if (tid == 0) s_ticket = atomicAdd(q.counter, 1u);
     __syncthreads();
     const long long tk = s_ticket;
-    if (tk >= p.tiles_per_unit) break;
-    const int cr = (int)(tk / p.B), b = (int)(tk - (long long)cr * p.B);
+    if (tk >= q.tiles) break;
+    const int cr = (int)(tk / q.n_b), b = q.first_b + (int)(tk - (long long)cr * q.n_b) * p.queues;
     const int c = p.nC - 1 - cr;
     const int t0 = c * TR;
 
     f32x16 ua[MT], ux[MT];
     float xv[EL];
-    gate_tile<IO, MT, NKG>(p, x + (long long)b * p.T * W, t0, p.T, w.k, w.slab, w.slab_ok, w_a_row, w_x_row,
-                           held_a, held_x, bias_a, bias_x, lds, ua, ux, xv);
+    if constexpr (NKG > 0) {
+      constexpr int VPR = KC / Tr::HW;
+      for (int idx = tid; idx < TR * VPR; idx += kThreads) {
+        const int row = idx / VPR, cv = idx - row * VPR;
+        Frag v = load_x_frag<IO>(p, x + (long long)b * p.T * W, (long long)t0 + row, p.T, w.k, cv * Tr::HW);
+        *reinterpret_cast<Frag*>(lds + row * LDSROW + cv * Tr::HW) = v;
+      }
+      __syncthreads();
+      if (w.slab_ok) gate_mfma_held<IO, MT, NKG>(lds, hw, 0, w.slab, w.r, hf, bias_a, bias_x, ua[0], ux[0], xv);
+      __syncthreads();
+    } else {
+      gate_tile_generic<IO, MT>(p, x + (long long)b * p.T * W, t0, p.T, w.k, w.slab, w.slab_ok, w_a_row, w_x_row,
+                                bias_a, bias_x, lds, ua, ux, xv);
+    }
     if (!w.slab_ok) continue;
 
     const long long trow = (long long)b * p.T + t0 + hf * EL;
@@ -356,9 +543,9 @@ __global__ __launch_bounds__(kThreads) void bwd_kernel(FusedArgs p) {
 #pragma unroll
     for (int e = 0; e < EL; ++e) {
       const bool in = t0 + hf * EL + e < p.T;
-      unsigned fl = in ? (p.flags ? (unsigned)p.flags[trow + e] : 0u) : RGLRU_FLAG_INACTIVE;
+      unsigned fl = token_flag(p, trow + e, in);
       flv[e] = fl;
-      GateOut go = gate_forward(ua[0][e], ux[0][e], xv[e], sp, fl);
+      GateOut go = gate_forward<Precise<IO>::value, true>(ua[0][e], ux[0][e], xv[e], sp, fl);
       r[e] = go.r; gi[e] = go.i; a[e] = go.a; g[e] = go.g; g2[e] = go.g2; z[e] = go.z;
       gy[e] = (in && w.ch_ok) ? (float)dy[(trow + e) * W + w.ch] : 0.f;
     }
@@ -389,22 +576,17 @@ __global__ __launch_bounds__(kThreads) void bwd_kernel(FusedArgs p) {
 
     CarryChain chain;
     const long long seq = (long long)b * p.nC * W + w.ch;
-    chain.agg_a = p.agg_a + seq; chain.agg_h = p.agg_h + seq; chain.incl = p.incl + seq;
-    chain.stride = W; chain.incl_stride = W;
-    chain.status = p.status + (long long)b * p.nC * p.slabs + (w.k * p.S + w.slab);
-    chain.status_stride = p.slabs;
+    chain.rec_a = p.rec_a + seq; chain.rec_h = p.rec_h + seq; chain.stride = W;
 
     float d_in;
     if (c == p.nC - 1) {
       d_in = (w.ch_ok && p.dh_last) ? p.dh_last[(long long)b * W + w.ch] : 0.f;
     } else {
-      if (w.ch_ok && hf == 0) { st_coherent(chain.agg_a + c * W, A_t); st_coherent(chain.agg_h + c * W, D_t); }
-      carry_publish(chain.status + (long long)c * chain.status_stride, 1u);
+      if (w.ch_ok && hf == 0) carry_publish(chain, c, A_t, D_t, kVerLocal);
       d_in = carry_lookback(chain, c, +1, p.nC, 0.f, w.ch_ok, p.limit, p.fail);
     }
     const float d_out = fmaf(A_t, d_in, D_t);
-    if (w.ch_ok && hf == 0) st_coherent(chain.incl + c * W, d_out);
-    carry_publish(chain.status + (long long)c * chain.status_stride, 2u);
+    if (w.ch_ok && hf == 0) carry_publish(chain, c, 0.f, d_out, kVerFinal);
     if (c == 0 && p.dh0 && w.ch_ok && hf == 0) p.dh0[(long long)b * W + w.ch] = d_out;
 
     carry = hf ? d_in : fmaf(A_hi, d_in, D_hi);
@@ -450,20 +632,31 @@ struct ReduceArgs {
   int W, bw, bwp, Wp, wg_per_unit; float c;
 };
 
-__global__ void reduce_kernel(ReduceArgs p) {
-  int ch = blockIdx.x * blockDim.x + threadIdx.x;
-  if (ch >= p.W) return;
-  int k = ch / p.bw, o = ch - k * p.bw;
-  int kp = k * p.bwp + o;
+__global__ __launch_bounds__(256) void reduce_kernel(ReduceArgs p) {
+  // 64 channels per workgroup; four quarter-sums per channel are combined through LDS
+  __shared__ float part_sum[3][4][64];
+  const int lane = threadIdx.x & 63, quarter = threadIdx.x >> 6;
+  const int ch = blockIdx.x * 64 + lane;
   float sa = 0.f, sx = 0.f, sl = 0.f;
-  for (int g = 0; g < p.wg_per_unit; ++g) {
-    const float* part = p.partial + (long long)g * 3 * p.Wp + kp;
-    sa += part[0]; sx += part[p.Wp]; sl += part[2 * p.Wp];
+  if (ch < p.W) {
+    const int k = ch / p.bw, o = ch - k * p.bw;
+    const int kp = k * p.bwp + o;
+    for (int g = quarter; g < p.wg_per_unit; g += 4) {
+      const float* part = p.partial + (long long)g * 3 * p.Wp + kp;
+      sa += part[0]; sx += part[p.Wp]; sl += part[2 * p.Wp];
+    }
   }
-  p.db_a[ch] = sa; p.db_x[ch] = sx;
-  float lam = p.lambda[ch];
-  float sig_neg = 1.0f / (1.0f + expf(lam));           // d/dLambda log sigmoid(Lambda) = sigmoid(-Lambda)
-  p.dlambda[ch] = p.c * sl * sig_neg;
+  part_sum[0][quarter][lane] = sa; part_sum[1][quarter][lane] = sx; part_sum[2][quarter][lane] = sl;
+  __syncthreads();
+  if (quarter == 0 && ch < p.W) {
+    sa = (part_sum[0][0][lane] + part_sum[0][1][lane]) + (part_sum[0][2][lane] + part_sum[0][3][lane]);
+    sx = (part_sum[1][0][lane] + part_sum[1][1][lane]) + (part_sum[1][2][lane] + part_sum[1][3][lane]);
+    sl = (part_sum[2][0][lane] + part_sum[2][1][lane]) + (part_sum[2][2][lane] + part_sum[2][3][lane]);
+    p.db_a[ch] = sa; p.db_x[ch] = sx;
+    const float lam = p.lambda[ch];
+    const float sig_neg = 1.0f / (1.0f + expf(lam));   // d/dLambda log sigmoid(Lambda) = sigmoid(-Lambda)
+    p.dlambda[ch] = p.c * sl * sig_neg;
+  }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -474,15 +667,15 @@ __global__ __launch_bounds__(kThreads) void step_kernel(FusedArgs p) {
   constexpr int MT = 1, TR = 32, EL = 16;
   typedef Io<IO> Tr;
   typedef typename Tr::Frag Frag;
-  __shared__ __attribute__((aligned(16))) IO lds[TR * (Tr::KCMAX + Tr::HW)];
+  constexpr int KC = NKG > 0 ? NKG * Tr::KG : Tr::KCMAX;
+  constexpr int LDSROW = KC + Tr::HW;
+  __shared__ __attribute__((aligned(16))) IO lds[TR * LDSROW];
 
   const WaveId w = wave_identity(p, blockIdx.x);
-  const int hf = w.hf;
+  const int hf = w.hf, tid = threadIdx.x;
   const IO* wg = (const IO*)p.wg;
   const IO* w_a_row = wg + ((long long)(0 * p.nb + w.k) * p.bwp + (w.slab_ok ? w.o : 0)) * p.bwp + hf * Tr::HW;
   const IO* w_x_row = wg + ((long long)(1 * p.nb + w.k) * p.bwp + (w.slab_ok ? w.o : 0)) * p.bwp + hf * Tr::HW;
-  Frag held_a[NKG > 0 ? NKG : 1], held_x[NKG > 0 ? NKG : 1];
-  load_held<IO, NKG>(w_a_row, w_x_row, held_a, held_x);
   const float bias_a = p.bias[w.kp], bias_x = p.bias[p.Wp + w.kp];
   const float sp = w.ch_ok ? p.sp[w.kp] : 0.f;
   const long long W = p.W;
@@ -490,8 +683,21 @@ __global__ __launch_bounds__(kThreads) void step_kernel(FusedArgs p) {
 
   f32x16 ua[MT], ux[MT];
   float xv[EL];
-  gate_tile<IO, MT, NKG>(p, (const IO*)p.x, row0, p.B, w.k, w.slab, w.slab_ok, w_a_row, w_x_row,
-                         held_a, held_x, bias_a, bias_x, lds, ua, ux, xv);
+  if constexpr (NKG > 0) {
+    HeldWeights<IO, NKG> hw;
+    hw.load(w_a_row, w_x_row);
+    constexpr int VPR = KC / Tr::HW;
+    for (int idx = tid; idx < TR * VPR; idx += kThreads) {
+      const int row = idx / VPR, cv = idx - row * VPR;
+      Frag v = load_x_frag<IO>(p, (const IO*)p.x, row0 + row, p.B, w.k, cv * Tr::HW);
+      *reinterpret_cast<Frag*>(lds + row * LDSROW + cv * Tr::HW) = v;
+    }
+    __syncthreads();
+    if (w.slab_ok) gate_mfma_held<IO, MT, NKG>(lds, hw, 0, w.slab, w.r, hf, bias_a, bias_x, ua[0], ux[0], xv);
+  } else {
+    gate_tile_generic<IO, MT>(p, (const IO*)p.x, row0, p.B, w.k, w.slab, w.slab_ok, w_a_row, w_x_row,
+                              bias_a, bias_x, lds, ua, ux, xv);
+  }
   if (!w.ch_ok) return;
   IO* y = (IO*)p.y;
 #pragma unroll
@@ -499,7 +705,7 @@ __global__ __launch_bounds__(kThreads) void step_kernel(FusedArgs p) {
     const long long row = row0 + hf * EL + e;
     if (row >= p.B) break;
     unsigned fl = p.flags ? (unsigned)p.flags[row] : 0u;
-    GateOut go = gate_forward(ua[0][e], ux[0][e], xv[e], sp, fl);
+    GateOut go = gate_forward<Precise<IO>::value, true>(ua[0][e], ux[0][e], xv[e], sp, fl);
     const long long at = row * W + w.ch;
     float h = fmaf(go.a, p.h_state[at], go.z);
     p.h_state[at] = h;
@@ -527,6 +733,7 @@ static void fill_common(FusedArgs& a, const Geometry& g, const void* prep, int d
   a.W = (int)g.W; a.nb = (int)g.nb; a.bw = (int)g.bw; a.bwp = (int)g.bwp; a.S = (int)g.S; a.Wp = (int)g.Wp;
   a.groups = (int)g.groups; a.units = (int)g.units;
   a.limit = spin_limit();
+  a.full_slabs = (g.bw % 32 == 0) ? 1 : 0;
 }
 
 static int is_aligned(const void* ptr, int64_t W, int64_t bw, size_t es) {
@@ -534,14 +741,26 @@ static int is_aligned(const void* ptr, int64_t W, int64_t bw, size_t es) {
 }
 
 // number of register-held K groups for this block width, or 0 for the streaming variant
-static int held_groups(const Geometry& g, int dtype) {
-  if (dtype == RGLRU_BF16) {
+static int held_groups(const Geometry& g, int dtype, int aligned) {
+  if (dtype == RGLRU_BF16 && aligned && g.bw == g.bwp) {
     if (g.bwp == 128) return 8;
     if (g.bwp == 64) return 4;
     if (g.bwp == 32) return 2;
   }
   return 0;
 }
+
+#define RGLRU_DISPATCH_FWD(grid, stream, args, dtype, nkg, masked)                                      \
+  do {                                                                                                 \
+    if ((dtype) == RGLRU_BF16 && (nkg) == 8 && !(masked)) hipLaunchKernelGGL((fwd_kernel<__bf16, 8, false>), grid, dim3(kThreads), 0, stream, args); \
+    else if ((dtype) == RGLRU_BF16 && (nkg) == 8) hipLaunchKernelGGL((fwd_kernel<__bf16, 8, true>), grid, dim3(kThreads), 0, stream, args); \
+    else if ((dtype) == RGLRU_BF16 && (nkg) == 4 && !(masked)) hipLaunchKernelGGL((fwd_kernel<__bf16, 4, false>), grid, dim3(kThreads), 0, stream, args); \
+    else if ((dtype) == RGLRU_BF16 && (nkg) == 4) hipLaunchKernelGGL((fwd_kernel<__bf16, 4, true>), grid, dim3(kThreads), 0, stream, args); \
+    else if ((dtype) == RGLRU_BF16 && (nkg) == 2 && !(masked)) hipLaunchKernelGGL((fwd_kernel<__bf16, 2, false>), grid, dim3(kThreads), 0, stream, args); \
+    else if ((dtype) == RGLRU_BF16 && (nkg) == 2) hipLaunchKernelGGL((fwd_kernel<__bf16, 2, true>), grid, dim3(kThreads), 0, stream, args); \
+    else if ((dtype) == RGLRU_BF16) hipLaunchKernelGGL((fwd_kernel<__bf16, 0, true>), grid, dim3(kThreads), 0, stream, args); \
+    else hipLaunchKernelGGL((fwd_kernel<float, 0, true>), grid, dim3(kThreads), 0, stream, args);      \
+  } while (0)
 
 #define RGLRU_DISPATCH(KERNEL, grid, stream, args, dtype, nkg)                                         \
   do {                                                                                                 \
@@ -557,10 +776,28 @@ static int held_groups(const Geometry& g, int dtype) {
 
 static int launch_clear(char* base, size_t begin, size_t end, hipStream_t s) {
   long long words = (long long)(end - begin) / 4;
-  int cb = (int)((words + 255) / 256); if (cb > 1024) cb = 1024; if (cb < 1) cb = 1;
+  int cb = (int)((words + 1023) / 1024); if (cb > 2048) cb = 2048; if (cb < 1) cb = 1;
   hipLaunchKernelGGL(clear_words_kernel, dim3(cb), dim3(256), 0, s, (unsigned*)(base + begin), words);
   return check_launch("workspace clear");
 }
+
+// Optional event bracket around the main kernel of an entry point (measurement hook).
+static std::atomic<int> g_timing{0};
+struct TimingSlot { hipEvent_t start = nullptr, stop = nullptr; bool armed = false; };
+static TimingSlot& timing_slot(int which) {
+  static TimingSlot slots[3];       // process-wide: backward runs on PyTorch's autograd thread
+  return slots[which];
+}
+struct KernelTimer {
+  TimingSlot* slot = nullptr; hipStream_t stream;
+  KernelTimer(int which, hipStream_t s) : stream(s) {
+    if (!g_timing.load(std::memory_order_relaxed)) return;
+    slot = &timing_slot(which);
+    if (!slot->start && (hipEventCreate(&slot->start) != hipSuccess || hipEventCreate(&slot->stop) != hipSuccess)) { slot = nullptr; return; }
+    hipEventRecord(slot->start, stream);
+  }
+  ~KernelTimer() { if (slot) { hipEventRecord(slot->stop, stream); slot->armed = true; } }
+};
 
 static int pick_wg_per_unit(const Geometry& g, long long tiles_per_unit, int per_cu, long long cap) {
   long long target = (long long)num_compute_units() * per_cu;
@@ -576,6 +813,11 @@ static int pick_wg_per_unit(const Geometry& g, long long tiles_per_unit, int per
 using namespace rglru;
 
 extern "C" {
+
+#ifdef RGLRU_TRACE
+static long long* g_trace = nullptr;
+void rglru_hip_debug_trace(void* buffer) { g_trace = (long long*)buffer; }
+#endif
 
 int rglru_hip_max_block_width(void) { return 512; }
 
@@ -622,20 +864,30 @@ int rglru_hip_fwd(const void* x, const void* prep, const float* h0, const uint8_
   WorkLayout L = make_work_layout(B, T, g);
   hipStream_t s = (hipStream_t)stream;
   char* wb = (char*)ws;
-  rc = launch_clear(wb, L.clear_begin, L.clear_end, s);
+  rc = launch_clear(wb, L.f_begin, L.f_end, s);
+  if (rc) return rc;
+  rc = launch_clear(wb, L.fail, L.fail + 256, s);
   if (rc) return rc;
   FusedArgs a;
   memset(&a, 0, sizeof(a));
   fill_common(a, g, prep, dtype);
   a.x = x; a.h0 = h0; a.flags = flags; a.y = y; a.h_last = h_last;
-  a.ckpt = (float*)(wb + L.ckpt); a.agg_a = (float*)(wb + L.f_agg_a); a.agg_h = (float*)(wb + L.f_agg_h);
-  a.status = (unsigned*)(wb + L.f_status); a.ticket = (unsigned*)(wb + L.f_ticket); a.fail = (unsigned*)(wb + L.fail);
-  a.B = (int)B; a.T = (int)T; a.nC = (int)L.nC; a.ckpt_nC = (int)L.nC; a.nCf = (int)L.nCf; a.slabs = (int)L.slabs;
+  a.ckpt = (float*)(wb + L.ckpt); a.rec_a = (rec_t*)(wb + L.f_rec_a); a.rec_h = (rec_t*)(wb + L.f_rec_h);
+  a.ticket = (unsigned*)(wb + L.f_ticket); a.fail = (unsigned*)(wb + L.fail);
+  a.B = (int)B; a.T = (int)T; a.nC = (int)L.nC; a.ckpt_nC = (int)L.nC;
+  a.nCf = (int)((T + 32 * kFwdMT - 1) / (32 * kFwdMT));
   a.aligned = is_aligned(x, W, g.bw, elem_size(dtype));
-  a.tiles_per_unit = B * L.nCf;
-  a.wg_per_unit = pick_wg_per_unit(g, a.tiles_per_unit, 2, 1 << 20);
+#ifdef RGLRU_TRACE
+  a.trace = g_trace;
+#endif
+  a.wg_per_unit = pick_wg_per_unit(g, B * (long long)a.nCf, 2, 1 << 20);
+  a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
   dim3 grid((unsigned)(a.wg_per_unit * g.units));
-  RGLRU_DISPATCH(fwd_kernel, grid, s, a, dtype, held_groups(g, dtype));
+  {
+    KernelTimer timer(0, s);
+    const int masked = (flags != nullptr) || (T % (32 * kFwdMT) != 0);
+    RGLRU_DISPATCH_FWD(grid, s, a, dtype, held_groups(g, dtype, a.aligned), masked);
+  }
   return check_launch("fwd");
 }
 
@@ -654,29 +906,31 @@ int rglru_hip_bwd(const void* x, const void* prep, const float* lambda, const fl
   WorkLayout L = make_work_layout(B, T, g);
   hipStream_t s = (hipStream_t)stream;
   char* wb = (char*)ws;
-  rc = launch_clear(wb, L.b_status, L.clear_end, s);      // backward status words, tickets, failure word
+  rc = launch_clear(wb, L.b_begin, L.b_end, s);           // backward carry records, tickets, failure word
   if (rc) return rc;
   FusedArgs a;
   memset(&a, 0, sizeof(a));
   fill_common(a, g, prep, dtype);
   a.x = x; a.h0 = h0; a.flags = flags; a.dy = dy; a.dh_last = dh_last;
   a.dx = dx; a.du_a = du_a; a.du_x = du_x; a.dh0 = dh0;
-  a.ckpt = (float*)(wb + L.ckpt); a.agg_a = (float*)(wb + L.b_agg_a); a.agg_h = (float*)(wb + L.b_agg_h);
-  a.incl = (float*)(wb + L.b_incl);
-  a.status = (unsigned*)(wb + L.b_status); a.ticket = (unsigned*)(wb + L.b_ticket); a.fail = (unsigned*)(wb + L.fail);
+  a.ckpt = (float*)(wb + L.ckpt); a.rec_a = (rec_t*)(wb + L.b_rec_a); a.rec_h = (rec_t*)(wb + L.b_rec_h);
+  a.ticket = (unsigned*)(wb + L.b_ticket); a.fail = (unsigned*)(wb + L.fail);
   a.partial = (float*)(wb + L.partial);
-  a.B = (int)B; a.T = (int)T; a.nC = (int)((T + kChunk - 1) / kChunk); a.ckpt_nC = (int)L.nC; a.nCf = (int)L.nCf; a.slabs = (int)L.slabs;
+  a.B = (int)B; a.T = (int)T; a.nC = (int)((T + kChunk - 1) / kChunk); a.ckpt_nC = (int)L.nC; a.nCf = (int)L.nCf;
   a.aligned = is_aligned(x, W, g.bw, elem_size(dtype));
-  a.tiles_per_unit = B * (long long)a.nC;
-  a.wg_per_unit = pick_wg_per_unit(g, a.tiles_per_unit, 2, L.max_wg);
+  a.wg_per_unit = pick_wg_per_unit(g, B * (long long)a.nC, 2, L.max_wg);
+  a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
   dim3 grid((unsigned)(a.wg_per_unit * g.units));
-  RGLRU_DISPATCH(bwd_kernel, grid, s, a, dtype, held_groups(g, dtype));
+  {
+    KernelTimer timer(1, s);
+    RGLRU_DISPATCH(bwd_kernel, grid, s, a, dtype, held_groups(g, dtype, a.aligned));
+  }
   rc = check_launch("bwd");
   if (rc) return rc;
   ReduceArgs r;
   r.partial = a.partial; r.lambda = lambda; r.db_a = db_a; r.db_x = db_x; r.dlambda = dlambda;
   r.W = (int)W; r.bw = (int)g.bw; r.bwp = (int)g.bwp; r.Wp = (int)g.Wp; r.wg_per_unit = a.wg_per_unit; r.c = c;
-  hipLaunchKernelGGL(reduce_kernel, dim3((unsigned)((W + 255) / 256)), dim3(256), 0, s, r);
+  hipLaunchKernelGGL(reduce_kernel, dim3((unsigned)((W + 63) / 64)), dim3(256), 0, s, r);
   return check_launch("bwd reduce");
 }
 
@@ -697,8 +951,22 @@ int rglru_hip_step(const void* x, const void* prep, float* h, const uint8_t* fla
   long long row_tiles = (B + 31) / 32;
   dim3 grid((unsigned)(row_tiles * g.units));
   hipStream_t s = (hipStream_t)stream;
-  RGLRU_DISPATCH(step_kernel, grid, s, a, dtype, held_groups(g, dtype));
+  {
+    KernelTimer timer(2, s);
+    RGLRU_DISPATCH(step_kernel, grid, s, a, dtype, held_groups(g, dtype, a.aligned));
+  }
   return check_launch("step");
+}
+
+int rglru_hip_set_timing(int enable) { return g_timing.exchange(enable ? 1 : 0); }
+
+float rglru_hip_kernel_ms(int which) {
+  if (which < 0 || which > 2) return -1.f;
+  TimingSlot& slot = timing_slot(which);
+  if (!slot.armed) return -1.f;
+  float ms = -1.f;
+  if (hipEventSynchronize(slot.stop) != hipSuccess || hipEventElapsedTime(&ms, slot.start, slot.stop) != hipSuccess) return -1.f;
+  return ms;
 }
 
 int rglru_hip_workspace_status(const void* ws, int64_t B, int64_t T, int64_t W, int64_t nb,

@@ -47,52 +47,54 @@ inline PrepLayout make_prep_layout(const Geometry& g, size_t elem) {
 }
 
 // Workspace of one forward/backward pair.  nC = chunks of 32 tokens (rounded up to even),
-// nCf = forward tiles of 64 tokens, slabs = nb * S status words per (sequence, chunk).
-//   ckpt        [B][nC][W]   fp32 state after each chunk (kept for backward)
-//   f_agg_a/h   [B][nCf][W]  forward carry records
-//   b_agg_a/h, b_incl [B][nC][W]  backward carry records
+// nCf = forward tiles of 64 tokens.
+//   ckpt        [B][nC][W]      fp32 state after each chunk (kept for backward)
 //   partial     [maxWg][3][Wp]  per-workgroup sums for db_a, db_x, dLambda
-//   --- cleared before each pass ---
-//   f_status    [B][nCf][slabs]   b_status [B][nC][slabs]
-//   f_ticket    [units]           b_ticket [units]
-//   fail        [1]
+//   --- cleared before the forward pass ---
+//   f_rec_a/h   [B][<=nC][W]    64-bit carry records of the forward chain
+//   f_ticket    [units][kMaxQueues]
+//   --- cleared before the backward pass ---
+//   b_rec_a/h   [B][nC][W]      64-bit carry records of the backward chain
+//   b_ticket    [units][kMaxQueues]
+//   fail        [1]             (cleared by both)
+constexpr int kMaxQueues = 64;          // ticket queues per unit (sequences are dealt round-robin to them)
+
 struct WorkLayout {
-  int64_t nC, nCf, slabs, max_wg;
-  size_t ckpt, f_agg_a, f_agg_h, b_agg_a, b_agg_h, b_incl, partial;
-  size_t clear_begin, f_status, b_status, f_ticket, b_ticket, fail, clear_end, total;
+  int64_t nC, nCf, max_wg;
+  size_t ckpt, partial;
+  size_t f_begin, f_rec_a, f_rec_h, f_ticket, f_end;
+  size_t b_begin, b_rec_a, b_rec_h, b_ticket, fail, b_end, total;
 };
 
 inline WorkLayout make_work_layout(int64_t B, int64_t T, const Geometry& g) {
   WorkLayout w;
   w.nCf = (T + 63) / 64;
   w.nC = 2 * w.nCf;
-  w.slabs = g.nb * g.S;
   w.max_wg = 256;                      // most workgroups one unit may use in backward
   size_t off = 0;
   auto take = [&](int64_t bytes) { size_t at = off; off += (size_t)round_up(bytes, 256); return at; };
   w.ckpt = take(B * w.nC * g.W * 4);
-  w.f_agg_a = take(B * w.nCf * g.W * 4);
-  w.f_agg_h = take(B * w.nCf * g.W * 4);
-  w.b_agg_a = take(B * w.nC * g.W * 4);
-  w.b_agg_h = take(B * w.nC * g.W * 4);
-  w.b_incl = take(B * w.nC * g.W * 4);
   w.partial = take(w.max_wg * 3 * g.Wp * 4);
-  w.clear_begin = off;
-  w.f_status = take(B * w.nCf * w.slabs * 4);
-  w.b_status = take(B * w.nC * w.slabs * 4);
-  w.f_ticket = take(g.units * 4);
-  w.b_ticket = take(g.units * 4);
+  w.f_begin = off;
+  w.f_rec_a = take(B * w.nC * g.W * 8);
+  w.f_rec_h = take(B * w.nC * g.W * 8);
+  w.f_ticket = take(g.units * kMaxQueues * 4);
+  w.f_end = off;
+  w.b_begin = off;
+  w.b_rec_a = take(B * w.nC * g.W * 8);
+  w.b_rec_h = take(B * w.nC * g.W * 8);
+  w.b_ticket = take(g.units * kMaxQueues * 4);
   w.fail = take(4);
-  w.clear_end = off;
+  w.b_end = off;
   w.total = off;
   return w;
 }
 
-// Scan-only workspace: chunks of 32 tokens, groups of 64 channels.
-//   agg_a, agg_h, incl [B][nC][W]; then (cleared) status [B][nC][groups], ticket, fail.
+// Scan-only workspace: chunks of 32 tokens; everything is cleared before each pass.
+//   rec_a, rec_h [B][nC][W] 64-bit carry records; ticket [B][groups]; fail.
 struct ScanLayout {
   int64_t nC, groups;
-  size_t agg_a, agg_h, incl, clear_begin, status, ticket, fail, clear_end, total;
+  size_t rec_a, rec_h, ticket, fail, total;
 };
 
 inline ScanLayout make_scan_layout(int64_t B, int64_t T, int64_t W) {
@@ -101,14 +103,10 @@ inline ScanLayout make_scan_layout(int64_t B, int64_t T, int64_t W) {
   s.groups = (W + 63) / 64;
   size_t off = 0;
   auto take = [&](int64_t bytes) { size_t at = off; off += (size_t)round_up(bytes, 256); return at; };
-  s.agg_a = take(B * s.nC * W * 4);
-  s.agg_h = take(B * s.nC * W * 4);
-  s.incl = take(B * s.nC * W * 4);
-  s.clear_begin = off;
-  s.status = take(B * s.nC * s.groups * 4);
-  s.ticket = take(4);
+  s.rec_a = take(B * s.nC * W * 8);
+  s.rec_h = take(B * s.nC * W * 8);
+  s.ticket = take(B * s.groups * 4);
   s.fail = take(4);
-  s.clear_end = off;
   s.total = off;
   return s;
 }

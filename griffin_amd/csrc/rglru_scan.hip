@@ -56,21 +56,24 @@ long long exchange_spin_limit(long long v) { return g_spin_limit.exchange(v); }
 struct ScanArgs {
   const float* a; const float* z; const float* h0; float* h;      // forward
   const float* dh; const float* h_saved; float* da; float* dz; float* dh0;   // backward
-  float* agg_a; float* agg_h; float* incl; unsigned* status; unsigned* ticket; unsigned* fail;
+  rec_t* rec_a; rec_t* rec_h; unsigned* ticket; unsigned* fail;
   int B, T, W, nC, groups;
   long long tiles, limit;
 };
 
 __global__ __launch_bounds__(kThreads) void scan_fwd_kernel(ScanArgs p) {
   const int lane = threadIdx.x & 63;
+  // one ticket counter per chain (sequence x channel group): the waves bound to a chain take its
+  // chunks in chain order
+  const long long gw = (long long)blockIdx.x * kWaves + (threadIdx.x >> 6);
+  if (gw >= p.tiles) return;
+  const int chains = p.B * p.groups;
+  const int chain_id = (int)(gw % chains);
   unsigned tk = 0;
-  if (lane == 0) tk = atomicAdd(p.ticket, 1u);
+  if (lane == 0) tk = atomicAdd(p.ticket + chain_id, 1u);
   tk = __builtin_amdgcn_readfirstlane(tk);
-  if ((long long)tk >= p.tiles) return;
-  const int per_chunk = p.B * p.groups;
-  const int c = tk / per_chunk;
-  const int rem = tk - c * per_chunk;
-  const int b = rem / p.groups, grp = rem - b * p.groups;
+  const int c = (int)tk;
+  const int b = chain_id / p.groups, grp = chain_id - b * p.groups;
   const int ch = grp * 64 + lane;
   const bool ok = ch < p.W;
   const int t0 = c * kChunk;
@@ -89,22 +92,17 @@ __global__ __launch_bounds__(kThreads) void scan_fwd_kernel(ScanArgs p) {
   for (int e = 0; e < kChunk; ++e) { H = fmaf(a[e], H, z[e]); A *= a[e]; }
 
   CarryChain chain;
-  const long long seq = (long long)b * p.nC * W + ch;
-  chain.agg_a = p.agg_a + seq; chain.agg_h = p.agg_h + seq; chain.incl = p.incl + seq;
-  chain.stride = W; chain.incl_stride = W;
-  chain.status = p.status + (long long)b * p.nC * p.groups + grp;
-  chain.status_stride = p.groups;
+  const long long seq = (long long)b * p.nC * W + (ok ? ch : 0);
+  chain.rec_a = p.rec_a + seq; chain.rec_h = p.rec_h + seq; chain.stride = W;
 
   float h_in;
   if (c == 0) {
     h_in = ok ? p.h0[(long long)b * W + ch] : 0.f;
   } else {
-    if (ok) { st_coherent(chain.agg_a + c * W, A); st_coherent(chain.agg_h + c * W, H); }
-    carry_publish(chain.status + c * chain.status_stride, 1u);
-    h_in = carry_lookback(chain, c, -1, -1, 0.f /*unused: chunk 0 always publishes inclusive*/, ok, p.limit, p.fail);
+    if (ok) carry_publish(chain, c, A, H, kVerLocal);
+    h_in = carry_lookback(chain, c, -1, -1, 0.f, ok, p.limit, p.fail);
   }
-  if (ok) st_coherent(chain.incl + c * W, fmaf(A, h_in, H));
-  carry_publish(chain.status + c * chain.status_stride, 2u);
+  if (ok) carry_publish(chain, c, 0.f, fmaf(A, h_in, H), kVerFinal);
 
   float h = h_in;
 #pragma unroll
@@ -116,15 +114,15 @@ __global__ __launch_bounds__(kThreads) void scan_fwd_kernel(ScanArgs p) {
 
 __global__ __launch_bounds__(kThreads) void scan_bwd_kernel(ScanArgs p) {
   const int lane = threadIdx.x & 63;
+  const long long gw = (long long)blockIdx.x * kWaves + (threadIdx.x >> 6);
+  if (gw >= p.tiles) return;
+  const int chains = p.B * p.groups;
+  const int chain_id = (int)(gw % chains);
   unsigned tk = 0;
-  if (lane == 0) tk = atomicAdd(p.ticket, 1u);
+  if (lane == 0) tk = atomicAdd(p.ticket + chain_id, 1u);
   tk = __builtin_amdgcn_readfirstlane(tk);
-  if ((long long)tk >= p.tiles) return;
-  const int per_chunk = p.B * p.groups;
-  const int cr = tk / per_chunk;
-  const int c = p.nC - 1 - cr;                       // the chain runs from the last chunk to the first
-  const int rem = tk - cr * per_chunk;
-  const int b = rem / p.groups, grp = rem - b * p.groups;
+  const int c = p.nC - 1 - (int)tk;                  // the chain runs from the last chunk to the first
+  const int b = chain_id / p.groups, grp = chain_id - b * p.groups;
   const int ch = grp * 64 + lane;
   const bool ok = ch < p.W;
   const int t0 = c * kChunk;
@@ -146,23 +144,18 @@ __global__ __launch_bounds__(kThreads) void scan_bwd_kernel(ScanArgs p) {
   const float H = carry;
 
   CarryChain chain;
-  const long long seq = (long long)b * p.nC * W + ch;
-  chain.agg_a = p.agg_a + seq; chain.agg_h = p.agg_h + seq; chain.incl = p.incl + seq;
-  chain.stride = W; chain.incl_stride = W;
-  chain.status = p.status + (long long)b * p.nC * p.groups + grp;
-  chain.status_stride = p.groups;
+  const long long seq = (long long)b * p.nC * W + (ok ? ch : 0);
+  chain.rec_a = p.rec_a + seq; chain.rec_h = p.rec_h + seq; chain.stride = W;
 
   float d_in;
   if (c == p.nC - 1) {
     d_in = 0.f;
   } else {
-    if (ok) { st_coherent(chain.agg_a + c * W, A); st_coherent(chain.agg_h + c * W, H); }
-    carry_publish(chain.status + c * chain.status_stride, 1u);
+    if (ok) carry_publish(chain, c, A, H, kVerLocal);
     d_in = carry_lookback(chain, c, +1, p.nC, 0.f, ok, p.limit, p.fail);
   }
   const float d_out = fmaf(A, d_in, H);
-  if (ok) st_coherent(chain.incl + c * W, d_out);
-  carry_publish(chain.status + c * chain.status_stride, 2u);
+  if (ok) carry_publish(chain, c, 0.f, d_out, kVerFinal);
   if (c == 0 && ok) p.dh0[(long long)b * W + ch] = d_out;
 
   carry = d_in;
@@ -184,14 +177,14 @@ static int scan_common(ScanArgs& p, void* ws, int64_t B, int64_t T, int64_t W, h
   ScanLayout L = make_scan_layout(B, T, W);
   if (B * L.nC * L.groups >= (1ll << 31)) return fail(RGLRU_E_UNSUPPORTED, "scan: too many tiles");
   char* base = (char*)ws;
-  p.agg_a = (float*)(base + L.agg_a); p.agg_h = (float*)(base + L.agg_h); p.incl = (float*)(base + L.incl);
-  p.status = (unsigned*)(base + L.status); p.ticket = (unsigned*)(base + L.ticket); p.fail = (unsigned*)(base + L.fail);
+  p.rec_a = (rec_t*)(base + L.rec_a); p.rec_h = (rec_t*)(base + L.rec_h);
+  p.ticket = (unsigned*)(base + L.ticket); p.fail = (unsigned*)(base + L.fail);
   p.B = (int)B; p.T = (int)T; p.W = (int)W; p.nC = (int)L.nC; p.groups = (int)L.groups;
   p.tiles = B * L.nC * L.groups;
   p.limit = spin_limit();
-  long long words = (long long)(L.clear_end - L.clear_begin) / 4;
-  int cb = (int)((words + 255) / 256); if (cb > 1024) cb = 1024;
-  hipLaunchKernelGGL(clear_words_kernel, dim3(cb), dim3(256), 0, s, (unsigned*)(base + L.clear_begin), words);
+  long long words = (long long)L.total / 4;
+  int cb = (int)((words + 1023) / 1024); if (cb > 2048) cb = 2048;
+  hipLaunchKernelGGL(clear_words_kernel, dim3(cb), dim3(256), 0, s, (unsigned*)base, words);
   return check_launch("scan workspace clear");
 }
 

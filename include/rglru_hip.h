@@ -116,6 +116,15 @@ int64_t rglru_hip_set_spin_limit(int64_t polls);
 int rglru_hip_workspace_status(const void* ws, int64_t B, int64_t T, int64_t W, int64_t nb,
                                int scan_only, void* stream, int* status);
 
+/* Measurement hook.  While enabled, rglru_hip_fwd / rglru_hip_bwd / rglru_hip_step bracket their
+ * main kernel (not the small clear / reduce launches) with HIP events on the call's stream.
+ * rglru_hip_kernel_ms(which) waits for the most recent bracket (process-wide, so enable it from one
+ * thread and keep calls sequential) and returns its
+ * duration in milliseconds (negative when none was recorded): which = 0 forward, 1 backward,
+ * 2 step.  Not for use under stream capture. */
+int rglru_hip_set_timing(int enable);
+float rglru_hip_kernel_ms(int which);
+
 #ifdef __cplusplus
 }
 #endif
