@@ -1,0 +1,74 @@
+"""The C-ABI library: it loads, exports every symbol the header declares, and validates arguments
+on the host before touching a GPU (no kernel is launched here)."""
+
+import ctypes
+import os
+import re
+
+import pytest
+
+from griffin_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "rglru_hip.h")
+
+
+def _declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(rglru_hip_[a-z_]+)\s*\(", text)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not os.path.exists(_lib.LIB_PATH):
+        from griffin_amd import build
+
+        build.build()
+    return _lib.load()
+
+
+def test_header_and_binding_agree():
+    assert _declared_symbols() == sorted(_lib.EXPORTED_SYMBOLS)
+
+
+def test_library_exports_every_declared_symbol(lib):
+    raw = ctypes.CDLL(_lib.LIB_PATH)
+    for name in _declared_symbols():
+        assert hasattr(raw, name), name
+    assert lib.rglru_hip_abi_version() == _lib.ABI_VERSION
+    assert lib.rglru_hip_max_block_width() == 512
+
+
+def test_size_queries(lib):
+    assert lib.rglru_hip_prep_bytes(1024, 8, _lib.RGLRU_BF16) > 2 * 8 * 128 * 128 * 2
+    assert lib.rglru_hip_prep_bytes(1024, 8, _lib.RGLRU_F32) > lib.rglru_hip_prep_bytes(1024, 8, _lib.RGLRU_BF16)
+    assert lib.rglru_hip_prep_bytes(1024, 7, _lib.RGLRU_F32) == 0          # width not divisible
+    assert lib.rglru_hip_prep_bytes(4096, 2, _lib.RGLRU_F32) == 0          # block wider than 512
+    small = lib.rglru_hip_workspace_bytes(2, 64, 256, 8)
+    large = lib.rglru_hip_workspace_bytes(2, 4096, 256, 8)
+    assert 0 < small < large
+    assert lib.rglru_hip_workspace_bytes(0, 64, 256, 8) == 0
+    assert lib.rglru_hip_scan_workspace_bytes(2, 100, 65) > 0
+    assert lib.rglru_hip_scan_workspace_bytes(2, 0, 65) == 0
+
+
+def test_argument_errors_are_reported_without_a_gpu(lib):
+    # null pointers and bad shapes are rejected on the host, with a message
+    assert lib.rglru_hip_scan_fwd(None, None, None, None, None, 1, 1, 1, None) == 1
+    assert b"null" in lib.rglru_hip_last_error()
+    assert lib.rglru_hip_fwd(None, None, None, None, None, None, None, 2, 8, 1024, 7, _lib.RGLRU_BF16, None) == 1
+    assert b"divisible" in lib.rglru_hip_last_error()
+    assert lib.rglru_hip_fwd(None, None, None, None, None, None, None, 2, 8, 4096, 2, _lib.RGLRU_BF16, None) == 2
+    assert b"512" in lib.rglru_hip_last_error()
+    assert lib.rglru_hip_step(None, None, None, None, None, 4, 64, 2, 7, None) == 1
+    assert b"dtype" in lib.rglru_hip_last_error()
+    with pytest.raises(ValueError):
+        _lib.check(1, "probe")
+    with pytest.raises(RuntimeError):
+        _lib.check(3, "probe")
+
+
+def test_spin_limit_hook_round_trips(lib):
+    previous = lib.rglru_hip_set_spin_limit(1234)
+    assert lib.rglru_hip_set_spin_limit(previous) == 1234
