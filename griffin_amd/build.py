@@ -35,7 +35,7 @@ def build(verbose: bool = False) -> str:
     cmd = [
         hipcc_path(), "-O3", "-std=c++17", "-fPIC", "-shared", f"--offload-arch={ARCH}",
         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-        "-Wno-unused-command-line-argument", "-ffp-contract=off",
+        "-Wno-unused-command-line-argument", "-ffp-contract=off", "-fno-strict-aliasing",
         "-I", os.path.join(os.path.dirname(HERE), "include"),
     ]
     cmd += [os.path.join(CSRC, s) for s in SOURCES]

@@ -91,6 +91,9 @@ template <> struct BufIo<float> {
 };
 RGLRU_DEVICE void buf_store_b128(i32x4 v, rsrc_t r, unsigned voff) {
   __builtin_amdgcn_raw_buffer_store_b128(v, r, voff, 0, 0);
+#ifdef RGLRU_EXP_STOREWAIT
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#endif
 }
 template <typename Frag> RGLRU_DEVICE Frag buf_load_frag(rsrc_t r, unsigned voff) {
   return __builtin_bit_cast(Frag, __builtin_amdgcn_raw_buffer_load_b128(r, voff, 0, 0));
@@ -110,8 +113,12 @@ template <int ROWS> struct WaveStage {
   static RGLRU_DEVICE unsigned row_offset(int row) { return (unsigned)row * kRowBytes + (row >= ROWS / 2 ? 64u : 0u); }
 };
 
+// LDS operations of one wave execute in program order, so lanes of the same wave may exchange data
+// through LDS as long as the COMPILER keeps the order: the asm statement is a full compiler barrier
+// for memory accesses (a fence alone does not order plain accesses of different types).
 RGLRU_DEVICE void wave_lds_fence() {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }

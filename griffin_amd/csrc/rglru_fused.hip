@@ -28,7 +28,7 @@ namespace rglru {
 // ------------------------------------------------------------------------------------------
 struct PrepArgs {
   const void* w_a; const void* w_x; const float* b_a; const float* b_x; const float* lambda;
-  void* wg; float* bias; float* sp; float* cs;
+  void* wg; float* bias; float* sp; float* cs; void* w2t;
   int W, nb, bw, bwp, Wp;
   float c;
 };
@@ -41,7 +41,7 @@ template <typename IO>
 __global__ void prepare_kernel(PrepArgs p) {
   const long long per_gate = (long long)p.nb * p.bwp * p.bwp;
   const long long n_w = 2 * per_gate;
-  const long long total = n_w + p.Wp;
+  const long long total = 2 * n_w + p.Wp;
   long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x;
   const long long stride = (long long)gridDim.x * blockDim.x;
   for (; i < total; i += stride) {
@@ -57,6 +57,20 @@ __global__ void prepare_kernel(PrepArgs p) {
         v = (float)src[((long long)k * p.bw + o) * p.bw + j];
       }
       ((IO*)p.wg)[i] = (IO)v;
+    } else if (i >= n_w + p.Wp) {
+      // w2t[k][j][2 * o + gate]
+      long long e = i - n_w - p.Wp;
+      const long long per_block = 2ll * p.bwp * p.bwp;
+      int k = (int)(e / per_block);
+      int rem = (int)(e - (long long)k * per_block);
+      int j = rem / (2 * p.bwp), kap = rem - j * 2 * p.bwp;
+      int o = kap >> 1, gate = kap & 1;
+      float v = 0.f;
+      if (o < p.bw && j < p.bw) {
+        const IO* src = (const IO*)(gate ? p.w_x : p.w_a);
+        v = (float)src[((long long)k * p.bw + o) * p.bw + j];
+      }
+      ((IO*)p.w2t)[e] = (IO)v;
     } else {
       int kp = (int)(i - n_w);
       int k = kp / p.bwp, o = kp - k * p.bwp;
@@ -87,7 +101,7 @@ __global__ void prepare_kernel(PrepArgs p) {
 // ------------------------------------------------------------------------------------------
 struct FusedArgs {
   // tensors
-  const void* x; const void* wg; const float* bias; const float* sp; const float* cs;
+  const void* x; const void* wg; const float* bias; const float* sp; const float* cs; const void* w2t;
   const float* h0; const uint8_t* flags;
   void* y; float* h_last;                                 // forward
   const void* dy; const float* dh_last;                   // backward in
@@ -95,7 +109,7 @@ struct FusedArgs {
   float* h_state;                                         // decode step (in place)
   // workspace
   float* ckpt; rec_t* rec_a; rec_t* rec_h; unsigned* ticket;
-  unsigned* fail; float* partial;
+  unsigned* fail; float* partial; float* dw_partial;
   // geometry
   int B, T, W, nb, bw, bwp, S, Wp, groups, units;
   int nC, nCf, ckpt_nC, wg_per_unit, aligned, full_slabs, queues;
@@ -300,21 +314,14 @@ RGLRU_DEVICE void fwd_scan_store(const FusedArgs& p, const WaveId& w, int b, int
   const long long seq = (long long)b * p.nCf * W + w.ch;
   chain.rec_a = p.rec_a + seq; chain.rec_h = p.rec_h + seq; chain.stride = W;
 
-  float h_in;
-  if (c == 0) {
-    h_in = (ch_ok && p.h0) ? p.h0[(long long)b * W + w.ch] : 0.f;
-    prefetch();
-  } else {
-    if (ch_ok && hf == 0) carry_publish(chain, c, A_t, H_t, kVerLocal);
-    prefetch();
-    RGLRU_STAMP(p, 5);
-#ifdef RGLRU_EXP_NOLOOKBACK
-    h_in = 0.f;
-#else
-    h_in = carry_lookback(chain, c, -1, -1, 0.f, ch_ok, p.limit, p.fail);
+  if (c != 0 && ch_ok && hf == 0) carry_publish(chain, c, A_t, H_t, kVerLocal);
+  prefetch();
+  float h_in = (c == 0 && ch_ok && p.h0) ? p.h0[(long long)b * W + w.ch] : 0.f;
+  RGLRU_STAMP(p, 5);
+#ifndef RGLRU_EXP_NOLOOKBACK
+  if (c != 0) h_in = carry_lookback(chain, c, -1, -1, 0.f, ch_ok, p.limit, p.fail);
 #endif
-    RGLRU_STAMP(p, 6);
-  }
+  RGLRU_STAMP(p, 6);
   const float h_end = fmaf(A_t, h_in, H_t);
   const float h_mid = fmaf(A_lo, h_in, H_lo);
   if (ch_ok) {
@@ -397,10 +404,12 @@ __global__ __launch_bounds__(kThreads, 2) void fwd_kernel(FusedArgs p) {
       pre_off[i] = (idx < TR * VPR) ? (unsigned)row * row_bytes + (unsigned)(w.k * p.bw + cv * Tr::HW) * (unsigned)sizeof(IO)
                                     : kOutOfRange;
     }
-    auto issue = [&](long long tk) {
-      if (tk >= q.tiles) return;
-      const int c = (int)(tk / q.n_b), b = q.first_b + (int)(tk - (long long)c * q.n_b) * p.queues;
-      const int rows = (p.T - c * TR) < TR ? (p.T - c * TR) : TR;
+    auto issue = [&](long long tk_in) {
+      // a ticket past the end keeps valid addresses (tile 0) but an empty extent: nothing is fetched
+      const bool live = tk_in < q.tiles;
+      const unsigned tk = live ? (unsigned)tk_in : 0u;
+      const int c = (int)(tk / (unsigned)q.n_b), b = q.first_b + (int)(tk - (unsigned)c * (unsigned)q.n_b) * p.queues;
+      const int rows = !live ? 0 : ((p.T - c * TR) < TR ? (p.T - c * TR) : TR);
       const rsrc_t rx = make_rsrc(x + ((long long)b * p.T + (long long)c * TR) * W, (unsigned)rows * row_bytes);
 #pragma unroll
       for (int i = 0; i < NV; ++i) pre[i] = buf_load_frag<Frag>(rx, pre_off[i]);
@@ -627,6 +636,418 @@ __global__ __launch_bounds__(kThreads) void bwd_kernel(FusedArgs p) {
   }
 }
 
+// ------------------------------------------------------------------------------------------
+// Fast backward, part 1 (16-bit storage, register-held weights): gate recomputation + both scans.
+// Same mathematics as bwd_kernel, but every global access is a 16-byte vector: x and dy tiles are
+// staged through LDS (prefetched one tile ahead), and the three outputs -- the direct input
+// gradient and the interleaved pair (du_a, du_x) per channel -- are transposed through per-wave LDS
+// areas.  `du2` is [B, T, nb, 2 * bw] with element 2 * o + gate, the layout the second part wants.
+// ------------------------------------------------------------------------------------------
+template <int ROWS> struct PairStage {                  // ROWS x 32 channels x 2 values of 16 bits
+  static constexpr int kRowBytes = 128;
+  static constexpr int kBytes = ROWS * kRowBytes + 256;
+  static RGLRU_DEVICE unsigned row_offset(int row) { return (unsigned)row * kRowBytes + (row >= ROWS / 2 ? 128u : 0u); }
+};
+
+template <typename IO, int NKG, bool MASKED>
+__global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
+  constexpr int MT = 1, TR = 32, EL = 16;
+  typedef Io<IO> Tr;
+  typedef typename Tr::Frag Frag;
+  constexpr int KC = NKG * Tr::KG;
+  constexpr int LDSROW = KC + Tr::HW;
+  static_assert(sizeof(IO) == 2 && NKG > 0, "fast backward is for 16-bit storage with held weights");
+  __shared__ __attribute__((aligned(16))) IO lds_x[TR * LDSROW];
+  __shared__ __attribute__((aligned(16))) IO lds_dy[TR * LDSROW];
+  __shared__ __attribute__((aligned(16))) unsigned char stage_dx_all[kWaves * WaveStage<TR>::kBytes];
+  __shared__ __attribute__((aligned(16))) unsigned char stage_du_all[kWaves * PairStage<TR>::kBytes];
+  __shared__ unsigned s_ticket[2];
+
+  const WaveId w = wave_identity(p, blockIdx.x);
+  const int hf = w.hf, tid = threadIdx.x;
+  unsigned char* stage_dx = stage_dx_all + w.wave * WaveStage<TR>::kBytes;
+  unsigned char* stage_du = stage_du_all + w.wave * PairStage<TR>::kBytes;
+  const IO* wg = (const IO*)p.wg;
+  const int o_safe = w.slab_ok ? w.o : 0;
+  const IO* w_a_row = wg + ((long long)(0 * p.nb + w.k) * p.bwp + o_safe) * p.bwp + hf * Tr::HW;
+  const IO* w_x_row = wg + ((long long)(1 * p.nb + w.k) * p.bwp + o_safe) * p.bwp + hf * Tr::HW;
+  HeldWeights<IO, NKG> hw;
+  hw.load(w_a_row, w_x_row);
+  const float bias_a = p.bias[w.kp], bias_x = p.bias[p.Wp + w.kp];
+  const float sp = p.sp[w.kp], cs = p.cs[w.kp];
+  const IO* x = (const IO*)p.x;
+  const IO* dy = (const IO*)p.dy;
+  const long long W = p.W;
+  const unsigned row_bytes = (unsigned)p.W * 2u;
+  float sum_ba = 0.f, sum_bx = 0.f, sum_l = 0.f;
+  const Queue q = make_queue(p, w.unit, w.wg_in_unit, p.nC);
+
+  constexpr int VPR = KC / Tr::HW;
+  constexpr int NV = (TR * VPR + kThreads - 1) / kThreads;
+  Frag pre_x[NV], pre_dy[NV];
+  unsigned pre_off[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int idx = tid + i * kThreads;
+    const int row = idx / VPR, cv = idx - row * VPR;
+    pre_off[i] = (idx < TR * VPR) ? (unsigned)row * row_bytes + (unsigned)(w.k * p.bw + cv * Tr::HW) * 2u : kOutOfRange;
+  }
+  auto decode = [&](unsigned tk, int& c, int& b) {
+    const unsigned cr = tk / (unsigned)q.n_b;
+    c = p.nC - 1 - (int)cr;
+    b = q.first_b + (int)(tk - cr * (unsigned)q.n_b) * p.queues;
+  };
+  auto issue = [&](unsigned tk) {
+    // a ticket past the end keeps valid addresses (tile 0) but an empty extent: nothing is fetched
+    const bool live = (long long)tk < q.tiles;
+    int c, b;
+    decode(live ? tk : 0u, c, b);
+    const int rows = !live ? 0 : ((p.T - c * TR) < TR ? (p.T - c * TR) : TR);
+    const long long first = ((long long)b * p.T + (long long)c * TR) * W;
+    const rsrc_t rx = make_rsrc(x + first, (unsigned)rows * row_bytes);
+    const rsrc_t rdy = make_rsrc(dy + first, (unsigned)rows * row_bytes);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) { pre_x[i] = buf_load_frag<Frag>(rx, pre_off[i]); pre_dy[i] = buf_load_frag<Frag>(rdy, pre_off[i]); }
+  };
+
+  if (tid == 0) s_ticket[0] = atomicAdd(q.counter, 1u);
+  __syncthreads();
+  unsigned tk = s_ticket[0];
+  int par = 0;
+  issue(tk);
+  while ((long long)tk < q.tiles) {
+    int c, b;
+    decode(tk, c, b);
+    const int t0 = c * TR;
+    const long long trow = (long long)b * p.T + t0 + hf * EL;
+    unsigned next_raw = 0;
+    if (tid == 0) next_raw = atomicAdd(q.counter, 1u);
+    // state at the start of the chunk (forward checkpoint), requested early
+    float h_start = 0.f;
+    if (c == 0) { if (p.h0) h_start = p.h0[(long long)b * W + w.ch]; }
+    else h_start = p.ckpt[((long long)b * p.ckpt_nC + (c - 1)) * W + w.ch];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int idx = tid + i * kThreads;
+      const int row = idx / VPR, cv = idx - row * VPR;
+      if (idx < TR * VPR) {
+        *reinterpret_cast<Frag*>(lds_x + row * LDSROW + cv * Tr::HW) = pre_x[i];
+        *reinterpret_cast<Frag*>(lds_dy + row * LDSROW + cv * Tr::HW) = pre_dy[i];
+      }
+    }
+    __syncthreads();
+    f32x16 ua, ux;
+    float xv[EL], gy[EL];
+    if (w.slab_ok) {
+      gate_mfma_held<IO, MT, NKG>(lds_x, hw, 0, w.slab, w.r, hf, bias_a, bias_x, ua, ux, xv);
+#pragma unroll
+      for (int e = 0; e < EL; ++e) gy[e] = (float)lds_dy[(hf * EL + e) * LDSROW + w.slab * 32 + w.r];
+    }
+    if (tid == 0) s_ticket[par ^ 1] = next_raw;
+    __syncthreads();
+    par ^= 1;
+    const unsigned tk_next = s_ticket[par];
+    if (!w.slab_ok) {                                    // a wave without a slab only helps with the loads
+      issue(tk_next);
+      tk = tk_next;
+      continue;
+    }
+
+    // gate recomputation; z is not kept (g * i * x is recomputed where needed)
+    float r[EL], gi[EL], a[EL], g[EL];
+    unsigned flbits = 0u;                                // two flag bits per local step
+    float A = 1.f, H = 0.f;
+#pragma unroll
+    for (int e = 0; e < EL; ++e) {
+      unsigned fl = 0u;
+      if constexpr (MASKED) { fl = token_flag(p, trow + e, t0 + hf * EL + e < p.T); flbits |= fl << (2 * e); }
+      GateOut go = gate_forward<false, MASKED>(ua[e], ux[e], xv[e], sp, fl);
+      r[e] = go.r; gi[e] = go.i; a[e] = go.a; g[e] = go.g;
+      H = fmaf(go.a, H, go.z); A *= go.a;
+    }
+    const float A_o = xhalf(A, hf), H_o = xhalf(H, hf);
+    const float A_lo = hf ? A_o : A, H_lo = hf ? H_o : H;
+    const float A_hi = hf ? A : A_o;
+    // reverse affine map of this lane's run and of the chunk
+    float carry = 0.f;
+#pragma unroll
+    for (int e = EL - 1; e >= 0; --e) { float d = gy[e] + carry; carry = a[e] * d; }
+    const float D = carry, D_o = xhalf(D, hf);
+    const float D_lo = hf ? D_o : D, D_hi = hf ? D : D_o;
+    const float A_t = A_lo * A_hi, D_t = fmaf(A_lo, D_hi, D_lo);
+
+    CarryChain chain;
+    const long long seq = (long long)b * p.nC * W + w.ch;
+    chain.rec_a = p.rec_a + seq; chain.rec_h = p.rec_h + seq; chain.stride = W;
+    const bool last_chunk = c == p.nC - 1;
+    if (!last_chunk && hf == 0) carry_publish(chain, c, A_t, D_t, kVerLocal);
+    issue(tk_next);
+    float d_in = (last_chunk && p.dh_last) ? p.dh_last[(long long)b * W + w.ch] : 0.f;
+    if (!last_chunk) d_in = carry_lookback(chain, c, +1, p.nC, 0.f, true, p.limit, p.fail);
+    const float d_out = fmaf(A_t, d_in, D_t);
+    if (hf == 0) carry_publish(chain, c, 0.f, d_out, kVerFinal);
+    if (hf == 0 && c == 0 && p.dh0) p.dh0[(long long)b * W + w.ch] = d_out;
+
+    // delta_t in place of dy_t (reverse), then one forward pass that carries h_{t-1} along
+    carry = hf ? d_in : fmaf(A_hi, d_in, D_hi);
+#pragma unroll
+    for (int e = EL - 1; e >= 0; --e) { const float d = gy[e] + carry; gy[e] = d; carry = a[e] * d; }
+    float h = hf ? fmaf(A_lo, h_start, H_lo) : h_start;
+    unsigned char* my_dx = stage_dx + WaveStage<TR>::row_offset(hf * EL) + w.r * 2;
+    unsigned char* my_du = stage_du + PairStage<TR>::row_offset(hf * EL) + w.r * 4;
+#pragma unroll
+    for (int e = 0; e < EL; ++e) {
+      const float d = gy[e];
+      const float xe = xv[e];
+      const float gx = g[e] * xe;                        // dz/di
+      float dg = d * gi[e] * xe;
+      float di = d * gx;
+      float dxd = d * g[e] * gi[e];
+      // g = sqrt(g2) with the bounded derivative; a = exp(l), g2 = 1 - a^2 (= g * g off reset)
+      const float a2 = a[e] * a[e];
+      float dg2 = dg * __builtin_amdgcn_rsqf(fmaxf(4.0f * (g[e] * g[e]), 1e-6f));
+      float dl = fmaf(d * h, a[e], -2.0f * a2 * dg2);
+      float ze = gx * gi[e];
+      if constexpr (MASKED) { if ((flbits >> (2 * e)) & 1u) dl = 0.f; }
+      float va = dl * cs * r[e] * (1.0f - r[e]);
+      float vx = di * gi[e] * (1.0f - gi[e]);
+      if constexpr (MASKED) { if ((flbits >> (2 * e)) & 2u) { dl = 0.f; va = 0.f; vx = 0.f; dxd = 0.f; ze = 0.f; } }
+      h = fmaf(a[e], h, ze);
+      sum_l = fmaf(dl, r[e], sum_l);
+      sum_ba += va; sum_bx += vx;
+      *reinterpret_cast<IO*>(my_dx + e * WaveStage<TR>::kRowBytes) = (IO)dxd;
+      typedef IO io2 __attribute__((ext_vector_type(2)));
+      io2 pair; pair[0] = (IO)va; pair[1] = (IO)vx;
+      *reinterpret_cast<io2*>(my_du + e * PairStage<TR>::kRowBytes) = pair;
+    }
+    wave_lds_fence();
+    {
+      const int rows = (p.T - t0) < TR ? (p.T - t0) : TR;
+      const rsrc_t rdx = make_rsrc((const IO*)p.dx + ((long long)b * p.T + t0) * W, (unsigned)rows * row_bytes);
+      stage_flush<TR>(stage_dx, rdx, row_bytes, (unsigned)(w.k * p.bw + w.slab * 32) * 2u, w.lane);
+      const unsigned du_row_bytes = 2u * row_bytes;
+      const rsrc_t rdu = make_rsrc((const IO*)p.du_a + ((long long)b * p.T + t0) * 2 * W, (unsigned)rows * du_row_bytes);
+      const unsigned du_col = (unsigned)(w.k * 2 * p.bw + w.slab * 64) * 2u;
+#pragma unroll
+      for (int i = 0; i < TR / 8; ++i) {
+        const int row = 8 * i + (w.lane >> 3);
+        const unsigned seg = (unsigned)(w.lane & 7) * 16u;
+        i32x4 v = *reinterpret_cast<const i32x4*>(stage_du + PairStage<TR>::row_offset(row) + seg);
+        buf_store_b128(v, rdu, (unsigned)row * du_row_bytes + du_col + seg);
+      }
+    }
+    wave_lds_fence();
+    tk = tk_next;
+  }
+  // per-workgroup partial sums (every slot is written, so the buffer needs no clearing)
+  sum_ba += xhalf(sum_ba, hf); sum_bx += xhalf(sum_bx, hf); sum_l += xhalf(sum_l, hf);
+  if (hf == 0 && w.slab_ok) {
+    float* part = p.partial + (long long)w.wg_in_unit * 3 * p.Wp + w.k * p.bwp + w.o;
+    part[0] = sum_ba; part[p.Wp] = sum_bx; part[2 * p.Wp] = sum_l;
+  }
+}
+
+// ------------------------------------------------------------------------------------------
+// Fast backward, part 2: the two block-diagonal GEMMs of the gate gradients,
+//     dx[n, j]   += sum_kappa du2[n, kappa] * w2t[j, kappa]          (kappa = 2 * o + gate)
+//     dW2T[j, kappa] = sum_n x[n, j] * du2[n, kappa]
+// over the flattened token axis n = b * T + t, one gate block per workgroup, 32 tokens per tile.
+// Each wave owns a 32-column slab j of the block: it keeps its w2t rows (the B operand of the first
+// GEMM) and its 32 x 2*bw slice of dW2T (the accumulator of the second) in registers for the whole
+// launch.  The second GEMM contracts over tokens, so both operands are needed with tokens running
+// along a lane's vector; tiles arrive token-major, and the transposition is done by the matrix
+// unit itself: multiplying a tile by the identity returns it in accumulator layout, where a lane
+// holds 16 consecutive tokens of one column.
+// ------------------------------------------------------------------------------------------
+template <typename IO, int NKG>
+__global__ __launch_bounds__(kThreads, 1) void gate_grad_kernel(FusedArgs p) {
+  typedef Io<IO> Tr;
+  typedef typename Tr::Frag Frag;
+  static_assert(sizeof(IO) == 2 && NKG > 0, "16-bit storage only");
+  constexpr int TR = 32;
+  constexpr int KC = NKG * Tr::KG;                       // block width
+  constexpr int S = KC / 32;                             // slabs in the block
+  constexpr int K2 = 2 * KC, NKG2 = 2 * NKG;             // contraction length of the first GEMM
+  constexpr int ROW_X = KC + Tr::HW, ROW_DU = K2 + Tr::HW, ROW_T = TR + Tr::HW;
+  __shared__ __attribute__((aligned(16))) IO lds_du[TR * ROW_DU];
+  __shared__ __attribute__((aligned(16))) IO lds_x[TR * ROW_X];
+  __shared__ __attribute__((aligned(16))) IO lds_dx[TR * ROW_X];
+  __shared__ __attribute__((aligned(16))) IO lds_dut[K2 * ROW_T];          // du2 transposed: [kappa][token]
+  __shared__ __attribute__((aligned(16))) unsigned char stage_all[kWaves * WaveStage<TR>::kBytes];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, hf = lane >> 5;
+  const int k = blockIdx.x % p.nb, wg_in_unit = blockIdx.x / p.nb, n_wg = gridDim.x / p.nb;
+  const bool slab_ok = wave < S;
+  unsigned char* stage = stage_all + wave * WaveStage<TR>::kBytes;
+  const long long rows_total = (long long)p.B * p.T;
+  const long long n_tiles = (rows_total + TR - 1) / TR;
+  const unsigned row_bytes = (unsigned)p.W * 2u;
+
+  // this wave's rows of w2t: B operand of the first GEMM, lane (n = j, hf) holds kappa = 16 kg + 8 hf + i
+  Frag w2[NKG2];
+  {
+    const IO* row = (const IO*)p.w2t + ((long long)k * p.bwp + (slab_ok ? wave * 32 + r : 0)) * (2 * p.bwp) + hf * Tr::HW;
+#pragma unroll
+    for (int kg = 0; kg < NKG2; ++kg) w2[kg] = *reinterpret_cast<const Frag*>(row + kg * Tr::KG);
+  }
+  // identity fragments: element i of ident[q] is 1 where 16 q + 8 hf + i == r
+  Frag ident[2];
+#pragma unroll
+  for (int qd = 0; qd < 2; ++qd)
+#pragma unroll
+    for (int i = 0; i < Tr::HW; ++i) ident[qd][i] = (IO)((16 * qd + 8 * hf + i == r) ? 1.0f : 0.0f);
+
+  f32x16 dw[2 * S];
+#pragma unroll
+  for (int kt = 0; kt < 2 * S; ++kt)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) dw[kt][v] = 0.f;
+
+  // cooperative tile loads: du2 (TR x K2), x and dx (TR x KC)
+  constexpr int VPR_DU = K2 / Tr::HW, VPR_X = KC / Tr::HW;
+  constexpr int NV_DU = (TR * VPR_DU + kThreads - 1) / kThreads, NV_X = (TR * VPR_X + kThreads - 1) / kThreads;
+  Frag pre_du[NV_DU], pre_x[NV_X], pre_dx[NV_X];
+  auto issue = [&](long long tile) {
+    if (tile >= n_tiles) return;
+    const long long row0 = tile * TR;
+    const int rows = (int)((rows_total - row0) < TR ? (rows_total - row0) : TR);
+    const rsrc_t rdu = make_rsrc((const IO*)p.du_a + row0 * 2 * p.W, (unsigned)rows * 2u * row_bytes);
+    const rsrc_t rx = make_rsrc((const IO*)p.x + row0 * p.W, (unsigned)rows * row_bytes);
+    const rsrc_t rdx = make_rsrc((const IO*)p.dx + row0 * p.W, (unsigned)rows * row_bytes);
+#pragma unroll
+    for (int i = 0; i < NV_DU; ++i) {
+      const int idx = tid + i * kThreads;
+      const int row = idx / VPR_DU, cv = idx - row * VPR_DU;
+      pre_du[i] = buf_load_frag<Frag>(rdu, idx < TR * VPR_DU ? (unsigned)row * 2u * row_bytes + (unsigned)(k * 2 * p.bw + cv * Tr::HW) * 2u : kOutOfRange);
+    }
+#pragma unroll
+    for (int i = 0; i < NV_X; ++i) {
+      const int idx = tid + i * kThreads;
+      const int row = idx / VPR_X, cv = idx - row * VPR_X;
+      const unsigned off = idx < TR * VPR_X ? (unsigned)row * row_bytes + (unsigned)(k * p.bw + cv * Tr::HW) * 2u : kOutOfRange;
+      pre_x[i] = buf_load_frag<Frag>(rx, off);
+      pre_dx[i] = buf_load_frag<Frag>(rdx, off);
+    }
+  };
+
+  long long tile = wg_in_unit;
+  issue(tile);
+  for (; tile < n_tiles; tile += n_wg) {
+#pragma unroll
+    for (int i = 0; i < NV_DU; ++i) {
+      const int idx = tid + i * kThreads;
+      const int row = idx / VPR_DU, cv = idx - row * VPR_DU;
+      if (idx < TR * VPR_DU) *reinterpret_cast<Frag*>(lds_du + row * ROW_DU + cv * Tr::HW) = pre_du[i];
+    }
+#pragma unroll
+    for (int i = 0; i < NV_X; ++i) {
+      const int idx = tid + i * kThreads;
+      const int row = idx / VPR_X, cv = idx - row * VPR_X;
+      if (idx < TR * VPR_X) {
+        *reinterpret_cast<Frag*>(lds_x + row * ROW_X + cv * Tr::HW) = pre_x[i];
+        *reinterpret_cast<Frag*>(lds_dx + row * ROW_X + cv * Tr::HW) = pre_dx[i];
+      }
+    }
+    __syncthreads();
+    issue(tile + n_wg);
+
+    const long long row0 = tile * TR;
+    const IO* a_row_du = lds_du + tile_row<1>(0, r) * ROW_DU + hf * Tr::HW;
+    const IO* a_row_x = lds_x + tile_row<1>(0, r) * ROW_X + hf * Tr::HW;
+    // transposes: kappa tiles 2 * wave and 2 * wave + 1 of du2 go to lds_dut
+#pragma unroll
+    for (int h2 = 0; h2 < 2; ++h2) {
+      const int kt = 2 * wave + h2;
+      if (kt < 2 * S) {
+        f32x16 dc;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) dc[v] = 0.f;
+        Tr::mma(dc, *reinterpret_cast<const Frag*>(a_row_du + (2 * kt) * Tr::KG), ident[0]);
+        Tr::mma(dc, *reinterpret_cast<const Frag*>(a_row_du + (2 * kt + 1) * Tr::KG), ident[1]);
+        Frag lo, hi;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { lo[i] = (IO)dc[i]; hi[i] = (IO)dc[8 + i]; }
+        IO* dst = lds_dut + (kt * 32 + r) * ROW_T + hf * 16;
+        *reinterpret_cast<Frag*>(dst) = lo;
+        *reinterpret_cast<Frag*>(dst + 8) = hi;
+      }
+    }
+    Frag xt_lo = Tr::zero(), xt_hi = Tr::zero();
+    if (slab_ok) {
+      // x of this wave's slab with tokens along the lane vector (A operand of the second GEMM)
+      f32x16 xc;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) xc[v] = 0.f;
+      Tr::mma(xc, *reinterpret_cast<const Frag*>(a_row_x + (2 * wave) * Tr::KG), ident[0]);
+      Tr::mma(xc, *reinterpret_cast<const Frag*>(a_row_x + (2 * wave + 1) * Tr::KG), ident[1]);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) { xt_lo[i] = (IO)xc[i]; xt_hi[i] = (IO)xc[8 + i]; }
+      // first GEMM: dx tile = direct part + du2 . w2t^T
+      f32x16 acc;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[v] = (float)lds_dx[(hf * 16 + v) * ROW_X + wave * 32 + r];
+#pragma unroll
+      for (int kg = 0; kg < NKG2; ++kg)
+        Tr::mma(acc, *reinterpret_cast<const Frag*>(a_row_du + kg * Tr::KG), w2[kg]);
+      unsigned char* my = stage + WaveStage<TR>::row_offset(hf * 16) + r * 2;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) *reinterpret_cast<IO*>(my + v * WaveStage<TR>::kRowBytes) = (IO)acc[v];
+      wave_lds_fence();
+      const int rows = (int)((rows_total - row0) < TR ? (rows_total - row0) : TR);
+      const rsrc_t rdx = make_rsrc((const IO*)p.dx + row0 * p.W, (unsigned)rows * row_bytes);
+      stage_flush<TR>(stage, rdx, row_bytes, (unsigned)(k * p.bw + wave * 32) * 2u, lane);
+      wave_lds_fence();
+    }
+    __syncthreads();
+    if (slab_ok) {
+      // second GEMM: dW2T[j, kappa] += sum over the tile's tokens
+#pragma unroll
+      for (int kt = 0; kt < 2 * S; ++kt) {
+        const IO* b_row = lds_dut + (kt * 32 + r) * ROW_T + hf * 16;
+        Tr::mma(dw[kt], xt_lo, *reinterpret_cast<const Frag*>(b_row));
+        Tr::mma(dw[kt], xt_hi, *reinterpret_cast<const Frag*>(b_row + 8));
+      }
+    }
+  }
+  // per-workgroup partial of dW2T: [wg][k][j][kappa]
+  if (slab_ok) {
+    float* part = p.dw_partial + (((long long)wg_in_unit * p.nb + k) * p.bwp) * (2 * p.bwp);
+#pragma unroll
+    for (int kt = 0; kt < 2 * S; ++kt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int j = wave * 32 + 8 * (v >> 2) + 4 * hf + (v & 3);
+        part[(long long)j * (2 * p.bwp) + kt * 32 + r] = dw[kt][v];
+      }
+  }
+}
+
+struct DwReduceArgs {
+  const float* dw_partial; float* dw_a; float* dw_x; int nb, bw, bwp, n_wg;
+};
+
+// dW_gate[k][o][j] = sum over workgroups of dW2T[wg][k][j][2 o + gate]
+__global__ void dw_reduce_kernel(DwReduceArgs p) {
+  const long long total = (long long)p.nb * p.bw * 2 * p.bw;
+  long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const int kap = (int)(i % (2 * p.bw));
+  const int j = (int)((i / (2 * p.bw)) % p.bw);
+  const int k = (int)(i / ((long long)2 * p.bw * p.bw));
+  const long long stride = (long long)p.nb * p.bwp * 2 * p.bwp;
+  const float* src = p.dw_partial + ((long long)k * p.bwp + j) * (2 * p.bwp) + kap;
+  float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+  int g = 0;
+  for (; g + 3 < p.n_wg; g += 4) {
+    s0 += src[(long long)g * stride]; s1 += src[(long long)(g + 1) * stride];
+    s2 += src[(long long)(g + 2) * stride]; s3 += src[(long long)(g + 3) * stride];
+  }
+  for (; g < p.n_wg; ++g) s0 += src[(long long)g * stride];
+  const float sum = (s0 + s1) + (s2 + s3);
+  float* dst = (kap & 1) ? p.dw_x : p.dw_a;
+  dst[((long long)k * p.bw + (kap >> 1)) * p.bw + j] = sum;
+}
+
 struct ReduceArgs {
   const float* partial; const float* lambda; float* db_a; float* db_x; float* dlambda;
   int W, bw, bwp, Wp, wg_per_unit; float c;
@@ -730,6 +1151,7 @@ static void fill_common(FusedArgs& a, const Geometry& g, const void* prep, int d
   PrepLayout pl = make_prep_layout(g, elem_size(dtype));
   const char* pb = (const char*)prep;
   a.wg = pb + pl.wg; a.bias = (const float*)(pb + pl.bias); a.sp = (const float*)(pb + pl.sp); a.cs = (const float*)(pb + pl.cs);
+  a.w2t = pb + pl.w2t;
   a.W = (int)g.W; a.nb = (int)g.nb; a.bw = (int)g.bw; a.bwp = (int)g.bwp; a.S = (int)g.S; a.Wp = (int)g.Wp;
   a.groups = (int)g.groups; a.units = (int)g.units;
   a.limit = spin_limit();
@@ -785,7 +1207,7 @@ static int launch_clear(char* base, size_t begin, size_t end, hipStream_t s) {
 static std::atomic<int> g_timing{0};
 struct TimingSlot { hipEvent_t start = nullptr, stop = nullptr; bool armed = false; };
 static TimingSlot& timing_slot(int which) {
-  static TimingSlot slots[3];       // process-wide: backward runs on PyTorch's autograd thread
+  static TimingSlot slots[4];       // process-wide: backward runs on PyTorch's autograd thread
   return slots[which];
 }
 struct KernelTimer {
@@ -838,8 +1260,9 @@ int rglru_hip_prepare(const void* w_a, const float* b_a, const void* w_x, const 
   PrepArgs a;
   a.w_a = w_a; a.w_x = w_x; a.b_a = b_a; a.b_x = b_x; a.lambda = lambda;
   a.wg = pb + pl.wg; a.bias = (float*)(pb + pl.bias); a.sp = (float*)(pb + pl.sp); a.cs = (float*)(pb + pl.cs);
+  a.w2t = pb + pl.w2t;
   a.W = (int)W; a.nb = (int)nb; a.bw = (int)g.bw; a.bwp = (int)g.bwp; a.Wp = (int)g.Wp; a.c = c;
-  long long total = 2 * g.nb * g.bwp * g.bwp + g.Wp;
+  long long total = 4 * g.nb * g.bwp * g.bwp + g.Wp;
   int blocks = (int)((total + 255) / 256); if (blocks > 2048) blocks = 2048;
   hipStream_t s = (hipStream_t)stream;
   if (dtype == RGLRU_BF16) hipLaunchKernelGGL(prepare_kernel<__bf16>, dim3(blocks), dim3(256), 0, s, a);
@@ -934,6 +1357,83 @@ int rglru_hip_bwd(const void* x, const void* prep, const float* lambda, const fl
   return check_launch("bwd reduce");
 }
 
+int rglru_hip_fast_path(int64_t W, int64_t nb, int dtype) {
+  if (dtype != RGLRU_BF16 || W <= 0 || nb <= 0 || W % nb) return 0;
+  const int64_t bw = W / nb;
+  return (bw == 32 || bw == 64 || bw == 128) ? 1 : 0;
+}
+
+int rglru_hip_bwd_full(const void* x, const void* prep, const float* lambda, const float* h0,
+                       const uint8_t* flags, const void* dy, const float* dh_last, void* ws,
+                       void* dx, float* dw_a, float* dw_x, float* db_a, float* db_x, float* dlambda,
+                       float* dh0, int64_t B, int64_t T, int64_t W, int64_t nb, float c, int dtype,
+                       void* stream) {
+  int rc = check_geometry("bwd_full", W, nb, dtype);
+  if (rc) return rc;
+  if (!rglru_hip_fast_path(W, nb, dtype))
+    return fail(RGLRU_E_UNSUPPORTED, "bwd_full: needs 16-bit storage and gate blocks of 32, 64 or 128 channels");
+  if (B <= 0 || T <= 0) return fail(RGLRU_E_ARG, "bwd_full: B and T must be positive (got %lld, %lld)", (long long)B, (long long)T);
+  if (!x || !prep || !lambda || !dy || !ws || !dx || !dw_a || !dw_x || !db_a || !db_x || !dlambda)
+    return fail(RGLRU_E_ARG, "bwd_full: null pointer");
+  if (B * T * W >= (1ll << 40) || B * T >= (1ll << 31)) return fail(RGLRU_E_UNSUPPORTED, "bwd_full: tensor too large");
+  Geometry g = make_geometry(W, nb);
+  if (!is_aligned(x, W, g.bw, 2) || !is_aligned(dy, W, g.bw, 2) || !is_aligned(dx, W, g.bw, 2))
+    return fail(RGLRU_E_UNSUPPORTED, "bwd_full: x, dy and dx must be 16-byte aligned");
+  WorkLayout L = make_work_layout(B, T, g);
+  hipStream_t s = (hipStream_t)stream;
+  char* wb = (char*)ws;
+  rc = launch_clear(wb, L.b_begin, L.b_end, s);
+  if (rc) return rc;
+  FusedArgs a;
+  memset(&a, 0, sizeof(a));
+  fill_common(a, g, prep, dtype);
+  a.x = x; a.h0 = h0; a.flags = flags; a.dy = dy; a.dh_last = dh_last;
+  a.dx = dx; a.du_a = wb + L.du2; a.dh0 = dh0;
+  a.ckpt = (float*)(wb + L.ckpt); a.rec_a = (rec_t*)(wb + L.b_rec_a); a.rec_h = (rec_t*)(wb + L.b_rec_h);
+  a.ticket = (unsigned*)(wb + L.b_ticket); a.fail = (unsigned*)(wb + L.fail);
+  a.partial = (float*)(wb + L.partial); a.dw_partial = (float*)(wb + L.dw_partial);
+  a.B = (int)B; a.T = (int)T; a.nC = (int)((T + kChunk - 1) / kChunk); a.ckpt_nC = (int)L.nC;
+  a.aligned = 1;
+  a.wg_per_unit = pick_wg_per_unit(g, B * (long long)a.nC, 2, L.max_wg);
+  a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
+  const int nkg = held_groups(g, dtype, 1);
+  const bool masked = (flags != nullptr) || (T % kChunk != 0);
+  dim3 grid((unsigned)(a.wg_per_unit * g.units));
+  {
+    KernelTimer timer(1, s);
+#define RGLRU_LAUNCH_SCAN(N)                                                                              \
+    if (masked) hipLaunchKernelGGL((bwd_scan_kernel<__bf16, N, true>), grid, dim3(kThreads), 0, s, a);      \
+    else hipLaunchKernelGGL((bwd_scan_kernel<__bf16, N, false>), grid, dim3(kThreads), 0, s, a)
+    if (nkg == 8) { RGLRU_LAUNCH_SCAN(8); } else if (nkg == 4) { RGLRU_LAUNCH_SCAN(4); } else { RGLRU_LAUNCH_SCAN(2); }
+#undef RGLRU_LAUNCH_SCAN
+  }
+  rc = check_launch("bwd_full scan");
+  if (rc) return rc;
+  int n_wg = num_compute_units() / (int)nb; if (n_wg < 1) n_wg = 1; if (n_wg > kGemmWgPerUnit) n_wg = kGemmWgPerUnit;
+  dim3 grid2((unsigned)(n_wg * nb));
+#ifndef RGLRU_EXP_NOGEMM
+  {
+    KernelTimer timer(3, s);
+    if (nkg == 8) hipLaunchKernelGGL((gate_grad_kernel<__bf16, 8>), grid2, dim3(kThreads), 0, s, a);
+    else if (nkg == 4) hipLaunchKernelGGL((gate_grad_kernel<__bf16, 4>), grid2, dim3(kThreads), 0, s, a);
+    else hipLaunchKernelGGL((gate_grad_kernel<__bf16, 2>), grid2, dim3(kThreads), 0, s, a);
+  }
+#endif
+  rc = check_launch("bwd_full gemm");
+  if (rc) return rc;
+  ReduceArgs r;
+  r.partial = a.partial; r.lambda = lambda; r.db_a = db_a; r.db_x = db_x; r.dlambda = dlambda;
+  r.W = (int)W; r.bw = (int)g.bw; r.bwp = (int)g.bwp; r.Wp = (int)g.Wp; r.wg_per_unit = a.wg_per_unit; r.c = c;
+  hipLaunchKernelGGL(reduce_kernel, dim3((unsigned)((W + 63) / 64)), dim3(256), 0, s, r);
+  rc = check_launch("bwd_full reduce");
+  if (rc) return rc;
+  DwReduceArgs d;
+  d.dw_partial = a.dw_partial; d.dw_a = dw_a; d.dw_x = dw_x; d.nb = (int)nb; d.bw = (int)g.bw; d.bwp = (int)g.bwp; d.n_wg = n_wg;
+  const long long total = nb * g.bw * 2 * g.bw;
+  hipLaunchKernelGGL(dw_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, d);
+  return check_launch("bwd_full weight reduce");
+}
+
 int rglru_hip_step(const void* x, const void* prep, float* h, const uint8_t* flags, void* y,
                    int64_t B, int64_t W, int64_t nb, int dtype, void* stream) {
   int rc = check_geometry("step", W, nb, dtype);
@@ -961,7 +1461,7 @@ int rglru_hip_step(const void* x, const void* prep, float* h, const uint8_t* fla
 int rglru_hip_set_timing(int enable) { return g_timing.exchange(enable ? 1 : 0); }
 
 float rglru_hip_kernel_ms(int which) {
-  if (which < 0 || which > 2) return -1.f;
+  if (which < 0 || which > 3) return -1.f;
   TimingSlot& slot = timing_slot(which);
   if (!slot.armed) return -1.f;
   float ms = -1.f;

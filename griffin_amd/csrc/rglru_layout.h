@@ -31,8 +31,10 @@ inline Geometry make_geometry(int64_t W, int64_t nb) {
 //   bias  [2][Wp]            fp32
 //   sp    [Wp]               fp32   c * log2(sigmoid(Lambda))
 //   cs    [Wp]               fp32   c * log(sigmoid(Lambda))
+//   w2t   [nb][bwp][2*bwp]   storage type: w2t[k][j][2*o + gate] = W_gate[k][o][j], the operand
+//                            of the input-gradient GEMM dx += du W
 struct PrepLayout {
-  size_t wg, bias, sp, cs, total;
+  size_t wg, bias, sp, cs, w2t, total;
 };
 
 inline PrepLayout make_prep_layout(const Geometry& g, size_t elem) {
@@ -42,6 +44,7 @@ inline PrepLayout make_prep_layout(const Geometry& g, size_t elem) {
   p.bias = off; off += (size_t)round_up(2 * g.Wp * 4, 256);
   p.sp = off;   off += (size_t)round_up(g.Wp * 4, 256);
   p.cs = off;   off += (size_t)round_up(g.Wp * 4, 256);
+  p.w2t = off;  off += (size_t)round_up(2 * g.nb * g.bwp * g.bwp * (int64_t)elem, 256);
   p.total = off;
   return p;
 }
@@ -50,6 +53,8 @@ inline PrepLayout make_prep_layout(const Geometry& g, size_t elem) {
 // nCf = forward tiles of 64 tokens.
 //   ckpt        [B][nC][W]      fp32 state after each chunk (kept for backward)
 //   partial     [maxWg][3][Wp]  per-workgroup sums for db_a, db_x, dLambda
+//   du2         [B][T][2W]      16-bit: gate pre-activation gradients (fast backward only)
+//   dw_partial  [kGemmWgPerUnit][nb][bwp][2*bwp] fp32 per-workgroup weight-gradient sums
 //   --- cleared before the forward pass ---
 //   f_rec_a/h   [B][<=nC][W]    64-bit carry records of the forward chain
 //   f_ticket    [units][kMaxQueues]
@@ -57,11 +62,12 @@ inline PrepLayout make_prep_layout(const Geometry& g, size_t elem) {
 //   b_rec_a/h   [B][nC][W]      64-bit carry records of the backward chain
 //   b_ticket    [units][kMaxQueues]
 //   fail        [1]             (cleared by both)
-constexpr int kMaxQueues = 64;          // ticket queues per unit (sequences are dealt round-robin to them)
+constexpr int kMaxQueues = 64;
+constexpr int kGemmWgPerUnit = 32;      // workgroups per gate block in the gradient GEMM kernel          // ticket queues per unit (sequences are dealt round-robin to them)
 
 struct WorkLayout {
   int64_t nC, nCf, max_wg;
-  size_t ckpt, partial;
+  size_t ckpt, partial, du2, dw_partial;
   size_t f_begin, f_rec_a, f_rec_h, f_ticket, f_end;
   size_t b_begin, b_rec_a, b_rec_h, b_ticket, fail, b_end, total;
 };
@@ -75,6 +81,8 @@ inline WorkLayout make_work_layout(int64_t B, int64_t T, const Geometry& g) {
   auto take = [&](int64_t bytes) { size_t at = off; off += (size_t)round_up(bytes, 256); return at; };
   w.ckpt = take(B * w.nC * g.W * 4);
   w.partial = take(w.max_wg * 3 * g.Wp * 4);
+  w.du2 = take(B * T * 2 * g.W * 2);                      // 16-bit storage only
+  w.dw_partial = take((int64_t)kGemmWgPerUnit * g.nb * g.bwp * 2 * g.bwp * 4);
   w.f_begin = off;
   w.f_rec_a = take(B * w.nC * g.W * 8);
   w.f_rec_h = take(B * w.nC * g.W * 8);

@@ -211,28 +211,38 @@ class _HipRGLRU(torch.autograd.Function):
         dhl = None if dh_last is None else dh_last.to(torch.float32).contiguous()
         with torch.cuda.device(device):
             dx = torch.empty_like(x)
-            du_a = torch.empty_like(x)
-            du_x = torch.empty_like(x)
             db_a = torch.empty(W, dtype=torch.float32, device=device)
             db_x = torch.empty(W, dtype=torch.float32, device=device)
             dlam = torch.empty(W, dtype=torch.float32, device=device)
             dh0 = torch.empty(B, W, dtype=torch.float32, device=device) if ctx.needs_input_grad[6] else None
-            _lib.check(lib.rglru_hip_bwd(x.data_ptr(), image.data_ptr(), lam32.data_ptr(), _ptr(h0c), _ptr(flags),
-                                         dy.data_ptr(), _ptr(dhl), ws.data_ptr(), dx.data_ptr(), du_a.data_ptr(),
-                                         du_x.data_ptr(), db_a.data_ptr(), db_x.data_ptr(), dlam.data_ptr(),
-                                         _ptr(dh0), B, T, W, nb, ctx.c, code, _stream_ptr(device)), "rglru_hip_bwd")
-            # block-diagonal GEMMs: dW[k] = du[:, k]^T x[:, k];  dx[:, k] += du[:, k] W[k]
-            n = B * T
-            xk = x.view(n, nb, bw).transpose(0, 1)               # [nb, n, bw] (strided view)
-            ua = du_a.view(n, nb, bw).transpose(0, 1)
-            ux = du_x.view(n, nb, bw).transpose(0, 1)
-            wa = w_a.detach().to(x.dtype)
-            wx = w_x.detach().to(x.dtype)
-            dw_a = torch.bmm(ua.transpose(1, 2), xk)
-            dw_x = torch.bmm(ux.transpose(1, 2), xk)
-            dxg = torch.bmm(ua, wa)
-            dxg = torch.baddbmm(dxg, ux, wx)
-            dx = (dx.view(n, nb, bw).float() + dxg.transpose(0, 1).float()).to(x.dtype).view(B, T, W)
+            if lib.rglru_hip_fast_path(W, nb, code) and dy.data_ptr() % 16 == 0 and x.data_ptr() % 16 == 0:
+                # everything in hand-written kernels, including the two gate GEMMs
+                dw_a = torch.empty(nb, bw, bw, dtype=torch.float32, device=device)
+                dw_x = torch.empty(nb, bw, bw, dtype=torch.float32, device=device)
+                _lib.check(lib.rglru_hip_bwd_full(x.data_ptr(), image.data_ptr(), lam32.data_ptr(), _ptr(h0c), _ptr(flags),
+                                                  dy.data_ptr(), _ptr(dhl), ws.data_ptr(), dx.data_ptr(), dw_a.data_ptr(),
+                                                  dw_x.data_ptr(), db_a.data_ptr(), db_x.data_ptr(), dlam.data_ptr(),
+                                                  _ptr(dh0), B, T, W, nb, ctx.c, code, _stream_ptr(device)),
+                           "rglru_hip_bwd_full")
+            else:
+                du_a = torch.empty_like(x)
+                du_x = torch.empty_like(x)
+                _lib.check(lib.rglru_hip_bwd(x.data_ptr(), image.data_ptr(), lam32.data_ptr(), _ptr(h0c), _ptr(flags),
+                                             dy.data_ptr(), _ptr(dhl), ws.data_ptr(), dx.data_ptr(), du_a.data_ptr(),
+                                             du_x.data_ptr(), db_a.data_ptr(), db_x.data_ptr(), dlam.data_ptr(),
+                                             _ptr(dh0), B, T, W, nb, ctx.c, code, _stream_ptr(device)), "rglru_hip_bwd")
+                # block-diagonal library GEMMs: dW[k] = du[:, k]^T x[:, k];  dx[:, k] += du[:, k] W[k]
+                n = B * T
+                xk = x.view(n, nb, bw).transpose(0, 1)               # [nb, n, bw] (strided view)
+                ua = du_a.view(n, nb, bw).transpose(0, 1)
+                ux = du_x.view(n, nb, bw).transpose(0, 1)
+                wa = w_a.detach().to(x.dtype)
+                wx = w_x.detach().to(x.dtype)
+                dw_a = torch.bmm(ua.transpose(1, 2), xk)
+                dw_x = torch.bmm(ux.transpose(1, 2), xk)
+                dxg = torch.bmm(ua, wa)
+                dxg = torch.baddbmm(dxg, ux, wx)
+                dx = (dx.view(n, nb, bw).float() + dxg.transpose(0, 1).float()).to(x.dtype).view(B, T, W)
         pd = ctx.param_dtypes
         grads = (dx, dw_a.to(pd[0]), db_a.view(nb, bw).to(pd[1]), dw_x.to(pd[2]), db_x.view(nb, bw).to(pd[3]),
                  dlam.to(pd[4]), None if dh0 is None else dh0.to(ctx.h0_dtype), None, None)

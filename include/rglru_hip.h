@@ -9,7 +9,7 @@
  *   griffin/triton_scan.py:207-244  _FusedRGLRUScan.forward   rglru_hip_scan_fwd
  *   griffin/triton_scan.py:246-271  _FusedRGLRUScan.backward  rglru_hip_scan_bwd
  *   griffin/griffin.py:237-289      RG_LRU.forward (gates + scan, T > 1)   rglru_hip_prepare + rglru_hip_fwd
- *   autograd of griffin/griffin.py:237-289                                   rglru_hip_bwd
+ *   autograd of griffin/griffin.py:237-289                                   rglru_hip_bwd, rglru_hip_bwd_full
  *   griffin/griffin.py:279-284 with T == 1 (decode step, carried state)     rglru_hip_step
  *
  * Conventions
@@ -104,6 +104,18 @@ int rglru_hip_bwd(const void* x, const void* prep, const float* lambda, const fl
                   float* dh0, int64_t B, int64_t T, int64_t W, int64_t nb, float c, int dtype,
                   void* stream);
 
+/* Complete backward for the fast configurations (rglru_hip_fast_path(W, nb, dtype) != 0: 16-bit
+ * storage, gate blocks of 32, 64 or 128 channels, 16-byte aligned tensors).  Same inputs as
+ * rglru_hip_bwd; dx[B,T,W] is the full input gradient and dw_a, dw_x [nb,bw,bw] fp32 the weight
+ * gradients: the two gate GEMMs run in a second hand-written kernel instead of being left to the
+ * caller.  Returns RGLRU_E_UNSUPPORTED for other configurations. */
+int rglru_hip_fast_path(int64_t W, int64_t nb, int dtype);
+int rglru_hip_bwd_full(const void* x, const void* prep, const float* lambda, const float* h0,
+                       const uint8_t* flags, const void* dy, const float* dh_last, void* ws,
+                       void* dx, float* dw_a, float* dw_x, float* db_a, float* db_x, float* dlambda,
+                       float* dh0, int64_t B, int64_t T, int64_t W, int64_t nb, float c, int dtype,
+                       void* stream);
+
 /* One decode step (T == 1): h[B,W] fp32 is updated in place, y[B,W] (dtype) = h as stored. */
 int rglru_hip_step(const void* x, const void* prep, float* h, const uint8_t* flags, void* y,
                    int64_t B, int64_t W, int64_t nb, int dtype, void* stream);
@@ -120,8 +132,8 @@ int rglru_hip_workspace_status(const void* ws, int64_t B, int64_t T, int64_t W, 
  * main kernel (not the small clear / reduce launches) with HIP events on the call's stream.
  * rglru_hip_kernel_ms(which) waits for the most recent bracket (process-wide, so enable it from one
  * thread and keep calls sequential) and returns its
- * duration in milliseconds (negative when none was recorded): which = 0 forward, 1 backward,
- * 2 step.  Not for use under stream capture. */
+ * duration in milliseconds (negative when none was recorded): which = 0 forward, 1 backward
+ * (scan part), 2 step, 3 backward gradient GEMMs (rglru_hip_bwd_full only).  Not for use under stream capture. */
 int rglru_hip_set_timing(int enable);
 float rglru_hip_kernel_ms(int which);
 
