@@ -66,7 +66,9 @@ template <> struct Io<float> {
 // ------------------------------------------------------------------------------------------
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef __amdgpu_buffer_rsrc_t rsrc_t;
-constexpr unsigned kOutOfRange = 0x7fffffffu;
+// Offset that no extent reaches.  It is 16-byte aligned: atomics must be naturally aligned even
+// when the range check is going to drop them.
+constexpr unsigned kOutOfRange = 0x7ffffff0u;
 
 RGLRU_DEVICE rsrc_t make_rsrc(const void* base, unsigned bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
@@ -91,9 +93,6 @@ template <> struct BufIo<float> {
 };
 RGLRU_DEVICE void buf_store_b128(i32x4 v, rsrc_t r, unsigned voff) {
   __builtin_amdgcn_raw_buffer_store_b128(v, r, voff, 0, 0);
-#ifdef RGLRU_EXP_STOREWAIT
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-#endif
 }
 template <typename Frag> RGLRU_DEVICE Frag buf_load_frag(rsrc_t r, unsigned voff) {
   return __builtin_bit_cast(Frag, __builtin_amdgcn_raw_buffer_load_b128(r, voff, 0, 0));
@@ -152,96 +151,148 @@ RGLRU_DEVICE float xhalf(float v, int hf) {
 
 // ------------------------------------------------------------------------------------------
 // Chunk carry protocol.  A scan over time is cut into chunks that are processed by different
-// waves.  Each (sequence, chunk, channel) owns two 64-bit records {fp32 value, 32-bit version}
-// that describe the chunk as an affine map of the carry: carry_out = A * carry_in + H.
-//   version 0            nothing published yet (records start out cleared)
-//   version kVerLocal    (A, H) is the chunk's own map: the reader must go on to the chunk before
-//   version kVerFinal    the chunk knows its carry_in: A = 0 and H = carry_out, the walk ends here
-// Value and version travel in one naturally aligned 8-byte access issued at device scope (sc1), so
-// a reader sees a record entirely or not at all and no fence is needed on either side; a reader
-// that catches the two records of a chunk at different versions simply polls again.  A wave that
-// needs its carry_in loads the records of the kDepth chunks before it in one round trip and
-// composes them in chain order until the accumulated A becomes 0 or the boundary is reached.
-// Chunks are handed out through ticket counters in chain order, so every record a wave waits for
-// belongs to a wave that is already running.
+// waves.  Each (sequence, chunk, channel) owns ONE 64-bit record that describes the chunk as an
+// affine map of the carry, carry_out = A * carry_in + H:  low word = bits of A with the lowest
+// mantissa bit forced to 1, high word = bits of H.
+//   low word == 0   nothing published yet (records start out cleared)
+//   low word == 1   A = 0: the chunk knows its carry_in and H is its carry_out; a walk ends here
+//   otherwise       (A, H) is the chunk's own map and the reader goes on to the chunk before
+// The record travels in one naturally aligned 8-byte access issued at device scope (sc1), so a reader
+// sees it entirely or not at all and no fence is needed on either side; a chunk that learns its
+// carry simply overwrites its record.  A wave that needs its carry_in loads the records of the
+// kDepth chunks before it in one round trip and composes them in chain order until A becomes 0 or
+// the boundary is reached.  Chunks are handed out through ticket counters in chain order, so every
+// record a wave waits for belongs to a wave that is already running.
 // ------------------------------------------------------------------------------------------
 typedef unsigned long long rec_t;
-constexpr unsigned kVerLocal = 1u, kVerFinal = 2u;
-constexpr int kDepth = 4;
+constexpr int kDepth = 8;
 
-RGLRU_DEVICE void rec_store(rec_t* p, float v, unsigned ver) {
-  __hip_atomic_store(p, ((rec_t)ver << 32) | (rec_t)__float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+RGLRU_DEVICE void rec_store(rec_t* p, float a, float h) {
+  const rec_t bits = ((rec_t)__float_as_uint(h) << 32) | (rec_t)(__float_as_uint(a) | 1u);
+  __hip_atomic_store(p, bits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// cache policy of a record access issued through a buffer descriptor: device scope (sc1)
+constexpr int kRecPolicy = 16;
 RGLRU_DEVICE rec_t rec_load(const rec_t* p) {
   return __hip_atomic_load(const_cast<rec_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-RGLRU_DEVICE unsigned rec_ver(rec_t r) { return (unsigned)(r >> 32); }
-RGLRU_DEVICE float rec_val(rec_t r) { return __uint_as_float((unsigned)r); }
 
 struct CarryChain {
-  rec_t* rec_a;       // per-lane pointers, already offset to (sequence, channel); chunk c at + c * stride
-  rec_t* rec_h;
+  rec_t* rec;         // per-lane pointer, already offset to (sequence, channel); chunk c at + c * stride
   long long stride;
 };
 
-RGLRU_DEVICE void carry_publish(const CarryChain& ch, int c, float a, float h, unsigned ver) {
-  rec_store(ch.rec_a + c * ch.stride, a, ver);
-  rec_store(ch.rec_h + c * ch.stride, h, ver);
+// Publish the chunk's own map (final = false) or its carry_out (final = true, `a` is ignored).
+RGLRU_DEVICE void carry_publish(const CarryChain& ch, int c, float a, float h, bool final) {
+  rec_store(ch.rec + c * ch.stride, final ? 0.f : a, h);
 }
 
-// carry_in of chunk c.  `step` is -1 when the chain runs forward in time (the chunk before c is
-// c - 1) and +1 when it runs backward; `end` is the index one past the first chunk of the chain
-// (-1 or the chunk count), where `boundary` is the carry.  After `limit` fruitless polls the wave
-// records the failure and returns an unspecified value, so every wave still reaches the end of the
-// kernel.
-RGLRU_DEVICE float carry_lookback(const CarryChain& ch, int c, int step, int end, float boundary,
-                                  bool lane_ok, long long limit, unsigned* fail_word) {
-  float acc_a = 1.f, acc_h = 0.f;
-  bool done = !lane_ok;
-  int p = c + step;
+// State of one walk along a chain: the composed map of the chunks consumed so far.
+struct CarryWalk {
+  float acc_a, acc_h;
+  bool done;
+  int p;              // next chunk to consume
+};
+
+// Compose one batch of records (chunks p, p + step, ...) into the walk.  Returns true when the
+// batch ran into a record that is not published yet; p then names that chunk.
+RGLRU_DEVICE bool carry_compose(const rec_t (&rec)[kDepth], CarryWalk& wk, int step, int end, float boundary) {
+#pragma unroll
+  for (int d = 0; d < kDepth; ++d) {
+    const int q = wk.p + d * step;
+    if (q == end) {                                      // wave-uniform
+      if (!wk.done) { wk.acc_h = fmaf(wk.acc_a, boundary, wk.acc_h); wk.acc_a = 0.f; wk.done = true; }
+      return false;
+    }
+    const unsigned lo = (unsigned)rec[d];
+    if (!__all(wk.done || lo != 0u)) { wk.p = q; return true; }
+    if (!wk.done) {
+      wk.acc_h = fmaf(wk.acc_a, __uint_as_float((unsigned)(rec[d] >> 32)), wk.acc_h);
+      if (lo == 1u) { wk.acc_a = 0.f; wk.done = true; }
+      else wk.acc_a *= __uint_as_float(lo);
+    }
+  }
+  wk.p += kDepth * step;
+  return false;
+}
+
+// Polling part of a walk: load a batch, compose, repeat until every lane has its carry.  After
+// `limit` fruitless polls the wave records the failure and returns an unspecified value, so every
+// wave still reaches the end of the kernel.
+RGLRU_DEVICE float carry_walk(const CarryChain& ch, CarryWalk& wk, int step, int end, float boundary,
+                              long long limit, unsigned* fail_word, int* stat) {
   long long polls = 0;
-  for (;;) {
-    rec_t ra[kDepth], rh[kDepth];
+  while (!__all(wk.done)) {
+    if (stat) stat[0] += 1;                              // development aid: round trips
+    rec_t rec[kDepth];
 #pragma unroll
     for (int d = 0; d < kDepth; ++d) {
-      const int q = p + d * step;
+      const int q = wk.p + d * step;
       const bool inside = (step < 0) ? (q > end) : (q < end);
-      ra[d] = 0; rh[d] = 0;
-      if (inside && !done) {
-        ra[d] = rec_load(ch.rec_a + q * ch.stride);
-        rh[d] = rec_load(ch.rec_h + q * ch.stride);
-      }
+      rec[d] = 0;
+      if (inside && !wk.done) rec[d] = rec_load(ch.rec + q * ch.stride);
     }
-    bool stalled = false;
-#pragma unroll
-    for (int d = 0; d < kDepth; ++d) {
-      if (stalled) break;
-      const int q = p + d * step;
-      if (q == end) {                                    // wave-uniform
-        if (!done) { acc_h = fmaf(acc_a, boundary, acc_h); acc_a = 0.f; done = true; }
-        break;
-      }
-      const unsigned va = rec_ver(ra[d]), vh = rec_ver(rh[d]);
-      const bool ready = done || (va == vh && va != 0u);
-      if (!__all(ready)) { stalled = true; p = q; break; }
-      if (!done) {
-        acc_h = fmaf(acc_a, rec_val(rh[d]), acc_h);
-        acc_a *= rec_val(ra[d]);
-        if (va == kVerFinal) { acc_a = 0.f; done = true; }
-      }
-    }
-    if (__all(done)) break;
-    if (stalled) {
+    if (carry_compose(rec, wk, step, end, boundary)) {
+      if (stat) stat[1] += 1;                            // development aid: stalls
       if (++polls > limit) {
         if ((threadIdx.x & 63) == 0) atomicOr(fail_word, 1u);
         break;
       }
       __builtin_amdgcn_s_sleep(1);
-    } else {
-      p += kDepth * step;
     }
   }
-  return acc_h;
+  return wk.acc_h;
+}
+
+// carry_in of chunk c.  `step` is -1 when the chain runs forward in time (the chunk before c is
+// c - 1) and +1 when it runs backward; `end` is the index one past the first chunk of the chain
+// (-1 or the chunk count), where `boundary` is the carry.
+RGLRU_DEVICE float carry_lookback(const CarryChain& ch, int c, int step, int end, float boundary,
+                                  bool lane_ok, long long limit, unsigned* fail_word, int* stat = nullptr) {
+  CarryWalk wk;
+  wk.acc_a = 1.f; wk.acc_h = 0.f; wk.done = !lane_ok; wk.p = c + step;
+  return carry_walk(ch, wk, step, end, boundary, limit, fail_word, stat);
+}
+
+// The first batch of a walk requested ahead of time.  A device-scope load takes a few
+// microseconds under load, far more than the gate math of a tile, so a caller that knows early
+// which chunk it will finish issues these loads before other work and resolves them afterwards.
+// They go through a buffer descriptor that covers the sequence's records (`lane_off` = byte offset
+// of the lane's channel, or kOutOfRange for a lane without one): chunks outside the chain are
+// masked by the offset instead of a branch, so the number of loads in flight is fixed and the
+// hardware counter can be waited on precisely.
+struct CarryBatch {
+  rec_t rec[kDepth];
+};
+
+// Record store through the same kind of descriptor; voff = kOutOfRange drops it.
+RGLRU_DEVICE void rec_store_buf(rsrc_t recs, unsigned voff, float a, float h) {
+  typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+  u32x2 v;
+  v[0] = __float_as_uint(a) | 1u; v[1] = __float_as_uint(h);
+  __builtin_amdgcn_raw_buffer_store_b64(v, recs, voff, 0, kRecPolicy);
+}
+
+RGLRU_DEVICE void carry_prefetch(rsrc_t recs, unsigned lane_off, unsigned stride_bytes, int c, int step, int end,
+                                 CarryBatch& batch) {
+  typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+  for (int d = 0; d < kDepth; ++d) {
+    const int q = c + step + d * step;
+    const bool inside = (step < 0) ? (q > end) : (q < end);
+    const unsigned voff = (inside && lane_off != kOutOfRange) ? (unsigned)q * stride_bytes + lane_off : kOutOfRange;
+    const u32x2 v = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(recs, voff, 0, kRecPolicy));
+    batch.rec[d] = ((rec_t)v[1] << 32) | (rec_t)v[0];
+  }
+}
+
+RGLRU_DEVICE float carry_lookback_from(const CarryBatch& first, const CarryChain& ch, int c, int step, int end,
+                                       float boundary, bool lane_ok, long long limit, unsigned* fail_word,
+                                       int* stat = nullptr) {
+  CarryWalk wk;
+  wk.acc_a = 1.f; wk.acc_h = 0.f; wk.done = !lane_ok; wk.p = c + step;
+  if (carry_compose(first.rec, wk, step, end, boundary) && stat) stat[1] += 1;
+  return carry_walk(ch, wk, step, end, boundary, limit, fail_word, stat);
 }
 
 // ------------------------------------------------------------------------------------------

@@ -108,7 +108,7 @@ struct FusedArgs {
   void* dx; void* du_a; void* du_x; float* dh0;           // backward out
   float* h_state;                                         // decode step (in place)
   // workspace
-  float* ckpt; rec_t* rec_a; rec_t* rec_h; unsigned* ticket;
+  float* ckpt; rec_t* rec_a; unsigned* ticket;
   unsigned* fail; float* partial; float* dw_partial;
   // geometry
   int B, T, W, nb, bw, bwp, S, Wp, groups, units;
@@ -288,55 +288,90 @@ RGLRU_DEVICE void fwd_gates(const FusedArgs& p, long long trow, int t_first, con
   }
 }
 
-// Local scan, carry exchange, final scan and stores of one wave's 64-token tile.
-// Local scan, carry exchange, final scan and stores of one wave's tile of 32 * MT tokens.
-// `prefetch` is called once the tile's own map has been published, i.e. right before the wave
-// starts waiting for its carry.
-template <typename IO, int MT, bool MASKED, bool STAGED, typename Prefetch>
-RGLRU_DEVICE void fwd_scan_store(const FusedArgs& p, const WaveId& w, int b, int c, const float (&a)[16 * MT],
-                                 const float (&z)[16 * MT], unsigned char* stage, Prefetch prefetch,
-                                 int trace_iter = 0) {
-  constexpr int EL = 16 * MT, TR = 32 * MT;
+// One wave's tile of 32 * MT tokens between its two stages: gate outputs in time order, the affine
+// maps of the lower lane run and of the whole tile, and where the tile sits.
+template <int MT>
+struct FwdTile {
+  float a[16 * MT], z[16 * MT];
+  float A_lo, H_lo, A_t, H_t;
+  int b, c;
+};
+
+// Descriptor of one sequence's forward carry records.
+RGLRU_DEVICE rsrc_t seq_records(const FusedArgs& p, int b) {
+  return make_rsrc(p.rec_a + (long long)b * p.nCf * p.W, (unsigned)p.nCf * (unsigned)p.W * 8u);
+}
+
+// Stage 1: affine map of the tile from (a, z); publishes it unless the tile starts its chain.
+template <int MT, bool MASKED>
+RGLRU_DEVICE void fwd_local(const FusedArgs& p, const WaveId& w, FwdTile<MT>& t, bool live = true) {
+  constexpr int EL = 16 * MT;
   const int hf = w.hf;
-  const long long W = p.W;
-  const int t0 = c * TR;
-  const bool ch_ok = MASKED ? w.ch_ok : true;
-  // affine map of this lane's run, then of the whole tile
   float A = 1.f, H = 0.f;
 #pragma unroll
-  for (int e = 0; e < EL; ++e) { H = fmaf(a[e], H, z[e]); A *= a[e]; }
+  for (int e = 0; e < EL; ++e) { H = fmaf(t.a[e], H, t.z[e]); A *= t.a[e]; }
   const float A_o = xhalf(A, hf), H_o = xhalf(H, hf);
-  const float A_lo = hf ? A_o : A, H_lo = hf ? H_o : H;
+  t.A_lo = hf ? A_o : A; t.H_lo = hf ? H_o : H;
   const float A_hi = hf ? A : A_o, H_hi = hf ? H : H_o;
-  const float A_t = A_hi * A_lo, H_t = fmaf(A_hi, H_lo, H_hi);
+  t.A_t = A_hi * t.A_lo; t.H_t = fmaf(A_hi, t.H_lo, H_hi);
+  const bool ch_ok = (MASKED ? w.ch_ok : true) && live;
+  // every store of the pipelined loop is issued unconditionally and masked through its offset, so
+  // the number of memory operations in flight is the same on every path
+  const unsigned voff = (t.c != 0 && ch_ok && hf == 0) ? ((unsigned)t.c * (unsigned)p.W + (unsigned)w.ch) * 8u : kOutOfRange;
+  rec_store_buf(seq_records(p, t.b), voff, t.A_t, t.H_t);
+}
 
+// Stage 2: carry in, carry out and checkpoint, then the recurrence itself and the stores.
+template <typename IO, int MT, bool MASKED, bool STAGED>
+RGLRU_DEVICE void fwd_finalize(const FusedArgs& p, const WaveId& w, const FwdTile<MT>& t, unsigned char* stage,
+                               const CarryBatch* first = nullptr, bool live = true, int trace_iter = 0) {
+  constexpr int EL = 16 * MT, TR = 32 * MT;
+  const int hf = w.hf, b = t.b, c = t.c;
+  const long long W = p.W;
+  const int t0 = c * TR;
+  const bool ch_ok = (MASKED ? w.ch_ok : true) && live;     // a dead call stores nothing
   CarryChain chain;
-  const long long seq = (long long)b * p.nCf * W + w.ch;
-  chain.rec_a = p.rec_a + seq; chain.rec_h = p.rec_h + seq; chain.stride = W;
+  chain.rec = p.rec_a + (long long)b * p.nCf * W + w.ch; chain.stride = W;
 
-  if (c != 0 && ch_ok && hf == 0) carry_publish(chain, c, A_t, H_t, kVerLocal);
-  prefetch();
-  float h_in = (c == 0 && ch_ok && p.h0) ? p.h0[(long long)b * W + w.ch] : 0.f;
+  float h_in = 0.f;
   RGLRU_STAMP(p, 5);
-#ifndef RGLRU_EXP_NOLOOKBACK
-  if (c != 0) h_in = carry_lookback(chain, c, -1, -1, 0.f, ch_ok, p.limit, p.fail);
+#ifdef RGLRU_TRACE
+  int stat[2] = {0, 0};
+  int* stat_p = stat;
+#else
+  int* stat_p = nullptr;
+#endif
+  if (c != 0) {
+    h_in = first ? carry_lookback_from(*first, chain, c, -1, -1, 0.f, ch_ok, p.limit, p.fail, stat_p)
+                 : carry_lookback(chain, c, -1, -1, 0.f, ch_ok, p.limit, p.fail, stat_p);
+  } else if (p.h0 && ch_ok) {
+    h_in = p.h0[(long long)b * W + w.ch];
+  }
+#ifdef RGLRU_TRACE
+  if (p.trace && w.lane == 0 && trace_iter < 8) {
+    long long* t_ = p.trace + (((long long)blockIdx.x * 4 + (threadIdx.x >> 6)) * 8 + trace_iter) * 12;
+    t_[8] = stat[0]; t_[9] = stat[1]; t_[10] = c;
+  }
 #endif
   RGLRU_STAMP(p, 6);
-  const float h_end = fmaf(A_t, h_in, H_t);
-  const float h_mid = fmaf(A_lo, h_in, H_lo);
-  if (ch_ok) {
-    if (hf == 0) {
-      carry_publish(chain, c, 0.f, h_end, kVerFinal);
-      p.ckpt[((long long)b * p.ckpt_nC + c * MT + (MT - 1)) * W + w.ch] = h_end;
-      if (c == p.nCf - 1 && p.h_last) p.h_last[(long long)b * W + w.ch] = h_end;
-    } else if (MT == 2) {
-      p.ckpt[((long long)b * p.ckpt_nC + c * MT) * W + w.ch] = h_mid;
-    }
+  const float h_end = fmaf(t.A_t, h_in, t.H_t);
+  const float h_mid = fmaf(t.A_lo, h_in, t.H_lo);
+  {
+    // carry out, checkpoint(s) and final state: unconditional stores masked through their offsets
+    const unsigned uW = (unsigned)W, ch = (unsigned)w.ch;
+    const bool lower = ch_ok && hf == 0;
+    rec_store_buf(seq_records(p, b), lower ? ((unsigned)c * uW + ch) * 8u : kOutOfRange, 0.f, h_end);
+    const rsrc_t rck = make_rsrc(p.ckpt + (long long)b * p.ckpt_nC * W, (unsigned)p.ckpt_nC * uW * 4u);
+    unsigned ck_off = lower ? ((unsigned)(c * MT + (MT - 1)) * uW + ch) * 4u : kOutOfRange;
+    if (MT == 2 && ch_ok && hf != 0) ck_off = ((unsigned)(c * MT) * uW + ch) * 4u;
+    BufIo<float>::store(hf ? h_mid : h_end, rck, ck_off, 0u);
+    const rsrc_t rhl = make_rsrc(p.h_last, p.h_last ? (unsigned)p.B * uW * 4u : 0u);
+    BufIo<float>::store(h_end, rhl, (lower && c == p.nCf - 1) ? ((unsigned)b * uW + ch) * 4u : kOutOfRange, 0u);
   }
 
   float h = hf ? h_mid : h_in;
   // y tile through a buffer descriptor: rows past the end of the sequence are dropped
-  const int rows = (p.T - t0) < TR ? (p.T - t0) : TR;
+  const int rows = !live ? 0 : ((p.T - t0) < TR ? (p.T - t0) : TR);
   const unsigned row_bytes = (unsigned)p.W * (unsigned)sizeof(IO);
   const rsrc_t ry = make_rsrc((const IO*)p.y + ((long long)b * p.T + t0) * W, (unsigned)rows * row_bytes);
   if constexpr (STAGED) {
@@ -344,7 +379,7 @@ RGLRU_DEVICE void fwd_scan_store(const FusedArgs& p, const WaveId& w, int b, int
     unsigned char* my = stage + WaveStage<TR>::row_offset(hf * EL) + w.r * 2;
 #pragma unroll
     for (int e = 0; e < EL; ++e) {
-      h = fmaf(a[e], h, z[e]);
+      h = fmaf(t.a[e], h, t.z[e]);
       *reinterpret_cast<IO*>(my + e * WaveStage<TR>::kRowBytes) = (IO)h;
     }
     wave_lds_fence();
@@ -356,7 +391,7 @@ RGLRU_DEVICE void fwd_scan_store(const FusedArgs& p, const WaveId& w, int b, int
     unsigned voff = ch_ok ? (unsigned)(hf * EL) * row_bytes + (unsigned)w.ch * (unsigned)sizeof(IO) : kOutOfRange;
 #pragma unroll
     for (int e = 0; e < EL; ++e) {
-      h = fmaf(a[e], h, z[e]);
+      h = fmaf(t.a[e], h, t.z[e]);
       BufIo<IO>::store((IO)h, ry, voff + (unsigned)e * row_bytes, 0u);
     }
   }
@@ -420,12 +455,34 @@ __global__ __launch_bounds__(kThreads, 2) void fwd_kernel(FusedArgs p) {
     int par = 0;
     issue(tk);
     int trace_iter = 0; (void)trace_iter;
+    // Two tiles are in flight per wave: the tile whose own map was published in the previous
+    // iteration is finished (carry in, recurrence, stores) after the gate math of the current one,
+    // so the wait for the neighbours' records overlaps with useful work.
+    FwdTile<MT> cur, prev;
+    bool have_prev = false;
+    prev.b = 0; prev.c = 0;                              // chunk 0 has no records to request
+#pragma unroll
+    for (int e = 0; e < EL; ++e) { prev.a[e] = 0.f; prev.z[e] = 0.f; }
+    prev.A_lo = prev.H_lo = prev.A_t = prev.H_t = 0.f;
+    // a gate block of 128 channels fills all four waves; narrower ones leave waves without a slab
+    const bool slab_ok = (NKG == 8) ? true : w.slab_ok;
+    const rsrc_t rticket = make_rsrc(q.counter, 4u);
+    const unsigned rec_stride = (unsigned)W * 8u;
+    const unsigned rec_lane = (slab_ok && w.ch_ok) ? (unsigned)w.ch * 8u : kOutOfRange;
+    // A dead finalize in front of the loop: the loop is entered with the same memory operations in
+    // flight as its back edge has, so the waits at its top are exact instead of worst case.
+    fwd_finalize<IO, MT, MASKED, sizeof(IO) == 2>(p, w, prev, stage, nullptr, false, 0);
     while (tk < q.tiles) {
       RGLRU_STAMP(p, 0);
-      const int c = (int)(tk / q.n_b), b = q.first_b + (int)(tk - (long long)c * q.n_b) * p.queues;
-      const long long trow = (long long)b * p.T + c * TR + hf * EL;
-      unsigned next_raw = 0;
-      if (tid == 0) next_raw = atomicAdd(q.counter, 1u);
+      cur.c = (int)((unsigned)tk / (unsigned)q.n_b);
+      cur.b = q.first_b + (int)((unsigned)tk - (unsigned)cur.c * (unsigned)q.n_b) * p.queues;
+      const long long trow = (long long)cur.b * p.T + cur.c * TR + hf * EL;
+      // next ticket: one instruction for the whole workgroup, live only in its first lane
+      const unsigned next_raw = (unsigned)__builtin_amdgcn_raw_ptr_buffer_atomic_add_i32(1, rticket, tid == 0 ? 0u : kOutOfRange, 0, 0);
+      // records the previous tile will need: requested now, used after this tile's gate math
+      CarryBatch ahead;
+      carry_prefetch(make_rsrc(p.rec_a + (long long)prev.b * p.nCf * W, (unsigned)p.nCf * rec_stride), rec_lane,
+                     rec_stride, prev.c, -1, -1, ahead);
 #pragma unroll
       for (int i = 0; i < NV; ++i) {
         const int idx = tid + i * kThreads;
@@ -434,32 +491,32 @@ __global__ __launch_bounds__(kThreads, 2) void fwd_kernel(FusedArgs p) {
       }
       __syncthreads();
       RGLRU_STAMP(p, 1);
-      float a[EL], z[EL];
-      if (w.slab_ok) {
+      if (slab_ok) {
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
           f32x16 ua, ux;
           float xv[16];
           gate_mfma_held<IO, MT, NKG>(lds, hw, mt, w.slab, w.r, hf, bias_a, bias_x, ua, ux, xv);
-          fwd_gates<IO, MASKED>(p, trow + 16 * mt, c * TR + hf * EL + 16 * mt, ua, ux, xv, sp, a + 16 * mt, z + 16 * mt);
+          fwd_gates<IO, MASKED>(p, trow + 16 * mt, cur.c * TR + hf * EL + 16 * mt, ua, ux, xv, sp, cur.a + 16 * mt, cur.z + 16 * mt);
         }
       }
+      fwd_local<MT, MASKED>(p, w, cur, slab_ok);
       RGLRU_STAMP(p, 2);
       if (tid == 0) s_ticket[par ^ 1] = next_raw;
       __syncthreads();
       RGLRU_STAMP(p, 3);
       par ^= 1;
       const long long tk_next = s_ticket[par];
-      if (w.slab_ok) {
-        RGLRU_STAMP(p, 4);
-        fwd_scan_store<IO, MT, MASKED, sizeof(IO) == 2>(p, w, b, c, a, z, stage, [&]() { issue(tk_next); }, trace_iter);
-      } else {
-        issue(tk_next);
-      }
+      issue(tk_next);
+      RGLRU_STAMP(p, 4);
+      fwd_finalize<IO, MT, MASKED, sizeof(IO) == 2>(p, w, prev, stage, &ahead, have_prev && slab_ok, trace_iter);
+      prev = cur;
+      have_prev = true;
       RGLRU_STAMP(p, 7);
       ++trace_iter;
       tk = tk_next;
     }
+    if (slab_ok && have_prev) fwd_finalize<IO, MT, MASKED, sizeof(IO) == 2>(p, w, prev, stage, nullptr, true, trace_iter);
   } else {
     for (;;) {
       if (tid == 0) s_ticket[0] = atomicAdd(q.counter, 1u);
@@ -473,15 +530,17 @@ __global__ __launch_bounds__(kThreads, 2) void fwd_kernel(FusedArgs p) {
                                 w_a_row, w_x_row, bias_a, bias_x, lds, ua, ux, xv);
       if (w.slab_ok) {
         const long long trow = (long long)b * p.T + c * TR + hf * EL;
-        float a[EL], z[EL];
+        FwdTile<MT> tile;
+        tile.b = b; tile.c = c;
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
           float xpart[16];
 #pragma unroll
           for (int e = 0; e < 16; ++e) xpart[e] = xv[16 * mt + e];
-          fwd_gates<IO, true>(p, trow + 16 * mt, c * TR + hf * EL + 16 * mt, ua[mt], ux[mt], xpart, sp, a + 16 * mt, z + 16 * mt);
+          fwd_gates<IO, true>(p, trow + 16 * mt, c * TR + hf * EL + 16 * mt, ua[mt], ux[mt], xpart, sp, tile.a + 16 * mt, tile.z + 16 * mt);
         }
-        fwd_scan_store<IO, MT, true, false>(p, w, b, c, a, z, stage, []() {});
+        fwd_local<MT, true>(p, w, tile);
+        fwd_finalize<IO, MT, true, false>(p, w, tile, stage);
       }
     }
   }
@@ -585,17 +644,17 @@ __global__ __launch_bounds__(kThreads) void bwd_kernel(FusedArgs p) {
 
     CarryChain chain;
     const long long seq = (long long)b * p.nC * W + w.ch;
-    chain.rec_a = p.rec_a + seq; chain.rec_h = p.rec_h + seq; chain.stride = W;
+    chain.rec = p.rec_a + seq; chain.stride = W;
 
     float d_in;
     if (c == p.nC - 1) {
       d_in = (w.ch_ok && p.dh_last) ? p.dh_last[(long long)b * W + w.ch] : 0.f;
     } else {
-      if (w.ch_ok && hf == 0) carry_publish(chain, c, A_t, D_t, kVerLocal);
+      if (w.ch_ok && hf == 0) carry_publish(chain, c, A_t, D_t, false);
       d_in = carry_lookback(chain, c, +1, p.nC, 0.f, w.ch_ok, p.limit, p.fail);
     }
     const float d_out = fmaf(A_t, d_in, D_t);
-    if (w.ch_ok && hf == 0) carry_publish(chain, c, 0.f, d_out, kVerFinal);
+    if (w.ch_ok && hf == 0) carry_publish(chain, c, 0.f, d_out, true);
     if (c == 0 && p.dh0 && w.ch_ok && hf == 0) p.dh0[(long long)b * W + w.ch] = d_out;
 
     carry = hf ? d_in : fmaf(A_hi, d_in, D_hi);
@@ -778,14 +837,14 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
 
     CarryChain chain;
     const long long seq = (long long)b * p.nC * W + w.ch;
-    chain.rec_a = p.rec_a + seq; chain.rec_h = p.rec_h + seq; chain.stride = W;
+    chain.rec = p.rec_a + seq; chain.stride = W;
     const bool last_chunk = c == p.nC - 1;
-    if (!last_chunk && hf == 0) carry_publish(chain, c, A_t, D_t, kVerLocal);
+    if (!last_chunk && hf == 0) carry_publish(chain, c, A_t, D_t, false);
     issue(tk_next);
     float d_in = (last_chunk && p.dh_last) ? p.dh_last[(long long)b * W + w.ch] : 0.f;
     if (!last_chunk) d_in = carry_lookback(chain, c, +1, p.nC, 0.f, true, p.limit, p.fail);
     const float d_out = fmaf(A_t, d_in, D_t);
-    if (hf == 0) carry_publish(chain, c, 0.f, d_out, kVerFinal);
+    if (hf == 0) carry_publish(chain, c, 0.f, d_out, true);
     if (hf == 0 && c == 0 && p.dh0) p.dh0[(long long)b * W + w.ch] = d_out;
 
     // delta_t in place of dy_t (reverse), then one forward pass that carries h_{t-1} along
@@ -1295,7 +1354,7 @@ int rglru_hip_fwd(const void* x, const void* prep, const float* h0, const uint8_
   memset(&a, 0, sizeof(a));
   fill_common(a, g, prep, dtype);
   a.x = x; a.h0 = h0; a.flags = flags; a.y = y; a.h_last = h_last;
-  a.ckpt = (float*)(wb + L.ckpt); a.rec_a = (rec_t*)(wb + L.f_rec_a); a.rec_h = (rec_t*)(wb + L.f_rec_h);
+  a.ckpt = (float*)(wb + L.ckpt); a.rec_a = (rec_t*)(wb + L.f_rec_a);
   a.ticket = (unsigned*)(wb + L.f_ticket); a.fail = (unsigned*)(wb + L.fail);
   a.B = (int)B; a.T = (int)T; a.nC = (int)L.nC; a.ckpt_nC = (int)L.nC;
   a.nCf = (int)((T + 32 * kFwdMT - 1) / (32 * kFwdMT));
@@ -1336,7 +1395,7 @@ int rglru_hip_bwd(const void* x, const void* prep, const float* lambda, const fl
   fill_common(a, g, prep, dtype);
   a.x = x; a.h0 = h0; a.flags = flags; a.dy = dy; a.dh_last = dh_last;
   a.dx = dx; a.du_a = du_a; a.du_x = du_x; a.dh0 = dh0;
-  a.ckpt = (float*)(wb + L.ckpt); a.rec_a = (rec_t*)(wb + L.b_rec_a); a.rec_h = (rec_t*)(wb + L.b_rec_h);
+  a.ckpt = (float*)(wb + L.ckpt); a.rec_a = (rec_t*)(wb + L.b_rec_a);
   a.ticket = (unsigned*)(wb + L.b_ticket); a.fail = (unsigned*)(wb + L.fail);
   a.partial = (float*)(wb + L.partial);
   a.B = (int)B; a.T = (int)T; a.nC = (int)((T + kChunk - 1) / kChunk); a.ckpt_nC = (int)L.nC; a.nCf = (int)L.nCf;
@@ -1389,7 +1448,7 @@ int rglru_hip_bwd_full(const void* x, const void* prep, const float* lambda, con
   fill_common(a, g, prep, dtype);
   a.x = x; a.h0 = h0; a.flags = flags; a.dy = dy; a.dh_last = dh_last;
   a.dx = dx; a.du_a = wb + L.du2; a.dh0 = dh0;
-  a.ckpt = (float*)(wb + L.ckpt); a.rec_a = (rec_t*)(wb + L.b_rec_a); a.rec_h = (rec_t*)(wb + L.b_rec_h);
+  a.ckpt = (float*)(wb + L.ckpt); a.rec_a = (rec_t*)(wb + L.b_rec_a);
   a.ticket = (unsigned*)(wb + L.b_ticket); a.fail = (unsigned*)(wb + L.fail);
   a.partial = (float*)(wb + L.partial); a.dw_partial = (float*)(wb + L.dw_partial);
   a.B = (int)B; a.T = (int)T; a.nC = (int)((T + kChunk - 1) / kChunk); a.ckpt_nC = (int)L.nC;

@@ -56,20 +56,20 @@ inline PrepLayout make_prep_layout(const Geometry& g, size_t elem) {
 //   du2         [B][T][2W]      16-bit: gate pre-activation gradients (fast backward only)
 //   dw_partial  [kGemmWgPerUnit][nb][bwp][2*bwp] fp32 per-workgroup weight-gradient sums
 //   --- cleared before the forward pass ---
-//   f_rec_a/h   [B][<=nC][W]    64-bit carry records of the forward chain
+//   f_rec_a     [B][<=nC][W]    64-bit carry records of the forward chain
 //   f_ticket    [units][kMaxQueues]
 //   --- cleared before the backward pass ---
-//   b_rec_a/h   [B][nC][W]      64-bit carry records of the backward chain
+//   b_rec_a     [B][nC][W]      64-bit carry records of the backward chain
 //   b_ticket    [units][kMaxQueues]
 //   fail        [1]             (cleared by both)
-constexpr int kMaxQueues = 64;
-constexpr int kGemmWgPerUnit = 32;      // workgroups per gate block in the gradient GEMM kernel          // ticket queues per unit (sequences are dealt round-robin to them)
+constexpr int kMaxQueues = 64;          // ticket queues per unit (sequences are dealt round-robin to them)
+constexpr int kGemmWgPerUnit = 32;      // workgroups per gate block in the gradient GEMM kernel
 
 struct WorkLayout {
   int64_t nC, nCf, max_wg;
   size_t ckpt, partial, du2, dw_partial;
-  size_t f_begin, f_rec_a, f_rec_h, f_ticket, f_end;
-  size_t b_begin, b_rec_a, b_rec_h, b_ticket, fail, b_end, total;
+  size_t f_begin, f_rec_a, f_ticket, f_end;
+  size_t b_begin, b_rec_a, b_ticket, fail, b_end, total;
 };
 
 inline WorkLayout make_work_layout(int64_t B, int64_t T, const Geometry& g) {
@@ -85,12 +85,10 @@ inline WorkLayout make_work_layout(int64_t B, int64_t T, const Geometry& g) {
   w.dw_partial = take((int64_t)kGemmWgPerUnit * g.nb * g.bwp * 2 * g.bwp * 4);
   w.f_begin = off;
   w.f_rec_a = take(B * w.nC * g.W * 8);
-  w.f_rec_h = take(B * w.nC * g.W * 8);
   w.f_ticket = take(g.units * kMaxQueues * 4);
   w.f_end = off;
   w.b_begin = off;
   w.b_rec_a = take(B * w.nC * g.W * 8);
-  w.b_rec_h = take(B * w.nC * g.W * 8);
   w.b_ticket = take(g.units * kMaxQueues * 4);
   w.fail = take(4);
   w.b_end = off;
@@ -99,10 +97,10 @@ inline WorkLayout make_work_layout(int64_t B, int64_t T, const Geometry& g) {
 }
 
 // Scan-only workspace: chunks of 32 tokens; everything is cleared before each pass.
-//   rec_a, rec_h [B][nC][W] 64-bit carry records; ticket [B][groups]; fail.
+//   rec_a [B][nC][W] 64-bit carry records; ticket [B][groups]; fail.
 struct ScanLayout {
   int64_t nC, groups;
-  size_t rec_a, rec_h, ticket, fail, total;
+  size_t rec_a, ticket, fail, total;
 };
 
 inline ScanLayout make_scan_layout(int64_t B, int64_t T, int64_t W) {
@@ -112,7 +110,6 @@ inline ScanLayout make_scan_layout(int64_t B, int64_t T, int64_t W) {
   size_t off = 0;
   auto take = [&](int64_t bytes) { size_t at = off; off += (size_t)round_up(bytes, 256); return at; };
   s.rec_a = take(B * s.nC * W * 8);
-  s.rec_h = take(B * s.nC * W * 8);
   s.ticket = take(B * s.groups * 4);
   s.fail = take(4);
   s.total = off;

@@ -56,7 +56,7 @@ long long exchange_spin_limit(long long v) { return g_spin_limit.exchange(v); }
 struct ScanArgs {
   const float* a; const float* z; const float* h0; float* h;      // forward
   const float* dh; const float* h_saved; float* da; float* dz; float* dh0;   // backward
-  rec_t* rec_a; rec_t* rec_h; unsigned* ticket; unsigned* fail;
+  rec_t* rec_a; unsigned* ticket; unsigned* fail;
   int B, T, W, nC, groups;
   long long tiles, limit;
 };
@@ -93,16 +93,16 @@ __global__ __launch_bounds__(kThreads) void scan_fwd_kernel(ScanArgs p) {
 
   CarryChain chain;
   const long long seq = (long long)b * p.nC * W + (ok ? ch : 0);
-  chain.rec_a = p.rec_a + seq; chain.rec_h = p.rec_h + seq; chain.stride = W;
+  chain.rec = p.rec_a + seq; chain.stride = W;
 
   float h_in;
   if (c == 0) {
     h_in = ok ? p.h0[(long long)b * W + ch] : 0.f;
   } else {
-    if (ok) carry_publish(chain, c, A, H, kVerLocal);
+    if (ok) carry_publish(chain, c, A, H, false);
     h_in = carry_lookback(chain, c, -1, -1, 0.f, ok, p.limit, p.fail);
   }
-  if (ok) carry_publish(chain, c, 0.f, fmaf(A, h_in, H), kVerFinal);
+  if (ok) carry_publish(chain, c, 0.f, fmaf(A, h_in, H), true);
 
   float h = h_in;
 #pragma unroll
@@ -145,17 +145,17 @@ __global__ __launch_bounds__(kThreads) void scan_bwd_kernel(ScanArgs p) {
 
   CarryChain chain;
   const long long seq = (long long)b * p.nC * W + (ok ? ch : 0);
-  chain.rec_a = p.rec_a + seq; chain.rec_h = p.rec_h + seq; chain.stride = W;
+  chain.rec = p.rec_a + seq; chain.stride = W;
 
   float d_in;
   if (c == p.nC - 1) {
     d_in = 0.f;
   } else {
-    if (ok) carry_publish(chain, c, A, H, kVerLocal);
+    if (ok) carry_publish(chain, c, A, H, false);
     d_in = carry_lookback(chain, c, +1, p.nC, 0.f, ok, p.limit, p.fail);
   }
   const float d_out = fmaf(A, d_in, H);
-  if (ok) carry_publish(chain, c, 0.f, d_out, kVerFinal);
+  if (ok) carry_publish(chain, c, 0.f, d_out, true);
   if (c == 0 && ok) p.dh0[(long long)b * W + ch] = d_out;
 
   carry = d_in;
@@ -177,7 +177,7 @@ static int scan_common(ScanArgs& p, void* ws, int64_t B, int64_t T, int64_t W, h
   ScanLayout L = make_scan_layout(B, T, W);
   if (B * L.nC * L.groups >= (1ll << 31)) return fail(RGLRU_E_UNSUPPORTED, "scan: too many tiles");
   char* base = (char*)ws;
-  p.rec_a = (rec_t*)(base + L.rec_a); p.rec_h = (rec_t*)(base + L.rec_h);
+  p.rec_a = (rec_t*)(base + L.rec_a);
   p.ticket = (unsigned*)(base + L.ticket); p.fail = (unsigned*)(base + L.fail);
   p.B = (int)B; p.T = (int)T; p.W = (int)W; p.nC = (int)L.nC; p.groups = (int)L.groups;
   p.tiles = B * L.nC * L.groups;
