@@ -24,10 +24,12 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes per launch of the backward kernel at the benchmark workload, from rocprofv3 --pmc
-# FETCH_SIZE / WRITE_SIZE runs scaled by a copy kernel of known size (see profiles/).  None until
-# measured.
-MEASURED_TRAFFIC_BYTES = {"bwd_kernel": None, "fwd_kernel": None}
+# HBM bytes per launch at the benchmark workload (B8 T2048 W1024 nb8 bf16), from two rocprofv3 --pmc
+# runs of this script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same
+# counter reads for the 64 MiB copy that --traffic-probe adds (profiles/ holds the summaries).  Only
+# valid for that workload; other shapes report null.
+MEASURED_TRAFFIC_BYTES = {"bwd_scan_kernel": 410250953, "fwd_kernel": 86420691, "gate_grad_kernel": 201985655}
+BENCH_SHAPE = (8, 2048, 1024, 8)
 
 
 def parse_args():
@@ -37,6 +39,8 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph replay")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="also run a plain 64 MiB device copy a few times (known traffic, for scaling profiler counters)")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--seq", type=int, default=2048)
     ap.add_argument("--width", type=int, default=1024)
@@ -129,37 +133,51 @@ def main():
 
     # per-kernel durations, HIP events on the launch stream (library measurement hook), eager launches
     lib.rglru_hip_set_timing(1)
-    fwd_ms, bwd_ms = [], []
+    names = {"fwd_kernel": 0, "bwd_scan_kernel": 1, "gate_grad_kernel": 3}
+    samples = {k: [] for k in names}
     for _ in range(20):
         step()
-        fwd_ms.append(lib.rglru_hip_kernel_ms(0))
-        bwd_ms.append(lib.rglru_hip_kernel_ms(1))
+        for k, slot in names.items():
+            samples[k].append(lib.rglru_hip_kernel_ms(slot))
     lib.rglru_hip_set_timing(0)
-    if min(fwd_ms) <= 0 or min(bwd_ms) <= 0:
-        raise RuntimeError(f"kernel timing hook returned no measurement: fwd {fwd_ms[:3]} bwd {bwd_ms[:3]}")
-    fwd_avg = sum(fwd_ms) / len(fwd_ms)
-    bwd_avg = sum(bwd_ms) / len(bwd_ms)
+    for k, v in samples.items():
+        if min(v) <= 0:
+            raise RuntimeError(f"kernel timing hook returned no measurement for {k}: {v[:3]}")
+    avg_ms = {k: sum(v) / len(v) for k, v in samples.items()}
 
+    if args.traffic_probe:
+        src = torch.empty(64 * 1024 * 1024 // 4, device=dev).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+
+    # Algorithmic bytes: the compulsory streams at the storage size.  Forward reads x and writes y;
+    # the backward scan kernel reads x and dy and writes the input gradient; the gradient GEMM kernel
+    # adds no compulsory stream of its own (everything it moves is overhead of the two-kernel split).
     n = B * T * W
     elem = 2
-    bytes_fwd, bytes_bwd = 2 * elem * n, 3 * elem * n
-    dominant = "bwd_kernel" if bwd_avg >= fwd_avg else "fwd_kernel"
-    dom_bytes, dom_ms = (bytes_bwd, bwd_avg) if dominant == "bwd_kernel" else (bytes_fwd, fwd_avg)
+    algo = {"fwd_kernel": 2 * elem * n, "bwd_scan_kernel": 3 * elem * n, "gate_grad_kernel": 0}
+    dominant = max(avg_ms, key=avg_ms.get)
+    dom_bytes, dom_ms = algo[dominant], avg_ms[dominant]
     achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
+    traffic = MEASURED_TRAFFIC_BYTES[dominant] if (B, T, W, nb) == BENCH_SHAPE else None
+    step_gbps = 5 * elem * n / (ms_per_step * 1e-3) / 1e9
     out = {
         "metric": "RG-LRU fwd+bwd tokens/s", "value": B * T / (ms_per_step * 1e-3), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16 storage, f32 state",
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": f"RG-LRU fwd+bwd B{B} T{T} W{W} nb{nb} bf16", "batch": B, "seq_len": T,
-                   "width": W, "gate_blocks": nb, "launch": "hip graph replay" if graph is not None else "eager"},
+                   "width": W, "gate_blocks": nb, "state_dtype": "f32", "launch": "hip graph replay" if graph is not None else "eager"},
         "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": MEASURED_TRAFFIC_BYTES[dominant],
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
                      "algorithmic_bytes": dom_bytes, "kernel_ms": dom_ms},
-        "kernels": {"fwd_kernel_ms": fwd_avg, "bwd_kernel_ms": bwd_avg,
-                    "fwd_GBps": bytes_fwd / (fwd_avg * 1e-3) / 1e9, "bwd_GBps": bytes_bwd / (bwd_avg * 1e-3) / 1e9,
-                    "fwd_bwd_GBps_whole_step": 5 * elem * n / (ms_per_step * 1e-3) / 1e9,
-                    "fwd_bwd_frac_of_peak_whole_step": 5 * elem * n / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS},
+        "kernels": {**{f"{k}_ms": v for k, v in avg_ms.items()},
+                    "fwd_GBps": algo["fwd_kernel"] / (avg_ms["fwd_kernel"] * 1e-3) / 1e9,
+                    "bwd_GBps": algo["bwd_scan_kernel"] / ((avg_ms["bwd_scan_kernel"] + avg_ms["gate_grad_kernel"]) * 1e-3) / 1e9,
+                    "fwd_bwd_GBps_whole_step": step_gbps,
+                    "fwd_bwd_frac_of_peak_whole_step": step_gbps / HBM_PEAK_GBS},
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(case)

@@ -842,7 +842,9 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
     if (!last_chunk && hf == 0) carry_publish(chain, c, A_t, D_t, false);
     issue(tk_next);
     float d_in = (last_chunk && p.dh_last) ? p.dh_last[(long long)b * W + w.ch] : 0.f;
+#ifndef RGLRU_EXP_BWD_NOLOOKBACK
     if (!last_chunk) d_in = carry_lookback(chain, c, +1, p.nC, 0.f, true, p.limit, p.fail);
+#endif
     const float d_out = fmaf(A_t, d_in, D_t);
     if (hf == 0) carry_publish(chain, c, 0.f, d_out, true);
     if (hf == 0 && c == 0 && p.dh0) p.dh0[(long long)b * W + w.ch] = d_out;
