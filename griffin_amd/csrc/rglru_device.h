@@ -173,11 +173,7 @@ RGLRU_DEVICE void rec_store(rec_t* p, float a, float h) {
 }
 // cache policy of a record access issued through a buffer descriptor: device scope (sc1)
 constexpr int kRecPolicy = 16;
-#ifdef RGLRU_EXP_SC0
-constexpr int kRecPrefetchPolicy = RGLRU_EXP_SC0;
-#else
-constexpr int kRecPrefetchPolicy = 16;
-#endif
+
 RGLRU_DEVICE rec_t rec_load(const rec_t* p) {
   return __hip_atomic_load(const_cast<rec_t*>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -286,7 +282,7 @@ RGLRU_DEVICE void carry_prefetch(rsrc_t recs, unsigned lane_off, unsigned stride
     const int q = c + step + d * step;
     const bool inside = (step < 0) ? (q > end) : (q < end);
     const unsigned voff = (inside && lane_off != kOutOfRange) ? (unsigned)q * stride_bytes + lane_off : kOutOfRange;
-    const u32x2 v = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(recs, voff, 0, kRecPrefetchPolicy));
+    const u32x2 v = __builtin_bit_cast(u32x2, __builtin_amdgcn_raw_buffer_load_b64(recs, voff, 0, kRecPolicy));
     batch.rec[d] = ((rec_t)v[1] << 32) | (rec_t)v[0];
   }
 }

@@ -27,11 +27,19 @@ namespace rglru {
 // Parameter preparation
 // ------------------------------------------------------------------------------------------
 struct PrepArgs {
-  const void* w_a; const void* w_x; const float* b_a; const float* b_x; const float* lambda;
-  void* wg; float* bias; float* sp; float* cs; void* w2t;
-  int W, nb, bw, bwp, Wp;
+  const void* w_a; const void* w_x; const void* b_a; const void* b_x; const void* lambda;
+  void* wg; float* bias; float* sp; float* cs; float* dsp; void* w2t;
+  int W, nb, bw, bwp, Wp, vec_dtype;
   float c;
 };
+
+// Element i of a vector stored as fp32 or bf16 (RGLRU_F32 / RGLRU_BF16).
+RGLRU_DEVICE float load_vec(const void* p, long long i, int dtype) {
+  return dtype == RGLRU_BF16 ? (float)((const __bf16*)p)[i] : ((const float*)p)[i];
+}
+RGLRU_DEVICE void store_vec(void* p, long long i, float v, int dtype) {
+  if (dtype == RGLRU_BF16) ((__bf16*)p)[i] = (__bf16)v; else ((float*)p)[i] = v;
+}
 
 RGLRU_DEVICE float log_sigmoid(float v) {
   return v >= 0.f ? -log1pf(expf(-v)) : v - log1pf(expf(v));
@@ -74,15 +82,17 @@ __global__ void prepare_kernel(PrepArgs p) {
     } else {
       int kp = (int)(i - n_w);
       int k = kp / p.bwp, o = kp - k * p.bwp;
-      float ba = 0.f, bx = 0.f, sp = 0.f, cs = 0.f;
+      float ba = 0.f, bx = 0.f, sp = 0.f, cs = 0.f, dsp = 0.f;
       if (o < p.bw) {
         int ch = k * p.bw + o;
-        ba = p.b_a[ch]; bx = p.b_x[ch];
-        float ls = log_sigmoid(p.lambda[ch]);
+        ba = load_vec(p.b_a, ch, p.vec_dtype); bx = load_vec(p.b_x, ch, p.vec_dtype);
+        const float lam = load_vec(p.lambda, ch, p.vec_dtype);
+        float ls = log_sigmoid(lam);
         cs = p.c * ls;
         sp = cs * kLog2e;
+        dsp = p.c / (1.0f + expf(lam));          // c * d/dLambda log sigmoid(Lambda) = c * sigmoid(-Lambda)
       }
-      p.bias[kp] = ba; p.bias[p.Wp + kp] = bx; p.sp[kp] = sp; p.cs[kp] = cs;
+      p.bias[kp] = ba; p.bias[p.Wp + kp] = bx; p.sp[kp] = sp; p.cs[kp] = cs; p.dsp[kp] = dsp;
     }
   }
 }
@@ -1083,46 +1093,46 @@ __global__ __launch_bounds__(kThreads, 1) void gate_grad_kernel(FusedArgs p) {
   }
 }
 
-struct DwReduceArgs {
-  const float* dw_partial; float* dw_a; float* dw_x; int nb, bw, bwp, n_wg;
+// Last launch of a backward pass: sums the per-workgroup partial results and writes the parameter
+// gradients in the caller's type.  Workgroups [0, vec_blocks) own 64 channels each of db_a, db_x and
+// dLambda; the rest (fast backward only) own 256 elements each of the two weight gradients,
+// dW_gate[k][o][j] = sum over workgroups of dW2T[wg][k][j][2 o + gate].
+struct FinishArgs {
+  const float* partial; const float* dsp; void* db_a; void* db_x; void* dlambda;
+  const float* dw_partial; void* dw_a; void* dw_x;
+  int W, nb, bw, bwp, Wp, wg_per_unit, n_wg, vec_blocks, grad_dtype;
 };
 
-// dW_gate[k][o][j] = sum over workgroups of dW2T[wg][k][j][2 o + gate]
-__global__ void dw_reduce_kernel(DwReduceArgs p) {
-  const long long total = (long long)p.nb * p.bw * 2 * p.bw;
-  long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x;
-  if (i >= total) return;
-  const int kap = (int)(i % (2 * p.bw));
-  const int j = (int)((i / (2 * p.bw)) % p.bw);
-  const int k = (int)(i / ((long long)2 * p.bw * p.bw));
-  const long long stride = (long long)p.nb * p.bwp * 2 * p.bwp;
-  const float* src = p.dw_partial + ((long long)k * p.bwp + j) * (2 * p.bwp) + kap;
-  float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
-  int g = 0;
-  for (; g + 3 < p.n_wg; g += 4) {
-    s0 += src[(long long)g * stride]; s1 += src[(long long)(g + 1) * stride];
-    s2 += src[(long long)(g + 2) * stride]; s3 += src[(long long)(g + 3) * stride];
-  }
-  for (; g < p.n_wg; ++g) s0 += src[(long long)g * stride];
-  const float sum = (s0 + s1) + (s2 + s3);
-  float* dst = (kap & 1) ? p.dw_x : p.dw_a;
-  dst[((long long)k * p.bw + (kap >> 1)) * p.bw + j] = sum;
-}
-
-struct ReduceArgs {
-  const float* partial; const float* lambda; float* db_a; float* db_x; float* dlambda;
-  int W, bw, bwp, Wp, wg_per_unit; float c;
-};
-
-__global__ __launch_bounds__(256) void reduce_kernel(ReduceArgs p) {
-  // 64 channels per workgroup; four quarter-sums per channel are combined through LDS
+__global__ __launch_bounds__(256) void finish_kernel(FinishArgs p) {
   __shared__ float part_sum[3][4][64];
+  if ((int)blockIdx.x >= p.vec_blocks) {
+    const long long total = (long long)p.nb * p.bw * 2 * p.bw;
+    const long long i = (long long)(blockIdx.x - p.vec_blocks) * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int kap = (int)(i % (2 * p.bw));
+    const int j = (int)((i / (2 * p.bw)) % p.bw);
+    const int k = (int)(i / ((long long)2 * p.bw * p.bw));
+    const long long stride = (long long)p.nb * p.bwp * 2 * p.bwp;
+    const float* src = p.dw_partial + ((long long)k * p.bwp + j) * (2 * p.bwp) + kap;
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    int g = 0;
+    for (; g + 3 < p.n_wg; g += 4) {
+      s0 += src[(long long)g * stride]; s1 += src[(long long)(g + 1) * stride];
+      s2 += src[(long long)(g + 2) * stride]; s3 += src[(long long)(g + 3) * stride];
+    }
+    for (; g < p.n_wg; ++g) s0 += src[(long long)g * stride];
+    const float sum = (s0 + s1) + (s2 + s3);
+    store_vec((kap & 1) ? p.dw_x : p.dw_a, ((long long)k * p.bw + (kap >> 1)) * p.bw + j, sum, p.grad_dtype);
+    return;
+  }
+  // 64 channels per workgroup; four quarter-sums per channel are combined through LDS
   const int lane = threadIdx.x & 63, quarter = threadIdx.x >> 6;
   const int ch = blockIdx.x * 64 + lane;
   float sa = 0.f, sx = 0.f, sl = 0.f;
+  int kp = 0;
   if (ch < p.W) {
     const int k = ch / p.bw, o = ch - k * p.bw;
-    const int kp = k * p.bwp + o;
+    kp = k * p.bwp + o;
     for (int g = quarter; g < p.wg_per_unit; g += 4) {
       const float* part = p.partial + (long long)g * 3 * p.Wp + kp;
       sa += part[0]; sx += part[p.Wp]; sl += part[2 * p.Wp];
@@ -1134,10 +1144,9 @@ __global__ __launch_bounds__(256) void reduce_kernel(ReduceArgs p) {
     sa = (part_sum[0][0][lane] + part_sum[0][1][lane]) + (part_sum[0][2][lane] + part_sum[0][3][lane]);
     sx = (part_sum[1][0][lane] + part_sum[1][1][lane]) + (part_sum[1][2][lane] + part_sum[1][3][lane]);
     sl = (part_sum[2][0][lane] + part_sum[2][1][lane]) + (part_sum[2][2][lane] + part_sum[2][3][lane]);
-    p.db_a[ch] = sa; p.db_x[ch] = sx;
-    const float lam = p.lambda[ch];
-    const float sig_neg = 1.0f / (1.0f + expf(lam));   // d/dLambda log sigmoid(Lambda) = sigmoid(-Lambda)
-    p.dlambda[ch] = p.c * sl * sig_neg;
+    store_vec(p.db_a, ch, sa, p.grad_dtype);
+    store_vec(p.db_x, ch, sx, p.grad_dtype);
+    store_vec(p.dlambda, ch, sl * p.dsp[kp], p.grad_dtype);
   }
 }
 
@@ -1217,6 +1226,10 @@ static void fill_common(FusedArgs& a, const Geometry& g, const void* prep, int d
   a.groups = (int)g.groups; a.units = (int)g.units;
   a.limit = spin_limit();
   a.full_slabs = (g.bw % 32 == 0) ? 1 : 0;
+}
+
+static const float* finish_dsp(const Geometry& g, const void* prep, int dtype) {
+  return (const float*)((const char*)prep + make_prep_layout(g, elem_size(dtype)).dsp);
 }
 
 static int is_aligned(const void* ptr, int64_t W, int64_t bw, size_t es) {
@@ -1309,11 +1322,12 @@ size_t rglru_hip_prep_bytes(int64_t W, int64_t nb, int dtype) {
   return make_prep_layout(make_geometry(W, nb), elem_size(dtype)).total;
 }
 
-int rglru_hip_prepare(const void* w_a, const float* b_a, const void* w_x, const float* b_x,
-                      const float* lambda, float c, int64_t W, int64_t nb, int dtype,
+int rglru_hip_prepare(const void* w_a, const void* b_a, const void* w_x, const void* b_x,
+                      const void* lambda, float c, int64_t W, int64_t nb, int dtype, int vec_dtype,
                       void* prep, void* stream) {
   int rc = check_geometry("prepare", W, nb, dtype);
   if (rc) return rc;
+  if (vec_dtype != RGLRU_F32 && vec_dtype != RGLRU_BF16) return fail(RGLRU_E_ARG, "prepare: unknown vector dtype %d", vec_dtype);
   if (!w_a || !b_a || !w_x || !b_x || !lambda || !prep) return fail(RGLRU_E_ARG, "prepare: null pointer");
   Geometry g = make_geometry(W, nb);
   PrepLayout pl = make_prep_layout(g, elem_size(dtype));
@@ -1321,6 +1335,7 @@ int rglru_hip_prepare(const void* w_a, const float* b_a, const void* w_x, const 
   PrepArgs a;
   a.w_a = w_a; a.w_x = w_x; a.b_a = b_a; a.b_x = b_x; a.lambda = lambda;
   a.wg = pb + pl.wg; a.bias = (float*)(pb + pl.bias); a.sp = (float*)(pb + pl.sp); a.cs = (float*)(pb + pl.cs);
+  a.dsp = (float*)(pb + pl.dsp); a.vec_dtype = vec_dtype;
   a.w2t = pb + pl.w2t;
   a.W = (int)W; a.nb = (int)nb; a.bw = (int)g.bw; a.bwp = (int)g.bwp; a.Wp = (int)g.Wp; a.c = c;
   long long total = 4 * g.nb * g.bwp * g.bwp + g.Wp;
@@ -1348,9 +1363,7 @@ int rglru_hip_fwd(const void* x, const void* prep, const float* h0, const uint8_
   WorkLayout L = make_work_layout(B, T, g);
   hipStream_t s = (hipStream_t)stream;
   char* wb = (char*)ws;
-  rc = launch_clear(wb, L.f_begin, L.f_end, s);
-  if (rc) return rc;
-  rc = launch_clear(wb, L.fail, L.fail + 256, s);
+  rc = launch_clear(wb, L.f_begin, L.f_end, s);         // forward carry records, tickets, failure word
   if (rc) return rc;
   FusedArgs a;
   memset(&a, 0, sizeof(a));
@@ -1375,15 +1388,22 @@ int rglru_hip_fwd(const void* x, const void* prep, const float* h0, const uint8_
   return check_launch("fwd");
 }
 
-int rglru_hip_bwd(const void* x, const void* prep, const float* lambda, const float* h0,
+static int check_grad_dtype(const char* who, int grad_dtype) {
+  if (grad_dtype != RGLRU_F32 && grad_dtype != RGLRU_BF16) return fail(RGLRU_E_ARG, "%s: unknown gradient dtype %d", who, grad_dtype);
+  return RGLRU_OK;
+}
+
+int rglru_hip_bwd(const void* x, const void* prep, const float* h0,
                   const uint8_t* flags, const void* dy, const float* dh_last, void* ws,
-                  void* dx, void* du_a, void* du_x, float* db_a, float* db_x, float* dlambda,
-                  float* dh0, int64_t B, int64_t T, int64_t W, int64_t nb, float c, int dtype,
+                  void* dx, void* du_a, void* du_x, void* db_a, void* db_x, void* dlambda,
+                  float* dh0, int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, int grad_dtype,
                   void* stream) {
   int rc = check_geometry("bwd", W, nb, dtype);
   if (rc) return rc;
+  rc = check_grad_dtype("bwd", grad_dtype);
+  if (rc) return rc;
   if (B <= 0 || T <= 0) return fail(RGLRU_E_ARG, "bwd: B and T must be positive (got %lld, %lld)", (long long)B, (long long)T);
-  if (!x || !prep || !lambda || !dy || !ws || !dx || !du_a || !du_x || !db_a || !db_x || !dlambda)
+  if (!x || !prep || !dy || !ws || !dx || !du_a || !du_x || !db_a || !db_x || !dlambda)
     return fail(RGLRU_E_ARG, "bwd: null pointer");
   if (B * T * W >= (1ll << 40) || B * T >= (1ll << 31)) return fail(RGLRU_E_UNSUPPORTED, "bwd: tensor too large");
   Geometry g = make_geometry(W, nb);
@@ -1411,11 +1431,13 @@ int rglru_hip_bwd(const void* x, const void* prep, const float* lambda, const fl
   }
   rc = check_launch("bwd");
   if (rc) return rc;
-  ReduceArgs r;
-  r.partial = a.partial; r.lambda = lambda; r.db_a = db_a; r.db_x = db_x; r.dlambda = dlambda;
-  r.W = (int)W; r.bw = (int)g.bw; r.bwp = (int)g.bwp; r.Wp = (int)g.Wp; r.wg_per_unit = a.wg_per_unit; r.c = c;
-  hipLaunchKernelGGL(reduce_kernel, dim3((unsigned)((W + 63) / 64)), dim3(256), 0, s, r);
-  return check_launch("bwd reduce");
+  FinishArgs r;
+  memset(&r, 0, sizeof(r));
+  r.partial = a.partial; r.dsp = finish_dsp(g, prep, dtype); r.db_a = db_a; r.db_x = db_x; r.dlambda = dlambda;
+  r.W = (int)W; r.nb = (int)nb; r.bw = (int)g.bw; r.bwp = (int)g.bwp; r.Wp = (int)g.Wp; r.wg_per_unit = a.wg_per_unit;
+  r.vec_blocks = (int)((W + 63) / 64); r.grad_dtype = grad_dtype;
+  hipLaunchKernelGGL(finish_kernel, dim3((unsigned)r.vec_blocks), dim3(256), 0, s, r);
+  return check_launch("bwd finish");
 }
 
 int rglru_hip_fast_path(int64_t W, int64_t nb, int dtype) {
@@ -1424,17 +1446,19 @@ int rglru_hip_fast_path(int64_t W, int64_t nb, int dtype) {
   return (bw == 32 || bw == 64 || bw == 128) ? 1 : 0;
 }
 
-int rglru_hip_bwd_full(const void* x, const void* prep, const float* lambda, const float* h0,
+int rglru_hip_bwd_full(const void* x, const void* prep, const float* h0,
                        const uint8_t* flags, const void* dy, const float* dh_last, void* ws,
-                       void* dx, float* dw_a, float* dw_x, float* db_a, float* db_x, float* dlambda,
-                       float* dh0, int64_t B, int64_t T, int64_t W, int64_t nb, float c, int dtype,
+                       void* dx, void* dw_a, void* dw_x, void* db_a, void* db_x, void* dlambda,
+                       float* dh0, int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, int grad_dtype,
                        void* stream) {
   int rc = check_geometry("bwd_full", W, nb, dtype);
+  if (rc) return rc;
+  rc = check_grad_dtype("bwd_full", grad_dtype);
   if (rc) return rc;
   if (!rglru_hip_fast_path(W, nb, dtype))
     return fail(RGLRU_E_UNSUPPORTED, "bwd_full: needs 16-bit storage and gate blocks of 32, 64 or 128 channels");
   if (B <= 0 || T <= 0) return fail(RGLRU_E_ARG, "bwd_full: B and T must be positive (got %lld, %lld)", (long long)B, (long long)T);
-  if (!x || !prep || !lambda || !dy || !ws || !dx || !dw_a || !dw_x || !db_a || !db_x || !dlambda)
+  if (!x || !prep || !dy || !ws || !dx || !dw_a || !dw_x || !db_a || !db_x || !dlambda)
     return fail(RGLRU_E_ARG, "bwd_full: null pointer");
   if (B * T * W >= (1ll << 40) || B * T >= (1ll << 31)) return fail(RGLRU_E_UNSUPPORTED, "bwd_full: tensor too large");
   Geometry g = make_geometry(W, nb);
@@ -1482,17 +1506,15 @@ int rglru_hip_bwd_full(const void* x, const void* prep, const float* lambda, con
 #endif
   rc = check_launch("bwd_full gemm");
   if (rc) return rc;
-  ReduceArgs r;
-  r.partial = a.partial; r.lambda = lambda; r.db_a = db_a; r.db_x = db_x; r.dlambda = dlambda;
-  r.W = (int)W; r.bw = (int)g.bw; r.bwp = (int)g.bwp; r.Wp = (int)g.Wp; r.wg_per_unit = a.wg_per_unit; r.c = c;
-  hipLaunchKernelGGL(reduce_kernel, dim3((unsigned)((W + 63) / 64)), dim3(256), 0, s, r);
-  rc = check_launch("bwd_full reduce");
-  if (rc) return rc;
-  DwReduceArgs d;
-  d.dw_partial = a.dw_partial; d.dw_a = dw_a; d.dw_x = dw_x; d.nb = (int)nb; d.bw = (int)g.bw; d.bwp = (int)g.bwp; d.n_wg = n_wg;
+  FinishArgs r;
+  memset(&r, 0, sizeof(r));
+  r.partial = a.partial; r.dsp = finish_dsp(g, prep, dtype); r.db_a = db_a; r.db_x = db_x; r.dlambda = dlambda;
+  r.dw_partial = a.dw_partial; r.dw_a = dw_a; r.dw_x = dw_x;
+  r.W = (int)W; r.nb = (int)nb; r.bw = (int)g.bw; r.bwp = (int)g.bwp; r.Wp = (int)g.Wp; r.wg_per_unit = a.wg_per_unit;
+  r.n_wg = n_wg; r.vec_blocks = (int)((W + 63) / 64); r.grad_dtype = grad_dtype;
   const long long total = nb * g.bw * 2 * g.bw;
-  hipLaunchKernelGGL(dw_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, d);
-  return check_launch("bwd_full weight reduce");
+  hipLaunchKernelGGL(finish_kernel, dim3((unsigned)(r.vec_blocks + (total + 255) / 256)), dim3(256), 0, s, r);
+  return check_launch("bwd_full finish");
 }
 
 int rglru_hip_step(const void* x, const void* prep, float* h, const uint8_t* flags, void* y,

@@ -31,10 +31,11 @@ inline Geometry make_geometry(int64_t W, int64_t nb) {
 //   bias  [2][Wp]            fp32
 //   sp    [Wp]               fp32   c * log2(sigmoid(Lambda))
 //   cs    [Wp]               fp32   c * log(sigmoid(Lambda))
+//   dsp   [Wp]               fp32   c * sigmoid(-Lambda), the factor of the Lambda gradient
 //   w2t   [nb][bwp][2*bwp]   storage type: w2t[k][j][2*o + gate] = W_gate[k][o][j], the operand
 //                            of the input-gradient GEMM dx += du W
 struct PrepLayout {
-  size_t wg, bias, sp, cs, w2t, total;
+  size_t wg, bias, sp, cs, dsp, w2t, total;
 };
 
 inline PrepLayout make_prep_layout(const Geometry& g, size_t elem) {
@@ -44,6 +45,7 @@ inline PrepLayout make_prep_layout(const Geometry& g, size_t elem) {
   p.bias = off; off += (size_t)round_up(2 * g.Wp * 4, 256);
   p.sp = off;   off += (size_t)round_up(g.Wp * 4, 256);
   p.cs = off;   off += (size_t)round_up(g.Wp * 4, 256);
+  p.dsp = off;  off += (size_t)round_up(g.Wp * 4, 256);
   p.w2t = off;  off += (size_t)round_up(2 * g.nb * g.bwp * g.bwp * (int64_t)elem, 256);
   p.total = off;
   return p;
@@ -55,13 +57,13 @@ inline PrepLayout make_prep_layout(const Geometry& g, size_t elem) {
 //   partial     [maxWg][3][Wp]  per-workgroup sums for db_a, db_x, dLambda
 //   du2         [B][T][2W]      16-bit: gate pre-activation gradients (fast backward only)
 //   dw_partial  [kGemmWgPerUnit][nb][bwp][2*bwp] fp32 per-workgroup weight-gradient sums
-//   --- cleared before the forward pass ---
+//   --- [f_begin, f_end) is cleared before the forward pass ---
 //   f_rec_a     [B][<=nC][W]    64-bit carry records of the forward chain
 //   f_ticket    [units][kMaxQueues]
-//   --- cleared before the backward pass ---
+//   fail        [1]             failure word; part of both regions, so either pass clears it
+//   --- [b_begin, b_end) is cleared before the backward pass ---
 //   b_rec_a     [B][nC][W]      64-bit carry records of the backward chain
 //   b_ticket    [units][kMaxQueues]
-//   fail        [1]             (cleared by both)
 constexpr int kMaxQueues = 64;          // ticket queues per unit (sequences are dealt round-robin to them)
 constexpr int kGemmWgPerUnit = 32;      // workgroups per gate block in the gradient GEMM kernel
 
@@ -86,11 +88,11 @@ inline WorkLayout make_work_layout(int64_t B, int64_t T, const Geometry& g) {
   w.f_begin = off;
   w.f_rec_a = take(B * w.nC * g.W * 8);
   w.f_ticket = take(g.units * kMaxQueues * 4);
+  w.b_begin = off;                     // the failure word belongs to both regions
+  w.fail = take(4);
   w.f_end = off;
-  w.b_begin = off;
   w.b_rec_a = take(B * w.nC * g.W * 8);
   w.b_ticket = take(g.units * kMaxQueues * 4);
-  w.fail = take(4);
   w.b_end = off;
   w.total = off;
   return w;

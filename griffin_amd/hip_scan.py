@@ -108,6 +108,9 @@ def hip_rglru_scan(decay: Tensor, current_input: Tensor, initial_state: Tensor) 
 # ----------------------------------------------------------------------------------------------
 # fused operator: gates + scan
 # ----------------------------------------------------------------------------------------------
+_DTYPE_CODES = {torch.float32: _lib.RGLRU_F32, torch.bfloat16: _lib.RGLRU_BF16}
+
+
 def _dtype_code(dtype: torch.dtype) -> int:
     if dtype == torch.float32:
         return _lib.RGLRU_F32
@@ -142,15 +145,18 @@ class PreparedParams:
         if size == 0:
             _lib.check(2, "rglru_hip_prep_bytes")
         device = w_a.device
-        self.lam32 = lam.detach().to(torch.float32).contiguous()
+        # gate weights in the storage type; biases and Lambda are read in their own type when the
+        # library knows it (fp32 or bf16), so the usual cases launch no conversion kernels
         w_a_c = w_a.detach().to(dtype).contiguous()
         w_x_c = w_x.detach().to(dtype).contiguous()
-        b_a_c = b_a.detach().to(torch.float32).contiguous()
-        b_x_c = b_x.detach().to(torch.float32).contiguous()
+        vec_dtype = b_a.dtype if (b_a.dtype == b_x.dtype == lam.dtype and b_a.dtype in _DTYPE_CODES) else torch.float32
+        b_a_c = b_a.detach().to(vec_dtype).contiguous()
+        b_x_c = b_x.detach().to(vec_dtype).contiguous()
+        lam_c = lam.detach().to(vec_dtype).contiguous()
         with torch.cuda.device(device):
             self.image = torch.empty(size, dtype=torch.uint8, device=device)
             _lib.check(lib.rglru_hip_prepare(w_a_c.data_ptr(), b_a_c.data_ptr(), w_x_c.data_ptr(), b_x_c.data_ptr(),
-                                             self.lam32.data_ptr(), self.c, self.width, nb, code,
+                                             lam_c.data_ptr(), self.c, self.width, nb, code, _DTYPE_CODES[vec_dtype],
                                              self.image.data_ptr(), _stream_ptr(device)), "rglru_hip_prepare")
 
 
@@ -192,16 +198,16 @@ class _HipRGLRU(torch.autograd.Function):
             _lib.check(lib.rglru_hip_fwd(x.data_ptr(), prep.image.data_ptr(), _ptr(h0c), _ptr(flags), y.data_ptr(),
                                          h_last.data_ptr(), ws.data_ptr(), B, T, W, nb, code, _stream_ptr(device)),
                        "rglru_hip_fwd")
-        ctx.save_for_backward(x, w_a, w_x, h0c, flags, ws, prep.image, prep.lam32)
-        ctx.c = float(c)
+        ctx.save_for_backward(x, w_a, w_x, h0c, flags, ws, prep.image)
         ctx.param_dtypes = (w_a.dtype, b_a.dtype, w_x.dtype, b_x.dtype, lam.dtype)
         ctx.h0_dtype = None if h0 is None else h0.dtype
+        ctx.set_materialize_grads(False)      # an unused output arrives as None, not as a tensor of zeros
         return y, h_last
 
     @staticmethod
     @once_differentiable
     def backward(ctx, dy, dh_last):
-        x, w_a, w_x, h0c, flags, ws, image, lam32 = ctx.saved_tensors
+        x, w_a, w_x, h0c, flags, ws, image = ctx.saved_tensors
         lib = _lib.load()
         B, T, W = x.shape
         nb, bw, _ = w_a.shape
@@ -209,28 +215,33 @@ class _HipRGLRU(torch.autograd.Function):
         device = x.device
         dy = torch.zeros_like(x) if dy is None else dy.to(x.dtype).contiguous()
         dhl = None if dh_last is None else dh_last.to(torch.float32).contiguous()
+        # parameter gradients come back in the parameters' own type when all five share one the
+        # library writes (fp32 or bf16); otherwise in fp32, converted below
+        pd = ctx.param_dtypes
+        gdt = pd[0] if (len(set(pd)) == 1 and pd[0] in _DTYPE_CODES) else torch.float32
+        gcode = _DTYPE_CODES[gdt]
         with torch.cuda.device(device):
             dx = torch.empty_like(x)
-            db_a = torch.empty(W, dtype=torch.float32, device=device)
-            db_x = torch.empty(W, dtype=torch.float32, device=device)
-            dlam = torch.empty(W, dtype=torch.float32, device=device)
+            db_a = torch.empty(nb, bw, dtype=gdt, device=device)
+            db_x = torch.empty(nb, bw, dtype=gdt, device=device)
+            dlam = torch.empty(W, dtype=gdt, device=device)
             dh0 = torch.empty(B, W, dtype=torch.float32, device=device) if ctx.needs_input_grad[6] else None
             if lib.rglru_hip_fast_path(W, nb, code) and dy.data_ptr() % 16 == 0 and x.data_ptr() % 16 == 0:
                 # everything in hand-written kernels, including the two gate GEMMs
-                dw_a = torch.empty(nb, bw, bw, dtype=torch.float32, device=device)
-                dw_x = torch.empty(nb, bw, bw, dtype=torch.float32, device=device)
-                _lib.check(lib.rglru_hip_bwd_full(x.data_ptr(), image.data_ptr(), lam32.data_ptr(), _ptr(h0c), _ptr(flags),
+                dw_a = torch.empty(nb, bw, bw, dtype=gdt, device=device)
+                dw_x = torch.empty(nb, bw, bw, dtype=gdt, device=device)
+                _lib.check(lib.rglru_hip_bwd_full(x.data_ptr(), image.data_ptr(), _ptr(h0c), _ptr(flags),
                                                   dy.data_ptr(), _ptr(dhl), ws.data_ptr(), dx.data_ptr(), dw_a.data_ptr(),
                                                   dw_x.data_ptr(), db_a.data_ptr(), db_x.data_ptr(), dlam.data_ptr(),
-                                                  _ptr(dh0), B, T, W, nb, ctx.c, code, _stream_ptr(device)),
+                                                  _ptr(dh0), B, T, W, nb, code, gcode, _stream_ptr(device)),
                            "rglru_hip_bwd_full")
             else:
                 du_a = torch.empty_like(x)
                 du_x = torch.empty_like(x)
-                _lib.check(lib.rglru_hip_bwd(x.data_ptr(), image.data_ptr(), lam32.data_ptr(), _ptr(h0c), _ptr(flags),
+                _lib.check(lib.rglru_hip_bwd(x.data_ptr(), image.data_ptr(), _ptr(h0c), _ptr(flags),
                                              dy.data_ptr(), _ptr(dhl), ws.data_ptr(), dx.data_ptr(), du_a.data_ptr(),
                                              du_x.data_ptr(), db_a.data_ptr(), db_x.data_ptr(), dlam.data_ptr(),
-                                             _ptr(dh0), B, T, W, nb, ctx.c, code, _stream_ptr(device)), "rglru_hip_bwd")
+                                             _ptr(dh0), B, T, W, nb, code, gcode, _stream_ptr(device)), "rglru_hip_bwd")
                 # block-diagonal library GEMMs: dW[k] = du[:, k]^T x[:, k];  dx[:, k] += du[:, k] W[k]
                 n = B * T
                 xk = x.view(n, nb, bw).transpose(0, 1)               # [nb, n, bw] (strided view)
@@ -243,8 +254,7 @@ class _HipRGLRU(torch.autograd.Function):
                 dxg = torch.bmm(ua, wa)
                 dxg = torch.baddbmm(dxg, ux, wx)
                 dx = (dx.view(n, nb, bw).float() + dxg.transpose(0, 1).float()).to(x.dtype).view(B, T, W)
-        pd = ctx.param_dtypes
-        grads = (dx, dw_a.to(pd[0]), db_a.view(nb, bw).to(pd[1]), dw_x.to(pd[2]), db_x.view(nb, bw).to(pd[3]),
+        grads = (dx, dw_a.to(pd[0]), db_a.to(pd[1]), dw_x.to(pd[2]), db_x.to(pd[3]),
                  dlam.to(pd[4]), None if dh0 is None else dh0.to(ctx.h0_dtype), None, None)
         return grads
 

@@ -21,7 +21,10 @@
  *   - the library keeps no per-call state: forward and backward may be issued from different
  *     host threads (PyTorch runs backward on its autograd thread);
  *   - `dtype` selects the storage type of x / y / dy / dx and of the gate weights:
- *     RGLRU_F32 or RGLRU_BF16.  State, biases, Lambda and every parameter gradient are fp32.
+ *     RGLRU_F32 or RGLRU_BF16.  The state is always fp32.  Biases and Lambda are read in
+ *     `vec_dtype` and the parameter gradients written in `grad_dtype` (each RGLRU_F32 or
+ *     RGLRU_BF16), so a caller never has to convert its parameters or their gradients; the
+ *     arithmetic and the accumulation are fp32 either way.
  *   - `flags` is one byte per token, [B, T]: bit 0 = reset (griffin/griffin.py:248-249: a <- 0,
  *     g <- 1), bit 1 = inactive / padding (griffin/griffin.py:252-255: a <- 1, z <- 0).
  *     NULL means no reset and all tokens active.
@@ -36,7 +39,7 @@
 extern "C" {
 #endif
 
-#define RGLRU_ABI_VERSION 1
+#define RGLRU_ABI_VERSION 2
 
 enum { RGLRU_F32 = 0, RGLRU_BF16 = 1 };
 
@@ -74,12 +77,13 @@ int rglru_hip_scan_bwd(const float* a, const float* h0, const float* h, const fl
 
 /* ---- fused RG-LRU ---------------------------------------------------------------------------
  * Parameters follow griffin/griffin.py:138-141, 174-176: w_a, w_x are [nb, bw, bw] (out, in) in
- * `param_dtype`; b_a, b_x are [nb, bw] and lambda is [W], fp32.  rglru_hip_prepare converts them
- * once into the padded, kernel-friendly image `prep` (rglru_hip_prep_bytes bytes) that fwd, bwd
- * and step consume; it must be re-run after the parameters change. */
+ * `dtype`; b_a, b_x are [nb, bw] and lambda is [W], in `vec_dtype`.  rglru_hip_prepare converts
+ * them once into the padded, kernel-friendly image `prep` (rglru_hip_prep_bytes bytes) that fwd,
+ * bwd and step consume (it also holds c * log sigmoid(Lambda) and c * sigmoid(-Lambda), so the
+ * other entry points take neither c nor Lambda); it must be re-run after the parameters change. */
 size_t rglru_hip_prep_bytes(int64_t W, int64_t nb, int dtype);
-int rglru_hip_prepare(const void* w_a, const float* b_a, const void* w_x, const float* b_x,
-                      const float* lambda, float c, int64_t W, int64_t nb, int dtype,
+int rglru_hip_prepare(const void* w_a, const void* b_a, const void* w_x, const void* b_x,
+                      const void* lambda, float c, int64_t W, int64_t nb, int dtype, int vec_dtype,
                       void* prep, void* stream);
 
 /* Workspace shared by one forward call and its backward call.  Forward fills it (chunk
@@ -96,24 +100,24 @@ int rglru_hip_fwd(const void* x, const void* prep, const float* h0, const uint8_
  * checkpoints in `ws` is kept from forward).  dy[B,T,W] (dtype); dh_last[B,W] fp32 or NULL.
  * Outputs: dx[B,T,W] (dtype) receives only the direct path dL/dz * g * i; du_a, du_x [B,T,W]
  * (dtype) receive the gradients at the two gate pre-activations, from which the caller forms
- * dW = du^T x, and dx += du W with two library GEMMs; db_a, db_x [nb*bw], dlambda [W] and
- * dh0 [B,W] (may be NULL) are fp32 and complete. */
-int rglru_hip_bwd(const void* x, const void* prep, const float* lambda, const float* h0,
+ * dW = du^T x, and dx += du W with two library GEMMs; db_a, db_x [nb*bw] and dlambda [W]
+ * (grad_dtype) and dh0 [B,W] (fp32, may be NULL) are complete. */
+int rglru_hip_bwd(const void* x, const void* prep, const float* h0,
                   const uint8_t* flags, const void* dy, const float* dh_last, void* ws,
-                  void* dx, void* du_a, void* du_x, float* db_a, float* db_x, float* dlambda,
-                  float* dh0, int64_t B, int64_t T, int64_t W, int64_t nb, float c, int dtype,
+                  void* dx, void* du_a, void* du_x, void* db_a, void* db_x, void* dlambda,
+                  float* dh0, int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, int grad_dtype,
                   void* stream);
 
 /* Complete backward for the fast configurations (rglru_hip_fast_path(W, nb, dtype) != 0: 16-bit
  * storage, gate blocks of 32, 64 or 128 channels, 16-byte aligned tensors).  Same inputs as
- * rglru_hip_bwd; dx[B,T,W] is the full input gradient and dw_a, dw_x [nb,bw,bw] fp32 the weight
- * gradients: the two gate GEMMs run in a second hand-written kernel instead of being left to the
- * caller.  Returns RGLRU_E_UNSUPPORTED for other configurations. */
+ * rglru_hip_bwd; dx[B,T,W] is the full input gradient and dw_a, dw_x [nb,bw,bw] (grad_dtype) the
+ * weight gradients: the two gate GEMMs run in a second hand-written kernel instead of being left
+ * to the caller.  Returns RGLRU_E_UNSUPPORTED for other configurations. */
 int rglru_hip_fast_path(int64_t W, int64_t nb, int dtype);
-int rglru_hip_bwd_full(const void* x, const void* prep, const float* lambda, const float* h0,
+int rglru_hip_bwd_full(const void* x, const void* prep, const float* h0,
                        const uint8_t* flags, const void* dy, const float* dh_last, void* ws,
-                       void* dx, float* dw_a, float* dw_x, float* db_a, float* db_x, float* dlambda,
-                       float* dh0, int64_t B, int64_t T, int64_t W, int64_t nb, float c, int dtype,
+                       void* dx, void* dw_a, void* dw_x, void* db_a, void* db_x, void* dlambda,
+                       float* dh0, int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, int grad_dtype,
                        void* stream);
 
 /* One decode step (T == 1): h[B,W] fp32 is updated in place, y[B,W] (dtype) = h as stored. */
