@@ -731,6 +731,11 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
   __shared__ __attribute__((aligned(16))) unsigned char stage_dx_all[kWaves * WaveStage<TR>::kBytes];
   __shared__ __attribute__((aligned(16))) unsigned char stage_du_all[kWaves * PairStage<TR>::kBytes];
   __shared__ unsigned s_ticket[2];
+  // With 128-channel blocks the weight registers (64) push the kernel into spilling; the input
+  // gate's weights then live in LDS instead (one copy per workgroup, read as B fragments per tile).
+  constexpr bool XLDS = (NKG == 8);
+  constexpr int WROW = KC + Tr::HW;
+  __shared__ __attribute__((aligned(16))) IO lds_wx[XLDS ? 32 * kWaves * WROW : Tr::HW];
 
   const WaveId w = wave_identity(p, blockIdx.x);
   const int hf = w.hf, tid = threadIdx.x;
@@ -741,7 +746,19 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
   const IO* w_a_row = wg + ((long long)(0 * p.nb + w.k) * p.bwp + o_safe) * p.bwp + hf * Tr::HW;
   const IO* w_x_row = wg + ((long long)(1 * p.nb + w.k) * p.bwp + o_safe) * p.bwp + hf * Tr::HW;
   HeldWeights<IO, NKG> hw;
-  hw.load(w_a_row, w_x_row);
+  if constexpr (XLDS) {
+#pragma unroll
+    for (int kg = 0; kg < NKG; ++kg) hw.a[kg] = *reinterpret_cast<const Frag*>(w_a_row + kg * Tr::KG);
+    // rows of this workgroup's four slabs of W_x
+    const IO* src = wg + ((long long)(1 * p.nb + w.k) * p.bwp + (w.unit % p.groups) * (32 * kWaves)) * p.bwp;
+    for (int idx = threadIdx.x; idx < 32 * kWaves * (KC / Tr::HW); idx += kThreads) {
+      const int row = idx / (KC / Tr::HW), v = idx - row * (KC / Tr::HW);
+      *reinterpret_cast<Frag*>(lds_wx + row * WROW + v * Tr::HW) = *reinterpret_cast<const Frag*>(src + (long long)row * p.bwp + v * Tr::HW);
+    }
+    __syncthreads();
+  } else {
+    hw.load(w_a_row, w_x_row);
+  }
   const float bias_a = p.bias[w.kp], bias_x = p.bias[p.Wp + w.kp];
   const float sp = p.sp[w.kp], cs = p.cs[w.kp];
   const IO* x = (const IO*)p.x;
@@ -808,7 +825,22 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
     f32x16 ua, ux;
     float xv[EL], gy[EL];
     if (w.slab_ok) {
-      gate_mfma_held<IO, MT, NKG>(lds_x, hw, 0, w.slab, w.r, hf, bias_a, bias_x, ua, ux, xv);
+      if constexpr (XLDS) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) { ua[v] = bias_a; ux[v] = bias_x; }
+        const IO* xrow = lds_x + tile_row<MT>(0, w.r) * LDSROW + hf * Tr::HW;
+        const IO* brow = lds_wx + (w.wave * 32 + w.r) * WROW + hf * Tr::HW;
+#pragma unroll
+        for (int kg = 0; kg < NKG; ++kg) {
+          const Frag xa = *reinterpret_cast<const Frag*>(xrow + kg * Tr::KG);
+          Tr::mma(ua, xa, hw.a[kg]);
+          Tr::mma(ux, xa, *reinterpret_cast<const Frag*>(brow + kg * Tr::KG));
+        }
+#pragma unroll
+        for (int e = 0; e < EL; ++e) xv[e] = (float)lds_x[(hf * EL + e) * LDSROW + w.slab * 32 + w.r];
+      } else {
+        gate_mfma_held<IO, MT, NKG>(lds_x, hw, 0, w.slab, w.r, hf, bias_a, bias_x, ua, ux, xv);
+      }
 #pragma unroll
       for (int e = 0; e < EL; ++e) gy[e] = (float)lds_dy[(hf * EL + e) * LDSROW + w.slab * 32 + w.r];
     }
