@@ -1133,10 +1133,15 @@ struct FinishArgs {
   const float* partial; const float* dsp; void* db_a; void* db_x; void* dlambda;
   const float* dw_partial; void* dw_a; void* dw_x;
   int W, nb, bw, bwp, Wp, wg_per_unit, n_wg, vec_blocks, grad_dtype;
+  uint4* clean; long long clean_n;                         // backward records and tickets, zeroed for the next pass
 };
 
 __global__ __launch_bounds__(256) void finish_kernel(FinishArgs p) {
   __shared__ float part_sum[3][4][64];
+  // the scan kernels of this pass are done: leave their records and tickets zeroed, so that another
+  // backward pass over the same forward needs no clearing launch of its own
+  for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < p.clean_n; i += (long long)gridDim.x * blockDim.x)
+    p.clean[i] = make_uint4(0u, 0u, 0u, 0u);
   if ((int)blockIdx.x >= p.vec_blocks) {
     const long long total = (long long)p.nb * p.bw * 2 * p.bw;
     const long long i = (long long)(blockIdx.x - p.vec_blocks) * blockDim.x + threadIdx.x;
@@ -1395,7 +1400,7 @@ int rglru_hip_fwd(const void* x, const void* prep, const float* h0, const uint8_
   WorkLayout L = make_work_layout(B, T, g);
   hipStream_t s = (hipStream_t)stream;
   char* wb = (char*)ws;
-  rc = launch_clear(wb, L.f_begin, L.f_end, s);         // forward carry records, tickets, failure word
+  rc = launch_clear(wb, L.f_begin, L.b_end, s);         // carry records and tickets of both passes, failure word
   if (rc) return rc;
   FusedArgs a;
   memset(&a, 0, sizeof(a));
@@ -1442,8 +1447,6 @@ int rglru_hip_bwd(const void* x, const void* prep, const float* h0,
   WorkLayout L = make_work_layout(B, T, g);
   hipStream_t s = (hipStream_t)stream;
   char* wb = (char*)ws;
-  rc = launch_clear(wb, L.b_begin, L.b_end, s);           // backward carry records, tickets, failure word
-  if (rc) return rc;
   FusedArgs a;
   memset(&a, 0, sizeof(a));
   fill_common(a, g, prep, dtype);
@@ -1468,6 +1471,7 @@ int rglru_hip_bwd(const void* x, const void* prep, const float* h0,
   r.partial = a.partial; r.dsp = finish_dsp(g, prep, dtype); r.db_a = db_a; r.db_x = db_x; r.dlambda = dlambda;
   r.W = (int)W; r.nb = (int)nb; r.bw = (int)g.bw; r.bwp = (int)g.bwp; r.Wp = (int)g.Wp; r.wg_per_unit = a.wg_per_unit;
   r.vec_blocks = (int)((W + 63) / 64); r.grad_dtype = grad_dtype;
+  r.clean = (uint4*)(wb + L.b_begin); r.clean_n = (long long)((L.b_end - L.b_begin) / 16);
   hipLaunchKernelGGL(finish_kernel, dim3((unsigned)r.vec_blocks), dim3(256), 0, s, r);
   return check_launch("bwd finish");
 }
@@ -1499,8 +1503,6 @@ int rglru_hip_bwd_full(const void* x, const void* prep, const float* h0,
   WorkLayout L = make_work_layout(B, T, g);
   hipStream_t s = (hipStream_t)stream;
   char* wb = (char*)ws;
-  rc = launch_clear(wb, L.b_begin, L.b_end, s);
-  if (rc) return rc;
   FusedArgs a;
   memset(&a, 0, sizeof(a));
   fill_common(a, g, prep, dtype);
@@ -1544,6 +1546,7 @@ int rglru_hip_bwd_full(const void* x, const void* prep, const float* h0,
   r.dw_partial = a.dw_partial; r.dw_a = dw_a; r.dw_x = dw_x;
   r.W = (int)W; r.nb = (int)nb; r.bw = (int)g.bw; r.bwp = (int)g.bwp; r.Wp = (int)g.Wp; r.wg_per_unit = a.wg_per_unit;
   r.n_wg = n_wg; r.vec_blocks = (int)((W + 63) / 64); r.grad_dtype = grad_dtype;
+  r.clean = (uint4*)(wb + L.b_begin); r.clean_n = (long long)((L.b_end - L.b_begin) / 16);
   const long long total = nb * g.bw * 2 * g.bw;
   hipLaunchKernelGGL(finish_kernel, dim3((unsigned)(r.vec_blocks + (total + 255) / 256)), dim3(256), 0, s, r);
   return check_launch("bwd_full finish");

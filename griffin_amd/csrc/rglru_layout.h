@@ -57,11 +57,11 @@ inline PrepLayout make_prep_layout(const Geometry& g, size_t elem) {
 //   partial     [maxWg][3][Wp]  per-workgroup sums for db_a, db_x, dLambda
 //   du2         [B][T][2W]      16-bit: gate pre-activation gradients (fast backward only)
 //   dw_partial  [kGemmWgPerUnit][nb][bwp][2*bwp] fp32 per-workgroup weight-gradient sums
-//   --- [f_begin, f_end) is cleared before the forward pass ---
+//   --- [f_begin, b_end) is cleared at the start of the forward pass ---
 //   f_rec_a     [B][<=nC][W]    64-bit carry records of the forward chain
 //   f_ticket    [units][kMaxQueues]
-//   fail        [1]             failure word; part of both regions, so either pass clears it
-//   --- [b_begin, b_end) is cleared before the backward pass ---
+//   fail        [1]             failure word (either pass sets it; only forward clears it)
+//   --- [b_begin, b_end): clean on entry to a backward pass, which cleans it again when it is done ---
 //   b_rec_a     [B][nC][W]      64-bit carry records of the backward chain
 //   b_ticket    [units][kMaxQueues]
 constexpr int kMaxQueues = 64;          // ticket queues per unit (sequences are dealt round-robin to them)
@@ -88,9 +88,9 @@ inline WorkLayout make_work_layout(int64_t B, int64_t T, const Geometry& g) {
   w.f_begin = off;
   w.f_rec_a = take(B * w.nC * g.W * 8);
   w.f_ticket = take(g.units * kMaxQueues * 4);
-  w.b_begin = off;                     // the failure word belongs to both regions
   w.fail = take(4);
   w.f_end = off;
+  w.b_begin = off;
   w.b_rec_a = take(B * w.nC * g.W * 8);
   w.b_ticket = take(g.units * kMaxQueues * 4);
   w.b_end = off;

@@ -86,9 +86,10 @@ int rglru_hip_prepare(const void* w_a, const void* b_a, const void* w_x, const v
                       const void* lambda, float c, int64_t W, int64_t nb, int dtype, int vec_dtype,
                       void* prep, void* stream);
 
-/* Workspace shared by one forward call and its backward call.  Forward fills it (chunk
- * checkpoints of the fp32 state, carry records); backward reads the checkpoints and uses the
- * rest as scratch.  Contents on entry to forward do not matter. */
+/* Workspace shared by one forward call and its backward call(s).  Forward initialises it (chunk
+ * checkpoints of the fp32 state, cleared carry records for both passes), so its contents on entry
+ * to forward do not matter; a backward call must be given the workspace of its forward call, reads
+ * the checkpoints, uses the rest as scratch and leaves it ready for another backward call. */
 size_t rglru_hip_workspace_bytes(int64_t B, int64_t T, int64_t W, int64_t nb);
 
 /* y[B,T,W] (dtype) and h_last[B,W] (fp32, may be NULL) from x[B,T,W], h0[B,W] (fp32, NULL = 0). */

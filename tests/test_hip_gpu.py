@@ -131,6 +131,29 @@ def test_fused_bf16_matches_fp32_oracle(cfg):
         assert err < BF16_TOL, (name, err)
 
 
+@pytest.mark.parametrize("dtype,shape", [(torch.bfloat16, (2, 200, 256, 2)), (torch.float32, (2, 70, 48, 3))])
+def test_backward_twice_over_one_forward(dtype, shape):
+    """A second backward pass over the same forward (retain_graph) reuses the workspace of the first
+    and must reproduce its gradients (up to the rounding of a different carry composition order: which
+    records a walk meets depends on timing); linearity in the upstream gradient is checked too."""
+    from griffin_amd import hip_rglru
+
+    B, T, W, nb = shape
+    _say("backward twice", dtype, shape)
+    case = orc.make_case(B, T, W, nb, seed=11)
+    leaves = [case[k].to(dtype).cuda().requires_grad_(True) for k in PARAMS]
+    dy = case["dy"].to(dtype).cuda()
+    y, _ = hip_rglru(*leaves, 8.0)
+    first = torch.autograd.grad(y, leaves, dy, retain_graph=True)
+    second = torch.autograd.grad(y, leaves, dy, retain_graph=True)
+    tol = 1e-5 if dtype == torch.float32 else BF16_TOL
+    for a, b in zip(first, second):
+        assert rel_err(b.float(), a.float()) < tol
+    doubled = torch.autograd.grad(y, leaves, dy * 2)
+    for a, b in zip(first, doubled):
+        assert rel_err(b.float(), 2 * a.float()) < tol
+
+
 # ------------------------------------------------------------------ golden vectors of the reference
 @pytest.mark.parametrize("name", ["rglru_plain_b2_t16_w32", "rglru_masks_b2_t16_w32", "rglru_odd_b3_t37_w65"])
 def test_fused_matches_reference_golden_vectors(golden_dir, name):
