@@ -962,8 +962,11 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
 // unit itself: multiplying a tile by the identity returns it in accumulator layout, where a lane
 // holds 16 consecutive tokens of one column.
 // ------------------------------------------------------------------------------------------
+constexpr int kGradWaves = 8;                            // waves per workgroup of the gradient GEMM kernel
+constexpr int kGradThreads = 64 * kGradWaves;
+
 template <typename IO, int NKG>
-__global__ __launch_bounds__(kThreads, 1) void gate_grad_kernel(FusedArgs p) {
+__global__ __launch_bounds__(kGradThreads, 1) void gate_grad_kernel(FusedArgs p) {
   typedef Io<IO> Tr;
   typedef typename Tr::Frag Frag;
   static_assert(sizeof(IO) == 2 && NKG > 0, "16-bit storage only");
@@ -971,27 +974,37 @@ __global__ __launch_bounds__(kThreads, 1) void gate_grad_kernel(FusedArgs p) {
   constexpr int KC = NKG * Tr::KG;                       // block width
   constexpr int S = KC / 32;                             // slabs in the block
   constexpr int K2 = 2 * KC, NKG2 = 2 * NKG;             // contraction length of the first GEMM
+  constexpr int NKT = 2 * S;                             // 32-wide kappa tiles of du2
+  constexpr int KT_HALF = (NKT + 1) / 2;                 // kappa tiles each half of the workgroup accumulates
   constexpr int ROW_X = KC + Tr::HW, ROW_DU = K2 + Tr::HW, ROW_T = TR + Tr::HW;
   __shared__ __attribute__((aligned(16))) IO lds_du[TR * ROW_DU];
   __shared__ __attribute__((aligned(16))) IO lds_x[TR * ROW_X];
   __shared__ __attribute__((aligned(16))) IO lds_dx[TR * ROW_X];
   __shared__ __attribute__((aligned(16))) IO lds_dut[K2 * ROW_T];          // du2 transposed: [kappa][token]
-  __shared__ __attribute__((aligned(16))) unsigned char stage_all[kWaves * WaveStage<TR>::kBytes];
+  __shared__ __attribute__((aligned(16))) unsigned char stage_all[4 * WaveStage<TR>::kBytes];
 
+  // Eight waves, two per SIMD: wave = 4 * half + slab.  Between the two barriers of a tile the lower
+  // half does the input-gradient GEMM of its slab and the stores, the upper half transposes du2;
+  // after the second barrier both halves accumulate their share of the kappa tiles of dW2T.
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, hf = lane >> 5;
+  const int slab = wave & 3, half = wave >> 2;
   const int k = blockIdx.x % p.nb, wg_in_unit = blockIdx.x / p.nb, n_wg = gridDim.x / p.nb;
-  const bool slab_ok = wave < S;
-  unsigned char* stage = stage_all + wave * WaveStage<TR>::kBytes;
+  const bool slab_ok = slab < S;
+  unsigned char* stage = stage_all + slab * WaveStage<TR>::kBytes;
   const long long rows_total = (long long)p.B * p.T;
   const long long n_tiles = (rows_total + TR - 1) / TR;
   const unsigned row_bytes = (unsigned)p.W * 2u;
 
-  // this wave's rows of w2t: B operand of the first GEMM, lane (n = j, hf) holds kappa = 16 kg + 8 hf + i
+  // lower half: this wave's rows of w2t, B operand of the first GEMM; lane (n = j, hf) holds
+  // kappa = 16 kg + 8 hf + i
   Frag w2[NKG2];
-  {
-    const IO* row = (const IO*)p.w2t + ((long long)k * p.bwp + (slab_ok ? wave * 32 + r : 0)) * (2 * p.bwp) + hf * Tr::HW;
+  if (half == 0) {
+    const IO* row = (const IO*)p.w2t + ((long long)k * p.bwp + (slab_ok ? slab * 32 + r : 0)) * (2 * p.bwp) + hf * Tr::HW;
 #pragma unroll
     for (int kg = 0; kg < NKG2; ++kg) w2[kg] = *reinterpret_cast<const Frag*>(row + kg * Tr::KG);
+  } else {
+#pragma unroll
+    for (int kg = 0; kg < NKG2; ++kg) w2[kg] = Tr::zero();
   }
   // identity fragments: element i of ident[q] is 1 where 16 q + 8 hf + i == r
   Frag ident[2];
@@ -1000,32 +1013,33 @@ __global__ __launch_bounds__(kThreads, 1) void gate_grad_kernel(FusedArgs p) {
 #pragma unroll
     for (int i = 0; i < Tr::HW; ++i) ident[qd][i] = (IO)((16 * qd + 8 * hf + i == r) ? 1.0f : 0.0f);
 
-  f32x16 dw[2 * S];
+  f32x16 dw[KT_HALF];                                    // kappa tiles half * KT_HALF + i of this wave's slab
 #pragma unroll
-  for (int kt = 0; kt < 2 * S; ++kt)
+  for (int kt = 0; kt < KT_HALF; ++kt)
 #pragma unroll
     for (int v = 0; v < 16; ++v) dw[kt][v] = 0.f;
 
   // cooperative tile loads: du2 (TR x K2), x and dx (TR x KC)
   constexpr int VPR_DU = K2 / Tr::HW, VPR_X = KC / Tr::HW;
-  constexpr int NV_DU = (TR * VPR_DU + kThreads - 1) / kThreads, NV_X = (TR * VPR_X + kThreads - 1) / kThreads;
+  constexpr int NV_DU = (TR * VPR_DU + kGradThreads - 1) / kGradThreads, NV_X = (TR * VPR_X + kGradThreads - 1) / kGradThreads;
   Frag pre_du[NV_DU], pre_x[NV_X], pre_dx[NV_X];
   auto issue = [&](long long tile) {
-    if (tile >= n_tiles) return;
-    const long long row0 = tile * TR;
-    const int rows = (int)((rows_total - row0) < TR ? (rows_total - row0) : TR);
+    // a tile past the end keeps valid addresses but an empty extent: nothing is fetched
+    const bool live = tile < n_tiles;
+    const long long row0 = live ? tile * TR : 0;
+    const int rows = !live ? 0 : (int)((rows_total - row0) < TR ? (rows_total - row0) : TR);
     const rsrc_t rdu = make_rsrc((const IO*)p.du_a + row0 * 2 * p.W, (unsigned)rows * 2u * row_bytes);
     const rsrc_t rx = make_rsrc((const IO*)p.x + row0 * p.W, (unsigned)rows * row_bytes);
     const rsrc_t rdx = make_rsrc((const IO*)p.dx + row0 * p.W, (unsigned)rows * row_bytes);
 #pragma unroll
     for (int i = 0; i < NV_DU; ++i) {
-      const int idx = tid + i * kThreads;
+      const int idx = tid + i * kGradThreads;
       const int row = idx / VPR_DU, cv = idx - row * VPR_DU;
       pre_du[i] = buf_load_frag<Frag>(rdu, idx < TR * VPR_DU ? (unsigned)row * 2u * row_bytes + (unsigned)(k * 2 * p.bw + cv * Tr::HW) * 2u : kOutOfRange);
     }
 #pragma unroll
     for (int i = 0; i < NV_X; ++i) {
-      const int idx = tid + i * kThreads;
+      const int idx = tid + i * kGradThreads;
       const int row = idx / VPR_X, cv = idx - row * VPR_X;
       const unsigned off = idx < TR * VPR_X ? (unsigned)row * row_bytes + (unsigned)(k * p.bw + cv * Tr::HW) * 2u : kOutOfRange;
       pre_x[i] = buf_load_frag<Frag>(rx, off);
@@ -1038,13 +1052,13 @@ __global__ __launch_bounds__(kThreads, 1) void gate_grad_kernel(FusedArgs p) {
   for (; tile < n_tiles; tile += n_wg) {
 #pragma unroll
     for (int i = 0; i < NV_DU; ++i) {
-      const int idx = tid + i * kThreads;
+      const int idx = tid + i * kGradThreads;
       const int row = idx / VPR_DU, cv = idx - row * VPR_DU;
       if (idx < TR * VPR_DU) *reinterpret_cast<Frag*>(lds_du + row * ROW_DU + cv * Tr::HW) = pre_du[i];
     }
 #pragma unroll
     for (int i = 0; i < NV_X; ++i) {
-      const int idx = tid + i * kThreads;
+      const int idx = tid + i * kGradThreads;
       const int row = idx / VPR_X, cv = idx - row * VPR_X;
       if (idx < TR * VPR_X) {
         *reinterpret_cast<Frag*>(lds_x + row * ROW_X + cv * Tr::HW) = pre_x[i];
@@ -1057,58 +1071,66 @@ __global__ __launch_bounds__(kThreads, 1) void gate_grad_kernel(FusedArgs p) {
     const long long row0 = tile * TR;
     const IO* a_row_du = lds_du + tile_row<1>(0, r) * ROW_DU + hf * Tr::HW;
     const IO* a_row_x = lds_x + tile_row<1>(0, r) * ROW_X + hf * Tr::HW;
-    // transposes: kappa tiles 2 * wave and 2 * wave + 1 of du2 go to lds_dut
-#pragma unroll
-    for (int h2 = 0; h2 < 2; ++h2) {
-      const int kt = 2 * wave + h2;
-      if (kt < 2 * S) {
-        f32x16 dc;
-#pragma unroll
-        for (int v = 0; v < 16; ++v) dc[v] = 0.f;
-        Tr::mma(dc, *reinterpret_cast<const Frag*>(a_row_du + (2 * kt) * Tr::KG), ident[0]);
-        Tr::mma(dc, *reinterpret_cast<const Frag*>(a_row_du + (2 * kt + 1) * Tr::KG), ident[1]);
-        Frag lo, hi;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) { lo[i] = (IO)dc[i]; hi[i] = (IO)dc[8 + i]; }
-        IO* dst = lds_dut + (kt * 32 + r) * ROW_T + hf * 16;
-        *reinterpret_cast<Frag*>(dst) = lo;
-        *reinterpret_cast<Frag*>(dst + 8) = hi;
-      }
-    }
+    // x of this wave's slab with tokens along the lane vector (A operand of the second GEMM)
     Frag xt_lo = Tr::zero(), xt_hi = Tr::zero();
     if (slab_ok) {
-      // x of this wave's slab with tokens along the lane vector (A operand of the second GEMM)
       f32x16 xc;
 #pragma unroll
       for (int v = 0; v < 16; ++v) xc[v] = 0.f;
-      Tr::mma(xc, *reinterpret_cast<const Frag*>(a_row_x + (2 * wave) * Tr::KG), ident[0]);
-      Tr::mma(xc, *reinterpret_cast<const Frag*>(a_row_x + (2 * wave + 1) * Tr::KG), ident[1]);
+      Tr::mma(xc, *reinterpret_cast<const Frag*>(a_row_x + (2 * slab) * Tr::KG), ident[0]);
+      Tr::mma(xc, *reinterpret_cast<const Frag*>(a_row_x + (2 * slab + 1) * Tr::KG), ident[1]);
 #pragma unroll
       for (int i = 0; i < 8; ++i) { xt_lo[i] = (IO)xc[i]; xt_hi[i] = (IO)xc[8 + i]; }
-      // first GEMM: dx tile = direct part + du2 . w2t^T
-      f32x16 acc;
+    }
+    if (half == 1) {
+      // transposes: the upper half's four waves share the kappa tiles of du2, written to lds_dut
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[v] = (float)lds_dx[(hf * 16 + v) * ROW_X + wave * 32 + r];
+      for (int h2 = 0; h2 < (NKT + 3) / 4; ++h2) {
+        const int kt = 4 * h2 + slab;
+        if (kt < NKT) {
+          f32x16 dc;
 #pragma unroll
-      for (int kg = 0; kg < NKG2; ++kg)
+          for (int v = 0; v < 16; ++v) dc[v] = 0.f;
+          Tr::mma(dc, *reinterpret_cast<const Frag*>(a_row_du + (2 * kt) * Tr::KG), ident[0]);
+          Tr::mma(dc, *reinterpret_cast<const Frag*>(a_row_du + (2 * kt + 1) * Tr::KG), ident[1]);
+          Frag lo, hi;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) { lo[i] = (IO)dc[i]; hi[i] = (IO)dc[8 + i]; }
+          IO* dst = lds_dut + (kt * 32 + r) * ROW_T + hf * 16;
+          *reinterpret_cast<Frag*>(dst) = lo;
+          *reinterpret_cast<Frag*>(dst + 8) = hi;
+        }
+      }
+    } else if (slab_ok) {
+      // first GEMM: dx tile = direct part + du2 . w2t^T, on two accumulators
+      f32x16 acc, acc_odd;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) { acc[v] = (float)lds_dx[(hf * 16 + v) * ROW_X + slab * 32 + r]; acc_odd[v] = 0.f; }
+#pragma unroll
+      for (int kg = 0; kg < NKG2; kg += 2) {
         Tr::mma(acc, *reinterpret_cast<const Frag*>(a_row_du + kg * Tr::KG), w2[kg]);
+        Tr::mma(acc_odd, *reinterpret_cast<const Frag*>(a_row_du + (kg + 1) * Tr::KG), w2[kg + 1]);
+      }
       unsigned char* my = stage + WaveStage<TR>::row_offset(hf * 16) + r * 2;
 #pragma unroll
-      for (int v = 0; v < 16; ++v) *reinterpret_cast<IO*>(my + v * WaveStage<TR>::kRowBytes) = (IO)acc[v];
+      for (int v = 0; v < 16; ++v) *reinterpret_cast<IO*>(my + v * WaveStage<TR>::kRowBytes) = (IO)(acc[v] + acc_odd[v]);
       wave_lds_fence();
       const int rows = (int)((rows_total - row0) < TR ? (rows_total - row0) : TR);
       const rsrc_t rdx = make_rsrc((const IO*)p.dx + row0 * p.W, (unsigned)rows * row_bytes);
-      stage_flush<TR>(stage, rdx, row_bytes, (unsigned)(k * p.bw + wave * 32) * 2u, lane);
+      stage_flush<TR>(stage, rdx, row_bytes, (unsigned)(k * p.bw + slab * 32) * 2u, lane);
       wave_lds_fence();
     }
     __syncthreads();
     if (slab_ok) {
-      // second GEMM: dW2T[j, kappa] += sum over the tile's tokens
+      // second GEMM: dW2T[j, kappa] += sum over the tile's tokens, this half's kappa tiles
 #pragma unroll
-      for (int kt = 0; kt < 2 * S; ++kt) {
-        const IO* b_row = lds_dut + (kt * 32 + r) * ROW_T + hf * 16;
-        Tr::mma(dw[kt], xt_lo, *reinterpret_cast<const Frag*>(b_row));
-        Tr::mma(dw[kt], xt_hi, *reinterpret_cast<const Frag*>(b_row + 8));
+      for (int i = 0; i < KT_HALF; ++i) {
+        const int kt = half * KT_HALF + i;
+        if (kt < NKT) {
+          const IO* b_row = lds_dut + (kt * 32 + r) * ROW_T + hf * 16;
+          Tr::mma(dw[i], xt_lo, *reinterpret_cast<const Frag*>(b_row));
+          Tr::mma(dw[i], xt_hi, *reinterpret_cast<const Frag*>(b_row + 8));
+        }
       }
     }
   }
@@ -1116,12 +1138,16 @@ __global__ __launch_bounds__(kThreads, 1) void gate_grad_kernel(FusedArgs p) {
   if (slab_ok) {
     float* part = p.dw_partial + (((long long)wg_in_unit * p.nb + k) * p.bwp) * (2 * p.bwp);
 #pragma unroll
-    for (int kt = 0; kt < 2 * S; ++kt)
+    for (int i = 0; i < KT_HALF; ++i) {
+      const int kt = half * KT_HALF + i;
+      if (kt < NKT) {
 #pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const int j = wave * 32 + 8 * (v >> 2) + 4 * hf + (v & 3);
-        part[(long long)j * (2 * p.bwp) + kt * 32 + r] = dw[kt][v];
+        for (int v = 0; v < 16; ++v) {
+          const int j = slab * 32 + 8 * (v >> 2) + 4 * hf + (v & 3);
+          part[(long long)j * (2 * p.bwp) + kt * 32 + r] = dw[i][v];
+        }
       }
+    }
   }
 }
 
@@ -1151,11 +1177,15 @@ __global__ __launch_bounds__(256) void finish_kernel(FinishArgs p) {
     const int k = (int)(i / ((long long)2 * p.bw * p.bw));
     const long long stride = (long long)p.nb * p.bwp * 2 * p.bwp;
     const float* src = p.dw_partial + ((long long)k * p.bwp + j) * (2 * p.bwp) + kap;
+    // fixed summation order; eight loads in flight per thread
     float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
     int g = 0;
-    for (; g + 3 < p.n_wg; g += 4) {
-      s0 += src[(long long)g * stride]; s1 += src[(long long)(g + 1) * stride];
-      s2 += src[(long long)(g + 2) * stride]; s3 += src[(long long)(g + 3) * stride];
+    for (; g + 7 < p.n_wg; g += 8) {
+      float v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = src[(long long)(g + u) * stride];
+      s0 += v[0]; s1 += v[1]; s2 += v[2]; s3 += v[3];
+      s0 += v[4]; s1 += v[5]; s2 += v[6]; s3 += v[7];
     }
     for (; g < p.n_wg; ++g) s0 += src[(long long)g * stride];
     const float sum = (s0 + s1) + (s2 + s3);
@@ -1533,9 +1563,9 @@ int rglru_hip_bwd_full(const void* x, const void* prep, const float* h0,
 #ifndef RGLRU_EXP_NOGEMM
   {
     KernelTimer timer(3, s);
-    if (nkg == 8) hipLaunchKernelGGL((gate_grad_kernel<__bf16, 8>), grid2, dim3(kThreads), 0, s, a);
-    else if (nkg == 4) hipLaunchKernelGGL((gate_grad_kernel<__bf16, 4>), grid2, dim3(kThreads), 0, s, a);
-    else hipLaunchKernelGGL((gate_grad_kernel<__bf16, 2>), grid2, dim3(kThreads), 0, s, a);
+    if (nkg == 8) hipLaunchKernelGGL((gate_grad_kernel<__bf16, 8>), grid2, dim3(kGradThreads), 0, s, a);
+    else if (nkg == 4) hipLaunchKernelGGL((gate_grad_kernel<__bf16, 4>), grid2, dim3(kGradThreads), 0, s, a);
+    else hipLaunchKernelGGL((gate_grad_kernel<__bf16, 2>), grid2, dim3(kGradThreads), 0, s, a);
   }
 #endif
   rc = check_launch("bwd_full gemm");
