@@ -335,9 +335,6 @@ RGLRU_DEVICE float one_minus_exp(float y, float a) {
 template <bool PRECISE, bool MASKED>
 RGLRU_DEVICE GateOut gate_forward(float ua, float ux, float x, float sp, unsigned fl) {
   GateOut o;
-#ifdef RGLRU_EXP_NOGATES
-  o.r = ua; o.i = ux; o.a = 0.9f; o.g = 0.4f; o.g2 = 0.16f; o.z = x * ux; return o;
-#endif
   o.r = sigmoid_fast(ua);
   o.i = sigmoid_fast(ux);
   float l2 = o.r * sp;                         // log2(a) <= 0

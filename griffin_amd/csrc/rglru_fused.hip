@@ -393,9 +393,7 @@ RGLRU_DEVICE void fwd_finalize(const FusedArgs& p, const WaveId& w, const FwdTil
       *reinterpret_cast<IO*>(my + e * WaveStage<TR>::kRowBytes) = (IO)h;
     }
     wave_lds_fence();
-#ifndef RGLRU_EXP_NOSTORE
     stage_flush<TR>(stage, ry, row_bytes, (unsigned)(w.k * p.bw + w.slab * 32) * 2u, w.lane);
-#endif
     wave_lds_fence();
   } else {
     unsigned voff = ch_ok ? (unsigned)(hf * EL) * row_bytes + (unsigned)w.ch * (unsigned)sizeof(IO) : kOutOfRange;
@@ -884,9 +882,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
     if (!last_chunk && hf == 0) carry_publish(chain, c, A_t, D_t, false);
     issue(tk_next);
     float d_in = (last_chunk && p.dh_last) ? p.dh_last[(long long)b * W + w.ch] : 0.f;
-#ifndef RGLRU_EXP_BWD_NOLOOKBACK
     if (!last_chunk) d_in = carry_lookback(chain, c, +1, p.nC, 0.f, true, p.limit, p.fail);
-#endif
     const float d_out = fmaf(A_t, d_in, D_t);
     if (hf == 0) carry_publish(chain, c, 0.f, d_out, true);
     if (hf == 0 && c == 0 && p.dh0) p.dh0[(long long)b * W + w.ch] = d_out;
@@ -1560,14 +1556,12 @@ int rglru_hip_bwd_full(const void* x, const void* prep, const float* h0,
   if (rc) return rc;
   int n_wg = num_compute_units() / (int)nb; if (n_wg < 1) n_wg = 1; if (n_wg > kGemmWgPerUnit) n_wg = kGemmWgPerUnit;
   dim3 grid2((unsigned)(n_wg * nb));
-#ifndef RGLRU_EXP_NOGEMM
   {
     KernelTimer timer(3, s);
     if (nkg == 8) hipLaunchKernelGGL((gate_grad_kernel<__bf16, 8>), grid2, dim3(kGradThreads), 0, s, a);
     else if (nkg == 4) hipLaunchKernelGGL((gate_grad_kernel<__bf16, 4>), grid2, dim3(kGradThreads), 0, s, a);
     else hipLaunchKernelGGL((gate_grad_kernel<__bf16, 2>), grid2, dim3(kGradThreads), 0, s, a);
   }
-#endif
   rc = check_launch("bwd_full gemm");
   if (rc) return rc;
   FinishArgs r;

@@ -95,6 +95,26 @@ class RG_LRU(nn.Module):
             and xt.numel() > 0
         )
 
+    def _gate_parameters(self):
+        return (self.recurrence_gate.weight, self.recurrence_gate.bias, self.input_gate.weight,
+                self.input_gate.bias, self.Lambda)
+
+    def _needs_grad(self, xt: Tensor, ht_minus_1: Tensor | None) -> bool:
+        if not torch.is_grad_enabled():
+            return False
+        tensors = (xt, ht_minus_1) + self._gate_parameters()
+        return any(t is not None and t.requires_grad for t in tensors)
+
+    def _prepared(self, dtype: torch.dtype, device: torch.device):
+        """Kernel-side parameter image for inference, rebuilt when a parameter is replaced or updated
+        in place (every in-place update bumps the tensor's version counter)."""
+        params = self._gate_parameters()
+        key = (dtype, device, float(self.c)) + tuple((q.data_ptr(), q._version) for q in params)
+        if getattr(self, "_prep_key", None) != key:
+            self._prep = hip_scan.PreparedParams(*params, self.c, dtype)
+            self._prep_key = key
+        return self._prep
+
     def forward(
         self,
         xt: Tensor,
@@ -138,6 +158,15 @@ class RG_LRU(nn.Module):
                     f'scan_mode="{mode}" requires CUDA/HIP tensors and the RG-LRU HIP library; '
                     f"got a {xt.device.type} tensor"
                 )
+            if steps == 1 and not self._needs_grad(xt, ht_minus_1):
+                # decode: the single-step kernel on a prepared parameter image kept between calls
+                prep = self._prepared(xt.dtype, xt.device)
+                state = (torch.zeros(batch, width, device=xt.device, dtype=torch.float32) if ht_minus_1 is None
+                         else ht_minus_1.to(torch.float32).clone(memory_format=torch.contiguous_format))
+                flags = hip_scan.pack_flags(reset_mask, active_mask)
+                y = hip_scan.hip_rglru_step(xt[:, 0], prep, state, None if flags is None else flags.reshape(batch))
+                y = y.unsqueeze(1)
+                return (y, state) if return_state else y
             y, state = hip_scan.hip_rglru(
                 xt, self.recurrence_gate.weight, self.recurrence_gate.bias, self.input_gate.weight,
                 self.input_gate.bias, self.Lambda, self.c, ht_minus_1, reset_mask, active_mask,

@@ -259,6 +259,48 @@ def test_config4_prefill_then_512_decode_steps():
         assert err < BF16_TOL
 
 
+def test_module_decode_uses_step_kernel_and_tracks_parameter_updates():
+    """T == 1 without gradients goes through the single-step kernel on a cached parameter image; the
+    image must follow in-place parameter updates.  Reference behaviour: griffin/griffin.py:279-284."""
+    case = orc.make_case(4, 6, 256, 2, seed=13, h0_std=0.5)
+    ref = _module_from_case(case, 2, "sequential", device="cpu")
+    hip = _module_from_case(case, 2, "hip")
+    x = case["x"]
+    reset = torch.zeros(4, 6, dtype=torch.bool)
+    reset[2, 3] = True
+    active = torch.ones(4, 6, dtype=torch.bool)
+    active[1, 4:] = False
+
+    def decode(module, device):
+        state = case["h0"].to(device)
+        outs = []
+        with torch.no_grad():
+            for t in range(6):
+                y, state = module(x[:, t:t + 1].to(device), state, reset_mask=reset[:, t:t + 1].to(device),
+                                  active_mask=active[:, t:t + 1].to(device), return_state=True)
+                outs.append(y)
+        return torch.cat(outs, dim=1).cpu(), state.cpu()
+
+    y_ref, h_ref = decode(ref, "cpu")
+    y_hip, h_hip = decode(hip, "cuda")
+    assert hip._prep_key is not None                          # the step path ran
+    assert rel_err(y_hip, y_ref) < FP32_TOL and rel_err(h_hip, h_ref) < FP32_TOL
+    # an optimiser-style in-place update must invalidate the cached image
+    with torch.no_grad():
+        for module in (ref, hip):
+            module.Lambda.add_(0.25)
+            module.input_gate.bias.add_(0.1)
+    y_ref2, h_ref2 = decode(ref, "cpu")
+    y_hip2, h_hip2 = decode(hip, "cuda")
+    assert rel_err(y_ref2, y_ref) > 1e-3                      # the update matters
+    assert rel_err(y_hip2, y_ref2) < FP32_TOL and rel_err(h_hip2, h_ref2) < FP32_TOL
+    # with gradients enabled the same call takes the differentiable path
+    xg = x[:, :1].cuda().requires_grad_(True)
+    yg = hip(xg)
+    yg.sum().backward()
+    assert xg.grad is not None
+
+
 def test_config5_recurrent_block_with_hip_scan():
     """d_model 768 -> width 1024 block: the HIP scan slotted into the block unchanged, forward and
     backward against the same block on the CPU with the sequential scan (fp32, reduced length),
