@@ -1148,7 +1148,7 @@ __global__ __launch_bounds__(kGradThreads, 1) void gate_grad_kernel(FusedArgs p)
 }
 
 // Last launch of a backward pass: sums the per-workgroup partial results and writes the parameter
-// gradients in the caller's type.  Workgroups [0, vec_blocks) own 64 channels each of db_a, db_x and
+// gradients in the caller's type.  Workgroups [0, vec_blocks) own 16 channels each of db_a, db_x and
 // dLambda; the rest (fast backward only) own 256 elements each of the two weight gradients,
 // dW_gate[k][o][j] = sum over workgroups of dW2T[wg][k][j][2 o + gate].
 struct FinishArgs {
@@ -1159,54 +1159,68 @@ struct FinishArgs {
 };
 
 __global__ __launch_bounds__(256) void finish_kernel(FinishArgs p) {
-  __shared__ float part_sum[3][4][64];
+  __shared__ float part_sum[3][16][16];
   // the scan kernels of this pass are done: leave their records and tickets zeroed, so that another
   // backward pass over the same forward needs no clearing launch of its own
   for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < p.clean_n; i += (long long)gridDim.x * blockDim.x)
     p.clean[i] = make_uint4(0u, 0u, 0u, 0u);
   if ((int)blockIdx.x >= p.vec_blocks) {
-    const long long total = (long long)p.nb * p.bw * 2 * p.bw;
-    const long long i = (long long)(blockIdx.x - p.vec_blocks) * blockDim.x + threadIdx.x;
-    if (i >= total) return;
+    // four consecutive kappa (two output channels x two gates) per thread, 16-byte loads; bw is a
+    // multiple of 32 on this path, so a group of four never crosses a row
+    const long long total4 = (long long)p.nb * p.bw * 2 * p.bw / 4;
+    const long long i4 = (long long)(blockIdx.x - p.vec_blocks) * blockDim.x + threadIdx.x;
+    if (i4 >= total4) return;
+    const long long i = i4 * 4;
     const int kap = (int)(i % (2 * p.bw));
     const int j = (int)((i / (2 * p.bw)) % p.bw);
     const int k = (int)(i / ((long long)2 * p.bw * p.bw));
     const long long stride = (long long)p.nb * p.bwp * 2 * p.bwp;
     const float* src = p.dw_partial + ((long long)k * p.bwp + j) * (2 * p.bwp) + kap;
     // fixed summation order; eight loads in flight per thread
-    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+    float4 s0 = make_float4(0.f, 0.f, 0.f, 0.f), s1 = s0;
     int g = 0;
     for (; g + 7 < p.n_wg; g += 8) {
-      float v[8];
+      float4 v[8];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) v[u] = src[(long long)(g + u) * stride];
-      s0 += v[0]; s1 += v[1]; s2 += v[2]; s3 += v[3];
-      s0 += v[4]; s1 += v[5]; s2 += v[6]; s3 += v[7];
+      for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const float4*>(src + (long long)(g + u) * stride);
+#pragma unroll
+      for (int u = 0; u < 8; u += 2) {
+        s0.x += v[u].x; s0.y += v[u].y; s0.z += v[u].z; s0.w += v[u].w;
+        s1.x += v[u + 1].x; s1.y += v[u + 1].y; s1.z += v[u + 1].z; s1.w += v[u + 1].w;
+      }
     }
-    for (; g < p.n_wg; ++g) s0 += src[(long long)g * stride];
-    const float sum = (s0 + s1) + (s2 + s3);
-    store_vec((kap & 1) ? p.dw_x : p.dw_a, ((long long)k * p.bw + (kap >> 1)) * p.bw + j, sum, p.grad_dtype);
+    for (; g < p.n_wg; ++g) {
+      const float4 v = *reinterpret_cast<const float4*>(src + (long long)g * stride);
+      s0.x += v.x; s0.y += v.y; s0.z += v.z; s0.w += v.w;
+    }
+    const long long o0 = ((long long)k * p.bw + (kap >> 1)) * p.bw + j;      // element (k, o, j); o + 1 is bw further
+    store_vec(p.dw_a, o0, s0.x + s1.x, p.grad_dtype);
+    store_vec(p.dw_x, o0, s0.y + s1.y, p.grad_dtype);
+    store_vec(p.dw_a, o0 + p.bw, s0.z + s1.z, p.grad_dtype);
+    store_vec(p.dw_x, o0 + p.bw, s0.w + s1.w, p.grad_dtype);
     return;
   }
-  // 64 channels per workgroup; four quarter-sums per channel are combined through LDS
-  const int lane = threadIdx.x & 63, quarter = threadIdx.x >> 6;
-  const int ch = blockIdx.x * 64 + lane;
+  // 16 channels per workgroup; sixteen threads per channel each sum a share of the per-workgroup
+  // partials (independent loads), combined through LDS in a fixed order
+  const int cl = threadIdx.x & 15, share = threadIdx.x >> 4;
+  const int ch = blockIdx.x * 16 + cl;
   float sa = 0.f, sx = 0.f, sl = 0.f;
   int kp = 0;
   if (ch < p.W) {
     const int k = ch / p.bw, o = ch - k * p.bw;
     kp = k * p.bwp + o;
-    for (int g = quarter; g < p.wg_per_unit; g += 4) {
+#pragma unroll 4
+    for (int g = share; g < p.wg_per_unit; g += 16) {
       const float* part = p.partial + (long long)g * 3 * p.Wp + kp;
       sa += part[0]; sx += part[p.Wp]; sl += part[2 * p.Wp];
     }
   }
-  part_sum[0][quarter][lane] = sa; part_sum[1][quarter][lane] = sx; part_sum[2][quarter][lane] = sl;
+  part_sum[0][share][cl] = sa; part_sum[1][share][cl] = sx; part_sum[2][share][cl] = sl;
   __syncthreads();
-  if (quarter == 0 && ch < p.W) {
-    sa = (part_sum[0][0][lane] + part_sum[0][1][lane]) + (part_sum[0][2][lane] + part_sum[0][3][lane]);
-    sx = (part_sum[1][0][lane] + part_sum[1][1][lane]) + (part_sum[1][2][lane] + part_sum[1][3][lane]);
-    sl = (part_sum[2][0][lane] + part_sum[2][1][lane]) + (part_sum[2][2][lane] + part_sum[2][3][lane]);
+  if (share == 0 && ch < p.W) {
+    sa = 0.f; sx = 0.f; sl = 0.f;
+#pragma unroll
+    for (int q = 0; q < 16; ++q) { sa += part_sum[0][q][cl]; sx += part_sum[1][q][cl]; sl += part_sum[2][q][cl]; }
     store_vec(p.db_a, ch, sa, p.grad_dtype);
     store_vec(p.db_x, ch, sx, p.grad_dtype);
     store_vec(p.dlambda, ch, sl * p.dsp[kp], p.grad_dtype);
@@ -1496,7 +1510,7 @@ int rglru_hip_bwd(const void* x, const void* prep, const float* h0,
   memset(&r, 0, sizeof(r));
   r.partial = a.partial; r.dsp = finish_dsp(g, prep, dtype); r.db_a = db_a; r.db_x = db_x; r.dlambda = dlambda;
   r.W = (int)W; r.nb = (int)nb; r.bw = (int)g.bw; r.bwp = (int)g.bwp; r.Wp = (int)g.Wp; r.wg_per_unit = a.wg_per_unit;
-  r.vec_blocks = (int)((W + 63) / 64); r.grad_dtype = grad_dtype;
+  r.vec_blocks = (int)((W + 15) / 16); r.grad_dtype = grad_dtype;
   r.clean = (uint4*)(wb + L.b_begin); r.clean_n = (long long)((L.b_end - L.b_begin) / 16);
   hipLaunchKernelGGL(finish_kernel, dim3((unsigned)r.vec_blocks), dim3(256), 0, s, r);
   return check_launch("bwd finish");
@@ -1569,10 +1583,10 @@ int rglru_hip_bwd_full(const void* x, const void* prep, const float* h0,
   r.partial = a.partial; r.dsp = finish_dsp(g, prep, dtype); r.db_a = db_a; r.db_x = db_x; r.dlambda = dlambda;
   r.dw_partial = a.dw_partial; r.dw_a = dw_a; r.dw_x = dw_x;
   r.W = (int)W; r.nb = (int)nb; r.bw = (int)g.bw; r.bwp = (int)g.bwp; r.Wp = (int)g.Wp; r.wg_per_unit = a.wg_per_unit;
-  r.n_wg = n_wg; r.vec_blocks = (int)((W + 63) / 64); r.grad_dtype = grad_dtype;
+  r.n_wg = n_wg; r.vec_blocks = (int)((W + 15) / 16); r.grad_dtype = grad_dtype;
   r.clean = (uint4*)(wb + L.b_begin); r.clean_n = (long long)((L.b_end - L.b_begin) / 16);
   const long long total = nb * g.bw * 2 * g.bw;
-  hipLaunchKernelGGL(finish_kernel, dim3((unsigned)(r.vec_blocks + (total + 255) / 256)), dim3(256), 0, s, r);
+  hipLaunchKernelGGL(finish_kernel, dim3((unsigned)(r.vec_blocks + (total / 4 + 255) / 256)), dim3(256), 0, s, r);
   return check_launch("bwd_full finish");
 }
 
