@@ -122,7 +122,7 @@ struct FusedArgs {
   unsigned* fail; float* partial; float* dw_partial;
   // geometry
   int B, T, W, nb, bw, bwp, S, Wp, groups, units;
-  int nC, nCf, ckpt_nC, wg_per_unit, aligned, full_slabs, queues;
+  int nC, nCf, ckpt_nC, wg_per_unit, aligned, full_slabs, queues, flags_vec;
   long long limit;
 #ifdef RGLRU_TRACE
   long long* trace;
@@ -281,6 +281,28 @@ RGLRU_DEVICE unsigned token_flag(const FusedArgs& p, long long token_row, bool i
   return p.flags ? (unsigned)p.flags[token_row] : 0u;
 }
 
+// Flags of a lane's run of 16 consecutive tokens, two bits per token (token e at bits 2e, 2e + 1);
+// tokens past the end of the sequence read as inactive.  When the sequence length is a multiple of
+// 16 and the flag array is 16-byte aligned (flags_vec), a run is wholly inside or outside the
+// sequence and its flags are one 16-byte load.
+RGLRU_DEVICE unsigned pack_flag_bytes(unsigned d) {
+  unsigned t = d & 0x03030303u;
+  t = (t | (t >> 6)) & 0x000F000Fu;
+  return (t | (t >> 12)) & 0xFFu;
+}
+RGLRU_DEVICE unsigned flag_run(const FusedArgs& p, long long token_row, int t_first) {
+  if (p.flags_vec) {
+    if (t_first >= p.T) return 0xAAAAAAAAu;
+    if (!p.flags) return 0u;
+    const uint4 w = *reinterpret_cast<const uint4*>(p.flags + token_row);
+    return pack_flag_bytes(w.x) | (pack_flag_bytes(w.y) << 8) | (pack_flag_bytes(w.z) << 16) | (pack_flag_bytes(w.w) << 24);
+  }
+  unsigned bits = 0u;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) bits |= token_flag(p, token_row + e, t_first + e < p.T) << (2 * e);
+  return bits;
+}
+
 // ------------------------------------------------------------------------------------------
 // Forward
 // ------------------------------------------------------------------------------------------
@@ -289,10 +311,11 @@ RGLRU_DEVICE unsigned token_flag(const FusedArgs& p, long long token_row, bool i
 template <typename IO, bool MASKED>
 RGLRU_DEVICE void fwd_gates(const FusedArgs& p, long long trow, int t_first, const f32x16& ua, const f32x16& ux,
                             const float (&xv)[16], float sp, float* a, float* z) {
+  unsigned flbits = 0u;
+  if constexpr (MASKED) flbits = flag_run(p, trow, t_first);
 #pragma unroll
   for (int v = 0; v < 16; ++v) {
-    unsigned fl = 0u;
-    if constexpr (MASKED) fl = token_flag(p, trow + v, t_first + v < p.T);
+    const unsigned fl = MASKED ? ((flbits >> (2 * v)) & 3u) : 0u;
     GateOut go = gate_forward<Precise<IO>::value, MASKED>(ua[v], ux[v], xv[v], sp, fl);
     a[v] = go.a; z[v] = go.z;
   }
@@ -855,11 +878,11 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
     // gate recomputation; z is not kept (g * i * x is recomputed where needed)
     float r[EL], gi[EL], a[EL], g[EL];
     unsigned flbits = 0u;                                // two flag bits per local step
+    if constexpr (MASKED) flbits = flag_run(p, trow, t0 + hf * EL);
     float A = 1.f, H = 0.f;
 #pragma unroll
     for (int e = 0; e < EL; ++e) {
-      unsigned fl = 0u;
-      if constexpr (MASKED) { fl = token_flag(p, trow + e, t0 + hf * EL + e < p.T); flbits |= fl << (2 * e); }
+      const unsigned fl = MASKED ? ((flbits >> (2 * e)) & 3u) : 0u;
       GateOut go = gate_forward<false, MASKED>(ua[e], ux[e], xv[e], sp, fl);
       r[e] = go.r; gi[e] = go.i; a[e] = go.a; g[e] = go.g;
       H = fmaf(go.a, H, go.z); A *= go.a;
@@ -1446,6 +1469,7 @@ int rglru_hip_fwd(const void* x, const void* prep, const float* h0, const uint8_
   memset(&a, 0, sizeof(a));
   fill_common(a, g, prep, dtype);
   a.x = x; a.h0 = h0; a.flags = flags; a.y = y; a.h_last = h_last;
+  a.flags_vec = (T % 16 == 0) && ((uintptr_t)flags % 16 == 0);
   a.ckpt = (float*)(wb + L.ckpt); a.rec_a = (rec_t*)(wb + L.f_rec_a);
   a.ticket = (unsigned*)(wb + L.f_ticket); a.fail = (unsigned*)(wb + L.fail);
   a.B = (int)B; a.T = (int)T; a.nC = (int)L.nC; a.ckpt_nC = (int)L.nC;
@@ -1491,6 +1515,7 @@ int rglru_hip_bwd(const void* x, const void* prep, const float* h0,
   memset(&a, 0, sizeof(a));
   fill_common(a, g, prep, dtype);
   a.x = x; a.h0 = h0; a.flags = flags; a.dy = dy; a.dh_last = dh_last;
+  a.flags_vec = (T % 16 == 0) && ((uintptr_t)flags % 16 == 0);
   a.dx = dx; a.du_a = du_a; a.du_x = du_x; a.dh0 = dh0;
   a.ckpt = (float*)(wb + L.ckpt); a.rec_a = (rec_t*)(wb + L.b_rec_a);
   a.ticket = (unsigned*)(wb + L.b_ticket); a.fail = (unsigned*)(wb + L.fail);
@@ -1547,6 +1572,7 @@ int rglru_hip_bwd_full(const void* x, const void* prep, const float* h0,
   memset(&a, 0, sizeof(a));
   fill_common(a, g, prep, dtype);
   a.x = x; a.h0 = h0; a.flags = flags; a.dy = dy; a.dh_last = dh_last;
+  a.flags_vec = (T % 16 == 0) && ((uintptr_t)flags % 16 == 0);
   a.dx = dx; a.du_a = wb + L.du2; a.dh0 = dh0;
   a.ckpt = (float*)(wb + L.ckpt); a.rec_a = (rec_t*)(wb + L.b_rec_a);
   a.ticket = (unsigned*)(wb + L.b_ticket); a.fail = (unsigned*)(wb + L.fail);
