@@ -110,6 +110,11 @@ BF16_CASES = [
     (2, 64, 64, 2, True, False),     # 32-wide blocks
     (1, 150, 640, 2, True, True),    # 320-wide blocks: streamed weights, two LDS slices
     (2, 33, 24, 3, True, True),      # unaligned rows (width 24 -> 48-byte rows, 8-wide blocks)
+    (2, 75, 256, 2, False, True),    # fast kernels with a ragged last tile and no flags
+    (2, 80, 256, 2, True, False),    # length a multiple of 16 but not of 32: vector flag loads, half-empty tile
+    (1, 700, 128, 1, True, True),    # one sequence: every workgroup of the block works on the same chain
+    (70, 40, 128, 1, False, False),  # more sequences than ticket queues
+    (3, 17, 128, 2, True, True),     # shorter than one tile
 ]
 
 
