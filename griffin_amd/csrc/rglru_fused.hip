@@ -875,20 +875,26 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
       continue;
     }
 
-    // gate recomputation; z is not kept (g * i * x is recomputed where needed)
+    // Gate recomputation in two steps.  The chunk's reverse map needs only the decay a_t (and dy),
+    // so the recurrence gate comes first and the map is published before the rest of the gate math:
+    // the neighbours see it that much earlier.  z is not kept (g * i * x is recomputed where needed).
     float r[EL], gi[EL], a[EL], g[EL];
     unsigned flbits = 0u;                                // two flag bits per local step
     if constexpr (MASKED) flbits = flag_run(p, trow, t0 + hf * EL);
-    float A = 1.f, H = 0.f;
+    float A = 1.f;
 #pragma unroll
     for (int e = 0; e < EL; ++e) {
-      const unsigned fl = MASKED ? ((flbits >> (2 * e)) & 3u) : 0u;
-      GateOut go = gate_forward<false, MASKED>(ua[e], ux[e], xv[e], sp, fl);
-      r[e] = go.r; gi[e] = go.i; a[e] = go.a; g[e] = go.g;
-      H = fmaf(go.a, H, go.z); A *= go.a;
+      const float re = sigmoid_fast(ua[e]);
+      float ae = __builtin_amdgcn_exp2f(re * sp);
+      if constexpr (MASKED) {                            // as in gate_forward: reset a = 0, then padding a = 1
+        if ((flbits >> (2 * e)) & 1u) ae = 0.f;
+        if ((flbits >> (2 * e)) & 2u) ae = 1.f;
+      }
+      r[e] = re; a[e] = ae;
+      A *= ae;
     }
-    const float A_o = xhalf(A, hf), H_o = xhalf(H, hf);
-    const float A_lo = hf ? A_o : A, H_lo = hf ? H_o : H;
+    const float A_o = xhalf(A, hf);
+    const float A_lo = hf ? A_o : A;
     const float A_hi = hf ? A : A_o;
     // reverse affine map of this lane's run and of the chunk
     float carry = 0.f;
@@ -903,6 +909,24 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
     chain.rec = p.rec_a + seq; chain.stride = W;
     const bool last_chunk = c == p.nC - 1;
     if (!last_chunk && hf == 0) carry_publish(chain, c, A_t, D_t, false);
+
+    // input gate, g = sqrt(1 - a^2) and the forward map of the lane's run (for h at the run's start)
+    float H = 0.f;
+#pragma unroll
+    for (int e = 0; e < EL; ++e) {
+      const unsigned fl = MASKED ? ((flbits >> (2 * e)) & 3u) : 0u;
+      const float ie = sigmoid_fast(ux[e]);
+      const float l2 = r[e] * sp;
+      const float a_raw = MASKED ? __builtin_amdgcn_exp2f(l2) : a[e];
+      float ge = __builtin_amdgcn_sqrtf(fmaxf(one_minus_exp<false>(l2 * (2.0f * kLn2), a_raw), 0.0f));
+      if constexpr (MASKED) { if (fl & 1u) ge = 1.f; }
+      float ze = ge * ie * xv[e];
+      if constexpr (MASKED) { if (fl & 2u) ze = 0.f; }
+      gi[e] = ie; g[e] = ge;
+      H = fmaf(a[e], H, ze);
+    }
+    const float H_o = xhalf(H, hf);
+    const float H_lo = hf ? H_o : H;
     issue(tk_next);
     float d_in = (last_chunk && p.dh_last) ? p.dh_last[(long long)b * W + w.ch] : 0.f;
     if (!last_chunk) d_in = carry_lookback(chain, c, +1, p.nC, 0.f, true, p.limit, p.fail);
