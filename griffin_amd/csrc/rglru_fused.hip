@@ -1475,6 +1475,11 @@ size_t rglru_hip_workspace_bytes(int64_t B, int64_t T, int64_t W, int64_t nb) {
   return make_work_layout(B, T, make_geometry(W, nb)).total;
 }
 
+size_t rglru_hip_bwd_scratch_bytes(int64_t B, int64_t T, int64_t W, int64_t nb, int dtype) {
+  if (B <= 0 || T <= 0 || W <= 0 || nb <= 0 || W % nb) return 0;
+  return make_scratch_layout(B, T, make_geometry(W, nb), rglru_hip_fast_path(W, nb, dtype) != 0).total;
+}
+
 int rglru_hip_fwd(const void* x, const void* prep, const float* h0, const uint8_t* flags,
                   void* y, float* h_last, void* ws,
                   int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, void* stream) {
@@ -1519,7 +1524,7 @@ static int check_grad_dtype(const char* who, int grad_dtype) {
 }
 
 int rglru_hip_bwd(const void* x, const void* prep, const float* h0,
-                  const uint8_t* flags, const void* dy, const float* dh_last, void* ws,
+                  const uint8_t* flags, const void* dy, const float* dh_last, void* ws, void* scratch,
                   void* dx, void* du_a, void* du_x, void* db_a, void* db_x, void* dlambda,
                   float* dh0, int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, int grad_dtype,
                   void* stream) {
@@ -1528,7 +1533,7 @@ int rglru_hip_bwd(const void* x, const void* prep, const float* h0,
   rc = check_grad_dtype("bwd", grad_dtype);
   if (rc) return rc;
   if (B <= 0 || T <= 0) return fail(RGLRU_E_ARG, "bwd: B and T must be positive (got %lld, %lld)", (long long)B, (long long)T);
-  if (!x || !prep || !dy || !ws || !dx || !du_a || !du_x || !db_a || !db_x || !dlambda)
+  if (!x || !prep || !dy || !ws || !scratch || !dx || !du_a || !du_x || !db_a || !db_x || !dlambda)
     return fail(RGLRU_E_ARG, "bwd: null pointer");
   if (B * T * W >= (1ll << 40) || B * T >= (1ll << 31)) return fail(RGLRU_E_UNSUPPORTED, "bwd: tensor too large");
   Geometry g = make_geometry(W, nb);
@@ -1543,7 +1548,7 @@ int rglru_hip_bwd(const void* x, const void* prep, const float* h0,
   a.dx = dx; a.du_a = du_a; a.du_x = du_x; a.dh0 = dh0;
   a.ckpt = (float*)(wb + L.ckpt); a.rec_a = (rec_t*)(wb + L.b_rec_a);
   a.ticket = (unsigned*)(wb + L.b_ticket); a.fail = (unsigned*)(wb + L.fail);
-  a.partial = (float*)(wb + L.partial);
+  a.partial = (float*)((char*)scratch + make_scratch_layout(B, T, g, false).partial);
   a.B = (int)B; a.T = (int)T; a.nC = (int)((T + kChunk - 1) / kChunk); a.ckpt_nC = (int)L.nC; a.nCf = (int)L.nCf;
   a.aligned = is_aligned(x, W, g.bw, elem_size(dtype));
   a.wg_per_unit = pick_wg_per_unit(g, B * (long long)a.nC, 2, L.max_wg);
@@ -1572,7 +1577,7 @@ int rglru_hip_fast_path(int64_t W, int64_t nb, int dtype) {
 }
 
 int rglru_hip_bwd_full(const void* x, const void* prep, const float* h0,
-                       const uint8_t* flags, const void* dy, const float* dh_last, void* ws,
+                       const uint8_t* flags, const void* dy, const float* dh_last, void* ws, void* scratch,
                        void* dx, void* dw_a, void* dw_x, void* db_a, void* db_x, void* dlambda,
                        float* dh0, int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, int grad_dtype,
                        void* stream) {
@@ -1583,7 +1588,7 @@ int rglru_hip_bwd_full(const void* x, const void* prep, const float* h0,
   if (!rglru_hip_fast_path(W, nb, dtype))
     return fail(RGLRU_E_UNSUPPORTED, "bwd_full: needs 16-bit storage and gate blocks of 32, 64 or 128 channels");
   if (B <= 0 || T <= 0) return fail(RGLRU_E_ARG, "bwd_full: B and T must be positive (got %lld, %lld)", (long long)B, (long long)T);
-  if (!x || !prep || !dy || !ws || !dx || !dw_a || !dw_x || !db_a || !db_x || !dlambda)
+  if (!x || !prep || !dy || !ws || !scratch || !dx || !dw_a || !dw_x || !db_a || !db_x || !dlambda)
     return fail(RGLRU_E_ARG, "bwd_full: null pointer");
   if (B * T * W >= (1ll << 40) || B * T >= (1ll << 31)) return fail(RGLRU_E_UNSUPPORTED, "bwd_full: tensor too large");
   Geometry g = make_geometry(W, nb);
@@ -1597,10 +1602,12 @@ int rglru_hip_bwd_full(const void* x, const void* prep, const float* h0,
   fill_common(a, g, prep, dtype);
   a.x = x; a.h0 = h0; a.flags = flags; a.dy = dy; a.dh_last = dh_last;
   a.flags_vec = (T % 16 == 0) && ((uintptr_t)flags % 16 == 0);
-  a.dx = dx; a.du_a = wb + L.du2; a.dh0 = dh0;
+  const ScratchLayout SL = make_scratch_layout(B, T, g, true);
+  char* sb = (char*)scratch;
+  a.dx = dx; a.du_a = sb + SL.du2; a.dh0 = dh0;
   a.ckpt = (float*)(wb + L.ckpt); a.rec_a = (rec_t*)(wb + L.b_rec_a);
   a.ticket = (unsigned*)(wb + L.b_ticket); a.fail = (unsigned*)(wb + L.fail);
-  a.partial = (float*)(wb + L.partial); a.dw_partial = (float*)(wb + L.dw_partial);
+  a.partial = (float*)(sb + SL.partial); a.dw_partial = (float*)(sb + SL.dw_partial);
   a.B = (int)B; a.T = (int)T; a.nC = (int)((T + kChunk - 1) / kChunk); a.ckpt_nC = (int)L.nC;
   a.aligned = 1;
   a.wg_per_unit = pick_wg_per_unit(g, B * (long long)a.nC, 2, L.max_wg);

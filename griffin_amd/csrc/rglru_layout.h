@@ -51,12 +51,10 @@ inline PrepLayout make_prep_layout(const Geometry& g, size_t elem) {
   return p;
 }
 
-// Workspace of one forward/backward pair.  nC = chunks of 32 tokens (rounded up to even),
-// nCf = forward tiles of 64 tokens.
+// Workspace of one forward/backward pair: what has to survive from forward to backward, plus the
+// carry records of both passes.  nC = chunks of 32 tokens (rounded up to even), nCf = forward tiles
+// of 64 tokens.
 //   ckpt        [B][nC][W]      fp32 state after each chunk (kept for backward)
-//   partial     [maxWg][3][Wp]  per-workgroup sums for db_a, db_x, dLambda
-//   du2         [B][T][2W]      16-bit: gate pre-activation gradients (fast backward only)
-//   dw_partial  [kGemmWgPerUnit][nb][bwp][2*bwp] fp32 per-workgroup weight-gradient sums
 //   --- [f_begin, b_end) is cleared at the start of the forward pass ---
 //   f_rec_a     [B][<=nC][W]    64-bit carry records of the forward chain
 //   f_ticket    [units][kMaxQueues]
@@ -69,7 +67,7 @@ constexpr int kGemmWgPerUnit = 32;      // workgroups per gate block in the grad
 
 struct WorkLayout {
   int64_t nC, nCf, max_wg;
-  size_t ckpt, partial, du2, dw_partial;
+  size_t ckpt;
   size_t f_begin, f_rec_a, f_ticket, f_end;
   size_t b_begin, b_rec_a, b_ticket, fail, b_end, total;
 };
@@ -82,9 +80,6 @@ inline WorkLayout make_work_layout(int64_t B, int64_t T, const Geometry& g) {
   size_t off = 0;
   auto take = [&](int64_t bytes) { size_t at = off; off += (size_t)round_up(bytes, 256); return at; };
   w.ckpt = take(B * w.nC * g.W * 4);
-  w.partial = take(w.max_wg * 3 * g.Wp * 4);
-  w.du2 = take(B * T * 2 * g.W * 2);                      // 16-bit storage only
-  w.dw_partial = take((int64_t)kGemmWgPerUnit * g.nb * g.bwp * 2 * g.bwp * 4);
   w.f_begin = off;
   w.f_rec_a = take(B * w.nC * g.W * 8);
   w.f_ticket = take(g.units * kMaxQueues * 4);
@@ -96,6 +91,25 @@ inline WorkLayout make_work_layout(int64_t B, int64_t T, const Geometry& g) {
   w.b_end = off;
   w.total = off;
   return w;
+}
+
+// Scratch of one backward call; nothing in it outlives the call, its contents on entry do not matter.
+//   partial     [maxWg][3][Wp]  per-workgroup sums for db_a, db_x, dLambda
+//   du2         [B][T][2W]      16-bit: gate pre-activation gradients (fast backward only)
+//   dw_partial  [kGemmWgPerUnit][nb][bwp][2*bwp] fp32 per-workgroup weight-gradient sums (fast backward only)
+struct ScratchLayout {
+  size_t partial, du2, dw_partial, total;
+};
+
+inline ScratchLayout make_scratch_layout(int64_t B, int64_t T, const Geometry& g, bool fast) {
+  ScratchLayout s;
+  size_t off = 0;
+  auto take = [&](int64_t bytes) { size_t at = off; off += (size_t)round_up(bytes, 256); return at; };
+  s.partial = take((int64_t)256 * 3 * g.Wp * 4);
+  s.du2 = take(fast ? B * T * 2 * g.W * 2 : 0);
+  s.dw_partial = take(fast ? (int64_t)kGemmWgPerUnit * g.nb * g.bwp * 2 * g.bwp * 4 : 0);
+  s.total = off;
+  return s;
 }
 
 // Scan-only workspace: chunks of 32 tokens; everything is cleared before each pass.

@@ -226,12 +226,14 @@ class _HipRGLRU(torch.autograd.Function):
             db_x = torch.empty(nb, bw, dtype=gdt, device=device)
             dlam = torch.empty(W, dtype=gdt, device=device)
             dh0 = torch.empty(B, W, dtype=torch.float32, device=device) if ctx.needs_input_grad[6] else None
+            # scratch of this call only (the workspace kept since forward holds just checkpoints and records)
+            scratch = torch.empty(lib.rglru_hip_bwd_scratch_bytes(B, T, W, nb, code), dtype=torch.uint8, device=device)
             if lib.rglru_hip_fast_path(W, nb, code) and dy.data_ptr() % 16 == 0 and x.data_ptr() % 16 == 0:
                 # everything in hand-written kernels, including the two gate GEMMs
                 dw_a = torch.empty(nb, bw, bw, dtype=gdt, device=device)
                 dw_x = torch.empty(nb, bw, bw, dtype=gdt, device=device)
                 _lib.check(lib.rglru_hip_bwd_full(x.data_ptr(), image.data_ptr(), _ptr(h0c), _ptr(flags),
-                                                  dy.data_ptr(), _ptr(dhl), ws.data_ptr(), dx.data_ptr(), dw_a.data_ptr(),
+                                                  dy.data_ptr(), _ptr(dhl), ws.data_ptr(), scratch.data_ptr(), dx.data_ptr(), dw_a.data_ptr(),
                                                   dw_x.data_ptr(), db_a.data_ptr(), db_x.data_ptr(), dlam.data_ptr(),
                                                   _ptr(dh0), B, T, W, nb, code, gcode, _stream_ptr(device)),
                            "rglru_hip_bwd_full")
@@ -239,7 +241,7 @@ class _HipRGLRU(torch.autograd.Function):
                 du_a = torch.empty_like(x)
                 du_x = torch.empty_like(x)
                 _lib.check(lib.rglru_hip_bwd(x.data_ptr(), image.data_ptr(), _ptr(h0c), _ptr(flags),
-                                             dy.data_ptr(), _ptr(dhl), ws.data_ptr(), dx.data_ptr(), du_a.data_ptr(),
+                                             dy.data_ptr(), _ptr(dhl), ws.data_ptr(), scratch.data_ptr(), dx.data_ptr(), du_a.data_ptr(),
                                              du_x.data_ptr(), db_a.data_ptr(), db_x.data_ptr(), dlam.data_ptr(),
                                              _ptr(dh0), B, T, W, nb, code, gcode, _stream_ptr(device)), "rglru_hip_bwd")
                 # block-diagonal library GEMMs: dW[k] = du[:, k]^T x[:, k];  dx[:, k] += du[:, k] W[k]

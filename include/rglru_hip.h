@@ -39,7 +39,7 @@
 extern "C" {
 #endif
 
-#define RGLRU_ABI_VERSION 2
+#define RGLRU_ABI_VERSION 3
 
 enum { RGLRU_F32 = 0, RGLRU_BF16 = 1 };
 
@@ -92,6 +92,12 @@ int rglru_hip_prepare(const void* w_a, const void* b_a, const void* w_x, const v
  * the checkpoints, uses the rest as scratch and leaves it ready for another backward call. */
 size_t rglru_hip_workspace_bytes(int64_t B, int64_t T, int64_t W, int64_t nb);
 
+/* Scratch of one backward call (per-workgroup partial sums; for the fast configurations also the
+ * gate pre-activation gradients between the two backward kernels).  Nothing in it outlives the
+ * call, so it is allocated when backward runs instead of being held since forward; its contents on
+ * entry do not matter.  The size depends on which backward entry point the configuration takes. */
+size_t rglru_hip_bwd_scratch_bytes(int64_t B, int64_t T, int64_t W, int64_t nb, int dtype);
+
 /* y[B,T,W] (dtype) and h_last[B,W] (fp32, may be NULL) from x[B,T,W], h0[B,W] (fp32, NULL = 0). */
 int rglru_hip_fwd(const void* x, const void* prep, const float* h0, const uint8_t* flags,
                   void* y, float* h_last, void* ws,
@@ -104,7 +110,7 @@ int rglru_hip_fwd(const void* x, const void* prep, const float* h0, const uint8_
  * dW = du^T x, and dx += du W with two library GEMMs; db_a, db_x [nb*bw] and dlambda [W]
  * (grad_dtype) and dh0 [B,W] (fp32, may be NULL) are complete. */
 int rglru_hip_bwd(const void* x, const void* prep, const float* h0,
-                  const uint8_t* flags, const void* dy, const float* dh_last, void* ws,
+                  const uint8_t* flags, const void* dy, const float* dh_last, void* ws, void* scratch,
                   void* dx, void* du_a, void* du_x, void* db_a, void* db_x, void* dlambda,
                   float* dh0, int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, int grad_dtype,
                   void* stream);
@@ -116,7 +122,7 @@ int rglru_hip_bwd(const void* x, const void* prep, const float* h0,
  * to the caller.  Returns RGLRU_E_UNSUPPORTED for other configurations. */
 int rglru_hip_fast_path(int64_t W, int64_t nb, int dtype);
 int rglru_hip_bwd_full(const void* x, const void* prep, const float* h0,
-                       const uint8_t* flags, const void* dy, const float* dh_last, void* ws,
+                       const uint8_t* flags, const void* dy, const float* dh_last, void* ws, void* scratch,
                        void* dx, void* dw_a, void* dw_x, void* db_a, void* db_x, void* dlambda,
                        float* dh0, int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, int grad_dtype,
                        void* stream);
