@@ -571,7 +571,10 @@ __global__ __launch_bounds__(kThreads, 2) void fwd_kernel(FusedArgs p) {
           fwd_gates<IO, true>(p, trow + 16 * mt, c * TR + hf * EL + 16 * mt, ua[mt], ux[mt], xpart, sp, tile.a + 16 * mt, tile.z + 16 * mt);
         }
         fwd_local<MT, true>(p, w, tile);
-        fwd_finalize<IO, MT, true, false>(p, w, tile, stage);
+        // 16-bit outputs go through the wave's staging area when whole 64-byte row segments can be
+        // written (aligned rows, blocks made of full slabs); else element by element
+        if (sizeof(IO) == 2 && p.aligned && p.full_slabs) fwd_finalize<IO, MT, true, true>(p, w, tile, stage);
+        else fwd_finalize<IO, MT, true, false>(p, w, tile, stage);
       }
     }
   }
@@ -1503,7 +1506,7 @@ int rglru_hip_fwd(const void* x, const void* prep, const float* h0, const uint8_
   a.ticket = (unsigned*)(wb + L.f_ticket); a.fail = (unsigned*)(wb + L.fail);
   a.B = (int)B; a.T = (int)T; a.nC = (int)L.nC; a.ckpt_nC = (int)L.nC;
   a.nCf = (int)((T + 32 * kFwdMT - 1) / (32 * kFwdMT));
-  a.aligned = is_aligned(x, W, g.bw, elem_size(dtype));
+  a.aligned = is_aligned(x, W, g.bw, elem_size(dtype)) && ((uintptr_t)y % 16 == 0);
 #ifdef RGLRU_TRACE
   a.trace = g_trace;
 #endif
