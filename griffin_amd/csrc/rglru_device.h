@@ -303,7 +303,7 @@ RGLRU_DEVICE float carry_lookback_from(const CarryBatch& first, const CarryChain
 //   fl     : RGLRU_FLAG_* bits of this token
 // ------------------------------------------------------------------------------------------
 struct GateOut {
-  float r, i, a, g, g2, z;   // a, g, z are post-mask; g2 = 1 - a_raw^2 is pre-mask
+  float r, i, a, g, g2, z;   // a, g, g2 = g * g and z include the token's masks
 };
 
 RGLRU_DEVICE float sigmoid_fast(float u) {
@@ -331,6 +331,18 @@ RGLRU_DEVICE float one_minus_exp(float y, float a) {
   }
 }
 
+// log2 of the decay under the token's flags.  Both masks of the reference act through it alone:
+//   padding (a <- 1, z <- 0): log2 a = 0 gives a = 1 and, through the series branch of
+//     one_minus_exp, g = 0 exactly, hence z = 0;
+//   reset (a <- 0, g <- 1): log2 a = -126 gives a = 2^-126 (the state it lets through is below
+//     1e-38 of its value) and g = sqrt(1 - a^2) = 1 exactly.
+// Padding wins when both are set, as in griffin/griffin.py:248-255.
+constexpr float kResetLog2 = -126.0f;
+RGLRU_DEVICE float masked_log2_decay(float l2, unsigned fl) {
+  l2 = (fl & 1u) ? kResetLog2 : l2;
+  return (fl & 2u) ? 0.0f : l2;
+}
+
 // MASKED = false: the token is known to be an ordinary one (no reset, active), fl is ignored.
 template <bool PRECISE, bool MASKED>
 RGLRU_DEVICE GateOut gate_forward(float ua, float ux, float x, float sp, unsigned fl) {
@@ -338,14 +350,12 @@ RGLRU_DEVICE GateOut gate_forward(float ua, float ux, float x, float sp, unsigne
   o.r = sigmoid_fast(ua);
   o.i = sigmoid_fast(ux);
   float l2 = o.r * sp;                         // log2(a) <= 0
-  float a = __builtin_amdgcn_exp2f(l2);
-  float g2 = fmaxf(one_minus_exp<PRECISE>(l2 * (2.0f * kLn2), a), 0.0f);
-  float g = __builtin_amdgcn_sqrtf(g2);
+  if constexpr (MASKED) l2 = masked_log2_decay(l2, fl);
+  const float a = __builtin_amdgcn_exp2f(l2);
+  const float g2 = fmaxf(one_minus_exp<PRECISE>(l2 * (2.0f * kLn2), a), 0.0f);
+  const float g = __builtin_amdgcn_sqrtf(g2);
   o.g2 = g2;
-  if constexpr (MASKED) { if (fl & 1u) { a = 0.f; g = 1.f; } }
-  float z = g * o.i * x;
-  if constexpr (MASKED) { if (fl & 2u) { a = 1.f; z = 0.f; } }
-  o.a = a; o.g = g; o.z = z;
+  o.a = a; o.g = g; o.z = g * o.i * x;
   return o;
 }
 

@@ -888,11 +888,9 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
 #pragma unroll
     for (int e = 0; e < EL; ++e) {
       const float re = sigmoid_fast(ua[e]);
-      float ae = __builtin_amdgcn_exp2f(re * sp);
-      if constexpr (MASKED) {                            // as in gate_forward: reset a = 0, then padding a = 1
-        if ((flbits >> (2 * e)) & 1u) ae = 0.f;
-        if ((flbits >> (2 * e)) & 2u) ae = 1.f;
-      }
+      float l2 = re * sp;
+      if constexpr (MASKED) l2 = masked_log2_decay(l2, (flbits >> (2 * e)) & 3u);
+      const float ae = __builtin_amdgcn_exp2f(l2);
       r[e] = re; a[e] = ae;
       A *= ae;
     }
@@ -917,14 +915,11 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
     float H = 0.f;
 #pragma unroll
     for (int e = 0; e < EL; ++e) {
-      const unsigned fl = MASKED ? ((flbits >> (2 * e)) & 3u) : 0u;
       const float ie = sigmoid_fast(ux[e]);
-      const float l2 = r[e] * sp;
-      const float a_raw = MASKED ? __builtin_amdgcn_exp2f(l2) : a[e];
-      float ge = __builtin_amdgcn_sqrtf(fmaxf(one_minus_exp<false>(l2 * (2.0f * kLn2), a_raw), 0.0f));
-      if constexpr (MASKED) { if (fl & 1u) ge = 1.f; }
-      float ze = ge * ie * xv[e];
-      if constexpr (MASKED) { if (fl & 2u) ze = 0.f; }
+      float l2 = r[e] * sp;
+      if constexpr (MASKED) l2 = masked_log2_decay(l2, (flbits >> (2 * e)) & 3u);     // gives g = 1 / g = 0
+      const float ge = __builtin_amdgcn_sqrtf(fmaxf(one_minus_exp<false>(l2 * (2.0f * kLn2), a[e]), 0.0f));
+      const float ze = ge * ie * xv[e];
       gi[e] = ie; g[e] = ge;
       H = fmaf(a[e], H, ze);
     }
@@ -956,11 +951,12 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
       const float a2 = a[e] * a[e];
       float dg2 = dg * __builtin_amdgcn_rsqf(fmaxf(4.0f * (g[e] * g[e]), 1e-6f));
       float dl = fmaf(d * h, a[e], -2.0f * a2 * dg2);
-      float ze = gx * gi[e];
-      if constexpr (MASKED) { if ((flbits >> (2 * e)) & 1u) dl = 0.f; }
+      const float ze = gx * gi[e];
+      // A reset token has a = 2^-126, which already switches dl off; a padded one has g = 0, which
+      // zeroes dxd, vx and z, but its bounded-sqrt term would leak into dl.
+      if constexpr (MASKED) { if ((flbits >> (2 * e)) & 2u) dl = 0.f; }
       float va = dl * cs * r[e] * (1.0f - r[e]);
       float vx = di * gi[e] * (1.0f - gi[e]);
-      if constexpr (MASKED) { if ((flbits >> (2 * e)) & 2u) { dl = 0.f; va = 0.f; vx = 0.f; dxd = 0.f; ze = 0.f; } }
       h = fmaf(a[e], h, ze);
       sum_l = fmaf(dl, r[e], sum_l);
       sum_ba += va; sum_bx += vx;
