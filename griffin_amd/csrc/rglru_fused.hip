@@ -941,24 +941,26 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
     unsigned char* my_du = stage_du + PairStage<TR>::row_offset(hf * EL) + w.r * 4;
 #pragma unroll
     for (int e = 0; e < EL; ++e) {
+      // With z = g i x, a = exp(l), g = sqrt(1 - a^2) (bounded derivative 1 / (2 max(g, 5e-4))):
+      //   dz = delta,  dx_direct = delta g i,  di = delta g x,  dl = delta a (h_{t-1} - 2 a i x / (2 g_b))
       const float d = gy[e];
       const float xe = xv[e];
-      const float gx = g[e] * xe;                        // dz/di
-      float dg = d * gi[e] * xe;
-      float di = d * gx;
-      float dxd = d * g[e] * gi[e];
-      // g = sqrt(g2) with the bounded derivative; a = exp(l), g2 = 1 - a^2 (= g * g off reset)
-      const float a2 = a[e] * a[e];
-      float dg2 = dg * __builtin_amdgcn_rsqf(fmaxf(4.0f * (g[e] * g[e]), 1e-6f));
-      float dl = fmaf(d * h, a[e], -2.0f * a2 * dg2);
-      const float ze = gx * gi[e];
+      // the factors below do not depend on delta; tying them to it keeps the compiler from computing
+      // all of them before the look-back, where they would only occupy registers
+      float ge = g[e], ie = gi[e], re = r[e];
+      asm volatile("" : "+v"(ge), "+v"(ie), "+v"(re) : "v"(d));
+      const float c1 = ge * ie;
+      const float dxd = d * c1;
+      const float ze = c1 * xe;
+      const float q = (ie * xe) * __builtin_amdgcn_rsqf(fmaxf(4.0f * (ge * ge), 1e-6f));
+      float dl = (a[e] * d) * fmaf(-2.0f * a[e], q, h);
       // A reset token has a = 2^-126, which already switches dl off; a padded one has g = 0, which
       // zeroes dxd, vx and z, but its bounded-sqrt term would leak into dl.
       if constexpr (MASKED) { if ((flbits >> (2 * e)) & 2u) dl = 0.f; }
-      float va = dl * cs * r[e] * (1.0f - r[e]);
-      float vx = di * gi[e] * (1.0f - gi[e]);
+      const float va = dl * (cs * fmaf(-re, re, re));
+      const float vx = (d * ze) * (1.0f - ie);
       h = fmaf(a[e], h, ze);
-      sum_l = fmaf(dl, r[e], sum_l);
+      sum_l = fmaf(dl, re, sum_l);
       sum_ba += va; sum_bx += vx;
       *reinterpret_cast<IO*>(my_dx + e * WaveStage<TR>::kRowBytes) = (IO)dxd;
       typedef IO io2 __attribute__((ext_vector_type(2)));
