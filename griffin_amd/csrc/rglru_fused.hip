@@ -31,6 +31,7 @@ struct PrepArgs {
   void* wg; float* bias; float* sp; float* cs; float* dsp; void* w2t;
   int W, nb, bw, bwp, Wp, vec_dtype;
   float c;
+  uint4* clear; long long clear_n;     // optional: a workspace region to zero in the same launch
 };
 
 // Element i of a vector stored as fp32 or bf16 (RGLRU_F32 / RGLRU_BF16).
@@ -52,6 +53,7 @@ __global__ void prepare_kernel(PrepArgs p) {
   const long long total = 2 * n_w + p.Wp;
   long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x;
   const long long stride = (long long)gridDim.x * blockDim.x;
+  for (long long z = i; z < p.clear_n; z += stride) p.clear[z] = make_uint4(0u, 0u, 0u, 0u);
   for (; i < total; i += stride) {
     if (i < n_w) {
       int gate = (int)(i / per_gate);
@@ -1447,9 +1449,9 @@ size_t rglru_hip_prep_bytes(int64_t W, int64_t nb, int dtype) {
   return make_prep_layout(make_geometry(W, nb), elem_size(dtype)).total;
 }
 
-int rglru_hip_prepare(const void* w_a, const void* b_a, const void* w_x, const void* b_x,
-                      const void* lambda, float c, int64_t W, int64_t nb, int dtype, int vec_dtype,
-                      void* prep, void* stream) {
+static int prepare_impl(const void* w_a, const void* b_a, const void* w_x, const void* b_x,
+                        const void* lambda, float c, int64_t W, int64_t nb, int dtype, int vec_dtype,
+                        void* prep, void* clear, size_t clear_bytes, void* stream) {
   int rc = check_geometry("prepare", W, nb, dtype);
   if (rc) return rc;
   if (vec_dtype != RGLRU_F32 && vec_dtype != RGLRU_BF16) return fail(RGLRU_E_ARG, "prepare: unknown vector dtype %d", vec_dtype);
@@ -1463,12 +1465,20 @@ int rglru_hip_prepare(const void* w_a, const void* b_a, const void* w_x, const v
   a.dsp = (float*)(pb + pl.dsp); a.vec_dtype = vec_dtype;
   a.w2t = pb + pl.w2t;
   a.W = (int)W; a.nb = (int)nb; a.bw = (int)g.bw; a.bwp = (int)g.bwp; a.Wp = (int)g.Wp; a.c = c;
+  a.clear = (uint4*)clear; a.clear_n = (long long)(clear_bytes / 16);
   long long total = 4 * g.nb * g.bwp * g.bwp + g.Wp;
+  if (a.clear_n > total) total = a.clear_n;
   int blocks = (int)((total + 255) / 256); if (blocks > 2048) blocks = 2048;
   hipStream_t s = (hipStream_t)stream;
   if (dtype == RGLRU_BF16) hipLaunchKernelGGL(prepare_kernel<__bf16>, dim3(blocks), dim3(256), 0, s, a);
   else hipLaunchKernelGGL(prepare_kernel<float>, dim3(blocks), dim3(256), 0, s, a);
   return check_launch("prepare");
+}
+
+int rglru_hip_prepare(const void* w_a, const void* b_a, const void* w_x, const void* b_x,
+                      const void* lambda, float c, int64_t W, int64_t nb, int dtype, int vec_dtype,
+                      void* prep, void* stream) {
+  return prepare_impl(w_a, b_a, w_x, b_x, lambda, c, W, nb, dtype, vec_dtype, prep, nullptr, 0, stream);
 }
 
 size_t rglru_hip_workspace_bytes(int64_t B, int64_t T, int64_t W, int64_t nb) {
@@ -1481,9 +1491,9 @@ size_t rglru_hip_bwd_scratch_bytes(int64_t B, int64_t T, int64_t W, int64_t nb, 
   return make_scratch_layout(B, T, make_geometry(W, nb), rglru_hip_fast_path(W, nb, dtype) != 0).total;
 }
 
-int rglru_hip_fwd(const void* x, const void* prep, const float* h0, const uint8_t* flags,
-                  void* y, float* h_last, void* ws,
-                  int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, void* stream) {
+static int fwd_impl(const void* x, const void* prep, const float* h0, const uint8_t* flags,
+                    void* y, float* h_last, void* ws,
+                    int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, bool cleared, void* stream) {
   int rc = check_geometry("fwd", W, nb, dtype);
   if (rc) return rc;
   if (B <= 0 || T <= 0) return fail(RGLRU_E_ARG, "fwd: B and T must be positive (got %lld, %lld)", (long long)B, (long long)T);
@@ -1493,8 +1503,10 @@ int rglru_hip_fwd(const void* x, const void* prep, const float* h0, const uint8_
   WorkLayout L = make_work_layout(B, T, g);
   hipStream_t s = (hipStream_t)stream;
   char* wb = (char*)ws;
-  rc = launch_clear(wb, L.f_begin, L.b_end, s);         // carry records and tickets of both passes, failure word
-  if (rc) return rc;
+  if (!cleared) {
+    rc = launch_clear(wb, L.f_begin, L.b_end, s);       // carry records and tickets of both passes, failure word
+    if (rc) return rc;
+  }
   FusedArgs a;
   memset(&a, 0, sizeof(a));
   fill_common(a, g, prep, dtype);
@@ -1517,6 +1529,28 @@ int rglru_hip_fwd(const void* x, const void* prep, const float* h0, const uint8_
     RGLRU_DISPATCH_FWD(grid, s, a, dtype, held_groups(g, dtype, a.aligned), masked);
   }
   return check_launch("fwd");
+}
+
+int rglru_hip_fwd(const void* x, const void* prep, const float* h0, const uint8_t* flags,
+                  void* y, float* h_last, void* ws,
+                  int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, void* stream) {
+  return fwd_impl(x, prep, h0, flags, y, h_last, ws, B, T, W, nb, dtype, false, stream);
+}
+
+int rglru_hip_prepare_fwd(const void* w_a, const void* b_a, const void* w_x, const void* b_x,
+                          const void* lambda, float c, int vec_dtype, void* prep,
+                          const void* x, const float* h0, const uint8_t* flags,
+                          void* y, float* h_last, void* ws,
+                          int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, void* stream) {
+  int rc = check_geometry("prepare_fwd", W, nb, dtype);
+  if (rc) return rc;
+  if (B <= 0 || T <= 0) return fail(RGLRU_E_ARG, "prepare_fwd: B and T must be positive (got %lld, %lld)", (long long)B, (long long)T);
+  if (!ws) return fail(RGLRU_E_ARG, "prepare_fwd: null pointer");
+  // one launch converts the parameters and zeroes the records, tickets and failure word of `ws`
+  const WorkLayout L = make_work_layout(B, T, make_geometry(W, nb));
+  rc = prepare_impl(w_a, b_a, w_x, b_x, lambda, c, W, nb, dtype, vec_dtype, prep, (char*)ws + L.f_begin, L.b_end - L.f_begin, stream);
+  if (rc) return rc;
+  return fwd_impl(x, prep, h0, flags, y, h_last, ws, B, T, W, nb, dtype, true, stream);
 }
 
 static int check_grad_dtype(const char* who, int grad_dtype) {

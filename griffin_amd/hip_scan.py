@@ -130,6 +130,24 @@ def pack_flags(reset_mask: Tensor | None, active_mask: Tensor | None) -> Tensor 
     return None if flags is None else flags.contiguous()
 
 
+def _parameter_operands(w_a: Tensor, b_a: Tensor, w_x: Tensor, b_x: Tensor, lam: Tensor, dtype: torch.dtype):
+    """The five parameters as the library reads them: gate weights in the storage type; biases and
+    Lambda in their own type when the library knows it (fp32 or bf16), so the usual cases launch no
+    conversion kernels.  Returns the tensors (kept alive by the caller) and the vector dtype code."""
+    vec_dtype = b_a.dtype if (b_a.dtype == b_x.dtype == lam.dtype and b_a.dtype in _DTYPE_CODES) else torch.float32
+    tensors = (w_a.detach().to(dtype).contiguous(), b_a.detach().to(vec_dtype).contiguous(),
+               w_x.detach().to(dtype).contiguous(), b_x.detach().to(vec_dtype).contiguous(),
+               lam.detach().to(vec_dtype).contiguous())
+    return tensors, _DTYPE_CODES[vec_dtype]
+
+
+def _prep_bytes(width: int, blocks: int, code: int) -> int:
+    size = _lib.load().rglru_hip_prep_bytes(width, blocks, code)
+    if size == 0:
+        _lib.check(2, "rglru_hip_prep_bytes")
+    return size
+
+
 class PreparedParams:
     """Kernel-side image of the RG-LRU parameters (see rglru_hip_prepare)."""
 
@@ -141,22 +159,12 @@ class PreparedParams:
         self.dtype = dtype
         self.c = float(c)
         code = _dtype_code(dtype)
-        size = lib.rglru_hip_prep_bytes(self.width, nb, code)
-        if size == 0:
-            _lib.check(2, "rglru_hip_prep_bytes")
+        size = _prep_bytes(self.width, nb, code)
         device = w_a.device
-        # gate weights in the storage type; biases and Lambda are read in their own type when the
-        # library knows it (fp32 or bf16), so the usual cases launch no conversion kernels
-        w_a_c = w_a.detach().to(dtype).contiguous()
-        w_x_c = w_x.detach().to(dtype).contiguous()
-        vec_dtype = b_a.dtype if (b_a.dtype == b_x.dtype == lam.dtype and b_a.dtype in _DTYPE_CODES) else torch.float32
-        b_a_c = b_a.detach().to(vec_dtype).contiguous()
-        b_x_c = b_x.detach().to(vec_dtype).contiguous()
-        lam_c = lam.detach().to(vec_dtype).contiguous()
+        operands, vec_code = _parameter_operands(w_a, b_a, w_x, b_x, lam, dtype)
         with torch.cuda.device(device):
             self.image = torch.empty(size, dtype=torch.uint8, device=device)
-            _lib.check(lib.rglru_hip_prepare(w_a_c.data_ptr(), b_a_c.data_ptr(), w_x_c.data_ptr(), b_x_c.data_ptr(),
-                                             lam_c.data_ptr(), self.c, self.width, nb, code, _DTYPE_CODES[vec_dtype],
+            _lib.check(lib.rglru_hip_prepare(*(t.data_ptr() for t in operands), self.c, self.width, nb, code, vec_code,
                                              self.image.data_ptr(), _stream_ptr(device)), "rglru_hip_prepare")
 
 
@@ -188,17 +196,20 @@ class _HipRGLRU(torch.autograd.Function):
         B, T, W = x.shape
         nb = w_a.shape[0]
         code = _dtype_code(x.dtype)
-        prep = PreparedParams(w_a, b_a, w_x, b_x, lam, c, x.dtype)
+        operands, vec_code = _parameter_operands(w_a, b_a, w_x, b_x, lam, x.dtype)
         h0c = None if h0 is None else h0.detach().to(torch.float32).contiguous()
         device = x.device
         with torch.cuda.device(device):
             y = torch.empty_like(x)
             h_last = torch.empty(B, W, dtype=torch.float32, device=device)
+            image = torch.empty(_prep_bytes(W, nb, code), dtype=torch.uint8, device=device)
             ws = torch.empty(lib.rglru_hip_workspace_bytes(B, T, W, nb), dtype=torch.uint8, device=device)
-            _lib.check(lib.rglru_hip_fwd(x.data_ptr(), prep.image.data_ptr(), _ptr(h0c), _ptr(flags), y.data_ptr(),
-                                         h_last.data_ptr(), ws.data_ptr(), B, T, W, nb, code, _stream_ptr(device)),
-                       "rglru_hip_fwd")
-        ctx.save_for_backward(x, w_a, w_x, h0c, flags, ws, prep.image)
+            # parameter conversion, workspace clearing and the forward kernel: two launches
+            _lib.check(lib.rglru_hip_prepare_fwd(*(t.data_ptr() for t in operands), float(c), vec_code, image.data_ptr(),
+                                                 x.data_ptr(), _ptr(h0c), _ptr(flags), y.data_ptr(), h_last.data_ptr(),
+                                                 ws.data_ptr(), B, T, W, nb, code, _stream_ptr(device)),
+                       "rglru_hip_prepare_fwd")
+        ctx.save_for_backward(x, w_a, w_x, h0c, flags, ws, image)
         ctx.param_dtypes = (w_a.dtype, b_a.dtype, w_x.dtype, b_x.dtype, lam.dtype)
         ctx.h0_dtype = None if h0 is None else h0.dtype
         ctx.set_materialize_grads(False)      # an unused output arrives as None, not as a tensor of zeros

@@ -103,6 +103,16 @@ int rglru_hip_fwd(const void* x, const void* prep, const float* h0, const uint8_
                   void* y, float* h_last, void* ws,
                   int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, void* stream);
 
+/* rglru_hip_prepare followed by rglru_hip_fwd on the same stream with one launch fewer: the
+ * parameter conversion and the clearing of the workspace share a kernel.  For training, where
+ * every forward (griffin/griffin.py:237-289) sees freshly updated parameters; `prep` is written
+ * and stays valid for the matching backward call. */
+int rglru_hip_prepare_fwd(const void* w_a, const void* b_a, const void* w_x, const void* b_x,
+                          const void* lambda, float c, int vec_dtype, void* prep,
+                          const void* x, const float* h0, const uint8_t* flags,
+                          void* y, float* h_last, void* ws,
+                          int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, void* stream);
+
 /* Backward of rglru_hip_fwd.  Recomputes the gates and the decay from x (nothing but the chunk
  * checkpoints in `ws` is kept from forward).  dy[B,T,W] (dtype); dh_last[B,W] fp32 or NULL.
  * Outputs: dx[B,T,W] (dtype) receives only the direct path dL/dz * g * i; du_a, du_x [B,T,W]
