@@ -124,6 +124,7 @@ struct FusedArgs {
   unsigned* fail; float* partial; float* dw_partial;
   // geometry
   int B, T, W, nb, bw, bwp, S, Wp, groups, units;
+  int bpu;                                                // gate blocks per unit (packed narrow blocks), else 1
   int nC, nCf, ckpt_nC, wg_per_unit, aligned, full_slabs, queues, flags_vec;
   long long limit;
 #ifdef RGLRU_TRACE
@@ -150,16 +151,31 @@ RGLRU_DEVICE Queue make_queue(const FusedArgs& p, int unit, int wg_in_unit, int 
 // Identity of the wave inside its unit; shared by the kernels below.
 struct WaveId {
   int lane, r, hf, wave, unit, wg_in_unit, k, slab, o, ch, kp;
+  int tile_col, kb;          // first channel of the unit's x tile; offset of the wave's block inside it
   bool slab_ok, ch_ok;
 };
+
+// Width of the x tile of the kernels with register-held weights.  Blocks of 64 or 32 channels are
+// packed two or four to a unit, so the four waves of a workgroup always have a slab each.
+constexpr int kPackedWidth = 128;
 
 RGLRU_DEVICE WaveId wave_identity(const FusedArgs& p, int block) {
   WaveId w;
   w.lane = threadIdx.x & 63; w.r = w.lane & 31; w.hf = w.lane >> 5; w.wave = threadIdx.x >> 6;
   w.unit = block % p.units; w.wg_in_unit = block / p.units;
-  w.k = w.unit / p.groups;
-  w.slab = (w.unit % p.groups) * kWaves + w.wave;
-  w.slab_ok = w.slab < p.S;
+  if (p.bpu > 1) {
+    // packed: the unit covers bpu consecutive blocks of S slabs each (bpu * S = waves per workgroup)
+    const int blk = w.wave / p.S, k = w.unit * p.bpu + blk;
+    w.slab = w.wave - blk * p.S;
+    w.slab_ok = k < p.nb;
+    w.k = w.slab_ok ? k : p.nb - 1;
+    w.tile_col = w.unit * p.bpu * p.bw; w.kb = blk * p.bw;
+  } else {
+    w.k = w.unit / p.groups;
+    w.slab = (w.unit % p.groups) * kWaves + w.wave;
+    w.slab_ok = w.slab < p.S;
+    w.tile_col = w.k * p.bw; w.kb = 0;
+  }
   w.o = w.slab * 32 + w.r;
   w.ch_ok = w.slab_ok && w.o < p.bw;
   w.ch = w.k * p.bw + (w.ch_ok ? w.o : 0);
@@ -258,16 +274,16 @@ struct HeldWeights {
 // MFMA phase for register-held weights, one accumulator tile: the whole block width (NKG * KG
 // columns) is in LDS with row stride NKG * KG + HW.  Also returns the 16 x values of the tile in
 // accumulator layout.
-template <typename IO, int MT, int NKG>
+template <typename IO, int MT, int NKG, int TW = NKG * Io<IO>::KG>
 RGLRU_DEVICE void gate_mfma_held(const IO* lds, const HeldWeights<IO, NKG>& hw, int mt, int slab, int r, int hf,
-                                 float bias_a, float bias_x, f32x16& ua, f32x16& ux, float (&xv)[16]) {
+                                 float bias_a, float bias_x, f32x16& ua, f32x16& ux, float (&xv)[16], int kb = 0) {
   typedef Io<IO> Tr;
   typedef typename Tr::Frag Frag;
   constexpr int KG = Tr::KG, HW = Tr::HW;
-  constexpr int LDSROW = NKG * KG + HW;
+  constexpr int LDSROW = TW + HW;                          // the tile is TW columns wide; the block starts at kb
 #pragma unroll
   for (int v = 0; v < 16; ++v) { ua[v] = bias_a; ux[v] = bias_x; }
-  const IO* row = lds + tile_row<MT>(mt, r) * LDSROW + hf * HW;
+  const IO* row = lds + tile_row<MT>(mt, r) * LDSROW + kb + hf * HW;
 #pragma unroll
   for (int kg = 0; kg < NKG; ++kg) {
     Frag xa = *reinterpret_cast<const Frag*>(row + kg * KG);
@@ -275,7 +291,7 @@ RGLRU_DEVICE void gate_mfma_held(const IO* lds, const HeldWeights<IO, NKG>& hw, 
     Tr::mma(ux, xa, hw.x[kg]);
   }
 #pragma unroll
-  for (int e = 0; e < 16; ++e) xv[e] = (float)lds[(hf * 16 * MT + 16 * mt + e) * LDSROW + slab * 32 + r];
+  for (int e = 0; e < 16; ++e) xv[e] = (float)lds[(hf * 16 * MT + 16 * mt + e) * LDSROW + kb + slab * 32 + r];
 }
 
 RGLRU_DEVICE unsigned token_flag(const FusedArgs& p, long long token_row, bool inside) {
@@ -437,7 +453,7 @@ __global__ __launch_bounds__(kThreads, 2) void fwd_kernel(FusedArgs p) {
   constexpr int MT = kFwdMT, TR = 32 * MT, EL = 16 * MT;
   typedef Io<IO> Tr;
   typedef typename Tr::Frag Frag;
-  constexpr int KC = NKG > 0 ? NKG * Tr::KG : Tr::KCMAX;           // LDS tile width in elements
+  constexpr int KC = NKG > 0 ? kPackedWidth : Tr::KCMAX;           // LDS tile width in elements
   constexpr int LDSROW = KC + Tr::HW;
   __shared__ __attribute__((aligned(16))) IO lds[TR * LDSROW];
   __shared__ __attribute__((aligned(16))) unsigned char stage_all[kWaves * WaveStage<TR>::kBytes];
@@ -469,7 +485,7 @@ __global__ __launch_bounds__(kThreads, 2) void fwd_kernel(FusedArgs p) {
     for (int i = 0; i < NV; ++i) {
       const int idx = tid + i * kThreads;
       const int row = idx / VPR, cv = idx - row * VPR;
-      pre_off[i] = (idx < TR * VPR) ? (unsigned)row * row_bytes + (unsigned)(w.k * p.bw + cv * Tr::HW) * (unsigned)sizeof(IO)
+      pre_off[i] = (idx < TR * VPR) ? (unsigned)row * row_bytes + (unsigned)(w.tile_col + cv * Tr::HW) * (unsigned)sizeof(IO)
                                     : kOutOfRange;
     }
     auto issue = [&](long long tk_in) {
@@ -497,7 +513,7 @@ __global__ __launch_bounds__(kThreads, 2) void fwd_kernel(FusedArgs p) {
 #pragma unroll
     for (int e = 0; e < EL; ++e) { prev.a[e] = 0.f; prev.z[e] = 0.f; }
     prev.A_lo = prev.H_lo = prev.A_t = prev.H_t = 0.f;
-    // a gate block of 128 channels fills all four waves; narrower ones leave waves without a slab
+    // every wave has a slab except in the last unit of a block count that does not fill it
     const bool slab_ok = (NKG == 8) ? true : w.slab_ok;
     const rsrc_t rticket = make_rsrc(q.counter, 4u);
     const unsigned rec_stride = (unsigned)W * 8u;
@@ -529,7 +545,7 @@ __global__ __launch_bounds__(kThreads, 2) void fwd_kernel(FusedArgs p) {
         for (int mt = 0; mt < MT; ++mt) {
           f32x16 ua, ux;
           float xv[16];
-          gate_mfma_held<IO, MT, NKG>(lds, hw, mt, w.slab, w.r, hf, bias_a, bias_x, ua, ux, xv);
+          gate_mfma_held<IO, MT, NKG, KC>(lds, hw, mt, w.slab, w.r, hf, bias_a, bias_x, ua, ux, xv, NKG == 8 ? 0 : w.kb);
           fwd_gates<IO, MASKED>(p, trow + 16 * mt, cur.c * TR + hf * EL + 16 * mt, ua, ux, xv, sp, cur.a + 16 * mt, cur.z + 16 * mt);
         }
       }
@@ -749,8 +765,9 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
   constexpr int MT = 1, TR = 32, EL = 16;
   typedef Io<IO> Tr;
   typedef typename Tr::Frag Frag;
-  constexpr int KC = NKG * Tr::KG;
-  constexpr int LDSROW = KC + Tr::HW;
+  constexpr int KC = NKG * Tr::KG;                       // block width
+  constexpr int TW = kPackedWidth;                       // tile width (narrow blocks are packed)
+  constexpr int LDSROW = TW + Tr::HW;
   static_assert(sizeof(IO) == 2 && NKG > 0, "fast backward is for 16-bit storage with held weights");
   __shared__ __attribute__((aligned(16))) IO lds_x[TR * LDSROW];
   __shared__ __attribute__((aligned(16))) IO lds_dy[TR * LDSROW];
@@ -794,7 +811,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
   float sum_ba = 0.f, sum_bx = 0.f, sum_l = 0.f;
   const Queue q = make_queue(p, w.unit, w.wg_in_unit, p.nC);
 
-  constexpr int VPR = KC / Tr::HW;
+  constexpr int VPR = TW / Tr::HW;
   constexpr int NV = (TR * VPR + kThreads - 1) / kThreads;
   Frag pre_x[NV], pre_dy[NV];
   unsigned pre_off[NV];
@@ -802,7 +819,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
   for (int i = 0; i < NV; ++i) {
     const int idx = tid + i * kThreads;
     const int row = idx / VPR, cv = idx - row * VPR;
-    pre_off[i] = (idx < TR * VPR) ? (unsigned)row * row_bytes + (unsigned)(w.k * p.bw + cv * Tr::HW) * 2u : kOutOfRange;
+    pre_off[i] = (idx < TR * VPR) ? (unsigned)row * row_bytes + (unsigned)(w.tile_col + cv * Tr::HW) * 2u : kOutOfRange;
   }
   auto decode = [&](unsigned tk, int& c, int& b) {
     const unsigned cr = tk / (unsigned)q.n_b;
@@ -865,10 +882,10 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
 #pragma unroll
         for (int e = 0; e < EL; ++e) xv[e] = (float)lds_x[(hf * EL + e) * LDSROW + w.slab * 32 + w.r];
       } else {
-        gate_mfma_held<IO, MT, NKG>(lds_x, hw, 0, w.slab, w.r, hf, bias_a, bias_x, ua, ux, xv);
+        gate_mfma_held<IO, MT, NKG, TW>(lds_x, hw, 0, w.slab, w.r, hf, bias_a, bias_x, ua, ux, xv, w.kb);
       }
 #pragma unroll
-      for (int e = 0; e < EL; ++e) gy[e] = (float)lds_dy[(hf * EL + e) * LDSROW + w.slab * 32 + w.r];
+      for (int e = 0; e < EL; ++e) gy[e] = (float)lds_dy[(hf * EL + e) * LDSROW + (NKG == 8 ? 0 : w.kb) + w.slab * 32 + w.r];
     }
     if (tid == 0) s_ticket[par ^ 1] = next_raw;
     __syncthreads();
@@ -1350,7 +1367,7 @@ static void fill_common(FusedArgs& a, const Geometry& g, const void* prep, int d
   a.wg = pb + pl.wg; a.bias = (const float*)(pb + pl.bias); a.sp = (const float*)(pb + pl.sp); a.cs = (const float*)(pb + pl.cs);
   a.w2t = pb + pl.w2t;
   a.W = (int)g.W; a.nb = (int)g.nb; a.bw = (int)g.bw; a.bwp = (int)g.bwp; a.S = (int)g.S; a.Wp = (int)g.Wp;
-  a.groups = (int)g.groups; a.units = (int)g.units;
+  a.groups = (int)g.groups; a.units = (int)g.units; a.bpu = 1;
   a.limit = spin_limit();
   a.full_slabs = (g.bw % 32 == 0) ? 1 : 0;
 }
@@ -1422,9 +1439,17 @@ struct KernelTimer {
   ~KernelTimer() { if (slot) { hipEventRecord(slot->stop, stream); slot->armed = true; } }
 };
 
-static int pick_wg_per_unit(const Geometry& g, long long tiles_per_unit, int per_cu, long long cap) {
+// Narrow blocks of the kernels with register-held weights share a unit (see kPackedWidth).
+static void pack_units(FusedArgs& a, const Geometry& g, int nkg) {
+  if (nkg == 4 || nkg == 2) {
+    a.bpu = kPackedWidth / (int)g.bw;
+    a.units = (int)((g.nb + a.bpu - 1) / a.bpu);
+  }
+}
+
+static int pick_wg_per_unit(int units, long long tiles_per_unit, int per_cu, long long cap) {
   long long target = (long long)num_compute_units() * per_cu;
-  long long n = (target + g.units - 1) / g.units;
+  long long n = (target + units - 1) / units;
   if (n > tiles_per_unit) n = tiles_per_unit;
   if (n > cap) n = cap;
   if (n < 1) n = 1;
@@ -1520,13 +1545,15 @@ static int fwd_impl(const void* x, const void* prep, const float* h0, const uint
 #ifdef RGLRU_TRACE
   a.trace = g_trace;
 #endif
-  a.wg_per_unit = pick_wg_per_unit(g, B * (long long)a.nCf, 2, 1 << 20);
+  const int nkg = held_groups(g, dtype, a.aligned);
+  pack_units(a, g, nkg);
+  a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nCf, 2, 1 << 20);
   a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
-  dim3 grid((unsigned)(a.wg_per_unit * g.units));
+  dim3 grid((unsigned)(a.wg_per_unit * a.units));
   {
     KernelTimer timer(0, s);
     const int masked = (flags != nullptr) || (T % (32 * kFwdMT) != 0);
-    RGLRU_DISPATCH_FWD(grid, s, a, dtype, held_groups(g, dtype, a.aligned), masked);
+    RGLRU_DISPATCH_FWD(grid, s, a, dtype, nkg, masked);
   }
   return check_launch("fwd");
 }
@@ -1586,9 +1613,9 @@ int rglru_hip_bwd(const void* x, const void* prep, const float* h0,
   a.partial = (float*)((char*)scratch + make_scratch_layout(B, T, g, false).partial);
   a.B = (int)B; a.T = (int)T; a.nC = (int)((T + kChunk - 1) / kChunk); a.ckpt_nC = (int)L.nC; a.nCf = (int)L.nCf;
   a.aligned = is_aligned(x, W, g.bw, elem_size(dtype));
-  a.wg_per_unit = pick_wg_per_unit(g, B * (long long)a.nC, 2, L.max_wg);
+  a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nC, 2, L.max_wg);
   a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
-  dim3 grid((unsigned)(a.wg_per_unit * g.units));
+  dim3 grid((unsigned)(a.wg_per_unit * a.units));
   {
     KernelTimer timer(1, s);
     RGLRU_DISPATCH(bwd_kernel, grid, s, a, dtype, held_groups(g, dtype, a.aligned));
@@ -1645,11 +1672,12 @@ int rglru_hip_bwd_full(const void* x, const void* prep, const float* h0,
   a.partial = (float*)(sb + SL.partial); a.dw_partial = (float*)(sb + SL.dw_partial);
   a.B = (int)B; a.T = (int)T; a.nC = (int)((T + kChunk - 1) / kChunk); a.ckpt_nC = (int)L.nC;
   a.aligned = 1;
-  a.wg_per_unit = pick_wg_per_unit(g, B * (long long)a.nC, 2, L.max_wg);
-  a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
   const int nkg = held_groups(g, dtype, 1);
+  pack_units(a, g, nkg);
+  a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nC, 2, L.max_wg);
+  a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
   const bool masked = (flags != nullptr) || (T % kChunk != 0);
-  dim3 grid((unsigned)(a.wg_per_unit * g.units));
+  dim3 grid((unsigned)(a.wg_per_unit * a.units));
   {
     KernelTimer timer(1, s);
 #define RGLRU_LAUNCH_SCAN(N)                                                                              \

@@ -114,7 +114,10 @@ BF16_CASES = [
     (2, 80, 256, 2, True, False),    # length a multiple of 16 but not of 32: vector flag loads, half-empty tile
     (1, 700, 128, 1, True, True),    # one sequence: every workgroup of the block works on the same chain
     (70, 40, 128, 1, False, False),  # more sequences than ticket queues
-    (3, 17, 128, 2, True, True),     # shorter than one tile
+    (3, 17, 128, 2, True, True),     # shorter than one tile    (2, 100, 192, 3, True, True),    # 64-wide blocks packed two to a unit, last unit half empty
+    (2, 70, 96, 3, False, True),     # 32-wide blocks packed four to a unit, last unit one block short
+    (1, 64, 64, 1, False, False),    # a single 64-wide block: half of the packed unit idles
+    (2, 64, 1024, 16, True, False),  # reference default of 16 gate blocks at width 1024
 ]
 
 
