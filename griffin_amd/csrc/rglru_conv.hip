@@ -1,0 +1,392 @@
+// Causal depthwise temporal convolution in front of the RG-LRU (griffin/griffin.py:474-487, the
+// all-tokens-active path of RecurrentBlock.forward), forward and backward.
+//
+//   out[b,t,c] = bias[c] + sum_{lag<K} taps[c][K-1-lag] * [segment_pos[b,t] >= lag] * padded[b,t-lag,c]
+//
+// where padded is the K-1 rows of carried state followed by the T rows of the input.  The work is
+// pure streaming: a thread owns V consecutive channels (one 16-byte vector, or one element when
+// the rows are not 16-byte aligned) and a run of consecutive tokens of one sequence, keeps the last
+// K-1 rows in registers and touches every input and output element once.  All global accesses go
+// through buffer descriptors of one sequence: rows past its end read as zero and stores to them
+// are dropped, so the token loops carry no bounds branches.
+
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+#include <initializer_list>
+
+#include "rglru_device.h"
+#include "rglru_host.h"
+
+namespace rglru {
+
+constexpr int kConvMaxTaps = 4;        // kernel sizes 1..4 (the reference uses 4)
+constexpr int kConvRunFwd = 16;        // tokens per thread, forward
+constexpr int kConvRunBwd = 32;        // tokens per thread, backward (one partial sum per run)
+constexpr int kConvThreads = 256;
+
+struct ConvArgs {
+  const void* u; const void* state; const void* taps; const void* bias; const long long* segpos;
+  void* out; void* new_state;                               // forward
+  const void* dout; void* du; void* dstate; float* partial;  // backward
+  int B, T, W, K, nvec, runs, vec_dtype;
+};
+
+// V values of one row, as floats.
+template <typename IO, int V> struct ConvRow;
+template <> struct ConvRow<__bf16, 8> {
+  static RGLRU_DEVICE void load(float (&v)[8], rsrc_t r, unsigned off) {
+    const bf16x8 f = buf_load_frag<bf16x8>(r, off);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = (float)f[i];
+  }
+  static RGLRU_DEVICE void store(const float (&v)[8], rsrc_t r, unsigned off) {
+    bf16x8 f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) f[i] = (__bf16)v[i];
+    buf_store_b128(__builtin_bit_cast(i32x4, f), r, off);
+  }
+};
+template <> struct ConvRow<float, 4> {
+  static RGLRU_DEVICE void load(float (&v)[4], rsrc_t r, unsigned off) {
+    const f32x4 f = buf_load_frag<f32x4>(r, off);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = f[i];
+  }
+  static RGLRU_DEVICE void store(const float (&v)[4], rsrc_t r, unsigned off) {
+    f32x4 f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) f[i] = v[i];
+    buf_store_b128(__builtin_bit_cast(i32x4, f), r, off);
+  }
+};
+template <typename IO> struct ConvRow<IO, 1> {
+  static RGLRU_DEVICE void load(float (&v)[1], rsrc_t r, unsigned off) { v[0] = BufIo<IO>::load(r, off, 0u); }
+  static RGLRU_DEVICE void store(const float (&v)[1], rsrc_t r, unsigned off) { BufIo<IO>::store((IO)v[0], r, off, 0u); }
+};
+
+RGLRU_DEVICE float conv_param(const void* base, long long i, int vec_dtype) {
+  return vec_dtype == RGLRU_BF16 ? (float)((const __bf16*)base)[i] : ((const float*)base)[i];
+}
+
+// Which (sequence, run, channel vector) a thread owns; vectors vary fastest, so the lanes of a wave
+// read consecutive addresses of one row.
+struct ConvItem { int b, run, c0; bool ok; };
+RGLRU_DEVICE ConvItem conv_item(const ConvArgs& p) {
+  ConvItem it;
+  const long long item = (long long)blockIdx.x * kConvThreads + threadIdx.x;
+  it.ok = item < (long long)p.B * p.runs * p.nvec;
+  const long long safe = it.ok ? item : 0;
+  const int vec = (int)(safe % p.nvec);
+  const long long rest = safe / p.nvec;
+  it.run = (int)(rest % p.runs); it.b = (int)(rest / p.runs);
+  it.c0 = vec * (p.W / p.nvec);
+  return it;
+}
+
+// Row `t` of the padded input of sequence b (t < 0: carried state, zeros when there is none).
+template <typename IO, int V, int K>
+RGLRU_DEVICE void padded_row(const ConvArgs& p, rsrc_t ru, int b, int t, int c0, float (&v)[V]) {
+  if (t >= 0) {
+    ConvRow<IO, V>::load(v, ru, ((unsigned)t * (unsigned)p.W + (unsigned)c0) * (unsigned)sizeof(IO));
+  } else if (p.state && K - 1 + t >= 0) {
+    const rsrc_t rs = make_rsrc((const IO*)p.state + (long long)b * (K - 1) * p.W, (unsigned)((K - 1) * p.W) * (unsigned)sizeof(IO));
+    ConvRow<IO, V>::load(v, rs, ((unsigned)(K - 1 + t) * (unsigned)p.W + (unsigned)c0) * (unsigned)sizeof(IO));
+  } else {
+#pragma unroll
+    for (int i = 0; i < V; ++i) v[i] = 0.f;
+  }
+}
+
+template <typename IO, int V, int K>
+__global__ __launch_bounds__(kConvThreads) void conv_fwd_kernel(ConvArgs p) {
+  const ConvItem it = conv_item(p);
+  if (!it.ok) return;
+  const int b = it.b, c0 = it.c0, t0 = it.run * kConvRunFwd;
+  const unsigned es = (unsigned)sizeof(IO), uW = (unsigned)p.W;
+  float tap[K][V], bias[V];
+#pragma unroll
+  for (int v = 0; v < V; ++v) {
+    bias[v] = p.bias ? conv_param(p.bias, c0 + v, p.vec_dtype) : 0.f;
+#pragma unroll
+    for (int j = 0; j < K; ++j) tap[j][v] = conv_param(p.taps, (long long)(c0 + v) * K + j, p.vec_dtype);
+  }
+  const unsigned seq_bytes = (unsigned)p.T * uW * es;
+  const rsrc_t ru = make_rsrc((const IO*)p.u + (long long)b * p.T * p.W, seq_bytes);
+  const rsrc_t ro = make_rsrc((const IO*)p.out + (long long)b * p.T * p.W, seq_bytes);
+  const long long* sp_row = p.segpos + (long long)b * p.T;
+
+  float win[K > 1 ? K - 1 : 1][V];                         // win[j] = padded row t - 1 - j
+#pragma unroll
+  for (int j = 0; j < K - 1; ++j) padded_row<IO, V, K>(p, ru, b, t0 - 1 - j, c0, win[j]);
+#pragma unroll
+  for (int tt = 0; tt < kConvRunFwd; ++tt) {
+    const int t = t0 + tt;
+    const unsigned off = ((unsigned)t * uW + (unsigned)c0) * es;
+    float cur[V], acc[V];
+    ConvRow<IO, V>::load(cur, ru, off);
+    const long long sp = sp_row[t < p.T ? t : p.T - 1];
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      float a = bias[v];
+      if (sp >= 0) a = fmaf(cur[v], tap[K - 1][v], a);
+#pragma unroll
+      for (int lag = 1; lag < K; ++lag)
+        if (sp >= lag) a = fmaf(win[lag - 1][v], tap[K - 1 - lag][v], a);
+      acc[v] = a;
+    }
+    ConvRow<IO, V>::store(acc, ro, off);
+#pragma unroll
+    for (int j = K - 2; j > 0; --j)
+#pragma unroll
+      for (int v = 0; v < V; ++v) win[j][v] = win[j - 1][v];
+    if (K > 1) {
+#pragma unroll
+      for (int v = 0; v < V; ++v) win[0][v] = cur[v];
+    }
+  }
+  // carried state for the next call: the last K-1 rows of the padded input
+  if (K > 1 && p.new_state && it.run == p.runs - 1) {
+    const rsrc_t rn = make_rsrc((IO*)p.new_state + (long long)b * (K - 1) * p.W, (unsigned)((K - 1) * p.W) * es);
+#pragma unroll
+    for (int j = 0; j < K - 1; ++j) {
+      float row[V];
+      padded_row<IO, V, K>(p, ru, b, p.T - (K - 1) + j, c0, row);
+      ConvRow<IO, V>::store(row, rn, ((unsigned)j * uW + (unsigned)c0) * es);
+    }
+  }
+}
+
+// Backward: du, the gradient at the carried state (optional) and per-run partial sums of the tap
+// and bias gradients, partial[((b * runs + run) * (K + 1) + j) * W + c] with j = K for the bias.
+template <typename IO, int V, int K>
+__global__ __launch_bounds__(kConvThreads) void conv_bwd_kernel(ConvArgs p) {
+  const ConvItem it = conv_item(p);
+  if (!it.ok) return;
+  const int b = it.b, c0 = it.c0, t0 = it.run * kConvRunBwd;
+  const unsigned es = (unsigned)sizeof(IO), uW = (unsigned)p.W;
+  float tap[K][V];
+#pragma unroll
+  for (int v = 0; v < V; ++v)
+#pragma unroll
+    for (int j = 0; j < K; ++j) tap[j][v] = conv_param(p.taps, (long long)(c0 + v) * K + j, p.vec_dtype);
+  const unsigned seq_bytes = (unsigned)p.T * uW * es;
+  const rsrc_t ru = make_rsrc((const IO*)p.u + (long long)b * p.T * p.W, seq_bytes);
+  const rsrc_t rd = make_rsrc((const IO*)p.dout + (long long)b * p.T * p.W, seq_bytes);
+  const rsrc_t rg = make_rsrc((const IO*)p.du + (long long)b * p.T * p.W, seq_bytes);
+  const long long* sp_row = p.segpos + (long long)b * p.T;
+  auto position = [&](int t) { return sp_row[t < p.T ? t : p.T - 1]; };
+
+  float dwin[K][V];                                        // dwin[j] = dout row t + j
+  long long spw[K];
+  float uwin[K > 1 ? K - 1 : 1][V];                        // uwin[j] = padded row t - 1 - j
+  float acc_tap[K][V], acc_bias[V];
+#pragma unroll
+  for (int v = 0; v < V; ++v) {
+    acc_bias[v] = 0.f;
+#pragma unroll
+    for (int j = 0; j < K; ++j) acc_tap[j][v] = 0.f;
+  }
+#pragma unroll
+  for (int j = 0; j < K - 1; ++j) {
+    ConvRow<IO, V>::load(dwin[j], rd, ((unsigned)(t0 + j) * uW + (unsigned)c0) * es);
+    spw[j] = position(t0 + j);
+    padded_row<IO, V, K>(p, ru, b, t0 - 1 - j, c0, uwin[j]);
+  }
+#pragma unroll
+  for (int tt = 0; tt < kConvRunBwd; ++tt) {
+    const int t = t0 + tt;
+    const unsigned off = ((unsigned)t * uW + (unsigned)c0) * es;
+    ConvRow<IO, V>::load(dwin[K - 1], rd, ((unsigned)(t + K - 1) * uW + (unsigned)c0) * es);
+    spw[K - 1] = position(t + K - 1);
+    float cur[V], g[V];
+    ConvRow<IO, V>::load(cur, ru, off);
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      // input gradient: token t feeds the outputs t .. t + K - 1
+      float a = 0.f;
+#pragma unroll
+      for (int lag = 0; lag < K; ++lag)
+        if (spw[lag] >= lag) a = fmaf(dwin[lag][v], tap[K - 1 - lag][v], a);
+      g[v] = a;
+      // parameter gradients of output t
+      const float d = dwin[0][v];
+      acc_bias[v] += d;
+      if (spw[0] >= 0) acc_tap[K - 1][v] = fmaf(d, cur[v], acc_tap[K - 1][v]);
+#pragma unroll
+      for (int lag = 1; lag < K; ++lag)
+        if (spw[0] >= lag) acc_tap[K - 1 - lag][v] = fmaf(d, uwin[lag - 1][v], acc_tap[K - 1 - lag][v]);
+    }
+    ConvRow<IO, V>::store(g, rg, off);
+#pragma unroll
+    for (int j = 0; j < K - 1; ++j) {
+      spw[j] = spw[j + 1];
+#pragma unroll
+      for (int v = 0; v < V; ++v) dwin[j][v] = dwin[j + 1][v];
+    }
+#pragma unroll
+    for (int j = K - 2; j > 0; --j)
+#pragma unroll
+      for (int v = 0; v < V; ++v) uwin[j][v] = uwin[j - 1][v];
+    if (K > 1) {
+#pragma unroll
+      for (int v = 0; v < V; ++v) uwin[0][v] = cur[v];
+    }
+  }
+  float* part = p.partial + ((long long)(b * p.runs + it.run) * (K + 1)) * p.W + c0;
+#pragma unroll
+  for (int j = 0; j < K; ++j)
+#pragma unroll
+    for (int v = 0; v < V; ++v) part[(long long)j * p.W + v] = acc_tap[j][v];
+#pragma unroll
+  for (int v = 0; v < V; ++v) part[(long long)K * p.W + v] = acc_bias[v];
+
+  // gradient at the carried state: state row j stands at time j - (K - 1) < 0
+  if (K > 1 && p.dstate && it.run == 0) {
+    const rsrc_t rs = make_rsrc((IO*)p.dstate + (long long)b * (K - 1) * p.W, (unsigned)((K - 1) * p.W) * es);
+#pragma unroll
+    for (int j = 0; j < K - 1; ++j) {
+      const int tau = j - (K - 1);
+      float a[V];
+#pragma unroll
+      for (int v = 0; v < V; ++v) a[v] = 0.f;
+#pragma unroll
+      for (int lag = 1; lag < K; ++lag) {
+        const int t = tau + lag;
+        if (t >= 0 && t < p.T && position(t) >= lag) {
+          float d[V];
+          ConvRow<IO, V>::load(d, rd, ((unsigned)t * uW + (unsigned)c0) * es);
+#pragma unroll
+          for (int v = 0; v < V; ++v) a[v] = fmaf(d[v], tap[K - 1 - lag][v], a[v]);
+        }
+      }
+      ConvRow<IO, V>::store(a, rs, ((unsigned)j * uW + (unsigned)c0) * es);
+    }
+  }
+}
+
+// Sums the per-run partials: one thread per (tap or bias, channel).
+struct ConvFinishArgs { const float* partial; void* dtaps; void* dbias; int W, K, slots, grad_dtype; };
+__global__ __launch_bounds__(256) void conv_finish_kernel(ConvFinishArgs p) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= (long long)(p.K + 1) * p.W) return;
+  const int j = (int)(i / p.W), c = (int)(i - (long long)j * p.W);
+  const float* src = p.partial + (long long)j * p.W + c;
+  const long long stride = (long long)(p.K + 1) * p.W;
+  float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+  int n = 0;
+  for (; n + 4 <= p.slots; n += 4) {
+    s0 += src[(long long)n * stride]; s1 += src[(long long)(n + 1) * stride];
+    s2 += src[(long long)(n + 2) * stride]; s3 += src[(long long)(n + 3) * stride];
+  }
+  for (; n < p.slots; ++n) s0 += src[(long long)n * stride];
+  const float s = (s0 + s1) + (s2 + s3);
+  void* dst = j < p.K ? p.dtaps : p.dbias;
+  if (!dst) return;
+  const long long at = j < p.K ? (long long)c * p.K + j : c;
+  if (p.grad_dtype == RGLRU_BF16) ((__bf16*)dst)[at] = (__bf16)s; else ((float*)dst)[at] = s;
+}
+
+// ------------------------------------------------------------------------------------------
+// host side
+// ------------------------------------------------------------------------------------------
+static int conv_check(const char* who, int64_t B, int64_t T, int64_t W, int64_t K, int dtype, int vec_dtype) {
+  if (dtype != RGLRU_F32 && dtype != RGLRU_BF16) return fail(RGLRU_E_ARG, "%s: dtype must be RGLRU_F32 or RGLRU_BF16, got %d", who, dtype);
+  if (vec_dtype != RGLRU_F32 && vec_dtype != RGLRU_BF16) return fail(RGLRU_E_ARG, "%s: unknown parameter dtype %d", who, vec_dtype);
+  if (B <= 0 || T <= 0 || W <= 0) return fail(RGLRU_E_ARG, "%s: empty shape B=%lld T=%lld W=%lld", who, (long long)B, (long long)T, (long long)W);
+  if (K < 1 || K > kConvMaxTaps) return fail(RGLRU_E_UNSUPPORTED, "%s: kernel size %lld outside 1..%d", who, (long long)K, kConvMaxTaps);
+  const int64_t es = dtype == RGLRU_BF16 ? 2 : 4;
+  if ((T + kConvRunBwd + K) * W * es >= (1ll << 31)) return fail(RGLRU_E_UNSUPPORTED, "%s: one sequence exceeds 2 GiB", who);
+  if (B * ((T + kConvRunFwd - 1) / kConvRunFwd) * W >= (1ll << 40)) return fail(RGLRU_E_UNSUPPORTED, "%s: tensor too large", who);
+  return RGLRU_OK;
+}
+
+static bool conv_vector_ok(int64_t W, int dtype, std::initializer_list<const void*> ptrs) {
+  const int v = dtype == RGLRU_BF16 ? 8 : 4;
+  if (W % v) return false;
+  for (const void* q : ptrs) if (q && (uintptr_t)q % 16) return false;
+  return true;
+}
+
+#define RGLRU_CONV_K(KERNEL, IO, V, grid, s, a)                                                     \
+  switch ((a).K) {                                                                                  \
+    case 1: hipLaunchKernelGGL((KERNEL<IO, V, 1>), grid, dim3(kConvThreads), 0, s, a); break;       \
+    case 2: hipLaunchKernelGGL((KERNEL<IO, V, 2>), grid, dim3(kConvThreads), 0, s, a); break;       \
+    case 3: hipLaunchKernelGGL((KERNEL<IO, V, 3>), grid, dim3(kConvThreads), 0, s, a); break;       \
+    default: hipLaunchKernelGGL((KERNEL<IO, V, 4>), grid, dim3(kConvThreads), 0, s, a); break;      \
+  }
+#define RGLRU_CONV_DISPATCH(KERNEL, dtype, vec, grid, s, a)                                          \
+  do {                                                                                              \
+    if ((dtype) == RGLRU_BF16) { if (vec) { RGLRU_CONV_K(KERNEL, __bf16, 8, grid, s, a) } else { RGLRU_CONV_K(KERNEL, __bf16, 1, grid, s, a) } } \
+    else { if (vec) { RGLRU_CONV_K(KERNEL, float, 4, grid, s, a) } else { RGLRU_CONV_K(KERNEL, float, 1, grid, s, a) } } \
+  } while (0)
+
+}  // namespace rglru
+
+using namespace rglru;
+
+extern "C" {
+
+int rglru_hip_conv_max_kernel_size(void) { return kConvMaxTaps; }
+
+int rglru_hip_conv_fwd(const void* u, const void* state, const void* taps, const void* bias,
+                       const int64_t* segment_pos, void* out, void* new_state,
+                       int64_t B, int64_t T, int64_t W, int64_t K, int dtype, int vec_dtype, void* stream) {
+  int rc = conv_check("conv_fwd", B, T, W, K, dtype, vec_dtype);
+  if (rc) return rc;
+  if (!u || !taps || !segment_pos || !out) return fail(RGLRU_E_ARG, "conv_fwd: null pointer");
+  ConvArgs a;
+  memset(&a, 0, sizeof(a));
+  a.u = u; a.state = state; a.taps = taps; a.bias = bias; a.segpos = (const long long*)segment_pos;
+  a.out = out; a.new_state = new_state;
+  a.B = (int)B; a.T = (int)T; a.W = (int)W; a.K = (int)K; a.vec_dtype = vec_dtype;
+  const bool vec = conv_vector_ok(W, dtype, {u, state, out, new_state});
+  a.nvec = (int)(vec ? W / (dtype == RGLRU_BF16 ? 8 : 4) : W);
+  a.runs = (int)((T + kConvRunFwd - 1) / kConvRunFwd);
+  const long long items = (long long)B * a.runs * a.nvec;
+  dim3 grid((unsigned)((items + kConvThreads - 1) / kConvThreads));
+  hipStream_t s = (hipStream_t)stream;
+  RGLRU_CONV_DISPATCH(conv_fwd_kernel, dtype, vec, grid, s, a);
+  return check_launch("conv_fwd");
+}
+
+size_t rglru_hip_conv_scratch_bytes(int64_t B, int64_t T, int64_t W, int64_t K) {
+  if (B <= 0 || T <= 0 || W <= 0 || K < 1 || K > kConvMaxTaps) return 0;
+  const int64_t runs = (T + kConvRunBwd - 1) / kConvRunBwd;
+  return (size_t)(B * runs * (K + 1) * W * 4);
+}
+
+int rglru_hip_conv_bwd(const void* u, const void* state, const void* taps, const int64_t* segment_pos,
+                       const void* dout, void* scratch, void* du, void* dstate, void* dtaps, void* dbias,
+                       int64_t B, int64_t T, int64_t W, int64_t K, int dtype, int vec_dtype, int grad_dtype,
+                       void* stream) {
+  int rc = conv_check("conv_bwd", B, T, W, K, dtype, vec_dtype);
+  if (rc) return rc;
+  if (grad_dtype != RGLRU_F32 && grad_dtype != RGLRU_BF16) return fail(RGLRU_E_ARG, "conv_bwd: unknown gradient dtype %d", grad_dtype);
+  if (!u || !taps || !segment_pos || !dout || !scratch || !du) return fail(RGLRU_E_ARG, "conv_bwd: null pointer");
+  ConvArgs a;
+  memset(&a, 0, sizeof(a));
+  a.u = u; a.state = state; a.taps = taps; a.segpos = (const long long*)segment_pos;
+  a.dout = dout; a.du = du; a.dstate = dstate; a.partial = (float*)scratch;
+  a.B = (int)B; a.T = (int)T; a.W = (int)W; a.K = (int)K; a.vec_dtype = vec_dtype;
+  const bool vec = conv_vector_ok(W, dtype, {u, state, dout, du, dstate});
+  a.nvec = (int)(vec ? W / (dtype == RGLRU_BF16 ? 8 : 4) : W);
+  a.runs = (int)((T + kConvRunBwd - 1) / kConvRunBwd);
+  const long long items = (long long)B * a.runs * a.nvec;
+  dim3 grid((unsigned)((items + kConvThreads - 1) / kConvThreads));
+  hipStream_t s = (hipStream_t)stream;
+  RGLRU_CONV_DISPATCH(conv_bwd_kernel, dtype, vec, grid, s, a);
+  rc = check_launch("conv_bwd");
+  if (rc) return rc;
+  if (dtaps || dbias) {
+    ConvFinishArgs f;
+    f.partial = a.partial; f.dtaps = dtaps; f.dbias = dbias; f.W = (int)W; f.K = (int)K;
+    f.slots = (int)(B * a.runs); f.grad_dtype = grad_dtype;
+    const long long n = (long long)(K + 1) * W;
+    hipLaunchKernelGGL(conv_finish_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, f);
+    rc = check_launch("conv_bwd finish");
+  }
+  return rc;
+}
+
+}  // extern "C"

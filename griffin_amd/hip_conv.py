@@ -1,0 +1,119 @@
+"""PyTorch operator for the causal depthwise convolution that feeds the RG-LRU inside the recurrent
+block (griffin/griffin.py:474-487, the all-tokens-active path), over ``rglru_hip_conv_fwd`` /
+``rglru_hip_conv_bwd`` of librglru_hip.so.
+
+There is no CPU fallback here: the operator raises when the library or a GPU is missing.
+"""
+
+from __future__ import annotations
+
+import torch
+from torch import Tensor
+from torch.autograd.function import once_differentiable
+
+from . import _lib
+from .hip_scan import _DTYPE_CODES, _dtype_code, _ptr, _require_gpu, _stream_ptr
+
+
+def max_kernel_size() -> int:
+    """Largest convolution kernel size the HIP kernels cover."""
+    return int(_lib.load().rglru_hip_conv_max_kernel_size())
+
+
+def _parameter_operand(t: Tensor | None, like: torch.dtype) -> Tensor | None:
+    """A parameter as the library reads it: its own type when that is fp32 or bf16, else converted."""
+    if t is None:
+        return None
+    if t.dtype not in _DTYPE_CODES:
+        t = t.to(like)
+    return t.contiguous()
+
+
+class _HipCausalConv(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, u: Tensor, state: Tensor | None, weight: Tensor, bias: Tensor | None, segment_pos: Tensor):
+        _require_gpu("hip_causal_conv", u, state, weight, bias, segment_pos)
+        if u.dim() != 3:
+            raise ValueError(f"hip_causal_conv expects [batch, sequence, width], got {tuple(u.shape)}")
+        batch, steps, width = u.shape
+        if weight.dim() != 3 or weight.size(0) != width or weight.size(1) != 1:
+            raise ValueError("weight must be that of a depthwise Conv1d: [width, 1, kernel_size]")
+        taps_count = weight.size(2)
+        if bias is not None and bias.shape != (width,):
+            raise ValueError("bias must have shape [width]")
+        if state is not None and state.shape != (batch, taps_count - 1, width):
+            raise ValueError("state must have shape [batch, kernel_size - 1, width]")
+        if segment_pos.shape != (batch, steps):
+            raise ValueError("segment_pos must have shape [batch, sequence]")
+        code = _dtype_code(u.dtype)
+        u_c = u.contiguous()
+        state_c = None if state is None or taps_count == 1 else state.to(u.dtype).contiguous()
+        taps = _parameter_operand(weight, u.dtype)
+        if bias is not None and bias.dtype != taps.dtype:
+            bias = bias.to(taps.dtype)
+        bias_c = _parameter_operand(bias, u.dtype)
+        pos = segment_pos.to(device=u.device, dtype=torch.int64).contiguous()
+        out = torch.empty_like(u_c)
+        lib = _lib.load()
+        with torch.cuda.device(u.device):
+            _lib.check(lib.rglru_hip_conv_fwd(
+                _ptr(u_c), _ptr(state_c), _ptr(taps), _ptr(bias_c), _ptr(pos), _ptr(out), None,
+                batch, steps, width, taps_count, code, _DTYPE_CODES[taps.dtype], _stream_ptr(u.device)),
+                "rglru_hip_conv_fwd")
+        ctx.save_for_backward(u_c, state_c, taps, pos)
+        ctx.meta = (None if state is None else state.dtype, weight.dtype, None if bias is None else bias.dtype, weight.shape)
+        ctx.set_materialize_grads(False)
+        return out
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, dout: Tensor | None):
+        u, state, taps, pos = ctx.saved_tensors
+        state_dtype, weight_dtype, bias_dtype, weight_shape = ctx.meta
+        if dout is None:
+            return None, None, None, None, None
+        batch, steps, width = u.shape
+        taps_count = weight_shape[2]
+        code = _dtype_code(u.dtype)
+        dout_c = dout.to(u.dtype).contiguous()
+        lib = _lib.load()
+        need_u, need_state, need_w, need_b = ctx.needs_input_grad[:4]
+        grad_dtype = taps.dtype
+        du = torch.empty_like(u)
+        dstate = torch.empty_like(state) if (need_state and state is not None) else None
+        dtaps = torch.empty(width, taps_count, device=u.device, dtype=grad_dtype) if need_w else None
+        dbias = torch.empty(width, device=u.device, dtype=grad_dtype) if (need_b and bias_dtype is not None) else None
+        scratch = torch.empty(lib.rglru_hip_conv_scratch_bytes(batch, steps, width, taps_count),
+                              device=u.device, dtype=torch.uint8)
+        with torch.cuda.device(u.device):
+            _lib.check(lib.rglru_hip_conv_bwd(
+                _ptr(u), _ptr(state), _ptr(taps), _ptr(pos), _ptr(dout_c), _ptr(scratch), _ptr(du),
+                _ptr(dstate), _ptr(dtaps), _ptr(dbias),
+                batch, steps, width, taps_count, code, _DTYPE_CODES[taps.dtype], _DTYPE_CODES[grad_dtype],
+                _stream_ptr(u.device)), "rglru_hip_conv_bwd")
+        dweight = None if dtaps is None else dtaps.view(weight_shape).to(weight_dtype)
+        if dbias is not None:
+            dbias = dbias.to(bias_dtype)
+        if need_state and state_dtype is not None:
+            dstate = (u.new_zeros(batch, taps_count - 1, width) if dstate is None else dstate).to(state_dtype)
+        return (du if need_u else None), dstate, dweight, dbias, None
+
+
+def hip_causal_conv(u: Tensor, state: Tensor | None, weight: Tensor, bias: Tensor | None,
+                    segment_pos: Tensor) -> tuple[Tensor, Tensor]:
+    """Depthwise causal convolution with per-document tap masking.
+
+    ``u`` [B, T, W]; ``state`` [B, K-1, W] or None (zeros); ``weight`` [W, 1, K] and ``bias`` [W] of a
+    depthwise ``nn.Conv1d``; ``segment_pos`` [B, T] integer positions (a tap reaching back ``lag`` tokens
+    contributes only where ``segment_pos >= lag``).  Returns ``(out [B, T, W], new_state [B, K-1, W])``;
+    ``new_state`` is the last K-1 rows of ``cat(state, u)`` (griffin/griffin.py:487).
+    """
+    out = _HipCausalConv.apply(u, state, weight, bias, segment_pos)
+    history = weight.size(2) - 1
+    steps = u.size(1)
+    if steps >= history:
+        new_state = u[:, steps - history:].clone()
+    else:
+        previous = u.new_zeros(u.size(0), history, u.size(2)) if state is None else state.to(u.dtype)
+        new_state = torch.cat((previous[:, steps:], u), dim=1)
+    return out, new_state

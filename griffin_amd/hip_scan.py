@@ -370,6 +370,30 @@ def _validate_hip_scan(device: torch.device) -> None:
         scale = max(1.0, float(want.abs().max()))
         torch.testing.assert_close(got, want, atol=3e-5 * scale, rtol=3e-5)
 
+    # the caller's temporal convolution: 4 taps, carried state, a document boundary inside
+    from .hip_conv import hip_causal_conv
+
+    taps = (0.2 * torch.cos(torch.arange(W * 4, device=device, dtype=torch.float32) / 3.0)).reshape(W, 1, 4)
+    conv_bias = 0.1 * torch.sin(kb / 4.0)
+    conv_state = torch.cos(torch.arange(B * 3 * W, device=device, dtype=torch.float32) / 19.0).reshape(B, 3, W)
+    positions = torch.arange(T, device=device).repeat(B, 1)
+    positions[1, 33:] -= 33
+
+    def run_conv(use_hip):
+        leaves = [t.detach().clone().requires_grad_(True) for t in (x, conv_state, taps, conv_bias)]
+        fn = hip_causal_conv if use_hip else (lambda u, s, w, b, pos: portable.causal_depthwise_conv(u, s, w, b, pos))
+        out, carried = fn(*leaves, positions)
+        return out, carried, torch.autograd.grad(out, leaves, upstream)
+
+    ref_o, ref_c, ref_g = run_conv(False)
+    hip_o, hip_c, hip_g = run_conv(True)
+    torch.cuda.synchronize(device)
+    torch.testing.assert_close(hip_o, ref_o, atol=2e-5, rtol=2e-5)
+    torch.testing.assert_close(hip_c, ref_c, atol=0.0, rtol=0.0)
+    for got, want in zip(hip_g, ref_g):
+        scale = max(1.0, float(want.abs().max()))
+        torch.testing.assert_close(got, want, atol=3e-5 * scale, rtol=3e-5)
+
 
 def hip_scan_is_usable(device: torch.device | str) -> bool:
     """Validate the HIP kernels once per device before ``scan_mode="auto"`` may use them."""

@@ -20,7 +20,7 @@ from torch import Tensor
 import torch.nn as nn
 import torch.nn.functional as F
 
-from . import hip_scan, portable
+from . import hip_conv, hip_scan, portable
 
 ScanMode = Literal["auto", "sequential", "associative", "hip", "fused"]
 SCAN_MODES = ("auto", "sequential", "associative", "hip", "fused")
@@ -263,18 +263,25 @@ class RecurrentBlock(nn.Module):
     def _empty_conv_state(self, x: Tensor) -> Tensor:
         return x.new_zeros(x.size(0), self.conv_kernel_size - 1, self.rnn_width)
 
+    def _hip_conv_covers(self, projected: Tensor) -> bool:
+        """The HIP convolution runs wherever the RG-LRU inside takes its HIP path."""
+        mode = self.rg_lru.scan_mode
+        if not projected.is_cuda or projected.dtype not in hip_scan.SUPPORTED_DTYPES or projected.numel() == 0:
+            return False
+        if mode == "auto":
+            if not (self.rg_lru._hip_covers(projected) and hip_scan.hip_scan_is_usable(projected.device)):
+                return False
+        elif mode not in ("hip", "fused"):
+            return False
+        return self.conv_kernel_size <= hip_conv.max_kernel_size()
+
     def _dense_conv(self, projected: Tensor, conv_state: Tensor, segment_pos: Tensor):
         """All-tokens-active path (griffin/griffin.py:476-487): taps are masked per document."""
-        taps = self.temporal_conv.weight[:, 0, :]
-        history = self.conv_kernel_size - 1
-        steps = projected.size(1)
-        padded = torch.cat((conv_state.to(projected), projected), dim=1)
-        out = projected.new_zeros(projected.shape) + self.temporal_conv.bias
-        for lag in range(self.conv_kernel_size):
-            window = padded[:, history - lag: history - lag + steps]
-            same_document = (segment_pos >= lag).to(window.dtype).unsqueeze(-1)
-            out = out + window * same_document * taps[:, history - lag]
-        return out, (padded[:, padded.size(1) - history:] if history else padded[:, :0])
+        if self._hip_conv_covers(projected):
+            return hip_conv.hip_causal_conv(projected, conv_state, self.temporal_conv.weight,
+                                            self.temporal_conv.bias, segment_pos)
+        return portable.causal_depthwise_conv(projected, conv_state, self.temporal_conv.weight,
+                                              self.temporal_conv.bias, segment_pos)
 
     def _padded_conv(self, projected: Tensor, conv_state: Tensor, segment_pos: Tensor, active_mask: Tensor):
         """Right-padded batches (griffin/griffin.py:488-510): padding never enters the history."""

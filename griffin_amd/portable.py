@@ -53,6 +53,25 @@ def decay_and_input(x, w_a, b_a, w_x, b_x, lam, c, reset_mask, active_mask, stat
     return a.to(state_dtype), z.to(state_dtype)
 
 
+def causal_depthwise_conv(projected: Tensor, conv_state: Tensor, weight: Tensor, bias: Tensor | None,
+                          segment_pos: Tensor):
+    """All-tokens-active temporal convolution of the recurrent block (griffin/griffin.py:474-487):
+    ``weight`` [W, 1, K] of a depthwise Conv1d, taps masked per document through ``segment_pos``.
+    Returns the convolved sequence and the last K-1 rows of the padded input."""
+    taps = weight[:, 0, :]
+    history = taps.size(1) - 1
+    steps = projected.size(1)
+    padded = torch.cat((conv_state.to(projected), projected), dim=1)
+    out = projected.new_zeros(projected.shape)
+    if bias is not None:
+        out = out + bias
+    for lag in range(history + 1):
+        window = padded[:, history - lag: history - lag + steps]
+        same_document = (segment_pos >= lag).to(window.dtype).unsqueeze(-1)
+        out = out + window * same_document * taps[:, history - lag]
+    return out, (padded[:, padded.size(1) - history:] if history else padded[:, :0])
+
+
 def sequential_scan(a: Tensor, z: Tensor, state: Tensor) -> Tensor:
     """One step per token (griffin/griffin.py:279-284)."""
     steps = []

@@ -11,6 +11,8 @@
  *   griffin/griffin.py:237-289      RG_LRU.forward (gates + scan, T > 1)   rglru_hip_prepare + rglru_hip_fwd
  *   autograd of griffin/griffin.py:237-289                                   rglru_hip_bwd, rglru_hip_bwd_full
  *   griffin/griffin.py:279-284 with T == 1 (decode step, carried state)     rglru_hip_step
+ *   griffin/griffin.py:474-487      causal depthwise convolution of the caller   rglru_hip_conv_fwd
+ *   autograd of griffin/griffin.py:474-487                                   rglru_hip_conv_bwd
  *
  * Conventions
  *   - every pointer is a DEVICE pointer owned by the caller; tensors are row-major with the
@@ -39,7 +41,7 @@
 extern "C" {
 #endif
 
-#define RGLRU_ABI_VERSION 3
+#define RGLRU_ABI_VERSION 4
 
 enum { RGLRU_F32 = 0, RGLRU_BF16 = 1 };
 
@@ -140,6 +142,29 @@ int rglru_hip_bwd_full(const void* x, const void* prep, const float* h0,
 /* One decode step (T == 1): h[B,W] fp32 is updated in place, y[B,W] (dtype) = h as stored. */
 int rglru_hip_step(const void* x, const void* prep, float* h, const uint8_t* flags, void* y,
                    int64_t B, int64_t W, int64_t nb, int dtype, void* stream);
+
+/* Causal depthwise temporal convolution that feeds the RG-LRU inside the recurrent block, all
+ * tokens active (griffin/griffin.py:474-487):
+ *   out[b,t,c] = bias[c] + sum_{lag<K} taps[c][K-1-lag] * [segment_pos[b,t] >= lag] * padded[b,t-lag,c]
+ * with padded = state[B,K-1,W] (NULL: zeros) followed by u[B,T,W].  taps[W,K] is the weight of a
+ * depthwise nn.Conv1d viewed as [W][K] (tap K-1 multiplies the current token), bias[W] may be NULL;
+ * both are read in vec_dtype.  u, state, out and new_state are `dtype`; segment_pos[B,T] is int64.
+ * new_state[B,K-1,W] (may be NULL) receives the last K-1 rows of padded (griffin/griffin.py:487).
+ * K = 1 .. rglru_hip_conv_max_kernel_size(); arithmetic in fp32. */
+int rglru_hip_conv_max_kernel_size(void);
+int rglru_hip_conv_fwd(const void* u, const void* state, const void* taps, const void* bias,
+                       const int64_t* segment_pos, void* out, void* new_state,
+                       int64_t B, int64_t T, int64_t W, int64_t K, int dtype, int vec_dtype, void* stream);
+
+/* Reverse mode of rglru_hip_conv_fwd.  dout[B,T,W] (dtype) is the gradient at `out`.  Writes
+ * du[B,T,W] and, when not NULL, dstate[B,K-1,W] (dtype), dtaps[W,K] and dbias[W] (grad_dtype).
+ * `scratch` holds rglru_hip_conv_scratch_bytes(B, T, W, K) bytes of per-run partial sums; its
+ * contents on entry do not matter. */
+size_t rglru_hip_conv_scratch_bytes(int64_t B, int64_t T, int64_t W, int64_t K);
+int rglru_hip_conv_bwd(const void* u, const void* state, const void* taps, const int64_t* segment_pos,
+                       const void* dout, void* scratch, void* du, void* dstate, void* dtaps, void* dbias,
+                       int64_t B, int64_t T, int64_t W, int64_t K, int dtype, int vec_dtype, int grad_dtype,
+                       void* stream);
 
 /* Test hook: number of polls a wave may spend waiting for a neighbouring chunk's carry before it
  * gives up, records the failure in the workspace and finishes with unspecified results.  The

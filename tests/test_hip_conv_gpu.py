@@ -1,0 +1,157 @@
+"""GPU parity of the causal depthwise convolution kernels (C ABI: rglru_hip_conv_fwd / _bwd) against the
+oracle's restatement of griffin/griffin.py:474-487 and autograd through it."""
+
+import pytest
+import torch
+
+from oracle import rglru_oracle as orc
+from tests.helpers import rel_err
+
+pytestmark = pytest.mark.gpu
+
+FP32_TOL = 1e-5     # norm-wise relative, fp32 storage
+BF16_TOL = 2e-2     # bf16 storage, fp32 arithmetic, against the fp32 oracle on the bf16-rounded inputs
+
+
+def _say(*args):
+    print(*args, flush=True)
+
+
+def _positions(B, T, kind, seed):
+    """Token positions: one document continued from earlier calls, fresh documents, or several
+    documents packed into each row."""
+    if kind == "continued":
+        return torch.arange(5, 5 + T).repeat(B, 1)
+    if kind == "fresh":
+        return torch.arange(T).repeat(B, 1)
+    g = torch.Generator().manual_seed(seed)
+    pos = torch.empty(B, T, dtype=torch.long)
+    for b in range(B):
+        p = int(torch.randint(0, 4, (1,), generator=g))
+        for t in range(T):
+            if t > 0 and float(torch.rand(1, generator=g)) < 0.15:
+                p = 0
+            pos[b, t] = p
+            p += 1
+    return pos
+
+
+def _case(B, T, W, K, seed, with_state, with_bias):
+    g = torch.Generator().manual_seed(seed)
+    u = torch.randn(B, T, W, generator=g)
+    w = torch.randn(W, K, generator=g) * (1.0 / K) ** 0.5
+    b = torch.randn(W, generator=g) * 0.1 if with_bias else None
+    state = torch.randn(B, K - 1, W, generator=g) if with_state else None
+    dout = torch.randn(B, T, W, generator=g)
+    return u, w, b, state, dout
+
+
+def _oracle(u, w, b, state, dout, pos, dtype):
+    def prep(t):
+        return None if t is None else t.to(dtype).to(torch.float32).requires_grad_(True)
+    u_, w_, b_, s_ = prep(u), prep(w), prep(b), prep(state)
+    B, T, W = u.shape
+    K = w.shape[1]
+    out, new_state = orc.causal_conv(u_, w_, torch.zeros(W) if b_ is None else b_,
+                                     torch.zeros(B, K - 1, W) if s_ is None else s_, pos)
+    leaves = [t for t in (u_, w_, b_, s_) if t is not None]
+    grads = torch.autograd.grad(out, leaves, dout.to(dtype).to(torch.float32))
+    names = [n for n, t in zip(("u", "w", "b", "state"), (u_, w_, b_, s_)) if t is not None]
+    return out.detach(), new_state.detach(), dict(zip(names, grads))
+
+
+def _hip(u, w, b, state, dout, pos, dtype):
+    from griffin_amd.hip_conv import hip_causal_conv
+
+    def prep(t):
+        return None if t is None else t.to(dtype).cuda().requires_grad_(True)
+    u_, b_, s_ = prep(u), prep(b), prep(state)
+    w_ = w.to(dtype)[:, None, :].contiguous().cuda().requires_grad_(True)
+    out, new_state = hip_causal_conv(u_, s_, w_, b_, pos.cuda())
+    leaves = [t for t in (u_, w_, b_, s_) if t is not None]
+    grads = list(torch.autograd.grad(out, leaves, dout.to(dtype).cuda()))
+    torch.cuda.synchronize()
+    names = [n for n, t in zip(("u", "w", "b", "state"), (u_, w_, b_, s_)) if t is not None]
+    grads[1] = grads[1][:, 0, :]
+    return out.detach(), new_state.detach(), dict(zip(names, grads))
+
+
+CASES = [
+    # B, T, W, K, positions, carried state, bias
+    (2, 50, 64, 4, "packed", True, True),      # vector path, several documents per row
+    (2, 37, 24, 4, "packed", True, True),      # fp32 rows of 96 bytes (vector path), bf16 rows of 48 (vector path)
+    (3, 33, 13, 4, "packed", True, True),      # odd width: one element per thread
+    (1, 2, 64, 4, "continued", True, True),    # shorter than the kernel: the new state mixes old state and input
+    (2, 100, 128, 3, "fresh", False, True),    # three taps, no carried state
+    (2, 40, 32, 2, "continued", True, False),  # two taps, no bias
+    (2, 19, 16, 1, "packed", False, True),     # a single tap: a per-channel scale and shift
+    (4, 300, 256, 4, "packed", True, True),    # several runs per sequence, halo across run boundaries
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("cfg", CASES)
+def test_conv_matches_oracle(cfg, dtype):
+    B, T, W, K, kind, with_state, with_bias = cfg
+    _say("conv case", cfg, dtype)
+    u, w, b, state, dout = _case(B, T, W, K, seed=3, with_state=with_state, with_bias=with_bias)
+    pos = _positions(B, T, kind, seed=4)
+    want_out, want_state, want_g = _oracle(u, w, b, state, dout, pos, dtype)
+    got_out, got_state, got_g = _hip(u, w, b, state, dout, pos, dtype)
+    tol = FP32_TOL if dtype == torch.float32 else BF16_TOL
+    errs = {"out": rel_err(got_out.float(), want_out)}
+    for name in want_g:
+        errs["d" + name] = rel_err(got_g[name].float(), want_g[name])
+    _say("  rel errors:", {k: "%.2e" % v for k, v in errs.items()})
+    for name, err in errs.items():
+        assert err < tol, (name, err)
+    # the carried state is a copy of input rows: exact in the storage type
+    assert torch.equal(got_state.float().cpu(), want_state.to(dtype).float())
+
+
+def test_conv_split_equals_one_pass_at_training_shape():
+    """B8 T2048 W1024 bf16: the sequence convolved in three pieces with the carried state equals one
+    pass bit for bit (each output depends on the same K rows either way), and the input gradient is
+    linear in the upstream gradient."""
+    from griffin_amd.hip_conv import hip_causal_conv
+
+    g = torch.Generator().manual_seed(9)
+    B, T, W, K = 8, 2048, 1024, 4
+    u = torch.randn(B, T, W, generator=g).bfloat16().cuda()
+    w = (torch.randn(W, 1, K, generator=g) * 0.5).bfloat16().cuda()
+    b = (torch.randn(W, generator=g) * 0.1).bfloat16().cuda()
+    pos = torch.arange(T).repeat(B, 1).cuda()
+    pos[3, 700:] -= 700
+    whole, last = hip_causal_conv(u, None, w, b, pos)
+    pieces, state, start = [], None, 0
+    for stop in (5, 1031, T):
+        piece, state = hip_causal_conv(u[:, start:stop].contiguous(), state, w, b, pos[:, start:stop].contiguous())
+        pieces.append(piece)
+        start = stop
+    assert torch.equal(torch.cat(pieces, dim=1), whole)
+    assert torch.equal(state, last)
+    uu = u.clone().requires_grad_(True)
+    out, _ = hip_causal_conv(uu, None, w, b, pos)
+    d1 = torch.randn(B, T, W, generator=g).bfloat16().cuda()
+    g1, = torch.autograd.grad(out, uu, d1, retain_graph=True)
+    g2, = torch.autograd.grad(out, uu, 2 * d1)
+    torch.cuda.synchronize()
+    assert rel_err(g2.float(), 2 * g1.float()) < 1e-2
+
+
+def test_conv_argument_errors():
+    from griffin_amd.hip_conv import hip_causal_conv
+
+    u = torch.randn(2, 8, 16, device="cuda")
+    w = torch.randn(16, 1, 4, device="cuda")
+    pos = torch.arange(8, device="cuda").repeat(2, 1)
+    with pytest.raises(RuntimeError):
+        hip_causal_conv(u.cpu(), None, w.cpu(), None, pos.cpu())
+    with pytest.raises(ValueError):
+        hip_causal_conv(u, None, torch.randn(16, 1, 9, device="cuda"), None, pos)      # kernel size beyond the maximum
+    with pytest.raises(ValueError):
+        hip_causal_conv(u, torch.zeros(2, 2, 16, device="cuda"), w, None, pos)         # state of the wrong length
+    with pytest.raises(ValueError):
+        hip_causal_conv(u, None, w, None, pos[:, :4])
+    with pytest.raises(TypeError):
+        hip_causal_conv(u.double(), None, w.double(), None, pos)

@@ -257,3 +257,68 @@ def test_initialisers_follow_reference_ranges():
     assert a8.min() >= 0.9 - 1e-6 and a8.max() <= 0.999 + 1e-6
     w, b = orc.gate_init(16, 4, gen)
     assert abs(w.std().item() - 0.5) < 0.08 and (b == 0).all()
+
+
+# ----------------------------------------------------------------------------------------------
+# causal depthwise convolution of the caller (griffin/griffin.py:474-487)
+# ----------------------------------------------------------------------------------------------
+def _conv_case(B=2, T=13, W=6, K=4, seed=21):
+    g = torch.Generator().manual_seed(seed)
+    px = torch.randn(B, T, W, generator=g, dtype=torch.float64)
+    w = torch.randn(W, K, generator=g, dtype=torch.float64)
+    b = torch.randn(W, generator=g, dtype=torch.float64)
+    state = torch.randn(B, K - 1, W, generator=g, dtype=torch.float64)
+    return px, w, b, state
+
+
+def test_oracle_conv_equals_library_conv1d_on_one_document():
+    """Positions 3, 4, ... (every tap live): the conv is F.conv1d over cat(state, input), depthwise."""
+    px, w, b, state = _conv_case()
+    B, T, W = px.shape
+    K = w.shape[1]
+    seg = torch.arange(K - 1, K - 1 + T).repeat(B, 1)
+    out, new_state = orc.causal_conv(px, w, b, state, seg)
+    padded = torch.cat([state, px], dim=1).transpose(1, 2)
+    want = torch.nn.functional.conv1d(padded, w[:, None, :], b, groups=W).transpose(1, 2)
+    torch.testing.assert_close(out, want, atol=1e-12, rtol=1e-12)
+    torch.testing.assert_close(new_state, px[:, T - (K - 1):])
+
+
+def test_oracle_conv_fresh_document_ignores_history_and_state():
+    """Positions 0, 1, ...: taps reaching before the document start are dropped, so the carried state
+    has no influence and the result is conv1d with zero left padding; a document that starts inside
+    the sequence sees nothing from before its first token."""
+    px, w, b, state = _conv_case()
+    B, T, W = px.shape
+    K = w.shape[1]
+    seg = torch.arange(T).repeat(B, 1)
+    out, _ = orc.causal_conv(px, w, b, state, seg)
+    zero_padded = torch.nn.functional.pad(px.transpose(1, 2), (K - 1, 0))
+    want = torch.nn.functional.conv1d(zero_padded, w[:, None, :], b, groups=W).transpose(1, 2)
+    torch.testing.assert_close(out, want, atol=1e-12, rtol=1e-12)
+    start = 5
+    seg2 = seg.clone()
+    seg2[:, start:] -= start
+    out2, _ = orc.causal_conv(px, w, b, state, seg2)
+    alone, _ = orc.causal_conv(px[:, start:], w, b, torch.zeros_like(state), seg[:, : T - start])
+    torch.testing.assert_close(out2[:, start:], alone, atol=1e-12, rtol=1e-12)
+    torch.testing.assert_close(out2[:, :start], out[:, :start], atol=1e-12, rtol=1e-12)
+
+
+def test_oracle_conv_brute_force_and_split_invariance():
+    px, w, b, state = _conv_case(B=1, T=7, W=3, K=3, seed=5)
+    seg = torch.tensor([[4, 5, 0, 1, 2, 3, 0]])
+    out, new_state = orc.causal_conv(px, w, b, state, seg)
+    padded = torch.cat([state, px], dim=1)
+    K = 3
+    for t in range(7):
+        for c in range(3):
+            want = b[c].item()
+            for lag in range(K):
+                if seg[0, t] >= lag:
+                    want += w[c, K - 1 - lag].item() * padded[0, K - 1 + t - lag, c].item()
+            assert out[0, t, c].item() == pytest.approx(want, abs=1e-12)
+    first, mid_state = orc.causal_conv(px[:, :4], w, b, state, seg[:, :4])
+    second, end_state = orc.causal_conv(px[:, 4:], w, b, mid_state, seg[:, 4:])
+    torch.testing.assert_close(torch.cat([first, second], dim=1), out, atol=1e-12, rtol=1e-12)
+    torch.testing.assert_close(end_state, new_state)
