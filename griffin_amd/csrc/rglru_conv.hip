@@ -24,6 +24,10 @@ constexpr int kConvMaxTaps = 4;        // kernel sizes 1..4 (the reference uses 
 constexpr int kConvRunFwd = 16;        // tokens per thread, forward
 constexpr int kConvRunBwd = 32;        // tokens per thread, backward (one partial sum per run)
 constexpr int kConvThreads = 256;
+constexpr int kConvBatch = 8;          // rows requested together, forward
+constexpr int kConvBatchBwd = 4;       // backward (two streams, more live state)
+constexpr int kConvBwdVecs = 32;       // backward: channel vectors per workgroup ...
+constexpr int kConvBwdRuns = kConvThreads / kConvBwdVecs;   // ... and runs, whose partial sums it adds up
 
 struct ConvArgs {
   const void* u; const void* state; const void* taps; const void* bias; const long long* segpos;
@@ -32,14 +36,17 @@ struct ConvArgs {
   int B, T, W, K, nvec, runs, vec_dtype;
 };
 
-// V values of one row, as floats.
+// V values of one row.  `Raw` is the row as loaded (requests are issued in batches before any of
+// them is used); unpack turns it into floats.
 template <typename IO, int V> struct ConvRow;
 template <> struct ConvRow<__bf16, 8> {
-  static RGLRU_DEVICE void load(float (&v)[8], rsrc_t r, unsigned off) {
-    const bf16x8 f = buf_load_frag<bf16x8>(r, off);
+  typedef bf16x8 Raw;
+  static RGLRU_DEVICE Raw request(rsrc_t r, unsigned off) { return buf_load_frag<bf16x8>(r, off); }
+  static RGLRU_DEVICE void unpack(float (&v)[8], const Raw& f) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) v[i] = (float)f[i];
   }
+  static RGLRU_DEVICE void load(float (&v)[8], rsrc_t r, unsigned off) { unpack(v, request(r, off)); }
   static RGLRU_DEVICE void store(const float (&v)[8], rsrc_t r, unsigned off) {
     bf16x8 f;
 #pragma unroll
@@ -48,11 +55,13 @@ template <> struct ConvRow<__bf16, 8> {
   }
 };
 template <> struct ConvRow<float, 4> {
-  static RGLRU_DEVICE void load(float (&v)[4], rsrc_t r, unsigned off) {
-    const f32x4 f = buf_load_frag<f32x4>(r, off);
+  typedef f32x4 Raw;
+  static RGLRU_DEVICE Raw request(rsrc_t r, unsigned off) { return buf_load_frag<f32x4>(r, off); }
+  static RGLRU_DEVICE void unpack(float (&v)[4], const Raw& f) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) v[i] = f[i];
   }
+  static RGLRU_DEVICE void load(float (&v)[4], rsrc_t r, unsigned off) { unpack(v, request(r, off)); }
   static RGLRU_DEVICE void store(const float (&v)[4], rsrc_t r, unsigned off) {
     f32x4 f;
 #pragma unroll
@@ -61,7 +70,10 @@ template <> struct ConvRow<float, 4> {
   }
 };
 template <typename IO> struct ConvRow<IO, 1> {
-  static RGLRU_DEVICE void load(float (&v)[1], rsrc_t r, unsigned off) { v[0] = BufIo<IO>::load(r, off, 0u); }
+  typedef float Raw;
+  static RGLRU_DEVICE Raw request(rsrc_t r, unsigned off) { return BufIo<IO>::load(r, off, 0u); }
+  static RGLRU_DEVICE void unpack(float (&v)[1], const Raw& f) { v[0] = f; }
+  static RGLRU_DEVICE void load(float (&v)[1], rsrc_t r, unsigned off) { v[0] = request(r, off); }
   static RGLRU_DEVICE void store(const float (&v)[1], rsrc_t r, unsigned off) { BufIo<IO>::store((IO)v[0], r, off, 0u); }
 };
 
@@ -119,13 +131,22 @@ __global__ __launch_bounds__(kConvThreads) void conv_fwd_kernel(ConvArgs p) {
   float win[K > 1 ? K - 1 : 1][V];                         // win[j] = padded row t - 1 - j
 #pragma unroll
   for (int j = 0; j < K - 1; ++j) padded_row<IO, V, K>(p, ru, b, t0 - 1 - j, c0, win[j]);
+  for (int t1 = 0; t1 < kConvRunFwd; t1 += kConvBatch) {
+   typename ConvRow<IO, V>::Raw raw[kConvBatch];
+   long long spb[kConvBatch];
 #pragma unroll
-  for (int tt = 0; tt < kConvRunFwd; ++tt) {
-    const int t = t0 + tt;
+   for (int i = 0; i < kConvBatch; ++i) {
+     const int t = t0 + t1 + i;
+     raw[i] = ConvRow<IO, V>::request(ru, ((unsigned)t * uW + (unsigned)c0) * es);
+     spb[i] = sp_row[t < p.T ? t : p.T - 1];
+   }
+#pragma unroll
+   for (int i = 0; i < kConvBatch; ++i) {
+    const int t = t0 + t1 + i;
     const unsigned off = ((unsigned)t * uW + (unsigned)c0) * es;
     float cur[V], acc[V];
-    ConvRow<IO, V>::load(cur, ru, off);
-    const long long sp = sp_row[t < p.T ? t : p.T - 1];
+    ConvRow<IO, V>::unpack(cur, raw[i]);
+    const long long sp = spb[i];
 #pragma unroll
     for (int v = 0; v < V; ++v) {
       float a = bias[v];
@@ -144,6 +165,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_fwd_kernel(ConvArgs p) {
 #pragma unroll
       for (int v = 0; v < V; ++v) win[0][v] = cur[v];
     }
+   }
   }
   // carried state for the next call: the last K-1 rows of the padded input
   if (K > 1 && p.new_state && it.run == p.runs - 1) {
@@ -157,20 +179,30 @@ __global__ __launch_bounds__(kConvThreads) void conv_fwd_kernel(ConvArgs p) {
   }
 }
 
-// Backward: du, the gradient at the carried state (optional) and per-run partial sums of the tap
-// and bias gradients, partial[((b * runs + run) * (K + 1) + j) * W + c] with j = K for the bias.
+// Backward: du, the gradient at the carried state (optional) and partial sums of the tap and bias
+// gradients.  A workgroup covers kConvBwdVecs channel vectors and kConvBwdRuns consecutive runs of
+// one sequence and adds the sums of its runs up in LDS:
+//   partial[((b * run_groups + run_group) * (K + 1) + j) * W + c],  j = K for the bias.
 template <typename IO, int V, int K>
 __global__ __launch_bounds__(kConvThreads) void conv_bwd_kernel(ConvArgs p) {
-  const ConvItem it = conv_item(p);
-  if (!it.ok) return;
-  const int b = it.b, c0 = it.c0, t0 = it.run * kConvRunBwd;
+  __shared__ float red[kConvBwdRuns][(K + 1) * V][kConvBwdVecs + 1];
+  const int vec_groups = (p.nvec + kConvBwdVecs - 1) / kConvBwdVecs;
+  const int run_groups = (p.runs + kConvBwdRuns - 1) / kConvBwdRuns;
+  const int vg = blockIdx.x % vec_groups;
+  const int rest = blockIdx.x / vec_groups;
+  const int rgp = rest % run_groups, b = rest / run_groups;
+  const int lane_vec = threadIdx.x % kConvBwdVecs, lane_run = threadIdx.x / kConvBwdVecs;
+  const int vec = vg * kConvBwdVecs + lane_vec, run = rgp * kConvBwdRuns + lane_run;
+  const bool ok = vec < p.nvec && run < p.runs;
+  const int c0 = (vec < p.nvec ? vec : 0) * V, t0 = run * kConvRunBwd;
   const unsigned es = (unsigned)sizeof(IO), uW = (unsigned)p.W;
   float tap[K][V];
 #pragma unroll
   for (int v = 0; v < V; ++v)
 #pragma unroll
     for (int j = 0; j < K; ++j) tap[j][v] = conv_param(p.taps, (long long)(c0 + v) * K + j, p.vec_dtype);
-  const unsigned seq_bytes = (unsigned)p.T * uW * es;
+  // a thread without work sees empty tensors: its loads return zero and its stores are dropped
+  const unsigned seq_bytes = ok ? (unsigned)p.T * uW * es : 0u;
   const rsrc_t ru = make_rsrc((const IO*)p.u + (long long)b * p.T * p.W, seq_bytes);
   const rsrc_t rd = make_rsrc((const IO*)p.dout + (long long)b * p.T * p.W, seq_bytes);
   const rsrc_t rg = make_rsrc((const IO*)p.du + (long long)b * p.T * p.W, seq_bytes);
@@ -191,58 +223,67 @@ __global__ __launch_bounds__(kConvThreads) void conv_bwd_kernel(ConvArgs p) {
   for (int j = 0; j < K - 1; ++j) {
     ConvRow<IO, V>::load(dwin[j], rd, ((unsigned)(t0 + j) * uW + (unsigned)c0) * es);
     spw[j] = position(t0 + j);
-    padded_row<IO, V, K>(p, ru, b, t0 - 1 - j, c0, uwin[j]);
-  }
+    if (ok) {
+      padded_row<IO, V, K>(p, ru, b, t0 - 1 - j, c0, uwin[j]);
+    } else {
 #pragma unroll
-  for (int tt = 0; tt < kConvRunBwd; ++tt) {
-    const int t = t0 + tt;
-    const unsigned off = ((unsigned)t * uW + (unsigned)c0) * es;
-    ConvRow<IO, V>::load(dwin[K - 1], rd, ((unsigned)(t + K - 1) * uW + (unsigned)c0) * es);
-    spw[K - 1] = position(t + K - 1);
-    float cur[V], g[V];
-    ConvRow<IO, V>::load(cur, ru, off);
-#pragma unroll
-    for (int v = 0; v < V; ++v) {
-      // input gradient: token t feeds the outputs t .. t + K - 1
-      float a = 0.f;
-#pragma unroll
-      for (int lag = 0; lag < K; ++lag)
-        if (spw[lag] >= lag) a = fmaf(dwin[lag][v], tap[K - 1 - lag][v], a);
-      g[v] = a;
-      // parameter gradients of output t
-      const float d = dwin[0][v];
-      acc_bias[v] += d;
-      if (spw[0] >= 0) acc_tap[K - 1][v] = fmaf(d, cur[v], acc_tap[K - 1][v]);
-#pragma unroll
-      for (int lag = 1; lag < K; ++lag)
-        if (spw[0] >= lag) acc_tap[K - 1 - lag][v] = fmaf(d, uwin[lag - 1][v], acc_tap[K - 1 - lag][v]);
-    }
-    ConvRow<IO, V>::store(g, rg, off);
-#pragma unroll
-    for (int j = 0; j < K - 1; ++j) {
-      spw[j] = spw[j + 1];
-#pragma unroll
-      for (int v = 0; v < V; ++v) dwin[j][v] = dwin[j + 1][v];
-    }
-#pragma unroll
-    for (int j = K - 2; j > 0; --j)
-#pragma unroll
-      for (int v = 0; v < V; ++v) uwin[j][v] = uwin[j - 1][v];
-    if (K > 1) {
-#pragma unroll
-      for (int v = 0; v < V; ++v) uwin[0][v] = cur[v];
+      for (int v = 0; v < V; ++v) uwin[j][v] = 0.f;
     }
   }
-  float* part = p.partial + ((long long)(b * p.runs + it.run) * (K + 1)) * p.W + c0;
+  for (int t1 = 0; t1 < kConvRunBwd; t1 += kConvBatchBwd) {
+    typename ConvRow<IO, V>::Raw raw_u[kConvBatchBwd], raw_d[kConvBatchBwd];
+    long long spb[kConvBatchBwd];
 #pragma unroll
-  for (int j = 0; j < K; ++j)
+    for (int i = 0; i < kConvBatchBwd; ++i) {
+      const int t = t0 + t1 + i;
+      raw_u[i] = ConvRow<IO, V>::request(ru, ((unsigned)t * uW + (unsigned)c0) * es);
+      raw_d[i] = ConvRow<IO, V>::request(rd, ((unsigned)(t + K - 1) * uW + (unsigned)c0) * es);
+      spb[i] = position(t + K - 1);
+    }
 #pragma unroll
-    for (int v = 0; v < V; ++v) part[(long long)j * p.W + v] = acc_tap[j][v];
+    for (int i = 0; i < kConvBatchBwd; ++i) {
+      const int t = t0 + t1 + i;
+      const unsigned off = ((unsigned)t * uW + (unsigned)c0) * es;
+      ConvRow<IO, V>::unpack(dwin[K - 1], raw_d[i]);
+      spw[K - 1] = spb[i];
+      float cur[V], g[V];
+      ConvRow<IO, V>::unpack(cur, raw_u[i]);
 #pragma unroll
-  for (int v = 0; v < V; ++v) part[(long long)K * p.W + v] = acc_bias[v];
+      for (int v = 0; v < V; ++v) {
+        // input gradient: token t feeds the outputs t .. t + K - 1
+        float a = 0.f;
+#pragma unroll
+        for (int lag = 0; lag < K; ++lag)
+          if (spw[lag] >= lag) a = fmaf(dwin[lag][v], tap[K - 1 - lag][v], a);
+        g[v] = a;
+        // parameter gradients of output t
+        const float d = dwin[0][v];
+        acc_bias[v] += d;
+        if (spw[0] >= 0) acc_tap[K - 1][v] = fmaf(d, cur[v], acc_tap[K - 1][v]);
+#pragma unroll
+        for (int lag = 1; lag < K; ++lag)
+          if (spw[0] >= lag) acc_tap[K - 1 - lag][v] = fmaf(d, uwin[lag - 1][v], acc_tap[K - 1 - lag][v]);
+      }
+      ConvRow<IO, V>::store(g, rg, off);
+#pragma unroll
+      for (int j = 0; j < K - 1; ++j) {
+        spw[j] = spw[j + 1];
+#pragma unroll
+        for (int v = 0; v < V; ++v) dwin[j][v] = dwin[j + 1][v];
+      }
+#pragma unroll
+      for (int j = K - 2; j > 0; --j)
+#pragma unroll
+        for (int v = 0; v < V; ++v) uwin[j][v] = uwin[j - 1][v];
+      if (K > 1) {
+#pragma unroll
+        for (int v = 0; v < V; ++v) uwin[0][v] = cur[v];
+      }
+    }
+  }
 
   // gradient at the carried state: state row j stands at time j - (K - 1) < 0
-  if (K > 1 && p.dstate && it.run == 0) {
+  if (K > 1 && p.dstate && ok && run == 0) {
     const rsrc_t rs = make_rsrc((IO*)p.dstate + (long long)b * (K - 1) * p.W, (unsigned)((K - 1) * p.W) * es);
 #pragma unroll
     for (int j = 0; j < K - 1; ++j) {
@@ -261,6 +302,27 @@ __global__ __launch_bounds__(kConvThreads) void conv_bwd_kernel(ConvArgs p) {
         }
       }
       ConvRow<IO, V>::store(a, rs, ((unsigned)j * uW + (unsigned)c0) * es);
+    }
+  }
+
+  // sums of the workgroup's runs (threads without work hold zeros)
+#pragma unroll
+  for (int j = 0; j < K; ++j)
+#pragma unroll
+    for (int v = 0; v < V; ++v) red[lane_run][j * V + v][lane_vec] = acc_tap[j][v];
+#pragma unroll
+  for (int v = 0; v < V; ++v) red[lane_run][K * V + v][lane_vec] = acc_bias[v];
+  __syncthreads();
+  float* part = p.partial + ((long long)(b * run_groups + rgp) * (K + 1)) * p.W;
+  for (int idx = threadIdx.x; idx < (K + 1) * V * kConvBwdVecs; idx += kConvThreads) {
+    const int row = idx / kConvBwdVecs, lv = idx - row * kConvBwdVecs;   // row = j * V + v
+    const int j = row / V, v = row - j * V;
+    const int ch = (vg * kConvBwdVecs + lv) * V + v;
+    if (ch < p.W) {
+      float sum = 0.f;
+#pragma unroll
+      for (int q = 0; q < kConvBwdRuns; ++q) sum += red[q][row][lv];
+      part[(long long)j * p.W + ch] = sum;
     }
   }
 }
@@ -353,7 +415,8 @@ int rglru_hip_conv_fwd(const void* u, const void* state, const void* taps, const
 size_t rglru_hip_conv_scratch_bytes(int64_t B, int64_t T, int64_t W, int64_t K) {
   if (B <= 0 || T <= 0 || W <= 0 || K < 1 || K > kConvMaxTaps) return 0;
   const int64_t runs = (T + kConvRunBwd - 1) / kConvRunBwd;
-  return (size_t)(B * runs * (K + 1) * W * 4);
+  const int64_t run_groups = (runs + kConvBwdRuns - 1) / kConvBwdRuns;
+  return (size_t)(B * run_groups * (K + 1) * W * 4);
 }
 
 int rglru_hip_conv_bwd(const void* u, const void* state, const void* taps, const int64_t* segment_pos,
@@ -372,8 +435,10 @@ int rglru_hip_conv_bwd(const void* u, const void* state, const void* taps, const
   const bool vec = conv_vector_ok(W, dtype, {u, state, dout, du, dstate});
   a.nvec = (int)(vec ? W / (dtype == RGLRU_BF16 ? 8 : 4) : W);
   a.runs = (int)((T + kConvRunBwd - 1) / kConvRunBwd);
-  const long long items = (long long)B * a.runs * a.nvec;
-  dim3 grid((unsigned)((items + kConvThreads - 1) / kConvThreads));
+  const long long run_groups = (a.runs + kConvBwdRuns - 1) / kConvBwdRuns;
+  const long long vec_groups = (a.nvec + kConvBwdVecs - 1) / kConvBwdVecs;
+  if (B * run_groups * vec_groups >= (1ll << 31)) return fail(RGLRU_E_UNSUPPORTED, "conv_bwd: tensor too large");
+  dim3 grid((unsigned)(B * run_groups * vec_groups));
   hipStream_t s = (hipStream_t)stream;
   RGLRU_CONV_DISPATCH(conv_bwd_kernel, dtype, vec, grid, s, a);
   rc = check_launch("conv_bwd");
@@ -381,7 +446,7 @@ int rglru_hip_conv_bwd(const void* u, const void* state, const void* taps, const
   if (dtaps || dbias) {
     ConvFinishArgs f;
     f.partial = a.partial; f.dtaps = dtaps; f.dbias = dbias; f.W = (int)W; f.K = (int)K;
-    f.slots = (int)(B * a.runs); f.grad_dtype = grad_dtype;
+    f.slots = (int)(B * run_groups); f.grad_dtype = grad_dtype;
     const long long n = (long long)(K + 1) * W;
     hipLaunchKernelGGL(conv_finish_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, f);
     rc = check_launch("conv_bwd finish");
