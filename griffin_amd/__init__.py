@@ -9,6 +9,7 @@ from .hip_scan import (
     hip_scan_available,
     hip_scan_is_usable,
 )
+from .hip_block_ops import hip_causal_conv, hip_gelu_gate
 from .modules import (
     BlockDiagonalLinear,
     RG_LRU,
@@ -22,6 +23,8 @@ __all__ = [
     "RG_LRU",
     "RecurrentBlock",
     "RecurrentBlockCache",
+    "hip_causal_conv",
+    "hip_gelu_gate",
     "hip_rglru",
     "hip_rglru_scan",
     "hip_rglru_step",

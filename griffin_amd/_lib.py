@@ -43,6 +43,8 @@ _SIGNATURES = {
     "rglru_hip_conv_fwd": (ctypes.c_int, [_P] * 7 + [_I, _I, _I, _I, ctypes.c_int, ctypes.c_int, _P]),
     "rglru_hip_conv_scratch_bytes": (ctypes.c_size_t, [_I, _I, _I, _I]),
     "rglru_hip_conv_bwd": (ctypes.c_int, [_P] * 10 + [_I, _I, _I, _I, ctypes.c_int, ctypes.c_int, ctypes.c_int, _P]),
+    "rglru_hip_gelu_gate_fwd": (ctypes.c_int, [_P, _P, _P, _I, ctypes.c_int, _P]),
+    "rglru_hip_gelu_gate_bwd": (ctypes.c_int, [_P, _P, _P, _P, _P, _I, ctypes.c_int, _P]),
     "rglru_hip_set_spin_limit": (ctypes.c_int64, [_I]),
     "rglru_hip_set_timing": (ctypes.c_int, [ctypes.c_int]),
     "rglru_hip_kernel_ms": (ctypes.c_float, [ctypes.c_int]),

@@ -1,14 +1,16 @@
-// Causal depthwise temporal convolution in front of the RG-LRU (griffin/griffin.py:474-487, the
-// all-tokens-active path of RecurrentBlock.forward), forward and backward.
+// Kernels for the two elementwise stages of the recurrent block that sit directly in front of and
+// behind the RG-LRU (griffin/griffin.py:439-529): the causal depthwise temporal convolution
+// (:474-487, the all-tokens-active path) and the output gate h * gelu_tanh(v) (:464, :520), each
+// forward and backward.  Both are pure streaming, bounded by HBM.
 //
+// Convolution:
 //   out[b,t,c] = bias[c] + sum_{lag<K} taps[c][K-1-lag] * [segment_pos[b,t] >= lag] * padded[b,t-lag,c]
-//
-// where padded is the K-1 rows of carried state followed by the T rows of the input.  The work is
-// pure streaming: a thread owns V consecutive channels (one 16-byte vector, or one element when
-// the rows are not 16-byte aligned) and a run of consecutive tokens of one sequence, keeps the last
-// K-1 rows in registers and touches every input and output element once.  All global accesses go
-// through buffer descriptors of one sequence: rows past its end read as zero and stores to them
-// are dropped, so the token loops carry no bounds branches.
+// where padded is the K-1 rows of carried state followed by the T rows of the input.  A thread owns
+// V consecutive channels (one 16-byte vector, or one element when the rows are not 16-byte
+// aligned) and a run of consecutive tokens of one sequence, keeps the last K-1 rows in registers
+// and touches every input and output element once.  All global accesses go through buffer
+// descriptors of one sequence: rows past its end read as zero and stores to them are dropped, so
+// the token loops carry no bounds branches.
 
 #include <hip/hip_runtime.h>
 
@@ -383,6 +385,110 @@ static bool conv_vector_ok(int64_t W, int dtype, std::initializer_list<const voi
     else { if (vec) { RGLRU_CONV_K(KERNEL, float, 4, grid, s, a) } else { RGLRU_CONV_K(KERNEL, float, 1, grid, s, a) } } \
   } while (0)
 
+
+// ------------------------------------------------------------------------------------------
+// Output gate: out = h * gelu_tanh(v) and its reverse mode, flat over n elements.
+//   gelu_tanh(v) = v/2 * (1 + tanh(u)),  u = sqrt(2/pi) * (v + 0.044715 v^3)
+// A thread handles 16-byte vectors in a grid-stride loop, four vectors requested at a time.
+// ------------------------------------------------------------------------------------------
+constexpr int kGateThreads = 256;
+constexpr int kGateBatch = 4;
+
+struct GeluParts { float gelu, dgelu; };
+RGLRU_DEVICE GeluParts gelu_tanh_parts(float v) {
+  const float k0 = 0.7978845608028654f, k1 = 0.044715f;
+  const float v2 = v * v;
+  const float u = k0 * v * fmaf(k1, v2, 1.0f);
+  // tanh(u) = 1 - 2 / (1 + exp(2u)); exp overflows to +inf for large u, which gives tanh = 1
+  const float e = __builtin_amdgcn_exp2f(u * (2.0f * kLog2e));
+  const float t = 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + e);
+  GeluParts g;
+  g.gelu = 0.5f * v * (1.0f + t);
+  const float du = k0 * fmaf(3.0f * k1, v2, 1.0f);
+  g.dgelu = fmaf(0.5f * v * fmaf(-t, t, 1.0f), du, 0.5f * (1.0f + t));
+  return g;
+}
+
+struct GateArgs { const void* h; const void* v; const void* dout; void* out; void* dh; void* dv; long long n; };
+
+template <typename IO, int V, bool BACKWARD>
+__global__ __launch_bounds__(kGateThreads) void gelu_gate_kernel(GateArgs p) {
+  typedef ConvRow<IO, V> Row;
+  const long long nvec = p.n / V;
+  const long long stride = (long long)gridDim.x * kGateThreads;
+  // descriptors cover at most 2 GiB: the loop walks windows of that size
+  constexpr long long WIN = (1ll << 30) / (long long)sizeof(IO) / V * V;    // elements per window (1 GiB)
+  for (long long w0 = 0; w0 < p.n; w0 += WIN) {
+    const long long wn = (p.n - w0) < WIN ? (p.n - w0) : WIN;
+    const unsigned bytes = (unsigned)(wn * (long long)sizeof(IO));
+    const rsrc_t rh = make_rsrc((const IO*)p.h + w0, bytes);
+    const rsrc_t rv = make_rsrc((const IO*)p.v + w0, bytes);
+    const rsrc_t rd = make_rsrc(BACKWARD ? (const IO*)p.dout + w0 : (const IO*)p.h, BACKWARD ? bytes : 0u);
+    const rsrc_t ro = make_rsrc(BACKWARD ? (IO*)p.dh + w0 : (IO*)p.out + w0, bytes);
+    const rsrc_t rw = make_rsrc(BACKWARD ? (IO*)p.dv + w0 : (IO*)p.out, BACKWARD ? bytes : 0u);
+    const long long wvec = (wn + V - 1) / V;
+    (void)nvec;
+    for (long long i0 = (long long)blockIdx.x * kGateThreads + threadIdx.x; i0 < wvec; i0 += stride * kGateBatch) {
+      typename Row::Raw raw_h[kGateBatch], raw_v[kGateBatch], raw_d[kGateBatch];
+#pragma unroll
+      for (int j = 0; j < kGateBatch; ++j) {
+        const long long i = i0 + (long long)j * stride;
+        const unsigned off = i < wvec ? (unsigned)(i * V * (long long)sizeof(IO)) : kOutOfRange;
+        raw_h[j] = Row::request(rh, off);
+        raw_v[j] = Row::request(rv, off);
+        if (BACKWARD) raw_d[j] = Row::request(rd, off);
+      }
+#pragma unroll
+      for (int j = 0; j < kGateBatch; ++j) {
+        const long long i = i0 + (long long)j * stride;
+        const unsigned off = i < wvec ? (unsigned)(i * V * (long long)sizeof(IO)) : kOutOfRange;
+        float h[V], v[V], a[V], b[V];
+        Row::unpack(h, raw_h[j]);
+        Row::unpack(v, raw_v[j]);
+        if (BACKWARD) {
+          float d[V];
+          Row::unpack(d, raw_d[j]);
+#pragma unroll
+          for (int e = 0; e < V; ++e) {
+            const GeluParts g = gelu_tanh_parts(v[e]);
+            a[e] = d[e] * g.gelu;
+            b[e] = (d[e] * h[e]) * g.dgelu;
+          }
+          Row::store(a, ro, off);
+          Row::store(b, rw, off);
+        } else {
+#pragma unroll
+          for (int e = 0; e < V; ++e) a[e] = h[e] * gelu_tanh_parts(v[e]).gelu;
+          Row::store(a, ro, off);
+        }
+      }
+    }
+  }
+}
+
+static int gate_launch(const char* who, bool backward, GateArgs a, int dtype, void* stream) {
+  if (dtype != RGLRU_F32 && dtype != RGLRU_BF16) return fail(RGLRU_E_ARG, "%s: dtype must be RGLRU_F32 or RGLRU_BF16, got %d", who, dtype);
+  if (a.n <= 0) return fail(RGLRU_E_ARG, "%s: empty tensor", who);
+  const int v = dtype == RGLRU_BF16 ? 8 : 4;
+  const bool vec = conv_vector_ok(a.n, dtype, {a.h, a.v, a.dout, a.out, a.dh, a.dv});
+  const long long items = vec ? (a.n + v - 1) / v : a.n;
+  long long blocks = (items + (long long)kGateThreads * kGateBatch - 1) / ((long long)kGateThreads * kGateBatch);
+  const long long cap = (long long)num_compute_units() * 16;
+  if (blocks > cap) blocks = cap;
+  if (blocks < 1) blocks = 1;
+  dim3 grid((unsigned)blocks);
+  hipStream_t s = (hipStream_t)stream;
+#define RGLRU_GATE_LAUNCH(IO, V)                                                                      \
+  do {                                                                                                \
+    if (backward) hipLaunchKernelGGL((gelu_gate_kernel<IO, V, true>), grid, dim3(kGateThreads), 0, s, a);  \
+    else hipLaunchKernelGGL((gelu_gate_kernel<IO, V, false>), grid, dim3(kGateThreads), 0, s, a);     \
+  } while (0)
+  if (dtype == RGLRU_BF16) { if (vec) RGLRU_GATE_LAUNCH(__bf16, 8); else RGLRU_GATE_LAUNCH(__bf16, 1); }
+  else { if (vec) RGLRU_GATE_LAUNCH(float, 4); else RGLRU_GATE_LAUNCH(float, 1); }
+#undef RGLRU_GATE_LAUNCH
+  return check_launch(who);
+}
+
 }  // namespace rglru
 
 using namespace rglru;
@@ -452,6 +558,23 @@ int rglru_hip_conv_bwd(const void* u, const void* state, const void* taps, const
     rc = check_launch("conv_bwd finish");
   }
   return rc;
+}
+
+int rglru_hip_gelu_gate_fwd(const void* h, const void* v, void* out, int64_t n, int dtype, void* stream) {
+  if (!h || !v || !out) return fail(RGLRU_E_ARG, "gelu_gate_fwd: null pointer");
+  GateArgs a;
+  memset(&a, 0, sizeof(a));
+  a.h = h; a.v = v; a.out = out; a.n = n;
+  return gate_launch("gelu_gate_fwd", false, a, dtype, stream);
+}
+
+int rglru_hip_gelu_gate_bwd(const void* dout, const void* h, const void* v, void* dh, void* dv,
+                            int64_t n, int dtype, void* stream) {
+  if (!dout || !h || !v || !dh || !dv) return fail(RGLRU_E_ARG, "gelu_gate_bwd: null pointer");
+  GateArgs a;
+  memset(&a, 0, sizeof(a));
+  a.h = h; a.v = v; a.dout = dout; a.dh = dh; a.dv = dv; a.n = n;
+  return gate_launch("gelu_gate_bwd", true, a, dtype, stream);
 }
 
 }  // extern "C"

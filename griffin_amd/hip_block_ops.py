@@ -1,6 +1,7 @@
-"""PyTorch operator for the causal depthwise convolution that feeds the RG-LRU inside the recurrent
-block (griffin/griffin.py:474-487, the all-tokens-active path), over ``rglru_hip_conv_fwd`` /
-``rglru_hip_conv_bwd`` of librglru_hip.so.
+"""PyTorch operators for the two elementwise stages around the RG-LRU inside the recurrent block: the
+causal depthwise convolution that feeds it (griffin/griffin.py:474-487, the all-tokens-active path)
+over ``rglru_hip_conv_fwd`` / ``rglru_hip_conv_bwd``, and the output gate ``h * gelu_tanh(v)``
+(griffin/griffin.py:464, :520) over ``rglru_hip_gelu_gate_fwd`` / ``_bwd`` of librglru_hip.so.
 
 There is no CPU fallback here: the operator raises when the library or a GPU is missing.
 """
@@ -117,3 +118,41 @@ def hip_causal_conv(u: Tensor, state: Tensor | None, weight: Tensor, bias: Tenso
         previous = u.new_zeros(u.size(0), history, u.size(2)) if state is None else state.to(u.dtype)
         new_state = torch.cat((previous[:, steps:], u), dim=1)
     return out, new_state
+
+
+class _HipGeluGate(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, h: Tensor, v: Tensor) -> Tensor:
+        _require_gpu("hip_gelu_gate", h, v)
+        if h.shape != v.shape:
+            raise ValueError(f"hip_gelu_gate expects equal shapes, got {tuple(h.shape)} and {tuple(v.shape)}")
+        if h.dtype != v.dtype:
+            raise TypeError(f"hip_gelu_gate expects equal dtypes, got {h.dtype} and {v.dtype}")
+        code = _dtype_code(h.dtype)
+        h_c, v_c = h.contiguous(), v.contiguous()
+        out = torch.empty_like(h_c)
+        if h_c.numel():
+            with torch.cuda.device(h.device):
+                _lib.check(_lib.load().rglru_hip_gelu_gate_fwd(
+                    _ptr(h_c), _ptr(v_c), _ptr(out), h_c.numel(), code, _stream_ptr(h.device)),
+                    "rglru_hip_gelu_gate_fwd")
+        ctx.save_for_backward(h_c, v_c)
+        return out
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, dout: Tensor):
+        h, v = ctx.saved_tensors
+        dout_c = dout.to(h.dtype).contiguous()
+        dh, dv = torch.empty_like(h), torch.empty_like(v)
+        if h.numel():
+            with torch.cuda.device(h.device):
+                _lib.check(_lib.load().rglru_hip_gelu_gate_bwd(
+                    _ptr(dout_c), _ptr(h), _ptr(v), _ptr(dh), _ptr(dv), h.numel(), _dtype_code(h.dtype),
+                    _stream_ptr(h.device)), "rglru_hip_gelu_gate_bwd")
+        return dh, dv
+
+
+def hip_gelu_gate(h: Tensor, v: Tensor) -> Tensor:
+    """``h * gelu(v, approximate="tanh")`` in one pass, differentiable in both arguments."""
+    return _HipGeluGate.apply(h, v)

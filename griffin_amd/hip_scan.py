@@ -371,7 +371,7 @@ def _validate_hip_scan(device: torch.device) -> None:
         torch.testing.assert_close(got, want, atol=3e-5 * scale, rtol=3e-5)
 
     # the caller's temporal convolution: 4 taps, carried state, a document boundary inside
-    from .hip_conv import hip_causal_conv
+    from .hip_block_ops import hip_causal_conv
 
     taps = (0.2 * torch.cos(torch.arange(W * 4, device=device, dtype=torch.float32) / 3.0)).reshape(W, 1, 4)
     conv_bias = 0.1 * torch.sin(kb / 4.0)
@@ -393,6 +393,21 @@ def _validate_hip_scan(device: torch.device) -> None:
     for got, want in zip(hip_g, ref_g):
         scale = max(1.0, float(want.abs().max()))
         torch.testing.assert_close(got, want, atol=3e-5 * scale, rtol=3e-5)
+
+    # the block's output gate h * gelu_tanh(v)
+    from .hip_block_ops import hip_gelu_gate
+
+    def run_gate(use_hip):
+        leaves = [t.detach().clone().requires_grad_(True) for t in (x, 4.0 * upstream)]
+        out = hip_gelu_gate(*leaves) if use_hip else leaves[0] * torch.nn.functional.gelu(leaves[1], approximate="tanh")
+        return out, torch.autograd.grad(out, leaves, upstream)
+
+    ref_o, ref_g = run_gate(False)
+    hip_o, hip_g = run_gate(True)
+    torch.cuda.synchronize(device)
+    torch.testing.assert_close(hip_o, ref_o, atol=2e-5, rtol=2e-5)
+    for got, want in zip(hip_g, ref_g):
+        torch.testing.assert_close(got, want, atol=3e-5, rtol=3e-5)
 
 
 def hip_scan_is_usable(device: torch.device | str) -> bool:

@@ -20,7 +20,7 @@ from torch import Tensor
 import torch.nn as nn
 import torch.nn.functional as F
 
-from . import hip_conv, hip_scan, portable
+from . import hip_block_ops, hip_scan, portable
 
 ScanMode = Literal["auto", "sequential", "associative", "hip", "fused"]
 SCAN_MODES = ("auto", "sequential", "associative", "hip", "fused")
@@ -263,7 +263,7 @@ class RecurrentBlock(nn.Module):
     def _empty_conv_state(self, x: Tensor) -> Tensor:
         return x.new_zeros(x.size(0), self.conv_kernel_size - 1, self.rnn_width)
 
-    def _hip_conv_covers(self, projected: Tensor) -> bool:
+    def _hip_block_ops_covers(self, projected: Tensor) -> bool:
         """The HIP convolution runs wherever the RG-LRU inside takes its HIP path."""
         mode = self.rg_lru.scan_mode
         if not projected.is_cuda or projected.dtype not in hip_scan.SUPPORTED_DTYPES or projected.numel() == 0:
@@ -273,12 +273,12 @@ class RecurrentBlock(nn.Module):
                 return False
         elif mode not in ("hip", "fused"):
             return False
-        return self.conv_kernel_size <= hip_conv.max_kernel_size()
+        return self.conv_kernel_size <= hip_block_ops.max_kernel_size()
 
     def _dense_conv(self, projected: Tensor, conv_state: Tensor, segment_pos: Tensor):
         """All-tokens-active path (griffin/griffin.py:476-487): taps are masked per document."""
-        if self._hip_conv_covers(projected):
-            return hip_conv.hip_causal_conv(projected, conv_state, self.temporal_conv.weight,
+        if self._hip_block_ops_covers(projected):
+            return hip_block_ops.hip_causal_conv(projected, conv_state, self.temporal_conv.weight,
                                             self.temporal_conv.bias, segment_pos)
         return portable.causal_depthwise_conv(projected, conv_state, self.temporal_conv.weight,
                                               self.temporal_conv.bias, segment_pos)
@@ -319,7 +319,7 @@ class RecurrentBlock(nn.Module):
         segment_pos = _resolve_segment_positions(
             x, segment_pos, previous_position, None if everything_active else active_mask)
 
-        gate_branch = F.gelu(self.linear_y(x), approximate="tanh")
+        gate_input = self.linear_y(x)
         projected = self.linear_x(x)
         conv_state = self._empty_conv_state(projected) if cache is None else cache.conv_state
         if conv_state.shape != (batch, self.conv_kernel_size - 1, self.rnn_width):
@@ -336,7 +336,11 @@ class RecurrentBlock(nn.Module):
             active_mask=None if everything_active else active_mask,
             return_state=True,
         )
-        output = self.linear_out(recurrent_out * gate_branch)
+        if self._hip_block_ops_covers(projected) and gate_input.dtype == recurrent_out.dtype:
+            gated = hip_block_ops.hip_gelu_gate(recurrent_out, gate_input)
+        else:
+            gated = recurrent_out * F.gelu(gate_input, approximate="tanh")
+        output = self.linear_out(gated)
         if not everything_active:
             output = output.masked_fill(~active_mask.unsqueeze(-1), 0.0)
         if return_cache:

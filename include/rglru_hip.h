@@ -13,6 +13,7 @@
  *   griffin/griffin.py:279-284 with T == 1 (decode step, carried state)     rglru_hip_step
  *   griffin/griffin.py:474-487      causal depthwise convolution of the caller   rglru_hip_conv_fwd
  *   autograd of griffin/griffin.py:474-487                                   rglru_hip_conv_bwd
+ *   griffin/griffin.py:464, :520    x_branch * gelu_tanh(linear_y(x))        rglru_hip_gelu_gate_fwd, _bwd
  *
  * Conventions
  *   - every pointer is a DEVICE pointer owned by the caller; tensors are row-major with the
@@ -165,6 +166,14 @@ int rglru_hip_conv_bwd(const void* u, const void* state, const void* taps, const
                        const void* dout, void* scratch, void* du, void* dstate, void* dtaps, void* dbias,
                        int64_t B, int64_t T, int64_t W, int64_t K, int dtype, int vec_dtype, int grad_dtype,
                        void* stream);
+
+/* Output gate of the recurrent block, out = h * gelu_tanh(v) (griffin/griffin.py:464 and :520: the
+ * GeLU of the second branch and the product with the RG-LRU output in one pass), flat over n
+ * elements of `dtype`; and its reverse mode: dh = dout * gelu_tanh(v), dv = dout * h * gelu_tanh'(v).
+ * Arithmetic in fp32. */
+int rglru_hip_gelu_gate_fwd(const void* h, const void* v, void* out, int64_t n, int dtype, void* stream);
+int rglru_hip_gelu_gate_bwd(const void* dout, const void* h, const void* v, void* dh, void* dv,
+                            int64_t n, int dtype, void* stream);
 
 /* Test hook: number of polls a wave may spend waiting for a neighbouring chunk's carry before it
  * gives up, records the failure in the workspace and finishes with unspecified results.  The

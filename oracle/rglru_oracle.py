@@ -278,6 +278,17 @@ def causal_conv(px, conv_w, conv_b, conv_state, seg_pos):
     return out, new_state
 
 
+def gelu_tanh(v):
+    """tanh approximation of GeLU, the activation of the block's second branch (griffin/griffin.py:464,
+    ``F.gelu(..., approximate="tanh")``): v/2 * (1 + tanh(sqrt(2/pi) * (v + 0.044715 v^3)))."""
+    return 0.5 * v * (1.0 + torch.tanh(0.7978845608028654 * (v + 0.044715 * v ** 3)))
+
+
+def gelu_gate(h, v):
+    """Output gate of the block: RG-LRU output times the GeLU branch (griffin/griffin.py:520)."""
+    return h * gelu_tanh(v)
+
+
 def recurrent_block_forward(x, p, c=8.0, cache=None):
     """All-active path of RecurrentBlock.forward (griffin/griffin.py:439-529).
 
@@ -287,7 +298,7 @@ def recurrent_block_forward(x, p, c=8.0, cache=None):
     B, T, _ = x.shape
     prev = None if cache is None else cache[2]
     seg = segment_positions(B, T, prev)
-    yb = torch.nn.functional.gelu(x @ p["ly_w"].T + p["ly_b"], approximate="tanh")
+    gate_in = x @ p["ly_w"].T + p["ly_b"]
     px = x @ p["lx_w"].T + p["lx_b"]
     K = p["conv_w"].shape[1]
     cstate = torch.zeros(B, K - 1, px.shape[2], dtype=px.dtype) if cache is None else cache[1]
@@ -295,5 +306,5 @@ def recurrent_block_forward(x, p, c=8.0, cache=None):
     h0 = None if cache is None else cache[0]
     yr, h_last = rglru_forward(xb, p["w_a"], p["b_a"], p["w_x"], p["b_x"], p["lam"], c, h0,
                                reset_mask=(seg == 0), active_mask=None)
-    out = (yr * yb) @ p["lo_w"].T + p["lo_b"]
+    out = gelu_gate(yr, gate_in) @ p["lo_w"].T + p["lo_b"]
     return out, (h_last, new_cstate, seg[:, -1].clone())

@@ -61,7 +61,7 @@ def _oracle(u, w, b, state, dout, pos, dtype):
 
 
 def _hip(u, w, b, state, dout, pos, dtype):
-    from griffin_amd.hip_conv import hip_causal_conv
+    from griffin_amd.hip_block_ops import hip_causal_conv
 
     def prep(t):
         return None if t is None else t.to(dtype).cuda().requires_grad_(True)
@@ -113,7 +113,7 @@ def test_conv_split_equals_one_pass_at_training_shape():
     """B8 T2048 W1024 bf16: the sequence convolved in three pieces with the carried state equals one
     pass bit for bit (each output depends on the same K rows either way), and the input gradient is
     linear in the upstream gradient."""
-    from griffin_amd.hip_conv import hip_causal_conv
+    from griffin_amd.hip_block_ops import hip_causal_conv
 
     g = torch.Generator().manual_seed(9)
     B, T, W, K = 8, 2048, 1024, 4
@@ -140,7 +140,7 @@ def test_conv_split_equals_one_pass_at_training_shape():
 
 
 def test_conv_argument_errors():
-    from griffin_amd.hip_conv import hip_causal_conv
+    from griffin_amd.hip_block_ops import hip_causal_conv
 
     u = torch.randn(2, 8, 16, device="cuda")
     w = torch.randn(16, 1, 4, device="cuda")
@@ -155,3 +155,65 @@ def test_conv_argument_errors():
         hip_causal_conv(u, None, w, None, pos[:, :4])
     with pytest.raises(TypeError):
         hip_causal_conv(u.double(), None, w.double(), None, pos)
+
+
+# ----------------------------------------------------------------------------------------------
+# output gate h * gelu_tanh(v) (C ABI: rglru_hip_gelu_gate_fwd / _bwd)
+# ----------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(2, 50, 64), (3, 7, 13), (1, 1, 1), (4, 300, 256), (5, 1023)])
+def test_gelu_gate_matches_oracle(shape, dtype):
+    from griffin_amd.hip_block_ops import hip_gelu_gate
+
+    _say("gelu gate case", shape, dtype)
+    g = torch.Generator().manual_seed(11)
+    h = torch.randn(*shape, generator=g) * 1.5
+    v = torch.randn(*shape, generator=g) * 3.0          # covers the saturated tails of tanh
+    dout = torch.randn(*shape, generator=g)
+    hr = h.to(dtype).float().requires_grad_(True)
+    vr = v.to(dtype).float().requires_grad_(True)
+    want = orc.gelu_gate(hr, vr)
+    want_dh, want_dv = torch.autograd.grad(want, (hr, vr), dout.to(dtype).float())
+    hh = h.to(dtype).cuda().requires_grad_(True)
+    vh = v.to(dtype).cuda().requires_grad_(True)
+    got = hip_gelu_gate(hh, vh)
+    got_dh, got_dv = torch.autograd.grad(got, (hh, vh), dout.to(dtype).cuda())
+    torch.cuda.synchronize()
+    tol = FP32_TOL if dtype == torch.float32 else BF16_TOL
+    errs = {"out": rel_err(got.float(), want), "dh": rel_err(got_dh.float(), want_dh), "dv": rel_err(got_dv.float(), want_dv)}
+    _say("  rel errors:", {k: "%.2e" % e for k, e in errs.items()})
+    for name, err in errs.items():
+        assert err < tol, (name, err)
+
+
+def test_gelu_gate_special_values_at_training_shape():
+    """B8 T2048 W1024 bf16: exact zeros where either factor is zero, the identity far in the positive
+    tail, zero far in the negative tail, and linearity in h."""
+    from griffin_amd.hip_block_ops import hip_gelu_gate
+
+    g = torch.Generator().manual_seed(12)
+    shape = (8, 2048, 1024)
+    h = torch.randn(*shape, generator=g).bfloat16().cuda()
+    v = (torch.randn(*shape, generator=g) * 2).bfloat16().cuda()
+    assert torch.count_nonzero(hip_gelu_gate(h, torch.zeros_like(v))) == 0
+    assert torch.count_nonzero(hip_gelu_gate(torch.zeros_like(h), v)) == 0
+    big = torch.full_like(v, 40.0)
+    assert torch.equal(hip_gelu_gate(h, big), (h.float() * 40.0).bfloat16())
+    assert torch.count_nonzero(hip_gelu_gate(h, -big)) == 0
+    out1 = hip_gelu_gate(h, v).float()
+    out2 = hip_gelu_gate(2 * h, v).float()
+    assert rel_err(out2, 2 * out1) < 1e-2
+
+
+def test_gelu_gate_argument_errors():
+    from griffin_amd.hip_block_ops import hip_gelu_gate
+
+    a = torch.randn(4, 8, device="cuda")
+    with pytest.raises(RuntimeError):
+        hip_gelu_gate(a.cpu(), a.cpu())
+    with pytest.raises(ValueError):
+        hip_gelu_gate(a, a[:, :4])
+    with pytest.raises(TypeError):
+        hip_gelu_gate(a, a.bfloat16())
+    with pytest.raises(TypeError):
+        hip_gelu_gate(a.double(), a.double())

@@ -322,3 +322,17 @@ def test_oracle_conv_brute_force_and_split_invariance():
     second, end_state = orc.causal_conv(px[:, 4:], w, b, mid_state, seg[:, 4:])
     torch.testing.assert_close(torch.cat([first, second], dim=1), out, atol=1e-12, rtol=1e-12)
     torch.testing.assert_close(end_state, new_state)
+
+
+def test_oracle_gelu_gate_is_the_library_tanh_gelu():
+    v = torch.linspace(-12.0, 12.0, 4001, dtype=torch.float64)
+    torch.testing.assert_close(orc.gelu_tanh(v), torch.nn.functional.gelu(v, approximate="tanh"), atol=1e-14, rtol=1e-13)
+    assert orc.gelu_tanh(torch.tensor(0.0)).item() == 0.0
+    assert orc.gelu_tanh(torch.tensor(30.0, dtype=torch.float64)).item() == pytest.approx(30.0, rel=1e-12)
+    assert abs(orc.gelu_tanh(torch.tensor(-30.0, dtype=torch.float64)).item()) < 1e-12
+    # close to, but not the same as, the exact GeLU x * Phi(x): the approximation error peaks near 5e-4
+    exact = torch.nn.functional.gelu(v)
+    gap = (orc.gelu_tanh(v) - exact).abs().max().item()
+    assert 1e-4 < gap < 1e-3
+    h = torch.linspace(-2.0, 3.0, 4001, dtype=torch.float64)
+    torch.testing.assert_close(orc.gelu_gate(h, v), h * torch.nn.functional.gelu(v, approximate="tanh"), atol=1e-14, rtol=1e-13)
