@@ -113,7 +113,7 @@ __global__ void prepare_kernel(PrepArgs p) {
 // ------------------------------------------------------------------------------------------
 struct FusedArgs {
   // tensors
-  const void* x; const void* wg; const float* bias; const float* sp; const float* cs; const void* w2t;
+  const void* x; const void* pre; const void* wg; const float* bias; const float* sp; const float* cs; const void* w2t;
   const float* h0; const uint8_t* flags;
   void* y; float* h_last;                                 // forward
   const void* dy; const float* dh_last;                   // backward in
@@ -125,6 +125,7 @@ struct FusedArgs {
   // geometry
   int B, T, W, nb, bw, bwp, S, Wp, groups, units;
   int bpu;                                                // gate blocks per unit (packed narrow blocks), else 1
+  long long rows_total;                                   // B * T, the row count of one block of `pre`
   int nC, nCf, ckpt_nC, wg_per_unit, aligned, full_slabs, queues, flags_vec;
   long long limit;
 #ifdef RGLRU_TRACE
@@ -453,9 +454,14 @@ __global__ __launch_bounds__(kThreads, 2) void fwd_kernel(FusedArgs p) {
   constexpr int MT = kFwdMT, TR = 32 * MT, EL = 16 * MT;
   typedef Io<IO> Tr;
   typedef typename Tr::Frag Frag;
-  constexpr int KC = NKG > 0 ? kPackedWidth : Tr::KCMAX;           // LDS tile width in elements
+  // NKG > 0: gate weights held in registers, pre-activations on MFMA.  NKG < 0: the caller supplies the
+  // pre-activations (blocks too wide to hold their weights: a library GEMM computes W x first).
+  // NKG == 0: the portable path (any width, alignment and storage type), weights streamed.
+  constexpr bool GIVEN = NKG < 0;
+  constexpr int KC = NKG != 0 ? kPackedWidth : Tr::KCMAX;          // LDS tile width in elements
   constexpr int LDSROW = KC + Tr::HW;
   __shared__ __attribute__((aligned(16))) IO lds[TR * LDSROW];
+  __shared__ __attribute__((aligned(16))) IO lds_pre[GIVEN ? 2 * TR * LDSROW : Tr::HW];   // W_a x | W_x x tiles
   __shared__ __attribute__((aligned(16))) unsigned char stage_all[kWaves * WaveStage<TR>::kBytes];
   __shared__ unsigned s_ticket[2];
 
@@ -471,21 +477,29 @@ __global__ __launch_bounds__(kThreads, 2) void fwd_kernel(FusedArgs p) {
   const long long W = p.W;
   const Queue q = make_queue(p, w.unit, w.wg_in_unit, p.nCf);
 
-  if constexpr (NKG > 0) {
+  if constexpr (NKG != 0) {
     // software-pipelined loop: the next ticket is taken while the current tile's MFMAs run and the
     // next x tile is requested right before the wave starts waiting for its carry
     HeldWeights<IO, NKG> hw;
     hw.load(w_a_row, w_x_row);
     constexpr int VPR = KC / Tr::HW;                     // 16-byte vectors per tile row
     constexpr int NV = (TR * VPR + kThreads - 1) / kThreads;
-    Frag pre[NV];
+    Frag pre[NV], pre_a[GIVEN ? NV : 1], pre_x[GIVEN ? NV : 1];
     const unsigned row_bytes = (unsigned)p.W * (unsigned)sizeof(IO);
+    // GIVEN: the tiles hold the 128 channels of this workgroup's four slabs, not the block's K range
+    const int group_col = GIVEN ? (w.unit % p.groups) * KC : 0;
+    const int x_col = GIVEN ? w.k * p.bw + group_col : w.tile_col;
+    const unsigned u_row_bytes = 2u * (unsigned)p.bw * (unsigned)sizeof(IO);   // a row of `pre`: W_a x | W_x x of one block
     unsigned pre_off[NV];                                // lane offsets inside a tile (fixed)
+    unsigned u_off[GIVEN ? NV : 1];
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int idx = tid + i * kThreads;
       const int row = idx / VPR, cv = idx - row * VPR;
-      pre_off[i] = (idx < TR * VPR) ? (unsigned)row * row_bytes + (unsigned)(w.tile_col + cv * Tr::HW) * (unsigned)sizeof(IO)
+      pre_off[i] = (idx < TR * VPR) ? (unsigned)row * row_bytes + (unsigned)(x_col + cv * Tr::HW) * (unsigned)sizeof(IO)
+                                    : kOutOfRange;
+      if constexpr (GIVEN)
+        u_off[i] = (idx < TR * VPR) ? (unsigned)row * u_row_bytes + (unsigned)(group_col + cv * Tr::HW) * (unsigned)sizeof(IO)
                                     : kOutOfRange;
     }
     auto issue = [&](long long tk_in) {
@@ -497,6 +511,17 @@ __global__ __launch_bounds__(kThreads, 2) void fwd_kernel(FusedArgs p) {
       const rsrc_t rx = make_rsrc(x + ((long long)b * p.T + (long long)c * TR) * W, (unsigned)rows * row_bytes);
 #pragma unroll
       for (int i = 0; i < NV; ++i) pre[i] = buf_load_frag<Frag>(rx, pre_off[i]);
+      if constexpr (GIVEN) {
+        // the x-gate half of a row starts bw elements after the a-gate half
+        const IO* ubase = (const IO*)p.pre + ((long long)w.k * p.rows_total + (long long)b * p.T + (long long)c * TR) * (2 * p.bw);
+        const rsrc_t ru = make_rsrc(ubase, (unsigned)rows * u_row_bytes);
+        const unsigned half = (unsigned)p.bw * (unsigned)sizeof(IO);
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+          pre_a[i] = buf_load_frag<Frag>(ru, u_off[i]);
+          pre_x[i] = buf_load_frag<Frag>(ru, u_off[i] == kOutOfRange ? kOutOfRange : u_off[i] + half);
+        }
+      }
     };
     if (tid == 0) s_ticket[0] = atomicAdd(q.counter, 1u);
     __syncthreads();
@@ -536,7 +561,13 @@ __global__ __launch_bounds__(kThreads, 2) void fwd_kernel(FusedArgs p) {
       for (int i = 0; i < NV; ++i) {
         const int idx = tid + i * kThreads;
         const int row = idx / VPR, cv = idx - row * VPR;
-        if (idx < TR * VPR) *reinterpret_cast<Frag*>(lds + row * LDSROW + cv * Tr::HW) = pre[i];
+        if (idx < TR * VPR) {
+          *reinterpret_cast<Frag*>(lds + row * LDSROW + cv * Tr::HW) = pre[i];
+          if constexpr (GIVEN) {
+            *reinterpret_cast<Frag*>(lds_pre + row * LDSROW + cv * Tr::HW) = pre_a[i];
+            *reinterpret_cast<Frag*>(lds_pre + (TR + row) * LDSROW + cv * Tr::HW) = pre_x[i];
+          }
+        }
       }
       __syncthreads();
       RGLRU_STAMP(p, 1);
@@ -545,6 +576,17 @@ __global__ __launch_bounds__(kThreads, 2) void fwd_kernel(FusedArgs p) {
         for (int mt = 0; mt < MT; ++mt) {
           f32x16 ua, ux;
           float xv[16];
+          if constexpr (GIVEN) {
+            static_assert(MT == 1, "one accumulator tile per wave");
+            const int col = w.wave * 32 + w.r;
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+              const int at = (hf * 16 + e) * LDSROW + col;
+              xv[e] = (float)lds[at];
+              ua[e] = bias_a + (float)lds_pre[at];
+              ux[e] = bias_x + (float)lds_pre[TR * LDSROW + at];
+            }
+          } else
           gate_mfma_held<IO, MT, NKG, KC>(lds, hw, mt, w.slab, w.r, hf, bias_a, bias_x, ua, ux, xv, NKG == 8 ? 0 : w.kb);
           fwd_gates<IO, MASKED>(p, trow + 16 * mt, cur.c * TR + hf * EL + 16 * mt, ua, ux, xv, sp, cur.a + 16 * mt, cur.z + 16 * mt);
         }
@@ -765,14 +807,19 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
   constexpr int MT = 1, TR = 32, EL = 16;
   typedef Io<IO> Tr;
   typedef typename Tr::Frag Frag;
-  constexpr int KC = NKG * Tr::KG;                       // block width
+  // NKG < 0: the caller supplies the gate pre-activations (see fwd_kernel) and gets the gradients at
+  // them back as two halves per block, [nb][B*T][du_a (bw) | du_x (bw)], the operand layout of the
+  // two GEMMs it runs afterwards; no weights are read here.
+  constexpr bool GIVEN = NKG < 0;
+  constexpr int KC = (GIVEN ? 8 : NKG) * Tr::KG;         // block width (held weights)
   constexpr int TW = kPackedWidth;                       // tile width (narrow blocks are packed)
   constexpr int LDSROW = TW + Tr::HW;
-  static_assert(sizeof(IO) == 2 && NKG > 0, "fast backward is for 16-bit storage with held weights");
+  static_assert(sizeof(IO) == 2 && NKG != 0, "fast backward is for 16-bit storage");
   __shared__ __attribute__((aligned(16))) IO lds_x[TR * LDSROW];
   __shared__ __attribute__((aligned(16))) IO lds_dy[TR * LDSROW];
+  __shared__ __attribute__((aligned(16))) IO lds_pre[GIVEN ? 2 * TR * LDSROW : Tr::HW];
   __shared__ __attribute__((aligned(16))) unsigned char stage_dx_all[kWaves * WaveStage<TR>::kBytes];
-  __shared__ __attribute__((aligned(16))) unsigned char stage_du_all[kWaves * PairStage<TR>::kBytes];
+  __shared__ __attribute__((aligned(16))) unsigned char stage_du_all[kWaves * (GIVEN ? 2 * WaveStage<TR>::kBytes : PairStage<TR>::kBytes)];
   __shared__ unsigned s_ticket[2];
   // With 128-channel blocks the weight registers (64) push the kernel into spilling; the input
   // gate's weights then live in LDS instead (one copy per workgroup, read as B fragments per tile).
@@ -783,7 +830,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
   const WaveId w = wave_identity(p, blockIdx.x);
   const int hf = w.hf, tid = threadIdx.x;
   unsigned char* stage_dx = stage_dx_all + w.wave * WaveStage<TR>::kBytes;
-  unsigned char* stage_du = stage_du_all + w.wave * PairStage<TR>::kBytes;
+  unsigned char* stage_du = stage_du_all + w.wave * (GIVEN ? 2 * WaveStage<TR>::kBytes : PairStage<TR>::kBytes);
   const IO* wg = (const IO*)p.wg;
   const int o_safe = w.slab_ok ? w.o : 0;
   const IO* w_a_row = wg + ((long long)(0 * p.nb + w.k) * p.bwp + o_safe) * p.bwp + hf * Tr::HW;
@@ -799,7 +846,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
       *reinterpret_cast<Frag*>(lds_wx + row * WROW + v * Tr::HW) = *reinterpret_cast<const Frag*>(src + (long long)row * p.bwp + v * Tr::HW);
     }
     __syncthreads();
-  } else {
+  } else if constexpr (!GIVEN) {
     hw.load(w_a_row, w_x_row);
   }
   const float bias_a = p.bias[w.kp], bias_x = p.bias[p.Wp + w.kp];
@@ -813,13 +860,19 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
 
   constexpr int VPR = TW / Tr::HW;
   constexpr int NV = (TR * VPR + kThreads - 1) / kThreads;
-  Frag pre_x[NV], pre_dy[NV];
-  unsigned pre_off[NV];
+  Frag pre_x[NV], pre_dy[NV], pre_ua[GIVEN ? NV : 1], pre_ux[GIVEN ? NV : 1];
+  unsigned pre_off[NV], u_off[GIVEN ? NV : 1];
+  // GIVEN: the tiles hold the 128 channels of this workgroup's four slabs
+  const int group_col = GIVEN ? (w.unit % p.groups) * TW : 0;
+  const int x_col = GIVEN ? w.k * p.bw + group_col : w.tile_col;
+  const unsigned u_row_bytes = 4u * (unsigned)p.bw;      // a row of `pre` and of du: two halves of bw 16-bit values
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
     const int idx = tid + i * kThreads;
     const int row = idx / VPR, cv = idx - row * VPR;
-    pre_off[i] = (idx < TR * VPR) ? (unsigned)row * row_bytes + (unsigned)(w.tile_col + cv * Tr::HW) * 2u : kOutOfRange;
+    pre_off[i] = (idx < TR * VPR) ? (unsigned)row * row_bytes + (unsigned)(x_col + cv * Tr::HW) * 2u : kOutOfRange;
+    if constexpr (GIVEN)
+      u_off[i] = (idx < TR * VPR) ? (unsigned)row * u_row_bytes + (unsigned)(group_col + cv * Tr::HW) * 2u : kOutOfRange;
   }
   auto decode = [&](unsigned tk, int& c, int& b) {
     const unsigned cr = tk / (unsigned)q.n_b;
@@ -837,6 +890,15 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
     const rsrc_t rdy = make_rsrc(dy + first, (unsigned)rows * row_bytes);
 #pragma unroll
     for (int i = 0; i < NV; ++i) { pre_x[i] = buf_load_frag<Frag>(rx, pre_off[i]); pre_dy[i] = buf_load_frag<Frag>(rdy, pre_off[i]); }
+    if constexpr (GIVEN) {
+      const IO* ubase = (const IO*)p.pre + ((long long)w.k * p.rows_total + (long long)b * p.T + (long long)c * TR) * (2 * p.bw);
+      const rsrc_t ru = make_rsrc(ubase, (unsigned)rows * u_row_bytes);
+#pragma unroll
+      for (int i = 0; i < NV; ++i) {
+        pre_ua[i] = buf_load_frag<Frag>(ru, u_off[i]);
+        pre_ux[i] = buf_load_frag<Frag>(ru, u_off[i] == kOutOfRange ? kOutOfRange : u_off[i] + 2u * (unsigned)p.bw);
+      }
+    }
   };
 
   if (tid == 0) s_ticket[0] = atomicAdd(q.counter, 1u);
@@ -862,13 +924,27 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
       if (idx < TR * VPR) {
         *reinterpret_cast<Frag*>(lds_x + row * LDSROW + cv * Tr::HW) = pre_x[i];
         *reinterpret_cast<Frag*>(lds_dy + row * LDSROW + cv * Tr::HW) = pre_dy[i];
+        if constexpr (GIVEN) {
+          *reinterpret_cast<Frag*>(lds_pre + row * LDSROW + cv * Tr::HW) = pre_ua[i];
+          *reinterpret_cast<Frag*>(lds_pre + (TR + row) * LDSROW + cv * Tr::HW) = pre_ux[i];
+        }
       }
     }
     __syncthreads();
     f32x16 ua, ux;
     float xv[EL], gy[EL];
     if (w.slab_ok) {
-      if constexpr (XLDS) {
+      if constexpr (GIVEN) {
+        const int col = w.wave * 32 + w.r;
+#pragma unroll
+        for (int e = 0; e < EL; ++e) {
+          const int at = (hf * EL + e) * LDSROW + col;
+          xv[e] = (float)lds_x[at];
+          gy[e] = (float)lds_dy[at];
+          ua[e] = bias_a + (float)lds_pre[at];
+          ux[e] = bias_x + (float)lds_pre[TR * LDSROW + at];
+        }
+      } else if constexpr (XLDS) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) { ua[v] = bias_a; ux[v] = bias_x; }
         const IO* xrow = lds_x + tile_row<MT>(0, w.r) * LDSROW + hf * Tr::HW;
@@ -884,8 +960,10 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
       } else {
         gate_mfma_held<IO, MT, NKG, TW>(lds_x, hw, 0, w.slab, w.r, hf, bias_a, bias_x, ua, ux, xv, w.kb);
       }
+      if constexpr (!GIVEN) {
 #pragma unroll
-      for (int e = 0; e < EL; ++e) gy[e] = (float)lds_dy[(hf * EL + e) * LDSROW + (NKG == 8 ? 0 : w.kb) + w.slab * 32 + w.r];
+        for (int e = 0; e < EL; ++e) gy[e] = (float)lds_dy[(hf * EL + e) * LDSROW + (NKG == 8 ? 0 : w.kb) + w.slab * 32 + w.r];
+      }
     }
     if (tid == 0) s_ticket[par ^ 1] = next_raw;
     __syncthreads();
@@ -957,7 +1035,8 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
     for (int e = EL - 1; e >= 0; --e) { const float d = gy[e] + carry; gy[e] = d; carry = a[e] * d; }
     float h = hf ? fmaf(A_lo, h_start, H_lo) : h_start;
     unsigned char* my_dx = stage_dx + WaveStage<TR>::row_offset(hf * EL) + w.r * 2;
-    unsigned char* my_du = stage_du + PairStage<TR>::row_offset(hf * EL) + w.r * 4;
+    unsigned char* my_du = GIVEN ? stage_du + WaveStage<TR>::row_offset(hf * EL) + w.r * 2
+                                 : stage_du + PairStage<TR>::row_offset(hf * EL) + w.r * 4;
 #pragma unroll
     for (int e = 0; e < EL; ++e) {
       // With z = g i x, a = exp(l), g = sqrt(1 - a^2) (bounded derivative 1 / (2 max(g, 5e-4))):
@@ -982,15 +1061,26 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
       sum_l = fmaf(dl, re, sum_l);
       sum_ba += va; sum_bx += vx;
       *reinterpret_cast<IO*>(my_dx + e * WaveStage<TR>::kRowBytes) = (IO)dxd;
-      typedef IO io2 __attribute__((ext_vector_type(2)));
-      io2 pair; pair[0] = (IO)va; pair[1] = (IO)vx;
-      *reinterpret_cast<io2*>(my_du + e * PairStage<TR>::kRowBytes) = pair;
+      if constexpr (GIVEN) {
+        *reinterpret_cast<IO*>(my_du + e * WaveStage<TR>::kRowBytes) = (IO)va;
+        *reinterpret_cast<IO*>(my_du + WaveStage<TR>::kBytes + e * WaveStage<TR>::kRowBytes) = (IO)vx;
+      } else {
+        typedef IO io2 __attribute__((ext_vector_type(2)));
+        io2 pair; pair[0] = (IO)va; pair[1] = (IO)vx;
+        *reinterpret_cast<io2*>(my_du + e * PairStage<TR>::kRowBytes) = pair;
+      }
     }
     wave_lds_fence();
     {
       const int rows = (p.T - t0) < TR ? (p.T - t0) : TR;
       const rsrc_t rdx = make_rsrc((const IO*)p.dx + ((long long)b * p.T + t0) * W, (unsigned)rows * row_bytes);
       stage_flush<TR>(stage_dx, rdx, row_bytes, (unsigned)(w.k * p.bw + w.slab * 32) * 2u, w.lane);
+      if constexpr (GIVEN) {
+        IO* dbase = (IO*)p.du_a + ((long long)w.k * p.rows_total + (long long)b * p.T + t0) * (2 * p.bw);
+        const rsrc_t rdu = make_rsrc(dbase, (unsigned)rows * u_row_bytes);
+        stage_flush<TR>(stage_du, rdu, u_row_bytes, (unsigned)(w.slab * 32) * 2u, w.lane);
+        stage_flush<TR>(stage_du + WaveStage<TR>::kBytes, rdu, u_row_bytes, (unsigned)(p.bw + w.slab * 32) * 2u, w.lane);
+      } else {
       const unsigned du_row_bytes = 2u * row_bytes;
       const rsrc_t rdu = make_rsrc((const IO*)p.du_a + ((long long)b * p.T + t0) * 2 * W, (unsigned)rows * du_row_bytes);
       const unsigned du_col = (unsigned)(w.k * 2 * p.bw + w.slab * 64) * 2u;
@@ -1000,6 +1090,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
         const unsigned seg = (unsigned)(w.lane & 7) * 16u;
         i32x4 v = *reinterpret_cast<const i32x4*>(stage_du + PairStage<TR>::row_offset(row) + seg);
         buf_store_b128(v, rdu, (unsigned)row * du_row_bytes + du_col + seg);
+      }
       }
     }
     wave_lds_fence();
@@ -1398,6 +1489,8 @@ static int held_groups(const Geometry& g, int dtype, int aligned) {
     else if ((dtype) == RGLRU_BF16 && (nkg) == 4) hipLaunchKernelGGL((fwd_kernel<__bf16, 4, true>), grid, dim3(kThreads), 0, stream, args); \
     else if ((dtype) == RGLRU_BF16 && (nkg) == 2 && !(masked)) hipLaunchKernelGGL((fwd_kernel<__bf16, 2, false>), grid, dim3(kThreads), 0, stream, args); \
     else if ((dtype) == RGLRU_BF16 && (nkg) == 2) hipLaunchKernelGGL((fwd_kernel<__bf16, 2, true>), grid, dim3(kThreads), 0, stream, args); \
+    else if ((dtype) == RGLRU_BF16 && (nkg) < 0 && !(masked)) hipLaunchKernelGGL((fwd_kernel<__bf16, -1, false>), grid, dim3(kThreads), 0, stream, args); \
+    else if ((dtype) == RGLRU_BF16 && (nkg) < 0) hipLaunchKernelGGL((fwd_kernel<__bf16, -1, true>), grid, dim3(kThreads), 0, stream, args); \
     else if ((dtype) == RGLRU_BF16) hipLaunchKernelGGL((fwd_kernel<__bf16, 0, true>), grid, dim3(kThreads), 0, stream, args); \
     else hipLaunchKernelGGL((fwd_kernel<float, 0, true>), grid, dim3(kThreads), 0, stream, args);      \
   } while (0)
@@ -1518,7 +1611,8 @@ size_t rglru_hip_bwd_scratch_bytes(int64_t B, int64_t T, int64_t W, int64_t nb, 
 
 static int fwd_impl(const void* x, const void* prep, const float* h0, const uint8_t* flags,
                     void* y, float* h_last, void* ws,
-                    int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, bool cleared, void* stream) {
+                    int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, bool cleared, void* stream,
+                    const void* pre = nullptr) {
   int rc = check_geometry("fwd", W, nb, dtype);
   if (rc) return rc;
   if (B <= 0 || T <= 0) return fail(RGLRU_E_ARG, "fwd: B and T must be positive (got %lld, %lld)", (long long)B, (long long)T);
@@ -1545,7 +1639,13 @@ static int fwd_impl(const void* x, const void* prep, const float* h0, const uint
 #ifdef RGLRU_TRACE
   a.trace = g_trace;
 #endif
-  const int nkg = held_groups(g, dtype, a.aligned);
+  int nkg = held_groups(g, dtype, a.aligned);
+  if (pre) {
+    if (!rglru_hip_pre_path(W, nb, dtype)) return fail(RGLRU_E_UNSUPPORTED, "fwd_pre: needs bf16 storage and gate blocks of a multiple of 32 channels");
+    if (!a.aligned || (uintptr_t)pre % 16) return fail(RGLRU_E_UNSUPPORTED, "fwd_pre: x, pre and y must be 16-byte aligned");
+    a.pre = pre; a.rows_total = B * T;
+    nkg = -1;
+  }
   pack_units(a, g, nkg);
   a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nCf, 2, 1 << 20);
   a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
@@ -1562,6 +1662,73 @@ int rglru_hip_fwd(const void* x, const void* prep, const float* h0, const uint8_
                   void* y, float* h_last, void* ws,
                   int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, void* stream) {
   return fwd_impl(x, prep, h0, flags, y, h_last, ws, B, T, W, nb, dtype, false, stream);
+}
+
+static int check_grad_dtype(const char* who, int grad_dtype);
+
+int rglru_hip_pre_path(int64_t W, int64_t nb, int dtype) {
+  if (dtype != RGLRU_BF16 || W <= 0 || nb <= 0 || W % nb) return 0;
+  const int64_t bw = W / nb;
+  return (bw % 32 == 0 && bw <= 512) ? 1 : 0;
+}
+
+int rglru_hip_fwd_pre(const void* x, const void* pre, const void* prep, const float* h0, const uint8_t* flags,
+                      void* y, float* h_last, void* ws,
+                      int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, void* stream) {
+  if (!pre) return fail(RGLRU_E_ARG, "fwd_pre: null pointer");
+  return fwd_impl(x, prep, h0, flags, y, h_last, ws, B, T, W, nb, dtype, false, stream, pre);
+}
+
+int rglru_hip_bwd_pre(const void* x, const void* pre, const void* prep, const float* h0,
+                      const uint8_t* flags, const void* dy, const float* dh_last, void* ws, void* scratch,
+                      void* dx, void* du, void* db_a, void* db_x, void* dlambda, float* dh0,
+                      int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, int grad_dtype, void* stream) {
+  int rc = check_geometry("bwd_pre", W, nb, dtype);
+  if (rc) return rc;
+  rc = check_grad_dtype("bwd_pre", grad_dtype);
+  if (rc) return rc;
+  if (!rglru_hip_pre_path(W, nb, dtype)) return fail(RGLRU_E_UNSUPPORTED, "bwd_pre: needs bf16 storage and gate blocks of a multiple of 32 channels");
+  if (B <= 0 || T <= 0) return fail(RGLRU_E_ARG, "bwd_pre: B and T must be positive (got %lld, %lld)", (long long)B, (long long)T);
+  if (!x || !pre || !prep || !dy || !ws || !scratch || !dx || !du || !db_a || !db_x || !dlambda)
+    return fail(RGLRU_E_ARG, "bwd_pre: null pointer");
+  if (B * T * W >= (1ll << 40) || B * T >= (1ll << 31)) return fail(RGLRU_E_UNSUPPORTED, "bwd_pre: tensor too large");
+  Geometry g = make_geometry(W, nb);
+  if (!is_aligned(x, W, g.bw, 2) || !is_aligned(dy, W, g.bw, 2) || !is_aligned(dx, W, g.bw, 2) ||
+      (uintptr_t)pre % 16 || (uintptr_t)du % 16)
+    return fail(RGLRU_E_UNSUPPORTED, "bwd_pre: x, pre, dy, dx and du must be 16-byte aligned");
+  WorkLayout L = make_work_layout(B, T, g);
+  hipStream_t s = (hipStream_t)stream;
+  char* wb = (char*)ws;
+  FusedArgs a;
+  memset(&a, 0, sizeof(a));
+  fill_common(a, g, prep, dtype);
+  a.x = x; a.pre = pre; a.rows_total = B * T; a.h0 = h0; a.flags = flags; a.dy = dy; a.dh_last = dh_last;
+  a.flags_vec = (T % 16 == 0) && ((uintptr_t)flags % 16 == 0);
+  a.dx = dx; a.du_a = du; a.dh0 = dh0;
+  a.ckpt = (float*)(wb + L.ckpt); a.rec_a = (rec_t*)(wb + L.b_rec_a);
+  a.ticket = (unsigned*)(wb + L.b_ticket); a.fail = (unsigned*)(wb + L.fail);
+  a.partial = (float*)((char*)scratch + make_scratch_layout(B, T, g, false).partial);
+  a.B = (int)B; a.T = (int)T; a.nC = (int)((T + kChunk - 1) / kChunk); a.ckpt_nC = (int)L.nC;
+  a.aligned = 1;
+  a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nC, 2, L.max_wg);
+  a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
+  const bool masked = (flags != nullptr) || (T % kChunk != 0);
+  dim3 grid((unsigned)(a.wg_per_unit * a.units));
+  {
+    KernelTimer timer(1, s);
+    if (masked) hipLaunchKernelGGL((bwd_scan_kernel<__bf16, -1, true>), grid, dim3(kThreads), 0, s, a);
+    else hipLaunchKernelGGL((bwd_scan_kernel<__bf16, -1, false>), grid, dim3(kThreads), 0, s, a);
+  }
+  rc = check_launch("bwd_pre scan");
+  if (rc) return rc;
+  FinishArgs r;
+  memset(&r, 0, sizeof(r));
+  r.partial = a.partial; r.dsp = finish_dsp(g, prep, dtype); r.db_a = db_a; r.db_x = db_x; r.dlambda = dlambda;
+  r.W = (int)W; r.nb = (int)nb; r.bw = (int)g.bw; r.bwp = (int)g.bwp; r.Wp = (int)g.Wp; r.wg_per_unit = a.wg_per_unit;
+  r.vec_blocks = (int)((W + 15) / 16); r.grad_dtype = grad_dtype;
+  r.clean = (uint4*)(wb + L.b_begin); r.clean_n = (long long)((L.b_end - L.b_begin) / 16);
+  hipLaunchKernelGGL(finish_kernel, dim3((unsigned)r.vec_blocks), dim3(256), 0, s, r);
+  return check_launch("bwd_pre finish");
 }
 
 int rglru_hip_prepare_fwd(const void* w_a, const void* b_a, const void* w_x, const void* b_x,

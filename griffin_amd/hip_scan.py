@@ -184,6 +184,23 @@ def _check_fused_inputs(x: Tensor, w_a: Tensor, h0: Tensor | None, flags: Tensor
     _dtype_code(x.dtype)
 
 
+def _uses_pre_path(lib, x: Tensor, W: int, nb: int, code: int) -> bool:
+    """Blocks the kernels cannot hold the weights of (and other widths that are a multiple of 32):
+    the gate projections run as one library GEMM, everything else in the HIP kernels."""
+    return bool(not lib.rglru_hip_fast_path(W, nb, code) and lib.rglru_hip_pre_path(W, nb, code)
+                and x.data_ptr() % 16 == 0)
+
+
+def _gate_projections(x: Tensor, w_a: Tensor, w_x: Tensor) -> tuple[Tensor, Tensor, Tensor]:
+    """pre[k][n] = [W_a[k] x[n, k] | W_x[k] x[n, k]] as one batched GEMM (griffin/griffin.py:149-154
+    without the bias).  Returns (pre [nb, n, 2 bw], the stacked weights [nb, 2 bw, bw], x as [nb, n, bw])."""
+    nb, bw, _ = w_a.shape
+    n = x.shape[0] * x.shape[1]
+    stacked = torch.cat((w_a.detach().to(x.dtype), w_x.detach().to(x.dtype)), dim=1)
+    xk = x.view(n, nb, bw).transpose(0, 1)
+    return torch.bmm(xk, stacked.transpose(1, 2)), stacked, xk
+
+
 class _HipRGLRU(torch.autograd.Function):
     """y, h_T = RG-LRU(x; W_a, b_a, W_x, b_x, Lambda) with a recomputing backward."""
 
@@ -204,11 +221,20 @@ class _HipRGLRU(torch.autograd.Function):
             h_last = torch.empty(B, W, dtype=torch.float32, device=device)
             image = torch.empty(_prep_bytes(W, nb, code), dtype=torch.uint8, device=device)
             ws = torch.empty(lib.rglru_hip_workspace_bytes(B, T, W, nb), dtype=torch.uint8, device=device)
-            # parameter conversion, workspace clearing and the forward kernel: two launches
-            _lib.check(lib.rglru_hip_prepare_fwd(*(t.data_ptr() for t in operands), float(c), vec_code, image.data_ptr(),
-                                                 x.data_ptr(), _ptr(h0c), _ptr(flags), y.data_ptr(), h_last.data_ptr(),
-                                                 ws.data_ptr(), B, T, W, nb, code, _stream_ptr(device)),
-                       "rglru_hip_prepare_fwd")
+            if _uses_pre_path(lib, x, W, nb, code):
+                pre, _, _ = _gate_projections(x, w_a, w_x)
+                _lib.check(lib.rglru_hip_prepare(*(t.data_ptr() for t in operands), float(c), W, nb, code, vec_code,
+                                                 image.data_ptr(), _stream_ptr(device)), "rglru_hip_prepare")
+                _lib.check(lib.rglru_hip_fwd_pre(x.data_ptr(), pre.data_ptr(), image.data_ptr(), _ptr(h0c), _ptr(flags),
+                                                 y.data_ptr(), h_last.data_ptr(), ws.data_ptr(), B, T, W, nb, code,
+                                                 _stream_ptr(device)), "rglru_hip_fwd_pre")
+                del pre
+            else:
+                # parameter conversion, workspace clearing and the forward kernel: two launches
+                _lib.check(lib.rglru_hip_prepare_fwd(*(t.data_ptr() for t in operands), float(c), vec_code,
+                                                     image.data_ptr(), x.data_ptr(), _ptr(h0c), _ptr(flags),
+                                                     y.data_ptr(), h_last.data_ptr(), ws.data_ptr(), B, T, W, nb, code,
+                                                     _stream_ptr(device)), "rglru_hip_prepare_fwd")
         ctx.save_for_backward(x, w_a, w_x, h0c, flags, ws, image)
         ctx.param_dtypes = (w_a.dtype, b_a.dtype, w_x.dtype, b_x.dtype, lam.dtype)
         ctx.h0_dtype = None if h0 is None else h0.dtype
@@ -248,6 +274,20 @@ class _HipRGLRU(torch.autograd.Function):
                                                   dw_x.data_ptr(), db_a.data_ptr(), db_x.data_ptr(), dlam.data_ptr(),
                                                   _ptr(dh0), B, T, W, nb, code, gcode, _stream_ptr(device)),
                            "rglru_hip_bwd_full")
+            elif _uses_pre_path(lib, x, W, nb, code) and dy.data_ptr() % 16 == 0:
+                # gate projections recomputed by the library GEMM, the scan and all gate math in the
+                # HIP kernel, then the two GEMMs of the gate gradients on the kernel's du
+                pre, stacked, xk = _gate_projections(x, w_a, w_x)
+                du = torch.empty_like(pre)
+                _lib.check(lib.rglru_hip_bwd_pre(x.data_ptr(), pre.data_ptr(), image.data_ptr(), _ptr(h0c), _ptr(flags),
+                                                 dy.data_ptr(), _ptr(dhl), ws.data_ptr(), scratch.data_ptr(), dx.data_ptr(),
+                                                 du.data_ptr(), db_a.data_ptr(), db_x.data_ptr(), dlam.data_ptr(),
+                                                 _ptr(dh0), B, T, W, nb, code, gcode, _stream_ptr(device)),
+                           "rglru_hip_bwd_pre")
+                del pre
+                dw = torch.bmm(du.transpose(1, 2), xk)                 # [nb, 2 bw, bw] = [dW_a ; dW_x]
+                dw_a, dw_x = dw[:, :bw], dw[:, bw:]
+                dx.view(B * T, nb, bw).transpose(0, 1).add_(torch.bmm(du, stacked))
             else:
                 du_a = torch.empty_like(x)
                 du_x = torch.empty_like(x)

@@ -10,6 +10,7 @@
  *   griffin/triton_scan.py:246-271  _FusedRGLRUScan.backward  rglru_hip_scan_bwd
  *   griffin/griffin.py:237-289      RG_LRU.forward (gates + scan, T > 1)   rglru_hip_prepare + rglru_hip_fwd
  *   autograd of griffin/griffin.py:237-289                                   rglru_hip_bwd, rglru_hip_bwd_full
+ *   the same with the gate projections (griffin/griffin.py:149-154) left to a BLAS GEMM   rglru_hip_fwd_pre, rglru_hip_bwd_pre
  *   griffin/griffin.py:279-284 with T == 1 (decode step, carried state)     rglru_hip_step
  *   griffin/griffin.py:474-487      causal depthwise convolution of the caller   rglru_hip_conv_fwd
  *   autograd of griffin/griffin.py:474-487                                   rglru_hip_conv_bwd
@@ -42,7 +43,7 @@
 extern "C" {
 #endif
 
-#define RGLRU_ABI_VERSION 4
+#define RGLRU_ABI_VERSION 5
 
 enum { RGLRU_F32 = 0, RGLRU_BF16 = 1 };
 
@@ -139,6 +140,29 @@ int rglru_hip_bwd_full(const void* x, const void* prep, const float* h0,
                        void* dx, void* dw_a, void* dw_x, void* db_a, void* db_x, void* dlambda,
                        float* dh0, int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, int grad_dtype,
                        void* stream);
+
+/* Variant for gate blocks too wide for the kernels to keep their weights on chip (and for any block
+ * width that is a multiple of 32 channels up to 512, bf16 storage, 16-byte aligned tensors;
+ * rglru_hip_pre_path() says whether a configuration qualifies).  The caller runs the two block-diagonal
+ * projections of griffin/griffin.py:149-154 as ONE batched GEMM of its BLAS library and hands the
+ * result in:
+ *   pre[nb][B*T][2*bw] (dtype):  pre[k][n][o] = sum_j W_a[k][o][j] x[n][k*bw+j],
+ *                                pre[k][n][bw+o] = the same with W_x        (biases NOT added)
+ * rglru_hip_fwd_pre is rglru_hip_fwd with that operand.  rglru_hip_bwd_pre takes the same `pre`
+ * (recomputed by the caller), writes the direct part of the input gradient into dx[B,T,W] and the
+ * gradients at the pre-activations into du[nb][B*T][2*bw] (dtype; same two halves), plus db_a, db_x,
+ * dlambda (grad_dtype) and dh0; the caller finishes with two batched GEMMs:
+ *   dx[n][k*bw+j] += sum_o du[k][n][o] W_a[k][o][j] + du[k][n][bw+o] W_x[k][o][j]
+ *   dW_a[k][o][j] = sum_n du[k][n][o] x[n][k*bw+j],  dW_x likewise from the second half.
+ * `prep`, `ws` and `scratch` (rglru_hip_bwd_scratch_bytes) are those of rglru_hip_fwd / rglru_hip_bwd. */
+int rglru_hip_pre_path(int64_t W, int64_t nb, int dtype);
+int rglru_hip_fwd_pre(const void* x, const void* pre, const void* prep, const float* h0, const uint8_t* flags,
+                      void* y, float* h_last, void* ws,
+                      int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, void* stream);
+int rglru_hip_bwd_pre(const void* x, const void* pre, const void* prep, const float* h0,
+                      const uint8_t* flags, const void* dy, const float* dh_last, void* ws, void* scratch,
+                      void* dx, void* du, void* db_a, void* db_x, void* dlambda, float* dh0,
+                      int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, int grad_dtype, void* stream);
 
 /* One decode step (T == 1): h[B,W] fp32 is updated in place, y[B,W] (dtype) = h as stored. */
 int rglru_hip_step(const void* x, const void* prep, float* h, const uint8_t* flags, void* y,

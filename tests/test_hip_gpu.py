@@ -117,7 +117,10 @@ BF16_CASES = [
     (3, 17, 128, 2, True, True),     # shorter than one tile    (2, 100, 192, 3, True, True),    # 64-wide blocks packed two to a unit, last unit half empty
     (2, 70, 96, 3, False, True),     # 32-wide blocks packed four to a unit, last unit one block short
     (1, 64, 64, 1, False, False),    # a single 64-wide block: half of the packed unit idles
-    (2, 64, 1024, 16, True, False),  # reference default of 16 gate blocks at width 1024
+    (2, 64, 1024, 16, True, False),  # reference default of 16 gate blocks at width 1024    (2, 100, 512, 2, True, True),    # 256-wide blocks: library GEMM for the projections, two workgroups per block
+    (2, 75, 480, 3, False, True),    # 160-wide blocks: five slabs, the second workgroup of a block has one
+    (1, 64, 96, 1, True, False),     # 96-wide block: three slabs in one workgroup
+    (3, 33, 384, 2, True, True),     # 192-wide blocks, ragged tile, flags
 ]
 
 
