@@ -287,7 +287,8 @@ class _HipRGLRU(torch.autograd.Function):
                 del pre
                 dw = torch.bmm(du.transpose(1, 2), xk)                 # [nb, 2 bw, bw] = [dW_a ; dW_x]
                 dw_a, dw_x = dw[:, :bw], dw[:, bw:]
-                dx.view(B * T, nb, bw).transpose(0, 1).add_(torch.bmm(du, stacked))
+                dx_blocks = dx.view(B * T, nb, bw).transpose(0, 1)     # [nb, n, bw], row stride W: written in place
+                torch.baddbmm(dx_blocks, du, stacked, out=dx_blocks)
             else:
                 du_a = torch.empty_like(x)
                 du_x = torch.empty_like(x)
