@@ -165,7 +165,10 @@ RGLRU_DEVICE float xhalf(float v, int hf) {
 // record a wave waits for belongs to a wave that is already running.
 // ------------------------------------------------------------------------------------------
 typedef unsigned long long rec_t;
-constexpr int kDepth = 8;
+#ifndef RGLRU_DEPTH
+#define RGLRU_DEPTH 2
+#endif
+constexpr int kDepth = RGLRU_DEPTH;
 
 RGLRU_DEVICE void rec_store(rec_t* p, float a, float h) {
   const rec_t bits = ((rec_t)__float_as_uint(h) << 32) | (rec_t)(__float_as_uint(a) | 1u);

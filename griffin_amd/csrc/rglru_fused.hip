@@ -1647,7 +1647,8 @@ static int fwd_impl(const void* x, const void* prep, const float* h0, const uint
     nkg = -1;
   }
   pack_units(a, g, nkg);
-  a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nCf, 2, 1 << 20);
+  // without weights in registers three workgroups fit a compute unit
+  a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nCf, nkg < 0 ? 3 : 2, 1 << 20);
   a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
   dim3 grid((unsigned)(a.wg_per_unit * a.units));
   {
