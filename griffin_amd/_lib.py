@@ -14,7 +14,7 @@ RGLRU_BF16 = 1
 FLAG_RESET = 1
 FLAG_INACTIVE = 2
 CHUNK = 32
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 _lock = threading.Lock()
 _lib = None
@@ -48,6 +48,8 @@ _SIGNATURES = {
     "rglru_hip_conv_bwd": (ctypes.c_int, [_P] * 10 + [_I, _I, _I, _I, ctypes.c_int, ctypes.c_int, ctypes.c_int, _P]),
     "rglru_hip_gelu_gate_fwd": (ctypes.c_int, [_P, _P, _P, _I, ctypes.c_int, _P]),
     "rglru_hip_gelu_gate_bwd": (ctypes.c_int, [_P, _P, _P, _P, _P, _I, ctypes.c_int, _P]),
+    "rglru_hip_decode_prepare": (ctypes.c_int, [_P] * 11 + [_I, _I, _I, ctypes.c_int, ctypes.c_int, _P]),
+    "rglru_hip_step_gated": (ctypes.c_int, [_P] * 7 + [_I, _I, _I, ctypes.c_int, _P]),
     "rglru_hip_set_spin_limit": (ctypes.c_int64, [_I]),
     "rglru_hip_set_timing": (ctypes.c_int, [ctypes.c_int]),
     "rglru_hip_kernel_ms": (ctypes.c_float, [ctypes.c_int]),

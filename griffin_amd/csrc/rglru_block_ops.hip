@@ -387,27 +387,85 @@ static bool conv_vector_ok(int64_t W, int dtype, std::initializer_list<const voi
 
 
 // ------------------------------------------------------------------------------------------
+// Everything a single-token step of the recurrent block needs in front of the RG-LRU step kernel,
+// in one launch (griffin/griffin.py:459-510 with one token per row): the row's position
+// (previous + 1, or the one given), its flags for the step kernel (reset at position 0, inactive),
+// the convolved input, the shifted convolution state and the position to carry on.  Without an
+// `active` array the rows follow the all-active path (:476-487: taps masked by the position, the
+// state simply shifted); with one they follow the padded path (:488-510: a document start clears
+// the history first, every tap counts, an inactive row keeps its state and position and gets a
+// zero input).
+// ------------------------------------------------------------------------------------------
+struct DecodeArgs {
+  const void* u; const void* state; const void* taps; const void* bias;
+  const long long* prev_pos; const long long* seg_pos; const unsigned char* active;
+  void* x; void* new_state; long long* new_pos; unsigned char* flags;
+  int B, W, K, nvec, vec_dtype;
+};
+
+template <typename IO, int V, int K>
+__global__ __launch_bounds__(kConvThreads) void decode_prepare_kernel(DecodeArgs p) {
+  typedef ConvRow<IO, V> Row;
+  const long long item = (long long)blockIdx.x * kConvThreads + threadIdx.x;
+  if (item >= (long long)p.B * p.nvec) return;
+  const int vec = (int)(item % p.nvec), b = (int)(item / p.nvec);
+  const int c0 = vec * V;
+  const unsigned es = (unsigned)sizeof(IO), uW = (unsigned)p.W;
+  const bool live = p.active ? p.active[b] != 0 : true;
+  const long long before = p.prev_pos ? p.prev_pos[b] : -1;
+  const long long pos = p.seg_pos ? p.seg_pos[b] : before + (live ? 1 : 0);
+  if (vec == 0) {
+    p.new_pos[b] = live ? pos : before;
+    p.flags[b] = (unsigned char)((live && pos == 0 ? RGLRU_FLAG_RESET : 0u) | (live ? 0u : RGLRU_FLAG_INACTIVE));
+  }
+  const rsrc_t ru = make_rsrc((const IO*)p.u + (long long)b * p.W, uW * es);
+  const rsrc_t rx = make_rsrc((IO*)p.x + (long long)b * p.W, uW * es);
+  const unsigned off = (unsigned)c0 * es;
+  float cur[V], acc[V], hist[K > 1 ? K - 1 : 1][V];          // hist[j] = state row j (oldest first)
+  Row::load(cur, ru, off);
+  const rsrc_t rs = make_rsrc(p.state ? (const IO*)p.state + (long long)b * (K - 1) * p.W : (const IO*)p.u,
+                              p.state ? (unsigned)((K - 1) * p.W) * es : 0u);
+#pragma unroll
+  for (int j = 0; j < K - 1; ++j) Row::load(hist[j], rs, ((unsigned)j * uW + (unsigned)c0) * es);
+  const bool padded = p.active != nullptr;
+  if (padded && live && pos == 0) {                         // griffin/griffin.py:491-492
+#pragma unroll
+    for (int j = 0; j < K - 1; ++j)
+#pragma unroll
+      for (int v = 0; v < V; ++v) hist[j][v] = 0.f;
+  }
+#pragma unroll
+  for (int v = 0; v < V; ++v) {
+    float a = p.bias ? conv_param(p.bias, c0 + v, p.vec_dtype) : 0.f;
+    if (padded || pos >= 0) a = fmaf(cur[v], conv_param(p.taps, (long long)(c0 + v) * K + (K - 1), p.vec_dtype), a);
+#pragma unroll
+    for (int lag = 1; lag < K; ++lag)
+      if (padded || pos >= lag) a = fmaf(hist[K - 1 - lag][v], conv_param(p.taps, (long long)(c0 + v) * K + (K - 1 - lag), p.vec_dtype), a);
+    acc[v] = live ? a : 0.f;
+  }
+  Row::store(acc, rx, off);
+  if (K > 1) {
+    const rsrc_t rn = make_rsrc((IO*)p.new_state + (long long)b * (K - 1) * p.W, (unsigned)((K - 1) * p.W) * es);
+#pragma unroll
+    for (int j = 0; j < K - 1; ++j) {
+      float row[V];
+#pragma unroll
+      for (int v = 0; v < V; ++v) {
+        const float shifted = (j + 1 < K - 1) ? hist[j + 1 < K - 1 ? j + 1 : 0][v] : cur[v];
+        row[v] = live ? shifted : hist[j][v];
+      }
+      Row::store(row, rn, ((unsigned)j * uW + (unsigned)c0) * es);
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------
 // Output gate: out = h * gelu_tanh(v) and its reverse mode, flat over n elements.
 //   gelu_tanh(v) = v/2 * (1 + tanh(u)),  u = sqrt(2/pi) * (v + 0.044715 v^3)
 // A thread handles 16-byte vectors in a grid-stride loop, four vectors requested at a time.
 // ------------------------------------------------------------------------------------------
 constexpr int kGateThreads = 256;
 constexpr int kGateBatch = 4;
-
-struct GeluParts { float gelu, dgelu; };
-RGLRU_DEVICE GeluParts gelu_tanh_parts(float v) {
-  const float k0 = 0.7978845608028654f, k1 = 0.044715f;
-  const float v2 = v * v;
-  const float u = k0 * v * fmaf(k1, v2, 1.0f);
-  // tanh(u) = 1 - 2 / (1 + exp(2u)); exp overflows to +inf for large u, which gives tanh = 1
-  const float e = __builtin_amdgcn_exp2f(u * (2.0f * kLog2e));
-  const float t = 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + e);
-  GeluParts g;
-  g.gelu = 0.5f * v * (1.0f + t);
-  const float du = k0 * fmaf(3.0f * k1, v2, 1.0f);
-  g.dgelu = fmaf(0.5f * v * fmaf(-t, t, 1.0f), du, 0.5f * (1.0f + t));
-  return g;
-}
 
 struct GateArgs { const void* h; const void* v; const void* dout; void* out; void* dh; void* dv; long long n; };
 
@@ -575,6 +633,29 @@ int rglru_hip_gelu_gate_bwd(const void* dout, const void* h, const void* v, void
   memset(&a, 0, sizeof(a));
   a.h = h; a.v = v; a.dout = dout; a.dh = dh; a.dv = dv; a.n = n;
   return gate_launch("gelu_gate_bwd", true, a, dtype, stream);
+}
+
+int rglru_hip_decode_prepare(const void* u, const void* conv_state, const void* taps, const void* bias,
+                             const int64_t* prev_pos, const int64_t* segment_pos, const uint8_t* active,
+                             void* x, void* new_conv_state, int64_t* new_pos, uint8_t* flags,
+                             int64_t B, int64_t W, int64_t K, int dtype, int vec_dtype, void* stream) {
+  int rc = conv_check("decode_prepare", B, 1, W, K, dtype, vec_dtype);
+  if (rc) return rc;
+  if (!u || !taps || !x || !new_pos || !flags || (K > 1 && !new_conv_state))
+    return fail(RGLRU_E_ARG, "decode_prepare: null pointer");
+  DecodeArgs a;
+  memset(&a, 0, sizeof(a));
+  a.u = u; a.state = conv_state; a.taps = taps; a.bias = bias;
+  a.prev_pos = (const long long*)prev_pos; a.seg_pos = (const long long*)segment_pos; a.active = active;
+  a.x = x; a.new_state = new_conv_state; a.new_pos = (long long*)new_pos; a.flags = flags;
+  a.B = (int)B; a.W = (int)W; a.K = (int)K; a.vec_dtype = vec_dtype;
+  const bool vec = conv_vector_ok(W, dtype, {u, conv_state, x, new_conv_state});
+  a.nvec = (int)(vec ? W / (dtype == RGLRU_BF16 ? 8 : 4) : W);
+  const long long items = (long long)B * a.nvec;
+  dim3 grid((unsigned)((items + kConvThreads - 1) / kConvThreads));
+  hipStream_t s = (hipStream_t)stream;
+  RGLRU_CONV_DISPATCH(decode_prepare_kernel, dtype, vec, grid, s, a);
+  return check_launch("decode_prepare");
 }
 
 }  // extern "C"

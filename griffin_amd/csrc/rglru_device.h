@@ -362,6 +362,23 @@ RGLRU_DEVICE GateOut gate_forward(float ua, float ux, float x, float sp, unsigne
   return o;
 }
 
+// gelu_tanh(v) = v/2 * (1 + tanh(u)), u = sqrt(2/pi) * (v + 0.044715 v^3), and its derivative
+// (activation of the recurrent block's second branch, griffin/griffin.py:464).
+struct GeluParts { float gelu, dgelu; };
+RGLRU_DEVICE GeluParts gelu_tanh_parts(float v) {
+  const float k0 = 0.7978845608028654f, k1 = 0.044715f;
+  const float v2 = v * v;
+  const float u = k0 * v * fmaf(k1, v2, 1.0f);
+  // tanh(u) = 1 - 2 / (1 + exp(2u)); exp overflows to +inf for large u, which gives tanh = 1
+  const float e = __builtin_amdgcn_exp2f(u * (2.0f * kLog2e));
+  const float t = 1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + e);
+  GeluParts g;
+  g.gelu = 0.5f * v * (1.0f + t);
+  const float du = k0 * fmaf(3.0f * k1, v2, 1.0f);
+  g.dgelu = fmaf(0.5f * v * fmaf(-t, t, 1.0f), du, 0.5f * (1.0f + t));
+  return g;
+}
+
 template <typename IO> struct Precise { static constexpr bool value = true; };
 template <> struct Precise<__bf16> { static constexpr bool value = false; };
 

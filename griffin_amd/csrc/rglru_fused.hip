@@ -118,7 +118,8 @@ struct FusedArgs {
   void* y; float* h_last;                                 // forward
   const void* dy; const float* dh_last;                   // backward in
   void* dx; void* du_a; void* du_x; float* dh0;           // backward out
-  float* h_state;                                         // decode step (in place)
+  float* h_state; const float* h_prev;                    // decode step: state out, state in (may be the same)
+  const void* gate_v;                                     // decode step: y = h * gelu_tanh(gate_v) when set
   // workspace
   float* ckpt; rec_t* rec_a; unsigned* ticket;
   unsigned* fail; float* partial; float* dw_partial;
@@ -1433,8 +1434,9 @@ __global__ __launch_bounds__(kThreads) void step_kernel(FusedArgs p) {
     unsigned fl = p.flags ? (unsigned)p.flags[row] : 0u;
     GateOut go = gate_forward<Precise<IO>::value, true>(ua[0][e], ux[0][e], xv[e], sp, fl);
     const long long at = row * W + w.ch;
-    float h = fmaf(go.a, p.h_state[at], go.z);
+    float h = fmaf(go.a, p.h_prev[at], go.z);
     p.h_state[at] = h;
+    if (p.gate_v) h *= gelu_tanh_parts((float)((const IO*)p.gate_v)[at]).gelu;
     y[at] = (IO)h;
   }
 }
@@ -1878,18 +1880,18 @@ int rglru_hip_bwd_full(const void* x, const void* prep, const float* h0,
   return check_launch("bwd_full finish");
 }
 
-int rglru_hip_step(const void* x, const void* prep, float* h, const uint8_t* flags, void* y,
-                   int64_t B, int64_t W, int64_t nb, int dtype, void* stream) {
+static int step_impl(const void* x, const void* prep, const float* h_in, float* h, const uint8_t* flags,
+                     const void* gate_v, void* y, int64_t B, int64_t W, int64_t nb, int dtype, void* stream) {
   int rc = check_geometry("step", W, nb, dtype);
   if (rc) return rc;
   if (B <= 0) return fail(RGLRU_E_ARG, "step: B must be positive (got %lld)", (long long)B);
-  if (!x || !prep || !h || !y) return fail(RGLRU_E_ARG, "step: null pointer");
+  if (!x || !prep || !h || !h_in || !y) return fail(RGLRU_E_ARG, "step: null pointer");
   if (B * W >= (1ll << 40)) return fail(RGLRU_E_UNSUPPORTED, "step: tensor too large");
   Geometry g = make_geometry(W, nb);
   FusedArgs a;
   memset(&a, 0, sizeof(a));
   fill_common(a, g, prep, dtype);
-  a.x = x; a.flags = flags; a.y = y; a.h_state = h;
+  a.x = x; a.flags = flags; a.y = y; a.h_state = h; a.h_prev = h_in; a.gate_v = gate_v;
   a.B = (int)B; a.T = 1;
   a.aligned = is_aligned(x, W, g.bw, elem_size(dtype));
   long long row_tiles = (B + 31) / 32;
@@ -1900,6 +1902,16 @@ int rglru_hip_step(const void* x, const void* prep, float* h, const uint8_t* fla
     RGLRU_DISPATCH(step_kernel, grid, s, a, dtype, held_groups(g, dtype, a.aligned));
   }
   return check_launch("step");
+}
+
+int rglru_hip_step(const void* x, const void* prep, float* h, const uint8_t* flags, void* y,
+                   int64_t B, int64_t W, int64_t nb, int dtype, void* stream) {
+  return step_impl(x, prep, h, h, flags, nullptr, y, B, W, nb, dtype, stream);
+}
+
+int rglru_hip_step_gated(const void* x, const void* prep, const float* h_in, float* h_out, const uint8_t* flags,
+                         const void* v, void* out, int64_t B, int64_t W, int64_t nb, int dtype, void* stream) {
+  return step_impl(x, prep, h_in, h_out, flags, v, out, B, W, nb, dtype, stream);
 }
 
 int rglru_hip_set_timing(int enable) { return g_timing.exchange(enable ? 1 : 0); }

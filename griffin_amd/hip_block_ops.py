@@ -156,3 +156,47 @@ class _HipGeluGate(torch.autograd.Function):
 def hip_gelu_gate(h: Tensor, v: Tensor) -> Tensor:
     """``h * gelu(v, approximate="tanh")`` in one pass, differentiable in both arguments."""
     return _HipGeluGate.apply(h, v)
+
+
+def hip_block_decode_step(u: Tensor, v: Tensor, conv_state: Tensor | None, weight: Tensor, bias: Tensor | None,
+                          prev_pos: Tensor | None, segment_pos: Tensor | None, active: Tensor | None,
+                          prep, rnn_state: Tensor | None):
+    """One token per row through conv -> RG-LRU step -> output gate (no autograd), two kernel launches.
+
+    ``u``, ``v`` [B, W]: the block's two projections of the token; ``conv_state`` [B, K-1, W] or None;
+    ``prev_pos`` [B] (None: -1) or explicit ``segment_pos`` [B]; ``active`` [B] uint8 or None (all
+    active); ``prep`` the prepared RG-LRU parameters; ``rnn_state`` [B, W] fp32 or None (zeros).
+    Returns ``(gated [B, W], new_rnn_state, new_conv_state, new_pos)``; the inputs are left untouched.
+    """
+    _require_gpu("hip_block_decode_step", u, v, conv_state, weight, bias, prev_pos, segment_pos, active, rnn_state)
+    if u.dim() != 2 or u.shape != v.shape or u.dtype != v.dtype:
+        raise ValueError("hip_block_decode_step expects two [batch, width] tensors of one dtype")
+    batch, width = u.shape
+    if width != prep.width or u.dtype != prep.dtype:
+        raise ValueError("the prepared RG-LRU parameters do not match the activations")
+    taps_count = weight.size(2)
+    code = _dtype_code(u.dtype)
+    u_c, v_c = u.contiguous(), v.contiguous()
+    state_c = None if conv_state is None or taps_count == 1 else conv_state.to(u.dtype).contiguous()
+    taps = _parameter_operand(weight.detach(), u.dtype)
+    bias_c = None if bias is None else _parameter_operand(bias.detach().to(taps.dtype), u.dtype)
+    device = u.device
+    lib = _lib.load()
+    with torch.cuda.device(device):
+        x_conv = torch.empty_like(u_c)
+        new_conv = u.new_empty(batch, taps_count - 1, width)
+        new_pos = torch.empty(batch, dtype=torch.int64, device=device)
+        flags = torch.empty(batch, dtype=torch.uint8, device=device)
+        h_in = (torch.zeros(batch, width, dtype=torch.float32, device=device) if rnn_state is None
+                else rnn_state.to(torch.float32).contiguous())
+        h_out = torch.empty_like(h_in)
+        out = torch.empty_like(u_c)
+        stream = _stream_ptr(device)
+        _lib.check(lib.rglru_hip_decode_prepare(
+            _ptr(u_c), _ptr(state_c), _ptr(taps), _ptr(bias_c), _ptr(prev_pos), _ptr(segment_pos), _ptr(active),
+            _ptr(x_conv), _ptr(new_conv) if taps_count > 1 else None, _ptr(new_pos), _ptr(flags),
+            batch, width, taps_count, code, _DTYPE_CODES[taps.dtype], stream), "rglru_hip_decode_prepare")
+        _lib.check(lib.rglru_hip_step_gated(
+            _ptr(x_conv), prep.image.data_ptr(), _ptr(h_in), _ptr(h_out), _ptr(flags), _ptr(v_c), _ptr(out),
+            batch, width, prep.blocks, code, stream), "rglru_hip_step_gated")
+    return out, h_out, new_conv, new_pos

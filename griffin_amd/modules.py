@@ -275,6 +275,58 @@ class RecurrentBlock(nn.Module):
             return False
         return self.conv_kernel_size <= hip_block_ops.max_kernel_size()
 
+    def _hip_decode_covers(self, x: Tensor, cache: RecurrentBlockCache | None) -> bool:
+        """Single-token inference takes the two-launch decode path of the HIP library."""
+        if not x.is_cuda or x.dtype not in hip_scan.SUPPORTED_DTYPES or x.numel() == 0:
+            return False
+        if torch.is_grad_enabled():
+            tensors = [x, *self.parameters()]
+            if cache is not None:
+                tensors += [cache.rnn_state, cache.conv_state]
+            if any(t.requires_grad for t in tensors):
+                return False
+        if self.linear_x.weight.dtype != x.dtype or self.linear_y.weight.dtype != x.dtype:
+            return False
+        probe = x.new_empty(x.size(0), 1, self.rnn_width)
+        return self._hip_block_ops_covers(probe)
+
+    def _hip_decode(self, x: Tensor, cache: RecurrentBlockCache | None, segment_pos: Tensor | None,
+                    active_mask: Tensor | None, return_cache: bool):
+        """One token per row (griffin/griffin.py:459-528 with T == 1): positions, convolution, RG-LRU
+        step and output gate in two kernel launches around the three projections."""
+        batch = x.size(0)
+        width = self.rnn_width
+        history = self.conv_kernel_size - 1
+        if segment_pos is not None:
+            if segment_pos.shape != (batch, 1):
+                raise ValueError(f"segment_pos must have shape ({batch}, 1), got {tuple(segment_pos.shape)}")
+            segment_pos = segment_pos.to(device=x.device, dtype=torch.long)[:, 0].contiguous()
+        conv_state = prev_pos = rnn_state = None
+        if cache is not None:
+            conv_state, prev_pos, rnn_state = cache.conv_state, cache.segment_position, cache.rnn_state
+            if conv_state.shape != (batch, history, width):
+                raise ValueError("Recurrent convolution cache has an incompatible shape")
+            if prev_pos.shape != (batch,):
+                raise ValueError("Cached segment positions have an incompatible shape")
+            if rnn_state is not None and rnn_state.shape != (batch, width):
+                raise ValueError(f"ht_minus_1 must have shape ({batch}, {width}), got {tuple(rnn_state.shape)}")
+            prev_pos = prev_pos.to(device=x.device, dtype=torch.long).contiguous()
+        active = None
+        if active_mask is not None and not bool(active_mask.all()):
+            active = active_mask[:, 0].to(torch.uint8).contiguous()
+        gate_input = self.linear_y(x)[:, 0]
+        projected = self.linear_x(x)[:, 0]
+        prep = self.rg_lru._prepared(projected.dtype, projected.device)
+        gated, new_rnn_state, new_conv_state, new_pos = hip_block_ops.hip_block_decode_step(
+            projected, gate_input, conv_state, self.temporal_conv.weight, self.temporal_conv.bias,
+            prev_pos, segment_pos, active, prep, rnn_state)
+        output = self.linear_out(gated).unsqueeze(1)
+        if active is not None:
+            output = output.masked_fill(~active_mask.unsqueeze(-1), 0.0)
+        if return_cache:
+            return output, RecurrentBlockCache(new_rnn_state, new_conv_state, new_pos)
+        return output
+
     def _dense_conv(self, projected: Tensor, conv_state: Tensor, segment_pos: Tensor):
         """All-tokens-active path (griffin/griffin.py:476-487): taps are masked per document."""
         if self._hip_block_ops_covers(projected):
@@ -316,6 +368,8 @@ class RecurrentBlock(nn.Module):
         else:
             active_mask = active_mask.to(device=x.device, dtype=torch.bool)
         previous_position = None if cache is None else cache.segment_position
+        if steps == 1 and self._hip_decode_covers(x, cache):
+            return self._hip_decode(x, cache, segment_pos, None if everything_active else active_mask, return_cache)
         segment_pos = _resolve_segment_positions(
             x, segment_pos, previous_position, None if everything_active else active_mask)
 

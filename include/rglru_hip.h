@@ -15,6 +15,7 @@
  *   griffin/griffin.py:474-487      causal depthwise convolution of the caller   rglru_hip_conv_fwd
  *   autograd of griffin/griffin.py:474-487                                   rglru_hip_conv_bwd
  *   griffin/griffin.py:464, :520    x_branch * gelu_tanh(linear_y(x))        rglru_hip_gelu_gate_fwd, _bwd
+ *   griffin/griffin.py:459-528 with T == 1 (block decode: positions, conv, step, gate)   rglru_hip_decode_prepare + rglru_hip_step_gated
  *
  * Conventions
  *   - every pointer is a DEVICE pointer owned by the caller; tensors are row-major with the
@@ -43,7 +44,7 @@
 extern "C" {
 #endif
 
-#define RGLRU_ABI_VERSION 5
+#define RGLRU_ABI_VERSION 6
 
 enum { RGLRU_F32 = 0, RGLRU_BF16 = 1 };
 
@@ -198,6 +199,24 @@ int rglru_hip_conv_bwd(const void* u, const void* state, const void* taps, const
 int rglru_hip_gelu_gate_fwd(const void* h, const void* v, void* out, int64_t n, int dtype, void* stream);
 int rglru_hip_gelu_gate_bwd(const void* dout, const void* h, const void* v, void* dh, void* dv,
                             int64_t n, int dtype, void* stream);
+
+/* Single-token step of the recurrent block (griffin/griffin.py:459-528 with one token per row) in
+ * two launches around the caller's three Linear layers:
+ *   rglru_hip_decode_prepare: per row, the position (prev_pos + 1, prev_pos NULL = -1, or
+ *     segment_pos[B] when given), the flags for the step (reset at position 0, inactive), the
+ *     convolved input x[B,W] = conv(u[B,W], conv_state[B,K-1,W] or NULL = zeros), the shifted state
+ *     new_conv_state[B,K-1,W] (must not alias conv_state) and new_pos[B].  active[B] (one byte per
+ *     row) NULL selects the all-active path (:476-487); otherwise the padded path (:488-510): a
+ *     document start clears the history, an inactive row keeps state and position, x = 0 for it.
+ *   rglru_hip_step_gated: rglru_hip_step with the state read from h_in and written to h_out (the two
+ *     may be the same buffer) and out[B,W] = h * gelu_tanh(v[B,W]) (v NULL: out = h), which is the
+ *     operand of the block's output projection (:520). */
+int rglru_hip_decode_prepare(const void* u, const void* conv_state, const void* taps, const void* bias,
+                             const int64_t* prev_pos, const int64_t* segment_pos, const uint8_t* active,
+                             void* x, void* new_conv_state, int64_t* new_pos, uint8_t* flags,
+                             int64_t B, int64_t W, int64_t K, int dtype, int vec_dtype, void* stream);
+int rglru_hip_step_gated(const void* x, const void* prep, const float* h_in, float* h_out, const uint8_t* flags,
+                         const void* v, void* out, int64_t B, int64_t W, int64_t nb, int dtype, void* stream);
 
 /* Test hook: number of polls a wave may spend waiting for a neighbouring chunk's carry before it
  * gives up, records the failure in the workspace and finishes with unspecified results.  The

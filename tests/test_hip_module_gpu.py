@@ -369,3 +369,90 @@ def test_bounded_wait_gives_up_instead_of_hanging():
     good = hip_rglru_scan(a, z, h0)
     want = 10.0 * (1.0 - 0.9 ** torch.arange(1, T + 1, dtype=torch.float64))
     assert rel_err(good[0, :, 0], want) < 1e-5
+
+
+# ----------------------------------------------------------------------------------------------
+# single-token decode of the recurrent block (rglru_hip_decode_prepare + rglru_hip_step_gated)
+# ----------------------------------------------------------------------------------------------
+def _block_params(block):
+    """Parameters of a RecurrentBlock in the oracle's naming, fp32 on the CPU."""
+    sd = {k: v.detach().float().cpu() for k, v in block.state_dict().items()}
+    return {"lx_w": sd["linear_x.weight"], "lx_b": sd["linear_x.bias"], "ly_w": sd["linear_y.weight"],
+            "ly_b": sd["linear_y.bias"], "conv_w": sd["temporal_conv.weight"][:, 0, :], "conv_b": sd["temporal_conv.bias"],
+            "w_a": sd["rg_lru.recurrence_gate.weight"], "b_a": sd["rg_lru.recurrence_gate.bias"],
+            "w_x": sd["rg_lru.input_gate.weight"], "b_x": sd["rg_lru.input_gate.bias"], "lam": sd["rg_lru.Lambda"],
+            "lo_w": sd["linear_out.weight"], "lo_b": sd["linear_out.bias"]}
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, FP32_TOL), (torch.bfloat16, BF16_TOL)])
+def test_block_decode_matches_oracle(dtype, tol):
+    """Prefill of 9 tokens, then 7 single-token steps with the carried cache, against the oracle's
+    block run the same way (analogue of the reference's tests/test_recurrentblock.py chunk test)."""
+    from griffin_amd import RecurrentBlock
+
+    torch.manual_seed(3)
+    block = RecurrentBlock(24, 64, gate_blocks=2, scan_mode="hip")
+    with torch.no_grad():
+        for prm in block.parameters():
+            prm.copy_(prm.to(dtype).float())            # parameters exactly representable in the storage type
+        block.temporal_conv.bias.copy_((0.1 * torch.randn(64)).to(dtype).float())
+    params = _block_params(block)
+    block = block.cuda().to(dtype).eval()
+    x = torch.randn(3, 16, 24).to(dtype).float()
+    want, cache_o = [], None
+    with torch.no_grad():
+        piece, cache_o = orc.recurrent_block_forward(x[:, :9], params, cache=cache_o)
+        want.append(piece)
+        for t in range(9, 16):
+            piece, cache_o = orc.recurrent_block_forward(x[:, t:t + 1], params, cache=cache_o)
+            want.append(piece)
+        xg = x.to(dtype).cuda()
+        got, cache = [], None
+        piece, cache = block(xg[:, :9], return_cache=True)
+        got.append(piece)
+        for t in range(9, 16):
+            piece, cache = block(xg[:, t:t + 1], cache=cache, return_cache=True)
+            got.append(piece)
+    torch.cuda.synchronize()
+    want, got = torch.cat(want, dim=1), torch.cat(got, dim=1)
+    errs = {"out": rel_err(got.float(), want), "rnn_state": rel_err(cache.rnn_state, cache_o[0]),
+            "conv_state": rel_err(cache.conv_state.float(), cache_o[1])}
+    _say("block decode", dtype, {k: "%.2e" % v for k, v in errs.items()})
+    for name, err in errs.items():
+        assert err < tol, (name, err)
+    assert torch.equal(cache.segment_position.cpu(), cache_o[2])
+    assert cache.rnn_state.dtype == torch.float32
+
+
+def test_block_decode_with_padding_and_restart_matches_portable_block():
+    """Rows that pause (inactive tokens) and a row that starts a new document mid-stream: the decode
+    kernels against the same block on the CPU with the sequential scan (whose padded path follows
+    griffin/griffin.py:488-510)."""
+    from griffin_amd import RecurrentBlock
+
+    torch.manual_seed(4)
+    cpu_block = RecurrentBlock(16, 32, gate_blocks=2, scan_mode="sequential").eval()
+    hip_block = copy.deepcopy(cpu_block).cuda()
+    hip_block.rg_lru.scan_mode = "hip"
+    B, steps = 4, 10
+    x = torch.randn(B, steps, 16)
+    active = torch.ones(B, steps, dtype=torch.bool)
+    active[1, 3:5] = False
+    active[2, 7] = False
+    active[3, :] = True
+    positions = torch.arange(steps).repeat(B, 1)
+    positions[0, 6:] -= 6                                    # row 0 starts a new document at step 6
+    with torch.no_grad():
+        cache_c = cache_h = None
+        for t in range(steps):
+            # explicit positions on some steps, positions derived from the cache on the others
+            explicit = positions[:, t:t + 1] if (t >= 6 or t < 3) else None
+            mask = active[:, t:t + 1]
+            oc, cache_c = cpu_block(x[:, t:t + 1], cache=cache_c, segment_pos=explicit, active_mask=mask, return_cache=True)
+            oh, cache_h = hip_block(x[:, t:t + 1].cuda(), cache=cache_h,
+                                    segment_pos=None if explicit is None else explicit.cuda(),
+                                    active_mask=mask.cuda(), return_cache=True)
+            torch.testing.assert_close(oh.cpu(), oc, atol=2e-5, rtol=2e-5)
+            torch.testing.assert_close(cache_h.rnn_state.cpu(), cache_c.rnn_state, atol=2e-5, rtol=2e-5)
+            torch.testing.assert_close(cache_h.conv_state.cpu(), cache_c.conv_state, atol=1e-6, rtol=1e-6)
+            assert torch.equal(cache_h.segment_position.cpu(), cache_c.segment_position), t
