@@ -907,9 +907,11 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
   unsigned tk = s_ticket[0];
   int par = 0;
   issue(tk);
+  int trace_iter = 0; (void)trace_iter;
   while ((long long)tk < q.tiles) {
     int c, b;
     decode(tk, c, b);
+    RGLRU_STAMP(p, 0);
     const int t0 = c * TR;
     const long long trow = (long long)b * p.T + t0 + hf * EL;
     unsigned next_raw = 0;
@@ -932,6 +934,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
       }
     }
     __syncthreads();
+    RGLRU_STAMP(p, 1);
     f32x16 ua, ux;
     float xv[EL], gy[EL];
     if (w.slab_ok) {
@@ -966,8 +969,10 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
         for (int e = 0; e < EL; ++e) gy[e] = (float)lds_dy[(hf * EL + e) * LDSROW + (NKG == 8 ? 0 : w.kb) + w.slab * 32 + w.r];
       }
     }
+    RGLRU_STAMP(p, 2);
     if (tid == 0) s_ticket[par ^ 1] = next_raw;
     __syncthreads();
+    RGLRU_STAMP(p, 3);
     par ^= 1;
     const unsigned tk_next = s_ticket[par];
     if (!w.slab_ok) {                                    // a wave without a slab only helps with the loads
@@ -1008,6 +1013,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
     chain.rec = p.rec_a + seq; chain.stride = W;
     const bool last_chunk = c == p.nC - 1;
     if (!last_chunk && hf == 0) carry_publish(chain, c, A_t, D_t, false);
+    RGLRU_STAMP(p, 4);
 
     // input gate, g = sqrt(1 - a^2) and the forward map of the lane's run (for h at the run's start)
     float H = 0.f;
@@ -1024,8 +1030,10 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
     const float H_o = xhalf(H, hf);
     const float H_lo = hf ? H_o : H;
     issue(tk_next);
+    RGLRU_STAMP(p, 5);
     float d_in = (last_chunk && p.dh_last) ? p.dh_last[(long long)b * W + w.ch] : 0.f;
     if (!last_chunk) d_in = carry_lookback(chain, c, +1, p.nC, 0.f, true, p.limit, p.fail);
+    RGLRU_STAMP(p, 6);
     const float d_out = fmaf(A_t, d_in, D_t);
     if (hf == 0) carry_publish(chain, c, 0.f, d_out, true);
     if (hf == 0 && c == 0 && p.dh0) p.dh0[(long long)b * W + w.ch] = d_out;
@@ -1095,6 +1103,8 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
       }
     }
     wave_lds_fence();
+    RGLRU_STAMP(p, 7);
+    ++trace_iter;
     tk = tk_next;
   }
   // per-workgroup partial sums (every slot is written, so the buffer needs no clearing)
@@ -1842,6 +1852,9 @@ int rglru_hip_bwd_full(const void* x, const void* prep, const float* h0,
   a.partial = (float*)(sb + SL.partial); a.dw_partial = (float*)(sb + SL.dw_partial);
   a.B = (int)B; a.T = (int)T; a.nC = (int)((T + kChunk - 1) / kChunk); a.ckpt_nC = (int)L.nC;
   a.aligned = 1;
+#ifdef RGLRU_TRACE
+  a.trace = g_trace;
+#endif
   const int nkg = held_groups(g, dtype, 1);
   pack_units(a, g, nkg);
   a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nC, 2, L.max_wg);
