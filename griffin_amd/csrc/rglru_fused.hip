@@ -1138,14 +1138,17 @@ __global__ __launch_bounds__(kGradThreads, 1) void gate_grad_kernel(FusedArgs p)
   constexpr int TR = 32;
   constexpr int KC = NKG * Tr::KG;                       // block width
   constexpr int S = KC / 32;                             // slabs in the block
-  constexpr int K2 = 2 * KC, NKG2 = 2 * NKG;             // contraction length of the first GEMM
-  constexpr int NKT = 2 * S;                             // 32-wide kappa tiles of du2
+  constexpr int BPU = 4 / S;                             // blocks per unit: narrow blocks share a workgroup (four slabs)
+  constexpr int UKC = KC * BPU, UK2 = 2 * UKC;           // width of the unit's x / dx tiles (128) and of its du2 tile (256)
+  constexpr int NKG2 = 2 * NKG;                          // K groups of the first GEMM (contraction over a block's 2 * KC kappa)
+  constexpr int NKT = 2 * S;                             // 32-wide kappa tiles of du2 per block
+  constexpr int NKT_U = UK2 / 32;                        // ... and per unit
   constexpr int KT_HALF = (NKT + 1) / 2;                 // kappa tiles each half of the workgroup accumulates
-  constexpr int ROW_X = KC + Tr::HW, ROW_DU = K2 + Tr::HW, ROW_T = TR + Tr::HW;
+  constexpr int ROW_X = UKC + Tr::HW, ROW_DU = UK2 + Tr::HW, ROW_T = TR + Tr::HW;
   __shared__ __attribute__((aligned(16))) IO lds_du[TR * ROW_DU];
   __shared__ __attribute__((aligned(16))) IO lds_x[TR * ROW_X];
   __shared__ __attribute__((aligned(16))) IO lds_dx[TR * ROW_X];
-  __shared__ __attribute__((aligned(16))) IO lds_dut[K2 * ROW_T];          // du2 transposed: [kappa][token]
+  __shared__ __attribute__((aligned(16))) IO lds_dut[UK2 * ROW_T];         // du2 transposed: [kappa][token]
   __shared__ __attribute__((aligned(16))) unsigned char stage_all[4 * WaveStage<TR>::kBytes];
 
   // Eight waves, two per SIMD: wave = 4 * half + slab.  Between the two barriers of a tile the lower
@@ -1153,8 +1156,11 @@ __global__ __launch_bounds__(kGradThreads, 1) void gate_grad_kernel(FusedArgs p)
   // after the second barrier both halves accumulate their share of the kappa tiles of dW2T.
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, hf = lane >> 5;
   const int slab = wave & 3, half = wave >> 2;
-  const int k = blockIdx.x % p.nb, wg_in_unit = blockIdx.x / p.nb, n_wg = gridDim.x / p.nb;
-  const bool slab_ok = slab < S;
+  const int units = (p.nb + BPU - 1) / BPU;
+  const int unit = blockIdx.x % units, wg_in_unit = blockIdx.x / units, n_wg = gridDim.x / units;
+  const int blk = slab / S, sl = slab - blk * S;           // the wave's block inside the unit and its slab inside the block
+  const bool slab_ok = unit * BPU + blk < p.nb;
+  const int k = slab_ok ? unit * BPU + blk : p.nb - 1;
   unsigned char* stage = stage_all + slab * WaveStage<TR>::kBytes;
   const long long rows_total = (long long)p.B * p.T;
   const long long n_tiles = (rows_total + TR - 1) / TR;
@@ -1164,7 +1170,7 @@ __global__ __launch_bounds__(kGradThreads, 1) void gate_grad_kernel(FusedArgs p)
   // kappa = 16 kg + 8 hf + i
   Frag w2[NKG2];
   if (half == 0) {
-    const IO* row = (const IO*)p.w2t + ((long long)k * p.bwp + (slab_ok ? slab * 32 + r : 0)) * (2 * p.bwp) + hf * Tr::HW;
+    const IO* row = (const IO*)p.w2t + ((long long)k * p.bwp + sl * 32 + r) * (2 * p.bwp) + hf * Tr::HW;
 #pragma unroll
     for (int kg = 0; kg < NKG2; ++kg) w2[kg] = *reinterpret_cast<const Frag*>(row + kg * Tr::KG);
   } else {
@@ -1185,7 +1191,8 @@ __global__ __launch_bounds__(kGradThreads, 1) void gate_grad_kernel(FusedArgs p)
     for (int v = 0; v < 16; ++v) dw[kt][v] = 0.f;
 
   // cooperative tile loads: du2 (TR x K2), x and dx (TR x KC)
-  constexpr int VPR_DU = K2 / Tr::HW, VPR_X = KC / Tr::HW;
+  constexpr int VPR_DU = UK2 / Tr::HW, VPR_X = UKC / Tr::HW;
+  const int unit_col = unit * BPU * p.bw;                  // first channel of the unit
   constexpr int NV_DU = (TR * VPR_DU + kGradThreads - 1) / kGradThreads, NV_X = (TR * VPR_X + kGradThreads - 1) / kGradThreads;
   Frag pre_du[NV_DU], pre_x[NV_X], pre_dx[NV_X];
   auto issue = [&](long long tile) {
@@ -1200,13 +1207,13 @@ __global__ __launch_bounds__(kGradThreads, 1) void gate_grad_kernel(FusedArgs p)
     for (int i = 0; i < NV_DU; ++i) {
       const int idx = tid + i * kGradThreads;
       const int row = idx / VPR_DU, cv = idx - row * VPR_DU;
-      pre_du[i] = buf_load_frag<Frag>(rdu, idx < TR * VPR_DU ? (unsigned)row * 2u * row_bytes + (unsigned)(k * 2 * p.bw + cv * Tr::HW) * 2u : kOutOfRange);
+      pre_du[i] = buf_load_frag<Frag>(rdu, idx < TR * VPR_DU ? (unsigned)row * 2u * row_bytes + (unsigned)(2 * unit_col + cv * Tr::HW) * 2u : kOutOfRange);
     }
 #pragma unroll
     for (int i = 0; i < NV_X; ++i) {
       const int idx = tid + i * kGradThreads;
       const int row = idx / VPR_X, cv = idx - row * VPR_X;
-      const unsigned off = idx < TR * VPR_X ? (unsigned)row * row_bytes + (unsigned)(k * p.bw + cv * Tr::HW) * 2u : kOutOfRange;
+      const unsigned off = idx < TR * VPR_X ? (unsigned)row * row_bytes + (unsigned)(unit_col + cv * Tr::HW) * 2u : kOutOfRange;
       pre_x[i] = buf_load_frag<Frag>(rx, off);
       pre_dx[i] = buf_load_frag<Frag>(rdx, off);
     }
@@ -1250,9 +1257,9 @@ __global__ __launch_bounds__(kGradThreads, 1) void gate_grad_kernel(FusedArgs p)
     if (half == 1) {
       // transposes: the upper half's four waves share the kappa tiles of du2, written to lds_dut
 #pragma unroll
-      for (int h2 = 0; h2 < (NKT + 3) / 4; ++h2) {
+      for (int h2 = 0; h2 < (NKT_U + 3) / 4; ++h2) {
         const int kt = 4 * h2 + slab;
-        if (kt < NKT) {
+        if (kt < NKT_U) {
           f32x16 dc;
 #pragma unroll
           for (int v = 0; v < 16; ++v) dc[v] = 0.f;
@@ -1273,8 +1280,8 @@ __global__ __launch_bounds__(kGradThreads, 1) void gate_grad_kernel(FusedArgs p)
       for (int v = 0; v < 16; ++v) { acc[v] = (float)lds_dx[(hf * 16 + v) * ROW_X + slab * 32 + r]; acc_odd[v] = 0.f; }
 #pragma unroll
       for (int kg = 0; kg < NKG2; kg += 2) {
-        Tr::mma(acc, *reinterpret_cast<const Frag*>(a_row_du + kg * Tr::KG), w2[kg]);
-        Tr::mma(acc_odd, *reinterpret_cast<const Frag*>(a_row_du + (kg + 1) * Tr::KG), w2[kg + 1]);
+        Tr::mma(acc, *reinterpret_cast<const Frag*>(a_row_du + (blk * NKG2 + kg) * Tr::KG), w2[kg]);
+        Tr::mma(acc_odd, *reinterpret_cast<const Frag*>(a_row_du + (blk * NKG2 + kg + 1) * Tr::KG), w2[kg + 1]);
       }
       unsigned char* my = stage + WaveStage<TR>::row_offset(hf * 16) + r * 2;
 #pragma unroll
@@ -1282,7 +1289,7 @@ __global__ __launch_bounds__(kGradThreads, 1) void gate_grad_kernel(FusedArgs p)
       wave_lds_fence();
       const int rows = (int)((rows_total - row0) < TR ? (rows_total - row0) : TR);
       const rsrc_t rdx = make_rsrc((const IO*)p.dx + row0 * p.W, (unsigned)rows * row_bytes);
-      stage_flush<TR>(stage, rdx, row_bytes, (unsigned)(k * p.bw + slab * 32) * 2u, lane);
+      stage_flush<TR>(stage, rdx, row_bytes, (unsigned)(unit_col + slab * 32) * 2u, lane);
       wave_lds_fence();
     }
     __syncthreads();
@@ -1292,7 +1299,7 @@ __global__ __launch_bounds__(kGradThreads, 1) void gate_grad_kernel(FusedArgs p)
       for (int i = 0; i < KT_HALF; ++i) {
         const int kt = half * KT_HALF + i;
         if (kt < NKT) {
-          const IO* b_row = lds_dut + (kt * 32 + r) * ROW_T + hf * 16;
+          const IO* b_row = lds_dut + ((blk * NKT + kt) * 32 + r) * ROW_T + hf * 16;
           Tr::mma(dw[i], xt_lo, *reinterpret_cast<const Frag*>(b_row));
           Tr::mma(dw[i], xt_hi, *reinterpret_cast<const Frag*>(b_row + 8));
         }
@@ -1308,7 +1315,7 @@ __global__ __launch_bounds__(kGradThreads, 1) void gate_grad_kernel(FusedArgs p)
       if (kt < NKT) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          const int j = slab * 32 + 8 * (v >> 2) + 4 * hf + (v & 3);
+          const int j = sl * 32 + 8 * (v >> 2) + 4 * hf + (v & 3);
           part[(long long)j * (2 * p.bwp) + kt * 32 + r] = dw[i][v];
         }
       }
@@ -1871,8 +1878,9 @@ int rglru_hip_bwd_full(const void* x, const void* prep, const float* h0,
   }
   rc = check_launch("bwd_full scan");
   if (rc) return rc;
-  int n_wg = num_compute_units() / (int)nb; if (n_wg < 1) n_wg = 1; if (n_wg > kGemmWgPerUnit) n_wg = kGemmWgPerUnit;
-  dim3 grid2((unsigned)(n_wg * nb));
+  // the gradient GEMM kernel packs narrow blocks into units the same way (a.units)
+  int n_wg = num_compute_units() / a.units; if (n_wg < 1) n_wg = 1; if (n_wg > kGemmWgPerUnit) n_wg = kGemmWgPerUnit;
+  dim3 grid2((unsigned)(n_wg * a.units));
   {
     KernelTimer timer(3, s);
     if (nkg == 8) hipLaunchKernelGGL((gate_grad_kernel<__bf16, 8>), grid2, dim3(kGradThreads), 0, s, a);
