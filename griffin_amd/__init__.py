@@ -9,7 +9,7 @@ from .hip_scan import (
     hip_scan_available,
     hip_scan_is_usable,
 )
-from .hip_block_ops import hip_causal_conv, hip_gelu_gate
+from .hip_block_ops import hip_causal_conv, hip_causal_conv_padded, hip_gelu_gate
 from .modules import (
     BlockDiagonalLinear,
     RG_LRU,
@@ -24,6 +24,7 @@ __all__ = [
     "RecurrentBlock",
     "RecurrentBlockCache",
     "hip_causal_conv",
+    "hip_causal_conv_padded",
     "hip_gelu_gate",
     "hip_rglru",
     "hip_rglru_scan",

@@ -387,6 +387,126 @@ static bool conv_vector_ok(int64_t W, int dtype, std::initializer_list<const voi
 
 
 // ------------------------------------------------------------------------------------------
+// Convolution over right-padded batches (griffin/griffin.py:488-510), forward only.  The reference
+// walks the tokens one by one with a window of the last K-1 ACTIVE inputs, cleared where an active
+// token starts a document.  Here the walk is split in two parallel kernels:
+//   conv_padded_index_kernel  one wave per row: the ordinal of every active token among the active
+//       ones, the ordinal at which its document started (-1: no start inside this call) and the
+//       list ordinal -> token, by ballots and population counts over 64 tokens at a time;
+//   conv_padded_fwd_kernel    per token and channel vector, like the dense kernel, gathering the
+//       rows of the K-1 previous active tokens (or carried state rows, or zeros) through that list.
+// Scratch (32-bit words): ord[B][T], start[B][T], list[B][T], count[B], final_start[B].
+// ------------------------------------------------------------------------------------------
+struct PaddedArgs {
+  const void* u; const void* state; const void* taps; const void* bias;
+  const long long* segpos; const unsigned char* active;
+  void* out; void* new_state; int* scratch;
+  int B, T, W, K, nvec, vec_dtype;
+};
+
+__global__ __launch_bounds__(64) void conv_padded_index_kernel(PaddedArgs p) {
+  const int b = blockIdx.x, lane = threadIdx.x;
+  int* ord = p.scratch + (long long)b * p.T;
+  int* start = p.scratch + ((long long)p.B + b) * p.T;
+  int* list = p.scratch + (2ll * p.B + b) * p.T;
+  int* tail = p.scratch + 3ll * p.B * p.T;
+  int count = 0, doc_start = -1;                           // wave-uniform running values
+  for (int t0 = 0; t0 < p.T; t0 += 64) {
+    const int t = t0 + lane;
+    const bool in = t < p.T;
+    const bool act = in && p.active[(long long)b * p.T + t] != 0;
+    const bool rst = act && p.segpos[(long long)b * p.T + t] == 0;
+    const unsigned long long am = __ballot(act), rm = __ballot(rst);
+    const unsigned long long below = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+    const int my_ord = count + __popcll(am & below);
+    // last document start at or before this token inside the chunk, else the running one
+    const unsigned long long upto = rm & (below | (1ull << lane));
+    int my_start = doc_start;
+    if (upto) {
+      const int at = 63 - __clzll(upto);
+      my_start = count + __popcll(am & ((at == 0) ? 0ull : (~0ull >> (64 - at))));
+    }
+    if (in) { ord[t] = act ? my_ord : -1; start[t] = my_start; }
+    if (act) list[my_ord] = t;
+    if (rm) {
+      const int at = 63 - __clzll(rm);
+      doc_start = count + __popcll(am & ((at == 0) ? 0ull : (~0ull >> (64 - at))));
+    }
+    count += __popcll(am);
+  }
+  if (lane == 0) { tail[b] = count; tail[p.B + b] = doc_start; }
+}
+
+// Row that stands `lag` active tokens before ordinal i of sequence b, as floats.
+template <typename IO, int V, int K>
+RGLRU_DEVICE void padded_source(const PaddedArgs& p, rsrc_t ru, rsrc_t rs, const int* list, int i, int lag, int doc_start,
+                                int c0, float (&v)[V]) {
+  const int j = i - lag;
+  const unsigned es = (unsigned)sizeof(IO), uW = (unsigned)p.W;
+  unsigned off = kOutOfRange;
+  bool from_state = false;
+  if (j >= 0 && j >= doc_start) off = ((unsigned)list[j] * uW + (unsigned)c0) * es;
+  else if (doc_start < 0 && j < 0 && K - 1 + j >= 0) { off = ((unsigned)(K - 1 + j) * uW + (unsigned)c0) * es; from_state = true; }
+  ConvRow<IO, V>::load(v, from_state ? rs : ru, off);
+}
+
+template <typename IO, int V, int K>
+__global__ __launch_bounds__(kConvThreads) void conv_padded_fwd_kernel(PaddedArgs p) {
+  const long long item = (long long)blockIdx.x * kConvThreads + threadIdx.x;
+  const long long per_seq = (long long)(p.T + 1) * p.nvec;    // one extra "token" per row writes the new state
+  if (item >= (long long)p.B * per_seq) return;
+  const int b = (int)(item / per_seq);
+  const long long rest = item - (long long)b * per_seq;
+  const int t = (int)(rest / p.nvec), c0 = (int)(rest - (long long)t * p.nvec) * V;
+  const unsigned es = (unsigned)sizeof(IO), uW = (unsigned)p.W;
+  const int* ord = p.scratch + (long long)b * p.T;
+  const int* start = p.scratch + ((long long)p.B + b) * p.T;
+  const int* list = p.scratch + (2ll * p.B + b) * p.T;
+  const int* tail = p.scratch + 3ll * p.B * p.T;
+  const rsrc_t ru = make_rsrc((const IO*)p.u + (long long)b * p.T * p.W, (unsigned)p.T * uW * es);
+  const rsrc_t rs = make_rsrc(p.state ? (const IO*)p.state + (long long)b * (K - 1) * p.W : (const IO*)p.u,
+                              p.state ? (unsigned)((K - 1) * p.W) * es : 0u);
+  if (t == p.T) {
+    // carried state: the last K-1 active inputs since the last document start, oldest first
+    if (K > 1 && p.new_state) {
+      const int n = tail[b], doc_start = tail[p.B + b];
+      const rsrc_t rn = make_rsrc((IO*)p.new_state + (long long)b * (K - 1) * p.W, (unsigned)((K - 1) * p.W) * es);
+#pragma unroll
+      for (int lag = 1; lag < K; ++lag) {
+        float row[V];
+        padded_source<IO, V, K>(p, ru, rs, list, n, lag, doc_start, c0, row);
+        ConvRow<IO, V>::store(row, rn, ((unsigned)(K - 1 - lag) * uW + (unsigned)c0) * es);
+      }
+    }
+    return;
+  }
+  const rsrc_t ro = make_rsrc((IO*)p.out + (long long)b * p.T * p.W, (unsigned)p.T * uW * es);
+  const unsigned off = ((unsigned)t * uW + (unsigned)c0) * es;
+  const int i = ord[t];
+  float acc[V];
+  if (i < 0) {
+#pragma unroll
+    for (int v = 0; v < V; ++v) acc[v] = 0.f;
+  } else {
+    const int doc_start = start[t];
+    float cur[V];
+    ConvRow<IO, V>::load(cur, ru, off);
+#pragma unroll
+    for (int v = 0; v < V; ++v)
+      acc[v] = fmaf(cur[v], conv_param(p.taps, (long long)(c0 + v) * K + (K - 1), p.vec_dtype),
+                    p.bias ? conv_param(p.bias, c0 + v, p.vec_dtype) : 0.f);
+#pragma unroll
+    for (int lag = 1; lag < K; ++lag) {
+      float row[V];
+      padded_source<IO, V, K>(p, ru, rs, list, i, lag, doc_start, c0, row);
+#pragma unroll
+      for (int v = 0; v < V; ++v) acc[v] = fmaf(row[v], conv_param(p.taps, (long long)(c0 + v) * K + (K - 1 - lag), p.vec_dtype), acc[v]);
+    }
+  }
+  ConvRow<IO, V>::store(acc, ro, off);
+}
+
+// ------------------------------------------------------------------------------------------
 // Everything a single-token step of the recurrent block needs in front of the RG-LRU step kernel,
 // in one launch (griffin/griffin.py:459-510 with one token per row): the row's position
 // (previous + 1, or the one given), its flags for the step kernel (reset at position 0, inactive),
@@ -656,6 +776,36 @@ int rglru_hip_decode_prepare(const void* u, const void* conv_state, const void* 
   hipStream_t s = (hipStream_t)stream;
   RGLRU_CONV_DISPATCH(decode_prepare_kernel, dtype, vec, grid, s, a);
   return check_launch("decode_prepare");
+}
+
+size_t rglru_hip_conv_padded_scratch_bytes(int64_t B, int64_t T) {
+  if (B <= 0 || T <= 0) return 0;
+  return (size_t)((3 * B * T + 2 * B) * 4);
+}
+
+int rglru_hip_conv_padded_fwd(const void* u, const void* state, const void* taps, const void* bias,
+                              const int64_t* segment_pos, const uint8_t* active, void* scratch,
+                              void* out, void* new_state,
+                              int64_t B, int64_t T, int64_t W, int64_t K, int dtype, int vec_dtype, void* stream) {
+  int rc = conv_check("conv_padded_fwd", B, T, W, K, dtype, vec_dtype);
+  if (rc) return rc;
+  if (!u || !taps || !segment_pos || !active || !scratch || !out) return fail(RGLRU_E_ARG, "conv_padded_fwd: null pointer");
+  if (B * T >= (1ll << 29)) return fail(RGLRU_E_UNSUPPORTED, "conv_padded_fwd: tensor too large");
+  PaddedArgs a;
+  memset(&a, 0, sizeof(a));
+  a.u = u; a.state = state; a.taps = taps; a.bias = bias; a.segpos = (const long long*)segment_pos; a.active = active;
+  a.out = out; a.new_state = new_state; a.scratch = (int*)scratch;
+  a.B = (int)B; a.T = (int)T; a.W = (int)W; a.K = (int)K; a.vec_dtype = vec_dtype;
+  const bool vec = conv_vector_ok(W, dtype, {u, state, out, new_state});
+  a.nvec = (int)(vec ? W / (dtype == RGLRU_BF16 ? 8 : 4) : W);
+  hipStream_t s = (hipStream_t)stream;
+  hipLaunchKernelGGL(conv_padded_index_kernel, dim3((unsigned)B), dim3(64), 0, s, a);
+  rc = check_launch("conv_padded_fwd index");
+  if (rc) return rc;
+  const long long items = (long long)B * (T + 1) * a.nvec;
+  dim3 grid((unsigned)((items + kConvThreads - 1) / kConvThreads));
+  RGLRU_CONV_DISPATCH(conv_padded_fwd_kernel, dtype, vec, grid, s, a);
+  return check_launch("conv_padded_fwd");
 }
 
 }  // extern "C"

@@ -120,6 +120,42 @@ def hip_causal_conv(u: Tensor, state: Tensor | None, weight: Tensor, bias: Tenso
     return out, new_state
 
 
+def hip_causal_conv_padded(u: Tensor, state: Tensor | None, weight: Tensor, bias: Tensor | None,
+                           segment_pos: Tensor, active_mask: Tensor) -> tuple[Tensor, Tensor]:
+    """The convolution over right-padded batches (griffin/griffin.py:488-510), forward only (no
+    autograd): inactive tokens give zeros and stay out of the window of previous inputs, an active
+    token at position 0 clears the window.  Returns ``(out [B, T, W], new_state [B, K-1, W])``."""
+    _require_gpu("hip_causal_conv_padded", u, state, weight, bias, segment_pos, active_mask)
+    if u.dim() != 3:
+        raise ValueError(f"hip_causal_conv_padded expects [batch, sequence, width], got {tuple(u.shape)}")
+    batch, steps, width = u.shape
+    if weight.dim() != 3 or weight.size(0) != width or weight.size(1) != 1:
+        raise ValueError("weight must be that of a depthwise Conv1d: [width, 1, kernel_size]")
+    taps_count = weight.size(2)
+    if state is not None and state.shape != (batch, taps_count - 1, width):
+        raise ValueError("state must have shape [batch, kernel_size - 1, width]")
+    if segment_pos.shape != (batch, steps) or active_mask.shape != (batch, steps):
+        raise ValueError("segment_pos and active_mask must have shape [batch, sequence]")
+    code = _dtype_code(u.dtype)
+    u_c = u.detach().contiguous()
+    state_c = None if state is None or taps_count == 1 else state.detach().to(u.dtype).contiguous()
+    taps = _parameter_operand(weight.detach(), u.dtype)
+    bias_c = None if bias is None else _parameter_operand(bias.detach().to(taps.dtype), u.dtype)
+    pos = segment_pos.to(device=u.device, dtype=torch.int64).contiguous()
+    live = active_mask.to(device=u.device, dtype=torch.uint8).contiguous()
+    lib = _lib.load()
+    with torch.cuda.device(u.device):
+        out = torch.empty_like(u_c)
+        new_state = u.new_empty(batch, taps_count - 1, width)
+        scratch = torch.empty(lib.rglru_hip_conv_padded_scratch_bytes(batch, steps), dtype=torch.uint8, device=u.device)
+        _lib.check(lib.rglru_hip_conv_padded_fwd(
+            _ptr(u_c), _ptr(state_c), _ptr(taps), _ptr(bias_c), _ptr(pos), _ptr(live), _ptr(scratch), _ptr(out),
+            _ptr(new_state) if taps_count > 1 else None,
+            batch, steps, width, taps_count, code, _DTYPE_CODES[taps.dtype], _stream_ptr(u.device)),
+            "rglru_hip_conv_padded_fwd")
+    return out, new_state
+
+
 class _HipGeluGate(torch.autograd.Function):
     @staticmethod
     def forward(ctx, h: Tensor, v: Tensor) -> Tensor:

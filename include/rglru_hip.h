@@ -14,6 +14,7 @@
  *   griffin/griffin.py:279-284 with T == 1 (decode step, carried state)     rglru_hip_step
  *   griffin/griffin.py:474-487      causal depthwise convolution of the caller   rglru_hip_conv_fwd
  *   autograd of griffin/griffin.py:474-487                                   rglru_hip_conv_bwd
+ *   griffin/griffin.py:488-510      the same over right-padded batches (forward)   rglru_hip_conv_padded_fwd
  *   griffin/griffin.py:464, :520    x_branch * gelu_tanh(linear_y(x))        rglru_hip_gelu_gate_fwd, _bwd
  *   griffin/griffin.py:459-528 with T == 1 (block decode: positions, conv, step, gate)   rglru_hip_decode_prepare + rglru_hip_step_gated
  *
@@ -44,7 +45,7 @@
 extern "C" {
 #endif
 
-#define RGLRU_ABI_VERSION 6
+#define RGLRU_ABI_VERSION 7
 
 enum { RGLRU_F32 = 0, RGLRU_BF16 = 1 };
 
@@ -191,6 +192,17 @@ int rglru_hip_conv_bwd(const void* u, const void* state, const void* taps, const
                        const void* dout, void* scratch, void* du, void* dstate, void* dtaps, void* dbias,
                        int64_t B, int64_t T, int64_t W, int64_t K, int dtype, int vec_dtype, int grad_dtype,
                        void* stream);
+
+/* The same convolution over right-padded batches (griffin/griffin.py:488-510), forward only: tokens
+ * with active[b,t] == 0 produce zeros and never enter the window of the K-1 previous ACTIVE inputs; an
+ * active token with segment_pos == 0 clears that window (and the carried state) before it is used.
+ * active[B,T] is one byte per token; new_state[B,K-1,W] (may be NULL) receives the window after the
+ * last token; `scratch` holds rglru_hip_conv_padded_scratch_bytes(B, T) bytes. */
+size_t rglru_hip_conv_padded_scratch_bytes(int64_t B, int64_t T);
+int rglru_hip_conv_padded_fwd(const void* u, const void* state, const void* taps, const void* bias,
+                              const int64_t* segment_pos, const uint8_t* active, void* scratch,
+                              void* out, void* new_state,
+                              int64_t B, int64_t T, int64_t W, int64_t K, int dtype, int vec_dtype, void* stream);
 
 /* Output gate of the recurrent block, out = h * gelu_tanh(v) (griffin/griffin.py:464 and :520: the
  * GeLU of the second branch and the product with the RG-LRU output in one pass), flat over n

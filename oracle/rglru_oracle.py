@@ -278,6 +278,28 @@ def causal_conv(px, conv_w, conv_b, conv_state, seg_pos):
     return out, new_state
 
 
+def causal_conv_padded(px, conv_w, conv_b, conv_state, seg_pos, active):
+    """Padded-path depthwise causal conv (griffin/griffin.py:488-510): a running window of the last
+    K-1 active inputs, cleared where an active token has position 0; inactive tokens yield zeros and
+    leave the window alone.  Shapes as in ``causal_conv``; ``active`` [B,T] bool.  Returns (out, window)."""
+    B, T, W = px.shape
+    K = conv_w.shape[1]
+    window = conv_state.to(px.dtype).clone()
+    rows = []
+    for t in range(T):
+        live = active[:, t]
+        fresh = live & (seg_pos[:, t] == 0)
+        window = torch.where(fresh[:, None, None], torch.zeros_like(window), window)
+        value = px[:, t] * conv_w[:, K - 1] + conv_b
+        for j in range(K - 1):
+            value = value + window[:, j] * conv_w[:, j]
+        rows.append(torch.where(live[:, None], value, torch.zeros_like(value)))
+        if K > 1:
+            moved = torch.cat([window[:, 1:], px[:, t][:, None]], dim=1)
+            window = torch.where(live[:, None, None], moved, window)
+    return torch.stack(rows, dim=1), window
+
+
 def gelu_tanh(v):
     """tanh approximation of GeLU, the activation of the block's second branch (griffin/griffin.py:464,
     ``F.gelu(..., approximate="tanh")``): v/2 * (1 + tanh(sqrt(2/pi) * (v + 0.044715 v^3)))."""

@@ -336,3 +336,34 @@ def test_oracle_gelu_gate_is_the_library_tanh_gelu():
     assert 1e-4 < gap < 1e-3
     h = torch.linspace(-2.0, 3.0, 4001, dtype=torch.float64)
     torch.testing.assert_close(orc.gelu_gate(h, v), h * torch.nn.functional.gelu(v, approximate="tanh"), atol=1e-14, rtol=1e-13)
+
+
+def test_oracle_padded_conv_reduces_to_dense_conv_and_skips_padding():
+    """With every token active and documents that start at position 0 the padded walk is the dense
+    convolution; inserting inactive tokens anywhere changes nothing for the active ones (they see the
+    same previous active inputs) and yields zeros at the inserted places; brute force on one row."""
+    px, w, b, state = _conv_case(B=2, T=11, W=5, K=4, seed=8)
+    B, T, W = px.shape
+    seg = torch.arange(3, 3 + T).repeat(B, 1)
+    seg[1, 6:] -= 9                                           # row 1 starts a new document at t = 6
+    ones = torch.ones(B, T, dtype=torch.bool)
+    dense, dense_state = orc.causal_conv(px, w, b, state, seg)
+    walk, walk_state = orc.causal_conv_padded(px, w, b, state, seg, ones)
+    torch.testing.assert_close(walk, dense, atol=1e-12, rtol=1e-12)
+    torch.testing.assert_close(walk_state[0], dense_state[0])
+    # row 1 restarted: rows of the state that predate the document are cleared, not carried
+    assert torch.equal(walk_state[1], px[1, T - 3:])
+    # pad: insert inactive tokens (random content) after t = 2 and t = 7
+    g = torch.Generator().manual_seed(1)
+    keep = [0, 1, 2, None, None, 3, 4, 5, 6, 7, None, 8, 9, 10]
+    px2 = torch.stack([px[:, k] if k is not None else torch.randn(B, W, generator=g, dtype=px.dtype) for k in keep], dim=1)
+    seg2 = torch.stack([seg[:, k] if k is not None else torch.zeros(B, dtype=torch.long) for k in keep], dim=1)
+    act2 = torch.tensor([k is not None for k in keep]).repeat(B, 1)
+    walk2, state2 = orc.causal_conv_padded(px2, w, b, state, seg2, act2)
+    live_cols = [i for i, k in enumerate(keep) if k is not None]
+    torch.testing.assert_close(walk2[:, live_cols], walk, atol=1e-12, rtol=1e-12)
+    assert torch.count_nonzero(walk2[:, [i for i, k in enumerate(keep) if k is None]]) == 0
+    torch.testing.assert_close(state2, walk_state)
+    # all tokens inactive: zeros out, state untouched
+    none, same = orc.causal_conv_padded(px, w, b, state, seg, torch.zeros(B, T, dtype=torch.bool))
+    assert torch.count_nonzero(none) == 0 and torch.equal(same, state)
