@@ -822,9 +822,9 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
   __shared__ __attribute__((aligned(16))) unsigned char stage_dx_all[kWaves * WaveStage<TR>::kBytes];
   __shared__ __attribute__((aligned(16))) unsigned char stage_du_all[kWaves * (GIVEN ? 2 * WaveStage<TR>::kBytes : PairStage<TR>::kBytes)];
   __shared__ unsigned s_ticket[2];
-  // With 128-channel blocks the weight registers (64) push the kernel into spilling; the input
-  // gate's weights then live in LDS instead (one copy per workgroup, read as B fragments per tile).
-  constexpr bool XLDS = (NKG == 8);
+  // With 128- and 64-channel blocks the weight registers (64, 32) push the kernel into spilling; the
+  // input gate's weights then live in LDS instead (each wave's 32 rows, read as B fragments per tile).
+  constexpr bool XLDS = (NKG == 8 || NKG == 4);
   constexpr int WROW = KC + Tr::HW;
   __shared__ __attribute__((aligned(16))) IO lds_wx[XLDS ? 32 * kWaves * WROW : Tr::HW];
 
@@ -840,11 +840,11 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
   if constexpr (XLDS) {
 #pragma unroll
     for (int kg = 0; kg < NKG; ++kg) hw.a[kg] = *reinterpret_cast<const Frag*>(w_a_row + kg * Tr::KG);
-    // rows of this workgroup's four slabs of W_x
-    const IO* src = wg + ((long long)(1 * p.nb + w.k) * p.bwp + (w.unit % p.groups) * (32 * kWaves)) * p.bwp;
-    for (int idx = threadIdx.x; idx < 32 * kWaves * (KC / Tr::HW); idx += kThreads) {
+    // each wave copies the 32 rows of W_x of its own slab (the waves of a packed unit belong to different blocks)
+    const IO* src = wg + ((long long)(1 * p.nb + w.k) * p.bwp + (w.slab_ok ? w.slab * 32 : 0)) * p.bwp;
+    for (int idx = w.lane; idx < 32 * (KC / Tr::HW); idx += 64) {
       const int row = idx / (KC / Tr::HW), v = idx - row * (KC / Tr::HW);
-      *reinterpret_cast<Frag*>(lds_wx + row * WROW + v * Tr::HW) = *reinterpret_cast<const Frag*>(src + (long long)row * p.bwp + v * Tr::HW);
+      *reinterpret_cast<Frag*>(lds_wx + (w.wave * 32 + row) * WROW + v * Tr::HW) = *reinterpret_cast<const Frag*>(src + (long long)row * p.bwp + v * Tr::HW);
     }
     __syncthreads();
   } else if constexpr (!GIVEN) {
@@ -951,7 +951,8 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
       } else if constexpr (XLDS) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) { ua[v] = bias_a; ux[v] = bias_x; }
-        const IO* xrow = lds_x + tile_row<MT>(0, w.r) * LDSROW + hf * Tr::HW;
+        const int kb = NKG == 8 ? 0 : w.kb;
+        const IO* xrow = lds_x + tile_row<MT>(0, w.r) * LDSROW + kb + hf * Tr::HW;
         const IO* brow = lds_wx + (w.wave * 32 + w.r) * WROW + hf * Tr::HW;
 #pragma unroll
         for (int kg = 0; kg < NKG; ++kg) {
@@ -960,7 +961,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
           Tr::mma(ux, xa, *reinterpret_cast<const Frag*>(brow + kg * Tr::KG));
         }
 #pragma unroll
-        for (int e = 0; e < EL; ++e) xv[e] = (float)lds_x[(hf * EL + e) * LDSROW + w.slab * 32 + w.r];
+        for (int e = 0; e < EL; ++e) xv[e] = (float)lds_x[(hf * EL + e) * LDSROW + kb + w.slab * 32 + w.r];
       } else {
         gate_mfma_held<IO, MT, NKG, TW>(lds_x, hw, 0, w.slab, w.r, hf, bias_a, bias_x, ua, ux, xv, w.kb);
       }
