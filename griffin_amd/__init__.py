@@ -9,10 +9,11 @@ from .hip_scan import (
     hip_scan_available,
     hip_scan_is_usable,
 )
-from .hip_block_ops import hip_causal_conv, hip_causal_conv_padded, hip_gelu_gate
+from .hip_block_ops import hip_causal_conv, hip_causal_conv_padded, hip_gelu_gate, hip_rmsnorm
 from .modules import (
     BlockDiagonalLinear,
     RG_LRU,
+    RMSNorm,
     RecurrentBlock,
     RecurrentBlockCache,
 )
@@ -21,11 +22,13 @@ __all__ = [
     "BlockDiagonalLinear",
     "PreparedParams",
     "RG_LRU",
+    "RMSNorm",
     "RecurrentBlock",
     "RecurrentBlockCache",
     "hip_causal_conv",
     "hip_causal_conv_padded",
     "hip_gelu_gate",
+    "hip_rmsnorm",
     "hip_rglru",
     "hip_rglru_scan",
     "hip_rglru_step",

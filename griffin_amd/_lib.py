@@ -14,7 +14,7 @@ RGLRU_BF16 = 1
 FLAG_RESET = 1
 FLAG_INACTIVE = 2
 CHUNK = 32
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 _lock = threading.Lock()
 _lib = None
@@ -50,6 +50,10 @@ _SIGNATURES = {
     "rglru_hip_conv_padded_fwd": (ctypes.c_int, [_P] * 9 + [_I, _I, _I, _I, ctypes.c_int, ctypes.c_int, _P]),
     "rglru_hip_gelu_gate_fwd": (ctypes.c_int, [_P, _P, _P, _I, ctypes.c_int, _P]),
     "rglru_hip_gelu_gate_bwd": (ctypes.c_int, [_P, _P, _P, _P, _P, _I, ctypes.c_int, _P]),
+    "rglru_hip_rmsnorm_max_width": (ctypes.c_int, [ctypes.c_int, ctypes.c_int]),
+    "rglru_hip_rmsnorm_fwd": (ctypes.c_int, [_P, _P, _P, _P, _I, _I, ctypes.c_float, ctypes.c_int, ctypes.c_int, _P]),
+    "rglru_hip_rmsnorm_scratch_bytes": (ctypes.c_size_t, [_I, _I]),
+    "rglru_hip_rmsnorm_bwd": (ctypes.c_int, [_P] * 7 + [_I, _I, ctypes.c_int, ctypes.c_int, ctypes.c_int, _P]),
     "rglru_hip_decode_prepare": (ctypes.c_int, [_P] * 11 + [_I, _I, _I, ctypes.c_int, ctypes.c_int, _P]),
     "rglru_hip_step_gated": (ctypes.c_int, [_P] * 7 + [_I, _I, _I, ctypes.c_int, _P]),
     "rglru_hip_set_spin_limit": (ctypes.c_int64, [_I]),

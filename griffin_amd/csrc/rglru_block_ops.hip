@@ -667,6 +667,175 @@ static int gate_launch(const char* who, bool backward, GateArgs a, int dtype, vo
   return check_launch(who);
 }
 
+
+// ------------------------------------------------------------------------------------------
+// RMSNorm in front of the block (griffin/griffin.py:68-80): y = x * rsqrt(mean(x^2) + eps) * (1 + g)
+// over the last axis, and its reverse mode.  One wave per row at a time (grid-stride over rows); a
+// lane holds the row's 16-byte vectors lane, lane + 64, ... in registers, so a row is read once.
+//   dx = inv * (w dy - x inv^2 mean(w dy x)),  w = 1 + g,  inv = rsqrt(mean(x^2) + eps)
+//   dg = sum over rows of dy x inv            (per-wave partial sums, reduced by a second kernel)
+// ------------------------------------------------------------------------------------------
+constexpr int kNormThreads = 256;
+constexpr int kNormSlots = 16;                 // most vectors per lane: rows of up to 64 * 16 vectors (1, 2, 4, 8 or 16 are compiled)
+
+struct NormArgs {
+  const void* x; const void* g; const void* dy; const float* inv_in;
+  void* y; void* dx; float* inv_out; float* partial;
+  long long rows; int D, nvec, vec_dtype; float eps;
+};
+
+RGLRU_DEVICE float wave_sum(float v) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
+  return v;
+}
+
+template <typename IO, int V, int SLOTS, bool BACKWARD>
+__global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(NormArgs p) {
+  typedef ConvRow<IO, V> Row;
+  constexpr int kNormSlots = SLOTS;                        // shadows the global maximum inside the kernel
+  const int lane = threadIdx.x & 63;
+  const long long wave = (long long)blockIdx.x * (kNormThreads / 64) + (threadIdx.x >> 6);
+  const long long n_waves = (long long)gridDim.x * (kNormThreads / 64);
+  const unsigned row_bytes = (unsigned)p.D * (unsigned)sizeof(IO);
+  float w[kNormSlots][V], dg[kNormSlots][V];
+#pragma unroll
+  for (int s = 0; s < kNormSlots; ++s)
+#pragma unroll
+    for (int v = 0; v < V; ++v) {
+      const int c = (lane + 64 * s) * V + v;
+      w[s][v] = (lane + 64 * s < p.nvec) ? 1.0f + conv_param(p.g, c, p.vec_dtype) : 0.f;
+      dg[s][v] = 0.f;
+    }
+  const float inv_d = 1.0f / (float)p.D;
+  for (long long row = wave; row < p.rows; row += n_waves) {
+    const rsrc_t rx = make_rsrc((const IO*)p.x + row * p.D, row_bytes);
+    typename Row::Raw raw_x[kNormSlots], raw_d[kNormSlots];
+#pragma unroll
+    for (int s = 0; s < kNormSlots; ++s) {
+      const unsigned off = (lane + 64 * s < p.nvec) ? (unsigned)((lane + 64 * s) * V) * (unsigned)sizeof(IO) : kOutOfRange;
+      raw_x[s] = Row::request(rx, off);
+      if (BACKWARD) raw_d[s] = Row::request(make_rsrc((const IO*)p.dy + row * p.D, row_bytes), off);
+    }
+    float x[kNormSlots][V];
+    float acc = 0.f;
+#pragma unroll
+    for (int s = 0; s < kNormSlots; ++s) {
+      Row::unpack(x[s], raw_x[s]);
+#pragma unroll
+      for (int v = 0; v < V; ++v) acc = fmaf(x[s][v], x[s][v], acc);
+    }
+    if (!BACKWARD) {
+      const float inv = __builtin_amdgcn_rsqf(wave_sum(acc) * inv_d + p.eps);
+      if (lane == 0 && p.inv_out) p.inv_out[row] = inv;
+      const rsrc_t ry = make_rsrc((IO*)p.y + row * p.D, row_bytes);
+#pragma unroll
+      for (int s = 0; s < kNormSlots; ++s) {
+        float y[V];
+#pragma unroll
+        for (int v = 0; v < V; ++v) y[v] = x[s][v] * inv * w[s][v];
+        Row::store(y, ry, (lane + 64 * s < p.nvec) ? (unsigned)((lane + 64 * s) * V) * (unsigned)sizeof(IO) : kOutOfRange);
+      }
+    } else {
+      const float inv = p.inv_in[row];
+      float d[kNormSlots][V];
+      float dot = 0.f;
+#pragma unroll
+      for (int s = 0; s < kNormSlots; ++s) {
+        Row::unpack(d[s], raw_d[s]);
+#pragma unroll
+        for (int v = 0; v < V; ++v) {
+          dg[s][v] = fmaf(d[s][v] * inv, x[s][v], dg[s][v]);
+          d[s][v] *= w[s][v];
+          dot = fmaf(d[s][v], x[s][v], dot);
+        }
+      }
+      const float k = wave_sum(dot) * inv_d * inv * inv;
+      const rsrc_t rdx = make_rsrc((IO*)p.dx + row * p.D, row_bytes);
+#pragma unroll
+      for (int s = 0; s < kNormSlots; ++s) {
+        float g[V];
+#pragma unroll
+        for (int v = 0; v < V; ++v) g[v] = inv * fmaf(-k, x[s][v], d[s][v]);
+        Row::store(g, rdx, (lane + 64 * s < p.nvec) ? (unsigned)((lane + 64 * s) * V) * (unsigned)sizeof(IO) : kOutOfRange);
+      }
+    }
+  }
+  if constexpr (BACKWARD) {
+    // the workgroup's waves add their sums up in LDS, one after the other; one partial row per workgroup
+    __shared__ float red[SLOTS * 64 * V];
+    for (int turn = 0; turn < kNormThreads / 64; ++turn) {
+      if ((int)(threadIdx.x >> 6) == turn) {
+#pragma unroll
+        for (int s = 0; s < kNormSlots; ++s)
+#pragma unroll
+          for (int v = 0; v < V; ++v) {
+            const int at = (lane + 64 * s) * V + v;
+            red[at] = turn == 0 ? dg[s][v] : red[at] + dg[s][v];
+          }
+      }
+      __syncthreads();
+    }
+    float* part = p.partial + (long long)blockIdx.x * p.D;
+    for (int c = threadIdx.x; c < p.D; c += kNormThreads) part[c] = red[c];
+  }
+}
+
+// Sums the per-workgroup partial rows: a workgroup owns 32 columns, eight threads share a column.
+struct NormFinishArgs { const float* partial; void* dg; int D, slots, grad_dtype; };
+__global__ __launch_bounds__(256) void rmsnorm_finish_kernel(NormFinishArgs p) {
+  __shared__ float red[8][32];
+  const int col = threadIdx.x & 31, share = threadIdx.x >> 5;
+  const int c = blockIdx.x * 32 + col;
+  float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+  if (c < p.D) {
+    int n = share;
+    for (; n + 24 < p.slots; n += 32) {
+      s0 += p.partial[(long long)n * p.D + c]; s1 += p.partial[(long long)(n + 8) * p.D + c];
+      s2 += p.partial[(long long)(n + 16) * p.D + c]; s3 += p.partial[(long long)(n + 24) * p.D + c];
+    }
+    for (; n < p.slots; n += 8) s0 += p.partial[(long long)n * p.D + c];
+  }
+  red[share][col] = (s0 + s1) + (s2 + s3);
+  __syncthreads();
+  if (share == 0 && c < p.D) {
+    float s = 0.f;
+#pragma unroll
+    for (int q = 0; q < 8; ++q) s += red[q][col];
+    if (p.grad_dtype == RGLRU_BF16) ((__bf16*)p.dg)[c] = (__bf16)s; else ((float*)p.dg)[c] = s;
+  }
+}
+
+template <typename IO, int V, bool BACKWARD>
+static void norm_launch(int nvec, dim3 grid, hipStream_t s, const NormArgs& a) {
+  const int slots = (nvec + 63) / 64;
+  if (slots <= 1) hipLaunchKernelGGL((rmsnorm_kernel<IO, V, 1, BACKWARD>), grid, dim3(kNormThreads), 0, s, a);
+  else if (slots <= 2) hipLaunchKernelGGL((rmsnorm_kernel<IO, V, 2, BACKWARD>), grid, dim3(kNormThreads), 0, s, a);
+  else if (slots <= 4) hipLaunchKernelGGL((rmsnorm_kernel<IO, V, 4, BACKWARD>), grid, dim3(kNormThreads), 0, s, a);
+  else if (slots <= 8) hipLaunchKernelGGL((rmsnorm_kernel<IO, V, 8, BACKWARD>), grid, dim3(kNormThreads), 0, s, a);
+  else hipLaunchKernelGGL((rmsnorm_kernel<IO, V, 16, BACKWARD>), grid, dim3(kNormThreads), 0, s, a);
+}
+
+static int norm_grid(long long rows) {
+  long long blocks = (rows + (kNormThreads / 64) - 1) / (kNormThreads / 64);
+  const long long cap = (long long)num_compute_units() * 4;
+  if (blocks > cap) blocks = cap;
+  return (int)(blocks < 1 ? 1 : blocks);
+}
+
+static int norm_check(const char* who, int64_t rows, int64_t D, int dtype, int vec_dtype, bool* vec, int* nvec,
+                      std::initializer_list<const void*> ptrs) {
+  if (dtype != RGLRU_F32 && dtype != RGLRU_BF16) return fail(RGLRU_E_ARG, "%s: dtype must be RGLRU_F32 or RGLRU_BF16, got %d", who, dtype);
+  if (vec_dtype != RGLRU_F32 && vec_dtype != RGLRU_BF16) return fail(RGLRU_E_ARG, "%s: unknown parameter dtype %d", who, vec_dtype);
+  if (rows <= 0 || D <= 0) return fail(RGLRU_E_ARG, "%s: empty shape rows=%lld D=%lld", who, (long long)rows, (long long)D);
+  *vec = conv_vector_ok(D, dtype, ptrs);
+  const int v = *vec ? (dtype == RGLRU_BF16 ? 8 : 4) : 1;
+  *nvec = (int)(D / v);
+  if (*nvec > 64 * kNormSlots) return fail(RGLRU_E_UNSUPPORTED, "%s: rows of %lld elements exceed the supported %d", who, (long long)D, 64 * kNormSlots * v);
+  if (rows * D >= (1ll << 40)) return fail(RGLRU_E_UNSUPPORTED, "%s: tensor too large", who);
+  return RGLRU_OK;
+}
+
 }  // namespace rglru
 
 using namespace rglru;
@@ -806,6 +975,63 @@ int rglru_hip_conv_padded_fwd(const void* u, const void* state, const void* taps
   dim3 grid((unsigned)((items + kConvThreads - 1) / kConvThreads));
   RGLRU_CONV_DISPATCH(conv_padded_fwd_kernel, dtype, vec, grid, s, a);
   return check_launch("conv_padded_fwd");
+}
+
+int rglru_hip_rmsnorm_max_width(int dtype, int aligned) {
+  const int v = aligned ? (dtype == RGLRU_BF16 ? 8 : 4) : 1;
+  return 64 * kNormSlots * v;
+}
+
+int rglru_hip_rmsnorm_fwd(const void* x, const void* g, void* y, float* inv, int64_t rows, int64_t D, float eps,
+                          int dtype, int vec_dtype, void* stream) {
+  if (!x || !g || !y) return fail(RGLRU_E_ARG, "rmsnorm_fwd: null pointer");
+  bool vec; int nvec;
+  int rc = norm_check("rmsnorm_fwd", rows, D, dtype, vec_dtype, &vec, &nvec, {x, y});
+  if (rc) return rc;
+  NormArgs a;
+  memset(&a, 0, sizeof(a));
+  a.x = x; a.g = g; a.y = y; a.inv_out = inv; a.rows = rows; a.D = (int)D; a.nvec = nvec; a.vec_dtype = vec_dtype; a.eps = eps;
+  dim3 grid((unsigned)norm_grid(rows));
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == RGLRU_BF16) {
+    if (vec) norm_launch<__bf16, 8, false>(nvec, grid, s, a); else norm_launch<__bf16, 1, false>(nvec, grid, s, a);
+  } else {
+    if (vec) norm_launch<float, 4, false>(nvec, grid, s, a); else norm_launch<float, 1, false>(nvec, grid, s, a);
+  }
+  return check_launch("rmsnorm_fwd");
+}
+
+size_t rglru_hip_rmsnorm_scratch_bytes(int64_t rows, int64_t D) {
+  if (rows <= 0 || D <= 0) return 0;
+  return (size_t)norm_grid(rows) * (size_t)D * 4;
+}
+
+int rglru_hip_rmsnorm_bwd(const void* x, const void* g, const float* inv, const void* dy, void* scratch,
+                          void* dx, void* dg, int64_t rows, int64_t D, int dtype, int vec_dtype, int grad_dtype,
+                          void* stream) {
+  if (!x || !g || !inv || !dy || !scratch || !dx) return fail(RGLRU_E_ARG, "rmsnorm_bwd: null pointer");
+  if (grad_dtype != RGLRU_F32 && grad_dtype != RGLRU_BF16) return fail(RGLRU_E_ARG, "rmsnorm_bwd: unknown gradient dtype %d", grad_dtype);
+  bool vec; int nvec;
+  int rc = norm_check("rmsnorm_bwd", rows, D, dtype, vec_dtype, &vec, &nvec, {x, dy, dx});
+  if (rc) return rc;
+  NormArgs a;
+  memset(&a, 0, sizeof(a));
+  a.x = x; a.g = g; a.dy = dy; a.inv_in = inv; a.dx = dx; a.partial = (float*)scratch;
+  a.rows = rows; a.D = (int)D; a.nvec = nvec; a.vec_dtype = vec_dtype;
+  const int blocks = norm_grid(rows);
+  dim3 grid((unsigned)blocks);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == RGLRU_BF16) {
+    if (vec) norm_launch<__bf16, 8, true>(nvec, grid, s, a); else norm_launch<__bf16, 1, true>(nvec, grid, s, a);
+  } else {
+    if (vec) norm_launch<float, 4, true>(nvec, grid, s, a); else norm_launch<float, 1, true>(nvec, grid, s, a);
+  }
+  rc = check_launch("rmsnorm_bwd");
+  if (rc || !dg) return rc;
+  NormFinishArgs f;
+  f.partial = a.partial; f.dg = dg; f.D = (int)D; f.slots = blocks; f.grad_dtype = grad_dtype;
+  hipLaunchKernelGGL(rmsnorm_finish_kernel, dim3((unsigned)((D + 31) / 32)), dim3(256), 0, s, f);
+  return check_launch("rmsnorm_bwd finish");
 }
 
 }  // extern "C"

@@ -236,3 +236,56 @@ def hip_block_decode_step(u: Tensor, v: Tensor, conv_state: Tensor | None, weigh
             _ptr(x_conv), prep.image.data_ptr(), _ptr(h_in), _ptr(h_out), _ptr(flags), _ptr(v_c), _ptr(out),
             batch, width, prep.blocks, code, stream), "rglru_hip_step_gated")
     return out, h_out, new_conv, new_pos
+
+
+class _HipRMSNorm(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x: Tensor, g: Tensor, eps: float) -> Tensor:
+        _require_gpu("hip_rmsnorm", x, g)
+        if g.dim() != 1 or x.dim() < 1 or x.size(-1) != g.numel():
+            raise ValueError(f"hip_rmsnorm expects a scale of shape [{x.size(-1) if x.dim() else '?'}], got {tuple(g.shape)}")
+        code = _dtype_code(x.dtype)
+        width = x.size(-1)
+        x_c = x.contiguous()
+        rows = x_c.numel() // width
+        scale = _parameter_operand(g.detach(), x.dtype)
+        lib = _lib.load()
+        with torch.cuda.device(x.device):
+            y = torch.empty_like(x_c)
+            inv = torch.empty(rows, dtype=torch.float32, device=x.device)
+            if rows:
+                _lib.check(lib.rglru_hip_rmsnorm_fwd(_ptr(x_c), _ptr(scale), _ptr(y), _ptr(inv), rows, width, float(eps), code,
+                                                     _DTYPE_CODES[scale.dtype], _stream_ptr(x.device)), "rglru_hip_rmsnorm_fwd")
+        ctx.save_for_backward(x_c, scale, inv)
+        ctx.scale_dtype = g.dtype
+        return y
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, dy: Tensor):
+        x, scale, inv = ctx.saved_tensors
+        width = x.size(-1)
+        rows = x.numel() // width
+        dy_c = dy.to(x.dtype).contiguous()
+        lib = _lib.load()
+        need_g = ctx.needs_input_grad[1]
+        with torch.cuda.device(x.device):
+            dx = torch.empty_like(x)
+            dg = torch.empty(width, dtype=scale.dtype, device=x.device) if need_g else None
+            if rows:
+                scratch = torch.empty(lib.rglru_hip_rmsnorm_scratch_bytes(rows, width), dtype=torch.uint8, device=x.device)
+                _lib.check(lib.rglru_hip_rmsnorm_bwd(_ptr(x), _ptr(scale), _ptr(inv), _ptr(dy_c), _ptr(scratch), _ptr(dx), _ptr(dg),
+                                                     rows, width, _dtype_code(x.dtype), _DTYPE_CODES[scale.dtype],
+                                                     _DTYPE_CODES[scale.dtype], _stream_ptr(x.device)), "rglru_hip_rmsnorm_bwd")
+            elif dg is not None:
+                dg.zero_()
+        return dx, (None if dg is None else dg.to(ctx.scale_dtype)), None
+
+
+def rmsnorm_max_width(dtype: torch.dtype, aligned: bool = True) -> int:
+    return int(_lib.load().rglru_hip_rmsnorm_max_width(_dtype_code(dtype), 1 if aligned else 0))
+
+
+def hip_rmsnorm(x: Tensor, g: Tensor, eps: float = 1e-6) -> Tensor:
+    """``x * rsqrt(mean(x^2, -1) + eps) * (1 + g)`` (griffin/griffin.py:68-80), differentiable in x and g."""
+    return _HipRMSNorm.apply(x, g, eps)

@@ -450,6 +450,25 @@ def _validate_hip_scan(device: torch.device) -> None:
     for got, want in zip(hip_g, ref_g):
         torch.testing.assert_close(got, want, atol=3e-5, rtol=3e-5)
 
+    # RMSNorm in front of the block
+    from .hip_block_ops import hip_rmsnorm
+
+    def run_norm(use_hip):
+        leaves = [t.detach().clone().requires_grad_(True) for t in (x, conv_bias)]
+        if use_hip:
+            out = hip_rmsnorm(*leaves, 1e-6)
+        else:
+            out = leaves[0] * torch.rsqrt(leaves[0].pow(2).mean(dim=-1, keepdim=True) + 1e-6) * (1.0 + leaves[1])
+        return out, torch.autograd.grad(out, leaves, upstream)
+
+    ref_o, ref_g = run_norm(False)
+    hip_o, hip_g = run_norm(True)
+    torch.cuda.synchronize(device)
+    torch.testing.assert_close(hip_o, ref_o, atol=2e-5, rtol=2e-5)
+    for got, want in zip(hip_g, ref_g):
+        scale = max(1.0, float(want.abs().max()))
+        torch.testing.assert_close(got, want, atol=3e-5 * scale, rtol=3e-5)
+
 
 def hip_scan_is_usable(device: torch.device | str) -> bool:
     """Validate the HIP kernels once per device before ``scan_mode="auto"`` may use them."""

@@ -231,6 +231,31 @@ def _last_active_position(segment_pos: Tensor, active_mask: Tensor, previous_pos
     return torch.where(last >= 0, picked, fallback)
 
 
+class RMSNorm(nn.Module):
+    """Root-mean-square normalisation with a learned per-channel scale (griffin/griffin.py:68-80), the
+    layer in front of the recurrent block.  GPU tensors the HIP library covers go through its kernels
+    (after the same per-device self-test as ``scan_mode="auto"``); everything else through PyTorch."""
+
+    def __init__(self, dim: int, eps: float = 1e-6):
+        super().__init__()
+        self.eps = eps
+        self.g = nn.Parameter(torch.zeros(dim))
+
+    def _hip_covers(self, x: Tensor) -> bool:
+        if not x.is_cuda or x.dtype not in hip_scan.SUPPORTED_DTYPES or x.numel() == 0:
+            return False
+        if not hip_scan.hip_scan_is_usable(x.device):
+            return False
+        aligned = x.size(-1) % (8 if x.dtype == torch.bfloat16 else 4) == 0
+        return x.size(-1) <= hip_block_ops.rmsnorm_max_width(x.dtype, aligned)
+
+    def forward(self, x: Tensor) -> Tensor:
+        if self._hip_covers(x):
+            return hip_block_ops.hip_rmsnorm(x, self.g, self.eps)
+        normalized = x * torch.rsqrt(x.pow(2).mean(dim=-1, keepdim=True) + self.eps)
+        return normalized * (1.0 + self.g)
+
+
 class RecurrentBlock(nn.Module):
     """Linear -> causal depthwise conv -> RG-LRU, gated by GeLU(Linear), then Linear out
     (griffin/griffin.py:361-529).  The RG-LRU inside honours ``scan_mode`` unchanged."""

@@ -16,6 +16,7 @@
  *   autograd of griffin/griffin.py:474-487                                   rglru_hip_conv_bwd
  *   griffin/griffin.py:488-510      the same over right-padded batches (forward)   rglru_hip_conv_padded_fwd
  *   griffin/griffin.py:464, :520    x_branch * gelu_tanh(linear_y(x))        rglru_hip_gelu_gate_fwd, _bwd
+ *   griffin/griffin.py:68-80        RMSNorm in front of the block and its autograd   rglru_hip_rmsnorm_fwd, _bwd
  *   griffin/griffin.py:459-528 with T == 1 (block decode: positions, conv, step, gate)   rglru_hip_decode_prepare + rglru_hip_step_gated
  *
  * Conventions
@@ -45,7 +46,7 @@
 extern "C" {
 #endif
 
-#define RGLRU_ABI_VERSION 7
+#define RGLRU_ABI_VERSION 8
 
 enum { RGLRU_F32 = 0, RGLRU_BF16 = 1 };
 
@@ -211,6 +212,20 @@ int rglru_hip_conv_padded_fwd(const void* u, const void* state, const void* taps
 int rglru_hip_gelu_gate_fwd(const void* h, const void* v, void* out, int64_t n, int dtype, void* stream);
 int rglru_hip_gelu_gate_bwd(const void* dout, const void* h, const void* v, void* dh, void* dv,
                             int64_t n, int dtype, void* stream);
+
+/* RMSNorm in front of the block (griffin/griffin.py:68-80), over the last axis of x[rows, D]:
+ *   y = x * rsqrt(mean(x^2) + eps) * (1 + g),   g[D] read in vec_dtype;
+ * inv[rows] (fp32, may be NULL) receives rsqrt(mean(x^2) + eps) for the backward pass, which writes
+ * dx[rows, D] (dtype) and, when not NULL, dg[D] (grad_dtype); `scratch` holds
+ * rglru_hip_rmsnorm_scratch_bytes(rows, D) bytes.  D is at most rglru_hip_rmsnorm_max_width(dtype,
+ * aligned) (aligned: 16-byte aligned tensors and rows).  Arithmetic in fp32. */
+int rglru_hip_rmsnorm_max_width(int dtype, int aligned);
+int rglru_hip_rmsnorm_fwd(const void* x, const void* g, void* y, float* inv, int64_t rows, int64_t D, float eps,
+                          int dtype, int vec_dtype, void* stream);
+size_t rglru_hip_rmsnorm_scratch_bytes(int64_t rows, int64_t D);
+int rglru_hip_rmsnorm_bwd(const void* x, const void* g, const float* inv, const void* dy, void* scratch,
+                          void* dx, void* dg, int64_t rows, int64_t D, int dtype, int vec_dtype, int grad_dtype,
+                          void* stream);
 
 /* Single-token step of the recurrent block (griffin/griffin.py:459-528 with one token per row) in
  * two launches around the caller's three Linear layers:

@@ -300,6 +300,11 @@ def causal_conv_padded(px, conv_w, conv_b, conv_state, seg_pos, active):
     return torch.stack(rows, dim=1), window
 
 
+def rmsnorm(x, g, eps=1e-6):
+    """RMSNorm in front of the block (griffin/griffin.py:68-80): x * rsqrt(mean(x^2) + eps) * (1 + g)."""
+    return x * torch.rsqrt(x.pow(2).mean(dim=-1, keepdim=True) + eps) * (1.0 + g)
+
+
 def gelu_tanh(v):
     """tanh approximation of GeLU, the activation of the block's second branch (griffin/griffin.py:464,
     ``F.gelu(..., approximate="tanh")``): v/2 * (1 + tanh(sqrt(2/pi) * (v + 0.044715 v^3)))."""

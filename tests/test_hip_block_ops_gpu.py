@@ -280,3 +280,52 @@ def test_padded_conv_all_active_equals_dense_kernel_at_training_shape():
     dense, _ = hip_causal_conv(u, None, w, b, pos)
     padded, _ = hip_causal_conv_padded(u, None, w, b, pos, active)
     assert torch.equal(dense, padded)
+
+
+# ----------------------------------------------------------------------------------------------
+# RMSNorm in front of the block (C ABI: rglru_hip_rmsnorm_fwd / _bwd)
+# ----------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(2, 50, 64), (3, 7, 13), (1, 1, 768), (4, 33, 1024), (2, 5, 2560), (300, 24)])
+def test_rmsnorm_matches_oracle(shape, dtype):
+    from griffin_amd.hip_block_ops import hip_rmsnorm
+
+    _say("rmsnorm case", shape, dtype)
+    gen = torch.Generator().manual_seed(21)
+    x = torch.randn(*shape, generator=gen) * 1.7 + 0.3
+    scale = torch.randn(shape[-1], generator=gen) * 0.2
+    dy = torch.randn(*shape, generator=gen)
+    xr = x.to(dtype).float().requires_grad_(True)
+    sr = scale.to(dtype).float().requires_grad_(True)
+    want = orc.rmsnorm(xr, sr)
+    want_dx, want_dg = torch.autograd.grad(want, (xr, sr), dy.to(dtype).float())
+    xh = x.to(dtype).cuda().requires_grad_(True)
+    sh = scale.to(dtype).cuda().requires_grad_(True)
+    got = hip_rmsnorm(xh, sh)
+    got_dx, got_dg = torch.autograd.grad(got, (xh, sh), dy.to(dtype).cuda())
+    torch.cuda.synchronize()
+    tol = FP32_TOL if dtype == torch.float32 else BF16_TOL
+    errs = {"y": rel_err(got.float(), want), "dx": rel_err(got_dx.float(), want_dx), "dg": rel_err(got_dg.float(), want_dg)}
+    _say("  rel errors:", {k: "%.2e" % e for k, e in errs.items()})
+    for name, err in errs.items():
+        assert err < tol, (name, err)
+
+
+def test_rmsnorm_module_and_properties_at_training_shape():
+    """B8 T2048 D768 bf16 through the module: rows leave with mean square (1 + g)^2-weighted ~ 1 for a
+    zero scale, a positive rescaling of the input changes nothing (eps aside), and the module's state
+    dict keeps the reference's single parameter name."""
+    from griffin_amd import RMSNorm
+
+    norm = RMSNorm(768).cuda().bfloat16()
+    assert list(norm.state_dict()) == ["g"]
+    gen = torch.Generator().manual_seed(22)
+    x = (torch.randn(8, 2048, 768, generator=gen) * 3).bfloat16().cuda()
+    y = norm(x)
+    ms = y.float().pow(2).mean(-1)
+    assert (ms - 1.0).abs().max().item() < 2e-2
+    y4 = norm(4 * x)                                          # a power of two: exact in bf16
+    assert rel_err(y4.float(), y.float()) < 1e-2
+    with pytest.raises(ValueError):
+        from griffin_amd.hip_block_ops import hip_rmsnorm
+        hip_rmsnorm(x, torch.zeros(5, device="cuda", dtype=torch.bfloat16))

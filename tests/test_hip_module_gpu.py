@@ -305,23 +305,28 @@ def test_config5_recurrent_block_with_hip_scan():
     """d_model 768 -> width 1024 block: the HIP scan slotted into the block unchanged, forward and
     backward against the same block on the CPU with the sequential scan (fp32, reduced length),
     then the bf16 training shape B8 T2048 for finiteness and cache semantics."""
-    from griffin_amd import RecurrentBlock
+    from griffin_amd import RMSNorm, RecurrentBlock
 
     torch.manual_seed(5)
     cpu_block = RecurrentBlock(768, 1024, gate_blocks=8, scan_mode="sequential")
+    cpu_norm = RMSNorm(768)                                  # the RMSNorm in front of the block
+    with torch.no_grad():
+        cpu_norm.g.copy_(0.1 * torch.randn(768))
     hip_block = copy.deepcopy(cpu_block).cuda()
+    hip_norm = copy.deepcopy(cpu_norm).cuda()
     hip_block.scan_mode = None
     hip_block.rg_lru.scan_mode = "hip"
     x = torch.randn(2, 160, 768)
     xc = x.clone().requires_grad_(True)
     xh = x.clone().cuda().requires_grad_(True)
     up = torch.randn(2, 160, 768)
-    yc = cpu_block(xc)
-    yh = hip_block(xh)
+    yc = cpu_block(cpu_norm(xc))
+    yh = hip_block(hip_norm(xh))
     yc.backward(up)
     yh.backward(up.cuda())
     assert rel_err(yh, yc) < 1e-4
     assert rel_err(xh.grad, xc.grad) < 1e-4
+    assert rel_err(hip_norm.g.grad, cpu_norm.g.grad) < 2e-4
     for (name, ph), (_, pc) in zip(hip_block.named_parameters(), cpu_block.named_parameters()):
         assert rel_err(ph.grad, pc.grad) < 2e-4, name
 

@@ -367,3 +367,18 @@ def test_oracle_padded_conv_reduces_to_dense_conv_and_skips_padding():
     # all tokens inactive: zeros out, state untouched
     none, same = orc.causal_conv_padded(px, w, b, state, seg, torch.zeros(B, T, dtype=torch.bool))
     assert torch.count_nonzero(none) == 0 and torch.equal(same, state)
+
+
+def test_oracle_rmsnorm_closed_forms():
+    """Unit scale: every row leaves with mean square 1 (up to eps); a constant row c becomes sign(c)
+    (1 + g); scaling the input by a positive factor changes nothing; matches the library's rms_norm."""
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(5, 7, 12, generator=g, dtype=torch.float64)
+    scale = torch.randn(12, generator=g, dtype=torch.float64) * 0.3
+    y = orc.rmsnorm(x, torch.zeros(12, dtype=torch.float64))
+    torch.testing.assert_close(y.pow(2).mean(-1), torch.ones(5, 7, dtype=torch.float64), atol=1e-5, rtol=0)
+    const = torch.full((3, 12), -2.5, dtype=torch.float64)
+    torch.testing.assert_close(orc.rmsnorm(const, scale), -(1.0 + scale).expand(3, 12), atol=1e-6, rtol=0)
+    torch.testing.assert_close(orc.rmsnorm(3.0 * x, scale, eps=0.0), orc.rmsnorm(x, scale, eps=0.0), atol=1e-12, rtol=1e-12)
+    want = torch.nn.functional.rms_norm(x, (12,), weight=1.0 + scale, eps=1e-6)
+    torch.testing.assert_close(orc.rmsnorm(x, scale), want, atol=1e-12, rtol=1e-12)
