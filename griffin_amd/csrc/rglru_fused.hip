@@ -448,7 +448,20 @@ RGLRU_DEVICE void fwd_finalize(const FusedArgs& p, const WaveId& w, const FwdTil
   }
 }
 
-constexpr int kFwdMT = 1;               // forward tile = 32 * kFwdMT tokens
+// Forward tile = 32 * kFwdMT tokens.  Two ways to run the loop, chosen by kFwdDefer:
+//   true   (needs kFwdMT = 1 to fit the registers) two tiles in flight, the previous tile is finished
+//          after the gate math of the current one, its records requested an iteration ahead;
+//   false  a tile is finished in the iteration that computed it.
+// 64-token tiles without the deferral halve the look-backs, barriers, tickets and records per token,
+// which is worth more than hiding them: 39.6 us against 43.5 us at B8 T2048 W1024, 84 us against
+// 104 us for one sequence of 32768 tokens.
+#ifdef RGLRU_FWD_DEFER
+constexpr int kFwdMT = 1;
+constexpr bool kFwdDefer = true;
+#else
+constexpr int kFwdMT = 2;
+constexpr bool kFwdDefer = false;
+#endif
 
 // workgroups per compute unit of the forward kernel without weights in registers (NKG < 0); 4 spills
 #define RGLRU_GIVEN_OCC 3
@@ -558,8 +571,12 @@ __global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : 2)) void fwd
       const unsigned next_raw = (unsigned)__builtin_amdgcn_raw_ptr_buffer_atomic_add_i32(1, rticket, tid == 0 ? 0u : kOutOfRange, 0, 0);
       // records the previous tile will need: requested now, used after this tile's gate math
       CarryBatch ahead;
-      carry_prefetch(make_rsrc(p.rec_a + (long long)prev.b * p.nCf * W, (unsigned)p.nCf * rec_stride), rec_lane,
-                     rec_stride, prev.c, -1, -1, ahead);
+      if constexpr (kFwdDefer)
+        carry_prefetch(make_rsrc(p.rec_a + (long long)prev.b * p.nCf * W, (unsigned)p.nCf * rec_stride), rec_lane,
+                       rec_stride, prev.c, -1, -1, ahead);
+      else
+        carry_prefetch(make_rsrc(p.rec_a + (long long)cur.b * p.nCf * W, (unsigned)p.nCf * rec_stride), rec_lane,
+                       rec_stride, cur.c, -1, -1, ahead);
 #pragma unroll
       for (int i = 0; i < NV; ++i) {
         const int idx = tid + i * kThreads;
@@ -580,11 +597,10 @@ __global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : 2)) void fwd
           f32x16 ua, ux;
           float xv[16];
           if constexpr (GIVEN) {
-            static_assert(MT == 1, "one accumulator tile per wave");
             const int col = w.wave * 32 + w.r;
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
-              const int at = (hf * 16 + e) * LDSROW + col;
+              const int at = (hf * 16 * MT + 16 * mt + e) * LDSROW + col;
               xv[e] = (float)lds[at];
               ua[e] = bias_a + (float)lds_pre[at];
               ux[e] = bias_x + (float)lds_pre[TR * LDSROW + at];
@@ -603,14 +619,18 @@ __global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : 2)) void fwd
       const long long tk_next = s_ticket[par];
       issue(tk_next);
       RGLRU_STAMP(p, 4);
-      fwd_finalize<IO, MT, MASKED, sizeof(IO) == 2>(p, w, prev, stage, &ahead, have_prev && slab_ok, trace_iter);
-      prev = cur;
-      have_prev = true;
+      if constexpr (kFwdDefer) {
+        fwd_finalize<IO, MT, MASKED, sizeof(IO) == 2>(p, w, prev, stage, &ahead, have_prev && slab_ok, trace_iter);
+        prev = cur;
+        have_prev = true;
+      } else {
+        fwd_finalize<IO, MT, MASKED, sizeof(IO) == 2>(p, w, cur, stage, &ahead, slab_ok, trace_iter);
+      }
       RGLRU_STAMP(p, 7);
       ++trace_iter;
       tk = tk_next;
     }
-    if (slab_ok && have_prev) fwd_finalize<IO, MT, MASKED, sizeof(IO) == 2>(p, w, prev, stage, nullptr, true, trace_iter);
+    if (kFwdDefer && slab_ok && have_prev) fwd_finalize<IO, MT, MASKED, sizeof(IO) == 2>(p, w, prev, stage, nullptr, true, trace_iter);
   } else {
     for (;;) {
       if (tid == 0) s_ticket[0] = atomicAdd(q.counter, 1u);
