@@ -28,7 +28,7 @@ HBM_PEAK_GBS = 8000.0
 # runs of this script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same
 # counter reads for the 64 MiB copy that --traffic-probe adds (profiles/ holds the summaries).  Only
 # valid for that workload; other shapes report null.
-MEASURED_TRAFFIC_BYTES = {"bwd_scan_kernel": 220572523, "fwd_kernel": 85709179, "gate_grad_kernel": 201903992}
+MEASURED_TRAFFIC_BYTES = {"bwd_scan_kernel": 220478428, "fwd_kernel": 79377614, "gate_grad_kernel": 201923976}
 BENCH_SHAPE = (8, 2048, 1024, 8)
 
 
