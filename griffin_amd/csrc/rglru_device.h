@@ -345,21 +345,43 @@ RGLRU_DEVICE float masked_log2_decay(float l2, unsigned fl) {
   l2 = (fl & 1u) ? kResetLog2 : l2;
   return (fl & 2u) ? 0.0f : l2;
 }
+// The same for token e of a packed run (two flag bits per token): bit-field extracts that sign-extend
+// a flag into an all-ones mask and bitwise selects, so no compare results are kept per token.
+RGLRU_DEVICE float masked_log2_decay_run(float l2, unsigned flbits, int e) {
+  unsigned m_reset = (unsigned)__builtin_amdgcn_sbfe((int)flbits, 2 * e, 1);
+  unsigned m_pad = (unsigned)__builtin_amdgcn_sbfe((int)flbits, 2 * e + 1, 1);
+  asm("" : "+v"(m_reset), "+v"(m_pad));          // opaque: keeps the compiler from turning the masks back into compares
+  unsigned u = __builtin_bit_cast(unsigned, l2);
+  u = (u & ~m_reset) | (__builtin_bit_cast(unsigned, kResetLog2) & m_reset);
+  u &= ~m_pad;
+  return __builtin_bit_cast(float, u);
+}
 
-// MASKED = false: the token is known to be an ordinary one (no reset, active), fl is ignored.
-template <bool PRECISE, bool MASKED>
-RGLRU_DEVICE GateOut gate_forward(float ua, float ux, float x, float sp, unsigned fl) {
+// Gate outputs from the two sigmoids and the (possibly masked) log2 of the decay.
+template <bool PRECISE>
+RGLRU_DEVICE GateOut gate_outputs(float r, float i, float x, float l2) {
   GateOut o;
-  o.r = sigmoid_fast(ua);
-  o.i = sigmoid_fast(ux);
-  float l2 = o.r * sp;                         // log2(a) <= 0
-  if constexpr (MASKED) l2 = masked_log2_decay(l2, fl);
+  o.r = r; o.i = i;
   const float a = __builtin_amdgcn_exp2f(l2);
   const float g2 = fmaxf(one_minus_exp<PRECISE>(l2 * (2.0f * kLn2), a), 0.0f);
   const float g = __builtin_amdgcn_sqrtf(g2);
   o.g2 = g2;
-  o.a = a; o.g = g; o.z = g * o.i * x;
+  o.a = a; o.g = g; o.z = g * i * x;
   return o;
+}
+// MASKED = false: the token is known to be an ordinary one (no reset, active), fl is ignored.
+template <bool PRECISE, bool MASKED>
+RGLRU_DEVICE GateOut gate_forward(float ua, float ux, float x, float sp, unsigned fl) {
+  const float r = sigmoid_fast(ua), i = sigmoid_fast(ux);
+  float l2 = r * sp;                           // log2(a) <= 0
+  if constexpr (MASKED) l2 = masked_log2_decay(l2, fl);
+  return gate_outputs<PRECISE>(r, i, x, l2);
+}
+// Token e of a run whose flags are packed two bits per token.
+template <bool PRECISE>
+RGLRU_DEVICE GateOut gate_forward_run(float ua, float ux, float x, float sp, unsigned flbits, int e) {
+  const float r = sigmoid_fast(ua), i = sigmoid_fast(ux);
+  return gate_outputs<PRECISE>(r, i, x, masked_log2_decay_run(r * sp, flbits, e));
 }
 
 // gelu_tanh(v) = v/2 * (1 + tanh(u)), u = sqrt(2/pi) * (v + 0.044715 v^3), and its derivative

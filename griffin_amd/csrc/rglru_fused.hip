@@ -329,14 +329,13 @@ RGLRU_DEVICE unsigned flag_run(const FusedArgs& p, long long token_row, int t_fi
 // Gate math of 16 consecutive local steps (first = index of the first one in this lane's run).
 // MASKED = false is the common case: no flags, the tile lies inside the sequence.
 template <typename IO, bool MASKED>
-RGLRU_DEVICE void fwd_gates(const FusedArgs& p, long long trow, int t_first, const f32x16& ua, const f32x16& ux,
+RGLRU_DEVICE void fwd_gates(unsigned flbits, const f32x16& ua, const f32x16& ux,
                             const float (&xv)[16], float sp, float* a, float* z) {
-  unsigned flbits = 0u;
-  if constexpr (MASKED) flbits = flag_run(p, trow, t_first);
 #pragma unroll
   for (int v = 0; v < 16; ++v) {
-    const unsigned fl = MASKED ? ((flbits >> (2 * v)) & 3u) : 0u;
-    GateOut go = gate_forward<Precise<IO>::value, MASKED>(ua[v], ux[v], xv[v], sp, fl);
+    GateOut go;
+    if constexpr (MASKED) go = gate_forward_run<Precise<IO>::value>(ua[v], ux[v], xv[v], sp, flbits, v);
+    else go = gate_forward<Precise<IO>::value, false>(ua[v], ux[v], xv[v], sp, 0u);
     a[v] = go.a; z[v] = go.z;
   }
 }
@@ -567,6 +566,10 @@ __global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : 2)) void fwd
       cur.c = (int)((unsigned)tk / (unsigned)q.n_b);
       cur.b = q.first_b + (int)((unsigned)tk - (unsigned)cur.c * (unsigned)q.n_b) * p.queues;
       const long long trow = (long long)cur.b * p.T + cur.c * TR + hf * EL;
+      // token flags of this lane's runs: requested first, so that the gate math waits for nothing younger
+      unsigned flbits[MT];
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) flbits[mt] = MASKED ? flag_run(p, trow + 16 * mt, cur.c * TR + hf * EL + 16 * mt) : 0u;
       // next ticket: one instruction for the whole workgroup, live only in its first lane
       const unsigned next_raw = (unsigned)__builtin_amdgcn_raw_ptr_buffer_atomic_add_i32(1, rticket, tid == 0 ? 0u : kOutOfRange, 0, 0);
       // records the previous tile will need: requested now, used after this tile's gate math
@@ -607,7 +610,7 @@ __global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : 2)) void fwd
             }
           } else
           gate_mfma_held<IO, MT, NKG, KC>(lds, hw, mt, w.slab, w.r, hf, bias_a, bias_x, ua, ux, xv, NKG == 8 ? 0 : w.kb);
-          fwd_gates<IO, MASKED>(p, trow + 16 * mt, cur.c * TR + hf * EL + 16 * mt, ua, ux, xv, sp, cur.a + 16 * mt, cur.z + 16 * mt);
+          fwd_gates<IO, MASKED>(flbits[mt], ua, ux, xv, sp, cur.a + 16 * mt, cur.z + 16 * mt);
         }
       }
       fwd_local<MT, MASKED>(p, w, cur, slab_ok);
@@ -651,7 +654,7 @@ __global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : 2)) void fwd
           float xpart[16];
 #pragma unroll
           for (int e = 0; e < 16; ++e) xpart[e] = xv[16 * mt + e];
-          fwd_gates<IO, true>(p, trow + 16 * mt, c * TR + hf * EL + 16 * mt, ua[mt], ux[mt], xpart, sp, tile.a + 16 * mt, tile.z + 16 * mt);
+          fwd_gates<IO, true>(flag_run(p, trow + 16 * mt, c * TR + hf * EL + 16 * mt), ua[mt], ux[mt], xpart, sp, tile.a + 16 * mt, tile.z + 16 * mt);
         }
         fwd_local<MT, true>(p, w, tile);
         // 16-bit outputs go through the wave's staging area when whole 64-byte row segments can be
@@ -938,7 +941,10 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
     const long long trow = (long long)b * p.T + t0 + hf * EL;
     unsigned next_raw = 0;
     if (tid == 0) next_raw = atomicAdd(q.counter, 1u);
-    // state at the start of the chunk (forward checkpoint), requested early
+    // token flags (two bits per local step) and the state at the start of the chunk (forward
+    // checkpoint), requested early
+    unsigned flbits = 0u;
+    if constexpr (MASKED) flbits = flag_run(p, trow, t0 + hf * EL);
     float h_start = 0.f;
     if (c == 0) { if (p.h0) h_start = p.h0[(long long)b * W + w.ch]; }
     else h_start = p.ckpt[((long long)b * p.ckpt_nC + (c - 1)) * W + w.ch];
@@ -1008,14 +1014,12 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
     // so the recurrence gate comes first and the map is published before the rest of the gate math:
     // the neighbours see it that much earlier.  z is not kept (g * i * x is recomputed where needed).
     float r[EL], gi[EL], a[EL], g[EL];
-    unsigned flbits = 0u;                                // two flag bits per local step
-    if constexpr (MASKED) flbits = flag_run(p, trow, t0 + hf * EL);
     float A = 1.f;
 #pragma unroll
     for (int e = 0; e < EL; ++e) {
       const float re = sigmoid_fast(ua[e]);
       float l2 = re * sp;
-      if constexpr (MASKED) l2 = masked_log2_decay(l2, (flbits >> (2 * e)) & 3u);
+      if constexpr (MASKED) l2 = masked_log2_decay_run(l2, flbits, e);
       const float ae = __builtin_amdgcn_exp2f(l2);
       r[e] = re; a[e] = ae;
       A *= ae;
@@ -1044,7 +1048,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
     for (int e = 0; e < EL; ++e) {
       const float ie = sigmoid_fast(ux[e]);
       float l2 = r[e] * sp;
-      if constexpr (MASKED) l2 = masked_log2_decay(l2, (flbits >> (2 * e)) & 3u);     // gives g = 1 / g = 0
+      if constexpr (MASKED) l2 = masked_log2_decay_run(l2, flbits, e);     // gives g = 1 / g = 0
       const float ge = __builtin_amdgcn_sqrtf(fmaxf(one_minus_exp<false>(l2 * (2.0f * kLn2), a[e]), 0.0f));
       const float ze = ge * ie * xv[e];
       gi[e] = ie; g[e] = ge;
