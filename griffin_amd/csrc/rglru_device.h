@@ -309,8 +309,10 @@ struct GateOut {
   float r, i, a, g, g2, z;   // a, g, g2 = g * g and z include the token's masks
 };
 
-RGLRU_DEVICE float sigmoid_fast(float u) {
-  return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-kLog2e * u));
+// sigmoid(u + b) with the bias passed as nb = -log2(e) * b: the addition rides on the multiplication
+// the exponent needs anyway, and a matrix product that feeds u can start from a zero accumulator.
+RGLRU_DEVICE float sigmoid_fast(float u, float nb = 0.0f) {
+  return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(fmaf(-kLog2e, u, nb)));
 }
 
 // 1 - exp(y) for y <= 0 without cancellation: Taylor series near zero, direct form elsewhere.
@@ -371,16 +373,17 @@ RGLRU_DEVICE GateOut gate_outputs(float r, float i, float x, float l2) {
 }
 // MASKED = false: the token is known to be an ordinary one (no reset, active), fl is ignored.
 template <bool PRECISE, bool MASKED>
-RGLRU_DEVICE GateOut gate_forward(float ua, float ux, float x, float sp, unsigned fl) {
-  const float r = sigmoid_fast(ua), i = sigmoid_fast(ux);
+RGLRU_DEVICE GateOut gate_forward(float ua, float ux, float x, float sp, unsigned fl, float nba = 0.0f, float nbx = 0.0f) {
+  const float r = sigmoid_fast(ua, nba), i = sigmoid_fast(ux, nbx);
   float l2 = r * sp;                           // log2(a) <= 0
   if constexpr (MASKED) l2 = masked_log2_decay(l2, fl);
   return gate_outputs<PRECISE>(r, i, x, l2);
 }
 // Token e of a run whose flags are packed two bits per token.
 template <bool PRECISE>
-RGLRU_DEVICE GateOut gate_forward_run(float ua, float ux, float x, float sp, unsigned flbits, int e) {
-  const float r = sigmoid_fast(ua), i = sigmoid_fast(ux);
+RGLRU_DEVICE GateOut gate_forward_run(float ua, float ux, float x, float sp, unsigned flbits, int e,
+                                      float nba = 0.0f, float nbx = 0.0f) {
+  const float r = sigmoid_fast(ua, nba), i = sigmoid_fast(ux, nbx);
   return gate_outputs<PRECISE>(r, i, x, masked_log2_decay_run(r * sp, flbits, e));
 }
 

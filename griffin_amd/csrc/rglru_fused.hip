@@ -330,12 +330,12 @@ RGLRU_DEVICE unsigned flag_run(const FusedArgs& p, long long token_row, int t_fi
 // MASKED = false is the common case: no flags, the tile lies inside the sequence.
 template <typename IO, bool MASKED>
 RGLRU_DEVICE void fwd_gates(unsigned flbits, const f32x16& ua, const f32x16& ux,
-                            const float (&xv)[16], float sp, float* a, float* z) {
+                            const float (&xv)[16], float sp, float* a, float* z, float nba = 0.0f, float nbx = 0.0f) {
 #pragma unroll
   for (int v = 0; v < 16; ++v) {
     GateOut go;
-    if constexpr (MASKED) go = gate_forward_run<Precise<IO>::value>(ua[v], ux[v], xv[v], sp, flbits, v);
-    else go = gate_forward<Precise<IO>::value, false>(ua[v], ux[v], xv[v], sp, 0u);
+    if constexpr (MASKED) go = gate_forward_run<Precise<IO>::value>(ua[v], ux[v], xv[v], sp, flbits, v, nba, nbx);
+    else go = gate_forward<Precise<IO>::value, false>(ua[v], ux[v], xv[v], sp, 0u, nba, nbx);
     a[v] = go.a; z[v] = go.z;
   }
 }
@@ -548,6 +548,7 @@ __global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : 2)) void fwd
     // iteration is finished (carry in, recurrence, stores) after the gate math of the current one,
     // so the wait for the neighbours' records overlaps with useful work.
     FwdTile<MT> cur, prev;
+    const float nba = -kLog2e * bias_a, nbx = -kLog2e * bias_x;
     bool have_prev = false;
     prev.b = 0; prev.c = 0;                              // chunk 0 has no records to request
 #pragma unroll
@@ -605,12 +606,13 @@ __global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : 2)) void fwd
             for (int e = 0; e < 16; ++e) {
               const int at = (hf * 16 * MT + 16 * mt + e) * LDSROW + col;
               xv[e] = (float)lds[at];
-              ua[e] = bias_a + (float)lds_pre[at];
-              ux[e] = bias_x + (float)lds_pre[TR * LDSROW + at];
+              ua[e] = (float)lds_pre[at];
+              ux[e] = (float)lds_pre[TR * LDSROW + at];
             }
           } else
-          gate_mfma_held<IO, MT, NKG, KC>(lds, hw, mt, w.slab, w.r, hf, bias_a, bias_x, ua, ux, xv, NKG == 8 ? 0 : w.kb);
-          fwd_gates<IO, MASKED>(flbits[mt], ua, ux, xv, sp, cur.a + 16 * mt, cur.z + 16 * mt);
+          gate_mfma_held<IO, MT, NKG, KC>(lds, hw, mt, w.slab, w.r, hf, 0.0f, 0.0f, ua, ux, xv, NKG == 8 ? 0 : w.kb);
+          // the biases enter inside the sigmoids
+          fwd_gates<IO, MASKED>(flbits[mt], ua, ux, xv, sp, cur.a + 16 * mt, cur.z + 16 * mt, nba, nbx);
         }
       }
       fwd_local<MT, MASKED>(p, w, cur, slab_ok);
@@ -875,7 +877,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
   } else if constexpr (!GIVEN) {
     hw.load(w_a_row, w_x_row);
   }
-  const float bias_a = p.bias[w.kp], bias_x = p.bias[p.Wp + w.kp];
+  const float nba = -kLog2e * p.bias[w.kp], nbx = -kLog2e * p.bias[p.Wp + w.kp];   // biases as the sigmoids take them
   const float sp = p.sp[w.kp], cs = p.cs[w.kp];
   const IO* x = (const IO*)p.x;
   const IO* dy = (const IO*)p.dy;
@@ -973,12 +975,12 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
           const int at = (hf * EL + e) * LDSROW + col;
           xv[e] = (float)lds_x[at];
           gy[e] = (float)lds_dy[at];
-          ua[e] = bias_a + (float)lds_pre[at];
-          ux[e] = bias_x + (float)lds_pre[TR * LDSROW + at];
+          ua[e] = (float)lds_pre[at];
+          ux[e] = (float)lds_pre[TR * LDSROW + at];
         }
       } else if constexpr (XLDS) {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) { ua[v] = bias_a; ux[v] = bias_x; }
+        for (int v = 0; v < 16; ++v) { ua[v] = 0.0f; ux[v] = 0.0f; }     // the biases enter inside the sigmoids
         const int kb = NKG == 8 ? 0 : w.kb;
         const IO* xrow = lds_x + tile_row<MT>(0, w.r) * LDSROW + kb + hf * Tr::HW;
         const IO* brow = lds_wx + (w.wave * 32 + w.r) * WROW + hf * Tr::HW;
@@ -991,7 +993,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
 #pragma unroll
         for (int e = 0; e < EL; ++e) xv[e] = (float)lds_x[(hf * EL + e) * LDSROW + kb + w.slab * 32 + w.r];
       } else {
-        gate_mfma_held<IO, MT, NKG, TW>(lds_x, hw, 0, w.slab, w.r, hf, bias_a, bias_x, ua, ux, xv, w.kb);
+        gate_mfma_held<IO, MT, NKG, TW>(lds_x, hw, 0, w.slab, w.r, hf, 0.0f, 0.0f, ua, ux, xv, w.kb);
       }
       if constexpr (!GIVEN) {
 #pragma unroll
@@ -1017,7 +1019,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
     float A = 1.f;
 #pragma unroll
     for (int e = 0; e < EL; ++e) {
-      const float re = sigmoid_fast(ua[e]);
+      const float re = sigmoid_fast(ua[e], nba);
       float l2 = re * sp;
       if constexpr (MASKED) l2 = masked_log2_decay_run(l2, flbits, e);
       const float ae = __builtin_amdgcn_exp2f(l2);
@@ -1046,7 +1048,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
     float H = 0.f;
 #pragma unroll
     for (int e = 0; e < EL; ++e) {
-      const float ie = sigmoid_fast(ux[e]);
+      const float ie = sigmoid_fast(ux[e], nbx);
       float l2 = r[e] * sp;
       if constexpr (MASKED) l2 = masked_log2_decay_run(l2, flbits, e);     // gives g = 1 / g = 0
       const float ge = __builtin_amdgcn_sqrtf(fmaxf(one_minus_exp<false>(l2 * (2.0f * kLn2), a[e]), 0.0f));
@@ -1086,8 +1088,9 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
       const float c1 = ge * ie;
       const float dxd = d * c1;
       const float ze = c1 * xe;
-      const float q = (ie * xe) * __builtin_amdgcn_rsqf(fmaxf(4.0f * (ge * ge), 1e-6f));
-      float dl = (a[e] * d) * fmaf(-2.0f * a[e], q, h);
+      // 2 q with q = i x / sqrt(max(4 g^2, 1e-6)): the factors 4 and 2 cancel exactly (powers of two)
+      const float q2 = (ie * xe) * __builtin_amdgcn_rsqf(fmaxf(ge * ge, 0.25f * 1e-6f));
+      float dl = (a[e] * d) * fmaf(-a[e], q2, h);
       // A reset token has a = 2^-126, which already switches dl off; a padded one has g = 0, which
       // zeroes dxd, vx and z, but its bounded-sqrt term would leak into dl.
       if constexpr (MASKED) { if ((flbits >> (2 * e)) & 2u) dl = 0.f; }
