@@ -114,10 +114,12 @@ BF16_CASES = [
     (2, 80, 256, 2, True, False),    # length a multiple of 16 but not of 32: vector flag loads, half-empty tile
     (1, 700, 128, 1, True, True),    # one sequence: every workgroup of the block works on the same chain
     (70, 40, 128, 1, False, False),  # more sequences than ticket queues
-    (3, 17, 128, 2, True, True),     # shorter than one tile    (2, 100, 192, 3, True, True),    # 64-wide blocks packed two to a unit, last unit half empty
+    (3, 17, 128, 2, True, True),     # shorter than one tile
+    (2, 100, 192, 3, True, True),    # 64-wide blocks packed two to a unit, last unit half empty
     (2, 70, 96, 3, False, True),     # 32-wide blocks packed four to a unit, last unit one block short
     (1, 64, 64, 1, False, False),    # a single 64-wide block: half of the packed unit idles
-    (2, 64, 1024, 16, True, False),  # reference default of 16 gate blocks at width 1024    (2, 100, 512, 2, True, True),    # 256-wide blocks: library GEMM for the projections, two workgroups per block
+    (2, 64, 1024, 16, True, False),  # reference default of 16 gate blocks at width 1024
+    (2, 100, 512, 2, True, True),    # 256-wide blocks: library GEMM for the projections, two workgroups per block
     (2, 75, 480, 3, False, True),    # 160-wide blocks: five slabs, the second workgroup of a block has one
     (1, 64, 96, 1, True, False),     # 96-wide block: three slabs in one workgroup
     (3, 33, 384, 2, True, True),     # 192-wide blocks, ragged tile, flags
@@ -129,6 +131,10 @@ def test_fused_bf16_matches_fp32_oracle(cfg):
     B, T, W, nb, masks, with_h0 = cfg
     _say("fused bf16 case", cfg)
     case = orc.make_case(B, T, W, nb, seed=2, h0_std=0.5 if with_h0 else 0.0)
+    # per-channel biases (the reference initialises them to zero, training does not keep them there)
+    gen = torch.Generator().manual_seed(7)
+    case["b_a"] = 0.5 * torch.randn(case["b_a"].shape, generator=gen)
+    case["b_x"] = 0.5 * torch.randn(case["b_x"].shape, generator=gen)
     reset, active = _masks(B, T, masks)
     dh_last = torch.randn(B, W, generator=torch.Generator().manual_seed(6)) if with_h0 else None
     y, h_last, grads = hip_run(case, torch.bfloat16, reset, active, dh_last)
