@@ -235,8 +235,11 @@ def lambda_init(width: int, gen: torch.Generator, lo=0.9, hi=0.999, c=8.0, dtype
     return torch.logit(base).to(dtype)
 
 
-def make_case(B, T, W, nb, seed=0, lo=0.9, hi=0.999, c=8.0, h0_std=0.0):
-    """Synthetic inputs of the benchmark configurations: fp32 tensors on the CPU."""
+def make_case(B, T, W, nb, seed=0, lo=0.9, hi=0.999, c=8.0, h0_std=0.0, bias_std=0.0):
+    """Synthetic inputs of the benchmark configurations: fp32 tensors on the CPU.  The gate biases
+    are zero, as the reference initialises them, unless bias_std > 0 (parity cases: a trained model
+    does not keep them at zero); they come from a generator of their own, so the other tensors do
+    not depend on bias_std."""
     gen = torch.Generator().manual_seed(seed)
     bw = W // nb
     x = torch.randn(B, T, W, generator=gen)
@@ -245,6 +248,10 @@ def make_case(B, T, W, nb, seed=0, lo=0.9, hi=0.999, c=8.0, h0_std=0.0):
     lam = lambda_init(W, gen, lo, hi, c)
     dy = torch.randn(B, T, W, generator=gen)
     h0 = torch.randn(B, W, generator=gen) * h0_std if h0_std > 0 else None
+    if bias_std > 0:
+        gen_b = torch.Generator().manual_seed(seed + 7919)
+        b_a = bias_std * torch.randn(nb, bw, generator=gen_b)
+        b_x = bias_std * torch.randn(nb, bw, generator=gen_b)
     return {"x": x, "w_a": w_a, "b_a": b_a, "w_x": w_x, "b_x": b_x, "lam": lam, "dy": dy, "h0": h0}
 
 

@@ -130,11 +130,8 @@ BF16_CASES = [
 def test_fused_bf16_matches_fp32_oracle(cfg):
     B, T, W, nb, masks, with_h0 = cfg
     _say("fused bf16 case", cfg)
-    case = orc.make_case(B, T, W, nb, seed=2, h0_std=0.5 if with_h0 else 0.0)
-    # per-channel biases (the reference initialises them to zero, training does not keep them there)
-    gen = torch.Generator().manual_seed(7)
-    case["b_a"] = 0.5 * torch.randn(case["b_a"].shape, generator=gen)
-    case["b_x"] = 0.5 * torch.randn(case["b_x"].shape, generator=gen)
+    # per-channel biases: the reference initialises them to zero, training does not keep them there
+    case = orc.make_case(B, T, W, nb, seed=2, h0_std=0.5 if with_h0 else 0.0, bias_std=0.5)
     reset, active = _masks(B, T, masks)
     dh_last = torch.randn(B, W, generator=torch.Generator().manual_seed(6)) if with_h0 else None
     y, h_last, grads = hip_run(case, torch.bfloat16, reset, active, dh_last)
@@ -196,7 +193,7 @@ def test_step_kernel_matches_oracle(dtype, tol):
     from griffin_amd import PreparedParams, hip_rglru_step
 
     B, W, nb, steps = 5, 96, 3, 6
-    case = orc.make_case(B, steps, W, nb, seed=3, h0_std=0.5)
+    case = orc.make_case(B, steps, W, nb, seed=3, h0_std=0.5, bias_std=0.5)
     p = [case[k].to(dtype) for k in PARAMS]
     prep = PreparedParams(*[t.cuda() for t in p[1:]], 8.0, dtype)
     state = case["h0"].float().cuda().clone()

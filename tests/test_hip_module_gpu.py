@@ -101,7 +101,7 @@ def test_saturated_gate_stays_finite_in_bf16():
 
 
 def test_chunked_calls_with_carried_state_equal_one_call():
-    case = orc.make_case(2, 200, 128, 2, seed=4)
+    case = orc.make_case(2, 200, 128, 2, seed=4, bias_std=0.3)
     module = _module_from_case(case, 2, "hip")
     x = case["x"].cuda()
     with torch.no_grad():
@@ -114,7 +114,7 @@ def test_chunked_calls_with_carried_state_equal_one_call():
 
 
 def test_causality_on_the_hip_path():
-    case = orc.make_case(2, 100, 64, 2, seed=5)
+    case = orc.make_case(2, 100, 64, 2, seed=5, bias_std=0.3)
     module = _module_from_case(case, 2, "hip")
     x = case["x"].cuda()
     changed = x.clone()
@@ -126,7 +126,7 @@ def test_causality_on_the_hip_path():
 
 
 def test_reset_isolates_documents_on_the_hip_path():
-    case = orc.make_case(2, 96, 64, 2, seed=6)
+    case = orc.make_case(2, 96, 64, 2, seed=6, bias_std=0.3)
     module = _module_from_case(case, 2, "hip")
     x = case["x"].cuda()
     reset = torch.zeros(2, 96, dtype=torch.bool, device="cuda")
@@ -262,7 +262,7 @@ def test_config4_prefill_then_512_decode_steps():
 def test_module_decode_uses_step_kernel_and_tracks_parameter_updates():
     """T == 1 without gradients goes through the single-step kernel on a cached parameter image; the
     image must follow in-place parameter updates.  Reference behaviour: griffin/griffin.py:279-284."""
-    case = orc.make_case(4, 6, 256, 2, seed=13, h0_std=0.5)
+    case = orc.make_case(4, 6, 256, 2, seed=13, h0_std=0.5, bias_std=0.3)
     ref = _module_from_case(case, 2, "sequential", device="cpu")
     hip = _module_from_case(case, 2, "hip")
     x = case["x"]
