@@ -137,12 +137,14 @@ def main():
     elapsed = time.perf_counter() - t0
     ms_per_step = elapsed * 1e3 / args.steps
 
-    # per-kernel durations, HIP events on the launch stream (library measurement hook), eager launches
+    # per-kernel durations, HIP events on the launch stream (library measurement hook), eager launches;
+    # the hook keeps the events of the latest launch of each kernel
     lib.rglru_hip_set_timing(1)
     names = {"fwd_kernel": 0, "bwd_scan_kernel": 1, "gate_grad_kernel": 3}
     samples = {k: [] for k in names}
     for _ in range(20):
-        step()
+        for _ in range(4):      # back to back: the last step's kernels run on a busy GPU, as in the timed region
+            step()
         for k, slot in names.items():
             samples[k].append(lib.rglru_hip_kernel_ms(slot))
     lib.rglru_hip_set_timing(0)
