@@ -486,7 +486,8 @@ __global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : 2)) void fwd
   const IO* wg = (const IO*)p.wg;
   const IO* w_a_row = wg + ((long long)(0 * p.nb + w.k) * p.bwp + (w.slab_ok ? w.o : 0)) * p.bwp + hf * Tr::HW;
   const IO* w_x_row = wg + ((long long)(1 * p.nb + w.k) * p.bwp + (w.slab_ok ? w.o : 0)) * p.bwp + hf * Tr::HW;
-  const float bias_a = p.bias[w.kp], bias_x = p.bias[p.Wp + w.kp];
+  // the biases enter inside the sigmoids (as -log2(e) * b), the matrix products start from zero
+  const float nba = -kLog2e * p.bias[w.kp], nbx = -kLog2e * p.bias[p.Wp + w.kp];
   const float sp = w.ch_ok ? p.sp[w.kp] : 0.f;
   const IO* x = (const IO*)p.x;
   const long long W = p.W;
@@ -548,7 +549,6 @@ __global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : 2)) void fwd
     // iteration is finished (carry in, recurrence, stores) after the gate math of the current one,
     // so the wait for the neighbours' records overlaps with useful work.
     FwdTile<MT> cur, prev;
-    const float nba = -kLog2e * bias_a, nbx = -kLog2e * bias_x;
     bool have_prev = false;
     prev.b = 0; prev.c = 0;                              // chunk 0 has no records to request
 #pragma unroll
@@ -611,7 +611,6 @@ __global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : 2)) void fwd
             }
           } else
           gate_mfma_held<IO, MT, NKG, KC>(lds, hw, mt, w.slab, w.r, hf, 0.0f, 0.0f, ua, ux, xv, NKG == 8 ? 0 : w.kb);
-          // the biases enter inside the sigmoids
           fwd_gates<IO, MASKED>(flbits[mt], ua, ux, xv, sp, cur.a + 16 * mt, cur.z + 16 * mt, nba, nbx);
         }
       }
@@ -646,7 +645,7 @@ __global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : 2)) void fwd
       f32x16 ua[MT], ux[MT];
       float xv[EL];
       gate_tile_generic<IO, MT>(p, x + (long long)b * p.T * W, (long long)c * TR, p.T, w.k, w.slab, w.slab_ok,
-                                w_a_row, w_x_row, bias_a, bias_x, lds, ua, ux, xv);
+                                w_a_row, w_x_row, 0.0f, 0.0f, lds, ua, ux, xv);
       if (w.slab_ok) {
         const long long trow = (long long)b * p.T + c * TR + hf * EL;
         FwdTile<MT> tile;
@@ -656,7 +655,7 @@ __global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : 2)) void fwd
           float xpart[16];
 #pragma unroll
           for (int e = 0; e < 16; ++e) xpart[e] = xv[16 * mt + e];
-          fwd_gates<IO, true>(flag_run(p, trow + 16 * mt, c * TR + hf * EL + 16 * mt), ua[mt], ux[mt], xpart, sp, tile.a + 16 * mt, tile.z + 16 * mt);
+          fwd_gates<IO, true>(flag_run(p, trow + 16 * mt, c * TR + hf * EL + 16 * mt), ua[mt], ux[mt], xpart, sp, tile.a + 16 * mt, tile.z + 16 * mt, nba, nbx);
         }
         fwd_local<MT, true>(p, w, tile);
         // 16-bit outputs go through the wave's staging area when whole 64-byte row segments can be
@@ -690,7 +689,7 @@ __global__ __launch_bounds__(kThreads) void bwd_kernel(FusedArgs p) {
   const IO* w_x_row = wg + ((long long)(1 * p.nb + w.k) * p.bwp + (w.slab_ok ? w.o : 0)) * p.bwp + hf * Tr::HW;
   HeldWeights<IO, NKG> hw;
   hw.load(w_a_row, w_x_row);
-  const float bias_a = p.bias[w.kp], bias_x = p.bias[p.Wp + w.kp];
+  const float nba = -kLog2e * p.bias[w.kp], nbx = -kLog2e * p.bias[p.Wp + w.kp];   // biases as the sigmoids take them
   const float sp = w.ch_ok ? p.sp[w.kp] : 0.f;
   const float cs = w.ch_ok ? p.cs[w.kp] : 0.f;
   const IO* x = (const IO*)p.x;
@@ -719,11 +718,11 @@ __global__ __launch_bounds__(kThreads) void bwd_kernel(FusedArgs p) {
         *reinterpret_cast<Frag*>(lds + row * LDSROW + cv * Tr::HW) = v;
       }
       __syncthreads();
-      if (w.slab_ok) gate_mfma_held<IO, MT, NKG>(lds, hw, 0, w.slab, w.r, hf, bias_a, bias_x, ua[0], ux[0], xv);
+      if (w.slab_ok) gate_mfma_held<IO, MT, NKG>(lds, hw, 0, w.slab, w.r, hf, 0.0f, 0.0f, ua[0], ux[0], xv);
       __syncthreads();
     } else {
       gate_tile_generic<IO, MT>(p, x + (long long)b * p.T * W, t0, p.T, w.k, w.slab, w.slab_ok, w_a_row, w_x_row,
-                                bias_a, bias_x, lds, ua, ux, xv);
+                                0.0f, 0.0f, lds, ua, ux, xv);
     }
     if (!w.slab_ok) continue;
 
@@ -735,7 +734,7 @@ __global__ __launch_bounds__(kThreads) void bwd_kernel(FusedArgs p) {
       const bool in = t0 + hf * EL + e < p.T;
       unsigned fl = token_flag(p, trow + e, in);
       flv[e] = fl;
-      GateOut go = gate_forward<Precise<IO>::value, true>(ua[0][e], ux[0][e], xv[e], sp, fl);
+      GateOut go = gate_forward<Precise<IO>::value, true>(ua[0][e], ux[0][e], xv[e], sp, fl, nba, nbx);
       r[e] = go.r; gi[e] = go.i; a[e] = go.a; g[e] = go.g; g2[e] = go.g2; z[e] = go.z;
       gy[e] = (in && w.ch_ok) ? (float)dy[(trow + e) * W + w.ch] : 0.f;
     }

@@ -305,9 +305,9 @@ class _HipRGLRU(torch.autograd.Function):
                 wx = w_x.detach().to(x.dtype)
                 dw_a = torch.bmm(ua.transpose(1, 2), xk)
                 dw_x = torch.bmm(ux.transpose(1, 2), xk)
-                dxg = torch.bmm(ua, wa)
-                dxg = torch.baddbmm(dxg, ux, wx)
-                dx = (dx.view(n, nb, bw).float() + dxg.transpose(0, 1).float()).to(x.dtype).view(B, T, W)
+                dx_blocks = dx.view(n, nb, bw).transpose(0, 1)       # [nb, n, bw], row stride W: written in place
+                torch.baddbmm(dx_blocks, ua, wa, out=dx_blocks)
+                torch.baddbmm(dx_blocks, ux, wx, out=dx_blocks)
         grads = (dx, dw_a.to(pd[0]), db_a.to(pd[1]), dw_x.to(pd[2]), db_x.to(pd[3]),
                  dlam.to(pd[4]), None if dh0 is None else dh0.to(ctx.h0_dtype), None, None)
         return grads
