@@ -673,7 +673,7 @@ __global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : 2)) void fwd
 // per-workgroup partial sums for the bias and Lambda gradients.
 // ------------------------------------------------------------------------------------------
 template <typename IO, int NKG>
-__global__ __launch_bounds__(kThreads) void bwd_kernel(FusedArgs p) {
+__global__ __launch_bounds__(kThreads, (NKG == 0 ? 2 : 1)) void bwd_kernel(FusedArgs p) {
   constexpr int MT = 1, TR = 32, EL = 16;
   typedef Io<IO> Tr;
   typedef typename Tr::Frag Frag;
@@ -727,21 +727,23 @@ __global__ __launch_bounds__(kThreads) void bwd_kernel(FusedArgs p) {
     if (!w.slab_ok) continue;
 
     const long long trow = (long long)b * p.T + t0 + hf * EL;
-    float r[EL], gi[EL], a[EL], g[EL], g2[EL], z[EL], gy[EL];
-    unsigned flv[EL];
+    // kept per local step: both gates, the decay, the input scale and dy; z = g i x is recomputed
+    // where it is needed (two workgroups per compute unit need the registers)
+    float r[EL], gi[EL], a[EL], g[EL], gy[EL];
+    unsigned flbits = 0u;                                // two flag bits per local step
 #pragma unroll
     for (int e = 0; e < EL; ++e) {
       const bool in = t0 + hf * EL + e < p.T;
-      unsigned fl = token_flag(p, trow + e, in);
-      flv[e] = fl;
+      const unsigned fl = token_flag(p, trow + e, in);
+      flbits |= fl << (2 * e);
       GateOut go = gate_forward<Precise<IO>::value, true>(ua[0][e], ux[0][e], xv[e], sp, fl, nba, nbx);
-      r[e] = go.r; gi[e] = go.i; a[e] = go.a; g[e] = go.g; g2[e] = go.g2; z[e] = go.z;
+      r[e] = go.r; gi[e] = go.i; a[e] = go.a; g[e] = go.g;
       gy[e] = (in && w.ch_ok) ? (float)dy[(trow + e) * W + w.ch] : 0.f;
     }
     // forward recomputation of h_{t-1} from the chunk checkpoint
     float A = 1.f, H = 0.f;
 #pragma unroll
-    for (int e = 0; e < EL; ++e) { H = fmaf(a[e], H, z[e]); A *= a[e]; }
+    for (int e = 0; e < EL; ++e) { H = fmaf(a[e], H, g[e] * gi[e] * xv[e]); A *= a[e]; }
     const float A_o = xhalf(A, hf), H_o = xhalf(H, hf);
     const float A_lo = hf ? A_o : A, H_lo = hf ? H_o : H;
     const float A_hi = hf ? A : A_o;
@@ -753,7 +755,7 @@ __global__ __launch_bounds__(kThreads) void bwd_kernel(FusedArgs p) {
     float h = hf ? fmaf(A_lo, h_start, H_lo) : h_start;
     float hp[EL];
 #pragma unroll
-    for (int e = 0; e < EL; ++e) { hp[e] = h; h = fmaf(a[e], h, z[e]); }
+    for (int e = 0; e < EL; ++e) { hp[e] = h; h = fmaf(a[e], h, g[e] * gi[e] * xv[e]); }
 
     // reverse affine map of this lane's run and of the chunk
     float carry = 0.f;
@@ -783,7 +785,7 @@ __global__ __launch_bounds__(kThreads) void bwd_kernel(FusedArgs p) {
     for (int e = EL - 1; e >= 0; --e) {
       const float d = gy[e] + carry;
       carry = a[e] * d;
-      const unsigned fl = flv[e];
+      const unsigned fl = (flbits >> (2 * e)) & 3u;
       const bool rst = fl & 1u, ina = fl & 2u;
       const float xe = xv[e];
       // z = g * i * x
@@ -791,7 +793,7 @@ __global__ __launch_bounds__(kThreads) void bwd_kernel(FusedArgs p) {
       float di = d * g[e] * xe;
       float dxd = d * g[e] * gi[e];
       // g = sqrt(g2) with the bounded derivative; a = exp(l), g2 = 1 - exp(2l)
-      float dg2 = dg * __builtin_amdgcn_rsqf(fmaxf(4.0f * g2[e], 1e-6f));
+      float dg2 = dg * __builtin_amdgcn_rsqf(fmaxf(4.0f * (g[e] * g[e]), 1e-6f));
       float dl = fmaf(d * hp[e], a[e], -2.0f * (a[e] * a[e]) * dg2);
       if (rst) dl = 0.f;
       float dr = dl * cs;
