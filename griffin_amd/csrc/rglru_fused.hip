@@ -30,6 +30,7 @@ struct PrepArgs {
   const void* w_a; const void* w_x; const void* b_a; const void* b_x; const void* lambda;
   void* wg; float* bias; float* sp; float* cs; float* dsp; void* w2t;
   int W, nb, bw, bwp, Wp, vec_dtype;
+  int vec_ok;                          // 16-bit weights, unpadded blocks, 16-byte aligned: eight elements per thread
   float c;
   uint4* clear; long long clear_n;     // optional: a workspace region to zero in the same launch
 };
@@ -46,6 +47,23 @@ RGLRU_DEVICE float log_sigmoid(float v) {
   return v >= 0.f ? -log1pf(expf(-v)) : v - log1pf(expf(v));
 }
 
+// Per-channel constants of padded channel kp: the two biases, c log sigmoid(Lambda) in natural and
+// binary logarithm, and the factor of the Lambda gradient.
+RGLRU_DEVICE void prepare_channel(const PrepArgs& p, int kp) {
+  const int k = kp / p.bwp, o = kp - k * p.bwp;
+  float ba = 0.f, bx = 0.f, sp = 0.f, cs = 0.f, dsp = 0.f;
+  if (o < p.bw) {
+    const int ch = k * p.bw + o;
+    ba = load_vec(p.b_a, ch, p.vec_dtype); bx = load_vec(p.b_x, ch, p.vec_dtype);
+    const float lam = load_vec(p.lambda, ch, p.vec_dtype);
+    const float ls = log_sigmoid(lam);
+    cs = p.c * ls;
+    sp = cs * kLog2e;
+    dsp = p.c / (1.0f + expf(lam));          // c * d/dLambda log sigmoid(Lambda) = c * sigmoid(-Lambda)
+  }
+  p.bias[kp] = ba; p.bias[p.Wp + kp] = bx; p.sp[kp] = sp; p.cs[kp] = cs; p.dsp[kp] = dsp;
+}
+
 template <typename IO>
 __global__ void prepare_kernel(PrepArgs p) {
   const long long per_gate = (long long)p.nb * p.bwp * p.bwp;
@@ -54,6 +72,33 @@ __global__ void prepare_kernel(PrepArgs p) {
   long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x;
   const long long stride = (long long)gridDim.x * blockDim.x;
   for (long long z = i; z < p.clear_n; z += stride) p.clear[z] = make_uint4(0u, 0u, 0u, 0u);
+  if (sizeof(IO) == 2 && p.vec_ok) {
+    // 16 bytes per thread: wg is a copy of [w_a ; w_x]; a vector of w2t is four output channels x two gates
+    const long long per_gate8 = per_gate / 8, n_w8 = 2 * per_gate8;
+    const int row8 = 2 * p.bw / 8;                         // vectors per row j of w2t
+    const long long per_block8 = (long long)p.bw * row8;
+    const unsigned short* wa = (const unsigned short*)p.w_a;
+    const unsigned short* wx = (const unsigned short*)p.w_x;
+    for (; i < 2 * n_w8 + p.Wp; i += stride) {
+      if (i < n_w8) {
+        const int gate = i >= per_gate8;
+        ((uint4*)p.wg)[i] = ((const uint4*)(gate ? p.w_x : p.w_a))[i - gate * per_gate8];
+      } else if (i < 2 * n_w8) {
+        const long long e8 = i - n_w8;
+        const int k = (int)(e8 / per_block8);
+        const int rem = (int)(e8 - (long long)k * per_block8);
+        const int j = rem / row8, c8 = rem - j * row8;
+        const long long at = ((long long)k * p.bw + 4 * c8) * p.bw + j;   // W[k][4 c8][j]
+        unsigned v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = (unsigned)wa[at + (long long)u * p.bw] | ((unsigned)wx[at + (long long)u * p.bw] << 16);
+        ((uint4*)p.w2t)[e8] = make_uint4(v[0], v[1], v[2], v[3]);
+      } else {
+        prepare_channel(p, (int)(i - 2 * n_w8));
+      }
+    }
+    return;
+  }
   for (; i < total; i += stride) {
     if (i < n_w) {
       int gate = (int)(i / per_gate);
@@ -82,19 +127,7 @@ __global__ void prepare_kernel(PrepArgs p) {
       }
       ((IO*)p.w2t)[e] = (IO)v;
     } else {
-      int kp = (int)(i - n_w);
-      int k = kp / p.bwp, o = kp - k * p.bwp;
-      float ba = 0.f, bx = 0.f, sp = 0.f, cs = 0.f, dsp = 0.f;
-      if (o < p.bw) {
-        int ch = k * p.bw + o;
-        ba = load_vec(p.b_a, ch, p.vec_dtype); bx = load_vec(p.b_x, ch, p.vec_dtype);
-        const float lam = load_vec(p.lambda, ch, p.vec_dtype);
-        float ls = log_sigmoid(lam);
-        cs = p.c * ls;
-        sp = cs * kLog2e;
-        dsp = p.c / (1.0f + expf(lam));          // c * d/dLambda log sigmoid(Lambda) = c * sigmoid(-Lambda)
-      }
-      p.bias[kp] = ba; p.bias[p.Wp + kp] = bx; p.sp[kp] = sp; p.cs[kp] = cs; p.dsp[kp] = dsp;
+      prepare_channel(p, (int)(i - n_w));
     }
   }
 }
@@ -1634,7 +1667,9 @@ static int prepare_impl(const void* w_a, const void* b_a, const void* w_x, const
   a.w2t = pb + pl.w2t;
   a.W = (int)W; a.nb = (int)nb; a.bw = (int)g.bw; a.bwp = (int)g.bwp; a.Wp = (int)g.Wp; a.c = c;
   a.clear = (uint4*)clear; a.clear_n = (long long)(clear_bytes / 16);
-  long long total = 4 * g.nb * g.bwp * g.bwp + g.Wp;
+  a.vec_ok = dtype == RGLRU_BF16 && g.bw == g.bwp && g.bw % 8 == 0 && (uintptr_t)w_a % 16 == 0 && (uintptr_t)w_x % 16 == 0 &&
+             (uintptr_t)a.wg % 16 == 0 && (uintptr_t)a.w2t % 16 == 0;
+  long long total = a.vec_ok ? 4 * g.nb * g.bwp * g.bwp / 8 + g.Wp : 4 * g.nb * g.bwp * g.bwp + g.Wp;
   if (a.clear_n > total) total = a.clear_n;
   int blocks = (int)((total + 255) / 256); if (blocks > 2048) blocks = 2048;
   hipStream_t s = (hipStream_t)stream;
