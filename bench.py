@@ -1,11 +1,19 @@
 """Benchmark of the fused RG-LRU forward + backward on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-graph]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-graph] [--workload NAME]
 
 One step = one forward + one backward of the RG-LRU (gates + scan, recomputing backward) over one
 batch of synthetic input, B=8, T=2048, W=1024, 8 gate blocks, bf16 storage with fp32 state: the
 configuration the headline metric is quoted on.  Inputs are resident in HBM before the timed region.
 Prints ONE JSON line.
+
+--workload selects one of the other measured configurations instead (eager launches, one JSON line
+without the roofline and CPU legs; their per-kernel figures come from rocprofv3 runs of the same
+command, summarised under profiles/):
+    block         RMSNorm + RecurrentBlock(768, 1024) forward + backward at B8 T2048, bf16
+    long_context  RG-LRU forward + backward at B1 T32768 W2560, 8 blocks of 320 channels, slow decay
+    decode        512 single-token RG-LRU steps at B256 W1024 after a T2048 prefill
+    block_decode  64 single-token RecurrentBlock(768, 1024) steps at B256 after a T128 prefill
 """
 
 from __future__ import annotations
@@ -45,7 +53,87 @@ def parse_args():
     ap.add_argument("--seq", type=int, default=2048)
     ap.add_argument("--width", type=int, default=1024)
     ap.add_argument("--blocks", type=int, default=8)
+    ap.add_argument("--workload", default="rglru", choices=["rglru", "block", "long_context", "decode", "block_decode"])
     return ap.parse_args()
+
+
+def _timed(run, steps, warmup):
+    """Milliseconds per call of run(), eager launches, synchronised on both sides."""
+    for _ in range(max(warmup, 1)):
+        run()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        run()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def secondary_workload(args):
+    """The configurations next to the headline one; see the module docstring."""
+    from griffin_amd import PreparedParams, hip_rglru, hip_rglru_step
+    from griffin_amd.modules import RMSNorm, RecurrentBlock
+    from oracle import rglru_oracle as orc
+
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    torch.manual_seed(0)
+    dt = torch.bfloat16
+    name = args.workload
+    if name == "block":
+        B, T, D, W = 8, 2048, 768, 1024
+        block = RecurrentBlock(D, W, scan_mode="hip").to(dev).to(dt)
+        norm = RMSNorm(D).to(dev).to(dt)
+        x = torch.randn(B, T, D, device=dev, dtype=dt, requires_grad=True)
+        dy = torch.randn(B, T, D, device=dev, dtype=dt)
+        leaves = [x] + list(block.parameters()) + list(norm.parameters())
+        ms = _timed(lambda: torch.autograd.grad(block(norm(x)), leaves, dy), args.steps, args.warmup)
+        metric, tokens = "RMSNorm + RecurrentBlock fwd+bwd tokens/s", B * T
+        workload = f"RMSNorm + RecurrentBlock({D}, {W}) fwd+bwd B{B} T{T} bf16"
+    elif name == "long_context":
+        B, T, W, nb = 1, 32768, 2560, 8
+        case = orc.make_case(B, T, W, nb, seed=0, lo=0.99, hi=0.9999)
+        x = case["x"].to(dt).to(dev).requires_grad_(True)
+        params = [case[k].to(dt).to(dev).requires_grad_(True) for k in ("w_a", "b_a", "w_x", "b_x", "lam")]
+        dy = case["dy"].to(dt).to(dev)
+        ms = _timed(lambda: torch.autograd.grad(hip_rglru(x, *params, 8.0)[0], [x] + params, dy), args.steps, args.warmup)
+        metric, tokens = "RG-LRU fwd+bwd tokens/s", B * T
+        workload = f"RG-LRU fwd+bwd B{B} T{T} W{W} nb{nb} bf16"
+    elif name == "decode":
+        B, T, W, nb, steps = 256, 2048, 1024, 8, 512
+        case = orc.make_case(1, 1, W, nb, seed=0)
+        params = [case[k].to(dt).to(dev) for k in ("w_a", "b_a", "w_x", "b_x", "lam")]
+        with torch.no_grad():
+            _, state = hip_rglru(torch.randn(B, T, W, device=dev, dtype=dt), *params, 8.0)
+            state = state.contiguous()
+            prep = PreparedParams(*params, 8.0, dt)
+            xs = torch.randn(steps, B, W, device=dev, dtype=dt)
+
+            def run():
+                for t in range(steps):
+                    hip_rglru_step(xs[t], prep, state)
+            ms = _timed(run, max(args.steps // 10, 1), 1) / steps
+        metric, tokens = "RG-LRU decode tokens/s", B
+        workload = f"RG-LRU decode B{B} W{W} nb{nb} bf16, {steps} steps after a T{T} prefill"
+    else:
+        B, D, W, steps = 256, 768, 1024, 64
+        block = RecurrentBlock(D, W, scan_mode="hip").to(dev).to(dt).eval()
+        with torch.no_grad():
+            _, cache = block(torch.randn(B, 128, D, device=dev, dtype=dt), return_cache=True)
+            xs = torch.randn(B, 1, D, device=dev, dtype=dt)
+            holder = [cache]
+
+            def run():
+                for _ in range(steps):
+                    _, holder[0] = block(xs, cache=holder[0], return_cache=True)
+            ms = _timed(run, max(args.steps // 10, 1), 1) / steps
+        metric, tokens = "RecurrentBlock decode tokens/s", B
+        workload = f"RecurrentBlock({D}, {W}) decode B{B} bf16, {steps} steps after a T128 prefill"
+    print(json.dumps({
+        "metric": metric, "value": tokens / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic", "config": {"workload": workload, "launch": "eager"},
+    }))
 
 
 def cpu_baseline(case, budget_s=20.0):
@@ -83,6 +171,9 @@ def main():
     lib = _lib.load()
     if not torch.cuda.is_available():
         raise RuntimeError("bench.py needs a GPU")
+    if args.workload != "rglru":
+        secondary_workload(args)
+        return
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
     B, T, W, nb = args.batch, args.seq, args.width, args.blocks
