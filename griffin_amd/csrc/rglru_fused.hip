@@ -446,15 +446,18 @@ RGLRU_DEVICE void fwd_finalize(const FusedArgs& p, const WaveId& w, const FwdTil
     const unsigned uW = (unsigned)W, ch = (unsigned)w.ch;
     const bool lower = ch_ok && hf == 0;
     rec_store_buf(seq_records(p, b), lower ? ((unsigned)c * uW + ch) * 8u : kOutOfRange, 0.f, h_end);
-    const rsrc_t rck = make_rsrc(p.ckpt + (long long)b * p.ckpt_nC * W, (unsigned)p.ckpt_nC * uW * 4u);
-    unsigned ck_off = lower ? ((unsigned)(c * MT + (MT - 1)) * uW + ch) * 4u : kOutOfRange;
-    if (MT == 2 && ch_ok && hf != 0) ck_off = ((unsigned)(c * MT) * uW + ch) * 4u;
-    BufIo<float>::store(hf ? h_mid : h_end, rck, ck_off, 0u);
     const rsrc_t rhl = make_rsrc(p.h_last, p.h_last ? (unsigned)p.B * uW * 4u : 0u);
     BufIo<float>::store(h_end, rhl, (lower && c == p.nCf - 1) ? ((unsigned)b * uW + ch) * 4u : kOutOfRange, 0u);
   }
 
   float h = hf ? h_mid : h_in;
+  // checkpoints for the backward pass: the state after every 16 tokens (slot = token / 16); slots past
+  // the end of the buffer are dropped by the descriptor
+  const rsrc_t rck = make_rsrc(p.ckpt + (long long)b * p.ckpt_nC * W, (unsigned)p.ckpt_nC * (unsigned)W * 4u);
+  unsigned ck_off[MT];
+#pragma unroll
+  for (int g16 = 0; g16 < MT; ++g16)
+    ck_off[g16] = ch_ok ? ((unsigned)(c * 2 * MT + hf * MT + g16) * (unsigned)W + (unsigned)w.ch) * 4u : kOutOfRange;
   // y tile through a buffer descriptor: rows past the end of the sequence are dropped
   const int rows = !live ? 0 : ((p.T - t0) < TR ? (p.T - t0) : TR);
   const unsigned row_bytes = (unsigned)p.W * (unsigned)sizeof(IO);
@@ -466,6 +469,7 @@ RGLRU_DEVICE void fwd_finalize(const FusedArgs& p, const WaveId& w, const FwdTil
     for (int e = 0; e < EL; ++e) {
       h = fmaf(t.a[e], h, t.z[e]);
       *reinterpret_cast<IO*>(my + e * WaveStage<TR>::kRowBytes) = (IO)h;
+      if ((e & 15) == 15) BufIo<float>::store(h, rck, ck_off[e >> 4], 0u);
     }
     wave_lds_fence();
     stage_flush<TR>(stage, ry, row_bytes, (unsigned)(w.k * p.bw + w.slab * 32) * 2u, w.lane);
@@ -476,6 +480,7 @@ RGLRU_DEVICE void fwd_finalize(const FusedArgs& p, const WaveId& w, const FwdTil
     for (int e = 0; e < EL; ++e) {
       h = fmaf(t.a[e], h, t.z[e]);
       BufIo<IO>::store((IO)h, ry, voff + (unsigned)e * row_bytes, 0u);
+      if ((e & 15) == 15) BufIo<float>::store(h, rck, ck_off[e >> 4], 0u);
     }
   }
 }
@@ -773,19 +778,19 @@ __global__ __launch_bounds__(kThreads, (NKG == 0 ? 2 : 1)) void bwd_kernel(Fused
       r[e] = go.r; gi[e] = go.i; a[e] = go.a; g[e] = go.g;
       gy[e] = (in && w.ch_ok) ? (float)dy[(trow + e) * W + w.ch] : 0.f;
     }
-    // forward recomputation of h_{t-1} from the chunk checkpoint
-    float A = 1.f, H = 0.f;
+    // forward recomputation of h_{t-1} from the checkpoint in front of the lane's 16 tokens
+    float A = 1.f;
 #pragma unroll
-    for (int e = 0; e < EL; ++e) { H = fmaf(a[e], H, g[e] * gi[e] * xv[e]); A *= a[e]; }
-    const float A_o = xhalf(A, hf), H_o = xhalf(H, hf);
-    const float A_lo = hf ? A_o : A, H_lo = hf ? H_o : H;
+    for (int e = 0; e < EL; ++e) A *= a[e];
+    const float A_o = xhalf(A, hf);
+    const float A_lo = hf ? A_o : A;
     const float A_hi = hf ? A : A_o;
     float h_start = 0.f;
     if (w.ch_ok) {
-      if (c == 0) h_start = p.h0 ? p.h0[(long long)b * W + w.ch] : 0.f;
-      else h_start = p.ckpt[((long long)b * p.ckpt_nC + (c - 1)) * W + w.ch];
+      if (c == 0 && hf == 0) h_start = p.h0 ? p.h0[(long long)b * W + w.ch] : 0.f;
+      else h_start = p.ckpt[((long long)b * p.ckpt_nC + (2 * c - 1 + hf)) * W + w.ch];
     }
-    float h = hf ? fmaf(A_lo, h_start, H_lo) : h_start;
+    float h = h_start;
     float hp[EL];
 #pragma unroll
     for (int e = 0; e < EL; ++e) { hp[e] = h; h = fmaf(a[e], h, g[e] * gi[e] * xv[e]); }
@@ -981,9 +986,9 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
     // checkpoint), requested early
     unsigned flbits = 0u;
     if constexpr (MASKED) flbits = flag_run(p, trow, t0 + hf * EL);
-    float h_start = 0.f;
-    if (c == 0) { if (p.h0) h_start = p.h0[(long long)b * W + w.ch]; }
-    else h_start = p.ckpt[((long long)b * p.ckpt_nC + (c - 1)) * W + w.ch];
+    float h_start = 0.f;                                 // state in front of this lane's 16 tokens
+    if (c == 0 && hf == 0) { if (p.h0) h_start = p.h0[(long long)b * W + w.ch]; }
+    else h_start = p.ckpt[((long long)b * p.ckpt_nC + (2 * c - 1 + hf)) * W + w.ch];
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int idx = tid + i * kThreads;
@@ -1078,20 +1083,15 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
     if (!last_chunk && hf == 0) carry_publish(chain, c, A_t, D_t, false);
     RGLRU_STAMP(p, 4);
 
-    // input gate, g = sqrt(1 - a^2) and the forward map of the lane's run (for h at the run's start)
-    float H = 0.f;
+    // input gate and g = sqrt(1 - a^2)
 #pragma unroll
     for (int e = 0; e < EL; ++e) {
       const float ie = sigmoid_fast(ux[e], nbx);
       float l2 = r[e] * sp;
       if constexpr (MASKED) l2 = masked_log2_decay_run(l2, flbits, e);     // gives g = 1 / g = 0
       const float ge = __builtin_amdgcn_sqrtf(fmaxf(one_minus_exp<false>(l2 * (2.0f * kLn2), a[e]), 0.0f));
-      const float ze = ge * ie * xv[e];
       gi[e] = ie; g[e] = ge;
-      H = fmaf(a[e], H, ze);
     }
-    const float H_o = xhalf(H, hf);
-    const float H_lo = hf ? H_o : H;
     issue(tk_next);
     RGLRU_STAMP(p, 5);
     float d_in = (last_chunk && p.dh_last) ? p.dh_last[(long long)b * W + w.ch] : 0.f;
@@ -1105,7 +1105,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
     carry = hf ? d_in : fmaf(A_hi, d_in, D_hi);
 #pragma unroll
     for (int e = EL - 1; e >= 0; --e) { const float d = gy[e] + carry; gy[e] = d; carry = a[e] * d; }
-    float h = hf ? fmaf(A_lo, h_start, H_lo) : h_start;
+    float h = h_start;                                   // the forward pass left a checkpoint every 16 tokens
     unsigned char* my_dx = stage_dx + WaveStage<TR>::row_offset(hf * EL) + w.r * 2;
     unsigned char* my_du = GIVEN ? stage_du + WaveStage<TR>::row_offset(hf * EL) + w.r * 2
                                  : stage_du + PairStage<TR>::row_offset(hf * EL) + w.r * 4;
@@ -1718,7 +1718,7 @@ static int fwd_impl(const void* x, const void* prep, const float* h0, const uint
   a.flags_vec = (T % 16 == 0) && ((uintptr_t)flags % 16 == 0);
   a.ckpt = (float*)(wb + L.ckpt); a.rec_a = (rec_t*)(wb + L.f_rec_a);
   a.ticket = (unsigned*)(wb + L.f_ticket); a.fail = (unsigned*)(wb + L.fail);
-  a.B = (int)B; a.T = (int)T; a.nC = (int)L.nC; a.ckpt_nC = (int)L.nC;
+  a.B = (int)B; a.T = (int)T; a.nC = (int)L.nC; a.ckpt_nC = 2 * (int)L.nC;
   a.nCf = (int)((T + 32 * kFwdMT - 1) / (32 * kFwdMT));
   a.aligned = is_aligned(x, W, g.bw, elem_size(dtype)) && ((uintptr_t)y % 16 == 0);
 #ifdef RGLRU_TRACE
@@ -1794,7 +1794,7 @@ int rglru_hip_bwd_pre(const void* x, const void* pre, const void* prep, const fl
   a.ckpt = (float*)(wb + L.ckpt); a.rec_a = (rec_t*)(wb + L.b_rec_a);
   a.ticket = (unsigned*)(wb + L.b_ticket); a.fail = (unsigned*)(wb + L.fail);
   a.partial = (float*)((char*)scratch + make_scratch_layout(B, T, g, false).partial);
-  a.B = (int)B; a.T = (int)T; a.nC = (int)((T + kChunk - 1) / kChunk); a.ckpt_nC = (int)L.nC;
+  a.B = (int)B; a.T = (int)T; a.nC = (int)((T + kChunk - 1) / kChunk); a.ckpt_nC = 2 * (int)L.nC;
   a.aligned = 1;
   a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nC, 2, L.max_wg);
   a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
@@ -1864,7 +1864,7 @@ int rglru_hip_bwd(const void* x, const void* prep, const float* h0,
   a.ckpt = (float*)(wb + L.ckpt); a.rec_a = (rec_t*)(wb + L.b_rec_a);
   a.ticket = (unsigned*)(wb + L.b_ticket); a.fail = (unsigned*)(wb + L.fail);
   a.partial = (float*)((char*)scratch + make_scratch_layout(B, T, g, false).partial);
-  a.B = (int)B; a.T = (int)T; a.nC = (int)((T + kChunk - 1) / kChunk); a.ckpt_nC = (int)L.nC; a.nCf = (int)L.nCf;
+  a.B = (int)B; a.T = (int)T; a.nC = (int)((T + kChunk - 1) / kChunk); a.ckpt_nC = 2 * (int)L.nC; a.nCf = (int)L.nCf;
   a.aligned = is_aligned(x, W, g.bw, elem_size(dtype));
   a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nC, 2, L.max_wg);
   a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
@@ -1923,7 +1923,7 @@ int rglru_hip_bwd_full(const void* x, const void* prep, const float* h0,
   a.ckpt = (float*)(wb + L.ckpt); a.rec_a = (rec_t*)(wb + L.b_rec_a);
   a.ticket = (unsigned*)(wb + L.b_ticket); a.fail = (unsigned*)(wb + L.fail);
   a.partial = (float*)(sb + SL.partial); a.dw_partial = (float*)(sb + SL.dw_partial);
-  a.B = (int)B; a.T = (int)T; a.nC = (int)((T + kChunk - 1) / kChunk); a.ckpt_nC = (int)L.nC;
+  a.B = (int)B; a.T = (int)T; a.nC = (int)((T + kChunk - 1) / kChunk); a.ckpt_nC = 2 * (int)L.nC;
   a.aligned = 1;
 #ifdef RGLRU_TRACE
   a.trace = g_trace;

@@ -54,7 +54,8 @@ inline PrepLayout make_prep_layout(const Geometry& g, size_t elem) {
 // Workspace of one forward/backward pair: what has to survive from forward to backward, plus the
 // carry records of both passes.  nC = chunks of 32 tokens (rounded up to even), nCf = forward tiles
 // of 64 tokens.
-//   ckpt        [B][nC][W]      fp32 state after each chunk (kept for backward)
+//   ckpt        [B][2 nC][W]    fp32 state after every 16 tokens (kept for backward: each lane of the
+//                               backward scan owns 16 consecutive tokens and starts from one of these)
 //   --- [f_begin, b_end) is cleared at the start of the forward pass ---
 //   f_rec_a     [B][<=nC][W]    64-bit carry records of the forward chain
 //   f_ticket    [units][kMaxQueues]
@@ -79,7 +80,7 @@ inline WorkLayout make_work_layout(int64_t B, int64_t T, const Geometry& g) {
   w.max_wg = 256;                      // most workgroups one unit may use in backward
   size_t off = 0;
   auto take = [&](int64_t bytes) { size_t at = off; off += (size_t)round_up(bytes, 256); return at; };
-  w.ckpt = take(B * w.nC * g.W * 4);
+  w.ckpt = take(B * 2 * w.nC * g.W * 4);
   w.f_begin = off;
   w.f_rec_a = take(B * w.nC * g.W * 8);
   w.f_ticket = take(g.units * kMaxQueues * 4);
