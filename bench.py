@@ -36,7 +36,7 @@ HBM_PEAK_GBS = 8000.0
 # runs of this script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same
 # counter reads for the 64 MiB copy that --traffic-probe adds (profiles/ holds the summaries).  Only
 # valid for that workload; other shapes report null.
-MEASURED_TRAFFIC_BYTES = {"bwd_scan_kernel": 186776975, "fwd_kernel": 79358381, "gate_grad_kernel": 201923077}
+MEASURED_TRAFFIC_BYTES = {"bwd_scan_kernel": 189019817, "fwd_kernel": 81510566, "gate_grad_kernel": 201920628}
 BENCH_SHAPE = (8, 2048, 1024, 8)
 
 
