@@ -17,7 +17,7 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
-constexpr int kChunk = 32;          // tokens per checkpoint chunk (RGLRU_CHUNK)
+constexpr int kChunk = 32;          // tokens per backward chunk (RGLRU_CHUNK); checkpoints every kChunk / 2
 constexpr int kWaves = 4;           // waves per workgroup in the fused kernels
 constexpr int kThreads = 64 * kWaves;
 constexpr float kLog2e = 1.4426950408889634f;

@@ -60,8 +60,9 @@ enum {
 #define RGLRU_FLAG_RESET 1u
 #define RGLRU_FLAG_INACTIVE 2u
 
-/* Time steps per checkpoint: forward stores the fp32 state after every RGLRU_CHUNK tokens and
- * backward restarts its recomputation from those. */
+/* Tokens per chunk of the backward scan (one carry record per sequence, chunk and channel).  Forward
+ * stores the fp32 state after every RGLRU_CHUNK / 2 tokens and backward restarts its recomputation
+ * from those checkpoints. */
 #define RGLRU_CHUNK 32
 
 int rglru_hip_abi_version(void);
