@@ -276,7 +276,11 @@ def main():
                     "fwd_GBps": algo["fwd_kernel"] / (avg_ms["fwd_kernel"] * 1e-3) / 1e9,
                     "bwd_GBps": algo["bwd_scan_kernel"] / ((avg_ms["bwd_scan_kernel"] + avg_ms["gate_grad_kernel"]) * 1e-3) / 1e9,
                     "fwd_bwd_GBps_whole_step": step_gbps,
-                    "fwd_bwd_frac_of_peak_whole_step": step_gbps / HBM_PEAK_GBS},
+                    "fwd_bwd_frac_of_peak_whole_step": step_gbps / HBM_PEAK_GBS,
+                    # block-diagonal gate projections on MFMA: 4 W bw flops per token forward (and again
+                    # in the backward scan's recomputation), twice that in the gradient GEMM kernel
+                    "gate_gemm_TFLOPs_fwd": 4.0 * W * (W // nb) * B * T / (avg_ms["fwd_kernel"] * 1e-3) / 1e12,
+                    "gate_gemm_TFLOPs_gate_grad": 8.0 * W * (W // nb) * B * T / (avg_ms["gate_grad_kernel"] * 1e-3) / 1e12},
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(case)
