@@ -1489,6 +1489,19 @@ __global__ __launch_bounds__(kThreads) void step_kernel(FusedArgs p) {
   const long long W = p.W;
   const long long row0 = (long long)w.wg_in_unit * TR;
 
+  // the lane's previous states, gate values and flags: requested first, they arrive while the
+  // projections are computed (the step is a chain of latencies, not of bytes)
+  float h_old[EL], gate[EL];
+  unsigned fls[EL];
+#pragma unroll
+  for (int e = 0; e < EL; ++e) {
+    const long long row = row0 + hf * EL + e;
+    const bool ok = w.ch_ok && row < p.B;
+    const long long at = ok ? row * W + w.ch : 0;
+    h_old[e] = ok ? p.h_prev[at] : 0.f;
+    gate[e] = (ok && p.gate_v) ? (float)((const IO*)p.gate_v)[at] : 0.f;
+    fls[e] = (ok && p.flags) ? (unsigned)p.flags[row] : 0u;
+  }
   f32x16 ua[MT], ux[MT];
   float xv[EL];
   if constexpr (NKG > 0) {
@@ -1512,12 +1525,11 @@ __global__ __launch_bounds__(kThreads) void step_kernel(FusedArgs p) {
   for (int e = 0; e < EL; ++e) {
     const long long row = row0 + hf * EL + e;
     if (row >= p.B) break;
-    unsigned fl = p.flags ? (unsigned)p.flags[row] : 0u;
-    GateOut go = gate_forward<Precise<IO>::value, true>(ua[0][e], ux[0][e], xv[e], sp, fl);
+    GateOut go = gate_forward<Precise<IO>::value, true>(ua[0][e], ux[0][e], xv[e], sp, fls[e]);
     const long long at = row * W + w.ch;
-    float h = fmaf(go.a, p.h_prev[at], go.z);
+    float h = fmaf(go.a, h_old[e], go.z);
     p.h_state[at] = h;
-    if (p.gate_v) h *= gelu_tanh_parts((float)((const IO*)p.gate_v)[at]).gelu;
+    if (p.gate_v) h *= gelu_tanh_parts(gate[e]).gelu;
     y[at] = (IO)h;
   }
 }
