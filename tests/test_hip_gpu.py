@@ -145,6 +145,56 @@ def test_fused_bf16_matches_fp32_oracle(cfg):
         assert err < BF16_TOL, (name, err)
 
 
+def _random_case(rng, index, seed):
+    """One random configuration: storage type, block width and count, batch, length, masks, state."""
+    dtype = rng.choice([torch.bfloat16, torch.bfloat16, torch.float32])
+    bw = rng.choice([8, 16, 24, 32, 32, 48, 64, 64, 96, 128, 128, 160, 320])
+    nb = rng.choice([1, 2, 3, 4, 5, 8, 16])
+    if bw * nb > 2048:
+        nb = max(1, 2048 // bw)
+    W = bw * nb
+    B = rng.choice([1, 2, 3, 5, 9])
+    T = rng.choice([1, 2, 7, 16, 31, 32, 33, 48, 64, 65, 100, 127, 128, 129, 200, 257, 400])
+    if B * T * W > 600000:
+        T = max(1, 600000 // (B * W))
+    masks = rng.random() < 0.6
+    with_h0 = rng.random() < 0.5
+    case = orc.make_case(B, T, W, nb, seed=index + 100 * seed, h0_std=0.5 if with_h0 else 0.0,
+                         bias_std=0.5 if rng.random() < 0.7 else 0.0)
+    reset = active = None
+    if masks:
+        gen = torch.Generator().manual_seed(index)
+        reset = torch.rand(B, T, generator=gen) < 0.1
+        active = torch.rand(B, T, generator=gen) > 0.1
+        if rng.random() < 0.5:
+            active = None
+    dh_last = torch.randn(B, W, generator=torch.Generator().manual_seed(6)) if rng.random() < 0.5 else None
+    return dtype, (B, T, W, nb), case, reset, active, dh_last
+
+
+def test_random_shapes_match_oracle():
+    """Sixty random configurations (fixed seed) across every kernel family: portable, register-held
+    weights, packed narrow blocks, library-GEMM wide blocks; ragged lengths, random resets and
+    padding, initial state and a gradient at the final state."""
+    import random
+
+    seed = 3
+    rng = random.Random(seed)
+    failures = []
+    for index in range(60):
+        dtype, shape, case, reset, active, dh_last = _random_case(rng, index, seed)
+        _say("random case", index, str(dtype), shape, "masks" if reset is not None else "plain")
+        y, h_last, grads = hip_run(case, dtype, reset, active, dh_last)
+        ry, rh, rgrads = oracle_run(case, dtype, reset, active, dh_last)
+        errs = {"y": rel_err(y.float(), ry), "h_last": rel_err(h_last, rh)}
+        for name in grads:
+            errs[name] = rel_err(grads[name].float(), rgrads[name])
+        tol = FP32_TOL if dtype == torch.float32 else BF16_TOL
+        if not max(errs.values()) < tol:
+            failures.append((index, shape, {k: "%.2e" % v for k, v in errs.items()}))
+    assert not failures, failures
+
+
 @pytest.mark.parametrize("dtype,shape", [(torch.bfloat16, (2, 200, 256, 2)), (torch.float32, (2, 70, 48, 3))])
 def test_backward_twice_over_one_forward(dtype, shape):
     """A second backward pass over the same forward (retain_graph) reuses the workspace of the first
