@@ -339,9 +339,12 @@ __global__ __launch_bounds__(256) void conv_finish_kernel(ConvFinishArgs p) {
   const long long stride = (long long)(p.K + 1) * p.W;
   float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
   int n = 0;
-  for (; n + 4 <= p.slots; n += 4) {
-    s0 += src[(long long)n * stride]; s1 += src[(long long)(n + 1) * stride];
-    s2 += src[(long long)(n + 2) * stride]; s3 += src[(long long)(n + 3) * stride];
+  for (; n + 16 <= p.slots; n += 16) {                   // sixteen loads in flight: latency, not bytes, is what this kernel waits for
+    float v[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) v[u] = src[(long long)(n + u) * stride];
+#pragma unroll
+    for (int u = 0; u < 16; u += 4) { s0 += v[u]; s1 += v[u + 1]; s2 += v[u + 2]; s3 += v[u + 3]; }
   }
   for (; n < p.slots; ++n) s0 += src[(long long)n * stride];
   const float s = (s0 + s1) + (s2 + s3);
@@ -789,10 +792,14 @@ __global__ __launch_bounds__(256) void rmsnorm_finish_kernel(NormFinishArgs p) {
   const int c = blockIdx.x * 32 + col;
   float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
   if (c < p.D) {
+    // sixteen loads in flight per thread: the kernel is a chain of memory round trips, not of bytes
     int n = share;
-    for (; n + 24 < p.slots; n += 32) {
-      s0 += p.partial[(long long)n * p.D + c]; s1 += p.partial[(long long)(n + 8) * p.D + c];
-      s2 += p.partial[(long long)(n + 16) * p.D + c]; s3 += p.partial[(long long)(n + 24) * p.D + c];
+    for (; n + 120 < p.slots; n += 128) {
+      float v[16];
+#pragma unroll
+      for (int u = 0; u < 16; ++u) v[u] = p.partial[(long long)(n + 8 * u) * p.D + c];
+#pragma unroll
+      for (int u = 0; u < 16; u += 4) { s0 += v[u]; s1 += v[u + 1]; s2 += v[u + 2]; s3 += v[u + 3]; }
     }
     for (; n < p.slots; n += 8) s0 += p.partial[(long long)n * p.D + c];
   }
