@@ -83,6 +83,59 @@ RGLRU_DEVICE float conv_param(const void* base, long long i, int vec_dtype) {
   return vec_dtype == RGLRU_BF16 ? (float)((const __bf16*)base)[i] : ((const float*)base)[i];
 }
 
+// N consecutive parameters starting at element `first`, as fp32.  With 16-byte alignment (of the
+// pointer, of the first element and of the length) they come as 16-byte loads: element-wise loads
+// of a lane's 8 channels x 4 taps touch 32 cache lines per instruction and wave.
+template <int N>
+RGLRU_DEVICE void conv_params(const void* base, long long first, int vec_dtype, float (&out)[N]) {
+  const int es = vec_dtype == RGLRU_BF16 ? 2 : 4;
+  if ((N * es) % 16 == 0 && (first * es) % 16 == 0 && (uintptr_t)base % 16 == 0) {
+    const uint4* src = reinterpret_cast<const uint4*>((const char*)base + first * es);
+    if (vec_dtype == RGLRU_BF16) {
+#pragma unroll
+      for (int q = 0; q < (N * 2 + 15) / 16; ++q) {
+        const uint4 v = src[q];
+        const unsigned w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (8 * q + 2 * i < N) out[8 * q + 2 * i] = __uint_as_float(w[i] << 16);
+          if (8 * q + 2 * i + 1 < N) out[8 * q + 2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int q = 0; q < (N * 4 + 15) / 16; ++q) {
+        const uint4 v = src[q];
+        const unsigned w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (4 * q + i < N) out[4 * q + i] = __uint_as_float(w[i]);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < N; ++i) out[i] = conv_param(base, first + i, vec_dtype);
+  }
+}
+
+// Taps [channel][K] and biases of the V channels that start at c0: tap[j][v], bias[v] (zero without a bias).
+template <int V, int K>
+RGLRU_DEVICE void conv_load_taps(const void* taps, const void* bias_ptr, int c0, int vec_dtype,
+                                 float (&tap)[K][V], float (&bias)[V]) {
+  float flat[V * K];
+  conv_params<V * K>(taps, (long long)c0 * K, vec_dtype, flat);
+#pragma unroll
+  for (int v = 0; v < V; ++v)
+#pragma unroll
+    for (int j = 0; j < K; ++j) tap[j][v] = flat[v * K + j];
+  if (bias_ptr) {
+    conv_params<V>(bias_ptr, c0, vec_dtype, bias);
+  } else {
+#pragma unroll
+    for (int v = 0; v < V; ++v) bias[v] = 0.f;
+  }
+}
+
 // Which (sequence, run, channel vector) a thread owns; vectors vary fastest, so the lanes of a wave
 // read consecutive addresses of one row.
 struct ConvItem { int b, run, c0; bool ok; };
@@ -119,12 +172,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_fwd_kernel(ConvArgs p) {
   const int b = it.b, c0 = it.c0, t0 = it.run * kConvRunFwd;
   const unsigned es = (unsigned)sizeof(IO), uW = (unsigned)p.W;
   float tap[K][V], bias[V];
-#pragma unroll
-  for (int v = 0; v < V; ++v) {
-    bias[v] = p.bias ? conv_param(p.bias, c0 + v, p.vec_dtype) : 0.f;
-#pragma unroll
-    for (int j = 0; j < K; ++j) tap[j][v] = conv_param(p.taps, (long long)(c0 + v) * K + j, p.vec_dtype);
-  }
+  conv_load_taps<V, K>(p.taps, p.bias, c0, p.vec_dtype, tap, bias);
   const unsigned seq_bytes = (unsigned)p.T * uW * es;
   const rsrc_t ru = make_rsrc((const IO*)p.u + (long long)b * p.T * p.W, seq_bytes);
   const rsrc_t ro = make_rsrc((const IO*)p.out + (long long)b * p.T * p.W, seq_bytes);
@@ -198,11 +246,8 @@ __global__ __launch_bounds__(kConvThreads) void conv_bwd_kernel(ConvArgs p) {
   const bool ok = vec < p.nvec && run < p.runs;
   const int c0 = (vec < p.nvec ? vec : 0) * V, t0 = run * kConvRunBwd;
   const unsigned es = (unsigned)sizeof(IO), uW = (unsigned)p.W;
-  float tap[K][V];
-#pragma unroll
-  for (int v = 0; v < V; ++v)
-#pragma unroll
-    for (int j = 0; j < K; ++j) tap[j][v] = conv_param(p.taps, (long long)(c0 + v) * K + j, p.vec_dtype);
+  float tap[K][V], bias_unused[V];
+  conv_load_taps<V, K>(p.taps, nullptr, c0, p.vec_dtype, tap, bias_unused);
   // a thread without work sees empty tensors: its loads return zero and its stores are dropped
   const unsigned seq_bytes = ok ? (unsigned)p.T * uW * es : 0u;
   const rsrc_t ru = make_rsrc((const IO*)p.u + (long long)b * p.T * p.W, seq_bytes);
@@ -492,18 +537,17 @@ __global__ __launch_bounds__(kConvThreads) void conv_padded_fwd_kernel(PaddedArg
     for (int v = 0; v < V; ++v) acc[v] = 0.f;
   } else {
     const int doc_start = start[t];
-    float cur[V];
+    float cur[V], tap[K][V], bias[V];
     ConvRow<IO, V>::load(cur, ru, off);
+    conv_load_taps<V, K>(p.taps, p.bias, c0, p.vec_dtype, tap, bias);
 #pragma unroll
-    for (int v = 0; v < V; ++v)
-      acc[v] = fmaf(cur[v], conv_param(p.taps, (long long)(c0 + v) * K + (K - 1), p.vec_dtype),
-                    p.bias ? conv_param(p.bias, c0 + v, p.vec_dtype) : 0.f);
+    for (int v = 0; v < V; ++v) acc[v] = fmaf(cur[v], tap[K - 1][v], bias[v]);
 #pragma unroll
     for (int lag = 1; lag < K; ++lag) {
       float row[V];
       padded_source<IO, V, K>(p, ru, rs, list, i, lag, doc_start, c0, row);
 #pragma unroll
-      for (int v = 0; v < V; ++v) acc[v] = fmaf(row[v], conv_param(p.taps, (long long)(c0 + v) * K + (K - 1 - lag), p.vec_dtype), acc[v]);
+      for (int v = 0; v < V; ++v) acc[v] = fmaf(row[v], tap[K - 1 - lag][v], acc[v]);
     }
   }
   ConvRow<IO, V>::store(acc, ro, off);
@@ -557,13 +601,15 @@ __global__ __launch_bounds__(kConvThreads) void decode_prepare_kernel(DecodeArgs
 #pragma unroll
       for (int v = 0; v < V; ++v) hist[j][v] = 0.f;
   }
+  float tap[K][V], bias[V];
+  conv_load_taps<V, K>(p.taps, p.bias, c0, p.vec_dtype, tap, bias);
 #pragma unroll
   for (int v = 0; v < V; ++v) {
-    float a = p.bias ? conv_param(p.bias, c0 + v, p.vec_dtype) : 0.f;
-    if (padded || pos >= 0) a = fmaf(cur[v], conv_param(p.taps, (long long)(c0 + v) * K + (K - 1), p.vec_dtype), a);
+    float a = bias[v];
+    if (padded || pos >= 0) a = fmaf(cur[v], tap[K - 1][v], a);
 #pragma unroll
     for (int lag = 1; lag < K; ++lag)
-      if (padded || pos >= lag) a = fmaf(hist[K - 1 - lag][v], conv_param(p.taps, (long long)(c0 + v) * K + (K - 1 - lag), p.vec_dtype), a);
+      if (padded || pos >= lag) a = fmaf(hist[K - 1 - lag][v], tap[K - 1 - lag][v], a);
     acc[v] = live ? a : 0.f;
   }
   Row::store(acc, rx, off);
@@ -703,13 +749,16 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(NormArgs p) {
   const unsigned row_bytes = (unsigned)p.D * (unsigned)sizeof(IO);
   float w[kNormSlots][V], dg[kNormSlots][V];
 #pragma unroll
-  for (int s = 0; s < kNormSlots; ++s)
+  for (int s = 0; s < kNormSlots; ++s) {
+    const bool has = lane + 64 * s < p.nvec;
+    float g[V];
+    conv_params<V>(p.g, has ? (long long)(lane + 64 * s) * V : 0, p.vec_dtype, g);
 #pragma unroll
     for (int v = 0; v < V; ++v) {
-      const int c = (lane + 64 * s) * V + v;
-      w[s][v] = (lane + 64 * s < p.nvec) ? 1.0f + conv_param(p.g, c, p.vec_dtype) : 0.f;
+      w[s][v] = has ? 1.0f + g[v] : 0.f;
       dg[s][v] = 0.f;
     }
+  }
   const float inv_d = 1.0f / (float)p.D;
   for (long long row = wave; row < p.rows; row += n_waves) {
     const rsrc_t rx = make_rsrc((const IO*)p.x + row * p.D, row_bytes);
