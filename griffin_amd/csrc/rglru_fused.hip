@@ -502,8 +502,12 @@ constexpr bool kFwdDefer = false;
 
 // workgroups per compute unit of the forward kernel without weights in registers (NKG < 0); 4 spills
 #define RGLRU_GIVEN_OCC 3
+// ... and with the weights of 64- or 32-wide blocks (NKG = 4, 2): 150-168 registers, three fit
+#ifndef RGLRU_NARROW_OCC
+#define RGLRU_NARROW_OCC 3
+#endif
 template <typename IO, int NKG, bool MASKED>
-__global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : 2)) void fwd_kernel(FusedArgs p) {
+__global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : (NKG == 4 || NKG == 2) ? RGLRU_NARROW_OCC : 2)) void fwd_kernel(FusedArgs p) {
   constexpr int MT = kFwdMT, TR = 32 * MT, EL = 16 * MT;
   typedef Io<IO> Tr;
   typedef typename Tr::Frag Frag;
@@ -1745,7 +1749,7 @@ static int fwd_impl(const void* x, const void* prep, const float* h0, const uint
   }
   pack_units(a, g, nkg);
   // without weights in registers three workgroups fit a compute unit
-  a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nCf, nkg < 0 ? RGLRU_GIVEN_OCC : 2, 1 << 20);
+  a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nCf, nkg < 0 ? RGLRU_GIVEN_OCC : ((nkg == 4 || nkg == 2) ? RGLRU_NARROW_OCC : 2), 1 << 20);
   a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
   dim3 grid((unsigned)(a.wg_per_unit * a.units));
   {
