@@ -221,13 +221,14 @@ RGLRU_DEVICE bool carry_compose(const rec_t (&rec)[kDepth], CarryWalk& wk, int s
 }
 
 // Polling part of a walk: load a batch, compose, repeat until every lane has its carry.  After
-// `limit` fruitless polls the wave records the failure and returns an unspecified value, so every
-// wave still reaches the end of the kernel.
+// `limit` fruitless polls the wave records the failure and returns NaN as the carry of the lanes that
+// are still waiting, so every wave still reaches the end of the kernel and the failure is visible in
+// the results themselves (the chunk's outputs and the carry it hands on turn NaN) without anybody
+// having to read the failure word.
 RGLRU_DEVICE float carry_walk(const CarryChain& ch, CarryWalk& wk, int step, int end, float boundary,
-                              long long limit, unsigned* fail_word, int* stat) {
+                              long long limit, unsigned* fail_word) {
   long long polls = 0;
   while (!__all(wk.done)) {
-    if (stat) stat[0] += 1;                              // development aid: round trips
     rec_t rec[kDepth];
 #pragma unroll
     for (int d = 0; d < kDepth; ++d) {
@@ -237,9 +238,9 @@ RGLRU_DEVICE float carry_walk(const CarryChain& ch, CarryWalk& wk, int step, int
       if (inside && !wk.done) rec[d] = rec_load(ch.rec + q * ch.stride);
     }
     if (carry_compose(rec, wk, step, end, boundary)) {
-      if (stat) stat[1] += 1;                            // development aid: stalls
       if (++polls > limit) {
         if ((threadIdx.x & 63) == 0) atomicOr(fail_word, 1u);
+        if (!wk.done) wk.acc_h = __builtin_nanf("");
         break;
       }
       __builtin_amdgcn_s_sleep(1);
@@ -252,10 +253,10 @@ RGLRU_DEVICE float carry_walk(const CarryChain& ch, CarryWalk& wk, int step, int
 // c - 1) and +1 when it runs backward; `end` is the index one past the first chunk of the chain
 // (-1 or the chunk count), where `boundary` is the carry.
 RGLRU_DEVICE float carry_lookback(const CarryChain& ch, int c, int step, int end, float boundary,
-                                  bool lane_ok, long long limit, unsigned* fail_word, int* stat = nullptr) {
+                                  bool lane_ok, long long limit, unsigned* fail_word) {
   CarryWalk wk;
   wk.acc_a = 1.f; wk.acc_h = 0.f; wk.done = !lane_ok; wk.p = c + step;
-  return carry_walk(ch, wk, step, end, boundary, limit, fail_word, stat);
+  return carry_walk(ch, wk, step, end, boundary, limit, fail_word);
 }
 
 // The first batch of a walk requested ahead of time.  A device-scope load takes a few
@@ -291,12 +292,11 @@ RGLRU_DEVICE void carry_prefetch(rsrc_t recs, unsigned lane_off, unsigned stride
 }
 
 RGLRU_DEVICE float carry_lookback_from(const CarryBatch& first, const CarryChain& ch, int c, int step, int end,
-                                       float boundary, bool lane_ok, long long limit, unsigned* fail_word,
-                                       int* stat = nullptr) {
+                                       float boundary, bool lane_ok, long long limit, unsigned* fail_word) {
   CarryWalk wk;
   wk.acc_a = 1.f; wk.acc_h = 0.f; wk.done = !lane_ok; wk.p = c + step;
-  if (carry_compose(first.rec, wk, step, end, boundary) && stat) stat[1] += 1;
-  return carry_walk(ch, wk, step, end, boundary, limit, fail_word, stat);
+  carry_compose(first.rec, wk, step, end, boundary);
+  return carry_walk(ch, wk, step, end, boundary, limit, fail_word);
 }
 
 // ------------------------------------------------------------------------------------------

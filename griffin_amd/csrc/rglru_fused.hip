@@ -132,14 +132,6 @@ __global__ void prepare_kernel(PrepArgs p) {
   }
 }
 
-#ifdef RGLRU_TRACE
-// Development aid (not part of the shipped library): per-wave phase timestamps.
-#define RGLRU_STAMP(p, slot) do { if ((p).trace && (threadIdx.x & 63) == 0) { \
-    long long* t_ = (p).trace + ((((long long)blockIdx.x * 4 + (threadIdx.x >> 6)) * 8 + trace_iter) * 12 + (slot)); \
-    if (trace_iter < 8) *t_ = (long long)__builtin_readcyclecounter(); } } while (0)
-#else
-#define RGLRU_STAMP(p, slot) do { } while (0)
-#endif
 
 // ------------------------------------------------------------------------------------------
 // Arguments common to the fused kernels
@@ -162,9 +154,6 @@ struct FusedArgs {
   long long rows_total;                                   // B * T, the row count of one block of `pre`
   int nC, nCf, ckpt_nC, wg_per_unit, aligned, full_slabs, queues, flags_vec;
   long long limit;
-#ifdef RGLRU_TRACE
-  long long* trace;
-#endif
 };
 
 // Ticket queues.  A unit's (chunk, sequence) tiles are dealt to `queues` counters: queue j owns the
@@ -409,7 +398,7 @@ RGLRU_DEVICE void fwd_local(const FusedArgs& p, const WaveId& w, FwdTile<MT>& t,
 // Stage 2: carry in, carry out and checkpoint, then the recurrence itself and the stores.
 template <typename IO, int MT, bool MASKED, bool STAGED>
 RGLRU_DEVICE void fwd_finalize(const FusedArgs& p, const WaveId& w, const FwdTile<MT>& t, unsigned char* stage,
-                               const CarryBatch* first = nullptr, bool live = true, int trace_iter = 0) {
+                               const CarryBatch* first = nullptr, bool live = true) {
   constexpr int EL = 16 * MT, TR = 32 * MT;
   const int hf = w.hf, b = t.b, c = t.c;
   const long long W = p.W;
@@ -419,26 +408,12 @@ RGLRU_DEVICE void fwd_finalize(const FusedArgs& p, const WaveId& w, const FwdTil
   chain.rec = p.rec_a + (long long)b * p.nCf * W + w.ch; chain.stride = W;
 
   float h_in = 0.f;
-  RGLRU_STAMP(p, 5);
-#ifdef RGLRU_TRACE
-  int stat[2] = {0, 0};
-  int* stat_p = stat;
-#else
-  int* stat_p = nullptr;
-#endif
   if (c != 0) {
-    h_in = first ? carry_lookback_from(*first, chain, c, -1, -1, 0.f, ch_ok, p.limit, p.fail, stat_p)
-                 : carry_lookback(chain, c, -1, -1, 0.f, ch_ok, p.limit, p.fail, stat_p);
+    h_in = first ? carry_lookback_from(*first, chain, c, -1, -1, 0.f, ch_ok, p.limit, p.fail)
+                 : carry_lookback(chain, c, -1, -1, 0.f, ch_ok, p.limit, p.fail);
   } else if (p.h0 && ch_ok) {
     h_in = p.h0[(long long)b * W + w.ch];
   }
-#ifdef RGLRU_TRACE
-  if (p.trace && w.lane == 0 && trace_iter < 8) {
-    long long* t_ = p.trace + (((long long)blockIdx.x * 4 + (threadIdx.x >> 6)) * 8 + trace_iter) * 12;
-    t_[8] = stat[0]; t_[9] = stat[1]; t_[10] = c;
-  }
-#endif
-  RGLRU_STAMP(p, 6);
   const float h_end = fmaf(t.A_t, h_in, t.H_t);
   const float h_mid = fmaf(t.A_lo, h_in, t.H_lo);
   {
@@ -485,20 +460,11 @@ RGLRU_DEVICE void fwd_finalize(const FusedArgs& p, const WaveId& w, const FwdTil
   }
 }
 
-// Forward tile = 32 * kFwdMT tokens.  Two ways to run the loop, chosen by kFwdDefer:
-//   true   (needs kFwdMT = 1 to fit the registers) two tiles in flight, the previous tile is finished
-//          after the gate math of the current one, its records requested an iteration ahead;
-//   false  a tile is finished in the iteration that computed it.
-// 64-token tiles without the deferral halve the look-backs, barriers, tickets and records per token,
-// which is worth more than hiding them: 39.6 us against 43.5 us at B8 T2048 W1024, 84 us against
-// 104 us for one sequence of 32768 tokens.
-#ifdef RGLRU_FWD_DEFER
-constexpr int kFwdMT = 1;
-constexpr bool kFwdDefer = true;
-#else
+// Forward tile = 32 * kFwdMT tokens; a tile is finished in the iteration that computed it.  64-token
+// tiles halve the look-backs, barriers, tickets and records per token (39.6 us against 43.5 us for
+// 32-token tiles with two tiles in flight at B8 T2048 W1024, 84 us against 104 us for one sequence of
+// 32768 tokens).
 constexpr int kFwdMT = 2;
-constexpr bool kFwdDefer = false;
-#endif
 
 // workgroups per compute unit of the forward kernel without weights in registers (NKG < 0); 4 spills
 #define RGLRU_GIVEN_OCC 3
@@ -586,16 +552,11 @@ __global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : (NKG == 4 ||
     long long tk = s_ticket[0];
     int par = 0;
     issue(tk);
-    int trace_iter = 0; (void)trace_iter;
-    // Two tiles are in flight per wave: the tile whose own map was published in the previous
-    // iteration is finished (carry in, recurrence, stores) after the gate math of the current one,
-    // so the wait for the neighbours' records overlaps with useful work.
-    FwdTile<MT> cur, prev;
-    bool have_prev = false;
-    prev.b = 0; prev.c = 0;                              // chunk 0 has no records to request
+    FwdTile<MT> cur;
+    cur.b = 0; cur.c = 0;
 #pragma unroll
-    for (int e = 0; e < EL; ++e) { prev.a[e] = 0.f; prev.z[e] = 0.f; }
-    prev.A_lo = prev.H_lo = prev.A_t = prev.H_t = 0.f;
+    for (int e = 0; e < EL; ++e) { cur.a[e] = 0.f; cur.z[e] = 0.f; }
+    cur.A_lo = cur.H_lo = cur.A_t = cur.H_t = 0.f;
     // every wave has a slab except in the last unit of a block count that does not fill it
     const bool slab_ok = (NKG == 8) ? true : w.slab_ok;
     const rsrc_t rticket = make_rsrc(q.counter, 4u);
@@ -603,9 +564,8 @@ __global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : (NKG == 4 ||
     const unsigned rec_lane = (slab_ok && w.ch_ok) ? (unsigned)w.ch * 8u : kOutOfRange;
     // A dead finalize in front of the loop: the loop is entered with the same memory operations in
     // flight as its back edge has, so the waits at its top are exact instead of worst case.
-    fwd_finalize<IO, MT, MASKED, sizeof(IO) == 2>(p, w, prev, stage, nullptr, false, 0);
+    fwd_finalize<IO, MT, MASKED, sizeof(IO) == 2>(p, w, cur, stage, nullptr, false);
     while (tk < q.tiles) {
-      RGLRU_STAMP(p, 0);
       cur.c = (int)((unsigned)tk / (unsigned)q.n_b);
       cur.b = q.first_b + (int)((unsigned)tk - (unsigned)cur.c * (unsigned)q.n_b) * p.queues;
       const long long trow = (long long)cur.b * p.T + cur.c * TR + hf * EL;
@@ -615,13 +575,9 @@ __global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : (NKG == 4 ||
       for (int mt = 0; mt < MT; ++mt) flbits[mt] = MASKED ? flag_run(p, trow + 16 * mt, cur.c * TR + hf * EL + 16 * mt) : 0u;
       // next ticket: one instruction for the whole workgroup, live only in its first lane
       const unsigned next_raw = (unsigned)__builtin_amdgcn_raw_ptr_buffer_atomic_add_i32(1, rticket, tid == 0 ? 0u : kOutOfRange, 0, 0);
-      // records the previous tile will need: requested now, used after this tile's gate math
+      // records this tile will need: requested now, used after its gate math
       CarryBatch ahead;
-      if constexpr (kFwdDefer)
-        carry_prefetch(make_rsrc(p.rec_a + (long long)prev.b * p.nCf * W, (unsigned)p.nCf * rec_stride), rec_lane,
-                       rec_stride, prev.c, -1, -1, ahead);
-      else
-        carry_prefetch(make_rsrc(p.rec_a + (long long)cur.b * p.nCf * W, (unsigned)p.nCf * rec_stride), rec_lane,
+      carry_prefetch(make_rsrc(p.rec_a + (long long)cur.b * p.nCf * W, (unsigned)p.nCf * rec_stride), rec_lane,
                        rec_stride, cur.c, -1, -1, ahead);
 #pragma unroll
       for (int i = 0; i < NV; ++i) {
@@ -636,7 +592,6 @@ __global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : (NKG == 4 ||
         }
       }
       __syncthreads();
-      RGLRU_STAMP(p, 1);
       if (slab_ok) {
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
@@ -657,26 +612,14 @@ __global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : (NKG == 4 ||
         }
       }
       fwd_local<MT, MASKED>(p, w, cur, slab_ok);
-      RGLRU_STAMP(p, 2);
       if (tid == 0) s_ticket[par ^ 1] = next_raw;
       __syncthreads();
-      RGLRU_STAMP(p, 3);
       par ^= 1;
       const long long tk_next = s_ticket[par];
       issue(tk_next);
-      RGLRU_STAMP(p, 4);
-      if constexpr (kFwdDefer) {
-        fwd_finalize<IO, MT, MASKED, sizeof(IO) == 2>(p, w, prev, stage, &ahead, have_prev && slab_ok, trace_iter);
-        prev = cur;
-        have_prev = true;
-      } else {
-        fwd_finalize<IO, MT, MASKED, sizeof(IO) == 2>(p, w, cur, stage, &ahead, slab_ok, trace_iter);
-      }
-      RGLRU_STAMP(p, 7);
-      ++trace_iter;
+      fwd_finalize<IO, MT, MASKED, sizeof(IO) == 2>(p, w, cur, stage, &ahead, slab_ok);
       tk = tk_next;
     }
-    if (kFwdDefer && slab_ok && have_prev) fwd_finalize<IO, MT, MASKED, sizeof(IO) == 2>(p, w, prev, stage, nullptr, true, trace_iter);
   } else {
     for (;;) {
       if (tid == 0) s_ticket[0] = atomicAdd(q.counter, 1u);
@@ -977,11 +920,9 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
   unsigned tk = s_ticket[0];
   int par = 0;
   issue(tk);
-  int trace_iter = 0; (void)trace_iter;
   while ((long long)tk < q.tiles) {
     int c, b;
     decode(tk, c, b);
-    RGLRU_STAMP(p, 0);
     const int t0 = c * TR;
     const long long trow = (long long)b * p.T + t0 + hf * EL;
     unsigned next_raw = 0;
@@ -1007,7 +948,6 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
       }
     }
     __syncthreads();
-    RGLRU_STAMP(p, 1);
     f32x16 ua, ux;
     float xv[EL], gy[EL];
     if (w.slab_ok) {
@@ -1043,10 +983,8 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
         for (int e = 0; e < EL; ++e) gy[e] = (float)lds_dy[(hf * EL + e) * LDSROW + (NKG == 8 ? 0 : w.kb) + w.slab * 32 + w.r];
       }
     }
-    RGLRU_STAMP(p, 2);
     if (tid == 0) s_ticket[par ^ 1] = next_raw;
     __syncthreads();
-    RGLRU_STAMP(p, 3);
     par ^= 1;
     const unsigned tk_next = s_ticket[par];
     if (!w.slab_ok) {                                    // a wave without a slab only helps with the loads
@@ -1085,7 +1023,6 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
     chain.rec = p.rec_a + seq; chain.stride = W;
     const bool last_chunk = c == p.nC - 1;
     if (!last_chunk && hf == 0) carry_publish(chain, c, A_t, D_t, false);
-    RGLRU_STAMP(p, 4);
 
     // input gate and g = sqrt(1 - a^2)
 #pragma unroll
@@ -1097,10 +1034,8 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
       gi[e] = ie; g[e] = ge;
     }
     issue(tk_next);
-    RGLRU_STAMP(p, 5);
     float d_in = (last_chunk && p.dh_last) ? p.dh_last[(long long)b * W + w.ch] : 0.f;
     if (!last_chunk) d_in = carry_lookback(chain, c, +1, p.nC, 0.f, true, p.limit, p.fail);
-    RGLRU_STAMP(p, 6);
     const float d_out = fmaf(A_t, d_in, D_t);
     if (hf == 0) carry_publish(chain, c, 0.f, d_out, true);
     if (hf == 0 && c == 0 && p.dh0) p.dh0[(long long)b * W + w.ch] = d_out;
@@ -1171,8 +1106,6 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
       }
     }
     wave_lds_fence();
-    RGLRU_STAMP(p, 7);
-    ++trace_iter;
     tk = tk_next;
   }
   // per-workgroup partial sums (every slot is written, so the buffer needs no clearing)
@@ -1549,6 +1482,20 @@ static int check_geometry(const char* who, int64_t W, int64_t nb, int dtype) {
   return RGLRU_OK;
 }
 
+// Sizes the kernels address with 32-bit offsets.  Tiles and per-sequence slices of the workspace are
+// reached through buffer descriptors whose lane offsets are 32-bit and whose "dropped access" offset
+// is 0x7ffffff0, so every such extent has to stay below 2^31 bytes: the checkpoints of one sequence
+// (the fp32 state after every 16 tokens, 4 W bytes each; the carry records of a sequence are no larger)
+// and the [B, W] fp32 state tensors.
+static int check_extents(const char* who, int64_t B, int64_t T, int64_t W) {
+  if (B * T * W >= (1ll << 40) || B * T >= (1ll << 31)) return fail(RGLRU_E_UNSUPPORTED, "%s: tensor too large", who);
+  const int64_t slots = 4 * ((T + 63) / 64);              // checkpoint slots per sequence
+  if (slots * W * 4 >= (1ll << 31))
+    return fail(RGLRU_E_UNSUPPORTED, "%s: one sequence of %lld tokens x %lld channels exceeds the 2 GiB per-sequence workspace limit; split the sequence and carry the state", who, (long long)T, (long long)W);
+  if (B * W * 4 >= (1ll << 31)) return fail(RGLRU_E_UNSUPPORTED, "%s: state tensor [%lld, %lld] too large", who, (long long)B, (long long)W);
+  return RGLRU_OK;
+}
+
 static size_t elem_size(int dtype) { return dtype == RGLRU_BF16 ? 2 : 4; }
 
 static void fill_common(FusedArgs& a, const Geometry& g, const void* prep, int dtype) {
@@ -1654,10 +1601,6 @@ using namespace rglru;
 
 extern "C" {
 
-#ifdef RGLRU_TRACE
-static long long* g_trace = nullptr;
-void rglru_hip_debug_trace(void* buffer) { g_trace = (long long*)buffer; }
-#endif
 
 int rglru_hip_max_block_width(void) { return 512; }
 
@@ -1718,7 +1661,8 @@ static int fwd_impl(const void* x, const void* prep, const float* h0, const uint
   if (rc) return rc;
   if (B <= 0 || T <= 0) return fail(RGLRU_E_ARG, "fwd: B and T must be positive (got %lld, %lld)", (long long)B, (long long)T);
   if (!x || !prep || !y || !ws) return fail(RGLRU_E_ARG, "fwd: null pointer");
-  if (B * T * W >= (1ll << 40) || B * T >= (1ll << 31)) return fail(RGLRU_E_UNSUPPORTED, "fwd: tensor too large");
+  rc = check_extents("fwd", B, T, W);
+  if (rc) return rc;
   Geometry g = make_geometry(W, nb);
   WorkLayout L = make_work_layout(B, T, g);
   hipStream_t s = (hipStream_t)stream;
@@ -1737,9 +1681,6 @@ static int fwd_impl(const void* x, const void* prep, const float* h0, const uint
   a.B = (int)B; a.T = (int)T; a.nC = (int)L.nC; a.ckpt_nC = 2 * (int)L.nC;
   a.nCf = (int)((T + 32 * kFwdMT - 1) / (32 * kFwdMT));
   a.aligned = is_aligned(x, W, g.bw, elem_size(dtype)) && ((uintptr_t)y % 16 == 0);
-#ifdef RGLRU_TRACE
-  a.trace = g_trace;
-#endif
   int nkg = held_groups(g, dtype, a.aligned);
   if (pre) {
     if (!rglru_hip_pre_path(W, nb, dtype)) return fail(RGLRU_E_UNSUPPORTED, "fwd_pre: needs bf16 storage and gate blocks of a multiple of 32 channels");
@@ -1793,7 +1734,8 @@ int rglru_hip_bwd_pre(const void* x, const void* pre, const void* prep, const fl
   if (B <= 0 || T <= 0) return fail(RGLRU_E_ARG, "bwd_pre: B and T must be positive (got %lld, %lld)", (long long)B, (long long)T);
   if (!x || !pre || !prep || !dy || !ws || !scratch || !dx || !du || !db_a || !db_x || !dlambda)
     return fail(RGLRU_E_ARG, "bwd_pre: null pointer");
-  if (B * T * W >= (1ll << 40) || B * T >= (1ll << 31)) return fail(RGLRU_E_UNSUPPORTED, "bwd_pre: tensor too large");
+  rc = check_extents("bwd_pre", B, T, W);
+  if (rc) return rc;
   Geometry g = make_geometry(W, nb);
   if (!is_aligned(x, W, g.bw, 2) || !is_aligned(dy, W, g.bw, 2) || !is_aligned(dx, W, g.bw, 2) ||
       (uintptr_t)pre % 16 || (uintptr_t)du % 16)
@@ -1866,7 +1808,8 @@ int rglru_hip_bwd(const void* x, const void* prep, const float* h0,
   if (B <= 0 || T <= 0) return fail(RGLRU_E_ARG, "bwd: B and T must be positive (got %lld, %lld)", (long long)B, (long long)T);
   if (!x || !prep || !dy || !ws || !scratch || !dx || !du_a || !du_x || !db_a || !db_x || !dlambda)
     return fail(RGLRU_E_ARG, "bwd: null pointer");
-  if (B * T * W >= (1ll << 40) || B * T >= (1ll << 31)) return fail(RGLRU_E_UNSUPPORTED, "bwd: tensor too large");
+  rc = check_extents("bwd", B, T, W);
+  if (rc) return rc;
   Geometry g = make_geometry(W, nb);
   WorkLayout L = make_work_layout(B, T, g);
   hipStream_t s = (hipStream_t)stream;
@@ -1921,7 +1864,8 @@ int rglru_hip_bwd_full(const void* x, const void* prep, const float* h0,
   if (B <= 0 || T <= 0) return fail(RGLRU_E_ARG, "bwd_full: B and T must be positive (got %lld, %lld)", (long long)B, (long long)T);
   if (!x || !prep || !dy || !ws || !scratch || !dx || !dw_a || !dw_x || !db_a || !db_x || !dlambda)
     return fail(RGLRU_E_ARG, "bwd_full: null pointer");
-  if (B * T * W >= (1ll << 40) || B * T >= (1ll << 31)) return fail(RGLRU_E_UNSUPPORTED, "bwd_full: tensor too large");
+  rc = check_extents("bwd_full", B, T, W);
+  if (rc) return rc;
   Geometry g = make_geometry(W, nb);
   if (!is_aligned(x, W, g.bw, 2) || !is_aligned(dy, W, g.bw, 2) || !is_aligned(dx, W, g.bw, 2))
     return fail(RGLRU_E_UNSUPPORTED, "bwd_full: x, dy and dx must be 16-byte aligned");
@@ -1941,9 +1885,6 @@ int rglru_hip_bwd_full(const void* x, const void* prep, const float* h0,
   a.partial = (float*)(sb + SL.partial); a.dw_partial = (float*)(sb + SL.dw_partial);
   a.B = (int)B; a.T = (int)T; a.nC = (int)((T + kChunk - 1) / kChunk); a.ckpt_nC = 2 * (int)L.nC;
   a.aligned = 1;
-#ifdef RGLRU_TRACE
-  a.trace = g_trace;
-#endif
   const int nkg = held_groups(g, dtype, 1);
   pack_units(a, g, nkg);
   a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nC, 2, L.max_wg);

@@ -69,6 +69,17 @@ def test_argument_errors_are_reported_without_a_gpu(lib):
         _lib.check(3, "probe")
 
 
+def test_oversized_sequences_are_rejected_on_the_host(lib):
+    """Per-sequence slices of the workspace are addressed with 32-bit offsets: a sequence whose
+    checkpoints (4 W bytes per 16 tokens) reach 2 GiB is refused before anything is launched."""
+    fake = ctypes.c_void_p(256)            # never dereferenced: the size checks come first
+    args = lambda T, W: (fake, fake, None, None, fake, None, fake, 1, T, W, W // 128, _lib.RGLRU_BF16, None)
+    assert lib.rglru_hip_fwd(*args(1 << 23, 1024)) == 2          # T W = 2^33
+    assert b"per-sequence" in lib.rglru_hip_last_error()
+    assert lib.rglru_hip_fwd(*args(1 << 24, 512)) == 2
+    assert lib.rglru_hip_fwd(fake, fake, None, None, fake, None, fake, 1 << 20, 2048, 1024, 8, _lib.RGLRU_BF16, None) == 2
+
+
 def test_spin_limit_hook_round_trips(lib):
     previous = lib.rglru_hip_set_spin_limit(1234)
     assert lib.rglru_hip_set_spin_limit(previous) == 1234

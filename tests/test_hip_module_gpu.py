@@ -346,7 +346,9 @@ def test_config5_recurrent_block_with_hip_scan():
 # ------------------------------------------------------------------ failure handling
 def test_bounded_wait_gives_up_instead_of_hanging():
     """With the poll budget forced to one, waves that do not find their carry at once record the
-    failure and still run to the end of the kernel; the next call with the normal budget is exact."""
+    failure and still run to the end of the kernel; a give-up is visible in the results themselves (the
+    carry it could not get is NaN, and with it the chunk's outputs and its carry out) and never a
+    silently wrong number; the next call with the normal budget is exact."""
     import ctypes
 
     from griffin_amd import _lib, hip_rglru_scan
@@ -371,8 +373,16 @@ def test_bounded_wait_gives_up_instead_of_hanging():
     assert lib.rglru_hip_workspace_status(ws.data_ptr(), B, T, W, 1, 1, stream, ctypes.byref(status)) == 0
     _say("failure word after a one-poll budget:", status.value)
     assert status.value in (0, 1)
-    good = hip_rglru_scan(a, z, h0)
     want = 10.0 * (1.0 - 0.9 ** torch.arange(1, T + 1, dtype=torch.float64))
+    bad = torch.isnan(out)
+    if status.value == 1:
+        assert bad.any(), "a wave gave up but no result was poisoned"
+    else:
+        assert not bad.any()
+    # whatever is not NaN is right: no silently wrong values
+    finite = ~bad[0, :, 0]
+    assert rel_err(out[0, :, 0][finite], want[finite.cpu()]) < 1e-5
+    good = hip_rglru_scan(a, z, h0)
     assert rel_err(good[0, :, 0], want) < 1e-5
 
 
