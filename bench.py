@@ -32,11 +32,6 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0
 
-# HBM bytes per launch at the benchmark workload (B8 T2048 W1024 nb8 bf16), from two rocprofv3 --pmc
-# runs of this script (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), each scaled by what the same
-# counter reads for the 64 MiB copy that --traffic-probe adds (profiles/ holds the summaries).  Only
-# valid for that workload; other shapes report null.
-MEASURED_TRAFFIC_BYTES = {"bwd_scan_kernel": 189019817, "fwd_kernel": 81510566, "gate_grad_kernel": 201920628}
 BENCH_SHAPE = (8, 2048, 1024, 8)
 
 
@@ -49,6 +44,9 @@ def parse_args():
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph replay")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also run a plain 64 MiB device copy a few times (known traffic, for scaling profiler counters)")
+    ap.add_argument("--repeats", type=int, default=5, help="timed regions of K steps each; the median is reported")
+    ap.add_argument("--input-sets", type=int, default=5,
+                    help="distinct (x, dy) sets the timed steps rotate through (1 = the same buffers every step)")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--seq", type=int, default=2048)
     ap.add_argument("--width", type=int, default=1024)
@@ -136,28 +134,75 @@ def secondary_workload(args):
     }))
 
 
-def cpu_baseline(case, budget_s=20.0):
-    """The oracle (port of the reference's CPU sequential path, fp32) on the host cores: forward +
-    autograd backward on the same workload, bf16-rounded inputs upcast to fp32."""
+def _median(values):
+    v = sorted(values)
+    return v[len(v) // 2]
+
+
+def cpu_baseline(case):
+    """The oracle (port of the reference's CPU sequential path, griffin/griffin.py:237-289, fp32) on the
+    host cores: forward + autograd backward on a bounded slice of the same workload (bf16-rounded
+    inputs upcast to fp32).  All host threads on the first two sequences, and one thread on the first
+    sequence; each the median of five iterations after one warm-up.  Sequences are independent, so
+    tokens/s of a slice is tokens/s of the workload."""
     from tests.helpers import oracle_run
 
+    def timed(rows, threads, iterations):
+        torch.set_num_threads(threads)
+        part = {k: (v[:rows] if (torch.is_tensor(v) and k in ("x", "dy", "h0")) else v) for k, v in case.items()}
+        oracle_run(part, torch.bfloat16)            # warm-up
+        times = []
+        for _ in range(iterations):
+            t0 = time.perf_counter()
+            oracle_run(part, torch.bfloat16)
+            times.append(time.perf_counter() - t0)
+        return _median(times), rows * case["x"].shape[1]
+
     threads = os.cpu_count() or 1
-    torch.set_num_threads(threads)
     B, T, _ = case["x"].shape
-    t0 = time.perf_counter()
-    oracle_run(case, torch.bfloat16)            # warm-up
-    first = time.perf_counter() - t0
-    times = []
-    while (not times) or (sum(times) + first < budget_s and len(times) < 5):
-        t0 = time.perf_counter()
-        oracle_run(case, torch.bfloat16)
-        times.append(time.perf_counter() - t0)
-    times.sort()
-    med = times[len(times) // 2]
+    rows_all = min(2, B)
+    med_all, tok_all = timed(rows_all, threads, 5)
+    med_one, tok_one = timed(1, 1, 5)
+    torch.set_num_threads(threads)
     return {
-        "value": B * T / med, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
-        "sample": f"{len(times)} fwd+bwd iterations of the full workload after 1 warm-up, median {med:.3f} s",
+        "value": tok_all / med_all, "unit": "tokens/s", "cores": threads, "kind": "port",
+        "sample": f"fwd+bwd of {rows_all} of the {B} sequences (T={T}), median of 5 iterations after 1 warm-up: {med_all:.3f} s on {threads} threads",
+        "one_thread": {"value": tok_one / med_one, "unit": "tokens/s", "cores": 1,
+                       "sample": f"fwd+bwd of 1 sequence (T={T}), median of 5 iterations after 1 warm-up: {med_one:.3f} s"},
     }
+
+
+def source_digest():
+    """sha256 over the kernel sources the library is built from (what a profile summary is keyed to)."""
+    import hashlib
+
+    h = hashlib.sha256()
+    csrc = os.path.join(ROOT, "griffin_amd", "csrc")
+    for name in sorted(os.listdir(csrc)):
+        if name.endswith((".hip", ".h")):
+            h.update(name.encode())
+            h.update(open(os.path.join(csrc, name), "rb").read())
+    return h.hexdigest()
+
+
+def measured_traffic():
+    """HBM bytes per launch from the committed rocprofv3 summary (FETCH_SIZE / WRITE_SIZE runs of this
+    script, scaled by a copy of known size).  The summary ends in a line `traffic-json: {...}` that names
+    the digest of the kernel sources it was measured on; a summary of other sources is not used."""
+    path = os.path.join(ROOT, "profiles", "rglru_fwd_bwd_B8_T2048_W1024_bf16_hbm_traffic.txt")
+    try:
+        for line in open(path):
+            if line.startswith("traffic-json:"):
+                rec = json.loads(line[len("traffic-json:"):])
+                if rec.get("source_sha256") != source_digest():
+                    return None, "profiles/ summary was measured on other kernel sources (stale); traffic not reported"
+                return rec, f"profiles/{os.path.basename(path)}, kernel sources {rec['source_sha256'][:12]}"
+    except OSError:
+        pass
+    return None, "no traffic summary under profiles/"
+
+
+KERNEL_SLOTS = {"fwd_kernel": 0, "bwd_scan_kernel": 1, "gate_grad_kernel": 3}
 
 
 def main():
@@ -179,70 +224,113 @@ def main():
     B, T, W, nb = args.batch, args.seq, args.width, args.blocks
     case = orc.make_case(B, T, W, nb, seed=0)
     dt = torch.bfloat16
-    x = case["x"].to(dt).to(dev).requires_grad_(True)
     params = [case[k].to(dt).to(dev).requires_grad_(True) for k in ("w_a", "b_a", "w_x", "b_x", "lam")]
-    dy = case["dy"].to(dt).to(dev)
-    leaves = [x] + params
+    # Input sets.  Set 0 is the seeded case; the others are fresh N(0,1) draws of the same shape.  The
+    # timed region walks through all of them, so no step finds its inputs (or the previous step's
+    # outputs) in the 256 MB memory-side cache: with the outputs and scratch of every step in between
+    # more than 1 GiB is touched before a buffer comes round again.
+    n_sets = max(args.input_sets, 1)
+    gen = torch.Generator(device=dev).manual_seed(1)
+    xs = [case["x"].to(dt).to(dev).requires_grad_(True)]
+    dys = [case["dy"].to(dt).to(dev)]
+    for _ in range(n_sets - 1):
+        xs.append(torch.randn(B, T, W, device=dev, generator=gen).to(dt).requires_grad_(True))
+        dys.append(torch.randn(B, T, W, device=dev, generator=gen).to(dt))
 
-    def step():
-        y, _ = hip_rglru(x, *params, 8.0)
-        return torch.autograd.grad(y, leaves, dy)
+    def step(i=0):
+        y, _ = hip_rglru(xs[i], *params, 8.0)
+        return (y,) + torch.autograd.grad(y, [xs[i]] + params, dys[i])
 
     for _ in range(max(args.warmup, 3)):
         step()
     torch.cuda.synchronize()
 
-    graph = None
+    def capture(sets, per_graph):
+        """A HIP graph of per_graph whole steps, step j on input set j % sets; returns (graph, outputs)."""
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for i in range(sets):
+                step(i)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            outs = [step(j % sets) for j in range(per_graph)]
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        return graph, outs
+
+    # One graph holds several whole steps: consecutive replays of a graph are ~8 us apart on this
+    # runtime, a launch cost that a training step amortises over all of its kernels and that says
+    # nothing about this operator.  A timed region is still exactly K steps.
+    per_graph = next(d for d in (10, 5, 4, 3, 2, 1) if args.steps % d == 0)
+    graphs = {}
     if not args.no_graph:
         try:
-            side = torch.cuda.Stream()
-            side.wait_stream(torch.cuda.current_stream())
-            with torch.cuda.stream(side):
-                step()
-            torch.cuda.current_stream().wait_stream(side)
-            torch.cuda.synchronize()
-            # One graph holds several whole steps: consecutive replays of a graph are ~8 us apart on
-            # this runtime, a launch cost that a training step amortises over all of its kernels and
-            # that says nothing about this operator.  The timed region is still exactly K steps.
-            per_graph = next(d for d in (10, 5, 4, 3, 2, 1) if args.steps % d == 0)
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                captured = [step() for _ in range(per_graph)]
-            for _ in range(3):
-                graph.replay()
-            torch.cuda.synchronize()
+            graphs["rotating"] = capture(n_sets, per_graph)
+            graphs["same"] = capture(1, per_graph)
         except Exception as error:  # fall back to eager timing, and say so
             print(f"bench.py: graph capture failed ({error}); timing eager launches", file=sys.stderr)
-            graph = None
-    if graph is None:
-        per_graph = 1
+            graphs = {}
 
-    run = graph.replay if graph is not None else step
-    for _ in range((args.warmup + per_graph - 1) // per_graph):     # at least W warm-up steps
-        run()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps // per_graph):
-        run()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed * 1e3 / args.steps
+    def time_region(run, calls):
+        """Median over `repeats` timed regions of exactly K steps each (ms per step)."""
+        for _ in range(max((args.warmup + per_graph - 1) // per_graph, 1)):
+            run()
+        samples = []
+        for _ in range(args.repeats):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(calls):
+                run()
+            torch.cuda.synchronize()
+            samples.append((time.perf_counter() - t0) * 1e3 / args.steps)
+        return _median(samples), samples
+
+    graph_check = None
+    if graphs:
+        ms_per_step, samples = time_region(graphs["rotating"][0].replay, args.steps // per_graph)
+        ms_same, _ = time_region(graphs["same"][0].replay, args.steps // per_graph)
+        # the timed launch mode against eager launches: the last captured step of the last replay
+        # (input set j) and one eager step on the same inputs.  Equal up to the rounding of a different
+        # carry composition order (which records a look-back meets depends on timing).
+        j = (per_graph - 1) % n_sets
+        captured = [t.detach().clone() for t in graphs["rotating"][1][-1]]
+        eager = step(j)
+        torch.cuda.synchronize()
+        worst = 0.0
+        for got, want in zip(captured, eager):
+            scale = want.float().abs().max().item() or 1.0
+            worst = max(worst, (got.float() - want.float()).abs().max().item() / scale)
+        graph_check = {"graph_matches_eager": bool(worst < 1e-2), "graph_vs_eager_max_rel_err": worst}
+        launch = f"hip graph replay, {per_graph} steps per graph, {n_sets} input sets in rotation"
+    else:
+        per_graph = 1
+        counter = [0]
+
+        def eager_rotating():
+            step(counter[0] % n_sets)
+            counter[0] += 1
+        ms_per_step, samples = time_region(eager_rotating, args.steps)
+        ms_same, _ = time_region(step, args.steps)
+        launch = f"eager, {n_sets} input sets in rotation"
 
     # per-kernel durations, HIP events on the launch stream (library measurement hook), eager launches;
     # the hook keeps the events of the latest launch of each kernel
     lib.rglru_hip_set_timing(1)
-    names = {"fwd_kernel": 0, "bwd_scan_kernel": 1, "gate_grad_kernel": 3}
-    samples = {k: [] for k in names}
-    for _ in range(20):
-        for _ in range(4):      # back to back: the last step's kernels run on a busy GPU, as in the timed region
-            step()
-        for k, slot in names.items():
-            samples[k].append(lib.rglru_hip_kernel_ms(slot))
+    kernel_samples = {k: [] for k in KERNEL_SLOTS}
+    for it in range(20):
+        for k4 in range(4):      # back to back: the last step's kernels run on a busy GPU, as in the timed region
+            step((4 * it + k4) % n_sets)
+        for k, slot in KERNEL_SLOTS.items():
+            kernel_samples[k].append(lib.rglru_hip_kernel_ms(slot))
     lib.rglru_hip_set_timing(0)
-    for k, v in samples.items():
+    for k, v in kernel_samples.items():
         if min(v) <= 0:
             raise RuntimeError(f"kernel timing hook returned no measurement for {k}: {v[:3]}")
-    avg_ms = {k: sum(v) / len(v) for k, v in samples.items()}
+    avg_ms = {k: sum(v) / len(v) for k, v in kernel_samples.items()}
 
     if args.traffic_probe:
         src = torch.empty(64 * 1024 * 1024 // 4, device=dev).normal_()
@@ -252,39 +340,50 @@ def main():
         torch.cuda.synchronize()
 
     # Algorithmic bytes: the compulsory streams at the storage size.  Forward reads x and writes y;
-    # the backward scan kernel reads x and dy and writes the input gradient; the gradient GEMM kernel
-    # adds no compulsory stream of its own (everything it moves is overhead of the two-kernel split).
+    # backward reads x and dy and writes dx: 5 s N per step (s = 2 bytes).  The roofline object is that
+    # of the whole step; the dominant kernel's own figure is under "kernels".
     n = B * T * W
     elem = 2
+    step_bytes = 5 * elem * n
     algo = {"fwd_kernel": 2 * elem * n, "bwd_scan_kernel": 3 * elem * n, "gate_grad_kernel": 0}
     dominant = max(avg_ms, key=avg_ms.get)
-    dom_bytes, dom_ms = algo[dominant], avg_ms[dominant]
-    achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
-    traffic = MEASURED_TRAFFIC_BYTES[dominant] if (B, T, W, nb) == BENCH_SHAPE else None
-    step_gbps = 5 * elem * n / (ms_per_step * 1e-3) / 1e9
+    step_gbps = step_bytes / (ms_per_step * 1e-3) / 1e9
+    traffic_rec, traffic_note = (None, "measured for the benchmark shape only")
+    if (B, T, W, nb) == BENCH_SHAPE:
+        traffic_rec, traffic_note = measured_traffic()
     out = {
         "metric": "RG-LRU fwd+bwd tokens/s", "value": B * T / (ms_per_step * 1e-3), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": f"RG-LRU fwd+bwd B{B} T{T} W{W} nb{nb} bf16", "batch": B, "seq_len": T,
-                   "width": W, "gate_blocks": nb, "state_dtype": "f32", "launch": f"hip graph replay, {per_graph} steps per graph" if graph is not None else "eager"},
-        "roofline": {"bound": "hbm", "kernel": dominant, "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": traffic,
-                     "algorithmic_bytes": dom_bytes, "kernel_ms": dom_ms},
+                   "width": W, "gate_blocks": nb, "state_dtype": "f32", "launch": launch,
+                   "timed_regions": args.repeats, "ms_per_step_samples": samples},
+        "roofline": {"bound": "hbm", "scope": "whole fwd+bwd step (5 s N algorithmic bytes over ms_per_step)",
+                     "achieved": step_gbps, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": step_gbps / HBM_PEAK_GBS,
+                     "traffic": None if traffic_rec is None else traffic_rec["whole_step_bytes"],
+                     "traffic_source": traffic_note, "algorithmic_bytes": step_bytes},
+        "ms_per_step_same_buffers": ms_same,
         "kernels": {**{f"{k}_ms": v for k, v in avg_ms.items()},
+                    "dominant": dominant,
+                    "dominant_algorithmic_bytes": algo[dominant],
+                    "dominant_GBps": algo[dominant] / (avg_ms[dominant] * 1e-3) / 1e9,
+                    "dominant_frac_of_peak": algo[dominant] / (avg_ms[dominant] * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                    "traffic_bytes": None if traffic_rec is None else traffic_rec["kernels"],
                     "fwd_GBps": algo["fwd_kernel"] / (avg_ms["fwd_kernel"] * 1e-3) / 1e9,
-                    "bwd_GBps": algo["bwd_scan_kernel"] / ((avg_ms["bwd_scan_kernel"] + avg_ms["gate_grad_kernel"]) * 1e-3) / 1e9,
-                    "fwd_bwd_GBps_whole_step": step_gbps,
-                    "fwd_bwd_frac_of_peak_whole_step": step_gbps / HBM_PEAK_GBS,
                     # block-diagonal gate projections on MFMA: 4 W bw flops per token forward (and again
                     # in the backward scan's recomputation), twice that in the gradient GEMM kernel
                     "gate_gemm_TFLOPs_fwd": 4.0 * W * (W // nb) * B * T / (avg_ms["fwd_kernel"] * 1e-3) / 1e12,
                     "gate_gemm_TFLOPs_gate_grad": 8.0 * W * (W // nb) * B * T / (avg_ms["gate_grad_kernel"] * 1e-3) / 1e12},
     }
+    if graph_check is not None:
+        out.update(graph_check)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(case)
     print(json.dumps(out))
+    if graph_check is not None and not graph_check["graph_matches_eager"]:
+        print("bench.py: results of the captured step differ from an eager step", file=sys.stderr)
+        sys.exit(1)
 
 
 if __name__ == "__main__":

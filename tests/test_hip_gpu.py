@@ -237,6 +237,59 @@ def test_fused_matches_reference_golden_vectors(golden_dir, name):
         assert err < FP32_TOL, (key, err)
 
 
+# ------------------------------------------------------------------ capped derivative of the square root
+def test_saturated_gate_fixture_on_the_hip_path(golden_dir):
+    """The reference's own saturated-gate case (tests/test_rglru.py:61-75: Lambda = 20, b_a = -100, W_a = 0,
+    loss mean(y^2)), as written by the reference into the fixture: a = 1 and g = 0, so the output and every
+    gradient are exactly zero unless the capped derivative of griffin/griffin.py:48-65 overflows."""
+    from griffin_amd import hip_rglru
+
+    data = np.load(os.path.join(golden_dir, "rglru_saturated_b2_t8_w16.npz"))
+    d = {k: torch.from_numpy(data[k]) for k in data.files}
+    for dtype in (torch.float32, torch.bfloat16):
+        leaves = [t.to(dtype).cuda().requires_grad_(True) for t in
+                  (d["x"], torch.zeros(4, 4, 4), torch.full((4, 4), -100.0), d["w_x"], d["b_x"], torch.full((16,), 20.0))]
+        y, _ = hip_rglru(*leaves, 8.0)
+        y.float().square().mean().backward()
+        torch.cuda.synchronize()
+        _say("saturated fixture", dtype, "max |y| %.2e" % y.abs().max().item())
+        tol = 1e-6 if dtype == torch.float32 else 1e-3
+        torch.testing.assert_close(y.float().cpu(), d["y"], atol=tol, rtol=0)
+        torch.testing.assert_close(leaves[0].grad.float().cpu(), d["g_x"], atol=tol, rtol=0)
+        torch.testing.assert_close(leaves[5].grad.float().cpu(), d["g_lam"], atol=tol, rtol=0)
+        torch.testing.assert_close(leaves[2].grad.float().cpu(), d["g_b_a"], atol=tol, rtol=0)
+
+
+@pytest.mark.parametrize("dtype,shape", [(torch.float32, (2, 96, 256, 2)), (torch.bfloat16, (2, 96, 256, 2)),
+                                         (torch.bfloat16, (2, 70, 640, 2)), (torch.float32, (2, 40, 24, 3))])
+def test_capped_sqrt_derivative_regime_matches_oracle(dtype, shape):
+    """g^2 = 1 - a^2 on both sides of 2.5e-7, where the derivative of the square root stops growing
+    (griffin/griffin.py:48-65: grad / sqrt(clamp(4 g^2, 1e-6)), i.e. capped at 1000).  Lambda = 12 and
+    recurrence-gate pre-activations around -5 put 1 - a^2 between 1e-8 and 1e-4; every kernel family is
+    covered (portable fp32, register-held bf16 weights, wide blocks)."""
+    B, T, W, nb = shape
+    case = orc.make_case(B, T, W, nb, seed=21)
+    case["lam"] = torch.full((W,), 12.0)
+    case["w_a"] = 2.5 * case["w_a"]
+    case["b_a"] = torch.full_like(case["b_a"], -5.0)
+    p = [case[k].to(dtype).float() for k in PARAMS]
+    gates = orc.gate_math(*p)
+    g2 = gates.g.double() ** 2
+    below = (g2 < 2.5e-7).double().mean().item()
+    _say("capped sqrt regime", dtype, shape, "fraction below the cap threshold %.2f" % below)
+    assert 0.15 < below < 0.85                                 # the case does straddle the threshold
+    y, h_last, grads = hip_run(case, dtype)
+    ry, rh, rgrads = oracle_run(case, dtype)
+    _, _, g64 = oracle_run(case, torch.float64) if dtype == torch.float32 else (None, None, rgrads)
+    errs = {"y": rel_err(y.float(), ry), "h_last": rel_err(h_last, rh)}
+    for name in grads:
+        errs[name] = min(rel_err(grads[name].float(), rgrads[name]), rel_err(grads[name].float(), g64[name]))
+    _say("  rel errors:", {k: "%.2e" % v for k, v in errs.items()})
+    tol = FP32_TOL if dtype == torch.float32 else BF16_TOL
+    for name, err in errs.items():
+        assert err < tol, (name, err)
+
+
 # ------------------------------------------------------------------ decode step
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, FP32_TOL), (torch.bfloat16, BF16_TOL)])
 def test_step_kernel_matches_oracle(dtype, tol):

@@ -343,6 +343,49 @@ def test_config5_recurrent_block_with_hip_scan():
     assert torch.isfinite(nxt).all()
 
 
+def test_config5_recurrent_block_bf16_matches_fp32_oracle():
+    """Config 5 at its stated storage type: RMSNorm(768) + RecurrentBlock(768, 1024), 8 gate blocks, bf16
+    parameters and activations on the HIP kernels, T = 2048, against the oracle's block
+    (griffin/griffin.py:68-80, 439-529) in fp32 on the same bf16-rounded parameters and inputs, forward
+    and every gradient.  Two sequences instead of eight keep the CPU side to a few seconds; nothing in
+    the block couples sequences."""
+    from griffin_amd import RMSNorm, RecurrentBlock
+
+    torch.manual_seed(9)
+    B, T, D, W = 2, 2048, 768, 1024
+    block = RecurrentBlock(D, W, gate_blocks=8, scan_mode="hip").to(torch.bfloat16)
+    norm = RMSNorm(D)
+    with torch.no_grad():
+        norm.g.copy_(0.1 * torch.randn(D))
+        block.rg_lru.recurrence_gate.bias.copy_(0.3 * torch.randn(8, W // 8))
+        block.rg_lru.input_gate.bias.copy_(0.3 * torch.randn(8, W // 8))
+    norm = norm.to(torch.bfloat16)
+    x = torch.randn(B, T, D).to(torch.bfloat16)
+    up = torch.randn(B, T, D).to(torch.bfloat16)
+
+    # oracle, fp32, on the rounded values
+    p = {k: v.clone().requires_grad_(True) for k, v in _block_params(block).items()}
+    g = norm.g.detach().float().clone().requires_grad_(True)
+    xr = x.float().requires_grad_(True)
+    want, _ = orc.recurrent_block_forward(orc.rmsnorm(xr, g), p)
+    names = list(p)
+    want_grads = torch.autograd.grad(want, [xr, g] + [p[k] for k in names], up.float())
+
+    hip_block, hip_norm = block.cuda(), norm.cuda()
+    xh = x.cuda().requires_grad_(True)
+    got = hip_block(hip_norm(xh))
+    got.backward(up.cuda())
+    torch.cuda.synchronize()
+    mine = _block_params_grads(hip_block)
+    errs = {"out": rel_err(got.float(), want), "x": rel_err(xh.grad.float(), want_grads[0]),
+            "norm.g": rel_err(hip_norm.g.grad.float(), want_grads[1])}
+    for name, ref in zip(names, want_grads[2:]):
+        errs[name] = rel_err(mine[name], ref)
+    _say("config 5 bf16 rel errors:", {k: "%.2e" % v for k, v in errs.items()})
+    for name, err in errs.items():
+        assert err < BF16_TOL, (name, err)
+
+
 # ------------------------------------------------------------------ failure handling
 def test_bounded_wait_gives_up_instead_of_hanging():
     """With the poll budget forced to one, waves that do not find their carry at once record the
@@ -397,6 +440,16 @@ def _block_params(block):
             "w_a": sd["rg_lru.recurrence_gate.weight"], "b_a": sd["rg_lru.recurrence_gate.bias"],
             "w_x": sd["rg_lru.input_gate.weight"], "b_x": sd["rg_lru.input_gate.bias"], "lam": sd["rg_lru.Lambda"],
             "lo_w": sd["linear_out.weight"], "lo_b": sd["linear_out.bias"]}
+
+
+def _block_params_grads(block):
+    """Gradients of a RecurrentBlock's parameters in the oracle's naming, fp32 on the CPU."""
+    gd = {k: v.grad.detach().float().cpu() for k, v in block.named_parameters()}
+    return {"lx_w": gd["linear_x.weight"], "lx_b": gd["linear_x.bias"], "ly_w": gd["linear_y.weight"],
+            "ly_b": gd["linear_y.bias"], "conv_w": gd["temporal_conv.weight"][:, 0, :], "conv_b": gd["temporal_conv.bias"],
+            "w_a": gd["rg_lru.recurrence_gate.weight"], "b_a": gd["rg_lru.recurrence_gate.bias"],
+            "w_x": gd["rg_lru.input_gate.weight"], "b_x": gd["rg_lru.input_gate.bias"], "lam": gd["rg_lru.Lambda"],
+            "lo_w": gd["linear_out.weight"], "lo_b": gd["linear_out.bias"]}
 
 
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, FP32_TOL), (torch.bfloat16, BF16_TOL)])
