@@ -14,7 +14,7 @@ RGLRU_BF16 = 1
 FLAG_RESET = 1
 FLAG_INACTIVE = 2
 CHUNK = 32
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 _lock = threading.Lock()
 _lib = None
@@ -34,6 +34,8 @@ _SIGNATURES = {
     "rglru_hip_workspace_bytes": (ctypes.c_size_t, [_I, _I, _I, _I]),
     "rglru_hip_bwd_scratch_bytes": (ctypes.c_size_t, [_I, _I, _I, _I, ctypes.c_int]),
     "rglru_hip_fwd": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, ctypes.c_int, _P]),
+    "rglru_hip_static_workspace_bytes": (ctypes.c_size_t, []),
+    "rglru_hip_fwd_static": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, ctypes.c_int, _P]),
     "rglru_hip_prepare_fwd": (ctypes.c_int, [_P, _P, _P, _P, _P, ctypes.c_float, ctypes.c_int, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, ctypes.c_int, _P]),
     "rglru_hip_bwd": (ctypes.c_int, [_P] * 15 + [_I, _I, _I, _I, ctypes.c_int, ctypes.c_int, _P]),
     "rglru_hip_fast_path": (ctypes.c_int, [_I, _I, ctypes.c_int]),

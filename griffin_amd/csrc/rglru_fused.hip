@@ -1707,6 +1707,40 @@ int rglru_hip_fwd(const void* x, const void* prep, const float* h0, const uint8_
   return fwd_impl(x, prep, h0, flags, y, h_last, ws, B, T, W, nb, dtype, false, stream);
 }
 
+// Forward pass for callers that cannot allocate: the workspace is a file-scope device array of this
+// library.  Every device holds its own copy of the array at its own address; the name `static_scratch`
+// is only a handle in host code, the address comes from hipGetSymbolAddress, once per device.
+static __device__ __align__(256) unsigned char static_scratch[RGLRU_STATIC_WORKSPACE_BYTES];
+
+static void* static_scratch_address() {
+  static std::atomic<void*> cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) { fail(RGLRU_E_LAUNCH, "fwd_static: no current device"); return nullptr; }
+  void* ptr = cached[dev].load(std::memory_order_acquire);
+  if (ptr) return ptr;
+  const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(static_scratch));
+  if (e != hipSuccess || !ptr) { fail(RGLRU_E_LAUNCH, "fwd_static: hipGetSymbolAddress: %s", hipGetErrorString(e)); return nullptr; }
+  cached[dev].store(ptr, std::memory_order_release);     // racing first calls store the same address
+  return ptr;
+}
+
+size_t rglru_hip_static_workspace_bytes(void) { return (size_t)RGLRU_STATIC_WORKSPACE_BYTES; }
+
+int rglru_hip_fwd_static(const void* x, const void* prep, const float* h0, const uint8_t* flags,
+                         void* y, float* h_last,
+                         int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, void* stream) {
+  int rc = check_geometry("fwd_static", W, nb, dtype);
+  if (rc) return rc;
+  if (B <= 0 || T <= 0) return fail(RGLRU_E_ARG, "fwd_static: B and T must be positive (got %lld, %lld)", (long long)B, (long long)T);
+  const size_t need = make_work_layout(B, T, make_geometry(W, nb)).total;
+  if (need > (size_t)RGLRU_STATIC_WORKSPACE_BYTES)
+    return fail(RGLRU_E_UNSUPPORTED, "fwd_static: B=%lld T=%lld W=%lld needs a workspace of %zu bytes, the built-in one holds %zu; use rglru_hip_fwd with a caller-provided workspace",
+                (long long)B, (long long)T, (long long)W, need, (size_t)RGLRU_STATIC_WORKSPACE_BYTES);
+  void* ws = static_scratch_address();
+  if (!ws) return RGLRU_E_LAUNCH;
+  return fwd_impl(x, prep, h0, flags, y, h_last, ws, B, T, W, nb, dtype, false, stream);
+}
+
 static int check_grad_dtype(const char* who, int grad_dtype);
 
 int rglru_hip_pre_path(int64_t W, int64_t nb, int dtype) {

@@ -46,7 +46,7 @@
 extern "C" {
 #endif
 
-#define RGLRU_ABI_VERSION 8
+#define RGLRU_ABI_VERSION 9
 
 enum { RGLRU_F32 = 0, RGLRU_BF16 = 1 };
 
@@ -110,6 +110,21 @@ size_t rglru_hip_bwd_scratch_bytes(int64_t B, int64_t T, int64_t W, int64_t nb, 
 int rglru_hip_fwd(const void* x, const void* prep, const float* h0, const uint8_t* flags,
                   void* y, float* h_last, void* ws,
                   int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, void* stream);
+
+/* rglru_hip_fwd without a workspace argument and without any allocation.  It has no counterpart in
+ * the reference: it exists for callers that cannot allocate device memory around the call -- code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc -- and want the
+ * forward pass (inference: prefill of a prompt, T > 1) only.  The workspace is a device array built
+ * into the library, RGLRU_STATIC_WORKSPACE_BYTES per GPU, held until the process ends; shapes whose
+ * rglru_hip_workspace_bytes() exceed it are rejected with RGLRU_E_UNSUPPORTED.  All calls on one GPU
+ * share that array: calls that overlap in time on one GPU (different streams, different threads)
+ * race and give wrong results; calls on one stream are safe.  Nothing of a call survives in it, so
+ * there is no backward pass for this entry point.  Same results as rglru_hip_fwd. */
+#define RGLRU_STATIC_WORKSPACE_BYTES (16u << 20)
+size_t rglru_hip_static_workspace_bytes(void);
+int rglru_hip_fwd_static(const void* x, const void* prep, const float* h0, const uint8_t* flags,
+                         void* y, float* h_last,
+                         int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, void* stream);
 
 /* rglru_hip_prepare followed by rglru_hip_fwd on the same stream with one launch fewer: the
  * parameter conversion and the clearing of the workspace share a kernel.  For training, where
