@@ -202,7 +202,7 @@ def measured_traffic():
     return None, "no traffic summary under profiles/"
 
 
-KERNEL_SLOTS = {"fwd_kernel": 0, "bwd_scan_kernel": 1, "gate_grad_kernel": 3}
+KERNEL_SLOTS = {"fwd_kernel": 0, "bwd_delta_kernel": 1, "bwd_grad_kernel": 3}
 
 
 def main():
@@ -345,7 +345,9 @@ def main():
     n = B * T * W
     elem = 2
     step_bytes = 5 * elem * n
-    algo = {"fwd_kernel": 2 * elem * n, "bwd_scan_kernel": 3 * elem * n, "gate_grad_kernel": 0}
+    # per kernel: forward x -> y; reverse scan x, dy -> (delta, not compulsory); gradients x -> dx
+    # (delta and y are re-reads the split costs)
+    algo = {"fwd_kernel": 2 * elem * n, "bwd_delta_kernel": 2 * elem * n, "bwd_grad_kernel": 2 * elem * n}
     dominant = max(avg_ms, key=avg_ms.get)
     step_gbps = step_bytes / (ms_per_step * 1e-3) / 1e9
     traffic_rec, traffic_note = (None, "measured for the benchmark shape only")
@@ -371,10 +373,10 @@ def main():
                     "dominant_frac_of_peak": algo[dominant] / (avg_ms[dominant] * 1e-3) / 1e9 / HBM_PEAK_GBS,
                     "traffic_bytes": None if traffic_rec is None else traffic_rec["kernels"],
                     "fwd_GBps": algo["fwd_kernel"] / (avg_ms["fwd_kernel"] * 1e-3) / 1e9,
-                    # block-diagonal gate projections on MFMA: 4 W bw flops per token forward (and again
-                    # in the backward scan's recomputation), twice that in the gradient GEMM kernel
+                    # block-diagonal gate projections on MFMA: 4 W bw flops per token forward; the gradient
+                    # kernel recomputes them and adds the input- and weight-gradient products (8 W bw)
                     "gate_gemm_TFLOPs_fwd": 4.0 * W * (W // nb) * B * T / (avg_ms["fwd_kernel"] * 1e-3) / 1e12,
-                    "gate_gemm_TFLOPs_gate_grad": 8.0 * W * (W // nb) * B * T / (avg_ms["gate_grad_kernel"] * 1e-3) / 1e12},
+                    "gate_gemm_TFLOPs_bwd_grad": 12.0 * W * (W // nb) * B * T / (avg_ms["bwd_grad_kernel"] * 1e-3) / 1e12},
     }
     if graph_check is not None:
         out.update(graph_check)

@@ -198,11 +198,17 @@ struct CarryWalk {
   int p;              // next chunk to consume
 };
 
+// DEPTH = records requested per round trip.  Chunks of one chain that are in flight at the same time
+// publish their maps at about the same moment, so a walk has to cross all of them before it meets a
+// final record: the depth should be near the number of workgroups that work on one chain at once (two
+// suits the kernels that are short of registers, eight the light ones that run many waves).
+
 // Compose one batch of records (chunks p, p + step, ...) into the walk.  Returns true when the
 // batch ran into a record that is not published yet; p then names that chunk.
-RGLRU_DEVICE bool carry_compose(const rec_t (&rec)[kDepth], CarryWalk& wk, int step, int end, float boundary) {
+template <int DEPTH>
+RGLRU_DEVICE bool carry_compose(const rec_t (&rec)[DEPTH], CarryWalk& wk, int step, int end, float boundary) {
 #pragma unroll
-  for (int d = 0; d < kDepth; ++d) {
+  for (int d = 0; d < DEPTH; ++d) {
     const int q = wk.p + d * step;
     if (q == end) {                                      // wave-uniform
       if (!wk.done) { wk.acc_h = fmaf(wk.acc_a, boundary, wk.acc_h); wk.acc_a = 0.f; wk.done = true; }
@@ -216,7 +222,7 @@ RGLRU_DEVICE bool carry_compose(const rec_t (&rec)[kDepth], CarryWalk& wk, int s
       else wk.acc_a *= __uint_as_float(lo);
     }
   }
-  wk.p += kDepth * step;
+  wk.p += DEPTH * step;
   return false;
 }
 
@@ -225,19 +231,20 @@ RGLRU_DEVICE bool carry_compose(const rec_t (&rec)[kDepth], CarryWalk& wk, int s
 // are still waiting, so every wave still reaches the end of the kernel and the failure is visible in
 // the results themselves (the chunk's outputs and the carry it hands on turn NaN) without anybody
 // having to read the failure word.
+template <int DEPTH>
 RGLRU_DEVICE float carry_walk(const CarryChain& ch, CarryWalk& wk, int step, int end, float boundary,
                               long long limit, unsigned* fail_word) {
   long long polls = 0;
   while (!__all(wk.done)) {
-    rec_t rec[kDepth];
+    rec_t rec[DEPTH];
 #pragma unroll
-    for (int d = 0; d < kDepth; ++d) {
+    for (int d = 0; d < DEPTH; ++d) {
       const int q = wk.p + d * step;
       const bool inside = (step < 0) ? (q > end) : (q < end);
       rec[d] = 0;
       if (inside && !wk.done) rec[d] = rec_load(ch.rec + q * ch.stride);
     }
-    if (carry_compose(rec, wk, step, end, boundary)) {
+    if (carry_compose<DEPTH>(rec, wk, step, end, boundary)) {
       if (++polls > limit) {
         if ((threadIdx.x & 63) == 0) atomicOr(fail_word, 1u);
         if (!wk.done) wk.acc_h = __builtin_nanf("");
@@ -252,11 +259,12 @@ RGLRU_DEVICE float carry_walk(const CarryChain& ch, CarryWalk& wk, int step, int
 // carry_in of chunk c.  `step` is -1 when the chain runs forward in time (the chunk before c is
 // c - 1) and +1 when it runs backward; `end` is the index one past the first chunk of the chain
 // (-1 or the chunk count), where `boundary` is the carry.
+template <int DEPTH = kDepth>
 RGLRU_DEVICE float carry_lookback(const CarryChain& ch, int c, int step, int end, float boundary,
                                   bool lane_ok, long long limit, unsigned* fail_word) {
   CarryWalk wk;
   wk.acc_a = 1.f; wk.acc_h = 0.f; wk.done = !lane_ok; wk.p = c + step;
-  return carry_walk(ch, wk, step, end, boundary, limit, fail_word);
+  return carry_walk<DEPTH>(ch, wk, step, end, boundary, limit, fail_word);
 }
 
 // The first batch of a walk requested ahead of time.  A device-scope load takes a few
@@ -266,8 +274,9 @@ RGLRU_DEVICE float carry_lookback(const CarryChain& ch, int c, int step, int end
 // of the lane's channel, or kOutOfRange for a lane without one): chunks outside the chain are
 // masked by the offset instead of a branch, so the number of loads in flight is fixed and the
 // hardware counter can be waited on precisely.
+template <int DEPTH = kDepth>
 struct CarryBatch {
-  rec_t rec[kDepth];
+  rec_t rec[DEPTH];
 };
 
 // Record store through the same kind of descriptor; voff = kOutOfRange drops it.
@@ -278,11 +287,12 @@ RGLRU_DEVICE void rec_store_buf(rsrc_t recs, unsigned voff, float a, float h) {
   __builtin_amdgcn_raw_buffer_store_b64(v, recs, voff, 0, kRecPolicy);
 }
 
+template <int DEPTH>
 RGLRU_DEVICE void carry_prefetch(rsrc_t recs, unsigned lane_off, unsigned stride_bytes, int c, int step, int end,
-                                 CarryBatch& batch) {
+                                 CarryBatch<DEPTH>& batch) {
   typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 #pragma unroll
-  for (int d = 0; d < kDepth; ++d) {
+  for (int d = 0; d < DEPTH; ++d) {
     const int q = c + step + d * step;
     const bool inside = (step < 0) ? (q > end) : (q < end);
     const unsigned voff = (inside && lane_off != kOutOfRange) ? (unsigned)q * stride_bytes + lane_off : kOutOfRange;
@@ -291,12 +301,13 @@ RGLRU_DEVICE void carry_prefetch(rsrc_t recs, unsigned lane_off, unsigned stride
   }
 }
 
-RGLRU_DEVICE float carry_lookback_from(const CarryBatch& first, const CarryChain& ch, int c, int step, int end,
+template <int DEPTH>
+RGLRU_DEVICE float carry_lookback_from(const CarryBatch<DEPTH>& first, const CarryChain& ch, int c, int step, int end,
                                        float boundary, bool lane_ok, long long limit, unsigned* fail_word) {
   CarryWalk wk;
   wk.acc_a = 1.f; wk.acc_h = 0.f; wk.done = !lane_ok; wk.p = c + step;
-  carry_compose(first.rec, wk, step, end, boundary);
-  return carry_walk(ch, wk, step, end, boundary, limit, fail_word);
+  carry_compose<DEPTH>(first.rec, wk, step, end, boundary);
+  return carry_walk<DEPTH>(ch, wk, step, end, boundary, limit, fail_word);
 }
 
 // ------------------------------------------------------------------------------------------

@@ -16,6 +16,7 @@
 #include <hip/hip_runtime.h>
 
 #include <cstring>
+#include <type_traits>
 
 #include "rglru_device.h"
 #include "rglru_host.h"
@@ -362,6 +363,12 @@ RGLRU_DEVICE void fwd_gates(unsigned flbits, const f32x16& ua, const f32x16& ux,
   }
 }
 
+// records a forward walk requests per round trip (see carry_compose)
+#ifndef RGLRU_FWD_DEPTH
+#define RGLRU_FWD_DEPTH 2
+#endif
+constexpr int kFwdDepth = RGLRU_FWD_DEPTH;
+
 // One wave's tile of 32 * MT tokens between its two stages: gate outputs in time order, the affine
 // maps of the lower lane run and of the whole tile, and where the tile sits.
 template <int MT>
@@ -398,7 +405,7 @@ RGLRU_DEVICE void fwd_local(const FusedArgs& p, const WaveId& w, FwdTile<MT>& t,
 // Stage 2: carry in, carry out and checkpoint, then the recurrence itself and the stores.
 template <typename IO, int MT, bool MASKED, bool STAGED>
 RGLRU_DEVICE void fwd_finalize(const FusedArgs& p, const WaveId& w, const FwdTile<MT>& t, unsigned char* stage,
-                               const CarryBatch* first = nullptr, bool live = true) {
+                               const CarryBatch<kFwdDepth>* first = nullptr, bool live = true) {
   constexpr int EL = 16 * MT, TR = 32 * MT;
   const int hf = w.hf, b = t.b, c = t.c;
   const long long W = p.W;
@@ -409,8 +416,8 @@ RGLRU_DEVICE void fwd_finalize(const FusedArgs& p, const WaveId& w, const FwdTil
 
   float h_in = 0.f;
   if (c != 0) {
-    h_in = first ? carry_lookback_from(*first, chain, c, -1, -1, 0.f, ch_ok, p.limit, p.fail)
-                 : carry_lookback(chain, c, -1, -1, 0.f, ch_ok, p.limit, p.fail);
+    h_in = first ? carry_lookback_from<kFwdDepth>(*first, chain, c, -1, -1, 0.f, ch_ok, p.limit, p.fail)
+                 : carry_lookback<kFwdDepth>(chain, c, -1, -1, 0.f, ch_ok, p.limit, p.fail);
   } else if (p.h0 && ch_ok) {
     h_in = p.h0[(long long)b * W + w.ch];
   }
@@ -576,8 +583,8 @@ __global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : (NKG == 4 ||
       // next ticket: one instruction for the whole workgroup, live only in its first lane
       const unsigned next_raw = (unsigned)__builtin_amdgcn_raw_ptr_buffer_atomic_add_i32(1, rticket, tid == 0 ? 0u : kOutOfRange, 0, 0);
       // records this tile will need: requested now, used after its gate math
-      CarryBatch ahead;
-      carry_prefetch(make_rsrc(p.rec_a + (long long)cur.b * p.nCf * W, (unsigned)p.nCf * rec_stride), rec_lane,
+      CarryBatch<kFwdDepth> ahead;
+      carry_prefetch<kFwdDepth>(make_rsrc(p.rec_a + (long long)cur.b * p.nCf * W, (unsigned)p.nCf * rec_stride), rec_lane,
                        rec_stride, cur.c, -1, -1, ahead);
 #pragma unroll
       for (int i = 0; i < NV; ++i) {
@@ -1117,208 +1124,477 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
 }
 
 // ------------------------------------------------------------------------------------------
-// Fast backward, part 2: the two block-diagonal GEMMs of the gate gradients,
-//     dx[n, j]   += sum_kappa du2[n, kappa] * w2t[j, kappa]          (kappa = 2 * o + gate)
-//     dW2T[j, kappa] = sum_n x[n, j] * du2[n, kappa]
-// over the flattened token axis n = b * T + t, one gate block per workgroup, 32 tokens per tile.
-// Each wave owns a 32-column slab j of the block: it keeps its w2t rows (the B operand of the first
-// GEMM) and its 32 x 2*bw slice of dW2T (the accumulator of the second) in registers for the whole
-// launch.  The second GEMM contracts over tokens, so both operands are needed with tokens running
-// along a lane's vector; tiles arrive token-major, and the transposition is done by the matrix
-// unit itself: multiplying a tile by the identity returns it in accumulator layout, where a lane
-// holds 16 consecutive tokens of one column.
+// Fast backward in two kernels that split the work along its one sequential dependency.
+//
+//   bwd_delta_kernel   the reverse scan  delta_t = dy_t + a_{t+1} delta_{t+1}  (and dh0 = a_0 delta_0).
+//                      It recomputes only the decay a_t (the recurrence gate: half of the gate
+//                      products, one sigmoid, one exp2 per element), runs the chunked scan with the
+//                      carry protocol in the reverse direction and writes delta in the storage type.
+//   bwd_grad_kernel    everything else, which has no dependency between tokens once delta is known:
+//                      both gates again, the gradient at every element, and the two block-diagonal
+//                      GEMMs (input gradient and weight gradients) straight from registers and LDS,
+//                      so the gradients at the gate pre-activations never leave the chip.  The state
+//                      in front of a token, h_{t-1}, is the forward output y_{t-1} as stored.
+//
+// The scan kernel is light (few registers, many waves per SIMD hide the look-back); the heavy
+// kernel has no chains, no tickets and no carries, so its tiles are known in advance and can be
+// prefetched, and its weight-gradient accumulators are shared by the eight waves of a workgroup.
 // ------------------------------------------------------------------------------------------
-constexpr int kGradWaves = 8;                            // waves per workgroup of the gradient GEMM kernel
+#ifndef RGLRU_DELTA_DEPTH
+#define RGLRU_DELTA_DEPTH 8
+#endif
+constexpr int kDeltaDepth = RGLRU_DELTA_DEPTH;         // records a walk of the reverse scan requests per round trip
+
+template <typename IO, int NKG, bool MASKED, int MT>
+__global__ __launch_bounds__(kThreads, (MT == 1 ? 4 : 2)) void bwd_delta_kernel(FusedArgs p) {
+  constexpr int TR = 32 * MT, EL = 16 * MT;
+  typedef Io<IO> Tr;
+  typedef typename Tr::Frag Frag;
+  constexpr int TW = kPackedWidth;                       // tile width (narrow blocks are packed)
+  constexpr int LDSROW = TW + Tr::HW;
+  static_assert(sizeof(IO) == 2 && NKG > 0, "fast backward is for 16-bit storage and register-held weights");
+  __shared__ __attribute__((aligned(16))) IO lds_x[TR * LDSROW];
+  __shared__ __attribute__((aligned(16))) IO lds_dy[TR * LDSROW];
+  __shared__ __attribute__((aligned(16))) unsigned char stage_all[kWaves * WaveStage<TR>::kBytes];
+  __shared__ unsigned s_ticket[2];
+
+  const WaveId w = wave_identity(p, blockIdx.x);
+  const int hf = w.hf, tid = threadIdx.x;
+  unsigned char* stage = stage_all + w.wave * WaveStage<TR>::kBytes;
+  const IO* wg = (const IO*)p.wg;
+  const IO* w_a_row = wg + ((long long)(0 * p.nb + w.k) * p.bwp + (w.slab_ok ? w.o : 0)) * p.bwp + hf * Tr::HW;
+  Frag wa[NKG];
+#pragma unroll
+  for (int kg = 0; kg < NKG; ++kg) wa[kg] = *reinterpret_cast<const Frag*>(w_a_row + kg * Tr::KG);
+  const float nba = -kLog2e * p.bias[w.kp];
+  const float sp = p.sp[w.kp];
+  const IO* x = (const IO*)p.x;
+  const IO* dy = (const IO*)p.dy;
+  const long long W = p.W;
+  const unsigned row_bytes = (unsigned)p.W * 2u;
+  const int nCk = (p.T + TR - 1) / TR;                   // chunks of this kernel's tile length
+  const Queue q = make_queue(p, w.unit, w.wg_in_unit, nCk);
+  const int kb = NKG == 8 ? 0 : w.kb;
+
+  constexpr int VPR = TW / Tr::HW;
+  constexpr int NV = (TR * VPR + kThreads - 1) / kThreads;
+  Frag pre_x[NV], pre_dy[NV];
+  unsigned pre_off[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int idx = tid + i * kThreads;
+    const int row = idx / VPR, cv = idx - row * VPR;
+    pre_off[i] = (idx < TR * VPR) ? (unsigned)row * row_bytes + (unsigned)(w.tile_col + cv * Tr::HW) * 2u : kOutOfRange;
+  }
+  auto decode = [&](unsigned tk, int& c, int& b) {
+    const unsigned cr = tk / (unsigned)q.n_b;
+    c = nCk - 1 - (int)cr;
+    b = q.first_b + (int)(tk - cr * (unsigned)q.n_b) * p.queues;
+  };
+  auto issue = [&](unsigned tk) {
+    // a ticket past the end keeps valid addresses (tile 0) but an empty extent: nothing is fetched
+    const bool live = (long long)tk < q.tiles;
+    int c, b;
+    decode(live ? tk : 0u, c, b);
+    const int rows = !live ? 0 : ((p.T - c * TR) < TR ? (p.T - c * TR) : TR);
+    const long long first = ((long long)b * p.T + (long long)c * TR) * W;
+    const rsrc_t rx = make_rsrc(x + first, (unsigned)rows * row_bytes);
+    const rsrc_t rdy = make_rsrc(dy + first, (unsigned)rows * row_bytes);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) { pre_x[i] = buf_load_frag<Frag>(rx, pre_off[i]); pre_dy[i] = buf_load_frag<Frag>(rdy, pre_off[i]); }
+  };
+
+  if (tid == 0) s_ticket[0] = atomicAdd(q.counter, 1u);
+  __syncthreads();
+  unsigned tk = s_ticket[0];
+  int par = 0;
+  issue(tk);
+  while ((long long)tk < q.tiles) {
+    int c, b;
+    decode(tk, c, b);
+    const int t0 = c * TR;
+    const long long trow = (long long)b * p.T + t0 + hf * EL;
+    unsigned next_raw = 0;
+    if (tid == 0) next_raw = atomicAdd(q.counter, 1u);
+    unsigned flbits[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) flbits[mt] = MASKED ? flag_run(p, trow + 16 * mt, t0 + hf * EL + 16 * mt) : 0u;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int idx = tid + i * kThreads;
+      const int row = idx / VPR, cv = idx - row * VPR;
+      if (idx < TR * VPR) {
+        *reinterpret_cast<Frag*>(lds_x + row * LDSROW + cv * Tr::HW) = pre_x[i];
+        *reinterpret_cast<Frag*>(lds_dy + row * LDSROW + cv * Tr::HW) = pre_dy[i];
+      }
+    }
+    __syncthreads();
+    float a[EL], gy[EL];
+    if (w.slab_ok) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        f32x16 ua;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) ua[v] = 0.0f;          // the bias enters inside the sigmoid
+        const IO* xrow = lds_x + tile_row<MT>(mt, w.r) * LDSROW + kb + hf * Tr::HW;
+#pragma unroll
+        for (int kg = 0; kg < NKG; ++kg) Tr::mma(ua, *reinterpret_cast<const Frag*>(xrow + kg * Tr::KG), wa[kg]);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          float l2 = sigmoid_fast(ua[v], nba) * sp;
+          if constexpr (MASKED) l2 = masked_log2_decay_run(l2, flbits[mt], v);
+          a[16 * mt + v] = __builtin_amdgcn_exp2f(l2);
+          gy[16 * mt + v] = (float)lds_dy[(hf * EL + 16 * mt + v) * LDSROW + kb + w.slab * 32 + w.r];
+        }
+      }
+    }
+    if (tid == 0) s_ticket[par ^ 1] = next_raw;
+    __syncthreads();
+    par ^= 1;
+    const unsigned tk_next = s_ticket[par];
+    issue(tk_next);
+    if (!w.slab_ok) {                                    // a wave without a slab only helps with the loads
+      tk = tk_next;
+      continue;
+    }
+    // reverse affine map of this lane's run and of the chunk: carry_out = A carry_in + D
+    float A = 1.f, carry = 0.f;
+#pragma unroll
+    for (int e = EL - 1; e >= 0; --e) { const float d = gy[e] + carry; carry = a[e] * d; A *= a[e]; }
+    const float D = carry;
+    const float A_o = xhalf(A, hf), D_o = xhalf(D, hf);
+    const float A_lo = hf ? A_o : A, A_hi = hf ? A : A_o;
+    const float D_lo = hf ? D_o : D, D_hi = hf ? D : D_o;
+    const float A_t = A_lo * A_hi, D_t = fmaf(A_lo, D_hi, D_lo);
+
+    CarryChain chain;
+    chain.rec = p.rec_a + (long long)b * p.nC * W + w.ch; chain.stride = W;
+    const bool last_chunk = c == nCk - 1;
+    if (!last_chunk && hf == 0) carry_publish(chain, c, A_t, D_t, false);
+    float d_in = (last_chunk && p.dh_last) ? p.dh_last[(long long)b * W + w.ch] : 0.f;
+    if (!last_chunk) d_in = carry_lookback<kDeltaDepth>(chain, c, +1, nCk, 0.f, true, p.limit, p.fail);
+    const float d_out = fmaf(A_t, d_in, D_t);
+    if (hf == 0) carry_publish(chain, c, 0.f, d_out, true);
+    if (hf == 0 && c == 0 && p.dh0) p.dh0[(long long)b * W + w.ch] = d_out;
+
+    // delta of every token, through the wave's staging area, as 16-byte row segments
+    carry = hf ? d_in : fmaf(A_hi, d_in, D_hi);
+    unsigned char* my = stage + WaveStage<TR>::row_offset(hf * EL) + w.r * 2;
+#pragma unroll
+    for (int e = EL - 1; e >= 0; --e) {
+      const float d = gy[e] + carry;
+      carry = a[e] * d;
+      *reinterpret_cast<IO*>(my + e * WaveStage<TR>::kRowBytes) = (IO)d;
+    }
+    wave_lds_fence();
+    {
+      const int rows = (p.T - t0) < TR ? (p.T - t0) : TR;
+      const rsrc_t rd = make_rsrc((const IO*)p.du_a + ((long long)b * p.T + t0) * W, (unsigned)rows * row_bytes);
+      stage_flush<TR>(stage, rd, row_bytes, (unsigned)(w.k * p.bw + w.slab * 32) * 2u, w.lane);
+    }
+    wave_lds_fence();
+    tk = tk_next;
+  }
+}
+
+constexpr int kGradWaves = 8;                            // waves per workgroup of the gradient kernel
 constexpr int kGradThreads = 64 * kGradWaves;
 
-template <typename IO, int NKG>
-__global__ __launch_bounds__(kGradThreads, 1) void gate_grad_kernel(FusedArgs p) {
+// One workgroup = one unit (a 128-channel gate block, or two / four narrower ones), eight waves in two
+// roles, one wave of each role per SIMD.  A tile is 32 tokens of one sequence.
+//   element waves (0-3, one per 32-channel slab): gate products on the matrix unit with the weights in
+//     registers, then the gate math and the gradient at every element of the tile.  With the row
+//     permutation of tile_row() a lane's accumulator registers are 16 consecutive tokens of one
+//     channel, which is exactly the fragment layout of the weight-gradient product
+//     dW[j][o] = sum_t x[t][j] du[t][o] (contraction over tokens): the x values and the du values of a
+//     lane ARE its A and B fragments, no transposition needed.  They go to LDS together with the
+//     token-major du tile and the direct part of the input gradient.  The lane's x, delta and h
+//     values reach that layout through the matrix unit as well (tile times identity).
+//   product waves (4-7, one per slab): for the tile the element waves finished one iteration earlier,
+//     dx[t][j] = direct + sum_kappa du[t][kappa] w2t[j][kappa] for the slab's input channels j, and the
+//     weight gradients of the slab's output channels against all input channels of the block, both
+//     gates, accumulated in registers for the whole launch.  They also move the x tiles into LDS.
+// The element waves are bound by the vector unit, the product waves by the matrix unit and LDS, so
+// each SIMD overlaps the two; neither role needs more than 256 registers (weights in one, weight
+// gradient accumulators in the other).  Exchange buffers and the x tile are double-buffered: one
+// barrier per tile.
+template <typename IO, int NKG, bool MASKED>
+__global__ __launch_bounds__(kGradThreads, 1) void bwd_grad_kernel(FusedArgs p) {
   typedef Io<IO> Tr;
   typedef typename Tr::Frag Frag;
   static_assert(sizeof(IO) == 2 && NKG > 0, "16-bit storage only");
   constexpr int TR = 32;
   constexpr int KC = NKG * Tr::KG;                       // block width
-  constexpr int S = KC / 32;                             // slabs in the block
-  constexpr int BPU = 4 / S;                             // blocks per unit: narrow blocks share a workgroup (four slabs)
-  constexpr int UKC = KC * BPU, UK2 = 2 * UKC;           // width of the unit's x / dx tiles (128) and of its du2 tile (256)
-  constexpr int NKG2 = 2 * NKG;                          // K groups of the first GEMM (contraction over a block's 2 * KC kappa)
-  constexpr int NKT = 2 * S;                             // 32-wide kappa tiles of du2 per block
-  constexpr int NKT_U = UK2 / 32;                        // ... and per unit
-  constexpr int KT_HALF = (NKT + 1) / 2;                 // kappa tiles each half of the workgroup accumulates
-  constexpr int ROW_X = UKC + Tr::HW, ROW_DU = UK2 + Tr::HW, ROW_T = TR + Tr::HW;
-  __shared__ __attribute__((aligned(16))) IO lds_du[TR * ROW_DU];
-  __shared__ __attribute__((aligned(16))) IO lds_x[TR * ROW_X];
-  __shared__ __attribute__((aligned(16))) IO lds_dx[TR * ROW_X];
-  __shared__ __attribute__((aligned(16))) IO lds_dut[UK2 * ROW_T];         // du2 transposed: [kappa][token]
+  constexpr int S = KC / 32;                             // slabs per block
+  constexpr int BPU = 4 / S;                             // blocks per unit
+  constexpr int TW = kPackedWidth;                       // unit width
+  constexpr int NKG2 = 2 * NKG;                          // K groups of the input-gradient product (2 * KC kappa)
+  constexpr int ROW = TW + Tr::HW, ROW_DU = 2 * TW + Tr::HW;
+  __shared__ __attribute__((aligned(16))) IO lds_x[2][TR * ROW];        // x tiles of two consecutive iterations
+  __shared__ __attribute__((aligned(16))) IO lds_du[2][TR * ROW_DU];    // [token][2 * unit channel + gate]
+  __shared__ __attribute__((aligned(16))) float lds_dxd[2][4][16][64];  // direct input gradient [slab][register][lane]
+  __shared__ __attribute__((aligned(16))) Frag lds_xt[2][4][2][64];     // x fragments [slab][K group][lane]
+  __shared__ __attribute__((aligned(16))) Frag lds_dub[2][4][2][2][64]; // du fragments [slab][gate][K group][lane]
   __shared__ __attribute__((aligned(16))) unsigned char stage_all[4 * WaveStage<TR>::kBytes];
 
-  // Eight waves, two per SIMD: wave = 4 * half + slab.  Between the two barriers of a tile the lower
-  // half does the input-gradient GEMM of its slab and the stores, the upper half transposes du2;
-  // after the second barrier both halves accumulate their share of the kappa tiles of dW2T.
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, hf = lane >> 5;
-  const int slab = wave & 3, half = wave >> 2;
+  const int slab = wave & 3;
+  const bool element_role = wave < 4;
   const int units = (p.nb + BPU - 1) / BPU;
   const int unit = blockIdx.x % units, wg_in_unit = blockIdx.x / units, n_wg = gridDim.x / units;
-  const int blk = slab / S, sl = slab - blk * S;           // the wave's block inside the unit and its slab inside the block
+  const int blk = slab / S, sl = slab - blk * S;           // the wave's block inside the unit, its slab inside the block
   const bool slab_ok = unit * BPU + blk < p.nb;
   const int k = slab_ok ? unit * BPU + blk : p.nb - 1;
+  const int uo = slab * 32 + r;                            // channel inside the unit
+  const int unit_col = unit * TW;                          // first channel of the unit
+  const int ch = slab_ok ? unit_col + uo : 0;
+  const int kb = blk * KC;
   unsigned char* stage = stage_all + slab * WaveStage<TR>::kBytes;
-  const long long rows_total = (long long)p.B * p.T;
-  const long long n_tiles = (rows_total + TR - 1) / TR;
+  const long long W = p.W;
   const unsigned row_bytes = (unsigned)p.W * 2u;
+  const int nC = (p.T + TR - 1) / TR;
+  const int n_tiles = p.B * nC;                            // tiles of the unit; the workgroup takes wg_in_unit, + n_wg, ...
 
-  // lower half: this wave's rows of w2t, B operand of the first GEMM; lane (n = j, hf) holds
-  // kappa = 16 kg + 8 hf + i
-  Frag w2[NKG2];
-  if (half == 0) {
-    const IO* row = (const IO*)p.w2t + ((long long)k * p.bwp + sl * 32 + r) * (2 * p.bwp) + hf * Tr::HW;
-#pragma unroll
-    for (int kg = 0; kg < NKG2; ++kg) w2[kg] = *reinterpret_cast<const Frag*>(row + kg * Tr::KG);
-  } else {
-#pragma unroll
-    for (int kg = 0; kg < NKG2; ++kg) w2[kg] = Tr::zero();
-  }
-  // identity fragments: element i of ident[q] is 1 where 16 q + 8 hf + i == r
-  Frag ident[2];
-#pragma unroll
-  for (int qd = 0; qd < 2; ++qd)
-#pragma unroll
-    for (int i = 0; i < Tr::HW; ++i) ident[qd][i] = (IO)((16 * qd + 8 * hf + i == r) ? 1.0f : 0.0f);
-
-  f32x16 dw[KT_HALF];                                    // kappa tiles half * KT_HALF + i of this wave's slab
-#pragma unroll
-  for (int kt = 0; kt < KT_HALF; ++kt)
-#pragma unroll
-    for (int v = 0; v < 16; ++v) dw[kt][v] = 0.f;
-
-  // cooperative tile loads: du2 (TR x K2), x and dx (TR x KC)
-  constexpr int VPR_DU = UK2 / Tr::HW, VPR_X = UKC / Tr::HW;
-  const int unit_col = unit * BPU * p.bw;                  // first channel of the unit
-  constexpr int NV_DU = (TR * VPR_DU + kGradThreads - 1) / kGradThreads, NV_X = (TR * VPR_X + kGradThreads - 1) / kGradThreads;
-  Frag pre_du[NV_DU], pre_x[NV_X], pre_dx[NV_X];
-  auto issue = [&](long long tile) {
-    // a tile past the end keeps valid addresses but an empty extent: nothing is fetched
-    const bool live = tile < n_tiles;
-    const long long row0 = live ? tile * TR : 0;
-    const int rows = !live ? 0 : (int)((rows_total - row0) < TR ? (rows_total - row0) : TR);
-    const rsrc_t rdu = make_rsrc((const IO*)p.du_a + row0 * 2 * p.W, (unsigned)rows * 2u * row_bytes);
-    const rsrc_t rx = make_rsrc((const IO*)p.x + row0 * p.W, (unsigned)rows * row_bytes);
-    const rsrc_t rdx = make_rsrc((const IO*)p.dx + row0 * p.W, (unsigned)rows * row_bytes);
-#pragma unroll
-    for (int i = 0; i < NV_DU; ++i) {
-      const int idx = tid + i * kGradThreads;
-      const int row = idx / VPR_DU, cv = idx - row * VPR_DU;
-      pre_du[i] = buf_load_frag<Frag>(rdu, idx < TR * VPR_DU ? (unsigned)row * 2u * row_bytes + (unsigned)(2 * unit_col + cv * Tr::HW) * 2u : kOutOfRange);
-    }
-#pragma unroll
-    for (int i = 0; i < NV_X; ++i) {
-      const int idx = tid + i * kGradThreads;
-      const int row = idx / VPR_X, cv = idx - row * VPR_X;
-      const unsigned off = idx < TR * VPR_X ? (unsigned)row * row_bytes + (unsigned)(unit_col + cv * Tr::HW) * 2u : kOutOfRange;
-      pre_x[i] = buf_load_frag<Frag>(rx, off);
-      pre_dx[i] = buf_load_frag<Frag>(rdx, off);
-    }
+  // Position of a tile, advanced by n_wg tiles at a time without divisions.
+  struct Place { int tile, b, c; };
+  const int step_b = n_wg / nC, step_c = n_wg - step_b * nC;
+  auto advance = [&](Place& q) {
+    q.tile += n_wg; q.b += step_b; q.c += step_c;
+    if (q.c >= nC) { q.c -= nC; q.b += 1; }
   };
+  Place first;
+  first.tile = wg_in_unit; first.b = wg_in_unit / nC; first.c = wg_in_unit - first.b * nC;
 
-  long long tile = wg_in_unit;
-  issue(tile);
-  for (; tile < n_tiles; tile += n_wg) {
-#pragma unroll
-    for (int i = 0; i < NV_DU; ++i) {
-      const int idx = tid + i * kGradThreads;
-      const int row = idx / VPR_DU, cv = idx - row * VPR_DU;
-      if (idx < TR * VPR_DU) *reinterpret_cast<Frag*>(lds_du + row * ROW_DU + cv * Tr::HW) = pre_du[i];
+  if (element_role) {
+    // ------------------------------------------------------------------ element waves
+    HeldWeights<IO, NKG> hw;
+    {
+      const IO* wg = (const IO*)p.wg;
+      const int o = sl * 32 + r;
+      hw.load(wg + ((long long)(0 * p.nb + k) * p.bwp + o) * p.bwp + hf * Tr::HW,
+              wg + ((long long)(1 * p.nb + k) * p.bwp + o) * p.bwp + hf * Tr::HW);
     }
+    const float nba = -kLog2e * p.bias[ch], nbx = -kLog2e * p.bias[p.Wp + ch];
+    const float sp = p.sp[ch], cs = p.cs[ch];
+    float sum_ba = 0.f, sum_bx = 0.f, sum_l = 0.f;
+    // The lane's x, delta and h_{t-1} values (16 consecutive tokens of its channel) come from the matrix
+    // unit: a 32 x 32 tile times the identity returns the tile in accumulator layout, which is that
+    // layout.  delta and y (shifted by one token) are loaded from memory directly as A fragments (row =
+    // token tile_row(r), 8 channels of the wave's slab each), so they never pass through LDS.
+    Frag ident[2];
 #pragma unroll
-    for (int i = 0; i < NV_X; ++i) {
-      const int idx = tid + i * kGradThreads;
-      const int row = idx / VPR_X, cv = idx - row * VPR_X;
-      if (idx < TR * VPR_X) {
-        *reinterpret_cast<Frag*>(lds_x + row * ROW_X + cv * Tr::HW) = pre_x[i];
-        *reinterpret_cast<Frag*>(lds_dx + row * ROW_X + cv * Tr::HW) = pre_dx[i];
+    for (int q = 0; q < 2; ++q)
+#pragma unroll
+      for (int i = 0; i < Tr::HW; ++i) ident[q][i] = (IO)((16 * q + 8 * hf + i == r) ? 1.0f : 0.0f);
+    Frag pre_d[2], pre_h[2];
+    const int my_row = tile_row<1>(0, r);
+    auto issue = [&](const Place& q) {
+      const bool live = q.tile < n_tiles;
+      const int b = live ? q.b : 0, c = live ? q.c : 0;
+      const int t0 = c * TR;
+      const int rows = !live ? 0 : ((p.T - t0) < TR ? (p.T - t0) : TR);
+      const rsrc_t rd = make_rsrc((const IO*)p.du_a + ((long long)b * p.T + t0) * W, (unsigned)rows * row_bytes);
+      // the state in front of token t is the output row t - 1; tile row i wants y row t0 - 1 + i.  The
+      // row in front of the sequence's first token does not exist (h0 takes its place further down).
+      const int shift = c == 0 ? 1 : 0;
+      const int y_first = t0 - 1 + shift;
+      const int y_rows = !live ? 0 : (t0 + rows - 1 - y_first);
+      const rsrc_t rh = make_rsrc((const IO*)p.y + ((long long)b * p.T + y_first) * W, (unsigned)(y_rows > 0 ? y_rows : 0) * row_bytes);
+#pragma unroll
+      for (int q2 = 0; q2 < 2; ++q2) {
+        const unsigned col = (unsigned)(unit_col + slab * 32 + q2 * Tr::KG + hf * Tr::HW) * 2u;
+        pre_d[q2] = buf_load_frag<Frag>(rd, (unsigned)my_row * row_bytes + col);
+        pre_h[q2] = buf_load_frag<Frag>(rh, my_row >= shift ? (unsigned)(my_row - shift) * row_bytes + col : kOutOfRange);
       }
-    }
-    __syncthreads();
-    issue(tile + n_wg);
+    };
+    Place at = first;
+    issue(at);
+    __syncthreads();                                     // x tile 0 is in LDS
+    for (int it = 0; at.tile < n_tiles + n_wg; ++it) {
+      const int cur = it & 1;
+      if (at.tile < n_tiles && slab_ok) {
+        const int b = at.b, c = at.c;
+        const int t0 = c * TR;
+        unsigned flbits = 0u;
+        if constexpr (MASKED) flbits = flag_run(p, (long long)b * p.T + t0 + hf * 16, t0 + hf * 16);
+        float h_first = 0.f;                             // h0 of the sequence, for the lane that owns token 0
+        if (c == 0 && hf == 0 && p.h0) h_first = p.h0[(long long)b * W + ch];
 
-    const long long row0 = tile * TR;
-    const IO* a_row_du = lds_du + tile_row<1>(0, r) * ROW_DU + hf * Tr::HW;
-    const IO* a_row_x = lds_x + tile_row<1>(0, r) * ROW_X + hf * Tr::HW;
-    // x of this wave's slab with tokens along the lane vector (A operand of the second GEMM)
-    Frag xt_lo = Tr::zero(), xt_hi = Tr::zero();
-    if (slab_ok) {
-      f32x16 xc;
+        const IO* tile_x = lds_x[cur];
+        f32x16 ua, ux, xc, dc, hc;
 #pragma unroll
-      for (int v = 0; v < 16; ++v) xc[v] = 0.f;
-      Tr::mma(xc, *reinterpret_cast<const Frag*>(a_row_x + (2 * slab) * Tr::KG), ident[0]);
-      Tr::mma(xc, *reinterpret_cast<const Frag*>(a_row_x + (2 * slab + 1) * Tr::KG), ident[1]);
+        for (int v = 0; v < 16; ++v) { ua[v] = 0.0f; ux[v] = 0.0f; xc[v] = 0.0f; dc[v] = 0.0f; hc[v] = 0.0f; }   // the biases enter inside the sigmoids
+        const IO* xrow = tile_x + my_row * ROW + hf * Tr::HW;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) { xt_lo[i] = (IO)xc[i]; xt_hi[i] = (IO)xc[8 + i]; }
-    }
-    if (half == 1) {
-      // transposes: the upper half's four waves share the kappa tiles of du2, written to lds_dut
-#pragma unroll
-      for (int h2 = 0; h2 < (NKT_U + 3) / 4; ++h2) {
-        const int kt = 4 * h2 + slab;
-        if (kt < NKT_U) {
-          f32x16 dc;
-#pragma unroll
-          for (int v = 0; v < 16; ++v) dc[v] = 0.f;
-          Tr::mma(dc, *reinterpret_cast<const Frag*>(a_row_du + (2 * kt) * Tr::KG), ident[0]);
-          Tr::mma(dc, *reinterpret_cast<const Frag*>(a_row_du + (2 * kt + 1) * Tr::KG), ident[1]);
-          Frag lo, hi;
-#pragma unroll
-          for (int i = 0; i < 8; ++i) { lo[i] = (IO)dc[i]; hi[i] = (IO)dc[8 + i]; }
-          IO* dst = lds_dut + (kt * 32 + r) * ROW_T + hf * 16;
-          *reinterpret_cast<Frag*>(dst) = lo;
-          *reinterpret_cast<Frag*>(dst + 8) = hi;
+        for (int q2 = 0; q2 < 2; ++q2) {
+          Tr::mma(dc, pre_d[q2], ident[q2]);
+          Tr::mma(hc, pre_h[q2], ident[q2]);
+          Tr::mma(xc, *reinterpret_cast<const Frag*>(xrow + slab * 32 + q2 * Tr::KG), ident[q2]);
         }
-      }
-    } else if (slab_ok) {
-      // first GEMM: dx tile = direct part + du2 . w2t^T, on two accumulators
-      f32x16 acc, acc_odd;
 #pragma unroll
-      for (int v = 0; v < 16; ++v) { acc[v] = (float)lds_dx[(hf * 16 + v) * ROW_X + slab * 32 + r]; acc_odd[v] = 0.f; }
-#pragma unroll
-      for (int kg = 0; kg < NKG2; kg += 2) {
-        Tr::mma(acc, *reinterpret_cast<const Frag*>(a_row_du + (blk * NKG2 + kg) * Tr::KG), w2[kg]);
-        Tr::mma(acc_odd, *reinterpret_cast<const Frag*>(a_row_du + (blk * NKG2 + kg + 1) * Tr::KG), w2[kg + 1]);
-      }
-      unsigned char* my = stage + WaveStage<TR>::row_offset(hf * 16) + r * 2;
-#pragma unroll
-      for (int v = 0; v < 16; ++v) *reinterpret_cast<IO*>(my + v * WaveStage<TR>::kRowBytes) = (IO)(acc[v] + acc_odd[v]);
-      wave_lds_fence();
-      const int rows = (int)((rows_total - row0) < TR ? (rows_total - row0) : TR);
-      const rsrc_t rdx = make_rsrc((const IO*)p.dx + row0 * p.W, (unsigned)rows * row_bytes);
-      stage_flush<TR>(stage, rdx, row_bytes, (unsigned)(unit_col + slab * 32) * 2u, lane);
-      wave_lds_fence();
-    }
-    __syncthreads();
-    if (slab_ok) {
-      // second GEMM: dW2T[j, kappa] += sum over the tile's tokens, this half's kappa tiles
-#pragma unroll
-      for (int i = 0; i < KT_HALF; ++i) {
-        const int kt = half * KT_HALF + i;
-        if (kt < NKT) {
-          const IO* b_row = lds_dut + ((blk * NKT + kt) * 32 + r) * ROW_T + hf * 16;
-          Tr::mma(dw[i], xt_lo, *reinterpret_cast<const Frag*>(b_row));
-          Tr::mma(dw[i], xt_hi, *reinterpret_cast<const Frag*>(b_row + 8));
+        for (int kg = 0; kg < NKG; ++kg) {
+          const Frag xa = *reinterpret_cast<const Frag*>(xrow + kb + kg * Tr::KG);
+          Tr::mma(ua, xa, hw.a[kg]);
+          Tr::mma(ux, xa, hw.x[kg]);
         }
-      }
-    }
-  }
-  // per-workgroup partial of dW2T: [wg][k][j][kappa]
-  if (slab_ok) {
-    float* part = p.dw_partial + (((long long)wg_in_unit * p.nb + k) * p.bwp) * (2 * p.bwp);
-#pragma unroll
-    for (int i = 0; i < KT_HALF; ++i) {
-      const int kt = half * KT_HALF + i;
-      if (kt < NKT) {
+        Place nxt = at;
+        advance(nxt);
+        issue(nxt);
+        if (c == 0 && hf == 0) hc[0] = h_first;
+
+        IO* du_tile = lds_du[cur];
+        Frag fx_t[2], fa[2], fx[2];                        // x, du_a, du_x of the lane's tokens, per K group
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-          const int j = sl * 32 + 8 * (v >> 2) + 4 * hf + (v & 3);
-          part[(long long)j * (2 * p.bwp) + kt * 32 + r] = dw[i][v];
+          const int tok = hf * 16 + v;
+          const float xe = xc[v];
+          const float d = dc[v];
+          const float hp = hc[v];
+          const float re = sigmoid_fast(ua[v], nba), ie = sigmoid_fast(ux[v], nbx);
+          float l2 = re * sp;
+          if constexpr (MASKED) l2 = masked_log2_decay_run(l2, flbits, v);
+          const float ae = __builtin_amdgcn_exp2f(l2);
+          const float g2 = fmaxf(one_minus_exp<false>(l2 * (2.0f * kLn2), ae), 0.0f);
+          const float ge = __builtin_amdgcn_sqrtf(g2);
+          // With z = g i x, a = exp(l), g = sqrt(1 - a^2) (bounded derivative 1 / sqrt(max(4 g^2, 1e-6))):
+          //   dx_direct = delta g i,  di = delta g x,  dl = delta a (h_{t-1} - a i x / sqrt(max(g^2, 2.5e-7)))
+          const float c1 = ge * ie;
+          const float dxd = d * c1;
+          const float ze = c1 * xe;
+          const float q2 = (ie * xe) * __builtin_amdgcn_rsqf(fmaxf(g2, 0.25f * 1e-6f));
+          float dl = (ae * d) * fmaf(-ae, q2, hp);
+          // A reset token has a = 2^-126, which already switches dl off; a padded one has g = 0, which
+          // zeroes dxd, vx and z, but its bounded-sqrt term would leak into dl.
+          if constexpr (MASKED) { if ((flbits >> (2 * v)) & 2u) dl = 0.f; }
+          const float va = dl * (cs * fmaf(-re, re, re));
+          const float vx = (d * ze) * (1.0f - ie);
+          sum_l = fmaf(dl, re, sum_l);
+          sum_ba += va; sum_bx += vx;
+          typedef IO io2 __attribute__((ext_vector_type(2)));
+          io2 pair; pair[0] = (IO)va; pair[1] = (IO)vx;
+          *reinterpret_cast<io2*>(du_tile + tok * ROW_DU + 2 * uo) = pair;
+          lds_dxd[cur][slab][v][lane] = dxd;
+          fx_t[v >> 3][v & 7] = (IO)xe; fa[v >> 3][v & 7] = pair[0]; fx[v >> 3][v & 7] = pair[1];
         }
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+          lds_xt[cur][slab][q][lane] = fx_t[q];
+          lds_dub[cur][slab][0][q][lane] = fa[q];
+          lds_dub[cur][slab][1][q][lane] = fx[q];
+        }
+      }
+      advance(at);
+      __syncthreads();
+    }
+    if (slab_ok) {
+      // per-workgroup partial of the bias and Lambda gradients
+      sum_ba += xhalf(sum_ba, hf); sum_bx += xhalf(sum_bx, hf); sum_l += xhalf(sum_l, hf);
+      if (hf == 0) {
+        float* ps = p.partial + (long long)wg_in_unit * 3 * p.Wp + ch;
+        ps[0] = sum_ba; ps[p.Wp] = sum_bx; ps[2 * p.Wp] = sum_l;
+      }
+    }
+  } else {
+    // ------------------------------------------------------------------ product waves
+    // this wave's rows of w2t, B operand of the input-gradient product; lane (n = j, hf) holds
+    // kappa = 16 kg + 8 hf + i
+    Frag w2[NKG2];
+    {
+      const IO* row = (const IO*)p.w2t + ((long long)k * p.bwp + sl * 32 + r) * (2 * p.bwp) + hf * Tr::HW;
+#pragma unroll
+      for (int kg = 0; kg < NKG2; ++kg) w2[kg] = *reinterpret_cast<const Frag*>(row + kg * Tr::KG);
+    }
+    f32x16 dw[2][S];                                     // [gate][input slab of the block] x own output slab
+#pragma unroll
+    for (int g = 0; g < 2; ++g)
+#pragma unroll
+      for (int js = 0; js < S; ++js)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) dw[g][js][v] = 0.f;
+    // x tiles: 32 rows x 16 vectors, two per thread of the four product waves
+    const int gid = tid - 4 * 64;
+    Frag pre_x[2];
+    auto issue = [&](const Place& q) {
+      const bool live = q.tile < n_tiles;
+      const int b = live ? q.b : 0, c = live ? q.c : 0;
+      const int t0 = c * TR;
+      const int rows = !live ? 0 : ((p.T - t0) < TR ? (p.T - t0) : TR);
+      const rsrc_t rx = make_rsrc((const IO*)p.x + ((long long)b * p.T + t0) * W, (unsigned)rows * row_bytes);
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int idx = gid + 256 * i, row = idx >> 4, cv = idx & 15;
+        pre_x[i] = buf_load_frag<Frag>(rx, (unsigned)row * row_bytes + (unsigned)(unit_col + cv * Tr::HW) * 2u);
+      }
+    };
+    auto store_x = [&](int buf) {
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int idx = gid + 256 * i, row = idx >> 4, cv = idx & 15;
+        *reinterpret_cast<Frag*>(lds_x[buf] + row * ROW + cv * Tr::HW) = pre_x[i];
+      }
+    };
+    // the x tile of iteration it + 1 goes to LDS in iteration it
+    Place ahead = first;
+    issue(ahead);
+    store_x(0);
+    advance(ahead);
+    issue(ahead);
+    __syncthreads();                                     // x tile 0 is in LDS
+    Place at = first, done = first;                      // `done`: the tile the element waves finished last
+    for (int it = 0; at.tile < n_tiles + n_wg; ++it) {
+      const int prev = (it & 1) ^ 1;
+      store_x(prev);
+      advance(ahead);
+      issue(ahead);
+      if (it > 0 && slab_ok) {
+        const int b = done.b, c = done.c;
+        const int t0 = c * TR;
+        // weight gradients: the fragments the element waves left in LDS
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+          const Frag ba = lds_dub[prev][slab][0][q][lane], bx = lds_dub[prev][slab][1][q][lane];
+#pragma unroll
+          for (int js = 0; js < S; ++js) {
+            const Frag xt = lds_xt[prev][blk * S + js][q][lane];
+            Tr::mma(dw[0][js], xt, ba);
+            Tr::mma(dw[1][js], xt, bx);
+          }
+        }
+        // input gradient of this slab's channels: direct part + du . w2t^T, on two accumulators
+        f32x16 acc, acc_odd;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) { acc[v] = lds_dxd[prev][slab][v][lane]; acc_odd[v] = 0.f; }
+        const IO* a_row_du = lds_du[prev] + tile_row<1>(0, r) * ROW_DU + 2 * kb + hf * Tr::HW;
+#pragma unroll
+        for (int kg = 0; kg < NKG2; kg += 2) {
+          Tr::mma(acc, *reinterpret_cast<const Frag*>(a_row_du + kg * Tr::KG), w2[kg]);
+          Tr::mma(acc_odd, *reinterpret_cast<const Frag*>(a_row_du + (kg + 1) * Tr::KG), w2[kg + 1]);
+        }
+        unsigned char* my = stage + WaveStage<TR>::row_offset(hf * 16) + r * 2;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) *reinterpret_cast<IO*>(my + v * WaveStage<TR>::kRowBytes) = (IO)(acc[v] + acc_odd[v]);
+        wave_lds_fence();
+        const int rows = (p.T - t0) < TR ? (p.T - t0) : TR;
+        const rsrc_t rdx = make_rsrc((const IO*)p.dx + ((long long)b * p.T + t0) * W, (unsigned)rows * row_bytes);
+        stage_flush<TR>(stage, rdx, row_bytes, (unsigned)(unit_col + slab * 32) * 2u, lane);
+        wave_lds_fence();
+      }
+      done = at;
+      advance(at);
+      __syncthreads();
+    }
+    if (slab_ok) {
+      // per-workgroup partial of the weight gradients: [wg][k][gate][j][o]
+#pragma unroll
+      for (int g = 0; g < 2; ++g) {
+        float* part = p.dw_partial + ((((long long)wg_in_unit * p.nb + k) * 2 + g) * p.bwp) * p.bwp;
+#pragma unroll
+        for (int js = 0; js < S; ++js)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const int j = js * 32 + 8 * (v >> 2) + 4 * hf + (v & 3);
+            part[(long long)j * p.bwp + sl * 32 + r] = dw[g][js][v];
+          }
       }
     }
   }
@@ -1326,8 +1602,8 @@ __global__ __launch_bounds__(kGradThreads, 1) void gate_grad_kernel(FusedArgs p)
 
 // Last launch of a backward pass: sums the per-workgroup partial results and writes the parameter
 // gradients in the caller's type.  Workgroups [0, vec_blocks) own 16 channels each of db_a, db_x and
-// dLambda; the rest (fast backward only) own 256 elements each of the two weight gradients,
-// dW_gate[k][o][j] = sum over workgroups of dW2T[wg][k][j][2 o + gate].
+// dLambda; the rest (fast backward only) own 1024 elements each of the two weight gradients,
+// dW_gate[k][o][j] = sum over workgroups of the partials [wg][k][gate][j][o].
 struct FinishArgs {
   const float* partial; const float* dsp; void* db_a; void* db_x; void* dlambda;
   const float* dw_partial; void* dw_a; void* dw_x;
@@ -1342,17 +1618,18 @@ __global__ __launch_bounds__(256) void finish_kernel(FinishArgs p) {
   for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < p.clean_n; i += (long long)gridDim.x * blockDim.x)
     p.clean[i] = make_uint4(0u, 0u, 0u, 0u);
   if ((int)blockIdx.x >= p.vec_blocks) {
-    // four consecutive kappa (two output channels x two gates) per thread, 16-byte loads; bw is a
-    // multiple of 32 on this path, so a group of four never crosses a row
-    const long long total4 = (long long)p.nb * p.bw * 2 * p.bw / 4;
+    // four consecutive output channels o of one (block, gate, input channel j) per thread, 16-byte
+    // loads; bw is a multiple of 32 on this path, so a group of four never crosses a row
+    const long long total4 = (long long)p.nb * 2 * p.bw * p.bw / 4;
     const long long i4 = (long long)(blockIdx.x - p.vec_blocks) * blockDim.x + threadIdx.x;
     if (i4 >= total4) return;
     const long long i = i4 * 4;
-    const int kap = (int)(i % (2 * p.bw));
-    const int j = (int)((i / (2 * p.bw)) % p.bw);
+    const int o = (int)(i % p.bw);
+    const int j = (int)((i / p.bw) % p.bw);
+    const int gate = (int)((i / ((long long)p.bw * p.bw)) % 2);
     const int k = (int)(i / ((long long)2 * p.bw * p.bw));
-    const long long stride = (long long)p.nb * p.bwp * 2 * p.bwp;
-    const float* src = p.dw_partial + ((long long)k * p.bwp + j) * (2 * p.bwp) + kap;
+    const long long stride = (long long)p.nb * 2 * p.bwp * p.bwp;
+    const float* src = p.dw_partial + i;
     // fixed summation order; eight loads in flight per thread
     float4 s0 = make_float4(0.f, 0.f, 0.f, 0.f), s1 = s0;
     int g = 0;
@@ -1370,11 +1647,12 @@ __global__ __launch_bounds__(256) void finish_kernel(FinishArgs p) {
       const float4 v = *reinterpret_cast<const float4*>(src + (long long)g * stride);
       s0.x += v.x; s0.y += v.y; s0.z += v.z; s0.w += v.w;
     }
-    const long long o0 = ((long long)k * p.bw + (kap >> 1)) * p.bw + j;      // element (k, o, j); o + 1 is bw further
-    store_vec(p.dw_a, o0, s0.x + s1.x, p.grad_dtype);
-    store_vec(p.dw_x, o0, s0.y + s1.y, p.grad_dtype);
-    store_vec(p.dw_a, o0 + p.bw, s0.z + s1.z, p.grad_dtype);
-    store_vec(p.dw_x, o0 + p.bw, s0.w + s1.w, p.grad_dtype);
+    void* dst = gate ? p.dw_x : p.dw_a;
+    const long long o0 = ((long long)k * p.bw + o) * p.bw + j;               // element (k, o, j); o + 1 is bw further
+    store_vec(dst, o0, s0.x + s1.x, p.grad_dtype);
+    store_vec(dst, o0 + p.bw, s0.y + s1.y, p.grad_dtype);
+    store_vec(dst, o0 + 2 * p.bw, s0.z + s1.z, p.grad_dtype);
+    store_vec(dst, o0 + 3 * p.bw, s0.w + s1.w, p.grad_dtype);
     return;
   }
   // 16 channels per workgroup; sixteen threads per channel each sum a share of the per-workgroup
@@ -1884,7 +2162,13 @@ int rglru_hip_fast_path(int64_t W, int64_t nb, int dtype) {
   return (bw == 32 || bw == 64 || bw == 128) ? 1 : 0;
 }
 
-int rglru_hip_bwd_full(const void* x, const void* prep, const float* h0,
+// tokens per tile of the reverse-scan kernel: 32 * kDeltaMT
+#ifndef RGLRU_DELTA_MT
+#define RGLRU_DELTA_MT 1
+#endif
+constexpr int kDeltaMT = RGLRU_DELTA_MT;
+
+int rglru_hip_bwd_full(const void* x, const void* y, const void* prep, const float* h0,
                        const uint8_t* flags, const void* dy, const float* dh_last, void* ws, void* scratch,
                        void* dx, void* dw_a, void* dw_x, void* db_a, void* db_x, void* dlambda,
                        float* dh0, int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, int grad_dtype,
@@ -1896,24 +2180,24 @@ int rglru_hip_bwd_full(const void* x, const void* prep, const float* h0,
   if (!rglru_hip_fast_path(W, nb, dtype))
     return fail(RGLRU_E_UNSUPPORTED, "bwd_full: needs 16-bit storage and gate blocks of 32, 64 or 128 channels");
   if (B <= 0 || T <= 0) return fail(RGLRU_E_ARG, "bwd_full: B and T must be positive (got %lld, %lld)", (long long)B, (long long)T);
-  if (!x || !prep || !dy || !ws || !scratch || !dx || !dw_a || !dw_x || !db_a || !db_x || !dlambda)
+  if (!x || !y || !prep || !dy || !ws || !scratch || !dx || !dw_a || !dw_x || !db_a || !db_x || !dlambda)
     return fail(RGLRU_E_ARG, "bwd_full: null pointer");
   rc = check_extents("bwd_full", B, T, W);
   if (rc) return rc;
   Geometry g = make_geometry(W, nb);
-  if (!is_aligned(x, W, g.bw, 2) || !is_aligned(dy, W, g.bw, 2) || !is_aligned(dx, W, g.bw, 2))
-    return fail(RGLRU_E_UNSUPPORTED, "bwd_full: x, dy and dx must be 16-byte aligned");
+  if (!is_aligned(x, W, g.bw, 2) || !is_aligned(y, W, g.bw, 2) || !is_aligned(dy, W, g.bw, 2) || !is_aligned(dx, W, g.bw, 2))
+    return fail(RGLRU_E_UNSUPPORTED, "bwd_full: x, y, dy and dx must be 16-byte aligned");
   WorkLayout L = make_work_layout(B, T, g);
   hipStream_t s = (hipStream_t)stream;
   char* wb = (char*)ws;
   FusedArgs a;
   memset(&a, 0, sizeof(a));
   fill_common(a, g, prep, dtype);
-  a.x = x; a.h0 = h0; a.flags = flags; a.dy = dy; a.dh_last = dh_last;
+  a.x = x; a.y = const_cast<void*>(y); a.h0 = h0; a.flags = flags; a.dy = dy; a.dh_last = dh_last;
   a.flags_vec = (T % 16 == 0) && ((uintptr_t)flags % 16 == 0);
   const ScratchLayout SL = make_scratch_layout(B, T, g, true);
   char* sb = (char*)scratch;
-  a.dx = dx; a.du_a = sb + SL.du2; a.dh0 = dh0;
+  a.dx = dx; a.du_a = sb + SL.delta; a.dh0 = dh0;
   a.ckpt = (float*)(wb + L.ckpt); a.rec_a = (rec_t*)(wb + L.b_rec_a);
   a.ticket = (unsigned*)(wb + L.b_ticket); a.fail = (unsigned*)(wb + L.fail);
   a.partial = (float*)(sb + SL.partial); a.dw_partial = (float*)(sb + SL.dw_partial);
@@ -1921,36 +2205,43 @@ int rglru_hip_bwd_full(const void* x, const void* prep, const float* h0,
   a.aligned = 1;
   const int nkg = held_groups(g, dtype, 1);
   pack_units(a, g, nkg);
-  a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nC, 2, L.max_wg);
+  // reverse scan: delta[B, T, W] (and dh0)
+  const long long chunks = (T + 32 * kDeltaMT - 1) / (32 * kDeltaMT);
+  a.wg_per_unit = pick_wg_per_unit(a.units, B * chunks, kDeltaMT == 1 ? 4 : 2, L.max_wg);
   a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
-  const bool masked = (flags != nullptr) || (T % kChunk != 0);
+  const bool masked = (flags != nullptr) || (T % (32 * kDeltaMT) != 0);
   dim3 grid((unsigned)(a.wg_per_unit * a.units));
   {
     KernelTimer timer(1, s);
-#define RGLRU_LAUNCH_SCAN(N)                                                                              \
-    if (masked) hipLaunchKernelGGL((bwd_scan_kernel<__bf16, N, true>), grid, dim3(kThreads), 0, s, a);      \
-    else hipLaunchKernelGGL((bwd_scan_kernel<__bf16, N, false>), grid, dim3(kThreads), 0, s, a)
-    if (nkg == 8) { RGLRU_LAUNCH_SCAN(8); } else if (nkg == 4) { RGLRU_LAUNCH_SCAN(4); } else { RGLRU_LAUNCH_SCAN(2); }
-#undef RGLRU_LAUNCH_SCAN
+#define RGLRU_LAUNCH_DELTA(N)                                                                                        \
+    if (masked) hipLaunchKernelGGL((bwd_delta_kernel<__bf16, N, true, kDeltaMT>), grid, dim3(kThreads), 0, s, a);      \
+    else hipLaunchKernelGGL((bwd_delta_kernel<__bf16, N, false, kDeltaMT>), grid, dim3(kThreads), 0, s, a)
+    if (nkg == 8) { RGLRU_LAUNCH_DELTA(8); } else if (nkg == 4) { RGLRU_LAUNCH_DELTA(4); } else { RGLRU_LAUNCH_DELTA(2); }
+#undef RGLRU_LAUNCH_DELTA
   }
   rc = check_launch("bwd_full scan");
   if (rc) return rc;
-  // the gradient GEMM kernel packs narrow blocks into units the same way (a.units)
+  // gradients: one workgroup per compute unit, the same units
   int n_wg = num_compute_units() / a.units; if (n_wg < 1) n_wg = 1; if (n_wg > kGemmWgPerUnit) n_wg = kGemmWgPerUnit;
+  const long long grad_tiles = B * ((T + 31) / 32);
+  if (n_wg > grad_tiles) n_wg = (int)grad_tiles;
+  const bool masked_grad = (flags != nullptr) || (T % 32 != 0);
   dim3 grid2((unsigned)(n_wg * a.units));
   {
     KernelTimer timer(3, s);
-    if (nkg == 8) hipLaunchKernelGGL((gate_grad_kernel<__bf16, 8>), grid2, dim3(kGradThreads), 0, s, a);
-    else if (nkg == 4) hipLaunchKernelGGL((gate_grad_kernel<__bf16, 4>), grid2, dim3(kGradThreads), 0, s, a);
-    else hipLaunchKernelGGL((gate_grad_kernel<__bf16, 2>), grid2, dim3(kGradThreads), 0, s, a);
+#define RGLRU_LAUNCH_GRAD(N)                                                                                          \
+    if (masked_grad) hipLaunchKernelGGL((bwd_grad_kernel<__bf16, N, true>), grid2, dim3(kGradThreads), 0, s, a);         \
+    else hipLaunchKernelGGL((bwd_grad_kernel<__bf16, N, false>), grid2, dim3(kGradThreads), 0, s, a)
+    if (nkg == 8) { RGLRU_LAUNCH_GRAD(8); } else if (nkg == 4) { RGLRU_LAUNCH_GRAD(4); } else { RGLRU_LAUNCH_GRAD(2); }
+#undef RGLRU_LAUNCH_GRAD
   }
-  rc = check_launch("bwd_full gemm");
+  rc = check_launch("bwd_full gradients");
   if (rc) return rc;
   FinishArgs r;
   memset(&r, 0, sizeof(r));
   r.partial = a.partial; r.dsp = finish_dsp(g, prep, dtype); r.db_a = db_a; r.db_x = db_x; r.dlambda = dlambda;
   r.dw_partial = a.dw_partial; r.dw_a = dw_a; r.dw_x = dw_x;
-  r.W = (int)W; r.nb = (int)nb; r.bw = (int)g.bw; r.bwp = (int)g.bwp; r.Wp = (int)g.Wp; r.wg_per_unit = a.wg_per_unit;
+  r.W = (int)W; r.nb = (int)nb; r.bw = (int)g.bw; r.bwp = (int)g.bwp; r.Wp = (int)g.Wp; r.wg_per_unit = n_wg;
   r.n_wg = n_wg; r.vec_blocks = (int)((W + 15) / 16); r.grad_dtype = grad_dtype;
   r.clean = (uint4*)(wb + L.b_begin); r.clean_n = (long long)((L.b_end - L.b_begin) / 16);
   const long long total = nb * g.bw * 2 * g.bw;

@@ -64,7 +64,7 @@ inline PrepLayout make_prep_layout(const Geometry& g, size_t elem) {
 //   b_rec_a     [B][nC][W]      64-bit carry records of the backward chain
 //   b_ticket    [units][kMaxQueues]
 constexpr int kMaxQueues = 64;          // ticket queues per unit (sequences are dealt round-robin to them)
-constexpr int kGemmWgPerUnit = 32;      // workgroups per gate block in the gradient GEMM kernel
+constexpr int kGemmWgPerUnit = 32;      // workgroups per unit in the gradient kernel of the fast backward
 
 struct WorkLayout {
   int64_t nC, nCf, max_wg;
@@ -96,10 +96,10 @@ inline WorkLayout make_work_layout(int64_t B, int64_t T, const Geometry& g) {
 
 // Scratch of one backward call; nothing in it outlives the call, its contents on entry do not matter.
 //   partial     [maxWg][3][Wp]  per-workgroup sums for db_a, db_x, dLambda
-//   du2         [B][T][2W]      16-bit: gate pre-activation gradients (fast backward only)
-//   dw_partial  [kGemmWgPerUnit][nb][bwp][2*bwp] fp32 per-workgroup weight-gradient sums (fast backward only)
+//   delta       [B][T][W]       16-bit: dL/dh_t after the reverse scan (fast backward only)
+//   dw_partial  [kGemmWgPerUnit][nb][2][bwp][bwp] fp32 per-workgroup weight-gradient sums (fast backward only)
 struct ScratchLayout {
-  size_t partial, du2, dw_partial, total;
+  size_t partial, delta, dw_partial, total;
 };
 
 inline ScratchLayout make_scratch_layout(int64_t B, int64_t T, const Geometry& g, bool fast) {
@@ -107,7 +107,7 @@ inline ScratchLayout make_scratch_layout(int64_t B, int64_t T, const Geometry& g
   size_t off = 0;
   auto take = [&](int64_t bytes) { size_t at = off; off += (size_t)round_up(bytes, 256); return at; };
   s.partial = take((int64_t)256 * 3 * g.Wp * 4);
-  s.du2 = take(fast ? B * T * 2 * g.W * 2 : 0);
+  s.delta = take(fast ? B * T * g.W * 2 : 0);
   s.dw_partial = take(fast ? (int64_t)kGemmWgPerUnit * g.nb * g.bwp * 2 * g.bwp * 4 : 0);
   s.total = off;
   return s;

@@ -235,7 +235,7 @@ class _HipRGLRU(torch.autograd.Function):
                                                      image.data_ptr(), x.data_ptr(), _ptr(h0c), _ptr(flags),
                                                      y.data_ptr(), h_last.data_ptr(), ws.data_ptr(), B, T, W, nb, code,
                                                      _stream_ptr(device)), "rglru_hip_prepare_fwd")
-        ctx.save_for_backward(x, w_a, w_x, h0c, flags, ws, image)
+        ctx.save_for_backward(x, w_a, w_x, h0c, flags, ws, image, y)
         ctx.param_dtypes = (w_a.dtype, b_a.dtype, w_x.dtype, b_x.dtype, lam.dtype)
         ctx.h0_dtype = None if h0 is None else h0.dtype
         ctx.set_materialize_grads(False)      # an unused output arrives as None, not as a tensor of zeros
@@ -244,7 +244,7 @@ class _HipRGLRU(torch.autograd.Function):
     @staticmethod
     @once_differentiable
     def backward(ctx, dy, dh_last):
-        x, w_a, w_x, h0c, flags, ws, image = ctx.saved_tensors
+        x, w_a, w_x, h0c, flags, ws, image, y = ctx.saved_tensors
         lib = _lib.load()
         B, T, W = x.shape
         nb, bw, _ = w_a.shape
@@ -265,11 +265,12 @@ class _HipRGLRU(torch.autograd.Function):
             dh0 = torch.empty(B, W, dtype=torch.float32, device=device) if ctx.needs_input_grad[6] else None
             # scratch of this call only (the workspace kept since forward holds just checkpoints and records)
             scratch = torch.empty(lib.rglru_hip_bwd_scratch_bytes(B, T, W, nb, code), dtype=torch.uint8, device=device)
-            if lib.rglru_hip_fast_path(W, nb, code) and dy.data_ptr() % 16 == 0 and x.data_ptr() % 16 == 0:
+            if (lib.rglru_hip_fast_path(W, nb, code) and dy.data_ptr() % 16 == 0 and x.data_ptr() % 16 == 0
+                    and y.data_ptr() % 16 == 0):
                 # everything in hand-written kernels, including the two gate GEMMs
                 dw_a = torch.empty(nb, bw, bw, dtype=gdt, device=device)
                 dw_x = torch.empty(nb, bw, bw, dtype=gdt, device=device)
-                _lib.check(lib.rglru_hip_bwd_full(x.data_ptr(), image.data_ptr(), _ptr(h0c), _ptr(flags),
+                _lib.check(lib.rglru_hip_bwd_full(x.data_ptr(), y.data_ptr(), image.data_ptr(), _ptr(h0c), _ptr(flags),
                                                   dy.data_ptr(), _ptr(dhl), ws.data_ptr(), scratch.data_ptr(), dx.data_ptr(), dw_a.data_ptr(),
                                                   dw_x.data_ptr(), db_a.data_ptr(), db_x.data_ptr(), dlam.data_ptr(),
                                                   _ptr(dh0), B, T, W, nb, code, gcode, _stream_ptr(device)),

@@ -46,7 +46,7 @@
 extern "C" {
 #endif
 
-#define RGLRU_ABI_VERSION 9
+#define RGLRU_ABI_VERSION 10
 
 enum { RGLRU_F32 = 0, RGLRU_BF16 = 1 };
 
@@ -150,11 +150,15 @@ int rglru_hip_bwd(const void* x, const void* prep, const float* h0,
 
 /* Complete backward for the fast configurations (rglru_hip_fast_path(W, nb, dtype) != 0: 16-bit
  * storage, gate blocks of 32, 64 or 128 channels, 16-byte aligned tensors).  Same inputs as
- * rglru_hip_bwd; dx[B,T,W] is the full input gradient and dw_a, dw_x [nb,bw,bw] (grad_dtype) the
- * weight gradients: the two gate GEMMs run in a second hand-written kernel instead of being left
- * to the caller.  Returns RGLRU_E_UNSUPPORTED for other configurations. */
+ * rglru_hip_bwd plus y[B,T,W], the output of the forward call as it was stored (the state in front of
+ * token t is read from row t - 1 of it; the checkpoints in `ws` are not used).  dx[B,T,W] is the full
+ * input gradient and dw_a, dw_x [nb,bw,bw] (grad_dtype) the weight gradients.  Two hand-written
+ * kernels: the reverse scan for dL/dh_t, which recomputes only the decay, then one kernel that
+ * recomputes both gates and forms every gradient including the two block-diagonal GEMMs, so the
+ * gradients at the gate pre-activations never reach memory.  Returns RGLRU_E_UNSUPPORTED for other
+ * configurations. */
 int rglru_hip_fast_path(int64_t W, int64_t nb, int dtype);
-int rglru_hip_bwd_full(const void* x, const void* prep, const float* h0,
+int rglru_hip_bwd_full(const void* x, const void* y, const void* prep, const float* h0,
                        const uint8_t* flags, const void* dy, const float* dh_last, void* ws, void* scratch,
                        void* dx, void* dw_a, void* dw_x, void* db_a, void* db_x, void* dlambda,
                        float* dh0, int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, int grad_dtype,
@@ -274,7 +278,7 @@ int rglru_hip_workspace_status(const void* ws, int64_t B, int64_t T, int64_t W, 
  * rglru_hip_kernel_ms(which) waits for the most recent bracket (process-wide, so enable it from one
  * thread and keep calls sequential) and returns its
  * duration in milliseconds (negative when none was recorded): which = 0 forward, 1 backward
- * (scan part), 2 step, 3 backward gradient GEMMs (rglru_hip_bwd_full only).  Not for use under stream capture. */
+ * (scan part), 2 step, 3 backward gradient kernel (rglru_hip_bwd_full only).  Not for use under stream capture. */
 int rglru_hip_set_timing(int enable);
 float rglru_hip_kernel_ms(int which);
 
