@@ -1141,12 +1141,15 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
 // prefetched, and its weight-gradient accumulators are shared by the eight waves of a workgroup.
 // ------------------------------------------------------------------------------------------
 #ifndef RGLRU_DELTA_DEPTH
-#define RGLRU_DELTA_DEPTH 8
+#define RGLRU_DELTA_DEPTH 2
 #endif
 constexpr int kDeltaDepth = RGLRU_DELTA_DEPTH;         // records a walk of the reverse scan requests per round trip
 
+#ifndef RGLRU_DELTA_OCC
+#define RGLRU_DELTA_OCC 2
+#endif
 template <typename IO, int NKG, bool MASKED, int MT>
-__global__ __launch_bounds__(kThreads, (MT == 1 ? 4 : 2)) void bwd_delta_kernel(FusedArgs p) {
+__global__ __launch_bounds__(kThreads, (MT == 1 ? 4 : RGLRU_DELTA_OCC)) void bwd_delta_kernel(FusedArgs p) {
   constexpr int TR = 32 * MT, EL = 16 * MT;
   typedef Io<IO> Tr;
   typedef typename Tr::Frag Frag;
@@ -1454,7 +1457,8 @@ __global__ __launch_bounds__(kGradThreads, 1) void bwd_grad_kernel(FusedArgs p) 
           float l2 = re * sp;
           if constexpr (MASKED) l2 = masked_log2_decay_run(l2, flbits, v);
           const float ae = __builtin_amdgcn_exp2f(l2);
-          const float g2 = fmaxf(one_minus_exp<false>(l2 * (2.0f * kLn2), ae), 0.0f);
+          // l2 <= 0 and a <= 1, so neither branch of one_minus_exp can turn negative: no clamp needed
+          const float g2 = one_minus_exp<false>(l2 * (2.0f * kLn2), ae);
           const float ge = __builtin_amdgcn_sqrtf(g2);
           // With z = g i x, a = exp(l), g = sqrt(1 - a^2) (bounded derivative 1 / sqrt(max(4 g^2, 1e-6))):
           //   dx_direct = delta g i,  di = delta g x,  dl = delta a (h_{t-1} - a i x / sqrt(max(g^2, 2.5e-7)))
@@ -1552,27 +1556,36 @@ __global__ __launch_bounds__(kGradThreads, 1) void bwd_grad_kernel(FusedArgs p) 
         // weight gradients: the fragments the element waves left in LDS
 #pragma unroll
         for (int q = 0; q < 2; ++q) {
+          // all fragments of a K group first, so that their LDS latencies overlap
           const Frag ba = lds_dub[prev][slab][0][q][lane], bx = lds_dub[prev][slab][1][q][lane];
+          Frag xt[S];
+#pragma unroll
+          for (int js = 0; js < S; ++js) xt[js] = lds_xt[prev][blk * S + js][q][lane];
 #pragma unroll
           for (int js = 0; js < S; ++js) {
-            const Frag xt = lds_xt[prev][blk * S + js][q][lane];
-            Tr::mma(dw[0][js], xt, ba);
-            Tr::mma(dw[1][js], xt, bx);
+            Tr::mma(dw[0][js], xt[js], ba);
+            Tr::mma(dw[1][js], xt[js], bx);
           }
         }
-        // input gradient of this slab's channels: direct part + du . w2t^T, on two accumulators
-        f32x16 acc, acc_odd;
+        // input gradient of this slab's channels: direct part + du . w2t^T.  The A fragments are
+        // requested four at a time so that their LDS latency overlaps (one fragment per product would
+        // expose it sixteen times).
+        f32x16 acc;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) { acc[v] = lds_dxd[prev][slab][v][lane]; acc_odd[v] = 0.f; }
+        for (int v = 0; v < 16; ++v) acc[v] = lds_dxd[prev][slab][v][lane];
         const IO* a_row_du = lds_du[prev] + tile_row<1>(0, r) * ROW_DU + 2 * kb + hf * Tr::HW;
+        constexpr int kBatch = NKG2 < 4 ? NKG2 : 4;
 #pragma unroll
-        for (int kg = 0; kg < NKG2; kg += 2) {
-          Tr::mma(acc, *reinterpret_cast<const Frag*>(a_row_du + kg * Tr::KG), w2[kg]);
-          Tr::mma(acc_odd, *reinterpret_cast<const Frag*>(a_row_du + (kg + 1) * Tr::KG), w2[kg + 1]);
+        for (int kg0 = 0; kg0 < NKG2; kg0 += kBatch) {
+          Frag af[kBatch];
+#pragma unroll
+          for (int j = 0; j < kBatch; ++j) af[j] = *reinterpret_cast<const Frag*>(a_row_du + (kg0 + j) * Tr::KG);
+#pragma unroll
+          for (int j = 0; j < kBatch; ++j) Tr::mma(acc, af[j], w2[kg0 + j]);
         }
         unsigned char* my = stage + WaveStage<TR>::row_offset(hf * 16) + r * 2;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) *reinterpret_cast<IO*>(my + v * WaveStage<TR>::kRowBytes) = (IO)(acc[v] + acc_odd[v]);
+        for (int v = 0; v < 16; ++v) *reinterpret_cast<IO*>(my + v * WaveStage<TR>::kRowBytes) = (IO)acc[v];
         wave_lds_fence();
         const int rows = (p.T - t0) < TR ? (p.T - t0) : TR;
         const rsrc_t rdx = make_rsrc((const IO*)p.dx + ((long long)b * p.T + t0) * W, (unsigned)rows * row_bytes);
@@ -1851,9 +1864,9 @@ struct KernelTimer {
     if (!g_timing.load(std::memory_order_relaxed)) return;
     slot = &timing_slot(which);
     if (!slot->start && (hipEventCreate(&slot->start) != hipSuccess || hipEventCreate(&slot->stop) != hipSuccess)) { slot = nullptr; return; }
-    hipEventRecord(slot->start, stream);
+    (void)hipEventRecord(slot->start, stream);
   }
-  ~KernelTimer() { if (slot) { hipEventRecord(slot->stop, stream); slot->armed = true; } }
+  ~KernelTimer() { if (slot) { (void)hipEventRecord(slot->stop, stream); slot->armed = true; } }
 };
 
 // Narrow blocks of the kernels with register-held weights share a unit (see kPackedWidth).
@@ -2164,7 +2177,7 @@ int rglru_hip_fast_path(int64_t W, int64_t nb, int dtype) {
 
 // tokens per tile of the reverse-scan kernel: 32 * kDeltaMT
 #ifndef RGLRU_DELTA_MT
-#define RGLRU_DELTA_MT 1
+#define RGLRU_DELTA_MT 2
 #endif
 constexpr int kDeltaMT = RGLRU_DELTA_MT;
 
@@ -2207,7 +2220,7 @@ int rglru_hip_bwd_full(const void* x, const void* y, const void* prep, const flo
   pack_units(a, g, nkg);
   // reverse scan: delta[B, T, W] (and dh0)
   const long long chunks = (T + 32 * kDeltaMT - 1) / (32 * kDeltaMT);
-  a.wg_per_unit = pick_wg_per_unit(a.units, B * chunks, kDeltaMT == 1 ? 4 : 2, L.max_wg);
+  a.wg_per_unit = pick_wg_per_unit(a.units, B * chunks, kDeltaMT == 1 ? 4 : RGLRU_DELTA_OCC, L.max_wg);
   a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
   const bool masked = (flags != nullptr) || (T % (32 * kDeltaMT) != 0);
   dim3 grid((unsigned)(a.wg_per_unit * a.units));
