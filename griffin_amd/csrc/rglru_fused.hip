@@ -1333,7 +1333,7 @@ __global__ __launch_bounds__(kGradThreads, 1) void bwd_grad_kernel(FusedArgs p) 
   constexpr int TW = kPackedWidth;                       // unit width
   constexpr int NKG2 = 2 * NKG;                          // K groups of the input-gradient product (2 * KC kappa)
   constexpr int ROW = TW + Tr::HW, ROW_DU = 2 * TW + Tr::HW;
-  __shared__ __attribute__((aligned(16))) IO lds_x[2][TR * ROW];        // x tiles of two consecutive iterations
+  __shared__ __attribute__((aligned(16))) IO lds_x[3][TR * ROW];        // x tiles of three consecutive iterations
   __shared__ __attribute__((aligned(16))) IO lds_du[2][TR * ROW_DU];    // [token][2 * unit channel + gate]
   __shared__ __attribute__((aligned(16))) float lds_dxd[2][4][16][64];  // direct input gradient [slab][register][lane]
   __shared__ __attribute__((aligned(16))) Frag lds_xt[2][4][2][64];     // x fragments [slab][K group][lane]
@@ -1410,11 +1410,28 @@ __global__ __launch_bounds__(kGradThreads, 1) void bwd_grad_kernel(FusedArgs p) 
         pre_h[q2] = buf_load_frag<Frag>(rh, my_row >= shift ? (unsigned)(my_row - shift) * row_bytes + col : kOutOfRange);
       }
     };
+    // gate products of one tile: issued one iteration before their results are used, so the matrix
+    // unit works on the next tile while the vector unit works on the current one
+    auto gate_products = [&](const IO* tile_x, f32x16& ua, f32x16& ux) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) { ua[v] = 0.0f; ux[v] = 0.0f; }       // the biases enter inside the sigmoids
+      const IO* xrow = tile_x + my_row * ROW + kb + hf * Tr::HW;
+#pragma unroll
+      for (int kg = 0; kg < NKG; ++kg) {
+        const Frag xa = *reinterpret_cast<const Frag*>(xrow + kg * Tr::KG);
+        Tr::mma(ua, xa, hw.a[kg]);
+        Tr::mma(ux, xa, hw.x[kg]);
+      }
+    };
     Place at = first;
     issue(at);
-    __syncthreads();                                     // x tile 0 is in LDS
+    __syncthreads();                                     // x tiles 0 and 1 are in LDS
+    f32x16 ua, ux;
+    gate_products(lds_x[0], ua, ux);
+    int xb = 0;                                          // x buffer of the current tile
     for (int it = 0; at.tile < n_tiles + n_wg; ++it) {
       const int cur = it & 1;
+      const int xn = xb == 2 ? 0 : xb + 1;
       if (at.tile < n_tiles && slab_ok) {
         const int b = at.b, c = at.c;
         const int t0 = c * TR;
@@ -1423,10 +1440,10 @@ __global__ __launch_bounds__(kGradThreads, 1) void bwd_grad_kernel(FusedArgs p) 
         float h_first = 0.f;                             // h0 of the sequence, for the lane that owns token 0
         if (c == 0 && hf == 0 && p.h0) h_first = p.h0[(long long)b * W + ch];
 
-        const IO* tile_x = lds_x[cur];
-        f32x16 ua, ux, xc, dc, hc;
+        const IO* tile_x = lds_x[xb];
+        f32x16 xc, dc, hc, ua_next, ux_next;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) { ua[v] = 0.0f; ux[v] = 0.0f; xc[v] = 0.0f; dc[v] = 0.0f; hc[v] = 0.0f; }   // the biases enter inside the sigmoids
+        for (int v = 0; v < 16; ++v) { xc[v] = 0.0f; dc[v] = 0.0f; hc[v] = 0.0f; }
         const IO* xrow = tile_x + my_row * ROW + hf * Tr::HW;
 #pragma unroll
         for (int q2 = 0; q2 < 2; ++q2) {
@@ -1434,21 +1451,19 @@ __global__ __launch_bounds__(kGradThreads, 1) void bwd_grad_kernel(FusedArgs p) 
           Tr::mma(hc, pre_h[q2], ident[q2]);
           Tr::mma(xc, *reinterpret_cast<const Frag*>(xrow + slab * 32 + q2 * Tr::KG), ident[q2]);
         }
-#pragma unroll
-        for (int kg = 0; kg < NKG; ++kg) {
-          const Frag xa = *reinterpret_cast<const Frag*>(xrow + kb + kg * Tr::KG);
-          Tr::mma(ua, xa, hw.a[kg]);
-          Tr::mma(ux, xa, hw.x[kg]);
-        }
+        gate_products(lds_x[xn], ua_next, ux_next);
         Place nxt = at;
         advance(nxt);
         issue(nxt);
         if (c == 0 && hf == 0) hc[0] = h_first;
 
         IO* du_tile = lds_du[cur];
-        Frag fx_t[2], fa[2], fx[2];                        // x, du_a, du_x of the lane's tokens, per K group
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
+        for (int q = 0; q < 2; ++q) {
+        Frag fx_t, fa, fx;                                 // x, du_a, du_x of the lane's tokens of K group q
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int v = 8 * q + i;
           const int tok = hf * 16 + v;
           const float xe = xc[v];
           const float d = dc[v];
@@ -1478,15 +1493,15 @@ __global__ __launch_bounds__(kGradThreads, 1) void bwd_grad_kernel(FusedArgs p) 
           io2 pair; pair[0] = (IO)va; pair[1] = (IO)vx;
           *reinterpret_cast<io2*>(du_tile + tok * ROW_DU + 2 * uo) = pair;
           lds_dxd[cur][slab][v][lane] = dxd;
-          fx_t[v >> 3][v & 7] = (IO)xe; fa[v >> 3][v & 7] = pair[0]; fx[v >> 3][v & 7] = pair[1];
+          fx_t[i] = (IO)xe; fa[i] = pair[0]; fx[i] = pair[1];
         }
-#pragma unroll
-        for (int q = 0; q < 2; ++q) {
-          lds_xt[cur][slab][q][lane] = fx_t[q];
-          lds_dub[cur][slab][0][q][lane] = fa[q];
-          lds_dub[cur][slab][1][q][lane] = fx[q];
+        lds_xt[cur][slab][q][lane] = fx_t;
+        lds_dub[cur][slab][0][q][lane] = fa;
+        lds_dub[cur][slab][1][q][lane] = fx;
         }
+        ua = ua_next; ux = ux_next;
       }
+      xb = xn;
       advance(at);
       __syncthreads();
     }
@@ -1537,17 +1552,22 @@ __global__ __launch_bounds__(kGradThreads, 1) void bwd_grad_kernel(FusedArgs p) 
         *reinterpret_cast<Frag*>(lds_x[buf] + row * ROW + cv * Tr::HW) = pre_x[i];
       }
     };
-    // the x tile of iteration it + 1 goes to LDS in iteration it
+    // the x tile of iteration it + 2 goes to LDS in iteration it
     Place ahead = first;
     issue(ahead);
     store_x(0);
     advance(ahead);
     issue(ahead);
-    __syncthreads();                                     // x tile 0 is in LDS
+    store_x(1);
+    advance(ahead);
+    issue(ahead);
+    __syncthreads();                                     // x tiles 0 and 1 are in LDS
     Place at = first, done = first;                      // `done`: the tile the element waves finished last
+    int xw = 2;                                          // x buffer written in this iteration
     for (int it = 0; at.tile < n_tiles + n_wg; ++it) {
       const int prev = (it & 1) ^ 1;
-      store_x(prev);
+      store_x(xw);
+      xw = xw == 2 ? 0 : xw + 1;
       advance(ahead);
       issue(ahead);
       if (it > 0 && slab_ok) {
