@@ -69,7 +69,7 @@ def _timed(run, steps, warmup):
 
 def secondary_workload(args):
     """The configurations next to the headline one; see the module docstring."""
-    from griffin_amd import PreparedParams, hip_rglru, hip_rglru_step
+    from griffin_amd import PreparedParams, hip_rglru, hip_rglru_step, hip_rglru_steps
     from griffin_amd.modules import RMSNorm, RecurrentBlock
     from oracle import rglru_oracle as orc
 
@@ -98,21 +98,69 @@ def secondary_workload(args):
         metric, tokens = "RG-LRU fwd+bwd tokens/s", B * T
         workload = f"RG-LRU fwd+bwd B{B} T{T} W{W} nb{nb} bf16"
     elif name == "decode":
+        # 512 decode steps after a prefill, three ways: one eager launch per step (host-bound), a HIP
+        # graph of 64 single-step launches replayed 8 times (what a serving loop that samples between
+        # steps can do), and one launch for all 512 steps (inputs known in advance)
         B, T, W, nb, steps = 256, 2048, 1024, 8, 512
         case = orc.make_case(1, 1, W, nb, seed=0)
         params = [case[k].to(dt).to(dev) for k in ("w_a", "b_a", "w_x", "b_x", "lam")]
+        extra = {}
         with torch.no_grad():
-            _, state = hip_rglru(torch.randn(B, T, W, device=dev, dtype=dt), *params, 8.0)
-            state = state.contiguous()
+            _, state0 = hip_rglru(torch.randn(B, T, W, device=dev, dtype=dt), *params, 8.0)
+            state0 = state0.contiguous()
             prep = PreparedParams(*params, 8.0, dt)
             xs = torch.randn(steps, B, W, device=dev, dtype=dt)
+            state = state0.clone()
 
             def run():
                 for t in range(steps):
                     hip_rglru_step(xs[t], prep, state)
-            ms = _timed(run, max(args.steps // 10, 1), 1) / steps
+            ms_eager = _timed(run, max(args.steps // 10, 1), 1) / steps
+
+            per_graph = 64
+            ys = torch.empty(per_graph, B, W, device=dev, dtype=dt)
+            from griffin_amd import _lib as binding
+            lib = binding.load()
+            stream_of = lambda: torch.cuda.current_stream().cuda_stream
+            code = binding.RGLRU_BF16
+
+            def raw_steps(first):
+                for t in range(per_graph):
+                    lib.rglru_hip_step(xs[first + t].data_ptr(), prep.image.data_ptr(), state.data_ptr(), None,
+                                       ys[t].data_ptr(), B, W, nb, code, stream_of())
+            graphs = []
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                raw_steps(0)
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            for first in range(0, steps, per_graph):
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    raw_steps(first)
+                graphs.append(g)
+
+            def run_graphs():
+                for g in graphs:
+                    g.replay()
+            ms_graph = _timed(run_graphs, max(args.steps // 10, 1), 1) / steps
+            ms_multi = _timed(lambda: hip_rglru_steps(xs, prep, state), max(args.steps // 10, 1), 1) / steps
+            # state parity of the three ways from the same start
+            state.copy_(state0); run(); torch.cuda.synchronize(); s_eager = state.clone()
+            state.copy_(state0); run_graphs(); torch.cuda.synchronize(); s_graph = state.clone()
+            state.copy_(state0); hip_rglru_steps(xs, prep, state); torch.cuda.synchronize()
+            scale = s_eager.abs().max().item()
+            extra = {"us_per_token_eager": ms_eager * 1e3, "us_per_token_graph64": ms_graph * 1e3,
+                     "us_per_token_one_launch": ms_multi * 1e3,
+                     "bytes_per_step": B * W * (2 + 2 + 4 + 4) + 2 * (W // nb) * W * 2,
+                     "states_agree": bool((s_graph - s_eager).abs().max().item() <= 1e-6 * scale
+                                          and (state - s_eager).abs().max().item() <= 1e-6 * scale)}
+            extra["GBps_graph64"] = extra["bytes_per_step"] / (ms_graph * 1e-3) / 1e9
+            extra["GBps_one_launch"] = extra["bytes_per_step"] / (ms_multi * 1e-3) / 1e9
+            ms = ms_graph
         metric, tokens = "RG-LRU decode tokens/s", B
-        workload = f"RG-LRU decode B{B} W{W} nb{nb} bf16, {steps} steps after a T{T} prefill"
+        workload = f"RG-LRU decode B{B} W{W} nb{nb} bf16, {steps} steps after a T{T} prefill (HIP graph of 64 single-step launches)"
     else:
         B, D, W, steps = 256, 768, 1024, 64
         block = RecurrentBlock(D, W, scan_mode="hip").to(dev).to(dt).eval()
@@ -130,7 +178,8 @@ def secondary_workload(args):
     print(json.dumps({
         "metric": metric, "value": tokens / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic", "config": {"workload": workload, "launch": "eager"},
+        "dtype": "bf16", "data": "synthetic", "config": {"workload": workload, "launch": "eager" if name != "decode" else "hip graph"},
+        **({"decode": extra} if name == "decode" else {}),
     }))
 
 

@@ -6,6 +6,7 @@ from .hip_scan import (
     hip_rglru,
     hip_rglru_scan,
     hip_rglru_step,
+    hip_rglru_steps,
     hip_scan_available,
     hip_scan_is_usable,
 )
@@ -32,6 +33,7 @@ __all__ = [
     "hip_rglru",
     "hip_rglru_scan",
     "hip_rglru_step",
+    "hip_rglru_steps",
     "hip_scan_available",
     "hip_scan_is_usable",
 ]

@@ -14,7 +14,7 @@ RGLRU_BF16 = 1
 FLAG_RESET = 1
 FLAG_INACTIVE = 2
 CHUNK = 32
-ABI_VERSION = 10
+ABI_VERSION = 11
 
 _lock = threading.Lock()
 _lib = None
@@ -44,6 +44,7 @@ _SIGNATURES = {
     "rglru_hip_fwd_pre": (ctypes.c_int, [_P] * 8 + [_I, _I, _I, _I, ctypes.c_int, _P]),
     "rglru_hip_bwd_pre": (ctypes.c_int, [_P] * 15 + [_I, _I, _I, _I, ctypes.c_int, ctypes.c_int, _P]),
     "rglru_hip_step": (ctypes.c_int, [_P, _P, _P, _P, _P, _I, _I, _I, ctypes.c_int, _P]),
+    "rglru_hip_steps": (ctypes.c_int, [_P, _P, _P, _P, _P, _I, _I, _I, _I, ctypes.c_int, _P]),
     "rglru_hip_conv_max_kernel_size": (ctypes.c_int, []),
     "rglru_hip_conv_fwd": (ctypes.c_int, [_P] * 7 + [_I, _I, _I, _I, ctypes.c_int, ctypes.c_int, _P]),
     "rglru_hip_conv_scratch_bytes": (ctypes.c_size_t, [_I, _I, _I, _I]),

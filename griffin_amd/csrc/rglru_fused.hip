@@ -1782,6 +1782,98 @@ __global__ __launch_bounds__(kThreads) void step_kernel(FusedArgs p) {
   }
 }
 
+// K consecutive decode steps in one launch (teacher-forced inputs x[K, B, W]): the state stays in
+// registers across the steps, the gate weights are loaded once, and the next step's x tile is requested
+// while the current step is computed.  Same arithmetic as step_kernel, step by step.
+template <typename IO, int NKG>
+__global__ __launch_bounds__(kThreads) void steps_kernel(FusedArgs p) {
+  constexpr int MT = 1, TR = 32, EL = 16;
+  typedef Io<IO> Tr;
+  typedef typename Tr::Frag Frag;
+  constexpr int KC = NKG > 0 ? NKG * Tr::KG : Tr::KCMAX;
+  constexpr int LDSROW = KC + Tr::HW;
+  __shared__ __attribute__((aligned(16))) IO lds[TR * LDSROW];
+
+  const WaveId w = wave_identity(p, blockIdx.x);
+  const int hf = w.hf, tid = threadIdx.x;
+  const IO* wg = (const IO*)p.wg;
+  const IO* w_a_row = wg + ((long long)(0 * p.nb + w.k) * p.bwp + (w.slab_ok ? w.o : 0)) * p.bwp + hf * Tr::HW;
+  const IO* w_x_row = wg + ((long long)(1 * p.nb + w.k) * p.bwp + (w.slab_ok ? w.o : 0)) * p.bwp + hf * Tr::HW;
+  const float bias_a = p.bias[w.kp], bias_x = p.bias[p.Wp + w.kp];
+  const float sp = w.ch_ok ? p.sp[w.kp] : 0.f;
+  const long long W = p.W;
+  const long long row0 = (long long)w.wg_in_unit * TR;
+  const long long step_elems = (long long)p.B * W;
+  const int steps = p.T;
+
+  float h[EL];
+#pragma unroll
+  for (int e = 0; e < EL; ++e) {
+    const long long row = row0 + hf * EL + e;
+    h[e] = (w.ch_ok && row < p.B) ? p.h_prev[row * W + w.ch] : 0.f;
+  }
+  HeldWeights<IO, NKG> hw;
+  hw.load(w_a_row, w_x_row);
+  constexpr int VPR = KC / Tr::HW;
+  constexpr int NVX = NKG > 0 ? (TR * VPR + kThreads - 1) / kThreads : 1;
+  Frag pre[NVX];
+  auto issue = [&](int k) {
+    if constexpr (NKG > 0) {
+#pragma unroll
+      for (int i = 0; i < NVX; ++i) {
+        const int idx = tid + i * kThreads, row = idx / VPR, cv = idx - row * VPR;
+        pre[i] = Tr::zero();
+        if (idx < TR * VPR && k < steps)
+          pre[i] = load_x_frag<IO>(p, (const IO*)p.x + (long long)k * step_elems, row0 + row, p.B, w.k, cv * Tr::HW);
+      }
+    }
+  };
+  issue(0);
+  for (int k = 0; k < steps; ++k) {
+    unsigned fls[EL];
+#pragma unroll
+    for (int e = 0; e < EL; ++e) {
+      const long long row = row0 + hf * EL + e;
+      fls[e] = (p.flags && w.ch_ok && row < p.B) ? (unsigned)p.flags[(long long)k * p.B + row] : 0u;
+    }
+    f32x16 ua[MT], ux[MT];
+    float xv[EL];
+    if constexpr (NKG > 0) {
+#pragma unroll
+      for (int i = 0; i < NVX; ++i) {
+        const int idx = tid + i * kThreads, row = idx / VPR, cv = idx - row * VPR;
+        if (idx < TR * VPR) *reinterpret_cast<Frag*>(lds + row * LDSROW + cv * Tr::HW) = pre[i];
+      }
+      __syncthreads();
+      issue(k + 1);
+      if (w.slab_ok) gate_mfma_held<IO, MT, NKG>(lds, hw, 0, w.slab, w.r, hf, bias_a, bias_x, ua[0], ux[0], xv);
+      __syncthreads();                                   // the tile is overwritten at the top of the next step
+    } else {
+      gate_tile_generic<IO, MT>(p, (const IO*)p.x + (long long)k * step_elems, row0, p.B, w.k, w.slab, w.slab_ok,
+                                w_a_row, w_x_row, bias_a, bias_x, lds, ua, ux, xv);
+    }
+    if (w.ch_ok) {
+      IO* y = (IO*)p.y + (long long)k * step_elems;
+#pragma unroll
+      for (int e = 0; e < EL; ++e) {
+        const long long row = row0 + hf * EL + e;
+        if (row < p.B) {
+          GateOut go = gate_forward<Precise<IO>::value, true>(ua[0][e], ux[0][e], xv[e], sp, fls[e]);
+          h[e] = fmaf(go.a, h[e], go.z);
+          y[row * W + w.ch] = (IO)h[e];
+        }
+      }
+    }
+  }
+  if (w.ch_ok) {
+#pragma unroll
+    for (int e = 0; e < EL; ++e) {
+      const long long row = row0 + hf * EL + e;
+      if (row < p.B) p.h_state[row * W + w.ch] = h[e];
+    }
+  }
+}
+
 // ------------------------------------------------------------------------------------------
 // Host side
 // ------------------------------------------------------------------------------------------
@@ -2314,6 +2406,30 @@ int rglru_hip_step(const void* x, const void* prep, float* h, const uint8_t* fla
 int rglru_hip_step_gated(const void* x, const void* prep, const float* h_in, float* h_out, const uint8_t* flags,
                          const void* v, void* out, int64_t B, int64_t W, int64_t nb, int dtype, void* stream) {
   return step_impl(x, prep, h_in, h_out, flags, v, out, B, W, nb, dtype, stream);
+}
+
+int rglru_hip_steps(const void* x, const void* prep, float* h, const uint8_t* flags, void* y,
+                    int64_t K, int64_t B, int64_t W, int64_t nb, int dtype, void* stream) {
+  int rc = check_geometry("steps", W, nb, dtype);
+  if (rc) return rc;
+  if (B <= 0 || K <= 0) return fail(RGLRU_E_ARG, "steps: K and B must be positive (got %lld, %lld)", (long long)K, (long long)B);
+  if (!x || !prep || !h || !y) return fail(RGLRU_E_ARG, "steps: null pointer");
+  if (K * B * W >= (1ll << 40) || K >= (1ll << 31)) return fail(RGLRU_E_UNSUPPORTED, "steps: tensor too large");
+  Geometry g = make_geometry(W, nb);
+  FusedArgs a;
+  memset(&a, 0, sizeof(a));
+  fill_common(a, g, prep, dtype);
+  a.x = x; a.flags = flags; a.y = y; a.h_state = h; a.h_prev = h;
+  a.B = (int)B; a.T = (int)K;
+  a.aligned = is_aligned(x, W, g.bw, elem_size(dtype));
+  long long row_tiles = (B + 31) / 32;
+  dim3 grid((unsigned)(row_tiles * g.units));
+  hipStream_t s = (hipStream_t)stream;
+  {
+    KernelTimer timer(2, s);
+    RGLRU_DISPATCH(steps_kernel, grid, s, a, dtype, held_groups(g, dtype, a.aligned));
+  }
+  return check_launch("steps");
 }
 
 int rglru_hip_set_timing(int enable) { return g_timing.exchange(enable ? 1 : 0); }

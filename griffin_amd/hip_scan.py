@@ -342,6 +342,32 @@ def hip_rglru_step(x: Tensor, prep: PreparedParams, state: Tensor, flags: Tensor
     return y
 
 
+def hip_rglru_steps(xs: Tensor, prep: PreparedParams, state: Tensor, flags: Tensor | None = None) -> Tensor:
+    """K decode steps in one launch for inputs known in advance: ``xs`` [K, B, W]; ``state`` [B, W] fp32
+    is updated in place to the state after the last step; returns y [K, B, W] in xs.dtype (the result
+    of K calls of ``hip_rglru_step``)."""
+    _require_gpu("hip RG-LRU steps", xs, state, flags)
+    if xs.dim() != 3 or xs.shape[2] != prep.width:
+        raise ValueError(f"steps expects x of shape [steps, batch, {prep.width}], got {tuple(xs.shape)}")
+    if state.shape != xs.shape[1:] or state.dtype != torch.float32 or not state.is_contiguous():
+        raise ValueError("steps expects a contiguous fp32 state of shape [batch, width]")
+    if flags is not None and (flags.shape != xs.shape[:2] or flags.dtype != torch.uint8):
+        raise ValueError("flags must be uint8 of shape [steps, batch]")
+    if xs.dtype != prep.dtype:
+        raise TypeError(f"parameters were prepared for {prep.dtype}, got activations in {xs.dtype}")
+    lib = _lib.load()
+    xs = xs.contiguous()
+    K, B, _ = xs.shape
+    with torch.cuda.device(xs.device):
+        ys = torch.empty_like(xs)
+        if K > 0 and B > 0:
+            _lib.check(lib.rglru_hip_steps(xs.data_ptr(), prep.image.data_ptr(), state.data_ptr(),
+                                           None if flags is None else flags.contiguous().data_ptr(), ys.data_ptr(),
+                                           K, B, prep.width, prep.blocks, _dtype_code(xs.dtype), _stream_ptr(xs.device)),
+                       "rglru_hip_steps")
+    return ys
+
+
 # ----------------------------------------------------------------------------------------------
 # one-time self-test (reference: griffin/triton_scan.py:130-204)
 # ----------------------------------------------------------------------------------------------

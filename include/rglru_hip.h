@@ -46,7 +46,7 @@
 extern "C" {
 #endif
 
-#define RGLRU_ABI_VERSION 10
+#define RGLRU_ABI_VERSION 11
 
 enum { RGLRU_F32 = 0, RGLRU_BF16 = 1 };
 
@@ -190,6 +190,14 @@ int rglru_hip_bwd_pre(const void* x, const void* pre, const void* prep, const fl
 /* One decode step (T == 1): h[B,W] fp32 is updated in place, y[B,W] (dtype) = h as stored. */
 int rglru_hip_step(const void* x, const void* prep, float* h, const uint8_t* flags, void* y,
                    int64_t B, int64_t W, int64_t nb, int dtype, void* stream);
+
+/* K consecutive decode steps in one launch, for inputs that are known in advance (scoring a given
+ * continuation, speculative verification, replaying a prefix token by token): x[K,B,W] and y[K,B,W]
+ * (dtype), flags[K,B] or NULL, h[B,W] fp32 updated in place to the state after the last step.  The
+ * same arithmetic as K calls of rglru_hip_step (griffin/griffin.py:279-284 with T == 1, K times), with
+ * the state in registers and the weights loaded once. */
+int rglru_hip_steps(const void* x, const void* prep, float* h, const uint8_t* flags, void* y,
+                    int64_t K, int64_t B, int64_t W, int64_t nb, int dtype, void* stream);
 
 /* Causal depthwise temporal convolution that feeds the RG-LRU inside the recurrent block, all
  * tokens active (griffin/griffin.py:474-487):

@@ -310,6 +310,37 @@ def test_step_kernel_matches_oracle(dtype, tol):
     assert rel_err(got, ry) < tol and rel_err(state, rh) < tol
 
 
+@pytest.mark.parametrize("dtype,tol,shape", [(torch.float32, FP32_TOL, (5, 96, 3, 6)), (torch.bfloat16, BF16_TOL, (5, 96, 3, 6)),
+                                             (torch.bfloat16, BF16_TOL, (70, 256, 2, 33)), (torch.bfloat16, BF16_TOL, (3, 128, 2, 5))])
+def test_multi_step_kernel_matches_oracle_and_single_steps(dtype, tol, shape):
+    """K steps in one launch (rglru_hip_steps): against the oracle's sequence run, and against K calls of
+    the single-step kernel (same arithmetic step by step: equal up to nothing but the order of
+    identical operations, so the comparison is tight); one reset and one inactive token on the way."""
+    from griffin_amd import PreparedParams, hip_rglru_step, hip_rglru_steps
+
+    B, W, nb, steps = shape
+    case = orc.make_case(B, steps, W, nb, seed=4, h0_std=0.5, bias_std=0.5)
+    p = [case[k].to(dtype) for k in PARAMS]
+    prep = PreparedParams(*[t.cuda() for t in p[1:]], 8.0, dtype)
+    reset = torch.zeros(B, steps, dtype=torch.bool)
+    reset[0, steps // 2] = True
+    active = torch.ones(B, steps, dtype=torch.bool)
+    active[B - 1, steps - 1] = False
+    flags = (reset.to(torch.uint8) + 2 * (~active).to(torch.uint8)).t().contiguous().cuda()      # [K, B]
+    xs = p[0].transpose(0, 1).contiguous().cuda()                                                 # [K, B, W]
+    state = case["h0"].float().cuda().clone()
+    ys = hip_rglru_steps(xs, prep, state, flags)
+    single_state = case["h0"].float().cuda().clone()
+    singles = [hip_rglru_step(xs[t], prep, single_state, flags[t]) for t in range(steps)]
+    torch.cuda.synchronize()
+    ry, rh = orc.rglru_forward(*[t.float() for t in p], h0=case["h0"].float(), reset_mask=reset, active_mask=active)
+    got = ys.transpose(0, 1).float()
+    _say("steps", dtype, shape, "y err %.2e state err %.2e" % (rel_err(got, ry), rel_err(state, rh)))
+    assert rel_err(got, ry) < tol and rel_err(state, rh) < tol
+    assert rel_err(ys.float(), torch.stack(singles).float()) < 1e-6
+    assert rel_err(state, single_state) < 1e-6
+
+
 @pytest.mark.skip(reason="the process died with a host segmentation fault inside torch.cuda.graph's capture_end the "
                          "one time this test ran (no GPU fault was reported); bench.py captures and replays the same "
                          "step without trouble; cause not found, so the case stays off the GPU")
