@@ -51,7 +51,7 @@ def parse_args():
     ap.add_argument("--seq", type=int, default=2048)
     ap.add_argument("--width", type=int, default=1024)
     ap.add_argument("--blocks", type=int, default=8)
-    ap.add_argument("--workload", default="rglru", choices=["rglru", "block", "long_context", "decode", "block_decode"])
+    ap.add_argument("--workload", default="rglru", choices=["rglru", "block", "long_context", "decode", "block_decode", "scan_only"])
     return ap.parse_args()
 
 
@@ -88,6 +88,54 @@ def secondary_workload(args):
         ms = _timed(lambda: torch.autograd.grad(block(norm(x)), leaves, dy), args.steps, args.warmup)
         metric, tokens = "RMSNorm + RecurrentBlock fwd+bwd tokens/s", B * T
         workload = f"RMSNorm + RecurrentBlock({D}, {W}) fwd+bwd B{B} T{T} bf16"
+    elif name == "scan_only":
+        # the scan-only operator (contract of the reference's fused_rglru_scan: fp32 a, z, h0 -> h) at the
+        # benchmark shape: forward reads a, z and writes h (12 N bytes), backward reads a, dh, h and writes
+        # da, dz (20 N bytes).  HIP graph of ten steps, median of five timed regions.
+        from griffin_amd import hip_rglru_scan
+
+        B, T, W = 8, 2048, 1024
+        gen = torch.Generator(device=dev).manual_seed(0)
+        a = torch.sigmoid(torch.randn(B, T, W, device=dev, generator=gen) + 2.0).requires_grad_(True)
+        z = torch.randn(B, T, W, device=dev, generator=gen).requires_grad_(True)
+        h0 = torch.randn(B, W, device=dev, generator=gen).requires_grad_(True)
+        dh = torch.randn(B, T, W, device=dev, generator=gen)
+
+        def one():
+            return torch.autograd.grad(hip_rglru_scan(a, z, h0), [a, z, h0], dh)
+        for _ in range(3):
+            one()
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            one()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        per_graph = 10
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            kept = [one() for _ in range(per_graph)]
+        samples = []
+        for _ in range(6):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(max(args.steps // per_graph, 1)):
+                graph.replay()
+            torch.cuda.synchronize()
+            samples.append((time.perf_counter() - t0) * 1e3 / (max(args.steps // per_graph, 1) * per_graph))
+        ms = _median(samples[1:])
+        n = B * T * W
+        gbps = 32.0 * n / (ms * 1e-3) / 1e9
+        print(json.dumps({
+            "metric": "RG-LRU scan-only fwd+bwd tokens/s", "value": B * T / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+            "config": {"workload": f"scan-only operator fwd+bwd B{B} T{T} W{W} fp32", "launch": f"hip graph replay, {per_graph} steps per graph"},
+            "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBS,
+                         "traffic": None, "algorithmic_bytes": 32 * n},
+        }))
+        return
     elif name == "long_context":
         B, T, W, nb = 1, 32768, 2560, 8
         case = orc.make_case(B, T, W, nb, seed=0, lo=0.99, hi=0.9999)

@@ -113,11 +113,13 @@ inline ScratchLayout make_scratch_layout(int64_t B, int64_t T, const Geometry& g
   return s;
 }
 
-// Scan-only workspace: chunks of 32 tokens; everything is cleared before each pass.
-//   rec_a [B][nC][W] 64-bit carry records; ticket [B][groups]; fail.
+// Scan-only workspace; what a pass uses is cleared at its start.  Tickets and the failure word come
+// first, so that the clearing launch covers them and only as many records as the kernel variant needs
+// (one per sequence, channel and 32-token chunk, or one per 128-token run of the vector kernels).
+//   ticket [B][groups]; fail; rec_a [B][nC][W] 64-bit carry records.
 struct ScanLayout {
   int64_t nC, groups;
-  size_t rec_a, ticket, fail, total;
+  size_t ticket, fail, rec_a, total;
 };
 
 inline ScanLayout make_scan_layout(int64_t B, int64_t T, int64_t W) {
@@ -126,9 +128,9 @@ inline ScanLayout make_scan_layout(int64_t B, int64_t T, int64_t W) {
   s.groups = (W + 63) / 64;
   size_t off = 0;
   auto take = [&](int64_t bytes) { size_t at = off; off += (size_t)round_up(bytes, 256); return at; };
-  s.rec_a = take(B * s.nC * W * 8);
   s.ticket = take(B * s.groups * 4);
   s.fail = take(4);
+  s.rec_a = take(B * s.nC * W * 8);
   s.total = off;
   return s;
 }

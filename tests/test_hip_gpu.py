@@ -20,7 +20,8 @@ def _say(*args):
 
 
 # ------------------------------------------------------------------ scan-only operator
-@pytest.mark.parametrize("shape", [(2, 37, 65), (1, 7, 257), (3, 300, 130), (2, 1, 64), (1, 1025, 32)])
+@pytest.mark.parametrize("shape", [(2, 37, 65), (1, 7, 257), (3, 300, 130), (2, 1, 64), (1, 1025, 32),
+                                   (2, 300, 260), (3, 129, 1024), (1, 4100, 64), (9, 128, 256)])
 def test_scan_op_matches_loop(shape):
     from griffin_amd import hip_rglru_scan
 
