@@ -449,7 +449,8 @@ struct PaddedArgs {
   const void* u; const void* state; const void* taps; const void* bias;
   const long long* segpos; const unsigned char* active;
   void* out; void* new_state; int* scratch;
-  int B, T, W, K, nvec, vec_dtype;
+  const void* dout; void* du; void* dstate; float* partial;   // backward
+  int B, T, W, K, nvec, runs, vec_dtype;
 };
 
 __global__ __launch_bounds__(64) void conv_padded_index_kernel(PaddedArgs p) {
@@ -551,6 +552,134 @@ __global__ __launch_bounds__(kConvThreads) void conv_padded_fwd_kernel(PaddedArg
     }
   }
   ConvRow<IO, V>::store(acc, ro, off);
+}
+
+// Reverse mode of the padded convolution.  In ordinal space (the active tokens of a row in order) the
+// forward pass is a plain causal convolution whose taps are cut at the output's document start, so the
+// gradient of the input at ordinal j collects the outputs at ordinals j .. j + K - 1 whose document
+// started at or before j; the carried state rows stand at ordinals -(K-1) .. -1 and feed only outputs
+// without a document start in front of them.  Threads are laid out as in conv_bwd_kernel (a thread owns
+// a run of kConvRunBwd consecutive tokens of one channel vector; tap and bias gradients are summed per
+// workgroup and written as one partial row per (sequence, group of runs)).
+template <typename IO, int V, int K>
+__global__ __launch_bounds__(kConvThreads) void conv_padded_bwd_kernel(PaddedArgs p) {
+  __shared__ float red[kConvBwdRuns][(K + 1) * V][kConvBwdVecs + 1];
+  const int vec_groups = (p.nvec + kConvBwdVecs - 1) / kConvBwdVecs;
+  const int run_groups = (p.runs + kConvBwdRuns - 1) / kConvBwdRuns;
+  const int vg = blockIdx.x % vec_groups;
+  const int rest = blockIdx.x / vec_groups;
+  const int rgp = rest % run_groups, b = rest / run_groups;
+  const int lane_vec = threadIdx.x % kConvBwdVecs, lane_run = threadIdx.x / kConvBwdVecs;
+  const int vec = vg * kConvBwdVecs + lane_vec, run = rgp * kConvBwdRuns + lane_run;
+  const bool ok = vec < p.nvec && run < p.runs;
+  const int c0 = (vec < p.nvec ? vec : 0) * V, t0 = run * kConvRunBwd;
+  const unsigned es = (unsigned)sizeof(IO), uW = (unsigned)p.W;
+  const int* ord = p.scratch + (long long)b * p.T;
+  const int* start = p.scratch + ((long long)p.B + b) * p.T;
+  const int* list = p.scratch + (2ll * p.B + b) * p.T;
+  const int* tail = p.scratch + 3ll * p.B * p.T;
+  const int n = tail[b];                                   // active tokens of the row
+  float tap[K][V], bias_unused[V];
+  conv_load_taps<V, K>(p.taps, nullptr, c0, p.vec_dtype, tap, bias_unused);
+  const unsigned seq_bytes = ok ? (unsigned)p.T * uW * es : 0u;
+  const rsrc_t ru = make_rsrc((const IO*)p.u + (long long)b * p.T * p.W, seq_bytes);
+  const rsrc_t rd = make_rsrc((const IO*)p.dout + (long long)b * p.T * p.W, seq_bytes);
+  const rsrc_t rg = make_rsrc((const IO*)p.du + (long long)b * p.T * p.W, seq_bytes);
+  const rsrc_t rs = make_rsrc(p.state ? (const IO*)p.state + (long long)b * (K - 1) * p.W : (const IO*)p.u,
+                              (p.state && ok) ? (unsigned)((K - 1) * p.W) * es : 0u);
+  float acc_tap[K][V], acc_bias[V];
+#pragma unroll
+  for (int v = 0; v < V; ++v) {
+    acc_bias[v] = 0.f;
+#pragma unroll
+    for (int j = 0; j < K; ++j) acc_tap[j][v] = 0.f;
+  }
+  for (int t1 = 0; t1 < kConvRunBwd; ++t1) {
+    const int t = t0 + t1;
+    if (!ok || t >= p.T) break;
+    const unsigned off = ((unsigned)t * uW + (unsigned)c0) * es;
+    const int i = ord[t];
+    float g[V];
+#pragma unroll
+    for (int v = 0; v < V; ++v) g[v] = 0.f;
+    if (i >= 0) {
+      // input gradient: ordinal i feeds the outputs at ordinals i .. i + K - 1 of its document
+#pragma unroll
+      for (int lag = 0; lag < K; ++lag) {
+        const int i2 = i + lag;
+        if (i2 < n) {
+          const int t2 = list[i2];
+          if (start[t2] <= i) {
+            float d[V];
+            ConvRow<IO, V>::load(d, rd, ((unsigned)t2 * uW + (unsigned)c0) * es);
+#pragma unroll
+            for (int v = 0; v < V; ++v) g[v] = fmaf(d[v], tap[K - 1 - lag][v], g[v]);
+          }
+        }
+      }
+      // parameter gradients of the output at this token
+      float d[V];
+      ConvRow<IO, V>::load(d, rd, off);
+      const int doc_start = start[t];
+#pragma unroll
+      for (int v = 0; v < V; ++v) acc_bias[v] += d[v];
+#pragma unroll
+      for (int lag = 0; lag < K; ++lag) {
+        float row[V];
+        padded_source<IO, V, K>(p, ru, rs, list, i, lag, doc_start, c0, row);
+#pragma unroll
+        for (int v = 0; v < V; ++v) acc_tap[K - 1 - lag][v] = fmaf(d[v], row[v], acc_tap[K - 1 - lag][v]);
+      }
+    }
+    ConvRow<IO, V>::store(g, rg, off);
+  }
+
+  // gradient at the carried state: row j stands at ordinal j - (K - 1) < 0
+  if (K > 1 && p.dstate && ok && run == 0) {
+    const rsrc_t rds = make_rsrc((IO*)p.dstate + (long long)b * (K - 1) * p.W, (unsigned)((K - 1) * p.W) * es);
+#pragma unroll
+    for (int j = 0; j < K - 1; ++j) {
+      const int tau = j - (K - 1);
+      float a[V];
+#pragma unroll
+      for (int v = 0; v < V; ++v) a[v] = 0.f;
+#pragma unroll
+      for (int lag = 1; lag < K; ++lag) {
+        const int i2 = tau + lag;
+        if (i2 >= 0 && i2 < n) {
+          const int t2 = list[i2];
+          if (start[t2] < 0) {
+            float d[V];
+            ConvRow<IO, V>::load(d, rd, ((unsigned)t2 * uW + (unsigned)c0) * es);
+#pragma unroll
+            for (int v = 0; v < V; ++v) a[v] = fmaf(d[v], tap[K - 1 - lag][v], a[v]);
+          }
+        }
+      }
+      ConvRow<IO, V>::store(a, rds, ((unsigned)j * uW + (unsigned)c0) * es);
+    }
+  }
+
+  // sums of the workgroup's runs (threads without work hold zeros)
+#pragma unroll
+  for (int j = 0; j < K; ++j)
+#pragma unroll
+    for (int v = 0; v < V; ++v) red[lane_run][j * V + v][lane_vec] = acc_tap[j][v];
+#pragma unroll
+  for (int v = 0; v < V; ++v) red[lane_run][K * V + v][lane_vec] = acc_bias[v];
+  __syncthreads();
+  float* part = p.partial + ((long long)(b * run_groups + rgp) * (K + 1)) * p.W;
+  for (int idx = threadIdx.x; idx < (K + 1) * V * kConvBwdVecs; idx += kConvThreads) {
+    const int row = idx / kConvBwdVecs, lv = idx - row * kConvBwdVecs;   // row = j * V + v
+    const int j = row / V, v = row - j * V;
+    const int ch = (vg * kConvBwdVecs + lv) * V + v;
+    if (ch < p.W) {
+      float sum = 0.f;
+#pragma unroll
+      for (int q = 0; q < kConvBwdRuns; ++q) sum += red[q][row][lv];
+      part[(long long)j * p.W + ch] = sum;
+    }
+  }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -959,6 +1088,47 @@ int rglru_hip_conv_bwd(const void* u, const void* state, const void* taps, const
     const long long n = (long long)(K + 1) * W;
     hipLaunchKernelGGL(conv_finish_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, f);
     rc = check_launch("conv_bwd finish");
+  }
+  return rc;
+}
+
+int rglru_hip_conv_padded_bwd(const void* u, const void* state, const void* taps,
+                              const int64_t* segment_pos, const uint8_t* active, const void* dout,
+                              void* index_scratch, void* scratch, void* du, void* dstate, void* dtaps, void* dbias,
+                              int64_t B, int64_t T, int64_t W, int64_t K, int dtype, int vec_dtype, int grad_dtype,
+                              void* stream) {
+  int rc = conv_check("conv_padded_bwd", B, T, W, K, dtype, vec_dtype);
+  if (rc) return rc;
+  if (grad_dtype != RGLRU_F32 && grad_dtype != RGLRU_BF16) return fail(RGLRU_E_ARG, "conv_padded_bwd: unknown gradient dtype %d", grad_dtype);
+  if (!u || !taps || !segment_pos || !active || !dout || !index_scratch || !scratch || !du)
+    return fail(RGLRU_E_ARG, "conv_padded_bwd: null pointer");
+  if (B * T >= (1ll << 29)) return fail(RGLRU_E_UNSUPPORTED, "conv_padded_bwd: tensor too large");
+  PaddedArgs a;
+  memset(&a, 0, sizeof(a));
+  a.u = u; a.state = state; a.taps = taps; a.segpos = (const long long*)segment_pos; a.active = active;
+  a.scratch = (int*)index_scratch; a.dout = dout; a.du = du; a.dstate = dstate; a.partial = (float*)scratch;
+  a.B = (int)B; a.T = (int)T; a.W = (int)W; a.K = (int)K; a.vec_dtype = vec_dtype;
+  const bool vec = conv_vector_ok(W, dtype, {u, state, dout, du, dstate});
+  a.nvec = (int)(vec ? W / (dtype == RGLRU_BF16 ? 8 : 4) : W);
+  a.runs = (int)((T + kConvRunBwd - 1) / kConvRunBwd);
+  hipStream_t s = (hipStream_t)stream;
+  hipLaunchKernelGGL(conv_padded_index_kernel, dim3((unsigned)B), dim3(64), 0, s, a);
+  rc = check_launch("conv_padded_bwd index");
+  if (rc) return rc;
+  const long long run_groups = (a.runs + kConvBwdRuns - 1) / kConvBwdRuns;
+  const long long vec_groups = (a.nvec + kConvBwdVecs - 1) / kConvBwdVecs;
+  if (B * run_groups * vec_groups >= (1ll << 31)) return fail(RGLRU_E_UNSUPPORTED, "conv_padded_bwd: tensor too large");
+  dim3 grid((unsigned)(B * run_groups * vec_groups));
+  RGLRU_CONV_DISPATCH(conv_padded_bwd_kernel, dtype, vec, grid, s, a);
+  rc = check_launch("conv_padded_bwd");
+  if (rc) return rc;
+  if (dtaps || dbias) {
+    ConvFinishArgs f;
+    f.partial = a.partial; f.dtaps = dtaps; f.dbias = dbias; f.W = (int)W; f.K = (int)K;
+    f.slots = (int)(B * run_groups); f.grad_dtype = grad_dtype;
+    const long long n = (long long)(K + 1) * W;
+    hipLaunchKernelGGL(conv_finish_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, f);
+    rc = check_launch("conv_padded_bwd finish");
   }
   return rc;
 }

@@ -120,40 +120,87 @@ def hip_causal_conv(u: Tensor, state: Tensor | None, weight: Tensor, bias: Tenso
     return out, new_state
 
 
+class _HipCausalConvPadded(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, u: Tensor, state: Tensor | None, weight: Tensor, bias: Tensor | None,
+                segment_pos: Tensor, active_mask: Tensor):
+        _require_gpu("hip_causal_conv_padded", u, state, weight, bias, segment_pos, active_mask)
+        if u.dim() != 3:
+            raise ValueError(f"hip_causal_conv_padded expects [batch, sequence, width], got {tuple(u.shape)}")
+        batch, steps, width = u.shape
+        if weight.dim() != 3 or weight.size(0) != width or weight.size(1) != 1:
+            raise ValueError("weight must be that of a depthwise Conv1d: [width, 1, kernel_size]")
+        taps_count = weight.size(2)
+        if state is not None and state.shape != (batch, taps_count - 1, width):
+            raise ValueError("state must have shape [batch, kernel_size - 1, width]")
+        if segment_pos.shape != (batch, steps) or active_mask.shape != (batch, steps):
+            raise ValueError("segment_pos and active_mask must have shape [batch, sequence]")
+        code = _dtype_code(u.dtype)
+        u_c = u.contiguous()
+        state_c = None if state is None or taps_count == 1 else state.to(u.dtype).contiguous()
+        taps = _parameter_operand(weight, u.dtype)
+        bias_c = None if bias is None else _parameter_operand(bias.to(taps.dtype), u.dtype)
+        pos = segment_pos.to(device=u.device, dtype=torch.int64).contiguous()
+        live = active_mask.to(device=u.device, dtype=torch.uint8).contiguous()
+        lib = _lib.load()
+        with torch.cuda.device(u.device):
+            out = torch.empty_like(u_c)
+            new_state = u.new_empty(batch, taps_count - 1, width)
+            scratch = torch.empty(lib.rglru_hip_conv_padded_scratch_bytes(batch, steps), dtype=torch.uint8, device=u.device)
+            _lib.check(lib.rglru_hip_conv_padded_fwd(
+                _ptr(u_c), _ptr(state_c), _ptr(taps), _ptr(bias_c), _ptr(pos), _ptr(live), _ptr(scratch), _ptr(out),
+                _ptr(new_state) if taps_count > 1 else None,
+                batch, steps, width, taps_count, code, _DTYPE_CODES[taps.dtype], _stream_ptr(u.device)),
+                "rglru_hip_conv_padded_fwd")
+        ctx.save_for_backward(u_c, state_c, taps, pos, live)
+        ctx.meta = (None if state is None else state.dtype, weight.dtype, None if bias is None else bias.dtype, weight.shape)
+        ctx.mark_non_differentiable(new_state)
+        ctx.set_materialize_grads(False)
+        return out, new_state
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, dout: Tensor | None, _dstate_out):
+        u, state, taps, pos, live = ctx.saved_tensors
+        state_dtype, weight_dtype, bias_dtype, weight_shape = ctx.meta
+        if dout is None:
+            return None, None, None, None, None, None
+        batch, steps, width = u.shape
+        taps_count = weight_shape[2]
+        dout_c = dout.to(u.dtype).contiguous()
+        lib = _lib.load()
+        need_u, need_state, need_w, need_b = ctx.needs_input_grad[:4]
+        grad_dtype = taps.dtype
+        with torch.cuda.device(u.device):
+            du = torch.empty_like(u)
+            dstate = u.new_empty(batch, taps_count - 1, width) if (need_state and taps_count > 1) else None
+            dtaps = torch.empty(width, taps_count, device=u.device, dtype=grad_dtype) if need_w else None
+            dbias = torch.empty(width, device=u.device, dtype=grad_dtype) if (need_b and bias_dtype is not None) else None
+            index = torch.empty(lib.rglru_hip_conv_padded_scratch_bytes(batch, steps), dtype=torch.uint8, device=u.device)
+            scratch = torch.empty(lib.rglru_hip_conv_scratch_bytes(batch, steps, width, taps_count),
+                                  device=u.device, dtype=torch.uint8)
+            _lib.check(lib.rglru_hip_conv_padded_bwd(
+                _ptr(u), _ptr(state), _ptr(taps), _ptr(pos), _ptr(live), _ptr(dout_c), _ptr(index), _ptr(scratch),
+                _ptr(du), _ptr(dstate), _ptr(dtaps), _ptr(dbias),
+                batch, steps, width, taps_count, _dtype_code(u.dtype), _DTYPE_CODES[taps.dtype],
+                _DTYPE_CODES[grad_dtype], _stream_ptr(u.device)), "rglru_hip_conv_padded_bwd")
+        dweight = None if dtaps is None else dtaps.view(weight_shape).to(weight_dtype)
+        if dbias is not None:
+            dbias = dbias.to(bias_dtype)
+        if need_state and state_dtype is not None:
+            dstate = (u.new_zeros(batch, taps_count - 1, width) if dstate is None else dstate).to(state_dtype)
+        else:
+            dstate = None
+        return (du if need_u else None), dstate, dweight, dbias, None, None
+
+
 def hip_causal_conv_padded(u: Tensor, state: Tensor | None, weight: Tensor, bias: Tensor | None,
                            segment_pos: Tensor, active_mask: Tensor) -> tuple[Tensor, Tensor]:
-    """The convolution over right-padded batches (griffin/griffin.py:488-510), forward only (no
-    autograd): inactive tokens give zeros and stay out of the window of previous inputs, an active
-    token at position 0 clears the window.  Returns ``(out [B, T, W], new_state [B, K-1, W])``."""
-    _require_gpu("hip_causal_conv_padded", u, state, weight, bias, segment_pos, active_mask)
-    if u.dim() != 3:
-        raise ValueError(f"hip_causal_conv_padded expects [batch, sequence, width], got {tuple(u.shape)}")
-    batch, steps, width = u.shape
-    if weight.dim() != 3 or weight.size(0) != width or weight.size(1) != 1:
-        raise ValueError("weight must be that of a depthwise Conv1d: [width, 1, kernel_size]")
-    taps_count = weight.size(2)
-    if state is not None and state.shape != (batch, taps_count - 1, width):
-        raise ValueError("state must have shape [batch, kernel_size - 1, width]")
-    if segment_pos.shape != (batch, steps) or active_mask.shape != (batch, steps):
-        raise ValueError("segment_pos and active_mask must have shape [batch, sequence]")
-    code = _dtype_code(u.dtype)
-    u_c = u.detach().contiguous()
-    state_c = None if state is None or taps_count == 1 else state.detach().to(u.dtype).contiguous()
-    taps = _parameter_operand(weight.detach(), u.dtype)
-    bias_c = None if bias is None else _parameter_operand(bias.detach().to(taps.dtype), u.dtype)
-    pos = segment_pos.to(device=u.device, dtype=torch.int64).contiguous()
-    live = active_mask.to(device=u.device, dtype=torch.uint8).contiguous()
-    lib = _lib.load()
-    with torch.cuda.device(u.device):
-        out = torch.empty_like(u_c)
-        new_state = u.new_empty(batch, taps_count - 1, width)
-        scratch = torch.empty(lib.rglru_hip_conv_padded_scratch_bytes(batch, steps), dtype=torch.uint8, device=u.device)
-        _lib.check(lib.rglru_hip_conv_padded_fwd(
-            _ptr(u_c), _ptr(state_c), _ptr(taps), _ptr(bias_c), _ptr(pos), _ptr(live), _ptr(scratch), _ptr(out),
-            _ptr(new_state) if taps_count > 1 else None,
-            batch, steps, width, taps_count, code, _DTYPE_CODES[taps.dtype], _stream_ptr(u.device)),
-            "rglru_hip_conv_padded_fwd")
-    return out, new_state
+    """The convolution over right-padded batches (griffin/griffin.py:488-510): inactive tokens give zeros
+    and stay out of the window of previous inputs, an active token at position 0 clears the window.
+    Returns ``(out [B, T, W], new_state [B, K-1, W])``.  ``out`` is differentiable in ``u``, ``state``,
+    ``weight`` and ``bias``; ``new_state`` (the cache handed to the next call) carries no gradient."""
+    return _HipCausalConvPadded.apply(u, state, weight, bias, segment_pos, active_mask)
 
 
 class _HipGeluGate(torch.autograd.Function):

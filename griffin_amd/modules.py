@@ -362,9 +362,7 @@ class RecurrentBlock(nn.Module):
 
     def _padded_conv(self, projected: Tensor, conv_state: Tensor, segment_pos: Tensor, active_mask: Tensor):
         """Right-padded batches (griffin/griffin.py:488-510): padding never enters the history."""
-        needs_grad = torch.is_grad_enabled() and any(
-            t.requires_grad for t in (projected, conv_state, self.temporal_conv.weight, self.temporal_conv.bias))
-        if not needs_grad and self._hip_block_ops_covers(projected):
+        if self._hip_block_ops_covers(projected):
             return hip_block_ops.hip_causal_conv_padded(projected, conv_state, self.temporal_conv.weight,
                                                         self.temporal_conv.bias, segment_pos, active_mask)
         taps = self.temporal_conv.weight[:, 0, :]

@@ -14,7 +14,7 @@
  *   griffin/griffin.py:279-284 with T == 1 (decode step, carried state)     rglru_hip_step
  *   griffin/griffin.py:474-487      causal depthwise convolution of the caller   rglru_hip_conv_fwd
  *   autograd of griffin/griffin.py:474-487                                   rglru_hip_conv_bwd
- *   griffin/griffin.py:488-510      the same over right-padded batches (forward)   rglru_hip_conv_padded_fwd
+ *   griffin/griffin.py:488-510      the same over right-padded batches and its autograd   rglru_hip_conv_padded_fwd, _bwd
  *   griffin/griffin.py:464, :520    x_branch * gelu_tanh(linear_y(x))        rglru_hip_gelu_gate_fwd, _bwd
  *   griffin/griffin.py:68-80        RMSNorm in front of the block and its autograd   rglru_hip_rmsnorm_fwd, _bwd
  *   griffin/griffin.py:459-528 with T == 1 (block decode: positions, conv, step, gate)   rglru_hip_decode_prepare + rglru_hip_step_gated
@@ -46,7 +46,7 @@
 extern "C" {
 #endif
 
-#define RGLRU_ABI_VERSION 11
+#define RGLRU_ABI_VERSION 12
 
 enum { RGLRU_F32 = 0, RGLRU_BF16 = 1 };
 
@@ -222,16 +222,26 @@ int rglru_hip_conv_bwd(const void* u, const void* state, const void* taps, const
                        int64_t B, int64_t T, int64_t W, int64_t K, int dtype, int vec_dtype, int grad_dtype,
                        void* stream);
 
-/* The same convolution over right-padded batches (griffin/griffin.py:488-510), forward only: tokens
- * with active[b,t] == 0 produce zeros and never enter the window of the K-1 previous ACTIVE inputs; an
+/* The same convolution over right-padded batches (griffin/griffin.py:488-510): tokens with
+ * active[b,t] == 0 produce zeros and never enter the window of the K-1 previous ACTIVE inputs; an
  * active token with segment_pos == 0 clears that window (and the carried state) before it is used.
  * active[B,T] is one byte per token; new_state[B,K-1,W] (may be NULL) receives the window after the
- * last token; `scratch` holds rglru_hip_conv_padded_scratch_bytes(B, T) bytes. */
+ * last token; `scratch` holds rglru_hip_conv_padded_scratch_bytes(B, T) bytes.
+ * rglru_hip_conv_padded_bwd is its reverse mode (the reference gets it from autograd through a
+ * per-token Python loop): dout[B,T,W] in; du[B,T,W] (zero at inactive tokens), dstate[B,K-1,W],
+ * dtaps[W,K], dbias[W] out (the last three may be NULL).  `index_scratch` holds
+ * rglru_hip_conv_padded_scratch_bytes(B, T) bytes and `scratch` rglru_hip_conv_scratch_bytes(B, T, W, K)
+ * bytes; their contents on entry do not matter. */
 size_t rglru_hip_conv_padded_scratch_bytes(int64_t B, int64_t T);
 int rglru_hip_conv_padded_fwd(const void* u, const void* state, const void* taps, const void* bias,
                               const int64_t* segment_pos, const uint8_t* active, void* scratch,
                               void* out, void* new_state,
                               int64_t B, int64_t T, int64_t W, int64_t K, int dtype, int vec_dtype, void* stream);
+int rglru_hip_conv_padded_bwd(const void* u, const void* state, const void* taps,
+                              const int64_t* segment_pos, const uint8_t* active, const void* dout,
+                              void* index_scratch, void* scratch, void* du, void* dstate, void* dtaps, void* dbias,
+                              int64_t B, int64_t T, int64_t W, int64_t K, int dtype, int vec_dtype, int grad_dtype,
+                              void* stream);
 
 /* Output gate of the recurrent block, out = h * gelu_tanh(v) (griffin/griffin.py:464 and :520: the
  * GeLU of the second branch and the product with the RG-LRU output in one pass), flat over n

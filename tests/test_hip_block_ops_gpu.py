@@ -282,6 +282,40 @@ def test_padded_conv_all_active_equals_dense_kernel_at_training_shape():
     assert torch.equal(dense, padded)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("cfg", [(3, 50, 64, 4, "right"), (4, 200, 24, 4, "holes"), (2, 130, 13, 3, "holes"),
+                                 (3, 65, 128, 2, "right"), (2, 7, 16, 1, "holes"), (2, 300, 1024, 4, "holes")])
+def test_padded_conv_gradients_match_oracle_autograd(cfg, dtype):
+    """Reverse mode of the padded convolution (C ABI: rglru_hip_conv_padded_bwd) against autograd through
+    the oracle's token-by-token loop: gradients at the input, the carried state, the taps and the bias."""
+    from griffin_amd.hip_block_ops import hip_causal_conv_padded
+
+    B, T, W, K, pattern = cfg
+    _say("padded conv gradient case", cfg, dtype)
+    u, w, b, state, pos, active = _padded_inputs(B, T, W, K, seed=29, pattern=pattern)
+    dout = torch.randn(B, T, W, generator=torch.Generator().manual_seed(31))
+    up = lambda t: t.to(dtype).float()
+    ref = [up(t).clone().requires_grad_(True) for t in (u, w, b, state)]
+    want, _ = orc.causal_conv_padded(ref[0], ref[1], ref[2], ref[3], pos, active)
+    want.backward(up(dout))
+    dev = [u.to(dtype).cuda().requires_grad_(True), w.to(dtype)[:, None, :].contiguous().cuda().requires_grad_(True),
+           b.to(dtype).cuda().requires_grad_(True), state.to(dtype).cuda().requires_grad_(True)]
+    got, _ = hip_causal_conv_padded(dev[0], dev[3], dev[1], dev[2], pos.cuda(), active.cuda())
+    got.backward(dout.to(dtype).cuda())
+    torch.cuda.synchronize()
+    tol = FP32_TOL if dtype == torch.float32 else BF16_TOL
+    names = ("input", "taps", "bias", "state")
+    for name, r, d in zip(names, ref, dev):
+        if K == 1 and name == "state":
+            continue
+        grad = d.grad.float().cpu().reshape(r.grad.shape)
+        err = rel_err(grad, r.grad)
+        _say("  d%s rel error: %.2e" % (name, err))
+        assert err < tol, name
+    # padding receives no gradient at all
+    assert torch.count_nonzero(dev[0].grad[~active.cuda()]) == 0
+
+
 # ----------------------------------------------------------------------------------------------
 # RMSNorm in front of the block (C ABI: rglru_hip_rmsnorm_fwd / _bwd)
 # ----------------------------------------------------------------------------------------------

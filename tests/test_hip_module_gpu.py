@@ -343,6 +343,38 @@ def test_config5_recurrent_block_with_hip_scan():
     assert torch.isfinite(nxt).all()
 
 
+def test_recurrent_block_right_padded_batch_trains_on_hip_kernels():
+    """A right-padded batch with a packed second document (griffin/griffin.py:488-510): output, cache and
+    every gradient of the block on the HIP kernels against the same block on the CPU, whose padded
+    convolution is the token-by-token loop."""
+    from griffin_amd import RecurrentBlock
+
+    torch.manual_seed(9)
+    cpu_block = RecurrentBlock(96, 128, gate_blocks=4, scan_mode="sequential")
+    hip_block = copy.deepcopy(cpu_block).cuda()
+    hip_block.scan_mode = None
+    hip_block.rg_lru.scan_mode = "hip"
+    B, T = 3, 90
+    x = torch.randn(B, T, 96)
+    active = torch.arange(T)[None, :] < torch.tensor([T, 41, 0])[:, None]
+    pos = torch.arange(T).repeat(B, 1)
+    pos[0, 50:] -= 50                                        # a second document in the full row
+    xc = x.clone().requires_grad_(True)
+    xh = x.clone().cuda().requires_grad_(True)
+    up = torch.randn(B, T, 96)
+    yc, cache_c = cpu_block(xc, segment_pos=pos, active_mask=active, return_cache=True)
+    yh, cache_h = hip_block(xh, segment_pos=pos.cuda(), active_mask=active.cuda(), return_cache=True)
+    yc.backward(up)
+    yh.backward(up.cuda())
+    assert rel_err(yh, yc) < 1e-4
+    assert rel_err(cache_h.conv_state, cache_c.conv_state) < 1e-6
+    assert rel_err(cache_h.rnn_state, cache_c.rnn_state) < 1e-4
+    assert rel_err(xh.grad, xc.grad) < 1e-4
+    assert torch.count_nonzero(xh.grad[~active.cuda()]) == 0
+    for (name, ph), (_, pc) in zip(hip_block.named_parameters(), cpu_block.named_parameters()):
+        assert rel_err(ph.grad, pc.grad) < 2e-4, name
+
+
 def test_config5_recurrent_block_bf16_matches_fp32_oracle():
     """Config 5 at its stated storage type: RMSNorm(768) + RecurrentBlock(768, 1024), 8 gate blocks, bf16
     parameters and activations on the HIP kernels, T = 2048, against the oracle's block
