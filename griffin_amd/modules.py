@@ -312,8 +312,11 @@ class RecurrentBlock(nn.Module):
                 return False
         if self.linear_x.weight.dtype != x.dtype or self.linear_y.weight.dtype != x.dtype:
             return False
-        probe = x.new_empty(x.size(0), 1, self.rnn_width)
-        return self._hip_block_ops_covers(probe)
+        mode = self.rg_lru.scan_mode
+        if mode == "auto":
+            probe = x.new_empty(x.size(0), 1, self.rnn_width)
+            return self._hip_block_ops_covers(probe)
+        return mode in ("hip", "fused") and self.conv_kernel_size <= hip_block_ops.max_kernel_size()
 
     def _hip_decode(self, x: Tensor, cache: RecurrentBlockCache | None, segment_pos: Tensor | None,
                     active_mask: Tensor | None, return_cache: bool):
@@ -389,15 +392,15 @@ class RecurrentBlock(nn.Module):
             raise ValueError(f"RecurrentBlock expects [batch, sequence, width], got {tuple(x.shape)}")
         batch, steps = x.shape[:2]
         everything_active = active_mask is None
-        if active_mask is None:
-            active_mask = torch.ones(batch, steps, device=x.device, dtype=torch.bool)
-        elif active_mask.shape != (batch, steps):
-            raise ValueError("active_mask must match the input [batch, sequence] dimensions")
-        else:
+        if not everything_active:
+            if active_mask.shape != (batch, steps):
+                raise ValueError("active_mask must match the input [batch, sequence] dimensions")
             active_mask = active_mask.to(device=x.device, dtype=torch.bool)
         previous_position = None if cache is None else cache.segment_position
         if steps == 1 and self._hip_decode_covers(x, cache):
-            return self._hip_decode(x, cache, segment_pos, None if everything_active else active_mask, return_cache)
+            return self._hip_decode(x, cache, segment_pos, active_mask, return_cache)
+        if everything_active:
+            active_mask = torch.ones(batch, steps, device=x.device, dtype=torch.bool)
         segment_pos = _resolve_segment_positions(
             x, segment_pos, previous_position, None if everything_active else active_mask)
 
