@@ -14,7 +14,7 @@ RGLRU_BF16 = 1
 FLAG_RESET = 1
 FLAG_INACTIVE = 2
 CHUNK = 32
-ABI_VERSION = 12
+ABI_VERSION = 13
 
 _lock = threading.Lock()
 _lib = None
@@ -39,7 +39,9 @@ _SIGNATURES = {
     "rglru_hip_prepare_fwd": (ctypes.c_int, [_P, _P, _P, _P, _P, ctypes.c_float, ctypes.c_int, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, ctypes.c_int, _P]),
     "rglru_hip_bwd": (ctypes.c_int, [_P] * 15 + [_I, _I, _I, _I, ctypes.c_int, ctypes.c_int, _P]),
     "rglru_hip_fast_path": (ctypes.c_int, [_I, _I, ctypes.c_int]),
+    "rglru_hip_wide_path": (ctypes.c_int, [_I, _I, ctypes.c_int]),
     "rglru_hip_bwd_full": (ctypes.c_int, [_P] * 16 + [_I, _I, _I, _I, ctypes.c_int, ctypes.c_int, _P]),
+    "rglru_hip_bwd_wide": (ctypes.c_int, [_P] * 15 + [_I, _I, _I, _I, ctypes.c_int, ctypes.c_int, _P]),
     "rglru_hip_pre_path": (ctypes.c_int, [_I, _I, ctypes.c_int]),
     "rglru_hip_fwd_pre": (ctypes.c_int, [_P] * 8 + [_I, _I, _I, _I, ctypes.c_int, _P]),
     "rglru_hip_bwd_pre": (ctypes.c_int, [_P] * 15 + [_I, _I, _I, _I, ctypes.c_int, ctypes.c_int, _P]),

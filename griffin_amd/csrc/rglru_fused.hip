@@ -480,15 +480,18 @@ constexpr int kFwdMT = 2;
 #define RGLRU_NARROW_OCC 3
 #endif
 template <typename IO, int NKG, bool MASKED>
-__global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : (NKG == 4 || NKG == 2) ? RGLRU_NARROW_OCC : 2)) void fwd_kernel(FusedArgs p) {
+__global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : (NKG == 4 || NKG == 2) ? RGLRU_NARROW_OCC : NKG > 8 ? 1 : 2)) void fwd_kernel(FusedArgs p) {
   constexpr int MT = kFwdMT, TR = 32 * MT, EL = 16 * MT;
   typedef Io<IO> Tr;
   typedef typename Tr::Frag Frag;
-  // NKG > 0: gate weights held in registers, pre-activations on MFMA.  NKG < 0: the caller supplies the
-  // pre-activations (blocks too wide to hold their weights: a library GEMM computes W x first).
-  // NKG == 0: the portable path (any width, alignment and storage type), weights streamed.
+  // NKG > 0: gate weights held in registers, pre-activations on MFMA.  Up to NKG = 8 (128 channels) a
+  // workgroup covers a whole block (or several narrow ones); a wider block (NKG = bw / 16 > 8) is
+  // shared by `groups` workgroups of four 32-channel slabs each, every one of which stages the block's
+  // whole x tile and holds its slabs' rows of both matrices (8 NKG registers a lane, one wave a SIMD).
+  // NKG < 0: the caller supplies the pre-activations.  NKG == 0: the portable path (any width,
+  // alignment and storage type), weights streamed.
   constexpr bool GIVEN = NKG < 0;
-  constexpr int KC = NKG != 0 ? kPackedWidth : Tr::KCMAX;          // LDS tile width in elements
+  constexpr int KC = NKG > 8 ? NKG * Tr::KG : NKG != 0 ? kPackedWidth : Tr::KCMAX;   // LDS tile width in elements
   constexpr int LDSROW = KC + Tr::HW;
   __shared__ __attribute__((aligned(16))) IO lds[TR * LDSROW];
   __shared__ __attribute__((aligned(16))) IO lds_pre[GIVEN ? 2 * TR * LDSROW : Tr::HW];   // W_a x | W_x x tiles
@@ -614,7 +617,7 @@ __global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : (NKG == 4 ||
               ux[e] = (float)lds_pre[TR * LDSROW + at];
             }
           } else
-          gate_mfma_held<IO, MT, NKG, KC>(lds, hw, mt, w.slab, w.r, hf, 0.0f, 0.0f, ua, ux, xv, NKG == 8 ? 0 : w.kb);
+          gate_mfma_held<IO, MT, NKG, KC>(lds, hw, mt, w.slab, w.r, hf, 0.0f, 0.0f, ua, ux, xv, NKG >= 8 ? 0 : w.kb);
           fwd_gates<IO, MASKED>(flbits[mt], ua, ux, xv, sp, cur.a + 16 * mt, cur.z + 16 * mt, nba, nbx);
         }
       }
@@ -824,20 +827,24 @@ template <int ROWS> struct PairStage {                  // ROWS x 32 channels x 
 };
 
 template <typename IO, int NKG, bool MASKED>
-__global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
+__global__ __launch_bounds__(kThreads, (NKG > 8 ? 1 : 2)) void bwd_scan_kernel(FusedArgs p) {
   constexpr int MT = 1, TR = 32, EL = 16;
   typedef Io<IO> Tr;
   typedef typename Tr::Frag Frag;
   // NKG < 0: the caller supplies the gate pre-activations (see fwd_kernel) and gets the gradients at
   // them back as two halves per block, [nb][B*T][du_a (bw) | du_x (bw)], the operand layout of the
   // two GEMMs it runs afterwards; no weights are read here.
+  // NKG > 8: a block wider than four slabs, shared by `groups` workgroups as in fwd_kernel: the x
+  // tile spans the block, the dy tile only the workgroup's own 128 channels.
   constexpr bool GIVEN = NKG < 0;
+  constexpr bool WIDE = NKG > 8;
   constexpr int KC = (GIVEN ? 8 : NKG) * Tr::KG;         // block width (held weights)
-  constexpr int TW = kPackedWidth;                       // tile width (narrow blocks are packed)
+  constexpr int TW = WIDE ? KC : kPackedWidth;           // tile width (narrow blocks are packed)
   constexpr int LDSROW = TW + Tr::HW;
+  constexpr int DYROW = kPackedWidth + Tr::HW;
   static_assert(sizeof(IO) == 2 && NKG != 0, "fast backward is for 16-bit storage");
   __shared__ __attribute__((aligned(16))) IO lds_x[TR * LDSROW];
-  __shared__ __attribute__((aligned(16))) IO lds_dy[TR * LDSROW];
+  __shared__ __attribute__((aligned(16))) IO lds_dy[TR * DYROW];
   __shared__ __attribute__((aligned(16))) IO lds_pre[GIVEN ? 2 * TR * LDSROW : Tr::HW];
   __shared__ __attribute__((aligned(16))) unsigned char stage_dx_all[kWaves * WaveStage<TR>::kBytes];
   __shared__ __attribute__((aligned(16))) unsigned char stage_du_all[kWaves * (GIVEN ? 2 * WaveStage<TR>::kBytes : PairStage<TR>::kBytes)];
@@ -881,11 +888,15 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
 
   constexpr int VPR = TW / Tr::HW;
   constexpr int NV = (TR * VPR + kThreads - 1) / kThreads;
-  Frag pre_x[NV], pre_dy[NV], pre_ua[GIVEN ? NV : 1], pre_ux[GIVEN ? NV : 1];
-  unsigned pre_off[NV], u_off[GIVEN ? NV : 1];
+  constexpr int VPR_DY = kPackedWidth / Tr::HW;
+  constexpr int NV_DY = (TR * VPR_DY + kThreads - 1) / kThreads;
+  Frag pre_x[NV], pre_dy[NV_DY], pre_ua[GIVEN ? NV : 1], pre_ux[GIVEN ? NV : 1];
+  unsigned pre_off[NV], dy_off[NV_DY], u_off[GIVEN ? NV : 1];
   // GIVEN: the tiles hold the 128 channels of this workgroup's four slabs
-  const int group_col = GIVEN ? (w.unit % p.groups) * TW : 0;
+  const int group_col = (GIVEN || WIDE) ? (w.unit % p.groups) * kPackedWidth : 0;
   const int x_col = GIVEN ? w.k * p.bw + group_col : w.tile_col;
+  const int dy_col = WIDE ? w.k * p.bw + group_col : x_col;
+  const int own_col = WIDE ? group_col : 0;              // the dy tile's first column inside the x tile
   const unsigned u_row_bytes = 4u * (unsigned)p.bw;      // a row of `pre` and of du: two halves of bw 16-bit values
 #pragma unroll
   for (int i = 0; i < NV; ++i) {
@@ -894,6 +905,14 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
     pre_off[i] = (idx < TR * VPR) ? (unsigned)row * row_bytes + (unsigned)(x_col + cv * Tr::HW) * 2u : kOutOfRange;
     if constexpr (GIVEN)
       u_off[i] = (idx < TR * VPR) ? (unsigned)row * u_row_bytes + (unsigned)(group_col + cv * Tr::HW) * 2u : kOutOfRange;
+  }
+#pragma unroll
+  for (int i = 0; i < NV_DY; ++i) {
+    const int idx = tid + i * kThreads;
+    const int row = idx / VPR_DY, cv = idx - row * VPR_DY;
+    // a wide block's last group may reach past the block: those columns belong to a wave without a slab
+    const bool in = idx < TR * VPR_DY && (!WIDE || own_col + cv * Tr::HW < p.bw);
+    dy_off[i] = in ? (unsigned)row * row_bytes + (unsigned)(dy_col + cv * Tr::HW) * 2u : kOutOfRange;
   }
   auto decode = [&](unsigned tk, int& c, int& b) {
     const unsigned cr = tk / (unsigned)q.n_b;
@@ -910,7 +929,9 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
     const rsrc_t rx = make_rsrc(x + first, (unsigned)rows * row_bytes);
     const rsrc_t rdy = make_rsrc(dy + first, (unsigned)rows * row_bytes);
 #pragma unroll
-    for (int i = 0; i < NV; ++i) { pre_x[i] = buf_load_frag<Frag>(rx, pre_off[i]); pre_dy[i] = buf_load_frag<Frag>(rdy, pre_off[i]); }
+    for (int i = 0; i < NV; ++i) pre_x[i] = buf_load_frag<Frag>(rx, pre_off[i]);
+#pragma unroll
+    for (int i = 0; i < NV_DY; ++i) pre_dy[i] = buf_load_frag<Frag>(rdy, dy_off[i]);
     if constexpr (GIVEN) {
       const IO* ubase = (const IO*)p.pre + ((long long)w.k * p.rows_total + (long long)b * p.T + (long long)c * TR) * (2 * p.bw);
       const rsrc_t ru = make_rsrc(ubase, (unsigned)rows * u_row_bytes);
@@ -947,12 +968,17 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
       const int row = idx / VPR, cv = idx - row * VPR;
       if (idx < TR * VPR) {
         *reinterpret_cast<Frag*>(lds_x + row * LDSROW + cv * Tr::HW) = pre_x[i];
-        *reinterpret_cast<Frag*>(lds_dy + row * LDSROW + cv * Tr::HW) = pre_dy[i];
         if constexpr (GIVEN) {
           *reinterpret_cast<Frag*>(lds_pre + row * LDSROW + cv * Tr::HW) = pre_ua[i];
           *reinterpret_cast<Frag*>(lds_pre + (TR + row) * LDSROW + cv * Tr::HW) = pre_ux[i];
         }
       }
+    }
+#pragma unroll
+    for (int i = 0; i < NV_DY; ++i) {
+      const int idx = tid + i * kThreads;
+      const int row = idx / VPR_DY, cv = idx - row * VPR_DY;
+      if (idx < TR * VPR_DY) *reinterpret_cast<Frag*>(lds_dy + row * DYROW + cv * Tr::HW) = pre_dy[i];
     }
     __syncthreads();
     f32x16 ua, ux;
@@ -964,14 +990,14 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
         for (int e = 0; e < EL; ++e) {
           const int at = (hf * EL + e) * LDSROW + col;
           xv[e] = (float)lds_x[at];
-          gy[e] = (float)lds_dy[at];
+          gy[e] = (float)lds_dy[(hf * EL + e) * DYROW + col];
           ua[e] = (float)lds_pre[at];
           ux[e] = (float)lds_pre[TR * LDSROW + at];
         }
       } else if constexpr (XLDS) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) { ua[v] = 0.0f; ux[v] = 0.0f; }     // the biases enter inside the sigmoids
-        const int kb = NKG == 8 ? 0 : w.kb;
+        const int kb = NKG >= 8 ? 0 : w.kb;
         const IO* xrow = lds_x + tile_row<MT>(0, w.r) * LDSROW + kb + hf * Tr::HW;
         const IO* brow = lds_wx + (w.wave * 32 + w.r) * WROW + hf * Tr::HW;
 #pragma unroll
@@ -987,7 +1013,7 @@ __global__ __launch_bounds__(kThreads, 2) void bwd_scan_kernel(FusedArgs p) {
       }
       if constexpr (!GIVEN) {
 #pragma unroll
-        for (int e = 0; e < EL; ++e) gy[e] = (float)lds_dy[(hf * EL + e) * LDSROW + (NKG == 8 ? 0 : w.kb) + w.slab * 32 + w.r];
+        for (int e = 0; e < EL; ++e) gy[e] = (float)lds_dy[(hf * EL + e) * DYROW + (NKG >= 8 ? 0 : w.kb) + w.slab * 32 - own_col + w.r];
       }
     }
     if (tid == 0) s_ticket[par ^ 1] = next_raw;
@@ -1633,6 +1659,222 @@ __global__ __launch_bounds__(kGradThreads, 1) void bwd_grad_kernel(FusedArgs p) 
   }
 }
 
+// ------------------------------------------------------------------------------------------
+// Backward of blocks wider than 128 channels, second part: the two block-diagonal GEMMs of the gate
+// gradients on the pairs du2[n][k][2 o + gate] that bwd_scan_kernel left in memory,
+//     dx[n, j]   += sum_kappa du2[n, kappa] * w2t[j, kappa]          (kappa = 2 * o + gate)
+//     dW[gate][j][o] = sum_n x[n, j] * du2[n, 2 o + gate]
+// over the flattened token axis n = b * T + t, 32 tokens per tile.  A unit is a group of two
+// 32-column slabs j of one gate block; its eight waves are (slab, quarter): a wave owns every fourth
+// 32-wide kappa tile, and for those it keeps its slab's w2t fragments (B operand of the first GEMM,
+// which it contracts over its own kappa only: the four quarters' partial tiles are added through LDS)
+// and its slab's 32 x 32 accumulators of the second GEMM in registers for the whole launch.  The
+// second GEMM contracts over tokens; both operands reach the layout it needs through the matrix
+// unit (a tile times the identity comes back in accumulator layout, where a lane holds 16 consecutive
+// tokens of one column), du2 once per tile for all waves (lds_dut).
+// ------------------------------------------------------------------------------------------
+template <typename IO, int NKG>
+__global__ __launch_bounds__(kGradThreads, 1) void gate_grad_wide_kernel(FusedArgs p) {
+  typedef Io<IO> Tr;
+  typedef typename Tr::Frag Frag;
+  static_assert(sizeof(IO) == 2 && NKG > 8, "16-bit storage, blocks wider than 128 channels");
+  constexpr int TR = 32;
+  constexpr int KC = NKG * Tr::KG;                       // block width
+  constexpr int K2 = 2 * KC;                             // kappa per block
+  constexpr int S = KC / 32;                             // slabs in the block
+  constexpr int JG = (S + 1) / 2;                        // units per block (two slabs each)
+  constexpr int NKT = K2 / 32;                           // kappa tiles
+  constexpr int NI = (NKT + 3) / 4;                      // ... per wave
+  constexpr int JW = 64;                                 // columns of the unit's x / dx tiles
+  constexpr int ROW_DU = K2 + Tr::HW, ROW_X = JW + Tr::HW, ROW_T = TR + Tr::HW;
+  __shared__ __attribute__((aligned(16))) IO lds_du[TR * ROW_DU];
+  __shared__ __attribute__((aligned(16))) IO lds_dut[K2 * ROW_T];          // du2 transposed: [kappa][token]
+  __shared__ __attribute__((aligned(16))) IO lds_x[TR * ROW_X];
+  __shared__ __attribute__((aligned(16))) IO lds_dx[TR * ROW_X];
+  __shared__ __attribute__((aligned(16))) float lds_red[2][3][16][64];     // partial dx tiles of quarters 1..3
+  __shared__ __attribute__((aligned(16))) unsigned char stage_all[2 * WaveStage<TR>::kBytes];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, hf = lane >> 5;
+  const int sl = wave & 1, q = wave >> 1;
+  const int units = p.nb * JG;
+  const int unit = blockIdx.x % units, wg_in_unit = blockIdx.x / units, n_wg = gridDim.x / units;
+  const int k = unit / JG, jg = unit - k * JG;
+  const int slab = jg * 2 + sl;
+  const bool slab_ok = slab < S;
+  const int j0 = (slab_ok ? slab : 0) * 32;                // the wave's first column inside the block
+  unsigned char* stage = stage_all + sl * WaveStage<TR>::kBytes;
+  const long long rows_total = (long long)p.B * p.T;
+  const long long n_tiles = (rows_total + TR - 1) / TR;
+  const unsigned row_bytes = (unsigned)p.W * 2u;
+
+  // this wave's w2t fragments: row j0 + r, kappa tiles q, q + 4, ...; lane (j, hf) holds kappa = 32 kt + 16 g + 8 hf + i
+  Frag w2[NI][2];
+  {
+    const IO* row = (const IO*)p.w2t + ((long long)k * p.bwp + j0 + r) * (2 * p.bwp) + hf * Tr::HW;
+#pragma unroll
+    for (int i = 0; i < NI; ++i)
+#pragma unroll
+      for (int g = 0; g < 2; ++g) {
+        const int kt = q + 4 * i;
+        w2[i][g] = (slab_ok && kt < NKT) ? *reinterpret_cast<const Frag*>(row + kt * 32 + g * Tr::KG) : Tr::zero();
+      }
+  }
+  // identity fragments: element i of ident[g] is 1 where 16 g + 8 hf + i == r
+  Frag ident[2];
+#pragma unroll
+  for (int g = 0; g < 2; ++g)
+#pragma unroll
+    for (int i = 0; i < Tr::HW; ++i) ident[g][i] = (IO)((16 * g + 8 * hf + i == r) ? 1.0f : 0.0f);
+
+  f32x16 dw[NI];
+#pragma unroll
+  for (int i = 0; i < NI; ++i)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) dw[i][v] = 0.f;
+
+  // cooperative tile loads: du2 (TR x K2 of block k), x and the direct part of dx (TR x 64 of the unit)
+  constexpr int VPR_DU = K2 / Tr::HW, VPR_X = JW / Tr::HW;
+  constexpr int NV_DU = (TR * VPR_DU + kGradThreads - 1) / kGradThreads;
+  static_assert(TR * VPR_X <= kGradThreads, "one x vector per thread");
+  const int unit_col = k * p.bw + jg * JW;                 // first channel of the unit
+  Frag pre_du[NV_DU], pre_x, pre_dx;
+  unsigned du_off[NV_DU], x_off;
+#pragma unroll
+  for (int i = 0; i < NV_DU; ++i) {
+    const int idx = tid + i * kGradThreads;
+    const int row = idx / VPR_DU, cv = idx - row * VPR_DU;
+    du_off[i] = idx < TR * VPR_DU ? (unsigned)row * 2u * row_bytes + (unsigned)(2 * k * p.bw + cv * Tr::HW) * 2u : kOutOfRange;
+  }
+  {
+    const int row = tid / VPR_X, cv = tid - row * VPR_X;
+    x_off = (tid < TR * VPR_X && jg * JW + cv * Tr::HW < KC) ? (unsigned)row * row_bytes + (unsigned)(unit_col + cv * Tr::HW) * 2u : kOutOfRange;
+  }
+  auto issue = [&](long long tile) {
+    // a tile past the end keeps valid addresses but an empty extent: nothing is fetched
+    const bool live = tile < n_tiles;
+    const long long row0 = live ? tile * TR : 0;
+    const int rows = !live ? 0 : (int)((rows_total - row0) < TR ? (rows_total - row0) : TR);
+    const rsrc_t rdu = make_rsrc((const IO*)p.du_a + row0 * 2 * p.W, (unsigned)rows * 2u * row_bytes);
+    const rsrc_t rx = make_rsrc((const IO*)p.x + row0 * p.W, (unsigned)rows * row_bytes);
+    const rsrc_t rdx = make_rsrc((const IO*)p.dx + row0 * p.W, (unsigned)rows * row_bytes);
+#pragma unroll
+    for (int i = 0; i < NV_DU; ++i) pre_du[i] = buf_load_frag<Frag>(rdu, du_off[i]);
+    pre_x = buf_load_frag<Frag>(rx, x_off);
+    pre_dx = buf_load_frag<Frag>(rdx, x_off);
+  };
+
+  long long tile = wg_in_unit;
+  issue(tile);
+  for (; tile < n_tiles; tile += n_wg) {
+#pragma unroll
+    for (int i = 0; i < NV_DU; ++i) {
+      const int idx = tid + i * kGradThreads;
+      const int row = idx / VPR_DU, cv = idx - row * VPR_DU;
+      if (idx < TR * VPR_DU) *reinterpret_cast<Frag*>(lds_du + row * ROW_DU + cv * Tr::HW) = pre_du[i];
+    }
+    if (tid < TR * VPR_X) {
+      const int row = tid / VPR_X, cv = tid - row * VPR_X;
+      *reinterpret_cast<Frag*>(lds_x + row * ROW_X + cv * Tr::HW) = pre_x;
+      *reinterpret_cast<Frag*>(lds_dx + row * ROW_X + cv * Tr::HW) = pre_dx;
+    }
+    __syncthreads();
+    issue(tile + n_wg);
+
+    const long long row0 = tile * TR;
+    const IO* a_row_du = lds_du + tile_row<1>(0, r) * ROW_DU + hf * Tr::HW;
+    const IO* a_row_x = lds_x + tile_row<1>(0, r) * ROW_X + hf * Tr::HW;
+    // x of this wave's slab with tokens along the lane vector (A operand of the second GEMM)
+    Frag xt_lo = Tr::zero(), xt_hi = Tr::zero();
+    if (slab_ok) {
+      f32x16 xc;
+#pragma unroll
+      for (int v = 0; v < 16; ++v) xc[v] = 0.f;
+      Tr::mma(xc, *reinterpret_cast<const Frag*>(a_row_x + (2 * sl) * Tr::KG), ident[0]);
+      Tr::mma(xc, *reinterpret_cast<const Frag*>(a_row_x + (2 * sl + 1) * Tr::KG), ident[1]);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) { xt_lo[i] = (IO)xc[i]; xt_hi[i] = (IO)xc[8 + i]; }
+    }
+    // transposes of du2: the eight waves share the kappa tiles
+#pragma unroll
+    for (int h = 0; h < (NKT + kGradWaves - 1) / kGradWaves; ++h) {
+      const int kt = kGradWaves * h + wave;
+      if (kt < NKT) {
+        f32x16 dc;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) dc[v] = 0.f;
+        Tr::mma(dc, *reinterpret_cast<const Frag*>(a_row_du + (2 * kt) * Tr::KG), ident[0]);
+        Tr::mma(dc, *reinterpret_cast<const Frag*>(a_row_du + (2 * kt + 1) * Tr::KG), ident[1]);
+        Frag lo, hi;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { lo[i] = (IO)dc[i]; hi[i] = (IO)dc[8 + i]; }
+        IO* dst = lds_dut + (kt * 32 + r) * ROW_T + hf * 16;
+        *reinterpret_cast<Frag*>(dst) = lo;
+        *reinterpret_cast<Frag*>(dst + 8) = hi;
+      }
+    }
+    // first GEMM, this wave's share of kappa; quarter 0 starts from the direct part and adds the others' tiles
+    f32x16 acc;
+    if (slab_ok) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[v] = (q == 0) ? (float)lds_dx[(hf * 16 + v) * ROW_X + sl * 32 + r] : 0.f;
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        const int kt = q + 4 * i;
+        if (kt < NKT) {
+          Tr::mma(acc, *reinterpret_cast<const Frag*>(a_row_du + (2 * kt) * Tr::KG), w2[i][0]);
+          Tr::mma(acc, *reinterpret_cast<const Frag*>(a_row_du + (2 * kt + 1) * Tr::KG), w2[i][1]);
+        }
+      }
+      if (q != 0) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) lds_red[sl][q - 1][v][lane] = acc[v];
+      }
+    }
+    __syncthreads();
+    if (slab_ok) {
+      // second GEMM: dW2T[j, kappa] += sum over the tile's tokens, this wave's kappa tiles
+#pragma unroll
+      for (int i = 0; i < NI; ++i) {
+        const int kt = q + 4 * i;
+        if (kt < NKT) {
+          const IO* b_row = lds_dut + (kt * 32 + r) * ROW_T + hf * 16;
+          Tr::mma(dw[i], xt_lo, *reinterpret_cast<const Frag*>(b_row));
+          Tr::mma(dw[i], xt_hi, *reinterpret_cast<const Frag*>(b_row + 8));
+        }
+      }
+      if (q == 0) {
+        unsigned char* my = stage + WaveStage<TR>::row_offset(hf * 16) + r * 2;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const float sum = acc[v] + (lds_red[sl][0][v][lane] + (lds_red[sl][1][v][lane] + lds_red[sl][2][v][lane]));
+          *reinterpret_cast<IO*>(my + v * WaveStage<TR>::kRowBytes) = (IO)sum;
+        }
+        wave_lds_fence();
+        const int rows = (int)((rows_total - row0) < TR ? (rows_total - row0) : TR);
+        const rsrc_t rdx = make_rsrc((const IO*)p.dx + row0 * p.W, (unsigned)rows * row_bytes);
+        stage_flush<TR>(stage, rdx, row_bytes, (unsigned)(k * p.bw + j0) * 2u, lane);
+        wave_lds_fence();
+      }
+    }
+  }
+  // per-workgroup partial of the weight gradients: [wg][k][gate][j][o]
+  if (slab_ok) {
+    float* part = p.dw_partial + ((long long)wg_in_unit * p.nb + k) * 2 * p.bwp * p.bwp;
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int kt = q + 4 * i;
+      if (kt < NKT) {
+        const int kappa = kt * 32 + r, o = kappa >> 1, gate = kappa & 1;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int j = j0 + 8 * (v >> 2) + 4 * hf + (v & 3);
+          part[((long long)gate * p.bwp + j) * p.bwp + o] = dw[i][v];
+        }
+      }
+    }
+  }
+}
+
 // Last launch of a backward pass: sums the per-workgroup partial results and writes the parameter
 // gradients in the caller's type.  Workgroups [0, vec_blocks) own 16 channels each of db_a, db_x and
 // dLambda; the rest (fast backward only) own 1024 elements each of the two weight gradients,
@@ -1930,6 +2172,19 @@ static int held_groups(const Geometry& g, int dtype, int aligned) {
   return 0;
 }
 
+// ... and for the blocks wider than a workgroup's four slabs whose weights the forward and the
+// gate-gradient kernels hold in registers: K groups (bw / 16), or 0
+static int wide_groups(const Geometry& g, int dtype, int aligned) {
+  if (dtype != RGLRU_BF16 || !aligned) return 0;
+  switch (g.bw) {
+    case 160: case 192: case 256: case 320: case 384: return (int)(g.bw / 16);
+    default: return 0;
+  }
+}
+
+#define RGLRU_FWD_WIDE_CASE(N, grid, stream, args, dtype, nkg, masked)                                              \
+    else if ((dtype) == RGLRU_BF16 && (nkg) == N && !(masked)) hipLaunchKernelGGL((fwd_kernel<__bf16, N, false>), grid, dim3(kThreads), 0, stream, args); \
+    else if ((dtype) == RGLRU_BF16 && (nkg) == N) hipLaunchKernelGGL((fwd_kernel<__bf16, N, true>), grid, dim3(kThreads), 0, stream, args);
 #define RGLRU_DISPATCH_FWD(grid, stream, args, dtype, nkg, masked)                                      \
   do {                                                                                                 \
     if ((dtype) == RGLRU_BF16 && (nkg) == 8 && !(masked)) hipLaunchKernelGGL((fwd_kernel<__bf16, 8, false>), grid, dim3(kThreads), 0, stream, args); \
@@ -1938,6 +2193,9 @@ static int held_groups(const Geometry& g, int dtype, int aligned) {
     else if ((dtype) == RGLRU_BF16 && (nkg) == 4) hipLaunchKernelGGL((fwd_kernel<__bf16, 4, true>), grid, dim3(kThreads), 0, stream, args); \
     else if ((dtype) == RGLRU_BF16 && (nkg) == 2 && !(masked)) hipLaunchKernelGGL((fwd_kernel<__bf16, 2, false>), grid, dim3(kThreads), 0, stream, args); \
     else if ((dtype) == RGLRU_BF16 && (nkg) == 2) hipLaunchKernelGGL((fwd_kernel<__bf16, 2, true>), grid, dim3(kThreads), 0, stream, args); \
+    RGLRU_FWD_WIDE_CASE(10, grid, stream, args, dtype, nkg, masked) RGLRU_FWD_WIDE_CASE(12, grid, stream, args, dtype, nkg, masked) \
+    RGLRU_FWD_WIDE_CASE(16, grid, stream, args, dtype, nkg, masked) RGLRU_FWD_WIDE_CASE(20, grid, stream, args, dtype, nkg, masked) \
+    RGLRU_FWD_WIDE_CASE(24, grid, stream, args, dtype, nkg, masked)                                                                  \
     else if ((dtype) == RGLRU_BF16 && (nkg) < 0 && !(masked)) hipLaunchKernelGGL((fwd_kernel<__bf16, -1, false>), grid, dim3(kThreads), 0, stream, args); \
     else if ((dtype) == RGLRU_BF16 && (nkg) < 0) hipLaunchKernelGGL((fwd_kernel<__bf16, -1, true>), grid, dim3(kThreads), 0, stream, args); \
     else if ((dtype) == RGLRU_BF16) hipLaunchKernelGGL((fwd_kernel<__bf16, 0, true>), grid, dim3(kThreads), 0, stream, args); \
@@ -2051,9 +2309,12 @@ size_t rglru_hip_workspace_bytes(int64_t B, int64_t T, int64_t W, int64_t nb) {
   return make_work_layout(B, T, make_geometry(W, nb)).total;
 }
 
+int rglru_hip_wide_path(int64_t W, int64_t nb, int dtype);
+
 size_t rglru_hip_bwd_scratch_bytes(int64_t B, int64_t T, int64_t W, int64_t nb, int dtype) {
   if (B <= 0 || T <= 0 || W <= 0 || nb <= 0 || W % nb) return 0;
-  return make_scratch_layout(B, T, make_geometry(W, nb), rglru_hip_fast_path(W, nb, dtype) != 0).total;
+  const int kind = rglru_hip_fast_path(W, nb, dtype) ? kScratchFast : rglru_hip_wide_path(W, nb, dtype) ? kScratchWide : kScratchPlain;
+  return make_scratch_layout(B, T, make_geometry(W, nb), kind).total;
 }
 
 static int fwd_impl(const void* x, const void* prep, const float* h0, const uint8_t* flags,
@@ -2085,6 +2346,7 @@ static int fwd_impl(const void* x, const void* prep, const float* h0, const uint
   a.nCf = (int)((T + 32 * kFwdMT - 1) / (32 * kFwdMT));
   a.aligned = is_aligned(x, W, g.bw, elem_size(dtype)) && ((uintptr_t)y % 16 == 0);
   int nkg = held_groups(g, dtype, a.aligned);
+  if (!nkg && !pre) nkg = wide_groups(g, dtype, a.aligned);
   if (pre) {
     if (!rglru_hip_pre_path(W, nb, dtype)) return fail(RGLRU_E_UNSUPPORTED, "fwd_pre: needs bf16 storage and gate blocks of a multiple of 32 channels");
     if (!a.aligned || (uintptr_t)pre % 16) return fail(RGLRU_E_UNSUPPORTED, "fwd_pre: x, pre and y must be 16-byte aligned");
@@ -2093,7 +2355,7 @@ static int fwd_impl(const void* x, const void* prep, const float* h0, const uint
   }
   pack_units(a, g, nkg);
   // without weights in registers three workgroups fit a compute unit
-  a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nCf, nkg < 0 ? RGLRU_GIVEN_OCC : ((nkg == 4 || nkg == 2) ? RGLRU_NARROW_OCC : 2), 1 << 20);
+  a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nCf, nkg < 0 ? RGLRU_GIVEN_OCC : ((nkg == 4 || nkg == 2) ? RGLRU_NARROW_OCC : nkg > 8 ? 1 : 2), 1 << 20);
   a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
   dim3 grid((unsigned)(a.wg_per_unit * a.units));
   {
@@ -2188,7 +2450,7 @@ int rglru_hip_bwd_pre(const void* x, const void* pre, const void* prep, const fl
   a.dx = dx; a.du_a = du; a.dh0 = dh0;
   a.ckpt = (float*)(wb + L.ckpt); a.rec_a = (rec_t*)(wb + L.b_rec_a);
   a.ticket = (unsigned*)(wb + L.b_ticket); a.fail = (unsigned*)(wb + L.fail);
-  a.partial = (float*)((char*)scratch + make_scratch_layout(B, T, g, false).partial);
+  a.partial = (float*)((char*)scratch + make_scratch_layout(B, T, g, kScratchPlain).partial);
   a.B = (int)B; a.T = (int)T; a.nC = (int)((T + kChunk - 1) / kChunk); a.ckpt_nC = 2 * (int)L.nC;
   a.aligned = 1;
   a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nC, 2, L.max_wg);
@@ -2259,7 +2521,7 @@ int rglru_hip_bwd(const void* x, const void* prep, const float* h0,
   a.dx = dx; a.du_a = du_a; a.du_x = du_x; a.dh0 = dh0;
   a.ckpt = (float*)(wb + L.ckpt); a.rec_a = (rec_t*)(wb + L.b_rec_a);
   a.ticket = (unsigned*)(wb + L.b_ticket); a.fail = (unsigned*)(wb + L.fail);
-  a.partial = (float*)((char*)scratch + make_scratch_layout(B, T, g, false).partial);
+  a.partial = (float*)((char*)scratch + make_scratch_layout(B, T, g, kScratchPlain).partial);
   a.B = (int)B; a.T = (int)T; a.nC = (int)((T + kChunk - 1) / kChunk); a.ckpt_nC = 2 * (int)L.nC; a.nCf = (int)L.nCf;
   a.aligned = is_aligned(x, W, g.bw, elem_size(dtype));
   a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nC, 2, L.max_wg);
@@ -2320,7 +2582,7 @@ int rglru_hip_bwd_full(const void* x, const void* y, const void* prep, const flo
   fill_common(a, g, prep, dtype);
   a.x = x; a.y = const_cast<void*>(y); a.h0 = h0; a.flags = flags; a.dy = dy; a.dh_last = dh_last;
   a.flags_vec = (T % 16 == 0) && ((uintptr_t)flags % 16 == 0);
-  const ScratchLayout SL = make_scratch_layout(B, T, g, true);
+  const ScratchLayout SL = make_scratch_layout(B, T, g, kScratchFast);
   char* sb = (char*)scratch;
   a.dx = dx; a.du_a = sb + SL.delta; a.dh0 = dh0;
   a.ckpt = (float*)(wb + L.ckpt); a.rec_a = (rec_t*)(wb + L.b_rec_a);
@@ -2372,6 +2634,98 @@ int rglru_hip_bwd_full(const void* x, const void* y, const void* prep, const flo
   const long long total = nb * g.bw * 2 * g.bw;
   hipLaunchKernelGGL(finish_kernel, dim3((unsigned)(r.vec_blocks + (total / 4 + 255) / 256)), dim3(256), 0, s, r);
   return check_launch("bwd_full finish");
+}
+
+int rglru_hip_wide_path(int64_t W, int64_t nb, int dtype) {
+  if (W <= 0 || nb <= 0 || W % nb) return 0;
+  return wide_groups(make_geometry(W, nb), dtype, 1) != 0 ? 1 : 0;
+}
+
+int rglru_hip_bwd_wide(const void* x, const void* prep, const float* h0,
+                       const uint8_t* flags, const void* dy, const float* dh_last, void* ws, void* scratch,
+                       void* dx, void* dw_a, void* dw_x, void* db_a, void* db_x, void* dlambda,
+                       float* dh0, int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, int grad_dtype,
+                       void* stream) {
+  int rc = check_geometry("bwd_wide", W, nb, dtype);
+  if (rc) return rc;
+  rc = check_grad_dtype("bwd_wide", grad_dtype);
+  if (rc) return rc;
+  if (!rglru_hip_wide_path(W, nb, dtype))
+    return fail(RGLRU_E_UNSUPPORTED, "bwd_wide: needs 16-bit storage and gate blocks of 160, 192, 256, 320 or 384 channels");
+  if (B <= 0 || T <= 0) return fail(RGLRU_E_ARG, "bwd_wide: B and T must be positive (got %lld, %lld)", (long long)B, (long long)T);
+  if (!x || !prep || !dy || !ws || !scratch || !dx || !dw_a || !dw_x || !db_a || !db_x || !dlambda)
+    return fail(RGLRU_E_ARG, "bwd_wide: null pointer");
+  rc = check_extents("bwd_wide", B, T, W);
+  if (rc) return rc;
+  Geometry g = make_geometry(W, nb);
+  if (!is_aligned(x, W, g.bw, 2) || !is_aligned(dy, W, g.bw, 2) || !is_aligned(dx, W, g.bw, 2))
+    return fail(RGLRU_E_UNSUPPORTED, "bwd_wide: x, dy and dx must be 16-byte aligned");
+  WorkLayout L = make_work_layout(B, T, g);
+  hipStream_t s = (hipStream_t)stream;
+  char* wb = (char*)ws;
+  FusedArgs a;
+  memset(&a, 0, sizeof(a));
+  fill_common(a, g, prep, dtype);
+  a.x = x; a.h0 = h0; a.flags = flags; a.dy = dy; a.dh_last = dh_last;
+  a.flags_vec = (T % 16 == 0) && ((uintptr_t)flags % 16 == 0);
+  const ScratchLayout SL = make_scratch_layout(B, T, g, kScratchWide);
+  char* sb = (char*)scratch;
+  a.dx = dx; a.du_a = sb + SL.delta; a.dh0 = dh0;
+  a.ckpt = (float*)(wb + L.ckpt); a.rec_a = (rec_t*)(wb + L.b_rec_a);
+  a.ticket = (unsigned*)(wb + L.b_ticket); a.fail = (unsigned*)(wb + L.fail);
+  a.partial = (float*)(sb + SL.partial); a.dw_partial = (float*)(sb + SL.dw_partial);
+  a.B = (int)B; a.T = (int)T; a.nC = (int)((T + kChunk - 1) / kChunk); a.ckpt_nC = 2 * (int)L.nC; a.nCf = (int)L.nCf;
+  a.aligned = 1;
+  const int nkg = wide_groups(g, dtype, 1);
+  // reverse scan and gate math: direct part of dx, du2, per-workgroup bias and Lambda sums
+  a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nC, 1, L.max_wg);
+  a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
+  const bool masked = (flags != nullptr) || (T % kChunk != 0);
+  dim3 grid((unsigned)(a.wg_per_unit * a.units));
+  {
+    KernelTimer timer(1, s);
+#define RGLRU_LAUNCH_WIDE_SCAN(N)                                                                                    \
+    case N:                                                                                                          \
+      if (masked) hipLaunchKernelGGL((bwd_scan_kernel<__bf16, N, true>), grid, dim3(kThreads), 0, s, a);              \
+      else hipLaunchKernelGGL((bwd_scan_kernel<__bf16, N, false>), grid, dim3(kThreads), 0, s, a);                     \
+      break
+    switch (nkg) {
+      RGLRU_LAUNCH_WIDE_SCAN(10); RGLRU_LAUNCH_WIDE_SCAN(12); RGLRU_LAUNCH_WIDE_SCAN(16); RGLRU_LAUNCH_WIDE_SCAN(20);
+      RGLRU_LAUNCH_WIDE_SCAN(24);
+      default: return fail(RGLRU_E_UNSUPPORTED, "bwd_wide: no kernel for blocks of %lld channels", (long long)g.bw);
+    }
+#undef RGLRU_LAUNCH_WIDE_SCAN
+  }
+  rc = check_launch("bwd_wide scan");
+  if (rc) return rc;
+  // the two gate-gradient GEMMs: units of two slabs, one workgroup per compute unit
+  const int grad_units = (int)(nb * ((g.S + 1) / 2));
+  int n_wg = num_compute_units() / grad_units; if (n_wg < 1) n_wg = 1; if (n_wg > kWideWgPerUnit) n_wg = kWideWgPerUnit;
+  const long long grad_tiles = (B * T + 31) / 32;
+  if (n_wg > grad_tiles) n_wg = (int)grad_tiles;
+  dim3 grid2((unsigned)(n_wg * grad_units));
+  {
+    KernelTimer timer(3, s);
+    switch (nkg) {
+      case 10: hipLaunchKernelGGL((gate_grad_wide_kernel<__bf16, 10>), grid2, dim3(kGradThreads), 0, s, a); break;
+      case 12: hipLaunchKernelGGL((gate_grad_wide_kernel<__bf16, 12>), grid2, dim3(kGradThreads), 0, s, a); break;
+      case 16: hipLaunchKernelGGL((gate_grad_wide_kernel<__bf16, 16>), grid2, dim3(kGradThreads), 0, s, a); break;
+      case 20: hipLaunchKernelGGL((gate_grad_wide_kernel<__bf16, 20>), grid2, dim3(kGradThreads), 0, s, a); break;
+      default: hipLaunchKernelGGL((gate_grad_wide_kernel<__bf16, 24>), grid2, dim3(kGradThreads), 0, s, a); break;
+    }
+  }
+  rc = check_launch("bwd_wide gate gradients");
+  if (rc) return rc;
+  FinishArgs r;
+  memset(&r, 0, sizeof(r));
+  r.partial = a.partial; r.dsp = finish_dsp(g, prep, dtype); r.db_a = db_a; r.db_x = db_x; r.dlambda = dlambda;
+  r.dw_partial = a.dw_partial; r.dw_a = dw_a; r.dw_x = dw_x;
+  r.W = (int)W; r.nb = (int)nb; r.bw = (int)g.bw; r.bwp = (int)g.bwp; r.Wp = (int)g.Wp; r.wg_per_unit = a.wg_per_unit;
+  r.n_wg = n_wg; r.vec_blocks = (int)((W + 15) / 16); r.grad_dtype = grad_dtype;
+  r.clean = (uint4*)(wb + L.b_begin); r.clean_n = (long long)((L.b_end - L.b_begin) / 16);
+  const long long total = nb * g.bw * 2 * g.bw;
+  hipLaunchKernelGGL(finish_kernel, dim3((unsigned)(r.vec_blocks + (total / 4 + 255) / 256)), dim3(256), 0, s, r);
+  return check_launch("bwd_wide finish");
 }
 
 static int step_impl(const void* x, const void* prep, const float* h_in, float* h, const uint8_t* flags,

@@ -65,6 +65,7 @@ inline PrepLayout make_prep_layout(const Geometry& g, size_t elem) {
 //   b_ticket    [units][kMaxQueues]
 constexpr int kMaxQueues = 64;          // ticket queues per unit (sequences are dealt round-robin to them)
 constexpr int kGemmWgPerUnit = 32;      // workgroups per unit in the gradient kernel of the fast backward
+constexpr int kWideWgPerUnit = 8;       // ... and in the gate-gradient kernel of blocks wider than 128 channels
 
 struct WorkLayout {
   int64_t nC, nCf, max_wg;
@@ -96,19 +97,24 @@ inline WorkLayout make_work_layout(int64_t B, int64_t T, const Geometry& g) {
 
 // Scratch of one backward call; nothing in it outlives the call, its contents on entry do not matter.
 //   partial     [maxWg][3][Wp]  per-workgroup sums for db_a, db_x, dLambda
-//   delta       [B][T][W]       16-bit: dL/dh_t after the reverse scan (fast backward only)
-//   dw_partial  [kGemmWgPerUnit][nb][2][bwp][bwp] fp32 per-workgroup weight-gradient sums (fast backward only)
+//   delta       fast backward (blocks of 32, 64, 128 channels): [B][T][W] 16-bit, dL/dh_t after the
+//               reverse scan; wide backward (blocks of 160 .. 384 channels): [B][T][nb][2 bw] 16-bit,
+//               the gradients at the gate pre-activations as pairs (element 2 o + gate)
+//   dw_partial  [sets][nb][2][bwp][bwp] fp32 per-workgroup weight-gradient sums, sets = kGemmWgPerUnit
+//               (fast) or kWideWgPerUnit (wide)
+enum ScratchKind { kScratchPlain = 0, kScratchFast = 1, kScratchWide = 2 };
 struct ScratchLayout {
   size_t partial, delta, dw_partial, total;
 };
 
-inline ScratchLayout make_scratch_layout(int64_t B, int64_t T, const Geometry& g, bool fast) {
+inline ScratchLayout make_scratch_layout(int64_t B, int64_t T, const Geometry& g, int kind) {
   ScratchLayout s;
   size_t off = 0;
   auto take = [&](int64_t bytes) { size_t at = off; off += (size_t)round_up(bytes, 256); return at; };
   s.partial = take((int64_t)256 * 3 * g.Wp * 4);
-  s.delta = take(fast ? B * T * g.W * 2 : 0);
-  s.dw_partial = take(fast ? (int64_t)kGemmWgPerUnit * g.nb * g.bwp * 2 * g.bwp * 4 : 0);
+  s.delta = take(kind == kScratchFast ? B * T * g.W * 2 : kind == kScratchWide ? B * T * g.W * 4 : 0);
+  const int64_t sets = kind == kScratchFast ? kGemmWgPerUnit : kind == kScratchWide ? kWideWgPerUnit : 0;
+  s.dw_partial = take(sets * g.nb * g.bwp * 2 * g.bwp * 4);
   s.total = off;
   return s;
 }

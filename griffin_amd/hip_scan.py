@@ -187,8 +187,8 @@ def _check_fused_inputs(x: Tensor, w_a: Tensor, h0: Tensor | None, flags: Tensor
 def _uses_pre_path(lib, x: Tensor, W: int, nb: int, code: int) -> bool:
     """Blocks the kernels cannot hold the weights of (and other widths that are a multiple of 32):
     the gate projections run as one library GEMM, everything else in the HIP kernels."""
-    return bool(not lib.rglru_hip_fast_path(W, nb, code) and lib.rglru_hip_pre_path(W, nb, code)
-                and x.data_ptr() % 16 == 0)
+    return bool(not lib.rglru_hip_fast_path(W, nb, code) and not lib.rglru_hip_wide_path(W, nb, code)
+                and lib.rglru_hip_pre_path(W, nb, code) and x.data_ptr() % 16 == 0)
 
 
 def _gate_projections(x: Tensor, w_a: Tensor, w_x: Tensor) -> tuple[Tensor, Tensor, Tensor]:
@@ -275,6 +275,15 @@ class _HipRGLRU(torch.autograd.Function):
                                                   dw_x.data_ptr(), db_a.data_ptr(), db_x.data_ptr(), dlam.data_ptr(),
                                                   _ptr(dh0), B, T, W, nb, code, gcode, _stream_ptr(device)),
                            "rglru_hip_bwd_full")
+            elif lib.rglru_hip_wide_path(W, nb, code) and dy.data_ptr() % 16 == 0 and x.data_ptr() % 16 == 0:
+                # blocks of 160 .. 384 channels: scan and gate math, then the two gate GEMMs, all hand-written
+                dw_a = torch.empty(nb, bw, bw, dtype=gdt, device=device)
+                dw_x = torch.empty(nb, bw, bw, dtype=gdt, device=device)
+                _lib.check(lib.rglru_hip_bwd_wide(x.data_ptr(), image.data_ptr(), _ptr(h0c), _ptr(flags),
+                                                  dy.data_ptr(), _ptr(dhl), ws.data_ptr(), scratch.data_ptr(), dx.data_ptr(), dw_a.data_ptr(),
+                                                  dw_x.data_ptr(), db_a.data_ptr(), db_x.data_ptr(), dlam.data_ptr(),
+                                                  _ptr(dh0), B, T, W, nb, code, gcode, _stream_ptr(device)),
+                           "rglru_hip_bwd_wide")
             elif _uses_pre_path(lib, x, W, nb, code) and dy.data_ptr() % 16 == 0:
                 # gate projections recomputed by the library GEMM, the scan and all gate math in the
                 # HIP kernel, then the two GEMMs of the gate gradients on the kernel's du

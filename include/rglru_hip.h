@@ -46,7 +46,7 @@
 extern "C" {
 #endif
 
-#define RGLRU_ABI_VERSION 12
+#define RGLRU_ABI_VERSION 13
 
 enum { RGLRU_F32 = 0, RGLRU_BF16 = 1 };
 
@@ -159,6 +159,21 @@ int rglru_hip_bwd(const void* x, const void* prep, const float* h0,
  * configurations. */
 int rglru_hip_fast_path(int64_t W, int64_t nb, int dtype);
 int rglru_hip_bwd_full(const void* x, const void* y, const void* prep, const float* h0,
+                       const uint8_t* flags, const void* dy, const float* dh_last, void* ws, void* scratch,
+                       void* dx, void* dw_a, void* dw_x, void* db_a, void* db_x, void* dlambda,
+                       float* dh0, int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, int grad_dtype,
+                       void* stream);
+
+/* Complete backward for gate blocks of 160, 192, 256, 320 or 384 channels (rglru_hip_wide_path(W, nb,
+ * dtype) != 0: 16-bit storage; griffin/griffin.py:149-154 at those widths and its autograd).  For these
+ * widths rglru_hip_fwd and rglru_hip_prepare_fwd hold a block's weights in the registers of several
+ * workgroups (four 32-channel slabs each), and this entry point is the matching backward: same inputs
+ * and outputs as rglru_hip_bwd_full without y (the states come from the checkpoints in `ws`).  Two
+ * hand-written kernels: reverse scan and gate math (direct part of dx, the gradients at the gate
+ * pre-activations as 16-bit pairs in `scratch`), then the two block-diagonal GEMMs on the matrix unit
+ * (dx += du W and dW = du^T x).  Returns RGLRU_E_UNSUPPORTED for other configurations. */
+int rglru_hip_wide_path(int64_t W, int64_t nb, int dtype);
+int rglru_hip_bwd_wide(const void* x, const void* prep, const float* h0,
                        const uint8_t* flags, const void* dy, const float* dh_last, void* ws, void* scratch,
                        void* dx, void* dw_a, void* dw_x, void* db_a, void* db_x, void* dlambda,
                        float* dh0, int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, int grad_dtype,

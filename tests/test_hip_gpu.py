@@ -109,7 +109,7 @@ BF16_CASES = [
     (2, 200, 256, 2, True, True),    # 128-wide blocks: register-held weights
     (2, 96, 128, 2, False, False),   # 64-wide blocks
     (2, 64, 64, 2, True, False),     # 32-wide blocks
-    (1, 150, 640, 2, True, True),    # 320-wide blocks: streamed weights, two LDS slices
+    (1, 150, 640, 2, True, True),    # 320-wide blocks: three workgroups share a block (4 + 4 + 2 slabs)
     (2, 33, 24, 3, True, True),      # unaligned rows (width 24 -> 48-byte rows, 8-wide blocks)
     (2, 75, 256, 2, False, True),    # fast kernels with a ragged last tile and no flags
     (2, 80, 256, 2, True, False),    # length a multiple of 16 but not of 32: vector flag loads, half-empty tile
@@ -120,10 +120,14 @@ BF16_CASES = [
     (2, 70, 96, 3, False, True),     # 32-wide blocks packed four to a unit, last unit one block short
     (1, 64, 64, 1, False, False),    # a single 64-wide block: half of the packed unit idles
     (2, 64, 1024, 16, True, False),  # reference default of 16 gate blocks at width 1024
-    (2, 100, 512, 2, True, True),    # 256-wide blocks: library GEMM for the projections, two workgroups per block
+    (2, 100, 512, 2, True, True),    # 256-wide blocks: two workgroups per block
     (2, 75, 480, 3, False, True),    # 160-wide blocks: five slabs, the second workgroup of a block has one
     (1, 64, 96, 1, True, False),     # 96-wide block: three slabs in one workgroup
     (3, 33, 384, 2, True, True),     # 192-wide blocks, ragged tile, flags
+    (2, 128, 640, 2, False, False),  # 320-wide blocks, whole tiles, no flags, no state: the unmasked wide kernels
+    (1, 300, 768, 2, True, True),    # 384-wide blocks, the widest the kernels hold in registers
+    (5, 70, 320, 1, True, False),    # one 320-wide block, more sequences than tiles per sequence
+    (1, 90, 448, 1, True, True),     # 448-wide block: not held in registers, projections by the library GEMM
 ]
 
 
