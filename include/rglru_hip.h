@@ -9,9 +9,11 @@
  *   griffin/triton_scan.py:207-244  _FusedRGLRUScan.forward   rglru_hip_scan_fwd
  *   griffin/triton_scan.py:246-271  _FusedRGLRUScan.backward  rglru_hip_scan_bwd
  *   griffin/griffin.py:237-289      RG_LRU.forward (gates + scan, T > 1)   rglru_hip_prepare + rglru_hip_fwd
- *   autograd of griffin/griffin.py:237-289                                   rglru_hip_bwd, rglru_hip_bwd_full
+ *   autograd of griffin/griffin.py:237-289                                   rglru_hip_bwd_full (blocks of 32/64/128 channels),
+ *                                                                            rglru_hip_bwd_wide (160 .. 384), rglru_hip_bwd (any)
  *   the same with the gate projections (griffin/griffin.py:149-154) left to a BLAS GEMM   rglru_hip_fwd_pre, rglru_hip_bwd_pre
- *   griffin/griffin.py:279-284 with T == 1 (decode step, carried state)     rglru_hip_step
+ *   griffin/griffin.py:279-284 with T == 1 (decode step, carried state)     rglru_hip_step, rglru_hip_steps (K steps a launch)
+ *   (no counterpart: forward for callers that cannot allocate)              rglru_hip_fwd_static
  *   griffin/griffin.py:474-487      causal depthwise convolution of the caller   rglru_hip_conv_fwd
  *   autograd of griffin/griffin.py:474-487                                   rglru_hip_conv_bwd
  *   griffin/griffin.py:488-510      the same over right-padded batches and its autograd   rglru_hip_conv_padded_fwd, _bwd
@@ -179,8 +181,8 @@ int rglru_hip_bwd_wide(const void* x, const void* prep, const float* h0,
                        float* dh0, int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, int grad_dtype,
                        void* stream);
 
-/* Variant for gate blocks too wide for the kernels to keep their weights on chip (and for any block
- * width that is a multiple of 32 channels up to 512, bf16 storage, 16-byte aligned tensors;
+/* Variant for the block widths that neither rglru_hip_fast_path nor rglru_hip_wide_path covers (any
+ * multiple of 32 channels up to 512, e.g. 224, 448, 480 or 512; bf16 storage, 16-byte aligned tensors;
  * rglru_hip_pre_path() says whether a configuration qualifies).  The caller runs the two block-diagonal
  * projections of griffin/griffin.py:149-154 as ONE batched GEMM of its BLAS library and hands the
  * result in:
