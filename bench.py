@@ -1,19 +1,27 @@
 """Benchmark of the fused RG-LRU forward + backward on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-graph] [--workload NAME]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--repeats R] [--input-sets S] [--no-cpu] [--no-graph]
+                    [--workload NAME]
 
 One step = one forward + one backward of the RG-LRU (gates + scan, recomputing backward) over one
 batch of synthetic input, B=8, T=2048, W=1024, 8 gate blocks, bf16 storage with fp32 state: the
 configuration the headline metric is quoted on.  Inputs are resident in HBM before the timed region.
-Prints ONE JSON line.
+The steps are replayed as HIP graphs of ten steps that rotate through S distinct input sets (cache-cold);
+the figure is the median of R timed regions of exactly K steps.  Prints ONE JSON line: metric, the
+whole-step HBM roofline (5 s N algorithmic bytes over the step time; measured traffic from the committed
+profile summary if it was taken on the current kernel sources), per-kernel HIP-event durations, a check
+of the captured step against an eager one (exit status 1 if they differ) and the CPU baseline (the oracle
+on a bounded sample of the same workload, all threads and one thread).
 
---workload selects one of the other measured configurations instead (eager launches, one JSON line
-without the roofline and CPU legs; their per-kernel figures come from rocprofv3 runs of the same
-command, summarised under profiles/):
-    block         RMSNorm + RecurrentBlock(768, 1024) forward + backward at B8 T2048, bf16
-    long_context  RG-LRU forward + backward at B1 T32768 W2560, 8 blocks of 320 channels, slow decay
-    decode        512 single-token RG-LRU steps at B256 W1024 after a T2048 prefill
-    block_decode  64 single-token RecurrentBlock(768, 1024) steps at B256 after a T128 prefill
+--workload selects one of the other measured configurations instead (one JSON line without the CPU
+leg; their per-kernel figures come from rocprofv3 runs of the same command, summarised under profiles/):
+    scan_only     the scan-only operator (fp32 a, z -> h) forward + backward at B8 T2048 W1024, HIP graph
+    block         RMSNorm + RecurrentBlock(768, 1024) forward + backward at B8 T2048, bf16, eager
+    long_context  RG-LRU forward + backward at B1 T32768 W2560, 8 blocks of 320 channels, slow decay, eager
+    decode        512 single-token RG-LRU steps at B256 W1024 after a T2048 prefill: eager, a HIP graph of
+                  64 single-step launches, and one launch for all steps
+    block_decode  64 single-token RecurrentBlock(768, 1024) steps at B256 after a T128 prefill: eager and
+                  as one HIP graph
 """
 
 from __future__ import annotations
