@@ -1979,33 +1979,49 @@ __global__ __launch_bounds__(kThreads) void step_kernel(FusedArgs p) {
   const long long W = p.W;
   const long long row0 = (long long)w.wg_in_unit * TR;
 
-  // the lane's previous states, gate values and flags: requested first, they arrive while the
-  // projections are computed (the step is a chain of latencies, not of bytes)
   float h_old[EL], gate[EL];
   unsigned fls[EL];
+  auto load_state = [&]() {
 #pragma unroll
-  for (int e = 0; e < EL; ++e) {
-    const long long row = row0 + hf * EL + e;
-    const bool ok = w.ch_ok && row < p.B;
-    const long long at = ok ? row * W + w.ch : 0;
-    h_old[e] = ok ? p.h_prev[at] : 0.f;
-    gate[e] = (ok && p.gate_v) ? (float)((const IO*)p.gate_v)[at] : 0.f;
-    fls[e] = (ok && p.flags) ? (unsigned)p.flags[row] : 0u;
-  }
+    for (int e = 0; e < EL; ++e) {
+      const long long row = row0 + hf * EL + e;
+      const bool ok = w.ch_ok && row < p.B;
+      const long long at = ok ? row * W + w.ch : 0;
+      h_old[e] = ok ? p.h_prev[at] : 0.f;
+      gate[e] = (ok && p.gate_v) ? (float)((const IO*)p.gate_v)[at] : 0.f;
+      fls[e] = (ok && p.flags) ? (unsigned)p.flags[row] : 0u;
+    }
+  };
   f32x16 ua[MT], ux[MT];
   float xv[EL];
   if constexpr (NKG > 0) {
+    // Loads return in issue order and the step is a chain of latencies, not of bytes: the x tile (which
+    // has to pass through LDS and a barrier) is requested first, the weights next, the lane's previous
+    // states, gate values and flags last; they arrive while the projections are computed.  (9.05 us per
+    // step with the states requested first, 7.66 us in this order, B256 W1024 in a HIP graph; x rows
+    // loaded straight into MFMA fragments instead of through LDS: 8.2 us, 32 rows per load instruction.)
+    constexpr int VPR = KC / Tr::HW;
+    constexpr int NVX = (TR * VPR + kThreads - 1) / kThreads;
+    Frag xin[NVX];
+#pragma unroll
+    for (int i = 0; i < NVX; ++i) {
+      const int idx = tid + i * kThreads;
+      const int row = idx / VPR, cv = idx - row * VPR;
+      xin[i] = idx < TR * VPR ? load_x_frag<IO>(p, (const IO*)p.x, row0 + row, p.B, w.k, cv * Tr::HW) : Tr::zero();
+    }
     HeldWeights<IO, NKG> hw;
     hw.load(w_a_row, w_x_row);
-    constexpr int VPR = KC / Tr::HW;
-    for (int idx = tid; idx < TR * VPR; idx += kThreads) {
+    load_state();
+#pragma unroll
+    for (int i = 0; i < NVX; ++i) {
+      const int idx = tid + i * kThreads;
       const int row = idx / VPR, cv = idx - row * VPR;
-      Frag v = load_x_frag<IO>(p, (const IO*)p.x, row0 + row, p.B, w.k, cv * Tr::HW);
-      *reinterpret_cast<Frag*>(lds + row * LDSROW + cv * Tr::HW) = v;
+      if (idx < TR * VPR) *reinterpret_cast<Frag*>(lds + row * LDSROW + cv * Tr::HW) = xin[i];
     }
     __syncthreads();
     if (w.slab_ok) gate_mfma_held<IO, MT, NKG>(lds, hw, 0, w.slab, w.r, hf, bias_a, bias_x, ua[0], ux[0], xv);
   } else {
+    load_state();
     gate_tile_generic<IO, MT>(p, (const IO*)p.x, row0, p.B, w.k, w.slab, w.slab_ok, w_a_row, w_x_row,
                               bias_a, bias_x, lds, ua, ux, xv);
   }
@@ -2020,6 +2036,76 @@ __global__ __launch_bounds__(kThreads) void step_kernel(FusedArgs p) {
     float h = fmaf(go.a, h_old[e], go.z);
     p.h_state[at] = h;
     if (p.gate_v) h *= gelu_tanh_parts(gate[e]).gelu;
+    y[at] = (IO)h;
+  }
+}
+
+// Decode step for 16-bit storage and gate blocks of 32, 64 or 128 channels, on 16 x 16 MFMA tiles: a wave
+// owns 16 sequences x 16 channels, a lane 4 sequences of one channel.  The step is a chain of latencies
+// (launch, loads, products, gate math, stores), so the work is cut as fine as the matrix unit allows:
+// four elements of gate math per lane instead of sixteen, 8 KB of weights per wave instead of 16, x rows
+// straight into A fragments (16 rows of 64 contiguous bytes per load instruction; no LDS, no barrier),
+// and at B256 W1024 one workgroup on every compute unit instead of on a quarter of them.
+template <int NKS>
+__global__ __launch_bounds__(kThreads) void step16_kernel(FusedArgs p) {
+  typedef __bf16 IO;
+  typedef bf16x8 Frag;
+  typedef float f32x4v __attribute__((ext_vector_type(4)));
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n = lane & 15, q = lane >> 4;
+  const int ctiles = p.W / 16;
+  const long long wv = (long long)blockIdx.x * kWaves + wave;
+  const int ct = (int)(wv % ctiles);
+  const long long row0 = (wv / ctiles) * 16;
+  if (row0 >= p.B) return;
+  const long long W = p.W;
+  const int ch = ct * 16 + n;                              // the lane's channel; a tile lies inside one gate block
+  const int k = ch / p.bw, o = ch - k * p.bw;
+  const int kp = k * p.bwp + o;
+  // A fragments: row m = lane % 16 is sequence row0 + m, element j of K step ks is input channel 32 ks + 8 q + j
+  const long long arow = row0 + n;
+  const bool arow_ok = arow < p.B;
+  const IO* xr = (const IO*)p.x + (arow_ok ? arow : 0) * W + k * p.bw + 8 * q;
+  Frag xa[NKS], fa[NKS], fx[NKS];
+#pragma unroll
+  for (int ks = 0; ks < NKS; ++ks) xa[ks] = arow_ok ? *reinterpret_cast<const Frag*>(xr + 32 * ks) : Io<IO>::zero();
+  // B fragments: column n is output channel o, same K elements: rows of the two weight matrices
+  const IO* wa = (const IO*)p.wg + ((long long)(0 * p.nb + k) * p.bwp + o) * p.bwp + 8 * q;
+  const IO* wx = (const IO*)p.wg + ((long long)(1 * p.nb + k) * p.bwp + o) * p.bwp + 8 * q;
+#pragma unroll
+  for (int ks = 0; ks < NKS; ++ks) {
+    fa[ks] = *reinterpret_cast<const Frag*>(wa + 32 * ks);
+    fx[ks] = *reinterpret_cast<const Frag*>(wx + 32 * ks);
+  }
+  // accumulator register v of the lane is sequence row0 + 4 q + v
+  float h_old[4], gate[4], xv[4];
+  unsigned fls[4];
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    const long long row = row0 + 4 * q + v;
+    const bool ok = row < p.B;
+    const long long at = ok ? row * W + ch : 0;
+    h_old[v] = ok ? p.h_prev[at] : 0.f;
+    xv[v] = ok ? (float)((const IO*)p.x)[at] : 0.f;
+    gate[v] = (ok && p.gate_v) ? (float)((const IO*)p.gate_v)[at] : 0.f;
+    fls[v] = (ok && p.flags) ? (unsigned)p.flags[row] : 0u;
+  }
+  const float bias_a = p.bias[kp], bias_x = p.bias[p.Wp + kp], sp = p.sp[kp];
+  f32x4v ua = {bias_a, bias_a, bias_a, bias_a}, ux = {bias_x, bias_x, bias_x, bias_x};
+#pragma unroll
+  for (int ks = 0; ks < NKS; ++ks) {
+    ua = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[ks], fa[ks], ua, 0, 0, 0);
+    ux = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[ks], fx[ks], ux, 0, 0, 0);
+  }
+  IO* y = (IO*)p.y;
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    const long long row = row0 + 4 * q + v;
+    if (row >= p.B) break;
+    const GateOut go = gate_forward<Precise<IO>::value, true>(ua[v], ux[v], xv[v], sp, fls[v]);
+    const long long at = row * W + ch;
+    float h = fmaf(go.a, h_old[v], go.z);
+    p.h_state[at] = h;
+    if (p.gate_v) h *= gelu_tanh_parts(gate[v]).gelu;
     y[at] = (IO)h;
   }
 }
@@ -2745,9 +2831,19 @@ static int step_impl(const void* x, const void* prep, const float* h_in, float* 
   long long row_tiles = (B + 31) / 32;
   dim3 grid((unsigned)(row_tiles * g.units));
   hipStream_t s = (hipStream_t)stream;
+  const int nkg = held_groups(g, dtype, a.aligned);
   {
     KernelTimer timer(2, s);
-    RGLRU_DISPATCH(step_kernel, grid, s, a, dtype, held_groups(g, dtype, a.aligned));
+    if (nkg > 0) {
+      // 16 sequences x 16 channels per wave, four waves per workgroup
+      const long long waves = ((B + 15) / 16) * (W / 16);
+      dim3 grid16((unsigned)((waves + kWaves - 1) / kWaves));
+      if (nkg == 8) hipLaunchKernelGGL((step16_kernel<4>), grid16, dim3(kThreads), 0, s, a);
+      else if (nkg == 4) hipLaunchKernelGGL((step16_kernel<2>), grid16, dim3(kThreads), 0, s, a);
+      else hipLaunchKernelGGL((step16_kernel<1>), grid16, dim3(kThreads), 0, s, a);
+    } else {
+      RGLRU_DISPATCH(step_kernel, grid, s, a, dtype, 0);
+    }
   }
   return check_launch("step");
 }
