@@ -2110,6 +2110,87 @@ __global__ __launch_bounds__(kThreads) void step16_kernel(FusedArgs p) {
   }
 }
 
+// K consecutive decode steps on the tiling of step16_kernel: weights and the lane's four states stay in
+// registers, the next step's x fragments, own x values and flags are requested before the current step
+// is computed.
+template <int NKS>
+__global__ __launch_bounds__(kThreads) void steps16_kernel(FusedArgs p) {
+  typedef __bf16 IO;
+  typedef bf16x8 Frag;
+  typedef float f32x4v __attribute__((ext_vector_type(4)));
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n = lane & 15, q = lane >> 4;
+  const int ctiles = p.W / 16;
+  const long long wv = (long long)blockIdx.x * kWaves + wave;
+  const int ct = (int)(wv % ctiles);
+  const long long row0 = (wv / ctiles) * 16;
+  if (row0 >= p.B) return;
+  const long long W = p.W;
+  const int ch = ct * 16 + n;
+  const int k = ch / p.bw, o = ch - k * p.bw;
+  const int kp = k * p.bwp + o;
+  const long long step_elems = (long long)p.B * W;
+  const int steps = p.T;
+  const long long arow = row0 + n;
+  const bool arow_ok = arow < p.B;
+  const IO* xr = (const IO*)p.x + (arow_ok ? arow : 0) * W + k * p.bw + 8 * q;
+  Frag fa[NKS], fx[NKS];
+  const IO* wa = (const IO*)p.wg + ((long long)(0 * p.nb + k) * p.bwp + o) * p.bwp + 8 * q;
+  const IO* wx = (const IO*)p.wg + ((long long)(1 * p.nb + k) * p.bwp + o) * p.bwp + 8 * q;
+#pragma unroll
+  for (int ks = 0; ks < NKS; ++ks) {
+    fa[ks] = *reinterpret_cast<const Frag*>(wa + 32 * ks);
+    fx[ks] = *reinterpret_cast<const Frag*>(wx + 32 * ks);
+  }
+  long long at[4];
+  bool ok[4];
+  float h[4];
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    const long long row = row0 + 4 * q + v;
+    ok[v] = row < p.B;
+    at[v] = ok[v] ? row * W + ch : 0;
+    h[v] = ok[v] ? p.h_prev[at[v]] : 0.f;
+  }
+  const float bias_a = p.bias[kp], bias_x = p.bias[p.Wp + kp], sp = p.sp[kp];
+  Frag xa[NKS];
+  IO xv[4];
+  unsigned fls[4];
+  auto issue = [&](int t) {
+    const bool live = t < steps;
+    const long long base = live ? (long long)t * step_elems : 0;
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) xa[ks] = (arow_ok && live) ? *reinterpret_cast<const Frag*>(xr + base + 32 * ks) : Io<IO>::zero();
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      xv[v] = (ok[v] && live) ? ((const IO*)p.x)[base + at[v]] : (IO)0.0f;
+      fls[v] = (p.flags && ok[v] && live) ? (unsigned)p.flags[(long long)t * p.B + row0 + 4 * q + v] : 0u;
+    }
+  };
+  issue(0);
+  for (int t = 0; t < steps; ++t) {
+    f32x4v ua = {bias_a, bias_a, bias_a, bias_a}, ux = {bias_x, bias_x, bias_x, bias_x};
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) {
+      ua = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[ks], fa[ks], ua, 0, 0, 0);
+      ux = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[ks], fx[ks], ux, 0, 0, 0);
+    }
+    float xcur[4];
+    unsigned fcur[4];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) { xcur[v] = (float)xv[v]; fcur[v] = fls[v]; }
+    issue(t + 1);
+    IO* y = (IO*)p.y + (long long)t * step_elems;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const GateOut go = gate_forward<Precise<IO>::value, true>(ua[v], ux[v], xcur[v], sp, fcur[v]);
+      h[v] = fmaf(go.a, h[v], go.z);
+      if (ok[v]) y[at[v]] = (IO)h[v];
+    }
+  }
+#pragma unroll
+  for (int v = 0; v < 4; ++v) if (ok[v]) p.h_state[at[v]] = h[v];
+}
+
 // K consecutive decode steps in one launch (teacher-forced inputs x[K, B, W]): the state stays in
 // registers across the steps, the gate weights are loaded once, and the next step's x tile is requested
 // while the current step is computed.  Same arithmetic as step_kernel, step by step.
@@ -2875,9 +2956,18 @@ int rglru_hip_steps(const void* x, const void* prep, float* h, const uint8_t* fl
   long long row_tiles = (B + 31) / 32;
   dim3 grid((unsigned)(row_tiles * g.units));
   hipStream_t s = (hipStream_t)stream;
+  const int nkg = held_groups(g, dtype, a.aligned);
   {
     KernelTimer timer(2, s);
-    RGLRU_DISPATCH(steps_kernel, grid, s, a, dtype, held_groups(g, dtype, a.aligned));
+    if (nkg > 0) {
+      const long long waves = ((B + 15) / 16) * (W / 16);
+      dim3 grid16((unsigned)((waves + kWaves - 1) / kWaves));
+      if (nkg == 8) hipLaunchKernelGGL((steps16_kernel<4>), grid16, dim3(kThreads), 0, s, a);
+      else if (nkg == 4) hipLaunchKernelGGL((steps16_kernel<2>), grid16, dim3(kThreads), 0, s, a);
+      else hipLaunchKernelGGL((steps16_kernel<1>), grid16, dim3(kThreads), 0, s, a);
+    } else {
+      RGLRU_DISPATCH(steps_kernel, grid, s, a, dtype, 0);
+    }
   }
   return check_launch("steps");
 }
