@@ -2344,7 +2344,7 @@ static int held_groups(const Geometry& g, int dtype, int aligned) {
 static int wide_groups(const Geometry& g, int dtype, int aligned) {
   if (dtype != RGLRU_BF16 || !aligned) return 0;
   switch (g.bw) {
-    case 160: case 192: case 256: case 320: case 384: return (int)(g.bw / 16);
+    case 160: case 192: case 224: case 256: case 288: case 320: case 352: case 384: return (int)(g.bw / 16);
     default: return 0;
   }
 }
@@ -2361,8 +2361,9 @@ static int wide_groups(const Geometry& g, int dtype, int aligned) {
     else if ((dtype) == RGLRU_BF16 && (nkg) == 2 && !(masked)) hipLaunchKernelGGL((fwd_kernel<__bf16, 2, false>), grid, dim3(kThreads), 0, stream, args); \
     else if ((dtype) == RGLRU_BF16 && (nkg) == 2) hipLaunchKernelGGL((fwd_kernel<__bf16, 2, true>), grid, dim3(kThreads), 0, stream, args); \
     RGLRU_FWD_WIDE_CASE(10, grid, stream, args, dtype, nkg, masked) RGLRU_FWD_WIDE_CASE(12, grid, stream, args, dtype, nkg, masked) \
-    RGLRU_FWD_WIDE_CASE(16, grid, stream, args, dtype, nkg, masked) RGLRU_FWD_WIDE_CASE(20, grid, stream, args, dtype, nkg, masked) \
-    RGLRU_FWD_WIDE_CASE(24, grid, stream, args, dtype, nkg, masked)                                                                  \
+    RGLRU_FWD_WIDE_CASE(14, grid, stream, args, dtype, nkg, masked) RGLRU_FWD_WIDE_CASE(16, grid, stream, args, dtype, nkg, masked) \
+    RGLRU_FWD_WIDE_CASE(18, grid, stream, args, dtype, nkg, masked) RGLRU_FWD_WIDE_CASE(20, grid, stream, args, dtype, nkg, masked) \
+    RGLRU_FWD_WIDE_CASE(22, grid, stream, args, dtype, nkg, masked) RGLRU_FWD_WIDE_CASE(24, grid, stream, args, dtype, nkg, masked) \
     else if ((dtype) == RGLRU_BF16 && (nkg) < 0 && !(masked)) hipLaunchKernelGGL((fwd_kernel<__bf16, -1, false>), grid, dim3(kThreads), 0, stream, args); \
     else if ((dtype) == RGLRU_BF16 && (nkg) < 0) hipLaunchKernelGGL((fwd_kernel<__bf16, -1, true>), grid, dim3(kThreads), 0, stream, args); \
     else if ((dtype) == RGLRU_BF16) hipLaunchKernelGGL((fwd_kernel<__bf16, 0, true>), grid, dim3(kThreads), 0, stream, args); \
@@ -2818,7 +2819,7 @@ int rglru_hip_bwd_wide(const void* x, const void* prep, const float* h0,
   rc = check_grad_dtype("bwd_wide", grad_dtype);
   if (rc) return rc;
   if (!rglru_hip_wide_path(W, nb, dtype))
-    return fail(RGLRU_E_UNSUPPORTED, "bwd_wide: needs 16-bit storage and gate blocks of 160, 192, 256, 320 or 384 channels");
+    return fail(RGLRU_E_UNSUPPORTED, "bwd_wide: needs 16-bit storage and gate blocks of 160 to 384 channels in steps of 32");
   if (B <= 0 || T <= 0) return fail(RGLRU_E_ARG, "bwd_wide: B and T must be positive (got %lld, %lld)", (long long)B, (long long)T);
   if (!x || !prep || !dy || !ws || !scratch || !dx || !dw_a || !dw_x || !db_a || !db_x || !dlambda)
     return fail(RGLRU_E_ARG, "bwd_wide: null pointer");
@@ -2857,8 +2858,8 @@ int rglru_hip_bwd_wide(const void* x, const void* prep, const float* h0,
       else hipLaunchKernelGGL((bwd_scan_kernel<__bf16, N, false>), grid, dim3(kThreads), 0, s, a);                     \
       break
     switch (nkg) {
-      RGLRU_LAUNCH_WIDE_SCAN(10); RGLRU_LAUNCH_WIDE_SCAN(12); RGLRU_LAUNCH_WIDE_SCAN(16); RGLRU_LAUNCH_WIDE_SCAN(20);
-      RGLRU_LAUNCH_WIDE_SCAN(24);
+      RGLRU_LAUNCH_WIDE_SCAN(10); RGLRU_LAUNCH_WIDE_SCAN(12); RGLRU_LAUNCH_WIDE_SCAN(14); RGLRU_LAUNCH_WIDE_SCAN(16);
+      RGLRU_LAUNCH_WIDE_SCAN(18); RGLRU_LAUNCH_WIDE_SCAN(20); RGLRU_LAUNCH_WIDE_SCAN(22); RGLRU_LAUNCH_WIDE_SCAN(24);
       default: return fail(RGLRU_E_UNSUPPORTED, "bwd_wide: no kernel for blocks of %lld channels", (long long)g.bw);
     }
 #undef RGLRU_LAUNCH_WIDE_SCAN
@@ -2876,8 +2877,11 @@ int rglru_hip_bwd_wide(const void* x, const void* prep, const float* h0,
     switch (nkg) {
       case 10: hipLaunchKernelGGL((gate_grad_wide_kernel<__bf16, 10>), grid2, dim3(kGradThreads), 0, s, a); break;
       case 12: hipLaunchKernelGGL((gate_grad_wide_kernel<__bf16, 12>), grid2, dim3(kGradThreads), 0, s, a); break;
+      case 14: hipLaunchKernelGGL((gate_grad_wide_kernel<__bf16, 14>), grid2, dim3(kGradThreads), 0, s, a); break;
       case 16: hipLaunchKernelGGL((gate_grad_wide_kernel<__bf16, 16>), grid2, dim3(kGradThreads), 0, s, a); break;
+      case 18: hipLaunchKernelGGL((gate_grad_wide_kernel<__bf16, 18>), grid2, dim3(kGradThreads), 0, s, a); break;
       case 20: hipLaunchKernelGGL((gate_grad_wide_kernel<__bf16, 20>), grid2, dim3(kGradThreads), 0, s, a); break;
+      case 22: hipLaunchKernelGGL((gate_grad_wide_kernel<__bf16, 22>), grid2, dim3(kGradThreads), 0, s, a); break;
       default: hipLaunchKernelGGL((gate_grad_wide_kernel<__bf16, 24>), grid2, dim3(kGradThreads), 0, s, a); break;
     }
   }

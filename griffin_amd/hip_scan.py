@@ -185,8 +185,8 @@ def _check_fused_inputs(x: Tensor, w_a: Tensor, h0: Tensor | None, flags: Tensor
 
 
 def _uses_pre_path(lib, x: Tensor, W: int, nb: int, code: int) -> bool:
-    """Block widths that are a multiple of 32 but have no kernel with register-held weights (224, 448,
-    480, 512, ...): the gate projections run as one library GEMM, everything else in the HIP kernels."""
+    """Block widths that are a multiple of 32 but have no kernel with register-held weights (416, 448,
+    480, 512): the gate projections run as one library GEMM, everything else in the HIP kernels."""
     return bool(not lib.rglru_hip_fast_path(W, nb, code) and not lib.rglru_hip_wide_path(W, nb, code)
                 and lib.rglru_hip_pre_path(W, nb, code) and x.data_ptr() % 16 == 0)
 

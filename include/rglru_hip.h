@@ -166,7 +166,7 @@ int rglru_hip_bwd_full(const void* x, const void* y, const void* prep, const flo
                        float* dh0, int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, int grad_dtype,
                        void* stream);
 
-/* Complete backward for gate blocks of 160, 192, 256, 320 or 384 channels (rglru_hip_wide_path(W, nb,
+/* Complete backward for gate blocks of 160 to 384 channels in steps of 32 (rglru_hip_wide_path(W, nb,
  * dtype) != 0: 16-bit storage; griffin/griffin.py:149-154 at those widths and its autograd).  For these
  * widths rglru_hip_fwd and rglru_hip_prepare_fwd hold a block's weights in the registers of several
  * workgroups (four 32-channel slabs each), and this entry point is the matching backward: same inputs
@@ -182,7 +182,7 @@ int rglru_hip_bwd_wide(const void* x, const void* prep, const float* h0,
                        void* stream);
 
 /* Variant for the block widths that neither rglru_hip_fast_path nor rglru_hip_wide_path covers (any
- * multiple of 32 channels up to 512, e.g. 224, 448, 480 or 512; bf16 storage, 16-byte aligned tensors;
+ * multiple of 32 channels up to 512, i.e. 416, 448, 480 or 512; bf16 storage, 16-byte aligned tensors;
  * rglru_hip_pre_path() says whether a configuration qualifies).  The caller runs the two block-diagonal
  * projections of griffin/griffin.py:149-154 as ONE batched GEMM of its BLAS library and hands the
  * result in:

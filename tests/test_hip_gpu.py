@@ -128,6 +128,9 @@ BF16_CASES = [
     (1, 300, 768, 2, True, True),    # 384-wide blocks, the widest the kernels hold in registers
     (5, 70, 320, 1, True, False),    # one 320-wide block, more sequences than tiles per sequence
     (1, 90, 448, 1, True, True),     # 448-wide block: not held in registers, projections by the library GEMM
+    (2, 70, 448, 2, True, True),     # 224-wide blocks: seven slabs, K tiles not a multiple of four
+    (1, 100, 288, 1, False, True),   # one 288-wide block
+    (1, 64, 704, 2, True, False),    # 352-wide blocks
     (2, 1, 320, 1, True, True),      # a single token through the wide training kernels
     (1, 31, 512, 2, False, True),    # 256-wide blocks, shorter than one backward chunk
 ]
