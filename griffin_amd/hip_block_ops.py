@@ -13,7 +13,7 @@ from torch import Tensor
 from torch.autograd.function import once_differentiable
 
 from . import _lib
-from .hip_scan import _DTYPE_CODES, _dtype_code, _ptr, _require_gpu, _stream_ptr
+from .hip_scan import _DTYPE_CODES, _dtype_code, _on_device, _ptr, _require_gpu, _stream_ptr
 
 
 def max_kernel_size() -> int:
@@ -56,7 +56,7 @@ class _HipCausalConv(torch.autograd.Function):
         pos = segment_pos.to(device=u.device, dtype=torch.int64).contiguous()
         out = torch.empty_like(u_c)
         lib = _lib.load()
-        with torch.cuda.device(u.device):
+        with _on_device(u.device):
             _lib.check(lib.rglru_hip_conv_fwd(
                 _ptr(u_c), _ptr(state_c), _ptr(taps), _ptr(bias_c), _ptr(pos), _ptr(out), None,
                 batch, steps, width, taps_count, code, _DTYPE_CODES[taps.dtype], _stream_ptr(u.device)),
@@ -86,7 +86,7 @@ class _HipCausalConv(torch.autograd.Function):
         dbias = torch.empty(width, device=u.device, dtype=grad_dtype) if (need_b and bias_dtype is not None) else None
         scratch = torch.empty(lib.rglru_hip_conv_scratch_bytes(batch, steps, width, taps_count),
                               device=u.device, dtype=torch.uint8)
-        with torch.cuda.device(u.device):
+        with _on_device(u.device):
             _lib.check(lib.rglru_hip_conv_bwd(
                 _ptr(u), _ptr(state), _ptr(taps), _ptr(pos), _ptr(dout_c), _ptr(scratch), _ptr(du),
                 _ptr(dstate), _ptr(dtaps), _ptr(dbias),
@@ -143,7 +143,7 @@ class _HipCausalConvPadded(torch.autograd.Function):
         pos = segment_pos.to(device=u.device, dtype=torch.int64).contiguous()
         live = active_mask.to(device=u.device, dtype=torch.uint8).contiguous()
         lib = _lib.load()
-        with torch.cuda.device(u.device):
+        with _on_device(u.device):
             out = torch.empty_like(u_c)
             new_state = u.new_empty(batch, taps_count - 1, width)
             scratch = torch.empty(lib.rglru_hip_conv_padded_scratch_bytes(batch, steps), dtype=torch.uint8, device=u.device)
@@ -171,7 +171,7 @@ class _HipCausalConvPadded(torch.autograd.Function):
         lib = _lib.load()
         need_u, need_state, need_w, need_b = ctx.needs_input_grad[:4]
         grad_dtype = taps.dtype
-        with torch.cuda.device(u.device):
+        with _on_device(u.device):
             du = torch.empty_like(u)
             dstate = u.new_empty(batch, taps_count - 1, width) if (need_state and taps_count > 1) else None
             dtaps = torch.empty(width, taps_count, device=u.device, dtype=grad_dtype) if need_w else None
@@ -215,7 +215,7 @@ class _HipGeluGate(torch.autograd.Function):
         h_c, v_c = h.contiguous(), v.contiguous()
         out = torch.empty_like(h_c)
         if h_c.numel():
-            with torch.cuda.device(h.device):
+            with _on_device(h.device):
                 _lib.check(_lib.load().rglru_hip_gelu_gate_fwd(
                     _ptr(h_c), _ptr(v_c), _ptr(out), h_c.numel(), code, _stream_ptr(h.device)),
                     "rglru_hip_gelu_gate_fwd")
@@ -229,7 +229,7 @@ class _HipGeluGate(torch.autograd.Function):
         dout_c = dout.to(h.dtype).contiguous()
         dh, dv = torch.empty_like(h), torch.empty_like(v)
         if h.numel():
-            with torch.cuda.device(h.device):
+            with _on_device(h.device):
                 _lib.check(_lib.load().rglru_hip_gelu_gate_bwd(
                     _ptr(dout_c), _ptr(h), _ptr(v), _ptr(dh), _ptr(dv), h.numel(), _dtype_code(h.dtype),
                     _stream_ptr(h.device)), "rglru_hip_gelu_gate_bwd")
@@ -265,7 +265,7 @@ def hip_block_decode_step(u: Tensor, v: Tensor, conv_state: Tensor | None, weigh
     bias_c = None if bias is None else _parameter_operand(bias.detach().to(taps.dtype), u.dtype)
     device = u.device
     lib = _lib.load()
-    with torch.cuda.device(device):
+    with _on_device(device):
         x_conv = torch.empty_like(u_c)
         new_conv = u.new_empty(batch, taps_count - 1, width)
         new_pos = torch.empty(batch, dtype=torch.int64, device=device)
@@ -297,7 +297,7 @@ class _HipRMSNorm(torch.autograd.Function):
         rows = x_c.numel() // width
         scale = _parameter_operand(g.detach(), x.dtype)
         lib = _lib.load()
-        with torch.cuda.device(x.device):
+        with _on_device(x.device):
             y = torch.empty_like(x_c)
             inv = torch.empty(rows, dtype=torch.float32, device=x.device)
             if rows:
@@ -316,7 +316,7 @@ class _HipRMSNorm(torch.autograd.Function):
         dy_c = dy.to(x.dtype).contiguous()
         lib = _lib.load()
         need_g = ctx.needs_input_grad[1]
-        with torch.cuda.device(x.device):
+        with _on_device(x.device):
             dx = torch.empty_like(x)
             dg = torch.empty(width, dtype=scale.dtype, device=x.device) if need_g else None
             if rows:

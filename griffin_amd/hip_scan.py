@@ -30,18 +30,51 @@ def hip_scan_available() -> bool:
     return _lib.available()
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_raw_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
 def _stream_ptr(device: torch.device) -> int:
+    """The current stream of ``device`` as a raw hipStream_t (the C ABI takes it as void*)."""
+    index = device.index
+    if _raw_stream is not None and index is not None:
+        return _raw_stream(index)                        # no Stream object: a fraction of a microsecond
     return torch.cuda.current_stream(device).cuda_stream
+
+
+class _NoSwitch:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def _on_device(device: torch.device):
+    """``torch.cuda.device(device)`` without the cost of the guard when ``device`` is current already
+    (the usual case; the guard costs several microseconds per call, as much as a decode step's kernel)."""
+    if _raw_device is not None and device.index is not None and _raw_device() == device.index:
+        return _NO_SWITCH
+    return torch.cuda.device(device)
 
 
 def _ptr(t: Tensor | None) -> int | None:
     return None if t is None else t.data_ptr()
 
 
+_gpu_seen = False
+
+
 def _require_gpu(name: str, *tensors: Tensor) -> None:
-    _lib.load()  # raises RuntimeError when the extension is missing
-    if not torch.cuda.is_available():
-        raise RuntimeError(f"{name} requires a CUDA/HIP device, none is available")
+    global _gpu_seen
+    if not _gpu_seen:
+        _lib.load()  # raises RuntimeError when the extension is missing
+        if not torch.cuda.is_available():
+            raise RuntimeError(f"{name} requires a CUDA/HIP device, none is available")
+        _gpu_seen = True                                 # both facts hold for the life of the process
     for t in tensors:
         if t is not None and not t.is_cuda:
             raise RuntimeError(f"{name} requires CUDA/HIP tensors, got a {t.device.type} tensor")
@@ -71,7 +104,7 @@ class _HipScan(torch.autograd.Function):
         if out.numel() == 0:
             ctx.save_for_backward(decay, initial_state, out)
             return out
-        with torch.cuda.device(decay.device):
+        with _on_device(decay.device):
             ws = torch.empty(lib.rglru_hip_scan_workspace_bytes(B, T, W), dtype=torch.uint8, device=decay.device)
             _lib.check(lib.rglru_hip_scan_fwd(decay.data_ptr(), current_input.data_ptr(), initial_state.data_ptr(),
                                               out.data_ptr(), ws.data_ptr(), B, T, W, _stream_ptr(decay.device)),
@@ -91,7 +124,7 @@ class _HipScan(torch.autograd.Function):
         d_state = torch.empty_like(initial_state)
         if decay.numel() == 0:
             return d_decay, d_input, d_state.zero_()
-        with torch.cuda.device(decay.device):
+        with _on_device(decay.device):
             ws = torch.empty(lib.rglru_hip_scan_workspace_bytes(B, T, W), dtype=torch.uint8, device=decay.device)
             _lib.check(lib.rglru_hip_scan_bwd(decay.data_ptr(), initial_state.data_ptr(), out.data_ptr(),
                                               grad_out.data_ptr(), d_decay.data_ptr(), d_input.data_ptr(),
@@ -162,7 +195,7 @@ class PreparedParams:
         size = _prep_bytes(self.width, nb, code)
         device = w_a.device
         operands, vec_code = _parameter_operands(w_a, b_a, w_x, b_x, lam, dtype)
-        with torch.cuda.device(device):
+        with _on_device(device):
             self.image = torch.empty(size, dtype=torch.uint8, device=device)
             _lib.check(lib.rglru_hip_prepare(*(t.data_ptr() for t in operands), self.c, self.width, nb, code, vec_code,
                                              self.image.data_ptr(), _stream_ptr(device)), "rglru_hip_prepare")
@@ -216,7 +249,7 @@ class _HipRGLRU(torch.autograd.Function):
         operands, vec_code = _parameter_operands(w_a, b_a, w_x, b_x, lam, x.dtype)
         h0c = None if h0 is None else h0.detach().to(torch.float32).contiguous()
         device = x.device
-        with torch.cuda.device(device):
+        with _on_device(device):
             y = torch.empty_like(x)
             h_last = torch.empty(B, W, dtype=torch.float32, device=device)
             image = torch.empty(_prep_bytes(W, nb, code), dtype=torch.uint8, device=device)
@@ -257,7 +290,7 @@ class _HipRGLRU(torch.autograd.Function):
         pd = ctx.param_dtypes
         gdt = pd[0] if (len(set(pd)) == 1 and pd[0] in _DTYPE_CODES) else torch.float32
         gcode = _DTYPE_CODES[gdt]
-        with torch.cuda.device(device):
+        with _on_device(device):
             dx = torch.empty_like(x)
             db_a = torch.empty(nb, bw, dtype=gdt, device=device)
             db_x = torch.empty(nb, bw, dtype=gdt, device=device)
@@ -343,7 +376,7 @@ def hip_rglru_step(x: Tensor, prep: PreparedParams, state: Tensor, flags: Tensor
         raise TypeError(f"parameters were prepared for {prep.dtype}, got activations in {x.dtype}")
     lib = _lib.load()
     x = x.contiguous()
-    with torch.cuda.device(x.device):
+    with _on_device(x.device):
         y = torch.empty_like(x)
         _lib.check(lib.rglru_hip_step(x.data_ptr(), prep.image.data_ptr(), state.data_ptr(), _ptr(flags),
                                       y.data_ptr(), x.shape[0], prep.width, prep.blocks, _dtype_code(x.dtype),
@@ -367,7 +400,7 @@ def hip_rglru_steps(xs: Tensor, prep: PreparedParams, state: Tensor, flags: Tens
     lib = _lib.load()
     xs = xs.contiguous()
     K, B, _ = xs.shape
-    with torch.cuda.device(xs.device):
+    with _on_device(xs.device):
         ys = torch.empty_like(xs)
         if K > 0 and B > 0:
             _lib.check(lib.rglru_hip_steps(xs.data_ptr(), prep.image.data_ptr(), state.data_ptr(),
