@@ -93,9 +93,29 @@ def secondary_workload(args):
         x = torch.randn(B, T, D, device=dev, dtype=dt, requires_grad=True)
         dy = torch.randn(B, T, D, device=dev, dtype=dt)
         leaves = [x] + list(block.parameters()) + list(norm.parameters())
-        ms = _timed(lambda: torch.autograd.grad(block(norm(x)), leaves, dy), args.steps, args.warmup)
+        one = lambda: torch.autograd.grad(block(norm(x)), leaves, dy)
+        ms_eager = _timed(one, args.steps, args.warmup)
+        # the same step as a HIP graph (what a training loop that captures its step pays: no host time)
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            one()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        per_graph = 5
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            kept = [one() for _ in range(per_graph)]
+        eager_out = [t.clone() for t in one()]
+        graph.replay()
+        torch.cuda.synchronize()
+        worst = max(((g.float() - e.float()).abs().max() / e.float().abs().max().clamp_min(1e-30)).item()
+                    for g, e in zip(kept[-1], eager_out))
+        ms = _timed(graph.replay, max(args.steps // per_graph, 1), 2) / per_graph
+        block_extra = {"ms_per_step_eager": ms_eager, "ms_per_step_graph": ms, "graph_matches_eager": bool(worst < 2e-2),
+                       "graph_vs_eager_max_rel_err": worst}
         metric, tokens = "RMSNorm + RecurrentBlock fwd+bwd tokens/s", B * T
-        workload = f"RMSNorm + RecurrentBlock({D}, {W}) fwd+bwd B{B} T{T} bf16"
+        workload = f"RMSNorm + RecurrentBlock({D}, {W}) fwd+bwd B{B} T{T} bf16 (HIP graph of {per_graph} steps)"
     elif name == "scan_only":
         # the scan-only operator (contract of the reference's fused_rglru_scan: fp32 a, z, h0 -> h) at the
         # benchmark shape: forward reads a, z and writes h (12 N bytes), backward reads a, dh, h and writes
@@ -268,8 +288,9 @@ def secondary_workload(args):
     print(json.dumps({
         "metric": metric, "value": tokens / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic", "config": {"workload": workload, "launch": "hip graph" if name in ("decode", "block_decode") else "eager"},
+        "dtype": "bf16", "data": "synthetic", "config": {"workload": workload, "launch": "hip graph" if name in ("decode", "block_decode", "block") else "eager"},
         **({"decode": extra} if name in ("decode", "block_decode") else {}),
+        **({"block": block_extra} if name == "block" else {}),
     }))
 
 

@@ -14,7 +14,7 @@ RGLRU_BF16 = 1
 FLAG_RESET = 1
 FLAG_INACTIVE = 2
 CHUNK = 32
-ABI_VERSION = 13
+ABI_VERSION = 14
 
 _lock = threading.Lock()
 _lib = None
@@ -54,6 +54,8 @@ _SIGNATURES = {
     "rglru_hip_conv_padded_scratch_bytes": (ctypes.c_size_t, [_I, _I]),
     "rglru_hip_conv_padded_fwd": (ctypes.c_int, [_P] * 9 + [_I, _I, _I, _I, ctypes.c_int, ctypes.c_int, _P]),
     "rglru_hip_conv_padded_bwd": (ctypes.c_int, [_P] * 12 + [_I, _I, _I, _I, ctypes.c_int, ctypes.c_int, ctypes.c_int, _P]),
+    "rglru_hip_colsum_scratch_bytes": (ctypes.c_size_t, [_I, _I]),
+    "rglru_hip_colsum": (ctypes.c_int, [_P, _P, _P, _I, _I, ctypes.c_int, ctypes.c_int, _P]),
     "rglru_hip_gelu_gate_fwd": (ctypes.c_int, [_P, _P, _P, _I, ctypes.c_int, _P]),
     "rglru_hip_gelu_gate_bwd": (ctypes.c_int, [_P, _P, _P, _P, _P, _I, ctypes.c_int, _P]),
     "rglru_hip_rmsnorm_max_width": (ctypes.c_int, [ctypes.c_int, ctypes.c_int]),

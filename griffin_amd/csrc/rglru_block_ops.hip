@@ -991,6 +991,55 @@ __global__ __launch_bounds__(256) void rmsnorm_finish_kernel(NormFinishArgs p) {
   }
 }
 
+// Column sums of a [rows, D] matrix (the bias gradient of a Linear layer: db = sum over rows of dy).  A
+// workgroup owns 32 vectors of columns and a slot of rows; its 8 row lanes stride through the slot with all
+// their loads in flight, add up in LDS and leave one partial row per slot, which rmsnorm_finish_kernel
+// sums in fixed order.
+constexpr int kColsumVecs = 32, kColsumLanes = 8, kColsumRowsPerLane = 8;
+struct ColsumArgs { const void* x; float* partial; long long rows; int D, nvec, vec_groups; };
+template <typename IO, int V>
+__global__ __launch_bounds__(256) void colsum_kernel(ColsumArgs p) {
+  __shared__ float red[kColsumLanes][V][kColsumVecs + 1];
+  const int lv = threadIdx.x % kColsumVecs, rl = threadIdx.x / kColsumVecs;
+  const int vg = blockIdx.x % p.vec_groups;
+  const long long slot = blockIdx.x / p.vec_groups;
+  const int vec = vg * kColsumVecs + lv;
+  const long long row0 = slot * (kColsumLanes * kColsumRowsPerLane) + rl;
+  float acc[V];
+#pragma unroll
+  for (int v = 0; v < V; ++v) acc[v] = 0.f;
+  if (vec < p.nvec) {
+    const unsigned es = (unsigned)sizeof(IO);
+    // the slot's rows through one descriptor: rows past the end read as zero
+    const long long first = slot * (kColsumLanes * kColsumRowsPerLane);
+    const long long left = p.rows - first;
+    const unsigned rows_here = (unsigned)(left < kColsumLanes * kColsumRowsPerLane ? left : kColsumLanes * kColsumRowsPerLane);
+    const rsrc_t r = make_rsrc((const IO*)p.x + first * p.D, rows_here * (unsigned)p.D * es);
+    float row[kColsumRowsPerLane][V];
+#pragma unroll
+    for (int i = 0; i < kColsumRowsPerLane; ++i)
+      ConvRow<IO, V>::load(row[i], r, ((unsigned)(rl + kColsumLanes * i) * (unsigned)p.D + (unsigned)vec * V) * es);
+#pragma unroll
+    for (int i = 0; i < kColsumRowsPerLane; ++i)
+#pragma unroll
+      for (int v = 0; v < V; ++v) acc[v] += row[i][v];
+  }
+  (void)row0;
+#pragma unroll
+  for (int v = 0; v < V; ++v) red[rl][v][lv] = acc[v];
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < V * kColsumVecs; idx += 256) {
+    const int v = idx / kColsumVecs, l = idx - v * kColsumVecs;
+    const int c = (vg * kColsumVecs + l) * V + v;
+    if (c < p.D) {
+      float sum = 0.f;
+#pragma unroll
+      for (int q = 0; q < kColsumLanes; ++q) sum += red[q][v][l];
+      p.partial[slot * p.D + c] = sum;
+    }
+  }
+}
+
 template <typename IO, int V, bool BACKWARD>
 static void norm_launch(int nvec, dim3 grid, hipStream_t s, const NormArgs& a) {
   const int slots = (nvec + 63) / 64;
@@ -1258,6 +1307,46 @@ int rglru_hip_rmsnorm_bwd(const void* x, const void* g, const float* inv, const 
   f.partial = a.partial; f.dg = dg; f.D = (int)D; f.slots = blocks; f.grad_dtype = grad_dtype;
   hipLaunchKernelGGL(rmsnorm_finish_kernel, dim3((unsigned)((D + 31) / 32)), dim3(256), 0, s, f);
   return check_launch("rmsnorm_bwd finish");
+}
+
+static long long colsum_slots(int64_t rows) {
+  return (rows + kColsumLanes * kColsumRowsPerLane - 1) / (kColsumLanes * kColsumRowsPerLane);
+}
+
+size_t rglru_hip_colsum_scratch_bytes(int64_t rows, int64_t D) {
+  if (rows <= 0 || D <= 0) return 0;
+  return (size_t)colsum_slots(rows) * (size_t)D * 4;
+}
+
+int rglru_hip_colsum(const void* x, void* scratch, void* out, int64_t rows, int64_t D, int dtype, int out_dtype,
+                     void* stream) {
+  if (!x || !scratch || !out) return fail(RGLRU_E_ARG, "colsum: null pointer");
+  if (dtype != RGLRU_F32 && dtype != RGLRU_BF16) return fail(RGLRU_E_ARG, "colsum: dtype must be RGLRU_F32 or RGLRU_BF16, got %d", dtype);
+  if (out_dtype != RGLRU_F32 && out_dtype != RGLRU_BF16) return fail(RGLRU_E_ARG, "colsum: unknown output dtype %d", out_dtype);
+  if (rows <= 0 || D <= 0) return fail(RGLRU_E_ARG, "colsum: rows and D must be positive (got %lld, %lld)", (long long)rows, (long long)D);
+  const long long slots = colsum_slots(rows);
+  if (D >= (1 << 24) || slots >= (1ll << 24)) return fail(RGLRU_E_UNSUPPORTED, "colsum: matrix too large");
+  const bool vec = conv_vector_ok(D, dtype, {x});
+  const int V = vec ? (dtype == RGLRU_BF16 ? 8 : 4) : 1;
+  ColsumArgs a;
+  a.x = x; a.partial = (float*)scratch; a.rows = rows; a.D = (int)D; a.nvec = (int)((D + V - 1) / V);
+  a.vec_groups = (a.nvec + kColsumVecs - 1) / kColsumVecs;
+  if (slots * a.vec_groups >= (1ll << 31)) return fail(RGLRU_E_UNSUPPORTED, "colsum: matrix too large");
+  dim3 grid((unsigned)(slots * a.vec_groups));
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == RGLRU_BF16) {
+    if (vec) hipLaunchKernelGGL((colsum_kernel<__bf16, 8>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((colsum_kernel<__bf16, 1>), grid, dim3(256), 0, s, a);
+  } else {
+    if (vec) hipLaunchKernelGGL((colsum_kernel<float, 4>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((colsum_kernel<float, 1>), grid, dim3(256), 0, s, a);
+  }
+  int rc = check_launch("colsum");
+  if (rc) return rc;
+  NormFinishArgs f;
+  f.partial = a.partial; f.dg = out; f.D = (int)D; f.slots = (int)slots; f.grad_dtype = out_dtype;
+  hipLaunchKernelGGL(rmsnorm_finish_kernel, dim3((unsigned)((D + 31) / 32)), dim3(256), 0, s, f);
+  return check_launch("colsum finish");
 }
 
 }  // extern "C"

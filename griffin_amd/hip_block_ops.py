@@ -285,6 +285,49 @@ def hip_block_decode_step(u: Tensor, v: Tensor, conv_state: Tensor | None, weigh
     return out, h_out, new_conv, new_pos
 
 
+class _HipLinear(torch.autograd.Function):
+    """``F.linear`` whose bias gradient is summed by ``rglru_hip_colsum`` (the two GEMMs of the backward
+    pass stay with the BLAS library, as in ``nn.Linear``)."""
+
+    @staticmethod
+    def forward(ctx, x: Tensor, weight: Tensor, bias: Tensor | None) -> Tensor:
+        ctx.save_for_backward(x, weight)
+        ctx.bias_dtype = None if bias is None else bias.dtype
+        return torch.nn.functional.linear(x, weight, bias)
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, dy: Tensor):
+        x, weight = ctx.saved_tensors
+        need_x, need_w, need_b = ctx.needs_input_grad
+        dy2 = dy.reshape(-1, dy.size(-1))
+        dx = dw = db = None
+        if need_x:
+            dx = torch.matmul(dy, weight.to(dy.dtype))
+        if need_w:
+            dw = torch.mm(dy2.t(), x.reshape(-1, x.size(-1)).to(dy.dtype)).to(weight.dtype)
+        if need_b and ctx.bias_dtype is not None:
+            rows, width = dy2.shape
+            dy_c = dy2.contiguous()
+            out_dtype = ctx.bias_dtype if ctx.bias_dtype in _DTYPE_CODES else torch.float32
+            lib = _lib.load()
+            with _on_device(dy.device):
+                db = torch.empty(width, dtype=out_dtype, device=dy.device)
+                scratch = torch.empty(lib.rglru_hip_colsum_scratch_bytes(rows, width), dtype=torch.uint8, device=dy.device)
+                _lib.check(lib.rglru_hip_colsum(_ptr(dy_c), _ptr(scratch), _ptr(db), rows, width, _dtype_code(dy.dtype),
+                                                _DTYPE_CODES[out_dtype], _stream_ptr(dy.device)), "rglru_hip_colsum")
+            db = db.to(ctx.bias_dtype)
+        return dx, dw, db
+
+
+def hip_linear(x: Tensor, weight: Tensor, bias: Tensor | None) -> Tensor:
+    """``x @ weight.T + bias`` (griffin/griffin.py:379-389, the block's Linear layers) with the bias
+    gradient reduced by a kernel of this library; differentiable in all three arguments."""
+    _require_gpu("hip_linear", x, weight, bias)
+    _dtype_code(x.dtype)
+    return _HipLinear.apply(x, weight, bias)
+
+
 class _HipRMSNorm(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x: Tensor, g: Tensor, eps: float) -> Tensor:

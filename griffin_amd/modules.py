@@ -355,6 +355,16 @@ class RecurrentBlock(nn.Module):
             return output, RecurrentBlockCache(new_rnn_state, new_conv_state, new_pos)
         return output
 
+    def _linear(self, layer: nn.Linear, x: Tensor) -> Tensor:
+        """A Linear layer of the block; in training on the HIP path its bias gradient is summed by a
+        kernel of the library instead of a generic reduction (the GEMMs are the BLAS library's either way)."""
+        if (torch.is_grad_enabled() and layer.bias is not None and layer.bias.requires_grad
+                and x.is_cuda and x.dtype in hip_scan.SUPPORTED_DTYPES and layer.weight.dtype == x.dtype
+                and self.rg_lru.scan_mode in ("hip", "fused", "auto") and x.numel() > 0
+                and (self.rg_lru.scan_mode != "auto" or hip_scan.hip_scan_is_usable(x.device))):
+            return hip_block_ops.hip_linear(x, layer.weight, layer.bias)
+        return layer(x)
+
     def _dense_conv(self, projected: Tensor, conv_state: Tensor, segment_pos: Tensor):
         """All-tokens-active path (griffin/griffin.py:476-487): taps are masked per document."""
         if self._hip_block_ops_covers(projected):
@@ -404,8 +414,8 @@ class RecurrentBlock(nn.Module):
         segment_pos = _resolve_segment_positions(
             x, segment_pos, previous_position, None if everything_active else active_mask)
 
-        gate_input = self.linear_y(x)
-        projected = self.linear_x(x)
+        gate_input = self._linear(self.linear_y, x)
+        projected = self._linear(self.linear_x, x)
         conv_state = self._empty_conv_state(projected) if cache is None else cache.conv_state
         if conv_state.shape != (batch, self.conv_kernel_size - 1, self.rnn_width):
             raise ValueError("Recurrent convolution cache has an incompatible shape")
@@ -425,7 +435,7 @@ class RecurrentBlock(nn.Module):
             gated = hip_block_ops.hip_gelu_gate(recurrent_out, gate_input)
         else:
             gated = recurrent_out * F.gelu(gate_input, approximate="tanh")
-        output = self.linear_out(gated)
+        output = self._linear(self.linear_out, gated)
         if not everything_active:
             output = output.masked_fill(~active_mask.unsqueeze(-1), 0.0)
         if return_cache:

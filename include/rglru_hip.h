@@ -20,6 +20,7 @@
  *   griffin/griffin.py:464, :520    x_branch * gelu_tanh(linear_y(x))        rglru_hip_gelu_gate_fwd, _bwd
  *   griffin/griffin.py:68-80        RMSNorm in front of the block and its autograd   rglru_hip_rmsnorm_fwd, _bwd
  *   griffin/griffin.py:459-528 with T == 1 (block decode: positions, conv, step, gate)   rglru_hip_decode_prepare + rglru_hip_step_gated
+ *   autograd of the bias of griffin/griffin.py:379-389 (the block's Linear layers)      rglru_hip_colsum
  *
  * Conventions
  *   - every pointer is a DEVICE pointer owned by the caller; tensors are row-major with the
@@ -48,7 +49,7 @@
 extern "C" {
 #endif
 
-#define RGLRU_ABI_VERSION 13
+#define RGLRU_ABI_VERSION 14
 
 enum { RGLRU_F32 = 0, RGLRU_BF16 = 1 };
 
@@ -281,6 +282,14 @@ size_t rglru_hip_rmsnorm_scratch_bytes(int64_t rows, int64_t D);
 int rglru_hip_rmsnorm_bwd(const void* x, const void* g, const float* inv, const void* dy, void* scratch,
                           void* dx, void* dg, int64_t rows, int64_t D, int dtype, int vec_dtype, int grad_dtype,
                           void* stream);
+
+/* Column sums of x[rows, D] (dtype) into out[D] (out_dtype), fp32 accumulation in a fixed order: the
+ * bias gradient of the block's three Linear layers (griffin/griffin.py:379-389; autograd of
+ * `nn.Linear`: db = sum over tokens of dy), which the caller's BLAS library leaves to a generic reduction.
+ * `scratch` holds rglru_hip_colsum_scratch_bytes(rows, D) bytes. */
+size_t rglru_hip_colsum_scratch_bytes(int64_t rows, int64_t D);
+int rglru_hip_colsum(const void* x, void* scratch, void* out, int64_t rows, int64_t D, int dtype, int out_dtype,
+                     void* stream);
 
 /* Single-token step of the recurrent block (griffin/griffin.py:459-528 with one token per row) in
  * two launches around the caller's three Linear layers:

@@ -363,3 +363,35 @@ def test_rmsnorm_module_and_properties_at_training_shape():
     with pytest.raises(ValueError):
         from griffin_amd.hip_block_ops import hip_rmsnorm
         hip_rmsnorm(x, torch.zeros(5, device="cuda", dtype=torch.bfloat16))
+
+
+# ----------------------------------------------------------------------------------------------
+# bias gradient of the block's Linear layers (C ABI: rglru_hip_colsum)
+# ----------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(2, 50, 64, 96), (3, 7, 13, 5), (1, 1, 768, 1024), (8, 2048, 768, 1024), (2, 129, 24, 1030)])
+def test_hip_linear_matches_torch_linear(shape, dtype):
+    """Output and all three gradients of hip_linear against torch.nn.functional.linear in fp64 on the same
+    (rounded) operands; the bias gradient is the column sum the library computes."""
+    from griffin_amd.hip_block_ops import hip_linear
+
+    B, T, D, W = shape
+    _say("linear case", shape, dtype)
+    gen = torch.Generator().manual_seed(33)
+    x = torch.randn(B, T, D, generator=gen).to(dtype)
+    w = (torch.randn(W, D, generator=gen) / D ** 0.5).to(dtype)
+    b = (torch.randn(W, generator=gen) * 0.1).to(dtype)
+    dy = torch.randn(B, T, W, generator=gen).to(dtype)
+    ref = [t.double().requires_grad_(True) for t in (x, w, b)]
+    torch.nn.functional.linear(*ref).backward(dy.double())
+    dev = [t.cuda().requires_grad_(True) for t in (x, w, b)]
+    out = hip_linear(*dev)
+    out.backward(dy.cuda())
+    torch.cuda.synchronize()
+    tol = 2e-5 if dtype == torch.float32 else BF16_TOL
+    want = torch.nn.functional.linear(x.double(), w.double(), b.double())
+    assert rel_err(out.double().cpu(), want) < tol
+    for name, r, d in zip(("x", "weight", "bias"), ref, dev):
+        err = rel_err(d.grad.double().cpu(), r.grad)
+        _say("  d%s rel error: %.2e" % (name, err))
+        assert err < tol, name
