@@ -305,7 +305,20 @@ class _HipLinear(torch.autograd.Function):
         if need_x:
             dx = torch.matmul(dy, weight.to(dy.dtype))
         if need_w:
-            dw = torch.mm(dy2.t(), x.reshape(-1, x.size(-1)).to(dy.dtype)).to(weight.dtype)
+            x2 = x.reshape(-1, x.size(-1)).to(dy.dtype)
+            rows = dy2.size(0)
+            # dW = dy^T x contracts over all tokens: one GEMM with K = rows runs at a fraction of the rate of
+            # the same work as a batch of GEMMs with K = 2048 whose results are added (100 us against 43 us
+            # for 16384 x 1024 x 768 in bf16 on this library), so long contractions are split
+            chunks = rows // 2048 if (rows % 2048 == 0 and dy2.is_contiguous() and x2.is_contiguous()) else 1
+            while chunks > 16 and chunks % 2 == 0:
+                chunks //= 2
+            if chunks > 1:
+                per = rows // chunks
+                dw = torch.bmm(dy2.view(chunks, per, -1).transpose(1, 2), x2.view(chunks, per, -1)).sum(0)
+            else:
+                dw = torch.mm(dy2.t(), x2)
+            dw = dw.to(weight.dtype)
         if need_b and ctx.bias_dtype is not None:
             rows, width = dy2.shape
             dy_c = dy2.contiguous()
