@@ -101,15 +101,18 @@ class _HipCausalConv(torch.autograd.Function):
 
 
 def hip_causal_conv(u: Tensor, state: Tensor | None, weight: Tensor, bias: Tensor | None,
-                    segment_pos: Tensor) -> tuple[Tensor, Tensor]:
+                    segment_pos: Tensor, need_state: bool = True) -> tuple[Tensor, Tensor | None]:
     """Depthwise causal convolution with per-document tap masking.
 
     ``u`` [B, T, W]; ``state`` [B, K-1, W] or None (zeros); ``weight`` [W, 1, K] and ``bias`` [W] of a
     depthwise ``nn.Conv1d``; ``segment_pos`` [B, T] integer positions (a tap reaching back ``lag`` tokens
     contributes only where ``segment_pos >= lag``).  Returns ``(out [B, T, W], new_state [B, K-1, W])``;
-    ``new_state`` is the last K-1 rows of ``cat(state, u)`` (griffin/griffin.py:487).
+    ``new_state`` is the last K-1 rows of ``cat(state, u)`` (griffin/griffin.py:487), or None when the
+    caller says it does not need it (a training step that returns no cache).
     """
     out = _HipCausalConv.apply(u, state, weight, bias, segment_pos)
+    if not need_state:
+        return out, None
     history = weight.size(2) - 1
     steps = u.size(1)
     if steps >= history:

@@ -10,6 +10,8 @@ There is no CPU fallback in this file: every operator raises when the library or
 
 from __future__ import annotations
 
+import weakref
+
 import threading
 import warnings
 
@@ -152,8 +154,22 @@ def _dtype_code(dtype: torch.dtype) -> int:
     raise TypeError(f"hip RG-LRU supports float32 and bfloat16 activations, got {dtype}")
 
 
+_PACKED_FLAGS: dict = {}       # id(mask) -> (weak reference to the mask, its version, the packed bytes)
+
+
 def pack_flags(reset_mask: Tensor | None, active_mask: Tensor | None) -> Tensor | None:
-    """One byte per token: bit 0 = reset, bit 1 = inactive.  None when no token is flagged."""
+    """One byte per token: bit 0 = reset, bit 1 = inactive.  None when no token is flagged.  The bytes
+    of a reset mask that comes without an activity mask are remembered for as long as that tensor lives
+    and is not written to (a module that passes the same mask every step pays for them once)."""
+    if reset_mask is not None and active_mask is None and reset_mask.dtype == torch.bool:
+        hit = _PACKED_FLAGS.get(id(reset_mask))
+        if hit is not None and hit[0]() is reset_mask and hit[1] == reset_mask._version:
+            return hit[2]
+        flags = reset_mask.to(torch.uint8).contiguous()
+        if len(_PACKED_FLAGS) >= 64:
+            _PACKED_FLAGS.clear()
+        _PACKED_FLAGS[id(reset_mask)] = (weakref.ref(reset_mask), reset_mask._version, flags)
+        return flags
     flags = None
     if reset_mask is not None:
         flags = reset_mask.to(torch.uint8)

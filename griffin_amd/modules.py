@@ -195,11 +195,32 @@ class RG_LRU(nn.Module):
     _associative_scan = staticmethod(portable.associative_scan)
 
 
+# Positions 0 .. T-1 for every row and their "document starts here" mask: what a call without cache,
+# explicit positions or padding resolves to.  They depend only on (batch, steps, device), so they are
+# built once (a training step would otherwise spend six small launches per block on them) and must
+# not be modified in place by anyone.
+_DEFAULT_POSITIONS: dict = {}
+
+
+def _default_positions(batch: int, steps: int, device: torch.device):
+    key = (batch, steps, device)
+    hit = _DEFAULT_POSITIONS.get(key)
+    if hit is None:
+        if len(_DEFAULT_POSITIONS) >= 16:
+            _DEFAULT_POSITIONS.clear()
+        pos = torch.arange(steps, device=device, dtype=torch.long).expand(batch, steps).contiguous()
+        hit = (pos, pos == 0)
+        _DEFAULT_POSITIONS[key] = hit
+    return hit
+
+
 def _resolve_segment_positions(x, segment_pos, previous_position=None, active_mask=None) -> Tensor:
     """Explicit positions, or previous + running count of active tokens (griffin/griffin.py:309-338)."""
     batch, steps = x.shape[:2]
     if steps == 0:
         raise ValueError("Empty token sequences are not supported")
+    if segment_pos is None and previous_position is None and active_mask is None:
+        return _default_positions(batch, steps, x.device)[0]
     if segment_pos is not None:
         if segment_pos.shape != (batch, steps):
             raise ValueError(f"segment_pos must have shape ({batch}, {steps}), got {tuple(segment_pos.shape)}")
@@ -365,11 +386,11 @@ class RecurrentBlock(nn.Module):
             return hip_block_ops.hip_linear(x, layer.weight, layer.bias)
         return layer(x)
 
-    def _dense_conv(self, projected: Tensor, conv_state: Tensor, segment_pos: Tensor):
+    def _dense_conv(self, projected: Tensor, conv_state: Tensor | None, segment_pos: Tensor, need_state: bool = True):
         """All-tokens-active path (griffin/griffin.py:476-487): taps are masked per document."""
         if self._hip_block_ops_covers(projected):
             return hip_block_ops.hip_causal_conv(projected, conv_state, self.temporal_conv.weight,
-                                            self.temporal_conv.bias, segment_pos)
+                                                 self.temporal_conv.bias, segment_pos, need_state)
         return portable.causal_depthwise_conv(projected, conv_state, self.temporal_conv.weight,
                                               self.temporal_conv.bias, segment_pos)
 
@@ -409,25 +430,26 @@ class RecurrentBlock(nn.Module):
         previous_position = None if cache is None else cache.segment_position
         if steps == 1 and self._hip_decode_covers(x, cache):
             return self._hip_decode(x, cache, segment_pos, active_mask, return_cache)
-        if everything_active:
-            active_mask = torch.ones(batch, steps, device=x.device, dtype=torch.bool)
         segment_pos = _resolve_segment_positions(
             x, segment_pos, previous_position, None if everything_active else active_mask)
 
         gate_input = self._linear(self.linear_y, x)
         projected = self._linear(self.linear_x, x)
-        conv_state = self._empty_conv_state(projected) if cache is None else cache.conv_state
-        if conv_state.shape != (batch, self.conv_kernel_size - 1, self.rnn_width):
+        on_hip = self._hip_block_ops_covers(projected)
+        # the HIP convolution takes "no carried state" as such; the portable path wants the zeros
+        conv_state = (None if on_hip else self._empty_conv_state(projected)) if cache is None else cache.conv_state
+        if conv_state is not None and conv_state.shape != (batch, self.conv_kernel_size - 1, self.rnn_width):
             raise ValueError("Recurrent convolution cache has an incompatible shape")
         if everything_active or bool(active_mask.all()):
-            recurrent_in, new_conv_state = self._dense_conv(projected, conv_state, segment_pos)
+            recurrent_in, new_conv_state = self._dense_conv(projected, conv_state, segment_pos, return_cache)
         else:
             recurrent_in, new_conv_state = self._padded_conv(projected, conv_state, segment_pos, active_mask)
 
+        default = _DEFAULT_POSITIONS.get((batch, steps, x.device))
         recurrent_out, new_rnn_state = self.rg_lru(
             recurrent_in,
             None if cache is None else cache.rnn_state,
-            reset_mask=segment_pos == 0,
+            reset_mask=default[1] if (default is not None and segment_pos is default[0]) else segment_pos == 0,
             active_mask=None if everything_active else active_mask,
             return_state=True,
         )
@@ -439,6 +461,9 @@ class RecurrentBlock(nn.Module):
         if not everything_active:
             output = output.masked_fill(~active_mask.unsqueeze(-1), 0.0)
         if return_cache:
-            return output, RecurrentBlockCache(
-                new_rnn_state, new_conv_state, _last_active_position(segment_pos, active_mask, previous_position))
+            if everything_active:
+                last_position = segment_pos[:, -1].clone()   # every token is active: the last one's position
+            else:
+                last_position = _last_active_position(segment_pos, active_mask, previous_position)
+            return output, RecurrentBlockCache(new_rnn_state, new_conv_state, last_position)
         return output
