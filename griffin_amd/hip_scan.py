@@ -166,9 +166,10 @@ def pack_flags(reset_mask: Tensor | None, active_mask: Tensor | None) -> Tensor 
         if hit is not None and hit[0]() is reset_mask and hit[1] == reset_mask._version:
             return hit[2]
         flags = reset_mask.to(torch.uint8).contiguous()
-        if len(_PACKED_FLAGS) >= 64:
-            _PACKED_FLAGS.clear()
-        _PACKED_FLAGS[id(reset_mask)] = (weakref.ref(reset_mask), reset_mask._version, flags)
+        if not (reset_mask.is_cuda and torch.cuda.is_current_stream_capturing()):   # made under capture: valid inside that graph only
+            if len(_PACKED_FLAGS) >= 64:
+                _PACKED_FLAGS.clear()
+            _PACKED_FLAGS[id(reset_mask)] = (weakref.ref(reset_mask), reset_mask._version, flags)
         return flags
     flags = None
     if reset_mask is not None:

@@ -206,11 +206,14 @@ def _default_positions(batch: int, steps: int, device: torch.device):
     key = (batch, steps, device)
     hit = _DEFAULT_POSITIONS.get(key)
     if hit is None:
-        if len(_DEFAULT_POSITIONS) >= 16:
-            _DEFAULT_POSITIONS.clear()
         pos = torch.arange(steps, device=device, dtype=torch.long).expand(batch, steps).contiguous()
         hit = (pos, pos == 0)
-        _DEFAULT_POSITIONS[key] = hit
+        # tensors made while a graph is being captured live in that graph's memory and hold nothing until
+        # it is replayed: they are used for this call only
+        if not (device.type == "cuda" and torch.cuda.is_current_stream_capturing()):
+            if len(_DEFAULT_POSITIONS) >= 16:
+                _DEFAULT_POSITIONS.clear()
+            _DEFAULT_POSITIONS[key] = hit
     return hit
 
 

@@ -239,3 +239,32 @@ def test_portable_module_agrees_with_oracle():
     ry, rh = orc.rglru_forward(*[case[k] for k in ("x", "w_a", "b_a", "w_x", "b_x", "lam")], h0=case["h0"])
     torch.testing.assert_close(y, ry, atol=1e-6, rtol=1e-6)
     torch.testing.assert_close(h, rh, atol=1e-6, rtol=1e-6)
+
+
+def test_default_positions_are_built_once_and_match_the_general_rule():
+    """A call without cache, explicit positions or padding resolves to positions 0 .. T-1; the tensors are
+    shared between calls (griffin/griffin.py:309-338 for previous position -1 and every token active)."""
+    from griffin_amd import modules
+
+    x = torch.zeros(3, 7, 4)
+    first = modules._resolve_segment_positions(x, None)
+    again = modules._resolve_segment_positions(x, None)
+    assert first is again
+    general = modules._resolve_segment_positions(x, None, torch.full((3,), -1), None)
+    assert torch.equal(first, general)
+    assert torch.equal(modules._default_positions(3, 7, x.device)[1], general == 0)
+
+
+def test_packed_flags_follow_in_place_updates_of_the_mask():
+    """pack_flags remembers the bytes of a reset mask only while the mask is not written to."""
+    from griffin_amd.hip_scan import pack_flags
+
+    mask = torch.zeros(2, 5, dtype=torch.bool)
+    mask[0, 0] = True
+    a = pack_flags(mask, None)
+    assert pack_flags(mask, None) is a and a.tolist() == [[1, 0, 0, 0, 0], [0, 0, 0, 0, 0]]
+    mask[1, 3] = True                                        # bumps the tensor's version counter
+    b = pack_flags(mask, None)
+    assert b is not a and b.tolist() == [[1, 0, 0, 0, 0], [0, 0, 0, 1, 0]]
+    both = pack_flags(mask, torch.ones(2, 5, dtype=torch.bool))
+    assert both.tolist() == b.tolist()
