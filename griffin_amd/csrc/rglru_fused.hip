@@ -2040,7 +2040,7 @@ __global__ __launch_bounds__(kThreads) void step_kernel(FusedArgs p) {
   }
 }
 
-// Decode step for 16-bit storage and gate blocks of 32, 64 or 128 channels, on 16 x 16 MFMA tiles: a wave
+// Decode step for 16-bit storage and gate blocks of 32 to 384 channels in steps of 32, on 16 x 16 MFMA tiles: a wave
 // owns 16 sequences x 16 channels, a lane 4 sequences of one channel.  The step is a chain of latencies
 // (launch, loads, products, gate math, stores), so the work is cut as fine as the matrix unit allows:
 // four elements of gate math per lane instead of sixteen, 8 KB of weights per wave instead of 16, x rows
@@ -2337,6 +2337,13 @@ static int held_groups(const Geometry& g, int dtype, int aligned) {
     if (g.bwp == 32) return 2;
   }
   return 0;
+}
+
+// K steps of 32 channels of the decode kernels on 16 x 16 tiles (gate blocks of 32 .. 384 channels in steps
+// of 32, 16-bit storage, aligned rows), or 0 for the portable decode kernels
+static int step16_groups(const Geometry& g, int dtype, int aligned) {
+  if (dtype != RGLRU_BF16 || !aligned || g.bw != g.bwp || g.bw > 384) return 0;
+  return (int)(g.bw / 32);
 }
 
 // ... and for the blocks wider than a workgroup's four slabs whose weights the forward and the
@@ -2916,16 +2923,20 @@ static int step_impl(const void* x, const void* prep, const float* h_in, float* 
   long long row_tiles = (B + 31) / 32;
   dim3 grid((unsigned)(row_tiles * g.units));
   hipStream_t s = (hipStream_t)stream;
-  const int nkg = held_groups(g, dtype, a.aligned);
+  const int nks = step16_groups(g, dtype, a.aligned);
   {
     KernelTimer timer(2, s);
-    if (nkg > 0) {
+    if (nks > 0) {
       // 16 sequences x 16 channels per wave, four waves per workgroup
       const long long waves = ((B + 15) / 16) * (W / 16);
       dim3 grid16((unsigned)((waves + kWaves - 1) / kWaves));
-      if (nkg == 8) hipLaunchKernelGGL((step16_kernel<4>), grid16, dim3(kThreads), 0, s, a);
-      else if (nkg == 4) hipLaunchKernelGGL((step16_kernel<2>), grid16, dim3(kThreads), 0, s, a);
-      else hipLaunchKernelGGL((step16_kernel<1>), grid16, dim3(kThreads), 0, s, a);
+      switch (nks) {
+#define RGLRU_STEP16_CASE(N) case N: hipLaunchKernelGGL((step16_kernel<N>), grid16, dim3(kThreads), 0, s, a); break
+        RGLRU_STEP16_CASE(1); RGLRU_STEP16_CASE(2); RGLRU_STEP16_CASE(3); RGLRU_STEP16_CASE(4); RGLRU_STEP16_CASE(5);
+        RGLRU_STEP16_CASE(6); RGLRU_STEP16_CASE(7); RGLRU_STEP16_CASE(8); RGLRU_STEP16_CASE(9); RGLRU_STEP16_CASE(10);
+        RGLRU_STEP16_CASE(11); default: RGLRU_STEP16_CASE(12);
+#undef RGLRU_STEP16_CASE
+      }
     } else {
       RGLRU_DISPATCH(step_kernel, grid, s, a, dtype, 0);
     }
@@ -2960,15 +2971,19 @@ int rglru_hip_steps(const void* x, const void* prep, float* h, const uint8_t* fl
   long long row_tiles = (B + 31) / 32;
   dim3 grid((unsigned)(row_tiles * g.units));
   hipStream_t s = (hipStream_t)stream;
-  const int nkg = held_groups(g, dtype, a.aligned);
+  const int nks = step16_groups(g, dtype, a.aligned);
   {
     KernelTimer timer(2, s);
-    if (nkg > 0) {
+    if (nks > 0) {
       const long long waves = ((B + 15) / 16) * (W / 16);
       dim3 grid16((unsigned)((waves + kWaves - 1) / kWaves));
-      if (nkg == 8) hipLaunchKernelGGL((steps16_kernel<4>), grid16, dim3(kThreads), 0, s, a);
-      else if (nkg == 4) hipLaunchKernelGGL((steps16_kernel<2>), grid16, dim3(kThreads), 0, s, a);
-      else hipLaunchKernelGGL((steps16_kernel<1>), grid16, dim3(kThreads), 0, s, a);
+      switch (nks) {
+#define RGLRU_STEPS16_CASE(N) case N: hipLaunchKernelGGL((steps16_kernel<N>), grid16, dim3(kThreads), 0, s, a); break
+        RGLRU_STEPS16_CASE(1); RGLRU_STEPS16_CASE(2); RGLRU_STEPS16_CASE(3); RGLRU_STEPS16_CASE(4); RGLRU_STEPS16_CASE(5);
+        RGLRU_STEPS16_CASE(6); RGLRU_STEPS16_CASE(7); RGLRU_STEPS16_CASE(8); RGLRU_STEPS16_CASE(9); RGLRU_STEPS16_CASE(10);
+        RGLRU_STEPS16_CASE(11); default: RGLRU_STEPS16_CASE(12);
+#undef RGLRU_STEPS16_CASE
+      }
     } else {
       RGLRU_DISPATCH(steps_kernel, grid, s, a, dtype, 0);
     }

@@ -321,7 +321,10 @@ def test_step_kernel_matches_oracle(dtype, tol):
 
 
 @pytest.mark.parametrize("dtype,tol,shape", [(torch.float32, FP32_TOL, (5, 96, 3, 6)), (torch.bfloat16, BF16_TOL, (5, 96, 3, 6)),
-                                             (torch.bfloat16, BF16_TOL, (70, 256, 2, 33)), (torch.bfloat16, BF16_TOL, (3, 128, 2, 5))])
+                                             (torch.bfloat16, BF16_TOL, (70, 256, 2, 33)), (torch.bfloat16, BF16_TOL, (3, 128, 2, 5)),
+                                             (torch.bfloat16, BF16_TOL, (20, 640, 2, 4)), (torch.bfloat16, BF16_TOL, (3, 768, 2, 3)),
+                                             (torch.bfloat16, BF16_TOL, (17, 96, 1, 3)), (torch.bfloat16, BF16_TOL, (4, 480, 3, 3)),
+                                             (torch.bfloat16, BF16_TOL, (2, 896, 2, 3))])
 def test_multi_step_kernel_matches_oracle_and_single_steps(dtype, tol, shape):
     """K steps in one launch (rglru_hip_steps): against the oracle's sequence run, and against K calls of
     the single-step kernel (same arithmetic step by step: equal up to nothing but the order of
