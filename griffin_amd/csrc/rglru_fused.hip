@@ -154,6 +154,7 @@ struct FusedArgs {
   int bpu;                                                // gate blocks per unit (packed narrow blocks), else 1
   long long rows_total;                                   // B * T, the row count of one block of `pre`
   int nC, nCf, ckpt_nC, wg_per_unit, aligned, full_slabs, queues, flags_vec;
+  int dw_bf16;                                            // fast backward: per-workgroup weight-gradient sums stored as bf16
   long long limit;
 };
 
@@ -1646,13 +1647,16 @@ __global__ __launch_bounds__(kGradThreads, 1) void bwd_grad_kernel(FusedArgs p) 
       // per-workgroup partial of the weight gradients: [wg][k][gate][j][o]
 #pragma unroll
       for (int g = 0; g < 2; ++g) {
-        float* part = p.dw_partial + ((((long long)wg_in_unit * p.nb + k) * 2 + g) * p.bwp) * p.bwp;
+        const long long first = ((((long long)wg_in_unit * p.nb + k) * 2 + g) * p.bwp) * p.bwp;
+        float* part = p.dw_partial + first;
+        __bf16* part16 = (__bf16*)p.dw_partial + first;
 #pragma unroll
         for (int js = 0; js < S; ++js)
 #pragma unroll
           for (int v = 0; v < 16; ++v) {
             const int j = js * 32 + 8 * (v >> 2) + 4 * hf + (v & 3);
-            part[(long long)j * p.bwp + sl * 32 + r] = dw[g][js][v];
+            if (p.dw_bf16) part16[(long long)j * p.bwp + sl * 32 + r] = (__bf16)dw[g][js][v];
+            else part[(long long)j * p.bwp + sl * 32 + r] = dw[g][js][v];
           }
       }
     }
@@ -1882,7 +1886,7 @@ __global__ __launch_bounds__(kGradThreads, 1) void gate_grad_wide_kernel(FusedAr
 struct FinishArgs {
   const float* partial; const float* dsp; void* db_a; void* db_x; void* dlambda;
   const float* dw_partial; void* dw_a; void* dw_x;
-  int W, nb, bw, bwp, Wp, wg_per_unit, n_wg, vec_blocks, grad_dtype;
+  int W, nb, bw, bwp, Wp, wg_per_unit, n_wg, vec_blocks, grad_dtype, dw_bf16;
   uint4* clean; long long clean_n;                         // backward records and tickets, zeroed for the next pass
 };
 
@@ -1908,6 +1912,24 @@ __global__ __launch_bounds__(256) void finish_kernel(FinishArgs p) {
     // fixed summation order; eight loads in flight per thread
     float4 s0 = make_float4(0.f, 0.f, 0.f, 0.f), s1 = s0;
     int g = 0;
+    if (p.dw_bf16) {
+      typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+      const __bf16* src16 = (const __bf16*)p.dw_partial + i;
+      for (; g + 7 < p.n_wg; g += 8) {
+        bf16x4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const bf16x4*>(src16 + (long long)(g + u) * stride);
+#pragma unroll
+        for (int u = 0; u < 8; u += 2) {
+          s0.x += (float)v[u][0]; s0.y += (float)v[u][1]; s0.z += (float)v[u][2]; s0.w += (float)v[u][3];
+          s1.x += (float)v[u + 1][0]; s1.y += (float)v[u + 1][1]; s1.z += (float)v[u + 1][2]; s1.w += (float)v[u + 1][3];
+        }
+      }
+      for (; g < p.n_wg; ++g) {
+        const bf16x4 v = *reinterpret_cast<const bf16x4*>(src16 + (long long)g * stride);
+        s0.x += (float)v[0]; s0.y += (float)v[1]; s0.z += (float)v[2]; s0.w += (float)v[3];
+      }
+    }
     for (; g + 7 < p.n_wg; g += 8) {
       float4 v[8];
 #pragma unroll
@@ -2767,6 +2789,12 @@ int rglru_hip_bwd_full(const void* x, const void* y, const void* prep, const flo
   a.aligned = 1;
   const int nkg = held_groups(g, dtype, 1);
   pack_units(a, g, nkg);
+#ifndef RGLRU_DW_BF16
+#define RGLRU_DW_BF16 1
+#endif
+  // 16-bit weight gradients asked for: the per-workgroup sums (fp32 in registers over a workgroup's share of
+  // the tokens) cross memory as bf16 too, which halves what the finish kernel reads back
+  a.dw_bf16 = (RGLRU_DW_BF16 && grad_dtype == RGLRU_BF16) ? 1 : 0;
   // reverse scan: delta[B, T, W] (and dh0)
   const long long chunks = (T + 32 * kDeltaMT - 1) / (32 * kDeltaMT);
   a.wg_per_unit = pick_wg_per_unit(a.units, B * chunks, kDeltaMT == 1 ? 4 : RGLRU_DELTA_OCC, L.max_wg);
@@ -2804,7 +2832,7 @@ int rglru_hip_bwd_full(const void* x, const void* y, const void* prep, const flo
   r.partial = a.partial; r.dsp = finish_dsp(g, prep, dtype); r.db_a = db_a; r.db_x = db_x; r.dlambda = dlambda;
   r.dw_partial = a.dw_partial; r.dw_a = dw_a; r.dw_x = dw_x;
   r.W = (int)W; r.nb = (int)nb; r.bw = (int)g.bw; r.bwp = (int)g.bwp; r.Wp = (int)g.Wp; r.wg_per_unit = n_wg;
-  r.n_wg = n_wg; r.vec_blocks = (int)((W + 15) / 16); r.grad_dtype = grad_dtype;
+  r.n_wg = n_wg; r.vec_blocks = (int)((W + 15) / 16); r.grad_dtype = grad_dtype; r.dw_bf16 = a.dw_bf16;
   r.clean = (uint4*)(wb + L.b_begin); r.clean_n = (long long)((L.b_end - L.b_begin) / 16);
   const long long total = nb * g.bw * 2 * g.bw;
   hipLaunchKernelGGL(finish_kernel, dim3((unsigned)(r.vec_blocks + (total / 4 + 255) / 256)), dim3(256), 0, s, r);

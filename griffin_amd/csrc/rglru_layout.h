@@ -100,8 +100,9 @@ inline WorkLayout make_work_layout(int64_t B, int64_t T, const Geometry& g) {
 //   delta       fast backward (blocks of 32, 64, 128 channels): [B][T][W] 16-bit, dL/dh_t after the
 //               reverse scan; wide backward (blocks of 160 .. 384 channels): [B][T][nb][2 bw] 16-bit,
 //               the gradients at the gate pre-activations as pairs (element 2 o + gate)
-//   dw_partial  [sets][nb][2][bwp][bwp] fp32 per-workgroup weight-gradient sums, sets = kGemmWgPerUnit
-//               (fast) or kWideWgPerUnit (wide)
+//   dw_partial  [sets][nb][2][bwp][bwp] per-workgroup weight-gradient sums, sets = kGemmWgPerUnit (fast)
+//               or kWideWgPerUnit (wide); fp32, or bf16 in the fast backward when 16-bit gradients are
+//               asked for (sized for fp32 either way)
 enum ScratchKind { kScratchPlain = 0, kScratchFast = 1, kScratchWide = 2 };
 struct ScratchLayout {
   size_t partial, delta, dw_partial, total;
