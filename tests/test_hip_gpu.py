@@ -300,6 +300,43 @@ def test_capped_sqrt_derivative_regime_matches_oracle(dtype, shape):
         assert err < tol, (name, err)
 
 
+@pytest.mark.parametrize("shape", [(2048, 16, 256, 2), (300, 33, 384, 2), (2, 9000, 128, 4), (1, 20000, 640, 2)])
+def test_unusual_shapes_split_equals_whole(shape):
+    """Many short sequences, long sequences, wide blocks: too large for the oracle in a test, so the check
+    is the size-independent one.  One call over T tokens equals two calls that carry the state across the
+    cut, in the outputs, the final state and every gradient (bf16 storage: equal up to one rounding step)."""
+    from griffin_amd import hip_rglru
+
+    B, T, W, nb = shape
+    _say("split-equals-whole case", shape)
+    gen = torch.Generator().manual_seed(41)
+    bw = W // nb
+    x = torch.randn(B, T, W, generator=gen).bfloat16().cuda()
+    params = [(torch.randn(nb, bw, bw, generator=gen) / bw ** 0.5).bfloat16().cuda(),
+              (0.3 * torch.randn(nb, bw, generator=gen)).bfloat16().cuda(),
+              (torch.randn(nb, bw, bw, generator=gen) / bw ** 0.5).bfloat16().cuda(),
+              (0.3 * torch.randn(nb, bw, generator=gen)).bfloat16().cuda(),
+              torch.logit((torch.rand(W, generator=gen) * 0.099 + 0.9) ** (1 / 8)).bfloat16().cuda()]
+    dy = torch.randn(B, T, W, generator=gen).bfloat16().cuda()
+    xs = x.clone().requires_grad_(True)
+    ps = [p.clone().requires_grad_(True) for p in params]
+    y, h_last = hip_rglru(xs, *ps, 8.0)
+    grads = torch.autograd.grad(y, [xs] + ps, dy)
+    cut = T // 2
+    xa, xb = x[:, :cut].clone().requires_grad_(True), x[:, cut:].clone().requires_grad_(True)
+    pa = [p.clone().requires_grad_(True) for p in params]
+    ya, ha = hip_rglru(xa, *pa, 8.0)
+    yb, hb = hip_rglru(xb, *pa, 8.0, h0=ha)
+    g2 = torch.autograd.grad([ya, yb], [xa, xb] + pa, [dy[:, :cut], dy[:, cut:]])
+    torch.cuda.synchronize()
+    assert all(torch.isfinite(t.float()).all() for t in (y, h_last, *grads))
+    assert rel_err(torch.cat((ya, yb), dim=1).float(), y.float()) < BF16_TOL
+    assert rel_err(hb, h_last) < 1e-5
+    assert rel_err(torch.cat(g2[:2], dim=1).float(), grads[0].float()) < BF16_TOL
+    for got, want, name in zip(g2[2:], grads[1:], PARAMS[1:]):
+        assert rel_err(got.float(), want.float()) < BF16_TOL, name
+
+
 # ------------------------------------------------------------------ decode step
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, FP32_TOL), (torch.bfloat16, BF16_TOL)])
 def test_step_kernel_matches_oracle(dtype, tol):
