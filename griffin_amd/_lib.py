@@ -14,7 +14,7 @@ RGLRU_BF16 = 1
 FLAG_RESET = 1
 FLAG_INACTIVE = 2
 CHUNK = 32
-ABI_VERSION = 14
+ABI_VERSION = 15
 
 _lock = threading.Lock()
 _lib = None
@@ -62,8 +62,15 @@ _SIGNATURES = {
     "rglru_hip_rmsnorm_fwd": (ctypes.c_int, [_P, _P, _P, _P, _I, _I, ctypes.c_float, ctypes.c_int, ctypes.c_int, _P]),
     "rglru_hip_rmsnorm_scratch_bytes": (ctypes.c_size_t, [_I, _I]),
     "rglru_hip_rmsnorm_bwd": (ctypes.c_int, [_P] * 7 + [_I, _I, ctypes.c_int, ctypes.c_int, ctypes.c_int, _P]),
-    "rglru_hip_decode_prepare": (ctypes.c_int, [_P] * 11 + [_I, _I, _I, ctypes.c_int, ctypes.c_int, _P]),
-    "rglru_hip_step_gated": (ctypes.c_int, [_P] * 7 + [_I, _I, _I, ctypes.c_int, _P]),
+    "rglru_hip_decode_prepare": (ctypes.c_int, [_P, _I] + [_P] * 10 + [_I, _I, _I, ctypes.c_int, ctypes.c_int, _P]),
+    "rglru_hip_block_fwd_path": (ctypes.c_int, [_I, _I, _I, ctypes.c_int]),
+    "rglru_hip_block_flags": (ctypes.c_int, [_P, _P, _I, _P]),
+    "rglru_hip_block_fwd": (ctypes.c_int, [_P, _I, _P, _I, _P, _P, _P, _I, ctypes.c_int] + [_P] * 9
+                            + [_I, _I, _I, _I, ctypes.c_int, _P]),
+    "rglru_hip_prepare_block_fwd": (ctypes.c_int, [_P] * 5 + [ctypes.c_float, ctypes.c_int, _P]
+                                    + [_P, _I, _P, _I, _P, _P, _P, _I] + [_P] * 8
+                                    + [_I, _I, _I, _I, ctypes.c_int, _P]),
+    "rglru_hip_step_gated": (ctypes.c_int, [_P] * 6 + [_I, _P] + [_I, _I, _I, ctypes.c_int, _P]),
     "rglru_hip_set_spin_limit": (ctypes.c_int64, [_I]),
     "rglru_hip_set_timing": (ctypes.c_int, [ctypes.c_int]),
     "rglru_hip_kernel_ms": (ctypes.c_float, [ctypes.c_int]),

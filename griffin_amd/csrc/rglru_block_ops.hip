@@ -696,6 +696,7 @@ struct DecodeArgs {
   const void* u; const void* state; const void* taps; const void* bias;
   const long long* prev_pos; const long long* seg_pos; const unsigned char* active;
   void* x; void* new_state; long long* new_pos; unsigned char* flags;
+  long long ldu;                                          // elements between rows of u (>= W)
   int B, W, K, nvec, vec_dtype;
 };
 
@@ -714,7 +715,7 @@ __global__ __launch_bounds__(kConvThreads) void decode_prepare_kernel(DecodeArgs
     p.new_pos[b] = live ? pos : before;
     p.flags[b] = (unsigned char)((live && pos == 0 ? RGLRU_FLAG_RESET : 0u) | (live ? 0u : RGLRU_FLAG_INACTIVE));
   }
-  const rsrc_t ru = make_rsrc((const IO*)p.u + (long long)b * p.W, uW * es);
+  const rsrc_t ru = make_rsrc((const IO*)p.u + (long long)b * p.ldu, uW * es);
   const rsrc_t rx = make_rsrc((IO*)p.x + (long long)b * p.W, uW * es);
   const unsigned off = (unsigned)c0 * es;
   float cur[V], acc[V], hist[K > 1 ? K - 1 : 1][V];          // hist[j] = state row j (oldest first)
@@ -1182,6 +1183,26 @@ int rglru_hip_conv_padded_bwd(const void* u, const void* state, const void* taps
   return rc;
 }
 
+// Flag bytes of the block forward from the token positions: reset where a document starts, and in bits 2-3
+// the number of convolution lags that reach in front of the document, 3 - min(position, 3).
+__global__ __launch_bounds__(256) void block_flags_kernel(const long long* pos, unsigned char* flags, long long n) {
+  const long long stride = (long long)gridDim.x * 256;
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += stride) {
+    const long long p = pos[i];
+    const unsigned near = p < 0 ? 3u : p < 3 ? (unsigned)(3 - p) : 0u;
+    flags[i] = (unsigned char)((p == 0 ? RGLRU_FLAG_RESET : 0u) | (near << 2));
+  }
+}
+
+int rglru_hip_block_flags(const int64_t* segment_pos, uint8_t* flags, int64_t n, void* stream) {
+  if (!segment_pos || !flags) return fail(RGLRU_E_ARG, "block_flags: null pointer");
+  if (n <= 0) return fail(RGLRU_E_ARG, "block_flags: empty tensor");
+  long long blocks = (n + 255) / 256; if (blocks > 4096) blocks = 4096;
+  hipLaunchKernelGGL(block_flags_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                     (const long long*)segment_pos, (unsigned char*)flags, (long long)n);
+  return check_launch("block_flags");
+}
+
 int rglru_hip_gelu_gate_fwd(const void* h, const void* v, void* out, int64_t n, int dtype, void* stream) {
   if (!h || !v || !out) return fail(RGLRU_E_ARG, "gelu_gate_fwd: null pointer");
   GateArgs a;
@@ -1199,7 +1220,7 @@ int rglru_hip_gelu_gate_bwd(const void* dout, const void* h, const void* v, void
   return gate_launch("gelu_gate_bwd", true, a, dtype, stream);
 }
 
-int rglru_hip_decode_prepare(const void* u, const void* conv_state, const void* taps, const void* bias,
+int rglru_hip_decode_prepare(const void* u, int64_t u_stride, const void* conv_state, const void* taps, const void* bias,
                              const int64_t* prev_pos, const int64_t* segment_pos, const uint8_t* active,
                              void* x, void* new_conv_state, int64_t* new_pos, uint8_t* flags,
                              int64_t B, int64_t W, int64_t K, int dtype, int vec_dtype, void* stream) {
@@ -1207,13 +1228,16 @@ int rglru_hip_decode_prepare(const void* u, const void* conv_state, const void* 
   if (rc) return rc;
   if (!u || !taps || !x || !new_pos || !flags || (K > 1 && !new_conv_state))
     return fail(RGLRU_E_ARG, "decode_prepare: null pointer");
+  if (u_stride == 0) u_stride = W;
+  if (u_stride < W) return fail(RGLRU_E_ARG, "decode_prepare: row stride %lld of u is smaller than the width %lld", (long long)u_stride, (long long)W);
   DecodeArgs a;
   memset(&a, 0, sizeof(a));
   a.u = u; a.state = conv_state; a.taps = taps; a.bias = bias;
   a.prev_pos = (const long long*)prev_pos; a.seg_pos = (const long long*)segment_pos; a.active = active;
   a.x = x; a.new_state = new_conv_state; a.new_pos = (long long*)new_pos; a.flags = flags;
-  a.B = (int)B; a.W = (int)W; a.K = (int)K; a.vec_dtype = vec_dtype;
-  const bool vec = conv_vector_ok(W, dtype, {u, conv_state, x, new_conv_state});
+  a.B = (int)B; a.W = (int)W; a.K = (int)K; a.vec_dtype = vec_dtype; a.ldu = u_stride;
+  const bool vec = conv_vector_ok(W, dtype, {u, conv_state, x, new_conv_state}) &&
+                   (u_stride * (dtype == RGLRU_BF16 ? 2 : 4)) % 16 == 0;
   a.nvec = (int)(vec ? W / (dtype == RGLRU_BF16 ? 8 : 4) : W);
   const long long items = (long long)B * a.nvec;
   dim3 grid((unsigned)((items + kConvThreads - 1) / kConvThreads));

@@ -146,6 +146,13 @@ struct FusedArgs {
   void* dx; void* du_a; void* du_x; float* dh0;           // backward out
   float* h_state; const float* h_prev;                    // decode step: state out, state in (may be the same)
   const void* gate_v;                                     // decode step: y = h * gelu_tanh(gate_v) when set
+  long long ld_gate;                                      // ... elements between rows of gate_v (>= W)
+  // block forward: x = causal depthwise conv of the rows at `x` (taps by lag, carried rows in conv_state),
+  // out `gated` = y * gelu_tanh(gate_v); x_out, y and conv_new_state are optional outputs
+  const void* conv_state; const void* conv_taps; const void* conv_bias;
+  void* x_out; void* conv_new_state; void* gated;
+  long long ld_x;                                         // elements between rows of x (>= W)
+  int conv_k, conv_vec_dtype;
   // workspace
   float* ckpt; rec_t* rec_a; unsigned* ticket;
   unsigned* fail; float* partial; float* dw_partial;
@@ -322,7 +329,7 @@ RGLRU_DEVICE void gate_mfma_held(const IO* lds, const HeldWeights<IO, NKG>& hw, 
 
 RGLRU_DEVICE unsigned token_flag(const FusedArgs& p, long long token_row, bool inside) {
   if (!inside) return RGLRU_FLAG_INACTIVE;
-  return p.flags ? (unsigned)p.flags[token_row] : 0u;
+  return p.flags ? (unsigned)p.flags[token_row] & 3u : 0u;   // bits 2-3 belong to the block forward's convolution
 }
 
 // Flags of a lane's run of 16 consecutive tokens, two bits per token (token e at bits 2e, 2e + 1);
@@ -404,9 +411,10 @@ RGLRU_DEVICE void fwd_local(const FusedArgs& p, const WaveId& w, FwdTile<MT>& t,
 }
 
 // Stage 2: carry in, carry out and checkpoint, then the recurrence itself and the stores.
-template <typename IO, int MT, bool MASKED, bool STAGED>
+template <typename IO, int MT, bool MASKED, bool STAGED, bool BLOCK = false>
 RGLRU_DEVICE void fwd_finalize(const FusedArgs& p, const WaveId& w, const FwdTile<MT>& t, unsigned char* stage,
-                               const CarryBatch<kFwdDepth>* first = nullptr, bool live = true) {
+                               const CarryBatch<kFwdDepth>* first = nullptr, bool live = true,
+                               const bf16x8* gate_rows = nullptr) {
   constexpr int EL = 16 * MT, TR = 32 * MT;
   const int hf = w.hf, b = t.b, c = t.c;
   const long long W = p.W;
@@ -444,7 +452,7 @@ RGLRU_DEVICE void fwd_finalize(const FusedArgs& p, const WaveId& w, const FwdTil
   // y tile through a buffer descriptor: rows past the end of the sequence are dropped
   const int rows = !live ? 0 : ((p.T - t0) < TR ? (p.T - t0) : TR);
   const unsigned row_bytes = (unsigned)p.W * (unsigned)sizeof(IO);
-  const rsrc_t ry = make_rsrc((const IO*)p.y + ((long long)b * p.T + t0) * W, (unsigned)rows * row_bytes);
+  const rsrc_t ry = make_rsrc((const IO*)p.y + ((long long)b * p.T + t0) * W, (BLOCK && !p.y) ? 0u : (unsigned)rows * row_bytes);
   if constexpr (STAGED) {
     // 16-bit outputs: transpose through the wave's staging area, then 16-byte stores
     unsigned char* my = stage + WaveStage<TR>::row_offset(hf * EL) + w.r * 2;
@@ -455,7 +463,26 @@ RGLRU_DEVICE void fwd_finalize(const FusedArgs& p, const WaveId& w, const FwdTil
       if ((e & 15) == 15) BufIo<float>::store(h, rck, ck_off[e >> 4], 0u);
     }
     wave_lds_fence();
-    stage_flush<TR>(stage, ry, row_bytes, (unsigned)(w.k * p.bw + w.slab * 32) * 2u, w.lane);
+    if constexpr (BLOCK) {
+      // output gate at the store: a lane holds the same 8 channels of a row of y and of the gate input
+      const rsrc_t rg = make_rsrc((const IO*)p.gated + ((long long)b * p.T + t0) * W, (unsigned)rows * row_bytes);
+      const unsigned col_bytes = (unsigned)(w.k * p.bw + w.slab * 32) * 2u;
+#pragma unroll
+      for (int i = 0; i < TR / 16; ++i) {
+        const int row = 16 * i + (w.lane >> 2);
+        const unsigned seg = (unsigned)(w.lane & 3) * 16u;
+        const i32x4 raw = *reinterpret_cast<const i32x4*>(stage + WaveStage<TR>::row_offset(row) + seg);
+        const unsigned off = (unsigned)row * row_bytes + col_bytes + seg;
+        buf_store_b128(raw, ry, off);                       // y itself: dropped unless the caller keeps it
+        const bf16x8 hv = __builtin_bit_cast(bf16x8, raw);
+        bf16x8 out;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) out[e] = (__bf16)((float)hv[e] * gelu_tanh_parts((float)gate_rows[i][e]).gelu);
+        buf_store_b128(__builtin_bit_cast(i32x4, out), rg, off);
+      }
+    } else {
+      stage_flush<TR>(stage, ry, row_bytes, (unsigned)(w.k * p.bw + w.slab * 32) * 2u, w.lane);
+    }
     wave_lds_fence();
   } else {
     unsigned voff = ch_ok ? (unsigned)(hf * EL) * row_bytes + (unsigned)w.ch * (unsigned)sizeof(IO) : kOutOfRange;
@@ -480,9 +507,15 @@ constexpr int kFwdMT = 2;
 #ifndef RGLRU_NARROW_OCC
 #define RGLRU_NARROW_OCC 3
 #endif
-template <typename IO, int NKG, bool MASKED>
-__global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : (NKG == 4 || NKG == 2) ? RGLRU_NARROW_OCC : NKG > 8 ? 1 : 2)) void fwd_kernel(FusedArgs p) {
+// BLOCK: the recurrent block's forward around the scan in the same launch (griffin/griffin.py:474-487 in
+// front, :464 and :520 behind).  The rows at p.x are the block's first projection; a lane loads four
+// consecutive rows of eight channels plus the three rows in front of them, convolves them (taps by lag
+// from LDS, lags masked per token through bits 2-3 of the flag bytes = 3 - min(position, 3)) and puts the
+// result where the plain kernel puts x; the store stage multiplies by gelu_tanh of the second projection.
+template <typename IO, int NKG, bool MASKED, bool BLOCK = false>
+__global__ __launch_bounds__(kThreads, (BLOCK ? 2 : NKG < 0 ? RGLRU_GIVEN_OCC : (NKG == 4 || NKG == 2) ? RGLRU_NARROW_OCC : NKG > 8 ? 1 : 2)) void fwd_kernel(FusedArgs p) {
   constexpr int MT = kFwdMT, TR = 32 * MT, EL = 16 * MT;
+  static_assert(!BLOCK || (sizeof(IO) == 2 && (NKG == 8 || NKG == 4 || NKG == 2)), "block forward: 16-bit storage, register-held weights");
   typedef Io<IO> Tr;
   typedef typename Tr::Frag Frag;
   // NKG > 0: gate weights held in registers, pre-activations on MFMA.  Up to NKG = 8 (128 channels) a
@@ -498,10 +531,26 @@ __global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : (NKG == 4 ||
   __shared__ __attribute__((aligned(16))) IO lds_pre[GIVEN ? 2 * TR * LDSROW : Tr::HW];   // W_a x | W_x x tiles
   __shared__ __attribute__((aligned(16))) unsigned char stage_all[kWaves * WaveStage<TR>::kBytes];
   __shared__ unsigned s_ticket[2];
+  __shared__ __attribute__((aligned(16))) float conv_w[BLOCK ? 5 * KC : 4];    // taps of lag 0..3, then the bias
 
   const WaveId w = wave_identity(p, blockIdx.x);
   const int hf = w.hf, tid = threadIdx.x;
   unsigned char* stage = stage_all + w.wave * WaveStage<TR>::kBytes;
+  if constexpr (BLOCK) {
+    // read after the barrier that follows the first ticket
+    for (int i = tid; i < 5 * KC; i += kThreads) {
+      const int j = i / KC, ch = w.tile_col + (i - j * KC);
+      float v = 0.f;
+      if (ch < p.W) {
+        if (j == 4) { if (p.conv_bias) v = p.conv_vec_dtype == RGLRU_BF16 ? (float)((const __bf16*)p.conv_bias)[ch] : ((const float*)p.conv_bias)[ch]; }
+        else if (j < p.conv_k) {
+          const long long at = (long long)ch * p.conv_k + (p.conv_k - 1 - j);     // the tap of lag j
+          v = p.conv_vec_dtype == RGLRU_BF16 ? (float)((const __bf16*)p.conv_taps)[at] : ((const float*)p.conv_taps)[at];
+        }
+      }
+      conv_w[i] = v;
+    }
+  }
   const IO* wg = (const IO*)p.wg;
   const IO* w_a_row = wg + ((long long)(0 * p.nb + w.k) * p.bwp + (w.slab_ok ? w.o : 0)) * p.bwp + hf * Tr::HW;
   const IO* w_x_row = wg + ((long long)(1 * p.nb + w.k) * p.bwp + (w.slab_ok ? w.o : 0)) * p.bwp + hf * Tr::HW;
@@ -527,10 +576,21 @@ __global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : (NKG == 4 ||
     const unsigned u_row_bytes = 2u * (unsigned)p.bw * (unsigned)sizeof(IO);   // a row of `pre`: W_a x | W_x x of one block
     unsigned pre_off[NV];                                // lane offsets inside a tile (fixed)
     unsigned u_off[GIVEN ? NV : 1];
+    // BLOCK: rows 4 rho .. 4 rho + 3 of channel vector bcv; the descriptor starts three rows before the tile
+    static_assert(!BLOCK || (NV == 4 && VPR == 16), "block forward: four rows of a 128-channel tile per lane");
+    const int rho = tid / VPR, bcv = tid - rho * VPR;
+    const unsigned x_row_bytes = BLOCK ? (unsigned)p.ld_x * (unsigned)sizeof(IO) : row_bytes;
+    const bool bcol_ok = BLOCK && (x_col + bcv * Tr::HW < p.W);
+    const unsigned bcol_bytes = (unsigned)(x_col + bcv * Tr::HW) * (unsigned)sizeof(IO);
+    Frag halo[BLOCK ? 3 : 1];
+    unsigned conv_fl = 0u;                               // flag bytes of the lane's four rows
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int idx = tid + i * kThreads;
       const int row = idx / VPR, cv = idx - row * VPR;
+      if constexpr (BLOCK)
+        pre_off[i] = bcol_ok ? (unsigned)(4 * rho + i + 3) * x_row_bytes + bcol_bytes : kOutOfRange;
+      else
       pre_off[i] = (idx < TR * VPR) ? (unsigned)row * row_bytes + (unsigned)(x_col + cv * Tr::HW) * (unsigned)sizeof(IO)
                                     : kOutOfRange;
       if constexpr (GIVEN)
@@ -543,9 +603,30 @@ __global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : (NKG == 4 ||
       const unsigned tk = live ? (unsigned)tk_in : 0u;
       const int c = (int)(tk / (unsigned)q.n_b), b = q.first_b + (int)(tk - (unsigned)c * (unsigned)q.n_b) * p.queues;
       const int rows = !live ? 0 : ((p.T - c * TR) < TR ? (p.T - c * TR) : TR);
+      if constexpr (BLOCK) {
+        const rsrc_t rx = make_rsrc(x + ((long long)b * p.T + (long long)c * TR - 3) * p.ld_x, rows ? (unsigned)(rows + 3) * x_row_bytes : 0u);
+#pragma unroll
+        for (int i = 0; i < NV; ++i) pre[i] = buf_load_frag<Frag>(rx, pre_off[i]);
+        // the rows in front of a sequence are the carried state (fetched where the tile is consumed) or zero
+        const bool front = c == 0 && rho == 0;
+#pragma unroll
+        for (int h = 0; h < 3; ++h)
+          halo[h] = buf_load_frag<Frag>(rx, (front || !bcol_ok) ? kOutOfRange : (unsigned)(4 * rho + h) * x_row_bytes + bcol_bytes);
+        if constexpr (MASKED) {
+          const rsrc_t rf = make_rsrc(p.flags + (long long)b * p.T + (long long)c * TR, p.flags ? (unsigned)rows : 0u);
+          if (p.flags_vec) {
+            conv_fl = (unsigned)__builtin_amdgcn_raw_buffer_load_b32(rf, (unsigned)(4 * rho), 0, 0);
+          } else {
+            conv_fl = 0u;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) conv_fl |= ((unsigned)__builtin_amdgcn_raw_buffer_load_b8(rf, (unsigned)(4 * rho + i), 0, 0) & 0xffu) << (8 * i);
+          }
+        }
+      } else {
       const rsrc_t rx = make_rsrc(x + ((long long)b * p.T + (long long)c * TR) * W, (unsigned)rows * row_bytes);
 #pragma unroll
       for (int i = 0; i < NV; ++i) pre[i] = buf_load_frag<Frag>(rx, pre_off[i]);
+      }
       if constexpr (GIVEN) {
         // the x-gate half of a row starts bw elements after the a-gate half
         const IO* ubase = (const IO*)p.pre + ((long long)w.k * p.rows_total + (long long)b * p.T + (long long)c * TR) * (2 * p.bw);
@@ -575,7 +656,12 @@ __global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : (NKG == 4 ||
     const unsigned rec_lane = (slab_ok && w.ch_ok) ? (unsigned)w.ch * 8u : kOutOfRange;
     // A dead finalize in front of the loop: the loop is entered with the same memory operations in
     // flight as its back edge has, so the waits at its top are exact instead of worst case.
-    fwd_finalize<IO, MT, MASKED, sizeof(IO) == 2>(p, w, cur, stage, nullptr, false);
+    bf16x8 gate_rows[BLOCK ? TR / 16 : 1];               // the lane's vectors of the second projection
+    if constexpr (BLOCK) {
+#pragma unroll
+      for (int i = 0; i < TR / 16; ++i) gate_rows[i] = Io<__bf16>::zero();
+    }
+    fwd_finalize<IO, MT, MASKED, sizeof(IO) == 2, BLOCK>(p, w, cur, stage, nullptr, false, gate_rows);
     while (tk < q.tiles) {
       cur.c = (int)((unsigned)tk / (unsigned)q.n_b);
       cur.b = q.first_b + (int)((unsigned)tk - (unsigned)cur.c * (unsigned)q.n_b) * p.queues;
@@ -590,6 +676,66 @@ __global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : (NKG == 4 ||
       CarryBatch<kFwdDepth> ahead;
       carry_prefetch<kFwdDepth>(make_rsrc(p.rec_a + (long long)cur.b * p.nCf * W, (unsigned)p.nCf * rec_stride), rec_lane,
                        rec_stride, cur.c, -1, -1, ahead);
+      if constexpr (BLOCK) {
+        const int t0 = cur.c * TR;
+        const int rows = (p.T - t0) < TR ? (p.T - t0) : TR;
+        Frag um[7] = {halo[0], halo[1], halo[2], pre[0], pre[1], pre[2], pre[3]};      // tokens t0 + 4 rho - 3 .. + 3
+        if (cur.c == 0 && p.conv_state && rho == 0 && bcol_ok) {
+          // carried rows of the previous call: state row j holds the token K - 1 - j steps back
+          const int K1 = p.conv_k - 1;
+          const rsrc_t rs = make_rsrc((const IO*)p.conv_state + (long long)cur.b * K1 * W, (unsigned)K1 * row_bytes);
+#pragma unroll
+          for (int h = 0; h < 3; ++h) {
+            const int j = K1 - 3 + h;
+            um[h] = buf_load_frag<Frag>(rs, j >= 0 ? (unsigned)j * row_bytes + bcol_bytes : kOutOfRange);
+          }
+        }
+        float tap[4][8], cbias[8];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const f32x4 lo = *reinterpret_cast<const f32x4*>(conv_w + j * KC + bcv * 8);
+          const f32x4 hi = *reinterpret_cast<const f32x4*>(conv_w + j * KC + bcv * 8 + 4);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) { tap[j][e] = lo[e]; tap[j][4 + e] = hi[e]; }
+        }
+        {
+          const f32x4 lo = *reinterpret_cast<const f32x4*>(conv_w + 4 * KC + bcv * 8);
+          const f32x4 hi = *reinterpret_cast<const f32x4*>(conv_w + 4 * KC + bcv * 8 + 4);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) { cbias[e] = lo[e]; cbias[4 + e] = hi[e]; }
+        }
+        const rsrc_t rxo = make_rsrc((const IO*)p.x_out + ((long long)cur.b * p.T + t0) * W, p.x_out ? (unsigned)rows * row_bytes : 0u);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int hidden = MASKED ? (int)((conv_fl >> (8 * i + 2)) & 3u) : 0;        // lags 4 - hidden .. 3 do not apply
+          Frag out;
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            float a = fmaf((float)um[3 + i][e], tap[0][e], cbias[e]);
+#pragma unroll
+            for (int lag = 1; lag < 4; ++lag) {
+              const float with = fmaf((float)um[3 + i - lag][e], tap[lag][e], a);
+              a = (MASKED && lag + hidden > 3) ? a : with;
+            }
+            out[e] = (IO)a;
+          }
+          *reinterpret_cast<Frag*>(lds + (4 * rho + i) * LDSROW + bcv * Tr::HW) = out;
+          buf_store_b128(__builtin_bit_cast(i32x4, out), rxo, bcol_ok ? (unsigned)(4 * rho + i) * row_bytes + bcol_bytes : kOutOfRange);
+        }
+        if (cur.c == p.nCf - 1 && p.conv_new_state && bcol_ok) {
+          // the last K - 1 rows of [carried rows ; input] become the next call's carried rows
+          const int K1 = p.conv_k - 1;
+          const int last = p.T - 1 - t0;                     // tile row of the sequence's last token
+          if (rho == last / 4) {
+            const rsrc_t rn = make_rsrc((IO*)p.conv_new_state + (long long)cur.b * K1 * W, (unsigned)K1 * row_bytes);
+#pragma unroll
+            for (int idx = 0; idx < 7; ++idx) {
+              const int srow = (4 * rho - 3 + idx) - (last - K1 + 1);
+              buf_store_b128(__builtin_bit_cast(i32x4, um[idx]), rn, (srow >= 0 && srow < K1) ? (unsigned)srow * row_bytes + bcol_bytes : kOutOfRange);
+            }
+          }
+        }
+      } else {
 #pragma unroll
       for (int i = 0; i < NV; ++i) {
         const int idx = tid + i * kThreads;
@@ -601,6 +747,7 @@ __global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : (NKG == 4 ||
             *reinterpret_cast<Frag*>(lds_pre + (TR + row) * LDSROW + cv * Tr::HW) = pre_x[i];
           }
         }
+      }
       }
       __syncthreads();
       if (slab_ok) {
@@ -627,8 +774,19 @@ __global__ __launch_bounds__(kThreads, (NKG < 0 ? RGLRU_GIVEN_OCC : (NKG == 4 ||
       __syncthreads();
       par ^= 1;
       const long long tk_next = s_ticket[par];
+      if constexpr (BLOCK) {
+        // the tile's rows of the second projection, in the layout of the store stage
+        const int t0 = cur.c * TR;
+        const int rows = (p.T - t0) < TR ? (p.T - t0) : TR;
+        const unsigned v_row_bytes = (unsigned)p.ld_gate * (unsigned)sizeof(IO);
+        const rsrc_t rv = make_rsrc((const IO*)p.gate_v + ((long long)cur.b * p.T + t0) * p.ld_gate, slab_ok ? (unsigned)rows * v_row_bytes : 0u);
+#pragma unroll
+        for (int i = 0; i < TR / 16; ++i)
+          gate_rows[i] = buf_load_frag<bf16x8>(rv, (unsigned)(16 * i + (w.lane >> 2)) * v_row_bytes +
+                                                   (unsigned)(w.k * p.bw + w.slab * 32) * 2u + (unsigned)(w.lane & 3) * 16u);
+      }
       issue(tk_next);
-      fwd_finalize<IO, MT, MASKED, sizeof(IO) == 2>(p, w, cur, stage, &ahead, slab_ok);
+      fwd_finalize<IO, MT, MASKED, sizeof(IO) == 2, BLOCK>(p, w, cur, stage, &ahead, slab_ok, gate_rows);
       tk = tk_next;
     }
   } else {
@@ -2010,7 +2168,7 @@ __global__ __launch_bounds__(kThreads) void step_kernel(FusedArgs p) {
       const bool ok = w.ch_ok && row < p.B;
       const long long at = ok ? row * W + w.ch : 0;
       h_old[e] = ok ? p.h_prev[at] : 0.f;
-      gate[e] = (ok && p.gate_v) ? (float)((const IO*)p.gate_v)[at] : 0.f;
+      gate[e] = (ok && p.gate_v) ? (float)((const IO*)p.gate_v)[row * p.ld_gate + w.ch] : 0.f;
       fls[e] = (ok && p.flags) ? (unsigned)p.flags[row] : 0u;
     }
   };
@@ -2108,7 +2266,7 @@ __global__ __launch_bounds__(kThreads) void step16_kernel(FusedArgs p) {
     const long long at = ok ? row * W + ch : 0;
     h_old[v] = ok ? p.h_prev[at] : 0.f;
     xv[v] = ok ? (float)((const IO*)p.x)[at] : 0.f;
-    gate[v] = (ok && p.gate_v) ? (float)((const IO*)p.gate_v)[at] : 0.f;
+    gate[v] = (ok && p.gate_v) ? (float)((const IO*)p.gate_v)[row * p.ld_gate + ch] : 0.f;
     fls[v] = (ok && p.flags) ? (unsigned)p.flags[row] : 0u;
   }
   const float bias_a = p.bias[kp], bias_x = p.bias[p.Wp + kp], sp = p.sp[kp];
@@ -2508,30 +2666,39 @@ size_t rglru_hip_workspace_bytes(int64_t B, int64_t T, int64_t W, int64_t nb) {
 
 int rglru_hip_wide_path(int64_t W, int64_t nb, int dtype);
 
+int rglru_hip_block_fwd_path(int64_t W, int64_t nb, int64_t K, int dtype) {
+  if (dtype != RGLRU_BF16 || W <= 0 || nb <= 0 || W % nb || K < 1 || K > 4) return 0;
+  const int64_t bw = W / nb;
+  return (bw == 32 || bw == 64 || bw == 128) ? 1 : 0;
+}
+
 size_t rglru_hip_bwd_scratch_bytes(int64_t B, int64_t T, int64_t W, int64_t nb, int dtype) {
   if (B <= 0 || T <= 0 || W <= 0 || nb <= 0 || W % nb) return 0;
   const int kind = rglru_hip_fast_path(W, nb, dtype) ? kScratchFast : rglru_hip_wide_path(W, nb, dtype) ? kScratchWide : kScratchPlain;
   return make_scratch_layout(B, T, make_geometry(W, nb), kind).total;
 }
 
+// What the block forward adds to the scan's arguments (x is then the block's first projection).
+struct BlockFwd {
+  const void* v; int64_t x_stride, v_stride;
+  const void* conv_state; const void* taps; const void* conv_bias; int64_t K; int vec_dtype;
+  void* x_conv; void* gated; void* new_conv_state;
+};
+
 static int fwd_impl(const void* x, const void* prep, const float* h0, const uint8_t* flags,
                     void* y, float* h_last, void* ws,
                     int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, bool cleared, void* stream,
-                    const void* pre = nullptr) {
+                    const void* pre = nullptr, const BlockFwd* blk = nullptr) {
   int rc = check_geometry("fwd", W, nb, dtype);
   if (rc) return rc;
   if (B <= 0 || T <= 0) return fail(RGLRU_E_ARG, "fwd: B and T must be positive (got %lld, %lld)", (long long)B, (long long)T);
-  if (!x || !prep || !y || !ws) return fail(RGLRU_E_ARG, "fwd: null pointer");
+  if (!x || !prep || (!y && !blk) || !ws) return fail(RGLRU_E_ARG, "fwd: null pointer");
   rc = check_extents("fwd", B, T, W);
   if (rc) return rc;
   Geometry g = make_geometry(W, nb);
   WorkLayout L = make_work_layout(B, T, g);
   hipStream_t s = (hipStream_t)stream;
   char* wb = (char*)ws;
-  if (!cleared) {
-    rc = launch_clear(wb, L.f_begin, L.b_end, s);       // carry records and tickets of both passes, failure word
-    if (rc) return rc;
-  }
   FusedArgs a;
   memset(&a, 0, sizeof(a));
   fill_common(a, g, prep, dtype);
@@ -2550,15 +2717,45 @@ static int fwd_impl(const void* x, const void* prep, const float* h0, const uint
     a.pre = pre; a.rows_total = B * T;
     nkg = -1;
   }
+  if (blk) {
+    const int64_t xs = blk->x_stride ? blk->x_stride : W, vs = blk->v_stride ? blk->v_stride : W;
+    if (!rglru_hip_block_fwd_path(W, nb, blk->K, dtype))
+      return fail(RGLRU_E_UNSUPPORTED, "block_fwd: needs bf16 storage, gate blocks of 32, 64 or 128 channels and 1 to 4 taps");
+    if (blk->vec_dtype != RGLRU_F32 && blk->vec_dtype != RGLRU_BF16) return fail(RGLRU_E_ARG, "block_fwd: unknown vector dtype %d", blk->vec_dtype);
+    if (!blk->v || !blk->taps || !blk->gated) return fail(RGLRU_E_ARG, "block_fwd: null pointer");
+    if (xs < W || vs < W) return fail(RGLRU_E_ARG, "block_fwd: a row stride is smaller than the width %lld", (long long)W);
+    const void* ptrs[] = {x, blk->v, blk->conv_state, blk->x_conv, blk->gated, blk->new_conv_state, y};
+    for (const void* q : ptrs) if ((uintptr_t)q % 16) return fail(RGLRU_E_UNSUPPORTED, "block_fwd: tensors must be 16-byte aligned");
+    if ((W * 2) % 16 || (xs * 2) % 16 || (vs * 2) % 16) return fail(RGLRU_E_UNSUPPORTED, "block_fwd: rows must be a multiple of 16 bytes");
+    if (!nkg) return fail(RGLRU_E_UNSUPPORTED, "block_fwd: no kernel for this shape");
+    a.gate_v = blk->v; a.ld_gate = vs; a.ld_x = xs;
+    a.conv_state = blk->K > 1 ? blk->conv_state : nullptr; a.conv_taps = blk->taps; a.conv_bias = blk->conv_bias;
+    a.conv_k = (int)blk->K; a.conv_vec_dtype = blk->vec_dtype;
+    a.x_out = blk->x_conv; a.gated = blk->gated; a.conv_new_state = blk->K > 1 ? blk->new_conv_state : nullptr;
+  }
+  if (!cleared) {
+    rc = launch_clear(wb, L.f_begin, L.b_end, s);       // carry records and tickets of both passes, failure word
+    if (rc) return rc;
+  }
   pack_units(a, g, nkg);
   // without weights in registers three workgroups fit a compute unit
-  a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nCf, nkg < 0 ? RGLRU_GIVEN_OCC : ((nkg == 4 || nkg == 2) ? RGLRU_NARROW_OCC : nkg > 8 ? 1 : 2), 1 << 20);
+  a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nCf, blk ? 2 : nkg < 0 ? RGLRU_GIVEN_OCC : ((nkg == 4 || nkg == 2) ? RGLRU_NARROW_OCC : nkg > 8 ? 1 : 2), 1 << 20);
   a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
   dim3 grid((unsigned)(a.wg_per_unit * a.units));
   {
     KernelTimer timer(0, s);
     const int masked = (flags != nullptr) || (T % (32 * kFwdMT) != 0);
-    RGLRU_DISPATCH_FWD(grid, s, a, dtype, nkg, masked);
+    if (blk) {
+#define RGLRU_BLOCK_CASE(N)                                                                                            \
+      if (nkg == N) {                                                                                                  \
+        if (masked) hipLaunchKernelGGL((fwd_kernel<__bf16, N, true, true>), grid, dim3(kThreads), 0, s, a);            \
+        else hipLaunchKernelGGL((fwd_kernel<__bf16, N, false, true>), grid, dim3(kThreads), 0, s, a);                  \
+      }
+      RGLRU_BLOCK_CASE(8) RGLRU_BLOCK_CASE(4) RGLRU_BLOCK_CASE(2)
+#undef RGLRU_BLOCK_CASE
+    } else {
+      RGLRU_DISPATCH_FWD(grid, s, a, dtype, nkg, masked);
+    }
   }
   return check_launch("fwd");
 }
@@ -2685,6 +2882,33 @@ int rglru_hip_prepare_fwd(const void* w_a, const void* b_a, const void* w_x, con
   rc = prepare_impl(w_a, b_a, w_x, b_x, lambda, c, W, nb, dtype, vec_dtype, prep, (char*)ws + L.f_begin, L.b_end - L.f_begin, stream);
   if (rc) return rc;
   return fwd_impl(x, prep, h0, flags, y, h_last, ws, B, T, W, nb, dtype, true, stream);
+}
+
+int rglru_hip_block_fwd(const void* u, int64_t u_stride, const void* v, int64_t v_stride,
+                        const void* conv_state, const void* taps, const void* conv_bias, int64_t K, int vec_dtype,
+                        const void* prep, const float* h0, const uint8_t* flags,
+                        void* x_conv, void* y, void* gated, void* new_conv_state, float* h_last, void* ws,
+                        int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, void* stream) {
+  const BlockFwd blk = {v, u_stride, v_stride, conv_state, taps, conv_bias, K, vec_dtype, x_conv, gated, new_conv_state};
+  return fwd_impl(u, prep, h0, flags, y, h_last, ws, B, T, W, nb, dtype, false, stream, nullptr, &blk);
+}
+
+int rglru_hip_prepare_block_fwd(const void* w_a, const void* b_a, const void* w_x, const void* b_x,
+                                const void* lambda, float c, int vec_dtype, void* prep,
+                                const void* u, int64_t u_stride, const void* v, int64_t v_stride,
+                                const void* conv_state, const void* taps, const void* conv_bias, int64_t K,
+                                const float* h0, const uint8_t* flags,
+                                void* x_conv, void* y, void* gated, void* new_conv_state, float* h_last, void* ws,
+                                int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, void* stream) {
+  int rc = check_geometry("prepare_block_fwd", W, nb, dtype);
+  if (rc) return rc;
+  if (B <= 0 || T <= 0) return fail(RGLRU_E_ARG, "prepare_block_fwd: B and T must be positive (got %lld, %lld)", (long long)B, (long long)T);
+  if (!ws) return fail(RGLRU_E_ARG, "prepare_block_fwd: null pointer");
+  const WorkLayout L = make_work_layout(B, T, make_geometry(W, nb));
+  rc = prepare_impl(w_a, b_a, w_x, b_x, lambda, c, W, nb, dtype, vec_dtype, prep, (char*)ws + L.f_begin, L.b_end - L.f_begin, stream);
+  if (rc) return rc;
+  const BlockFwd blk = {v, u_stride, v_stride, conv_state, taps, conv_bias, K, vec_dtype, x_conv, gated, new_conv_state};
+  return fwd_impl(u, prep, h0, flags, y, h_last, ws, B, T, W, nb, dtype, true, stream, nullptr, &blk);
 }
 
 static int check_grad_dtype(const char* who, int grad_dtype) {
@@ -2935,7 +3159,8 @@ int rglru_hip_bwd_wide(const void* x, const void* prep, const float* h0,
 }
 
 static int step_impl(const void* x, const void* prep, const float* h_in, float* h, const uint8_t* flags,
-                     const void* gate_v, void* y, int64_t B, int64_t W, int64_t nb, int dtype, void* stream) {
+                     const void* gate_v, int64_t gate_stride, void* y, int64_t B, int64_t W, int64_t nb, int dtype,
+                     void* stream) {
   int rc = check_geometry("step", W, nb, dtype);
   if (rc) return rc;
   if (B <= 0) return fail(RGLRU_E_ARG, "step: B must be positive (got %lld)", (long long)B);
@@ -2945,7 +3170,9 @@ static int step_impl(const void* x, const void* prep, const float* h_in, float* 
   FusedArgs a;
   memset(&a, 0, sizeof(a));
   fill_common(a, g, prep, dtype);
-  a.x = x; a.flags = flags; a.y = y; a.h_state = h; a.h_prev = h_in; a.gate_v = gate_v;
+  if (gate_stride == 0) gate_stride = W;
+  if (gate_v && gate_stride < W) return fail(RGLRU_E_ARG, "step: row stride %lld of the gate input is smaller than the width %lld", (long long)gate_stride, (long long)W);
+  a.x = x; a.flags = flags; a.y = y; a.h_state = h; a.h_prev = h_in; a.gate_v = gate_v; a.ld_gate = gate_stride;
   a.B = (int)B; a.T = 1;
   a.aligned = is_aligned(x, W, g.bw, elem_size(dtype));
   long long row_tiles = (B + 31) / 32;
@@ -2974,12 +3201,13 @@ static int step_impl(const void* x, const void* prep, const float* h_in, float* 
 
 int rglru_hip_step(const void* x, const void* prep, float* h, const uint8_t* flags, void* y,
                    int64_t B, int64_t W, int64_t nb, int dtype, void* stream) {
-  return step_impl(x, prep, h, h, flags, nullptr, y, B, W, nb, dtype, stream);
+  return step_impl(x, prep, h, h, flags, nullptr, 0, y, B, W, nb, dtype, stream);
 }
 
 int rglru_hip_step_gated(const void* x, const void* prep, const float* h_in, float* h_out, const uint8_t* flags,
-                         const void* v, void* out, int64_t B, int64_t W, int64_t nb, int dtype, void* stream) {
-  return step_impl(x, prep, h_in, h_out, flags, v, out, B, W, nb, dtype, stream);
+                         const void* v, int64_t v_stride, void* out, int64_t B, int64_t W, int64_t nb, int dtype,
+                         void* stream) {
+  return step_impl(x, prep, h_in, h_out, flags, v, v_stride, out, B, W, nb, dtype, stream);
 }
 
 int rglru_hip_steps(const void* x, const void* prep, float* h, const uint8_t* flags, void* y,

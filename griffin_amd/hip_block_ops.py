@@ -13,7 +13,8 @@ from torch import Tensor
 from torch.autograd.function import once_differentiable
 
 from . import _lib
-from .hip_scan import _DTYPE_CODES, _dtype_code, _on_device, _ptr, _require_gpu, _stream_ptr
+from .hip_scan import (_DTYPE_CODES, _dtype_code, _on_device, _parameter_operands, _prep_bytes, _ptr, _require_gpu,
+                       _stream_ptr, rglru_backward)
 
 
 def max_kernel_size() -> int:
@@ -69,35 +70,41 @@ class _HipCausalConv(torch.autograd.Function):
     @staticmethod
     @once_differentiable
     def backward(ctx, dout: Tensor | None):
-        u, state, taps, pos = ctx.saved_tensors
-        state_dtype, weight_dtype, bias_dtype, weight_shape = ctx.meta
         if dout is None:
             return None, None, None, None, None
-        batch, steps, width = u.shape
-        taps_count = weight_shape[2]
-        code = _dtype_code(u.dtype)
-        dout_c = dout.to(u.dtype).contiguous()
-        lib = _lib.load()
-        need_u, need_state, need_w, need_b = ctx.needs_input_grad[:4]
-        grad_dtype = taps.dtype
-        du = torch.empty_like(u)
-        dstate = torch.empty_like(state) if (need_state and state is not None) else None
-        dtaps = torch.empty(width, taps_count, device=u.device, dtype=grad_dtype) if need_w else None
-        dbias = torch.empty(width, device=u.device, dtype=grad_dtype) if (need_b and bias_dtype is not None) else None
-        scratch = torch.empty(lib.rglru_hip_conv_scratch_bytes(batch, steps, width, taps_count),
-                              device=u.device, dtype=torch.uint8)
-        with _on_device(u.device):
-            _lib.check(lib.rglru_hip_conv_bwd(
-                _ptr(u), _ptr(state), _ptr(taps), _ptr(pos), _ptr(dout_c), _ptr(scratch), _ptr(du),
-                _ptr(dstate), _ptr(dtaps), _ptr(dbias),
-                batch, steps, width, taps_count, code, _DTYPE_CODES[taps.dtype], _DTYPE_CODES[grad_dtype],
-                _stream_ptr(u.device)), "rglru_hip_conv_bwd")
-        dweight = None if dtaps is None else dtaps.view(weight_shape).to(weight_dtype)
-        if dbias is not None:
-            dbias = dbias.to(bias_dtype)
-        if need_state and state_dtype is not None:
-            dstate = (u.new_zeros(batch, taps_count - 1, width) if dstate is None else dstate).to(state_dtype)
-        return (du if need_u else None), dstate, dweight, dbias, None
+        u, state, taps, pos = ctx.saved_tensors
+        return (*_conv_backward(u, state, taps, pos, dout, ctx.meta, ctx.needs_input_grad[:4]), None)
+
+
+def _conv_backward(u: Tensor, state: Tensor | None, taps: Tensor, pos: Tensor, dout: Tensor, meta, needs):
+    """Reverse mode of the dense convolution on contiguous operands: (du, dstate, dweight, dbias) in the types
+    of the forward's arguments; ``meta`` = (state dtype, weight dtype, bias dtype, weight shape)."""
+    state_dtype, weight_dtype, bias_dtype, weight_shape = meta
+    batch, steps, width = u.shape
+    taps_count = weight_shape[2]
+    code = _dtype_code(u.dtype)
+    dout_c = dout.to(u.dtype).contiguous()
+    lib = _lib.load()
+    need_u, need_state, need_w, need_b = needs
+    grad_dtype = taps.dtype
+    du = torch.empty_like(u)
+    dstate = torch.empty_like(state) if (need_state and state is not None) else None
+    dtaps = torch.empty(width, taps_count, device=u.device, dtype=grad_dtype) if need_w else None
+    dbias = torch.empty(width, device=u.device, dtype=grad_dtype) if (need_b and bias_dtype is not None) else None
+    scratch = torch.empty(lib.rglru_hip_conv_scratch_bytes(batch, steps, width, taps_count),
+                          device=u.device, dtype=torch.uint8)
+    with _on_device(u.device):
+        _lib.check(lib.rglru_hip_conv_bwd(
+            _ptr(u), _ptr(state), _ptr(taps), _ptr(pos), _ptr(dout_c), _ptr(scratch), _ptr(du),
+            _ptr(dstate), _ptr(dtaps), _ptr(dbias),
+            batch, steps, width, taps_count, code, _DTYPE_CODES[taps.dtype], _DTYPE_CODES[grad_dtype],
+            _stream_ptr(u.device)), "rglru_hip_conv_bwd")
+    dweight = None if dtaps is None else dtaps.view(weight_shape).to(weight_dtype)
+    if dbias is not None:
+        dbias = dbias.to(bias_dtype)
+    if need_state and state_dtype is not None:
+        dstate = (u.new_zeros(batch, taps_count - 1, width) if dstate is None else dstate).to(state_dtype)
+    return (du if need_u else None), dstate, dweight, dbias
 
 
 def hip_causal_conv(u: Tensor, state: Tensor | None, weight: Tensor, bias: Tensor | None,
@@ -244,12 +251,146 @@ def hip_gelu_gate(h: Tensor, v: Tensor) -> Tensor:
     return _HipGeluGate.apply(h, v)
 
 
+def hip_block_forward_covers(width: int, blocks: int, taps_count: int, dtype: torch.dtype) -> bool:
+    """Whether ``hip_block_forward`` has a kernel for this shape (rglru_hip_block_fwd_path)."""
+    if dtype not in _DTYPE_CODES or blocks <= 0 or width % blocks:
+        return False
+    return bool(_lib.load().rglru_hip_block_fwd_path(width, blocks, taps_count, _DTYPE_CODES[dtype]))
+
+
+def _row_view(t: Tensor) -> Tensor:
+    """[B, T, W] as the library addresses it: channels contiguous, one row stride for all tokens."""
+    batch, steps, width = t.shape
+    if t.stride(2) == 1 and t.stride(1) >= width and (batch == 1 or t.stride(0) == steps * t.stride(1)) \
+            and (t.stride(1) * t.element_size()) % 16 == 0 and t.data_ptr() % 16 == 0:
+        return t
+    return t.contiguous()
+
+
+class _HipBlockForward(torch.autograd.Function):
+    """conv -> RG-LRU -> output gate of the recurrent block in one forward launch (rglru_hip_block_fwd); the
+    backward pass runs the three reverse kernels one after the other on the x and y the forward kept."""
+
+    @staticmethod
+    def forward(ctx, u, v, conv_state, weight, bias, segment_pos, flags, w_a, b_a, w_x, b_x, lam, h0, c, prep):
+        _require_gpu("hip_block_forward", u, v, conv_state, weight, bias, segment_pos, w_a, b_a, w_x, b_x, lam, h0)
+        if u.dim() != 3 or u.shape != v.shape or u.dtype != v.dtype:
+            raise ValueError("hip_block_forward expects two [batch, sequence, width] tensors of one dtype")
+        B, T, W = u.shape
+        nb = w_a.shape[0]
+        taps_count = weight.size(2)
+        if weight.dim() != 3 or weight.size(0) != W or weight.size(1) != 1:
+            raise ValueError("weight must be that of a depthwise Conv1d: [width, 1, kernel_size]")
+        if conv_state is not None and conv_state.shape != (B, taps_count - 1, W):
+            raise ValueError("conv_state must have shape [batch, kernel_size - 1, width]")
+        if segment_pos.shape != (B, T):
+            raise ValueError("segment_pos must have shape [batch, sequence]")
+        if h0 is not None and h0.shape != (B, W):
+            raise ValueError(f"initial state must have shape ({B}, {W}), got {tuple(h0.shape)}")
+        if flags is not None and (flags.shape != (B, T) or flags.dtype != torch.uint8 or not flags.is_contiguous()):
+            raise ValueError("flags must be a contiguous uint8 tensor of shape [batch, sequence]")
+        code = _dtype_code(u.dtype)
+        lib = _lib.load()
+        training = any(ctx.needs_input_grad)
+        u_r, v_r = _row_view(u), _row_view(v)
+        state_c = None if conv_state is None or taps_count == 1 else conv_state.to(u.dtype).contiguous()
+        taps = _parameter_operand(weight.detach(), u.dtype)
+        bias_c = None if bias is None else _parameter_operand(bias.detach().to(taps.dtype), u.dtype)
+        pos = segment_pos.to(device=u.device, dtype=torch.int64).contiguous()
+        h0c = None if h0 is None else h0.detach().to(torch.float32).contiguous()
+        device = u.device
+        with _on_device(device):
+            stream = _stream_ptr(device)
+            if flags is None:
+                flags = hip_block_flags(pos)
+            gated = u.new_empty(B, T, W)
+            x_conv = u.new_empty(B, T, W) if training else None
+            y = u.new_empty(B, T, W) if training else None
+            new_conv = u.new_empty(B, taps_count - 1, W)
+            h_last = torch.empty(B, W, dtype=torch.float32, device=device)
+            ws = torch.empty(lib.rglru_hip_workspace_bytes(B, T, W, nb), dtype=torch.uint8, device=device)
+            tail = (_ptr(h0c), _ptr(flags), _ptr(x_conv), _ptr(y), _ptr(gated), _ptr(new_conv) if taps_count > 1 else None,
+                    _ptr(h_last), _ptr(ws), B, T, W, nb, code, stream)
+            if training or prep is None:
+                operands, vec_code = _parameter_operands(w_a, b_a, w_x, b_x, lam, u.dtype)
+                image = torch.empty(_prep_bytes(W, nb, code), dtype=torch.uint8, device=device)
+                _lib.check(lib.rglru_hip_prepare_block_fwd(
+                    *(t.data_ptr() for t in operands), float(c), vec_code, image.data_ptr(),
+                    _ptr(u_r), u_r.stride(1), _ptr(v_r), v_r.stride(1), _ptr(state_c), _ptr(taps), _ptr(bias_c), taps_count,
+                    *tail), "rglru_hip_prepare_block_fwd")
+            else:
+                image = prep.image
+                _lib.check(lib.rglru_hip_block_fwd(
+                    _ptr(u_r), u_r.stride(1), _ptr(v_r), v_r.stride(1), _ptr(state_c), _ptr(taps), _ptr(bias_c), taps_count,
+                    _DTYPE_CODES[taps.dtype], image.data_ptr(), *tail), "rglru_hip_block_fwd")
+        if training:
+            ctx.save_for_backward(u_r, v_r, state_c, taps, pos, x_conv, y, w_a, w_x, h0c, flags, ws, image)
+            ctx.conv_meta = (None if conv_state is None else conv_state.dtype, weight.dtype,
+                             None if bias is None else bias.dtype, weight.shape)
+            ctx.param_dtypes = (w_a.dtype, b_a.dtype, w_x.dtype, b_x.dtype, lam.dtype)
+            ctx.h0_dtype = None if h0 is None else h0.dtype
+        ctx.mark_non_differentiable(new_conv)
+        ctx.set_materialize_grads(False)
+        return gated, h_last, new_conv
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, dgated, dh_last, _dnew_conv):
+        u, v, state, taps, pos, x_conv, y, w_a, w_x, h0c, flags, ws, image = ctx.saved_tensors
+        need = ctx.needs_input_grad
+        lib = _lib.load()
+        dy = dv = None
+        if dgated is not None:
+            dout_c = dgated.to(y.dtype).contiguous()
+            v_c = v.contiguous()
+            dy, dv = torch.empty_like(y), torch.empty_like(v_c)
+            with _on_device(y.device):
+                _lib.check(lib.rglru_hip_gelu_gate_bwd(
+                    _ptr(dout_c), _ptr(y), _ptr(v_c), _ptr(dy), _ptr(dv), y.numel(), _dtype_code(y.dtype),
+                    _stream_ptr(y.device)), "rglru_hip_gelu_gate_bwd")
+        dx, dw_a, db_a, dw_x, db_x, dlam, dh0 = rglru_backward(
+            x_conv, y, w_a, w_x, h0c, flags, ws, image, dy, dh_last, ctx.param_dtypes, need[12])
+        u_c = u.contiguous()
+        du, dstate, dweight, dbias = _conv_backward(u_c, state, taps, pos, dx, ctx.conv_meta, (need[0], need[2], need[3], need[4]))
+        return (du, dv if need[1] else None, dstate, dweight, dbias, None, None, dw_a, db_a, dw_x, db_x, dlam,
+                None if dh0 is None else dh0.to(ctx.h0_dtype), None, None)
+
+
+def hip_block_flags(segment_pos: Tensor) -> Tensor:
+    """Per-token flag bytes of ``hip_block_forward`` for integer positions [B, T] (rglru_hip_block_flags):
+    reset where a document starts (position 0) and, in bits 2-3, how many convolution lags reach in front
+    of the token's document."""
+    _require_gpu("hip_block_flags", segment_pos)
+    pos = segment_pos.to(torch.int64).contiguous()
+    flags = torch.empty(pos.shape, dtype=torch.uint8, device=pos.device)
+    if pos.numel():
+        with _on_device(pos.device):
+            _lib.check(_lib.load().rglru_hip_block_flags(_ptr(pos), _ptr(flags), pos.numel(), _stream_ptr(pos.device)),
+                       "rglru_hip_block_flags")
+    return flags
+
+
+def hip_block_forward(u: Tensor, v: Tensor, conv_state: Tensor | None, weight: Tensor, bias: Tensor | None,
+                      segment_pos: Tensor, flags: Tensor | None, w_a: Tensor, b_a: Tensor, w_x: Tensor, b_x: Tensor,
+                      lam: Tensor, h0: Tensor | None, c: float = 8.0, prep=None):
+    """``gelu_tanh(v) * RG_LRU(conv(u))`` for whole sequences with every token active, one forward launch.
+
+    ``u``, ``v`` [B, T, W]: the block's two projections; ``conv_state`` [B, K-1, W] or None; ``weight``
+    [W, 1, K], ``bias`` [W] of the depthwise ``nn.Conv1d`` (K <= 4); ``segment_pos`` [B, T]; ``flags``:
+    ``hip_block_flags(segment_pos)`` if the caller has it already, else None; the five RG-LRU parameters, ``h0`` [B, W] or None; ``prep``: a prepared parameter image to use
+    when no gradient is asked for.  Returns ``(gated [B, T, W], final state [B, W] fp32, new_conv_state
+    [B, K-1, W])``; differentiable in u, v, the parameters, conv_state and h0 (not through new_conv_state).
+    """
+    return _HipBlockForward.apply(u, v, conv_state, weight, bias, segment_pos, flags, w_a, b_a, w_x, b_x, lam, h0, c, prep)
+
+
 def hip_block_decode_step(u: Tensor, v: Tensor, conv_state: Tensor | None, weight: Tensor, bias: Tensor | None,
                           prev_pos: Tensor | None, segment_pos: Tensor | None, active: Tensor | None,
                           prep, rnn_state: Tensor | None):
     """One token per row through conv -> RG-LRU step -> output gate (no autograd), two kernel launches.
 
-    ``u``, ``v`` [B, W]: the block's two projections of the token; ``conv_state`` [B, K-1, W] or None;
+    ``u``, ``v`` [B, W]: the block's two projections of the token (rows may be strided views of one wider
+    buffer); ``conv_state`` [B, K-1, W] or None;
     ``prev_pos`` [B] (None: -1) or explicit ``segment_pos`` [B]; ``active`` [B] uint8 or None (all
     active); ``prep`` the prepared RG-LRU parameters; ``rnn_state`` [B, W] fp32 or None (zeros).
     Returns ``(gated [B, W], new_rnn_state, new_conv_state, new_pos)``; the inputs are left untouched.
@@ -262,29 +403,31 @@ def hip_block_decode_step(u: Tensor, v: Tensor, conv_state: Tensor | None, weigh
         raise ValueError("the prepared RG-LRU parameters do not match the activations")
     taps_count = weight.size(2)
     code = _dtype_code(u.dtype)
-    u_c, v_c = u.contiguous(), v.contiguous()
+    # rows may be views into a wider buffer (the two halves of one fused projection)
+    u_c = u if u.stride(1) == 1 and u.stride(0) >= width else u.contiguous()
+    v_c = v if v.stride(1) == 1 and v.stride(0) >= width else v.contiguous()
     state_c = None if conv_state is None or taps_count == 1 else conv_state.to(u.dtype).contiguous()
     taps = _parameter_operand(weight.detach(), u.dtype)
     bias_c = None if bias is None else _parameter_operand(bias.detach().to(taps.dtype), u.dtype)
     device = u.device
     lib = _lib.load()
     with _on_device(device):
-        x_conv = torch.empty_like(u_c)
+        x_conv = u.new_empty(batch, width)
         new_conv = u.new_empty(batch, taps_count - 1, width)
         new_pos = torch.empty(batch, dtype=torch.int64, device=device)
         flags = torch.empty(batch, dtype=torch.uint8, device=device)
         h_in = (torch.zeros(batch, width, dtype=torch.float32, device=device) if rnn_state is None
                 else rnn_state.to(torch.float32).contiguous())
         h_out = torch.empty_like(h_in)
-        out = torch.empty_like(u_c)
+        out = u.new_empty(batch, width)
         stream = _stream_ptr(device)
         _lib.check(lib.rglru_hip_decode_prepare(
-            _ptr(u_c), _ptr(state_c), _ptr(taps), _ptr(bias_c), _ptr(prev_pos), _ptr(segment_pos), _ptr(active),
+            _ptr(u_c), u_c.stride(0), _ptr(state_c), _ptr(taps), _ptr(bias_c), _ptr(prev_pos), _ptr(segment_pos), _ptr(active),
             _ptr(x_conv), _ptr(new_conv) if taps_count > 1 else None, _ptr(new_pos), _ptr(flags),
             batch, width, taps_count, code, _DTYPE_CODES[taps.dtype], stream), "rglru_hip_decode_prepare")
         _lib.check(lib.rglru_hip_step_gated(
-            _ptr(x_conv), prep.image.data_ptr(), _ptr(h_in), _ptr(h_out), _ptr(flags), _ptr(v_c), _ptr(out),
-            batch, width, prep.blocks, code, stream), "rglru_hip_step_gated")
+            _ptr(x_conv), prep.image.data_ptr(), _ptr(h_in), _ptr(h_out), _ptr(flags), _ptr(v_c), v_c.stride(0),
+            _ptr(out), batch, width, prep.blocks, code, stream), "rglru_hip_step_gated")
     return out, h_out, new_conv, new_pos
 
 

@@ -295,82 +295,89 @@ class _HipRGLRU(torch.autograd.Function):
     @once_differentiable
     def backward(ctx, dy, dh_last):
         x, w_a, w_x, h0c, flags, ws, image, y = ctx.saved_tensors
-        lib = _lib.load()
-        B, T, W = x.shape
-        nb, bw, _ = w_a.shape
-        code = _dtype_code(x.dtype)
-        device = x.device
-        dy = torch.zeros_like(x) if dy is None else dy.to(x.dtype).contiguous()
-        dhl = None if dh_last is None else dh_last.to(torch.float32).contiguous()
-        # parameter gradients come back in the parameters' own type when all five share one the
-        # library writes (fp32 or bf16); otherwise in fp32, converted below
-        pd = ctx.param_dtypes
-        gdt = pd[0] if (len(set(pd)) == 1 and pd[0] in _DTYPE_CODES) else torch.float32
-        gcode = _DTYPE_CODES[gdt]
-        with _on_device(device):
-            dx = torch.empty_like(x)
-            db_a = torch.empty(nb, bw, dtype=gdt, device=device)
-            db_x = torch.empty(nb, bw, dtype=gdt, device=device)
-            dlam = torch.empty(W, dtype=gdt, device=device)
-            dh0 = torch.empty(B, W, dtype=torch.float32, device=device) if ctx.needs_input_grad[6] else None
-            # scratch of this call only (the workspace kept since forward holds just checkpoints and records)
-            scratch = torch.empty(lib.rglru_hip_bwd_scratch_bytes(B, T, W, nb, code), dtype=torch.uint8, device=device)
-            if (lib.rglru_hip_fast_path(W, nb, code) and dy.data_ptr() % 16 == 0 and x.data_ptr() % 16 == 0
-                    and y.data_ptr() % 16 == 0):
-                # everything in hand-written kernels, including the two gate GEMMs
-                dw_a = torch.empty(nb, bw, bw, dtype=gdt, device=device)
-                dw_x = torch.empty(nb, bw, bw, dtype=gdt, device=device)
-                _lib.check(lib.rglru_hip_bwd_full(x.data_ptr(), y.data_ptr(), image.data_ptr(), _ptr(h0c), _ptr(flags),
-                                                  dy.data_ptr(), _ptr(dhl), ws.data_ptr(), scratch.data_ptr(), dx.data_ptr(), dw_a.data_ptr(),
-                                                  dw_x.data_ptr(), db_a.data_ptr(), db_x.data_ptr(), dlam.data_ptr(),
-                                                  _ptr(dh0), B, T, W, nb, code, gcode, _stream_ptr(device)),
-                           "rglru_hip_bwd_full")
-            elif lib.rglru_hip_wide_path(W, nb, code) and dy.data_ptr() % 16 == 0 and x.data_ptr() % 16 == 0:
-                # blocks of 160 .. 384 channels: scan and gate math, then the two gate GEMMs, all hand-written
-                dw_a = torch.empty(nb, bw, bw, dtype=gdt, device=device)
-                dw_x = torch.empty(nb, bw, bw, dtype=gdt, device=device)
-                _lib.check(lib.rglru_hip_bwd_wide(x.data_ptr(), image.data_ptr(), _ptr(h0c), _ptr(flags),
-                                                  dy.data_ptr(), _ptr(dhl), ws.data_ptr(), scratch.data_ptr(), dx.data_ptr(), dw_a.data_ptr(),
-                                                  dw_x.data_ptr(), db_a.data_ptr(), db_x.data_ptr(), dlam.data_ptr(),
-                                                  _ptr(dh0), B, T, W, nb, code, gcode, _stream_ptr(device)),
-                           "rglru_hip_bwd_wide")
-            elif _uses_pre_path(lib, x, W, nb, code) and dy.data_ptr() % 16 == 0:
-                # gate projections recomputed by the library GEMM, the scan and all gate math in the
-                # HIP kernel, then the two GEMMs of the gate gradients on the kernel's du
-                pre, stacked, xk = _gate_projections(x, w_a, w_x)
-                du = torch.empty_like(pre)
-                _lib.check(lib.rglru_hip_bwd_pre(x.data_ptr(), pre.data_ptr(), image.data_ptr(), _ptr(h0c), _ptr(flags),
-                                                 dy.data_ptr(), _ptr(dhl), ws.data_ptr(), scratch.data_ptr(), dx.data_ptr(),
-                                                 du.data_ptr(), db_a.data_ptr(), db_x.data_ptr(), dlam.data_ptr(),
-                                                 _ptr(dh0), B, T, W, nb, code, gcode, _stream_ptr(device)),
-                           "rglru_hip_bwd_pre")
-                del pre
-                dw = torch.bmm(du.transpose(1, 2), xk)                 # [nb, 2 bw, bw] = [dW_a ; dW_x]
-                dw_a, dw_x = dw[:, :bw], dw[:, bw:]
-                dx_blocks = dx.view(B * T, nb, bw).transpose(0, 1)     # [nb, n, bw], row stride W: written in place
-                torch.baddbmm(dx_blocks, du, stacked, out=dx_blocks)
-            else:
-                du_a = torch.empty_like(x)
-                du_x = torch.empty_like(x)
-                _lib.check(lib.rglru_hip_bwd(x.data_ptr(), image.data_ptr(), _ptr(h0c), _ptr(flags),
-                                             dy.data_ptr(), _ptr(dhl), ws.data_ptr(), scratch.data_ptr(), dx.data_ptr(), du_a.data_ptr(),
-                                             du_x.data_ptr(), db_a.data_ptr(), db_x.data_ptr(), dlam.data_ptr(),
-                                             _ptr(dh0), B, T, W, nb, code, gcode, _stream_ptr(device)), "rglru_hip_bwd")
-                # block-diagonal library GEMMs: dW[k] = du[:, k]^T x[:, k];  dx[:, k] += du[:, k] W[k]
-                n = B * T
-                xk = x.view(n, nb, bw).transpose(0, 1)               # [nb, n, bw] (strided view)
-                ua = du_a.view(n, nb, bw).transpose(0, 1)
-                ux = du_x.view(n, nb, bw).transpose(0, 1)
-                wa = w_a.detach().to(x.dtype)
-                wx = w_x.detach().to(x.dtype)
-                dw_a = torch.bmm(ua.transpose(1, 2), xk)
-                dw_x = torch.bmm(ux.transpose(1, 2), xk)
-                dx_blocks = dx.view(n, nb, bw).transpose(0, 1)       # [nb, n, bw], row stride W: written in place
-                torch.baddbmm(dx_blocks, ua, wa, out=dx_blocks)
-                torch.baddbmm(dx_blocks, ux, wx, out=dx_blocks)
-        grads = (dx, dw_a.to(pd[0]), db_a.to(pd[1]), dw_x.to(pd[2]), db_x.to(pd[3]),
-                 dlam.to(pd[4]), None if dh0 is None else dh0.to(ctx.h0_dtype), None, None)
-        return grads
+        dx, dw_a, db_a, dw_x, db_x, dlam, dh0 = rglru_backward(
+            x, y, w_a, w_x, h0c, flags, ws, image, dy, dh_last, ctx.param_dtypes, ctx.needs_input_grad[6])
+        return (dx, dw_a, db_a, dw_x, db_x, dlam, None if dh0 is None else dh0.to(ctx.h0_dtype), None, None)
+
+
+def rglru_backward(x, y, w_a, w_x, h0c, flags, ws, image, dy, dh_last, param_dtypes, need_dh0):
+    """Backward pass of the RG-LRU on what its forward kept (the workspace with checkpoints and records, the
+    parameter image): returns (dx, dW_a, db_a, dW_x, db_x, dLambda, dh0 in fp32 or None), the parameter
+    gradients in the parameters' types."""
+    lib = _lib.load()
+    B, T, W = x.shape
+    nb, bw, _ = w_a.shape
+    code = _dtype_code(x.dtype)
+    device = x.device
+    dy = torch.zeros_like(x) if dy is None else dy.to(x.dtype).contiguous()
+    dhl = None if dh_last is None else dh_last.to(torch.float32).contiguous()
+    # parameter gradients come back in the parameters' own type when all five share one the
+    # library writes (fp32 or bf16); otherwise in fp32, converted below
+    pd = param_dtypes
+    gdt = pd[0] if (len(set(pd)) == 1 and pd[0] in _DTYPE_CODES) else torch.float32
+    gcode = _DTYPE_CODES[gdt]
+    with _on_device(device):
+        dx = torch.empty_like(x)
+        db_a = torch.empty(nb, bw, dtype=gdt, device=device)
+        db_x = torch.empty(nb, bw, dtype=gdt, device=device)
+        dlam = torch.empty(W, dtype=gdt, device=device)
+        dh0 = torch.empty(B, W, dtype=torch.float32, device=device) if need_dh0 else None
+        # scratch of this call only (the workspace kept since forward holds just checkpoints and records)
+        scratch = torch.empty(lib.rglru_hip_bwd_scratch_bytes(B, T, W, nb, code), dtype=torch.uint8, device=device)
+        if (lib.rglru_hip_fast_path(W, nb, code) and dy.data_ptr() % 16 == 0 and x.data_ptr() % 16 == 0
+                and y.data_ptr() % 16 == 0):
+            # everything in hand-written kernels, including the two gate GEMMs
+            dw_a = torch.empty(nb, bw, bw, dtype=gdt, device=device)
+            dw_x = torch.empty(nb, bw, bw, dtype=gdt, device=device)
+            _lib.check(lib.rglru_hip_bwd_full(x.data_ptr(), y.data_ptr(), image.data_ptr(), _ptr(h0c), _ptr(flags),
+                                              dy.data_ptr(), _ptr(dhl), ws.data_ptr(), scratch.data_ptr(), dx.data_ptr(), dw_a.data_ptr(),
+                                              dw_x.data_ptr(), db_a.data_ptr(), db_x.data_ptr(), dlam.data_ptr(),
+                                              _ptr(dh0), B, T, W, nb, code, gcode, _stream_ptr(device)),
+                       "rglru_hip_bwd_full")
+        elif lib.rglru_hip_wide_path(W, nb, code) and dy.data_ptr() % 16 == 0 and x.data_ptr() % 16 == 0:
+            # blocks of 160 .. 384 channels: scan and gate math, then the two gate GEMMs, all hand-written
+            dw_a = torch.empty(nb, bw, bw, dtype=gdt, device=device)
+            dw_x = torch.empty(nb, bw, bw, dtype=gdt, device=device)
+            _lib.check(lib.rglru_hip_bwd_wide(x.data_ptr(), image.data_ptr(), _ptr(h0c), _ptr(flags),
+                                              dy.data_ptr(), _ptr(dhl), ws.data_ptr(), scratch.data_ptr(), dx.data_ptr(), dw_a.data_ptr(),
+                                              dw_x.data_ptr(), db_a.data_ptr(), db_x.data_ptr(), dlam.data_ptr(),
+                                              _ptr(dh0), B, T, W, nb, code, gcode, _stream_ptr(device)),
+                       "rglru_hip_bwd_wide")
+        elif _uses_pre_path(lib, x, W, nb, code) and dy.data_ptr() % 16 == 0:
+            # gate projections recomputed by the library GEMM, the scan and all gate math in the
+            # HIP kernel, then the two GEMMs of the gate gradients on the kernel's du
+            pre, stacked, xk = _gate_projections(x, w_a, w_x)
+            du = torch.empty_like(pre)
+            _lib.check(lib.rglru_hip_bwd_pre(x.data_ptr(), pre.data_ptr(), image.data_ptr(), _ptr(h0c), _ptr(flags),
+                                             dy.data_ptr(), _ptr(dhl), ws.data_ptr(), scratch.data_ptr(), dx.data_ptr(),
+                                             du.data_ptr(), db_a.data_ptr(), db_x.data_ptr(), dlam.data_ptr(),
+                                             _ptr(dh0), B, T, W, nb, code, gcode, _stream_ptr(device)),
+                       "rglru_hip_bwd_pre")
+            del pre
+            dw = torch.bmm(du.transpose(1, 2), xk)                 # [nb, 2 bw, bw] = [dW_a ; dW_x]
+            dw_a, dw_x = dw[:, :bw], dw[:, bw:]
+            dx_blocks = dx.view(B * T, nb, bw).transpose(0, 1)     # [nb, n, bw], row stride W: written in place
+            torch.baddbmm(dx_blocks, du, stacked, out=dx_blocks)
+        else:
+            du_a = torch.empty_like(x)
+            du_x = torch.empty_like(x)
+            _lib.check(lib.rglru_hip_bwd(x.data_ptr(), image.data_ptr(), _ptr(h0c), _ptr(flags),
+                                         dy.data_ptr(), _ptr(dhl), ws.data_ptr(), scratch.data_ptr(), dx.data_ptr(), du_a.data_ptr(),
+                                         du_x.data_ptr(), db_a.data_ptr(), db_x.data_ptr(), dlam.data_ptr(),
+                                         _ptr(dh0), B, T, W, nb, code, gcode, _stream_ptr(device)), "rglru_hip_bwd")
+            # block-diagonal library GEMMs: dW[k] = du[:, k]^T x[:, k];  dx[:, k] += du[:, k] W[k]
+            n = B * T
+            xk = x.view(n, nb, bw).transpose(0, 1)               # [nb, n, bw] (strided view)
+            ua = du_a.view(n, nb, bw).transpose(0, 1)
+            ux = du_x.view(n, nb, bw).transpose(0, 1)
+            wa = w_a.detach().to(x.dtype)
+            wx = w_x.detach().to(x.dtype)
+            dw_a = torch.bmm(ua.transpose(1, 2), xk)
+            dw_x = torch.bmm(ux.transpose(1, 2), xk)
+            dx_blocks = dx.view(n, nb, bw).transpose(0, 1)       # [nb, n, bw], row stride W: written in place
+            torch.baddbmm(dx_blocks, ua, wa, out=dx_blocks)
+            torch.baddbmm(dx_blocks, ux, wx, out=dx_blocks)
+    return dx, dw_a.to(pd[0]), db_a.to(pd[1]), dw_x.to(pd[2]), db_x.to(pd[3]), dlam.to(pd[4]), dh0
 
 
 def hip_rglru(x: Tensor, w_a: Tensor, b_a: Tensor, w_x: Tensor, b_x: Tensor, lam: Tensor, c: float = 8.0,

@@ -217,6 +217,21 @@ def _default_positions(batch: int, steps: int, device: torch.device):
     return hit
 
 
+_DEFAULT_BLOCK_FLAGS: dict = {}
+
+
+def _default_block_flags(batch: int, steps: int, device: torch.device) -> Tensor | None:
+    """Flag bytes of the one-launch block forward for the default positions, built once like them (None
+    while a graph is being captured: the operator then derives them inside the capture)."""
+    key = (batch, steps, device)
+    hit = _DEFAULT_BLOCK_FLAGS.get(key)
+    if hit is None and not torch.cuda.is_current_stream_capturing():
+        if len(_DEFAULT_BLOCK_FLAGS) >= 16:
+            _DEFAULT_BLOCK_FLAGS.clear()
+        hit = _DEFAULT_BLOCK_FLAGS[key] = hip_block_ops.hip_block_flags(_default_positions(batch, steps, device)[0])
+    return hit
+
+
 def _resolve_segment_positions(x, segment_pos, previous_position=None, active_mask=None) -> Tensor:
     """Explicit positions, or previous + running count of active tokens (griffin/griffin.py:309-338)."""
     batch, steps = x.shape[:2]
@@ -324,6 +339,15 @@ class RecurrentBlock(nn.Module):
             return False
         return self.conv_kernel_size <= hip_block_ops.max_kernel_size()
 
+    def _hip_block_forward_covers(self, projected: Tensor, gate_input: Tensor, cache: RecurrentBlockCache | None) -> bool:
+        """The one-launch forward (convolution, RG-LRU, output gate) exists for this shape and these types."""
+        if gate_input.dtype != projected.dtype or gate_input.shape != projected.shape:
+            return False
+        if cache is not None and cache.rnn_state is not None and cache.rnn_state.shape != (projected.size(0), self.rnn_width):
+            return False                                     # the RG-LRU reports the shape error
+        return hip_block_ops.hip_block_forward_covers(self.rnn_width, self.rg_lru.recurrence_gate.weight.shape[0],
+                                                      self.conv_kernel_size, projected.dtype)
+
     def _hip_decode_covers(self, x: Tensor, cache: RecurrentBlockCache | None) -> bool:
         """Single-token inference takes the two-launch decode path of the HIP library."""
         if not x.is_cuda or x.dtype not in hip_scan.SUPPORTED_DTYPES or x.numel() == 0:
@@ -366,8 +390,7 @@ class RecurrentBlock(nn.Module):
         active = None
         if active_mask is not None and not bool(active_mask.all()):
             active = active_mask[:, 0].to(torch.uint8).contiguous()
-        gate_input = self.linear_y(x)[:, 0]
-        projected = self.linear_x(x)[:, 0]
+        projected, gate_input = self._decode_projections(x[:, 0])
         prep = self.rg_lru._prepared(projected.dtype, projected.device)
         gated, new_rnn_state, new_conv_state, new_pos = hip_block_ops.hip_block_decode_step(
             projected, gate_input, conv_state, self.temporal_conv.weight, self.temporal_conv.bias,
@@ -378,6 +401,26 @@ class RecurrentBlock(nn.Module):
         if return_cache:
             return output, RecurrentBlockCache(new_rnn_state, new_conv_state, new_pos)
         return output
+
+    def _decode_projections(self, token: Tensor):
+        """``linear_x`` and ``linear_y`` of one token per row as ONE GEMM against the two weights stacked
+        (the decode kernels take the halves of its output as strided rows).  The stacked copy is kept
+        until a weight or bias changes (storage or version counter)."""
+        layers = (self.linear_x, self.linear_y)
+        tensors = [t for layer in layers for t in (layer.weight, layer.bias) if t is not None]
+        key = tuple((t.data_ptr(), t._version, t.dtype, t.device) for t in tensors)
+        cached = getattr(self, "_stacked_projection", None)
+        if cached is None or cached[0] != key:
+            if len(tensors) != 4 or (token.is_cuda and torch.cuda.is_current_stream_capturing()):
+                # nothing allocated during a graph capture may outlive it: two GEMMs this time
+                return self.linear_x(token), self.linear_y(token)
+            with torch.no_grad():
+                weight = torch.cat([self.linear_x.weight, self.linear_y.weight], 0).contiguous()
+                bias = torch.cat([self.linear_x.bias, self.linear_y.bias], 0).contiguous()
+            cached = (key, weight, bias)
+            self._stacked_projection = cached
+        both = torch.nn.functional.linear(token, cached[1], cached[2])
+        return both[:, :self.rnn_width], both[:, self.rnn_width:]
 
     def _linear(self, layer: nn.Linear, x: Tensor) -> Tensor:
         """A Linear layer of the block; in training on the HIP path its bias gradient is summed by a
@@ -443,23 +486,36 @@ class RecurrentBlock(nn.Module):
         conv_state = (None if on_hip else self._empty_conv_state(projected)) if cache is None else cache.conv_state
         if conv_state is not None and conv_state.shape != (batch, self.conv_kernel_size - 1, self.rnn_width):
             raise ValueError("Recurrent convolution cache has an incompatible shape")
-        if everything_active or bool(active_mask.all()):
-            recurrent_in, new_conv_state = self._dense_conv(projected, conv_state, segment_pos, return_cache)
-        else:
-            recurrent_in, new_conv_state = self._padded_conv(projected, conv_state, segment_pos, active_mask)
-
+        dense = everything_active or bool(active_mask.all())
         default = _DEFAULT_POSITIONS.get((batch, steps, x.device))
-        recurrent_out, new_rnn_state = self.rg_lru(
-            recurrent_in,
-            None if cache is None else cache.rnn_state,
-            reset_mask=default[1] if (default is not None and segment_pos is default[0]) else segment_pos == 0,
-            active_mask=None if everything_active else active_mask,
-            return_state=True,
-        )
-        if self._hip_block_ops_covers(projected) and gate_input.dtype == recurrent_out.dtype:
-            gated = hip_block_ops.hip_gelu_gate(recurrent_out, gate_input)
+        if dense and on_hip and self._hip_block_forward_covers(projected, gate_input, cache):
+            # convolution, RG-LRU and output gate in one forward launch
+            rnn_state = None if cache is None else cache.rnn_state
+            needs_grad = torch.is_grad_enabled() and any(
+                t is not None and t.requires_grad
+                for t in (projected, gate_input, conv_state, rnn_state, self.temporal_conv.weight,
+                          self.temporal_conv.bias, *self.rg_lru._gate_parameters()))
+            gated, new_rnn_state, new_conv_state = hip_block_ops.hip_block_forward(
+                projected, gate_input, conv_state, self.temporal_conv.weight, self.temporal_conv.bias, segment_pos,
+                _default_block_flags(batch, steps, x.device) if (default is not None and segment_pos is default[0]) else None,
+                *self.rg_lru._gate_parameters(), rnn_state, self.rg_lru.c,
+                None if needs_grad else self.rg_lru._prepared(projected.dtype, projected.device))
         else:
-            gated = recurrent_out * F.gelu(gate_input, approximate="tanh")
+            if dense:
+                recurrent_in, new_conv_state = self._dense_conv(projected, conv_state, segment_pos, return_cache)
+            else:
+                recurrent_in, new_conv_state = self._padded_conv(projected, conv_state, segment_pos, active_mask)
+            recurrent_out, new_rnn_state = self.rg_lru(
+                recurrent_in,
+                None if cache is None else cache.rnn_state,
+                reset_mask=default[1] if (default is not None and segment_pos is default[0]) else segment_pos == 0,
+                active_mask=None if everything_active else active_mask,
+                return_state=True,
+            )
+            if on_hip and gate_input.dtype == recurrent_out.dtype:
+                gated = hip_block_ops.hip_gelu_gate(recurrent_out, gate_input)
+            else:
+                gated = recurrent_out * F.gelu(gate_input, approximate="tanh")
         output = self._linear(self.linear_out, gated)
         if not everything_active:
             output = output.masked_fill(~active_mask.unsqueeze(-1), 0.0)

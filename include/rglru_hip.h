@@ -18,6 +18,7 @@
  *   autograd of griffin/griffin.py:474-487                                   rglru_hip_conv_bwd
  *   griffin/griffin.py:488-510      the same over right-padded batches and its autograd   rglru_hip_conv_padded_fwd, _bwd
  *   griffin/griffin.py:464, :520    x_branch * gelu_tanh(linear_y(x))        rglru_hip_gelu_gate_fwd, _bwd
+ *   griffin/griffin.py:464-520      convolution, RG-LRU and output gate in one launch   rglru_hip_block_fwd, rglru_hip_prepare_block_fwd
  *   griffin/griffin.py:68-80        RMSNorm in front of the block and its autograd   rglru_hip_rmsnorm_fwd, _bwd
  *   griffin/griffin.py:459-528 with T == 1 (block decode: positions, conv, step, gate)   rglru_hip_decode_prepare + rglru_hip_step_gated
  *   autograd of the bias of griffin/griffin.py:379-389 (the block's Linear layers)      rglru_hip_colsum
@@ -49,7 +50,7 @@
 extern "C" {
 #endif
 
-#define RGLRU_ABI_VERSION 14
+#define RGLRU_ABI_VERSION 15
 
 enum { RGLRU_F32 = 0, RGLRU_BF16 = 1 };
 
@@ -62,6 +63,9 @@ enum {
 
 #define RGLRU_FLAG_RESET 1u
 #define RGLRU_FLAG_INACTIVE 2u
+/* Bits 2-3 of a flag byte are read by rglru_hip_block_fwd only (convolution lags that reach in front of the
+ * token's document); every other entry point ignores them. */
+#define RGLRU_FLAG_CONV_SHIFT 2
 
 /* Tokens per chunk of the backward scan (one carry record per sequence, chunk and channel).  Forward
  * stores the fp32 state after every RGLRU_CHUNK / 2 tokens and backward restarts its recomputation
@@ -301,13 +305,45 @@ int rglru_hip_colsum(const void* x, void* scratch, void* out, int64_t rows, int6
  *     document start clears the history, an inactive row keeps state and position, x = 0 for it.
  *   rglru_hip_step_gated: rglru_hip_step with the state read from h_in and written to h_out (the two
  *     may be the same buffer) and out[B,W] = h * gelu_tanh(v[B,W]) (v NULL: out = h), which is the
- *     operand of the block's output projection (:520). */
-int rglru_hip_decode_prepare(const void* u, const void* conv_state, const void* taps, const void* bias,
+ *     operand of the block's output projection (:520).
+ * u and v may be rows of a wider buffer (the two halves of one GEMM that computes both projections):
+ * u_stride and v_stride are the distances between their rows in elements, 0 meaning W. */
+int rglru_hip_decode_prepare(const void* u, int64_t u_stride, const void* conv_state, const void* taps, const void* bias,
                              const int64_t* prev_pos, const int64_t* segment_pos, const uint8_t* active,
                              void* x, void* new_conv_state, int64_t* new_pos, uint8_t* flags,
                              int64_t B, int64_t W, int64_t K, int dtype, int vec_dtype, void* stream);
 int rglru_hip_step_gated(const void* x, const void* prep, const float* h_in, float* h_out, const uint8_t* flags,
-                         const void* v, void* out, int64_t B, int64_t W, int64_t nb, int dtype, void* stream);
+                         const void* v, int64_t v_stride, void* out, int64_t B, int64_t W, int64_t nb, int dtype,
+                         void* stream);
+
+/* The recurrent block's forward between its projections in ONE launch (griffin/griffin.py:474-487, the
+ * RG-LRU of :97-286, and :464, :520): x = causal depthwise convolution of u[B,T,W] (taps[W][K], K <= 4,
+ * conv_bias[W] or NULL, both in vec_dtype; conv_state[B,K-1,W] or NULL = zeros in front of every row),
+ * y = RG-LRU(x) and gated[B,T,W] = y * gelu_tanh(v[B,T,W]).  u and v may be rows of wider buffers
+ * (u_stride, v_stride in elements, 0 = W).  Every token is active; the flag bytes carry, next to
+ * RGLRU_FLAG_RESET, in bits 2-3 how many convolution lags reach in front of the token's document,
+ * 3 - min(segment_pos, 3) (rglru_hip_block_flags writes them from segment_pos[n]); flags NULL means no
+ * document starts inside the rows and position >= K - 1 or an all-zero history at their beginning.
+ * Optional outputs (NULL to skip): x_conv[B,T,W] and y[B,T,W] (what a backward pass needs),
+ * new_conv_state[B,K-1,W], h_last[B,W].  ws as for rglru_hip_fwd.  Only where
+ * rglru_hip_block_fwd_path() returns 1 (bf16 storage, gate blocks of 32, 64 or 128 channels, 16-byte
+ * aligned rows); otherwise RGLRU_E_UNSUPPORTED, and the caller runs rglru_hip_conv_fwd, rglru_hip_fwd and
+ * rglru_hip_gelu_gate_fwd one after the other.  rglru_hip_prepare_block_fwd is rglru_hip_prepare +
+ * rglru_hip_block_fwd in two launches (as rglru_hip_prepare_fwd). */
+int rglru_hip_block_fwd_path(int64_t W, int64_t nb, int64_t K, int dtype);
+int rglru_hip_block_flags(const int64_t* segment_pos, uint8_t* flags, int64_t n, void* stream);
+int rglru_hip_block_fwd(const void* u, int64_t u_stride, const void* v, int64_t v_stride,
+                        const void* conv_state, const void* taps, const void* conv_bias, int64_t K, int vec_dtype,
+                        const void* prep, const float* h0, const uint8_t* flags,
+                        void* x_conv, void* y, void* gated, void* new_conv_state, float* h_last, void* ws,
+                        int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, void* stream);
+int rglru_hip_prepare_block_fwd(const void* w_a, const void* b_a, const void* w_x, const void* b_x,
+                                const void* lambda, float c, int vec_dtype, void* prep,
+                                const void* u, int64_t u_stride, const void* v, int64_t v_stride,
+                                const void* conv_state, const void* taps, const void* conv_bias, int64_t K,
+                                const float* h0, const uint8_t* flags,
+                                void* x_conv, void* y, void* gated, void* new_conv_state, float* h_last, void* ws,
+                                int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, void* stream);
 
 /* Test hook: number of polls a wave may spend waiting for a neighbouring chunk's carry before it
  * gives up, records the failure in the workspace and finishes with unspecified results.  The

@@ -556,3 +556,46 @@ def test_block_decode_with_padding_and_restart_matches_portable_block():
             torch.testing.assert_close(cache_h.rnn_state.cpu(), cache_c.rnn_state, atol=2e-5, rtol=2e-5)
             torch.testing.assert_close(cache_h.conv_state.cpu(), cache_c.conv_state, atol=1e-6, rtol=1e-6)
             assert torch.equal(cache_h.segment_position.cpu(), cache_c.segment_position), t
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("cfg", [(5, 64, 2, 0), (256, 1024, 8, 0), (3, 40, 1, 3), (7, 320, 1, 8)])
+def test_block_decode_step_takes_strided_rows(cfg, dtype):
+    """The decode kernels read their two projections as rows of a wider buffer (row strides through the
+    C ABI): results are bit-identical to the same call on contiguous copies, on the vector path
+    (16-byte-aligned strides) and on the element path (the padded buffers)."""
+    from griffin_amd import RG_LRU
+    from griffin_amd.hip_block_ops import hip_block_decode_step
+
+    B, W, nb, pad = cfg
+    torch.manual_seed(B + W)
+    rg = RG_LRU(W, gate_blocks=nb, scan_mode="hip").cuda().to(dtype)
+    prep = rg._prepared(dtype, torch.device("cuda", 0))
+    both = torch.randn(B, 2 * W + pad, device="cuda").to(dtype)
+    u, v = both[:, :W], both[:, W + pad:]
+    assert not u.is_contiguous() and not v.is_contiguous()
+    taps = (0.3 * torch.randn(W, 1, 4, device="cuda")).to(dtype)
+    bias = (0.1 * torch.randn(W, device="cuda")).to(dtype)
+    conv_state = torch.randn(B, 3, W, device="cuda").to(dtype)
+    prev_pos = torch.randint(-1, 5, (B,), device="cuda")
+    active = (torch.rand(B, device="cuda") < 0.8).to(torch.uint8)
+    h = torch.randn(B, W, device="cuda")
+    _say("strided decode rows", cfg, dtype)
+    got = hip_block_decode_step(u, v, conv_state, taps, bias, prev_pos, None, active, prep, h)
+    want = hip_block_decode_step(u.contiguous(), v.contiguous(), conv_state, taps, bias, prev_pos, None, active,
+                                 prep, h)
+    torch.cuda.synchronize()
+    for name, a, b in zip(("gated", "rnn_state", "conv_state", "position"), got, want):
+        assert torch.equal(a, b), name
+    assert got[0].is_contiguous() and got[0].shape == (B, W)
+
+
+def test_decode_row_stride_below_width_is_rejected():
+    """Row strides smaller than the width are argument errors (checked on the host, nothing is launched)."""
+    from griffin_amd import _lib
+
+    lib = _lib.load()
+    buf = torch.zeros(4096, device="cuda")
+    p = buf.data_ptr()
+    rc = lib.rglru_hip_decode_prepare(p, 16, None, p, None, None, None, None, p, p, p, p, 2, 32, 4, 0, 0, None)
+    assert rc != 0 and b"stride" in lib.rglru_hip_last_error()

@@ -268,3 +268,28 @@ def test_packed_flags_follow_in_place_updates_of_the_mask():
     assert b is not a and b.tolist() == [[1, 0, 0, 0, 0], [0, 0, 0, 1, 0]]
     both = pack_flags(mask, torch.ones(2, 5, dtype=torch.bool))
     assert both.tolist() == b.tolist()
+
+
+def test_stacked_decode_projection_follows_the_two_linear_layers():
+    """The one-GEMM form of linear_x / linear_y used by single-token decode (griffin/griffin.py:462-464)
+    returns what the two layers return, and is rebuilt when a weight or bias is written to."""
+    from griffin_amd import RecurrentBlock
+
+    torch.manual_seed(0)
+    block = RecurrentBlock(12, 16, gate_blocks=2, scan_mode="sequential")
+    token = torch.randn(5, 12)
+    with torch.no_grad():
+        px, py = block._decode_projections(token)
+        assert px.shape == py.shape == (5, 16) and px.stride(0) == 32
+        assert torch.allclose(px, block.linear_x(token), atol=1e-6)
+        assert torch.allclose(py, block.linear_y(token), atol=1e-6)
+        held = block._stacked_projection
+        block._decode_projections(token)
+        assert block._stacked_projection is held
+        block.linear_y.bias.add_(1.0)
+        block.linear_x.weight.mul_(2.0)
+        px, py = block._decode_projections(token)
+        assert block._stacked_projection is not held
+        assert torch.allclose(px, block.linear_x(token), atol=1e-6)
+        assert torch.allclose(py, block.linear_y(token), atol=1e-6)
+    assert "_stacked_projection" not in block.state_dict()
