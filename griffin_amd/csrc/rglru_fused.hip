@@ -162,6 +162,7 @@ struct FusedArgs {
   long long rows_total;                                   // B * T, the row count of one block of `pre`
   int nC, nCf, ckpt_nC, wg_per_unit, aligned, full_slabs, queues, flags_vec;
   int dw_bf16;                                            // fast backward: per-workgroup weight-gradient sums stored as bf16
+  int xcd_map;                                            // wide blocks: the workgroups that share a block's x tiles sit on one XCD
   long long limit;
 };
 
@@ -196,6 +197,16 @@ RGLRU_DEVICE WaveId wave_identity(const FusedArgs& p, int block) {
   WaveId w;
   w.lane = threadIdx.x & 63; w.r = w.lane & 31; w.hf = w.lane >> 5; w.wave = threadIdx.x >> 6;
   w.unit = block % p.units; w.wg_in_unit = block / p.units;
+  if (p.xcd_map) {
+    // Workgroups go to the eight XCDs round-robin by index and each XCD has its own L2.  The `groups` units
+    // of a wide block stage the same x tiles: index = xcd + 8 * slot keeps the members of a (block,
+    // workgroup number) pair in consecutive slots of one XCD, so the tile comes from memory once.  The grid
+    // is rounded up to whole rounds of eight pairs; a workgroup number past the end means "nothing to do".
+    const int xcd = block & 7, slot = block >> 3;
+    const int pair = xcd + 8 * (slot / p.groups);
+    w.unit = (pair % p.nb) * p.groups + slot % p.groups;
+    w.wg_in_unit = pair / p.nb;
+  }
   if (p.bpu > 1) {
     // packed: the unit covers bpu consecutive blocks of S slabs each (bpu * S = waves per workgroup)
     const int blk = w.wave / p.S, k = w.unit * p.bpu + blk;
@@ -500,6 +511,14 @@ RGLRU_DEVICE void fwd_finalize(const FusedArgs& p, const WaveId& w, const FwdTil
 // 32-token tiles with two tiles in flight at B8 T2048 W1024, 84 us against 104 us for one sequence of
 // 32768 tokens).
 constexpr int kFwdMT = 2;
+// ... except where a block wider than 128 channels needs the registers: each wave holds 8 NKG registers of
+// weights, and with one wave a SIMD nothing covers a tile's latency chain.  Measured per block width at
+// B1 T32768 and B4 T2048 (forward, ms; 64-token tiles and one workgroup a compute unit first):
+//   160: 0.185 -> 0.147, 192: 0.224 -> 0.161, 224: 0.199 -> 0.176 with 64-token tiles and two workgroups
+//   (224: 7 spilled registers); 288: 0.370 -> 0.302, 320: 0.390 -> 0.347 with 32-token tiles and two
+//   workgroups (320: 14 spilled registers); 256, 352, 384 are fastest as they were.
+constexpr int fwd_mt(int nkg) { return (nkg == 18 || nkg == 20) ? 1 : kFwdMT; }
+constexpr int fwd_wide_occ(int nkg) { return (nkg == 16 || nkg > 20) ? 1 : 2; }
 
 // workgroups per compute unit of the forward kernel without weights in registers (NKG < 0); 4 spills
 #define RGLRU_GIVEN_OCC 3
@@ -513,8 +532,8 @@ constexpr int kFwdMT = 2;
 // from LDS, lags masked per token through bits 2-3 of the flag bytes = 3 - min(position, 3)) and puts the
 // result where the plain kernel puts x; the store stage multiplies by gelu_tanh of the second projection.
 template <typename IO, int NKG, bool MASKED, bool BLOCK = false>
-__global__ __launch_bounds__(kThreads, (BLOCK ? 2 : NKG < 0 ? RGLRU_GIVEN_OCC : (NKG == 4 || NKG == 2) ? RGLRU_NARROW_OCC : NKG > 8 ? 1 : 2)) void fwd_kernel(FusedArgs p) {
-  constexpr int MT = kFwdMT, TR = 32 * MT, EL = 16 * MT;
+__global__ __launch_bounds__(kThreads, (BLOCK ? 2 : NKG < 0 ? RGLRU_GIVEN_OCC : (NKG == 4 || NKG == 2) ? RGLRU_NARROW_OCC : NKG > 8 ? fwd_wide_occ(NKG) : 2)) void fwd_kernel(FusedArgs p) {
+  constexpr int MT = fwd_mt(NKG), TR = 32 * MT, EL = 16 * MT;
   static_assert(!BLOCK || (sizeof(IO) == 2 && (NKG == 8 || NKG == 4 || NKG == 2)), "block forward: 16-bit storage, register-held weights");
   typedef Io<IO> Tr;
   typedef typename Tr::Frag Frag;
@@ -534,6 +553,7 @@ __global__ __launch_bounds__(kThreads, (BLOCK ? 2 : NKG < 0 ? RGLRU_GIVEN_OCC : 
   __shared__ __attribute__((aligned(16))) float conv_w[BLOCK ? 5 * KC : 4];    // taps of lag 0..3, then the bias
 
   const WaveId w = wave_identity(p, blockIdx.x);
+  if (w.wg_in_unit >= p.wg_per_unit) return;             // only with xcd_map: the grid's last round is not full
   const int hf = w.hf, tid = threadIdx.x;
   unsigned char* stage = stage_all + w.wave * WaveStage<TR>::kBytes;
   if constexpr (BLOCK) {
@@ -1015,6 +1035,7 @@ __global__ __launch_bounds__(kThreads, (NKG > 8 ? 1 : 2)) void bwd_scan_kernel(F
   __shared__ __attribute__((aligned(16))) IO lds_wx[XLDS ? 32 * kWaves * WROW : Tr::HW];
 
   const WaveId w = wave_identity(p, blockIdx.x);
+  if (w.wg_in_unit >= p.wg_per_unit) return;             // only with xcd_map: the grid's last round is not full
   const int hf = w.hf, tid = threadIdx.x;
   unsigned char* stage_dx = stage_dx_all + w.wave * WaveStage<TR>::kBytes;
   unsigned char* stage_du = stage_du_all + w.wave * (GIVEN ? 2 * WaveStage<TR>::kBytes : PairStage<TR>::kBytes);
@@ -1858,9 +1879,14 @@ __global__ __launch_bounds__(kGradThreads, 1) void gate_grad_wide_kernel(FusedAr
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, hf = lane >> 5;
   const int sl = wave & 1, q = wave >> 1;
-  const int units = p.nb * JG;
-  const int unit = blockIdx.x % units, wg_in_unit = blockIdx.x / units, n_wg = gridDim.x / units;
-  const int k = unit / JG, jg = unit - k * JG;
+  // The JG units of a block that walk the same tiles read the same du2 rows.  Workgroups go to the eight XCDs
+  // round-robin by index, each XCD has its own L2: index = xcd + 8 * slot puts the JG members of a
+  // (block, tile sequence) pair into consecutive slots of ONE XCD, so that du2 comes from memory once.
+  const int n_wg = p.wg_per_unit;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int pair = xcd + 8 * (slot / JG), jg = slot % JG;
+  const int k = pair % p.nb, wg_in_unit = pair / p.nb;
+  if (wg_in_unit >= n_wg) return;                          // the grid is rounded up to whole rounds of eight pairs
   const int slab = jg * 2 + sl;
   const bool slab_ok = slab < S;
   const int j0 = (slab_ok ? slab : 0) * 32;                // the wave's first column inside the block
@@ -2707,7 +2733,6 @@ static int fwd_impl(const void* x, const void* prep, const float* h0, const uint
   a.ckpt = (float*)(wb + L.ckpt); a.rec_a = (rec_t*)(wb + L.f_rec_a);
   a.ticket = (unsigned*)(wb + L.f_ticket); a.fail = (unsigned*)(wb + L.fail);
   a.B = (int)B; a.T = (int)T; a.nC = (int)L.nC; a.ckpt_nC = 2 * (int)L.nC;
-  a.nCf = (int)((T + 32 * kFwdMT - 1) / (32 * kFwdMT));
   a.aligned = is_aligned(x, W, g.bw, elem_size(dtype)) && ((uintptr_t)y % 16 == 0);
   int nkg = held_groups(g, dtype, a.aligned);
   if (!nkg && !pre) nkg = wide_groups(g, dtype, a.aligned);
@@ -2738,13 +2763,19 @@ static int fwd_impl(const void* x, const void* prep, const float* h0, const uint
     if (rc) return rc;
   }
   pack_units(a, g, nkg);
+  const int tile_tokens = 32 * fwd_mt(nkg);
+  a.nCf = (int)((T + tile_tokens - 1) / tile_tokens);
   // without weights in registers three workgroups fit a compute unit
-  a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nCf, blk ? 2 : nkg < 0 ? RGLRU_GIVEN_OCC : ((nkg == 4 || nkg == 2) ? RGLRU_NARROW_OCC : nkg > 8 ? 1 : 2), 1 << 20);
+  a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nCf, blk ? 2 : nkg < 0 ? RGLRU_GIVEN_OCC : ((nkg == 4 || nkg == 2) ? RGLRU_NARROW_OCC : nkg > 8 ? fwd_wide_occ(nkg) : 2), 1 << 20);
   a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
   dim3 grid((unsigned)(a.wg_per_unit * a.units));
+  if (nkg > 8) {
+    a.xcd_map = 1;
+    grid = dim3((unsigned)(8 * (((long long)nb * a.wg_per_unit + 7) / 8) * a.groups));
+  }
   {
     KernelTimer timer(0, s);
-    const int masked = (flags != nullptr) || (T % (32 * kFwdMT) != 0);
+    const int masked = (flags != nullptr) || (T % tile_tokens != 0);
     if (blk) {
 #define RGLRU_BLOCK_CASE(N)                                                                                            \
       if (nkg == N) {                                                                                                  \
@@ -3108,7 +3139,8 @@ int rglru_hip_bwd_wide(const void* x, const void* prep, const float* h0,
   a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nC, 1, L.max_wg);
   a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
   const bool masked = (flags != nullptr) || (T % kChunk != 0);
-  dim3 grid((unsigned)(a.wg_per_unit * a.units));
+  a.xcd_map = 1;
+  dim3 grid((unsigned)(8 * (((long long)nb * a.wg_per_unit + 7) / 8) * a.groups));
   {
     KernelTimer timer(1, s);
 #define RGLRU_LAUNCH_WIDE_SCAN(N)                                                                                    \
@@ -3130,7 +3162,10 @@ int rglru_hip_bwd_wide(const void* x, const void* prep, const float* h0,
   int n_wg = num_compute_units() / grad_units; if (n_wg < 1) n_wg = 1; if (n_wg > kWideWgPerUnit) n_wg = kWideWgPerUnit;
   const long long grad_tiles = (B * T + 31) / 32;
   if (n_wg > grad_tiles) n_wg = (int)grad_tiles;
-  dim3 grid2((unsigned)(n_wg * grad_units));
+  const int scan_wg_per_unit = a.wg_per_unit;
+  a.wg_per_unit = n_wg;
+  const long long grad_pairs = (long long)nb * n_wg;      // (block, tile sequence) pairs, dealt to the XCDs in rounds of eight
+  dim3 grid2((unsigned)(8 * ((grad_pairs + 7) / 8) * ((g.S + 1) / 2)));
   {
     KernelTimer timer(3, s);
     switch (nkg) {
@@ -3150,7 +3185,7 @@ int rglru_hip_bwd_wide(const void* x, const void* prep, const float* h0,
   memset(&r, 0, sizeof(r));
   r.partial = a.partial; r.dsp = finish_dsp(g, prep, dtype); r.db_a = db_a; r.db_x = db_x; r.dlambda = dlambda;
   r.dw_partial = a.dw_partial; r.dw_a = dw_a; r.dw_x = dw_x;
-  r.W = (int)W; r.nb = (int)nb; r.bw = (int)g.bw; r.bwp = (int)g.bwp; r.Wp = (int)g.Wp; r.wg_per_unit = a.wg_per_unit;
+  r.W = (int)W; r.nb = (int)nb; r.bw = (int)g.bw; r.bwp = (int)g.bwp; r.Wp = (int)g.Wp; r.wg_per_unit = scan_wg_per_unit;
   r.n_wg = n_wg; r.vec_blocks = (int)((W + 15) / 16); r.grad_dtype = grad_dtype;
   r.clean = (uint4*)(wb + L.b_begin); r.clean_n = (long long)((L.b_end - L.b_begin) / 16);
   const long long total = nb * g.bw * 2 * g.bw;
