@@ -9,8 +9,10 @@ from .hip_scan import (
     hip_rglru_steps,
     hip_scan_available,
     hip_scan_is_usable,
+    set_reproducible,
 )
-from .hip_block_ops import hip_causal_conv, hip_causal_conv_padded, hip_gelu_gate, hip_rmsnorm
+from .hip_block_ops import (hip_block_forward, hip_causal_conv, hip_causal_conv_padded, hip_gelu_gate, hip_linear,
+                            hip_linear_pair, hip_rmsnorm)
 from .modules import (
     BlockDiagonalLinear,
     RG_LRU,
@@ -26,9 +28,12 @@ __all__ = [
     "RMSNorm",
     "RecurrentBlock",
     "RecurrentBlockCache",
+    "hip_block_forward",
     "hip_causal_conv",
     "hip_causal_conv_padded",
     "hip_gelu_gate",
+    "hip_linear",
+    "hip_linear_pair",
     "hip_rmsnorm",
     "hip_rglru",
     "hip_rglru_scan",
@@ -36,4 +41,5 @@ __all__ = [
     "hip_rglru_steps",
     "hip_scan_available",
     "hip_scan_is_usable",
+    "set_reproducible",
 ]

@@ -72,6 +72,7 @@ _SIGNATURES = {
                                     + [_I, _I, _I, _I, ctypes.c_int, _P]),
     "rglru_hip_step_gated": (ctypes.c_int, [_P] * 6 + [_I, _P] + [_I, _I, _I, ctypes.c_int, _P]),
     "rglru_hip_set_spin_limit": (ctypes.c_int64, [_I]),
+    "rglru_hip_set_reproducible": (ctypes.c_int, [ctypes.c_int]),
     "rglru_hip_set_timing": (ctypes.c_int, [ctypes.c_int]),
     "rglru_hip_kernel_ms": (ctypes.c_float, [ctypes.c_int]),
     "rglru_hip_workspace_status": (ctypes.c_int, [_P, _I, _I, _I, _I, ctypes.c_int, _P, ctypes.POINTER(ctypes.c_int)]),

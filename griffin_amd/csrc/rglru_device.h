@@ -204,8 +204,12 @@ struct CarryWalk {
 
 // Compose one batch of records (chunks p, p + step, ...) into the walk.  Returns true when the
 // batch ran into a record that is not published yet; p then names that chunk.
+// finals_only: a record counts as published only once it is final, so every chunk takes its carry from
+// the chunk right before it and the result does not depend on which records happened to be final when
+// they were read (bit-reproducible; the chain is then as slow as one round trip per chunk).
 template <int DEPTH>
-RGLRU_DEVICE bool carry_compose(const rec_t (&rec)[DEPTH], CarryWalk& wk, int step, int end, float boundary) {
+RGLRU_DEVICE bool carry_compose(const rec_t (&rec)[DEPTH], CarryWalk& wk, int step, int end, float boundary,
+                                bool finals_only = false) {
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d) {
     const int q = wk.p + d * step;
@@ -214,7 +218,7 @@ RGLRU_DEVICE bool carry_compose(const rec_t (&rec)[DEPTH], CarryWalk& wk, int st
       return false;
     }
     const unsigned lo = (unsigned)rec[d];
-    if (!__all(wk.done || lo != 0u)) { wk.p = q; return true; }
+    if (!__all(wk.done || (finals_only ? lo == 1u : lo != 0u))) { wk.p = q; return true; }
     if (!wk.done) {
       wk.acc_h = fmaf(wk.acc_a, __uint_as_float((unsigned)(rec[d] >> 32)), wk.acc_h);
       if (lo == 1u) { wk.acc_a = 0.f; wk.done = true; }
@@ -230,9 +234,12 @@ RGLRU_DEVICE bool carry_compose(const rec_t (&rec)[DEPTH], CarryWalk& wk, int st
 // are still waiting, so every wave still reaches the end of the kernel and the failure is visible in
 // the results themselves (the chunk's outputs and the carry it hands on turn NaN) without anybody
 // having to read the failure word.
+// A negative `limit` asks for finals_only with -limit polls (one argument carries both through the kernels).
 template <int DEPTH>
 RGLRU_DEVICE float carry_walk(const CarryChain& ch, CarryWalk& wk, int step, int end, float boundary,
                               long long limit, unsigned* fail_word) {
+  const bool finals_only = limit < 0;
+  if (finals_only) limit = -limit;
   long long polls = 0;
   while (!__all(wk.done)) {
     rec_t rec[DEPTH];
@@ -243,7 +250,7 @@ RGLRU_DEVICE float carry_walk(const CarryChain& ch, CarryWalk& wk, int step, int
       rec[d] = 0;
       if (inside && !wk.done) rec[d] = rec_load(ch.rec + q * ch.stride);
     }
-    if (carry_compose<DEPTH>(rec, wk, step, end, boundary)) {
+    if (carry_compose<DEPTH>(rec, wk, step, end, boundary, finals_only)) {
       if (++polls > limit) {
         if ((threadIdx.x & 63) == 0) atomicOr(fail_word, 1u);
         if (!wk.done) wk.acc_h = __builtin_nanf("");
@@ -305,7 +312,7 @@ RGLRU_DEVICE float carry_lookback_from(const CarryBatch<DEPTH>& first, const Car
                                        float boundary, bool lane_ok, long long limit, unsigned* fail_word) {
   CarryWalk wk;
   wk.acc_a = 1.f; wk.acc_h = 0.f; wk.done = !lane_ok; wk.p = c + step;
-  carry_compose<DEPTH>(first.rec, wk, step, end, boundary);
+  carry_compose<DEPTH>(first.rec, wk, step, end, boundary, limit < 0);
   return carry_walk<DEPTH>(ch, wk, step, end, boundary, limit, fail_word);
 }
 

@@ -49,7 +49,12 @@ int num_compute_units() {
 }
 
 static std::atomic<long long> g_spin_limit{1ll << 22};
-long long spin_limit() { return g_spin_limit.load(std::memory_order_relaxed); }
+static std::atomic<int> g_reproducible{0};
+// what the kernels get as `limit`: negative selects the look-back that accepts final records only
+long long spin_limit() {
+  const long long polls = g_spin_limit.load(std::memory_order_relaxed);
+  return g_reproducible.load(std::memory_order_relaxed) ? -polls : polls;
+}
 long long exchange_spin_limit(long long v) { return g_spin_limit.exchange(v); }
 
 // ------------------------------------------------------------------------------------------
@@ -203,6 +208,8 @@ RGLRU_DEVICE float4 carry_lookback4(const rec_t* rec, long long stride, int c, i
   bool done = !lane_ok;
   int q = c + step;
   long long polls = 0;
+  const bool finals_only = limit < 0;                    // see carry_compose
+  if (finals_only) limit = -limit;
   while (!__all(done)) {
     if (q == end) {                                      // wave-uniform
       if (!done) {
@@ -217,7 +224,8 @@ RGLRU_DEVICE float4 carry_lookback4(const rec_t* rec, long long stride, int c, i
 #pragma unroll
       for (int i = 0; i < 4; ++i) r[i] = rec_load(rec + (long long)q * stride + i);
     }
-    const bool ready = done || ((unsigned)r[0] != 0u && (unsigned)r[1] != 0u && (unsigned)r[2] != 0u && (unsigned)r[3] != 0u);
+    const bool ready = done || (finals_only ? ((unsigned)r[0] == 1u && (unsigned)r[1] == 1u && (unsigned)r[2] == 1u && (unsigned)r[3] == 1u)
+                                            : ((unsigned)r[0] != 0u && (unsigned)r[1] != 0u && (unsigned)r[2] != 0u && (unsigned)r[3] != 0u));
     if (!__all(ready)) {
       if (++polls > limit) {
         if ((threadIdx.x & 63) == 0) atomicOr(fail_word, 1u);
@@ -390,6 +398,8 @@ int64_t rglru_hip_set_spin_limit(int64_t polls) {
   if (polls < 1) polls = 1;
   return (int64_t)g_spin_limit.exchange((long long)polls);
 }
+
+int rglru_hip_set_reproducible(int enable) { return g_reproducible.exchange(enable ? 1 : 0); }
 
 size_t rglru_hip_scan_workspace_bytes(int64_t B, int64_t T, int64_t W) {
   if (B <= 0 || T <= 0 || W <= 0) return 0;

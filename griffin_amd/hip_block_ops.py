@@ -446,37 +446,77 @@ class _HipLinear(torch.autograd.Function):
     def backward(ctx, dy: Tensor):
         x, weight = ctx.saved_tensors
         need_x, need_w, need_b = ctx.needs_input_grad
-        dy2 = dy.reshape(-1, dy.size(-1))
-        dx = dw = db = None
-        if need_x:
-            dx = torch.matmul(dy, weight.to(dy.dtype))
-        if need_w:
-            x2 = x.reshape(-1, x.size(-1)).to(dy.dtype)
-            rows = dy2.size(0)
-            # dW = dy^T x contracts over all tokens: one GEMM with K = rows runs at a fraction of the rate of
-            # the same work as a batch of GEMMs with K = 2048 whose results are added (100 us against 43 us
-            # for 16384 x 1024 x 768 in bf16 on this library), so long contractions are split
-            chunks = rows // 2048 if (rows % 2048 == 0 and dy2.is_contiguous() and x2.is_contiguous()) else 1
-            while chunks > 16 and chunks % 2 == 0:
-                chunks //= 2
-            if chunks > 1:
-                per = rows // chunks
-                dw = torch.bmm(dy2.view(chunks, per, -1).transpose(1, 2), x2.view(chunks, per, -1)).sum(0)
-            else:
-                dw = torch.mm(dy2.t(), x2)
-            dw = dw.to(weight.dtype)
-        if need_b and ctx.bias_dtype is not None:
-            rows, width = dy2.shape
-            dy_c = dy2.contiguous()
-            out_dtype = ctx.bias_dtype if ctx.bias_dtype in _DTYPE_CODES else torch.float32
-            lib = _lib.load()
-            with _on_device(dy.device):
-                db = torch.empty(width, dtype=out_dtype, device=dy.device)
-                scratch = torch.empty(lib.rglru_hip_colsum_scratch_bytes(rows, width), dtype=torch.uint8, device=dy.device)
-                _lib.check(lib.rglru_hip_colsum(_ptr(dy_c), _ptr(scratch), _ptr(db), rows, width, _dtype_code(dy.dtype),
-                                                _DTYPE_CODES[out_dtype], _stream_ptr(dy.device)), "rglru_hip_colsum")
-            db = db.to(ctx.bias_dtype)
+        dx = torch.matmul(dy, weight.to(dy.dtype)) if need_x else None
+        dw, db = _linear_parameter_grads(x, weight, dy, need_w, ctx.bias_dtype if need_b else None)
         return dx, dw, db
+
+
+def _linear_parameter_grads(x: Tensor, weight: Tensor, dy: Tensor, need_w: bool, bias_dtype):
+    """(dW, db) of ``y = x W^T + b`` for the incoming ``dy``; ``bias_dtype`` None skips db."""
+    dy2 = dy.reshape(-1, dy.size(-1))
+    dw = db = None
+    if need_w:
+        x2 = x.reshape(-1, x.size(-1)).to(dy.dtype)
+        rows = dy2.size(0)
+        # dW = dy^T x contracts over all tokens: one GEMM with K = rows runs at a fraction of the rate of
+        # the same work as a batch of GEMMs with K = 2048 whose results are added (100 us against 43 us
+        # for 16384 x 1024 x 768 in bf16 on this library), so long contractions are split
+        chunks = rows // 2048 if (rows % 2048 == 0 and dy2.is_contiguous() and x2.is_contiguous()) else 1
+        while chunks > 16 and chunks % 2 == 0:
+            chunks //= 2
+        if chunks > 1:
+            per = rows // chunks
+            dw = torch.bmm(dy2.view(chunks, per, -1).transpose(1, 2), x2.view(chunks, per, -1)).sum(0)
+        else:
+            dw = torch.mm(dy2.t(), x2)
+        dw = dw.to(weight.dtype)
+    if bias_dtype is not None:
+        rows, width = dy2.shape
+        dy_c = dy2.contiguous()
+        out_dtype = bias_dtype if bias_dtype in _DTYPE_CODES else torch.float32
+        lib = _lib.load()
+        with _on_device(dy.device):
+            db = torch.empty(width, dtype=out_dtype, device=dy.device)
+            scratch = torch.empty(lib.rglru_hip_colsum_scratch_bytes(rows, width), dtype=torch.uint8, device=dy.device)
+            _lib.check(lib.rglru_hip_colsum(_ptr(dy_c), _ptr(scratch), _ptr(db), rows, width, _dtype_code(dy.dtype),
+                                            _DTYPE_CODES[out_dtype], _stream_ptr(dy.device)), "rglru_hip_colsum")
+        db = db.to(bias_dtype)
+    return dw, db
+
+
+class _HipLinearPair(torch.autograd.Function):
+    """Two Linear layers on one input (the block's two branches).  Their input gradients are one GEMM that
+    accumulates into the other's result instead of two results and an addition."""
+
+    @staticmethod
+    def forward(ctx, x: Tensor, w1: Tensor, b1: Tensor | None, w2: Tensor, b2: Tensor | None):
+        ctx.save_for_backward(x, w1, w2)
+        ctx.bias_dtypes = (None if b1 is None else b1.dtype, None if b2 is None else b2.dtype)
+        ctx.set_materialize_grads(False)
+        return torch.nn.functional.linear(x, w1, b1), torch.nn.functional.linear(x, w2, b2)
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, dy1: Tensor | None, dy2: Tensor | None):
+        x, w1, w2 = ctx.saved_tensors
+        need_x, need_w1, need_b1, need_w2, need_b2 = ctx.needs_input_grad
+        dx = None
+        if need_x:
+            for dy, w in ((dy1, w1), (dy2, w2)):
+                if dy is None:
+                    continue
+                flat = dy.reshape(-1, dy.size(-1))
+                if dx is None:
+                    dx = torch.mm(flat, w.to(dy.dtype))
+                else:
+                    dx.addmm_(flat, w.to(dy.dtype))
+            dx = None if dx is None else dx.view(x.shape)
+        dw1 = db1 = dw2 = db2 = None
+        if dy1 is not None:
+            dw1, db1 = _linear_parameter_grads(x, w1, dy1, need_w1, ctx.bias_dtypes[0] if need_b1 else None)
+        if dy2 is not None:
+            dw2, db2 = _linear_parameter_grads(x, w2, dy2, need_w2, ctx.bias_dtypes[1] if need_b2 else None)
+        return dx, dw1, db1, dw2, db2
 
 
 def hip_linear(x: Tensor, weight: Tensor, bias: Tensor | None) -> Tensor:
@@ -485,6 +525,14 @@ def hip_linear(x: Tensor, weight: Tensor, bias: Tensor | None) -> Tensor:
     _require_gpu("hip_linear", x, weight, bias)
     _dtype_code(x.dtype)
     return _HipLinear.apply(x, weight, bias)
+
+
+def hip_linear_pair(x: Tensor, w1: Tensor, b1: Tensor | None, w2: Tensor, b2: Tensor | None) -> tuple[Tensor, Tensor]:
+    """``(x @ w1.T + b1, x @ w2.T + b2)``: two ``hip_linear`` calls whose backward passes share the input
+    gradient (the second GEMM accumulates into the first one's result)."""
+    _require_gpu("hip_linear_pair", x, w1, b1, w2, b2)
+    _dtype_code(x.dtype)
+    return _HipLinearPair.apply(x, w1, b1, w2, b2)
 
 
 class _HipRMSNorm(torch.autograd.Function):

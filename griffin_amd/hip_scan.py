@@ -32,6 +32,13 @@ def hip_scan_available() -> bool:
     return _lib.available()
 
 
+def set_reproducible(enable: bool) -> bool:
+    """Bit-reproducible results from run to run (rglru_hip_set_reproducible): every chunk of a sequence then
+    takes its carry from the finished chunk before it instead of combining whatever its neighbours have
+    published so far.  Slower, mostly for long sequences; off by default.  Returns the previous setting."""
+    return bool(_lib.load().rglru_hip_set_reproducible(1 if enable else 0))
+
+
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 _raw_device = getattr(torch._C, "_cuda_getDevice", None)
 

@@ -425,12 +425,15 @@ class RecurrentBlock(nn.Module):
     def _linear(self, layer: nn.Linear, x: Tensor) -> Tensor:
         """A Linear layer of the block; in training on the HIP path its bias gradient is summed by a
         kernel of the library instead of a generic reduction (the GEMMs are the BLAS library's either way)."""
-        if (torch.is_grad_enabled() and layer.bias is not None and layer.bias.requires_grad
-                and x.is_cuda and x.dtype in hip_scan.SUPPORTED_DTYPES and layer.weight.dtype == x.dtype
-                and self.rg_lru.scan_mode in ("hip", "fused", "auto") and x.numel() > 0
-                and (self.rg_lru.scan_mode != "auto" or hip_scan.hip_scan_is_usable(x.device))):
+        if self._linear_on_hip(layer, x):
             return hip_block_ops.hip_linear(x, layer.weight, layer.bias)
         return layer(x)
+
+    def _linear_on_hip(self, layer: nn.Linear, x: Tensor) -> bool:
+        return (torch.is_grad_enabled() and layer.bias is not None and layer.bias.requires_grad
+                and x.is_cuda and x.dtype in hip_scan.SUPPORTED_DTYPES and layer.weight.dtype == x.dtype
+                and self.rg_lru.scan_mode in ("hip", "fused", "auto") and x.numel() > 0
+                and (self.rg_lru.scan_mode != "auto" or hip_scan.hip_scan_is_usable(x.device)))
 
     def _dense_conv(self, projected: Tensor, conv_state: Tensor | None, segment_pos: Tensor, need_state: bool = True):
         """All-tokens-active path (griffin/griffin.py:476-487): taps are masked per document."""
@@ -479,8 +482,12 @@ class RecurrentBlock(nn.Module):
         segment_pos = _resolve_segment_positions(
             x, segment_pos, previous_position, None if everything_active else active_mask)
 
-        gate_input = self._linear(self.linear_y, x)
-        projected = self._linear(self.linear_x, x)
+        if self._linear_on_hip(self.linear_x, x) and self._linear_on_hip(self.linear_y, x):
+            projected, gate_input = hip_block_ops.hip_linear_pair(
+                x, self.linear_x.weight, self.linear_x.bias, self.linear_y.weight, self.linear_y.bias)
+        else:
+            gate_input = self._linear(self.linear_y, x)
+            projected = self._linear(self.linear_x, x)
         on_hip = self._hip_block_ops_covers(projected)
         # the HIP convolution takes "no carried state" as such; the portable path wants the zeros
         conv_state = (None if on_hip else self._empty_conv_state(projected)) if cache is None else cache.conv_state

@@ -349,6 +349,15 @@ int rglru_hip_prepare_block_fwd(const void* w_a, const void* b_a, const void* w_
  * gives up, records the failure in the workspace and finishes with unspecified results.  The
  * default is large enough never to trigger in normal operation.  Returns the previous value. */
 int64_t rglru_hip_set_spin_limit(int64_t polls);
+/* Reproducible mode (off by default; no counterpart in the reference, whose scans are sequential and therefore
+ * reproducible).  Chunks of a sequence exchange carries through a look-back that normally combines whatever
+ * records it finds, final or not, so results agree between runs to rounding only.  With the mode on, a chunk
+ * waits for the FINAL record of the chunk before it: y, h_last and everything the backward entry points
+ * rglru_hip_bwd_full, rglru_hip_scan_fwd and rglru_hip_scan_bwd return are then bit-identical from run to run
+ * (the bias and Lambda gradients of the other backward entry points still add per-workgroup sums whose
+ * composition follows the ticket order).  The chain becomes one memory round trip per chunk: slower,
+ * mostly for long sequences.  Applies to launches made after the call; returns the previous setting. */
+int rglru_hip_set_reproducible(int enable);
 /* Synchronising debug helper: copies the failure word of a workspace to the host (0 = clean). */
 int rglru_hip_workspace_status(const void* ws, int64_t B, int64_t T, int64_t W, int64_t nb,
                                int scan_only, void* stream, int* status);

@@ -397,6 +397,42 @@ def test_hip_linear_matches_torch_linear(shape, dtype):
         assert err < tol, name
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(2, 50, 64, 96), (3, 7, 13, 5), (8, 2048, 768, 1024)])
+@pytest.mark.parametrize("used", ["both", "first", "second"])
+def test_hip_linear_pair_matches_two_linear_layers(shape, dtype, used):
+    """The block's two input projections as one autograd node (griffin/griffin.py:462-464): outputs and all
+    five gradients against two torch.nn.functional.linear calls in fp64, also when only one of the two
+    outputs takes part in the loss."""
+    from griffin_amd.hip_block_ops import hip_linear_pair
+
+    B, T, D, W = shape
+    _say("linear pair case", shape, dtype, used)
+    gen = torch.Generator().manual_seed(34)
+    x = torch.randn(B, T, D, generator=gen).to(dtype)
+    ws = [(torch.randn(W, D, generator=gen) / D ** 0.5).to(dtype) for _ in range(2)]
+    bs = [(torch.randn(W, generator=gen) * 0.1).to(dtype) for _ in range(2)]
+    dys = [torch.randn(B, T, W, generator=gen).to(dtype) for _ in range(2)]
+    take = [used in ("both", "first"), used in ("both", "second")]
+    ref = [t.double().requires_grad_(True) for t in (x, ws[0], bs[0], ws[1], bs[1])]
+    outs = (torch.nn.functional.linear(ref[0], ref[1], ref[2]), torch.nn.functional.linear(ref[0], ref[3], ref[4]))
+    sum((o * d.double()).sum() for o, d, t in zip(outs, dys, take) if t).backward()
+    dev = [t.cuda().requires_grad_(True) for t in (x, ws[0], bs[0], ws[1], bs[1])]
+    got = hip_linear_pair(*dev)
+    sum((o.float() * d.cuda().float()).sum() for o, d, t in zip(got, dys, take) if t).backward()
+    torch.cuda.synchronize()
+    tol = 2e-5 if dtype == torch.float32 else BF16_TOL
+    for o, w in zip(got, outs):
+        assert rel_err(o.double().cpu(), w.detach()) < tol
+    for name, r, d in zip(("x", "w1", "b1", "w2", "b2"), ref, dev):
+        if r.grad is None:
+            assert d.grad is None, name
+            continue
+        err = rel_err(d.grad.double().cpu(), r.grad)
+        _say("  d%s rel error: %.2e" % (name, err))
+        assert err < tol, name
+
+
 # ----------------------------------------------------------------------------------------------
 # convolution + RG-LRU + output gate in one forward launch (rglru_hip_block_fwd), griffin/griffin.py:464-520
 # ----------------------------------------------------------------------------------------------

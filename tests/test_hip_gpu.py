@@ -228,6 +228,85 @@ def test_backward_twice_over_one_forward(dtype, shape):
         assert rel_err(b.float(), 2 * a.float()) < tol
 
 
+@pytest.mark.parametrize("dtype,shape,everything", [
+    (torch.bfloat16, (8, 2048, 1024, 8), True),      # the benchmark shape: forward, reverse scan and gradient kernels
+    (torch.bfloat16, (3, 1000, 256, 4), True),       # masked variants (T is not a multiple of the tile), 64-wide blocks
+    (torch.bfloat16, (1, 4096, 640, 2), False),      # 320-wide blocks
+    (torch.float32, (2, 300, 48, 3), False),         # portable kernels
+])
+def test_reproducible_mode_repeats_bit_for_bit(dtype, shape, everything):
+    """With rglru_hip_set_reproducible(1) a chunk takes its carry from the finished chunk before it, so
+    repeated runs agree bit for bit (the reference's sequential scan does, griffin/griffin.py:279-284) and
+    still match the oracle.  `everything`: all gradients (blocks of 32/64/128 channels in bf16); elsewhere the
+    bias and Lambda gradients add per-workgroup sums in ticket order and are compared to rounding only."""
+    from griffin_amd import hip_rglru, set_reproducible
+
+    B, T, W, nb = shape
+    _say("reproducible mode", dtype, shape)
+    case = orc.make_case(B, T, W, nb, seed=23, lo=0.9, hi=0.999)
+    dy = case["dy"].to(dtype).cuda()
+    dh = torch.randn(B, W, generator=torch.Generator().manual_seed(5)).cuda()
+
+    def run():
+        leaves = [case[k].to(dtype).cuda().requires_grad_(True) for k in PARAMS]
+        y, h_last = hip_rglru(*leaves, 8.0)
+        grads = torch.autograd.grad([y, h_last], leaves, [dy, dh])
+        torch.cuda.synchronize()
+        return [y.detach(), h_last.detach()] + list(grads)
+
+    names = ["y", "h_last"] + ["d" + k for k in PARAMS]
+    was = set_reproducible(True)
+    try:
+        runs = [run() for _ in range(3)]
+    finally:
+        set_reproducible(was)
+    exact = set(names) if everything else {"y", "h_last", "dx"}
+    for other in runs[1:]:
+        for name, a, b in zip(names, runs[0], other):
+            if name in exact:
+                assert torch.equal(a, b), name
+            else:
+                assert rel_err(b.float(), a.float()) < 1e-5, name
+    # the mode changes how carries travel, not what is computed
+    ry, rh, rgrads = oracle_run(case, dtype, None, None, dh.cpu())
+    tol = FP32_TOL if dtype == torch.float32 else BF16_TOL
+    assert rel_err(runs[0][0].float().cpu(), ry) < tol and rel_err(runs[0][1].cpu(), rh) < tol
+    for k, g in zip(PARAMS, runs[0][2:]):
+        assert rel_err(g.float().cpu(), rgrads[k]) < tol, k
+
+
+def test_reproducible_mode_of_the_scan_only_operator():
+    """The scan-only operator (contract of triton_scan.py:274) in reproducible mode: forward and both gradients
+    repeat bit for bit and equal the default mode to rounding."""
+    from griffin_amd import hip_rglru_scan, set_reproducible
+
+    B, T, W = 4, 3000, 192
+    gen = torch.Generator().manual_seed(2)
+    a0 = torch.sigmoid(torch.randn(B, T, W, generator=gen) + 2.0).cuda()
+    z0 = torch.randn(B, T, W, generator=gen).cuda()
+    h0 = torch.randn(B, W, generator=gen).cuda()
+    dh = torch.randn(B, T, W, generator=gen).cuda()
+
+    def run():
+        a, z, h = (t.clone().requires_grad_(True) for t in (a0, z0, h0))
+        out = hip_rglru_scan(a, z, h)
+        grads = torch.autograd.grad(out, [a, z, h], dh)
+        torch.cuda.synchronize()
+        return [out.detach()] + list(grads)
+
+    default = run()
+    was = set_reproducible(True)
+    try:
+        runs = [run() for _ in range(3)]
+    finally:
+        set_reproducible(was)
+    for other in runs[1:]:
+        for a, b in zip(runs[0], other):
+            assert torch.equal(a, b)
+    for a, b in zip(runs[0], default):
+        assert rel_err(a, b) < 1e-5
+
+
 # ------------------------------------------------------------------ golden vectors of the reference
 @pytest.mark.parametrize("name", ["rglru_plain_b2_t16_w32", "rglru_masks_b2_t16_w32", "rglru_odd_b3_t37_w65"])
 def test_fused_matches_reference_golden_vectors(golden_dir, name):
