@@ -379,9 +379,19 @@ def hip_block_forward(u: Tensor, v: Tensor, conv_state: Tensor | None, weight: T
     [W, 1, K], ``bias`` [W] of the depthwise ``nn.Conv1d`` (K <= 4); ``segment_pos`` [B, T]; ``flags``:
     ``hip_block_flags(segment_pos)`` if the caller has it already, else None; the five RG-LRU parameters, ``h0`` [B, W] or None; ``prep``: a prepared parameter image to use
     when no gradient is asked for.  Returns ``(gated [B, T, W], final state [B, W] fp32, new_conv_state
-    [B, K-1, W])``; differentiable in u, v, the parameters, conv_state and h0 (not through new_conv_state).
+    [B, K-1, W])``; differentiable in u, v, the parameters, conv_state and h0.
     """
-    return _HipBlockForward.apply(u, v, conv_state, weight, bias, segment_pos, flags, w_a, b_a, w_x, b_x, lam, h0, c, prep)
+    gated, h_last, new_conv = _HipBlockForward.apply(u, v, conv_state, weight, bias, segment_pos, flags,
+                                                     w_a, b_a, w_x, b_x, lam, h0, c, prep)
+    if torch.is_grad_enabled() and (u.requires_grad or (conv_state is not None and conv_state.requires_grad)):
+        # the carried rows as a differentiable function of u and conv_state (the kernel's copy carries no gradient)
+        history, steps = weight.size(2) - 1, u.size(1)
+        if steps >= history:
+            new_conv = u[:, steps - history:].clone()
+        else:
+            previous = u.new_zeros(u.size(0), history, u.size(2)) if conv_state is None else conv_state.to(u.dtype)
+            new_conv = torch.cat((previous[:, steps:], u), dim=1)
+    return gated, h_last, new_conv
 
 
 def hip_block_decode_step(u: Tensor, v: Tensor, conv_state: Tensor | None, weight: Tensor, bias: Tensor | None,

@@ -325,7 +325,8 @@ int rglru_hip_step_gated(const void* x, const void* prep, const float* h_in, flo
  * 3 - min(segment_pos, 3) (rglru_hip_block_flags writes them from segment_pos[n]); flags NULL means no
  * document starts inside the rows and position >= K - 1 or an all-zero history at their beginning.
  * Optional outputs (NULL to skip): x_conv[B,T,W] and y[B,T,W] (what a backward pass needs),
- * new_conv_state[B,K-1,W], h_last[B,W].  ws as for rglru_hip_fwd.  Only where
+ * new_conv_state[B,K-1,W], h_last[B,W].  No output may overlap an input (a tile reads the three rows of u in
+ * front of it while its neighbour writes).  ws as for rglru_hip_fwd.  Only where
  * rglru_hip_block_fwd_path() returns 1 (bf16 storage, gate blocks of 32, 64 or 128 channels, 16-byte
  * aligned rows); otherwise RGLRU_E_UNSUPPORTED, and the caller runs rglru_hip_conv_fwd, rglru_hip_fwd and
  * rglru_hip_gelu_gate_fwd one after the other.  rglru_hip_prepare_block_fwd is rglru_hip_prepare +

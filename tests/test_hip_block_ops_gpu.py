@@ -522,6 +522,7 @@ def test_block_forward_gradients_match_the_three_kernels(case):
     names = [n for n in ("u", "v", "conv_state", "weight", "bias", "w_a", "b_a", "w_x", "b_x", "lam", "h0") if p[n] is not None]
     dg = torch.randn(B, T, W).to(torch.bfloat16).cuda()
     dh = torch.randn(B, W).cuda()
+    dc = torch.randn(B, K - 1, W).to(torch.bfloat16).cuda()   # a later call's gradient at the carried rows
     _say("block forward gradients", case)
 
     def grads(fused):
@@ -529,12 +530,17 @@ def test_block_forward_gradients_match_the_three_kernels(case):
         for n in names:
             q[n] = p[n].detach().clone().requires_grad_(True)
         if fused:
-            gated, h_last, _ = hip_block_forward(q["u"], q["v"], q["conv_state"], q["weight"], q["bias"], q["pos"],
-                                                 hip_block_flags(q["pos"]) if B % 2 else None,
-                                                 q["w_a"], q["b_a"], q["w_x"], q["b_x"], q["lam"], q["h0"], 8.0)
+            gated, h_last, carried_rows = hip_block_forward(
+                q["u"], q["v"], q["conv_state"], q["weight"], q["bias"], q["pos"],
+                hip_block_flags(q["pos"]) if B % 2 else None,
+                q["w_a"], q["b_a"], q["w_x"], q["b_x"], q["lam"], q["h0"], 8.0)
         else:
-            gated, h_last, _ = _three_kernels(q)
-        return torch.autograd.grad([gated, h_last], [q[n] for n in names], [dg, dh])
+            gated, h_last, carried_rows = _three_kernels(q)
+        outs, ups = [gated, h_last], [dg, dh]
+        if K > 1:
+            outs.append(carried_rows)
+            ups.append(dc)
+        return torch.autograd.grad(outs, [q[n] for n in names], ups)
 
     want, got = grads(False), grads(True)
     torch.cuda.synchronize()
