@@ -163,6 +163,7 @@ struct FusedArgs {
   int nC, nCf, ckpt_nC, wg_per_unit, aligned, full_slabs, queues, flags_vec;
   int dw_bf16;                                            // fast backward: per-workgroup weight-gradient sums stored as bf16
   int xcd_map;                                            // wide blocks: the workgroups that share a block's x tiles sit on one XCD
+  int first_reset;                                        // token 0 of every sequence carries RGLRU_FLAG_RESET (and flags is null)
   long long limit;
 };
 
@@ -353,13 +354,15 @@ RGLRU_DEVICE unsigned pack_flag_bytes(unsigned d) {
   return (t | (t >> 12)) & 0xFFu;
 }
 RGLRU_DEVICE unsigned flag_run(const FusedArgs& p, long long token_row, int t_first) {
+  // first_reset: "every sequence starts a document" without a flag array (the run that holds token 0)
+  const unsigned first = (p.first_reset && t_first == 0) ? RGLRU_FLAG_RESET : 0u;
   if (p.flags_vec) {
     if (t_first >= p.T) return 0xAAAAAAAAu;
-    if (!p.flags) return 0u;
+    if (!p.flags) return first;
     const uint4 w = *reinterpret_cast<const uint4*>(p.flags + token_row);
-    return pack_flag_bytes(w.x) | (pack_flag_bytes(w.y) << 8) | (pack_flag_bytes(w.z) << 16) | (pack_flag_bytes(w.w) << 24);
+    return pack_flag_bytes(w.x) | (pack_flag_bytes(w.y) << 8) | (pack_flag_bytes(w.z) << 16) | (pack_flag_bytes(w.w) << 24) | first;
   }
-  unsigned bits = 0u;
+  unsigned bits = first;
 #pragma unroll
   for (int e = 0; e < 16; ++e) bits |= token_flag(p, token_row + e, t_first + e < p.T) << (2 * e);
   return bits;
@@ -370,13 +373,16 @@ RGLRU_DEVICE unsigned flag_run(const FusedArgs& p, long long token_row, int t_fi
 // ------------------------------------------------------------------------------------------
 // Gate math of 16 consecutive local steps (first = index of the first one in this lane's run).
 // MASKED = false is the common case: no flags, the tile lies inside the sequence.
+// reset0 (plain variant only): the run's first token starts a document although there is no flag array.
 template <typename IO, bool MASKED>
 RGLRU_DEVICE void fwd_gates(unsigned flbits, const f32x16& ua, const f32x16& ux,
-                            const float (&xv)[16], float sp, float* a, float* z, float nba = 0.0f, float nbx = 0.0f) {
+                            const float (&xv)[16], float sp, float* a, float* z, float nba = 0.0f, float nbx = 0.0f,
+                            bool reset0 = false) {
 #pragma unroll
   for (int v = 0; v < 16; ++v) {
     GateOut go;
     if constexpr (MASKED) go = gate_forward_run<Precise<IO>::value>(ua[v], ux[v], xv[v], sp, flbits, v, nba, nbx);
+    else if (v == 0) go = gate_forward<Precise<IO>::value, true>(ua[v], ux[v], xv[v], sp, reset0 ? RGLRU_FLAG_RESET : 0u, nba, nbx);
     else go = gate_forward<Precise<IO>::value, false>(ua[v], ux[v], xv[v], sp, 0u, nba, nbx);
     a[v] = go.a; z[v] = go.z;
   }
@@ -786,7 +792,8 @@ __global__ __launch_bounds__(kThreads, (BLOCK ? 2 : NKG < 0 ? RGLRU_GIVEN_OCC : 
             }
           } else
           gate_mfma_held<IO, MT, NKG, KC>(lds, hw, mt, w.slab, w.r, hf, 0.0f, 0.0f, ua, ux, xv, NKG >= 8 ? 0 : w.kb);
-          fwd_gates<IO, MASKED>(flbits[mt], ua, ux, xv, sp, cur.a + 16 * mt, cur.z + 16 * mt, nba, nbx);
+          fwd_gates<IO, MASKED>(flbits[mt], ua, ux, xv, sp, cur.a + 16 * mt, cur.z + 16 * mt, nba, nbx,
+                                p.first_reset && mt == 0 && cur.c == 0 && hf == 0);
         }
       }
       fwd_local<MT, MASKED>(p, w, cur, slab_ok);
@@ -908,7 +915,7 @@ __global__ __launch_bounds__(kThreads, (NKG == 0 ? 2 : 1)) void bwd_kernel(Fused
 #pragma unroll
     for (int e = 0; e < EL; ++e) {
       const bool in = t0 + hf * EL + e < p.T;
-      const unsigned fl = token_flag(p, trow + e, in);
+      const unsigned fl = token_flag(p, trow + e, in) | ((p.first_reset && t0 + hf * EL + e == 0) ? RGLRU_FLAG_RESET : 0u);
       flbits |= fl << (2 * e);
       GateOut go = gate_forward<Precise<IO>::value, true>(ua[0][e], ux[0][e], xv[e], sp, fl, nba, nbx);
       r[e] = go.r; gi[e] = go.i; a[e] = go.a; g[e] = go.g;
@@ -1452,6 +1459,7 @@ __global__ __launch_bounds__(kThreads, (MT == 1 ? 4 : RGLRU_DELTA_OCC)) void bwd
         for (int v = 0; v < 16; ++v) {
           float l2 = sigmoid_fast(ua[v], nba) * sp;
           if constexpr (MASKED) l2 = masked_log2_decay_run(l2, flbits[mt], v);
+          else if (mt == 0 && v == 0) l2 = (p.first_reset && c == 0 && hf == 0) ? kResetLog2 : l2;
           a[16 * mt + v] = __builtin_amdgcn_exp2f(l2);
           gy[16 * mt + v] = (float)lds_dy[(hf * EL + 16 * mt + v) * LDSROW + kb + w.slab * 32 + w.r];
         }
@@ -1677,6 +1685,7 @@ __global__ __launch_bounds__(kGradThreads, 1) void bwd_grad_kernel(FusedArgs p) 
           const float re = sigmoid_fast(ua[v], nba), ie = sigmoid_fast(ux[v], nbx);
           float l2 = re * sp;
           if constexpr (MASKED) l2 = masked_log2_decay_run(l2, flbits, v);
+          else if (v == 0) l2 = (p.first_reset && c == 0 && hf == 0) ? kResetLog2 : l2;
           const float ae = __builtin_amdgcn_exp2f(l2);
           // l2 <= 0 and a <= 1, so neither branch of one_minus_exp can turn negative: no clamp needed
           const float g2 = one_minus_exp<false>(l2 * (2.0f * kLn2), ae);
@@ -2728,6 +2737,9 @@ static int fwd_impl(const void* x, const void* prep, const float* h0, const uint
   FusedArgs a;
   memset(&a, 0, sizeof(a));
   fill_common(a, g, prep, dtype);
+  const bool first_reset = flags == RGLRU_FLAGS_FIRST_RESET;    // no flag array: token 0 of every row starts a document
+  if (first_reset) flags = nullptr;
+  a.first_reset = first_reset;
   a.x = x; a.h0 = h0; a.flags = flags; a.y = y; a.h_last = h_last;
   a.flags_vec = (T % 16 == 0) && ((uintptr_t)flags % 16 == 0);
   a.ckpt = (float*)(wb + L.ckpt); a.rec_a = (rec_t*)(wb + L.f_rec_a);
@@ -2754,7 +2766,8 @@ static int fwd_impl(const void* x, const void* prep, const float* h0, const uint
     if ((W * 2) % 16 || (xs * 2) % 16 || (vs * 2) % 16) return fail(RGLRU_E_UNSUPPORTED, "block_fwd: rows must be a multiple of 16 bytes");
     if (!nkg) return fail(RGLRU_E_UNSUPPORTED, "block_fwd: no kernel for this shape");
     a.gate_v = blk->v; a.ld_gate = vs; a.ld_x = xs;
-    a.conv_state = blk->K > 1 ? blk->conv_state : nullptr; a.conv_taps = blk->taps; a.conv_bias = blk->conv_bias;
+    // rows that start a document have no history
+    a.conv_state = (blk->K > 1 && !first_reset) ? blk->conv_state : nullptr; a.conv_taps = blk->taps; a.conv_bias = blk->conv_bias;
     a.conv_k = (int)blk->K; a.conv_vec_dtype = blk->vec_dtype;
     a.x_out = blk->x_conv; a.gated = blk->gated; a.conv_new_state = blk->K > 1 ? blk->new_conv_state : nullptr;
   }
@@ -2775,7 +2788,9 @@ static int fwd_impl(const void* x, const void* prep, const float* h0, const uint
   }
   {
     KernelTimer timer(0, s);
-    const int masked = (flags != nullptr) || (T % tile_tokens != 0);
+    // the plain kernels with register-held weights of up to 128 channels know first_reset; the others take it
+    // through the flag logic of their masked variant
+    const int masked = (flags != nullptr) || (T % tile_tokens != 0) || (first_reset && !(nkg == 8 || nkg == 4 || nkg == 2));
     if (blk) {
 #define RGLRU_BLOCK_CASE(N)                                                                                            \
       if (nkg == N) {                                                                                                  \
@@ -2870,6 +2885,7 @@ int rglru_hip_bwd_pre(const void* x, const void* pre, const void* prep, const fl
   FusedArgs a;
   memset(&a, 0, sizeof(a));
   fill_common(a, g, prep, dtype);
+  if (flags == RGLRU_FLAGS_FIRST_RESET) { flags = nullptr; a.first_reset = 1; }
   a.x = x; a.pre = pre; a.rows_total = B * T; a.h0 = h0; a.flags = flags; a.dy = dy; a.dh_last = dh_last;
   a.flags_vec = (T % 16 == 0) && ((uintptr_t)flags % 16 == 0);
   a.dx = dx; a.du_a = du; a.dh0 = dh0;
@@ -2880,7 +2896,7 @@ int rglru_hip_bwd_pre(const void* x, const void* pre, const void* prep, const fl
   a.aligned = 1;
   a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nC, 2, L.max_wg);
   a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
-  const bool masked = (flags != nullptr) || (T % kChunk != 0);
+  const bool masked = (flags != nullptr) || a.first_reset || (T % kChunk != 0);
   dim3 grid((unsigned)(a.wg_per_unit * a.units));
   {
     KernelTimer timer(1, s);
@@ -2968,6 +2984,7 @@ int rglru_hip_bwd(const void* x, const void* prep, const float* h0,
   FusedArgs a;
   memset(&a, 0, sizeof(a));
   fill_common(a, g, prep, dtype);
+  if (flags == RGLRU_FLAGS_FIRST_RESET) { flags = nullptr; a.first_reset = 1; }
   a.x = x; a.h0 = h0; a.flags = flags; a.dy = dy; a.dh_last = dh_last;
   a.flags_vec = (T % 16 == 0) && ((uintptr_t)flags % 16 == 0);
   a.dx = dx; a.du_a = du_a; a.du_x = du_x; a.dh0 = dh0;
@@ -3032,6 +3049,7 @@ int rglru_hip_bwd_full(const void* x, const void* y, const void* prep, const flo
   FusedArgs a;
   memset(&a, 0, sizeof(a));
   fill_common(a, g, prep, dtype);
+  if (flags == RGLRU_FLAGS_FIRST_RESET) { flags = nullptr; a.first_reset = 1; }
   a.x = x; a.y = const_cast<void*>(y); a.h0 = h0; a.flags = flags; a.dy = dy; a.dh_last = dh_last;
   a.flags_vec = (T % 16 == 0) && ((uintptr_t)flags % 16 == 0);
   const ScratchLayout SL = make_scratch_layout(B, T, g, kScratchFast);
@@ -3124,6 +3142,7 @@ int rglru_hip_bwd_wide(const void* x, const void* prep, const float* h0,
   FusedArgs a;
   memset(&a, 0, sizeof(a));
   fill_common(a, g, prep, dtype);
+  if (flags == RGLRU_FLAGS_FIRST_RESET) { flags = nullptr; a.first_reset = 1; }
   a.x = x; a.h0 = h0; a.flags = flags; a.dy = dy; a.dh_last = dh_last;
   a.flags_vec = (T % 16 == 0) && ((uintptr_t)flags % 16 == 0);
   const ScratchLayout SL = make_scratch_layout(B, T, g, kScratchWide);
@@ -3138,7 +3157,7 @@ int rglru_hip_bwd_wide(const void* x, const void* prep, const float* h0,
   // reverse scan and gate math: direct part of dx, du2, per-workgroup bias and Lambda sums
   a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nC, 1, L.max_wg);
   a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
-  const bool masked = (flags != nullptr) || (T % kChunk != 0);
+  const bool masked = (flags != nullptr) || a.first_reset || (T % kChunk != 0);
   a.xcd_map = 1;
   dim3 grid((unsigned)(8 * (((long long)nb * a.wg_per_unit + 7) / 8) * a.groups));
   {
@@ -3207,6 +3226,7 @@ static int step_impl(const void* x, const void* prep, const float* h_in, float* 
   fill_common(a, g, prep, dtype);
   if (gate_stride == 0) gate_stride = W;
   if (gate_v && gate_stride < W) return fail(RGLRU_E_ARG, "step: row stride %lld of the gate input is smaller than the width %lld", (long long)gate_stride, (long long)W);
+  if (flags == RGLRU_FLAGS_FIRST_RESET) return fail(RGLRU_E_ARG, "step: RGLRU_FLAGS_FIRST_RESET is for whole sequences; pass one flag byte per row");
   a.x = x; a.flags = flags; a.y = y; a.h_state = h; a.h_prev = h_in; a.gate_v = gate_v; a.ld_gate = gate_stride;
   a.B = (int)B; a.T = 1;
   a.aligned = is_aligned(x, W, g.bw, elem_size(dtype));
@@ -3251,6 +3271,7 @@ int rglru_hip_steps(const void* x, const void* prep, float* h, const uint8_t* fl
   if (rc) return rc;
   if (B <= 0 || K <= 0) return fail(RGLRU_E_ARG, "steps: K and B must be positive (got %lld, %lld)", (long long)K, (long long)B);
   if (!x || !prep || !h || !y) return fail(RGLRU_E_ARG, "steps: null pointer");
+  if (flags == RGLRU_FLAGS_FIRST_RESET) return fail(RGLRU_E_ARG, "steps: RGLRU_FLAGS_FIRST_RESET is for whole sequences; pass one flag byte per step and row");
   if (K * B * W >= (1ll << 40) || K >= (1ll << 31)) return fail(RGLRU_E_UNSUPPORTED, "steps: tensor too large");
   Geometry g = make_geometry(W, nb);
   FusedArgs a;

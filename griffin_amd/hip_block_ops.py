@@ -13,8 +13,8 @@ from torch import Tensor
 from torch.autograd.function import once_differentiable
 
 from . import _lib
-from .hip_scan import (_DTYPE_CODES, _dtype_code, _on_device, _parameter_operands, _prep_bytes, _ptr, _require_gpu,
-                       _stream_ptr, rglru_backward)
+from .hip_scan import (FIRST_TOKEN_RESET, _DTYPE_CODES, _dtype_code, _flags_ptr, _on_device, _parameter_operands,
+                       _prep_bytes, _ptr, _require_gpu, _stream_ptr, rglru_backward)
 
 
 def max_kernel_size() -> int:
@@ -287,7 +287,9 @@ class _HipBlockForward(torch.autograd.Function):
             raise ValueError("segment_pos must have shape [batch, sequence]")
         if h0 is not None and h0.shape != (B, W):
             raise ValueError(f"initial state must have shape ({B}, {W}), got {tuple(h0.shape)}")
-        if flags is not None and (flags.shape != (B, T) or flags.dtype != torch.uint8 or not flags.is_contiguous()):
+        first_reset = flags is FIRST_TOKEN_RESET
+        if flags is not None and not first_reset and (
+                flags.shape != (B, T) or flags.dtype != torch.uint8 or not flags.is_contiguous()):
             raise ValueError("flags must be a contiguous uint8 tensor of shape [batch, sequence]")
         code = _dtype_code(u.dtype)
         lib = _lib.load()
@@ -309,7 +311,7 @@ class _HipBlockForward(torch.autograd.Function):
             new_conv = u.new_empty(B, taps_count - 1, W)
             h_last = torch.empty(B, W, dtype=torch.float32, device=device)
             ws = torch.empty(lib.rglru_hip_workspace_bytes(B, T, W, nb), dtype=torch.uint8, device=device)
-            tail = (_ptr(h0c), _ptr(flags), _ptr(x_conv), _ptr(y), _ptr(gated), _ptr(new_conv) if taps_count > 1 else None,
+            tail = (_ptr(h0c), _flags_ptr(flags), _ptr(x_conv), _ptr(y), _ptr(gated), _ptr(new_conv) if taps_count > 1 else None,
                     _ptr(h_last), _ptr(ws), B, T, W, nb, code, stream)
             if training or prep is None:
                 operands, vec_code = _parameter_operands(w_a, b_a, w_x, b_x, lam, u.dtype)
@@ -324,7 +326,8 @@ class _HipBlockForward(torch.autograd.Function):
                     _ptr(u_r), u_r.stride(1), _ptr(v_r), v_r.stride(1), _ptr(state_c), _ptr(taps), _ptr(bias_c), taps_count,
                     _DTYPE_CODES[taps.dtype], image.data_ptr(), *tail), "rglru_hip_block_fwd")
         if training:
-            ctx.save_for_backward(u_r, v_r, state_c, taps, pos, x_conv, y, w_a, w_x, h0c, flags, ws, image)
+            ctx.save_for_backward(u_r, v_r, state_c, taps, pos, x_conv, y, w_a, w_x, h0c, None if first_reset else flags, ws, image)
+            ctx.first_reset = first_reset
             ctx.conv_meta = (None if conv_state is None else conv_state.dtype, weight.dtype,
                              None if bias is None else bias.dtype, weight.shape)
             ctx.param_dtypes = (w_a.dtype, b_a.dtype, w_x.dtype, b_x.dtype, lam.dtype)
@@ -337,6 +340,8 @@ class _HipBlockForward(torch.autograd.Function):
     @once_differentiable
     def backward(ctx, dgated, dh_last, _dnew_conv):
         u, v, state, taps, pos, x_conv, y, w_a, w_x, h0c, flags, ws, image = ctx.saved_tensors
+        if ctx.first_reset:
+            flags = FIRST_TOKEN_RESET
         need = ctx.needs_input_grad
         lib = _lib.load()
         dy = dv = None
@@ -377,7 +382,8 @@ def hip_block_forward(u: Tensor, v: Tensor, conv_state: Tensor | None, weight: T
 
     ``u``, ``v`` [B, T, W]: the block's two projections; ``conv_state`` [B, K-1, W] or None; ``weight``
     [W, 1, K], ``bias`` [W] of the depthwise ``nn.Conv1d`` (K <= 4); ``segment_pos`` [B, T]; ``flags``:
-    ``hip_block_flags(segment_pos)`` if the caller has it already, else None; the five RG-LRU parameters, ``h0`` [B, W] or None; ``prep``: a prepared parameter image to use
+    ``hip_block_flags(segment_pos)`` if the caller has it already, ``hip_scan.FIRST_TOKEN_RESET`` when the
+    positions are 0 .. T-1 in every row (no flag tensor is needed then), else None; the five RG-LRU parameters, ``h0`` [B, W] or None; ``prep``: a prepared parameter image to use
     when no gradient is asked for.  Returns ``(gated [B, T, W], final state [B, W] fp32, new_conv_state
     [B, K-1, W])``; differentiable in u, v, the parameters, conv_state and h0.
     """

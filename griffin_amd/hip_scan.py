@@ -70,6 +70,21 @@ def _on_device(device: torch.device):
     return torch.cuda.device(device)
 
 
+class _FirstTokenReset:
+    """In place of a flag tensor: token 0 of every sequence starts a document, no other token carries a flag
+    (RGLRU_FLAGS_FIRST_RESET of the C ABI).  The kernels then run their variants without per-token flags."""
+
+    def __repr__(self):
+        return "FIRST_TOKEN_RESET"
+
+
+FIRST_TOKEN_RESET = _FirstTokenReset()
+
+
+def _flags_ptr(flags) -> int | None:
+    return 1 if flags is FIRST_TOKEN_RESET else _ptr(flags)
+
+
 def _ptr(t: Tensor | None) -> int | None:
     return None if t is None else t.data_ptr()
 
@@ -234,7 +249,7 @@ def _check_fused_inputs(x: Tensor, w_a: Tensor, h0: Tensor | None, flags: Tensor
         raise ValueError(f"gate weights {tuple(w_a.shape)} do not match width {W}")
     if h0 is not None and h0.shape != (B, W):
         raise ValueError(f"initial state must have shape ({B}, {W}), got {tuple(h0.shape)}")
-    if flags is not None and flags.shape != (B, T):
+    if flags is not None and flags is not FIRST_TOKEN_RESET and flags.shape != (B, T):
         raise ValueError(f"token flags must have shape ({B}, {T}), got {tuple(flags.shape)}")
     if T == 0 or B == 0:
         raise ValueError("hip RG-LRU does not accept empty batches or sequences")
@@ -263,7 +278,8 @@ class _HipRGLRU(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, x, w_a, b_a, w_x, b_x, lam, h0, flags, c):
-        _require_gpu("hip RG-LRU", x, w_a, b_a, w_x, b_x, lam, h0, flags)
+        first_reset = flags is FIRST_TOKEN_RESET
+        _require_gpu("hip RG-LRU", x, w_a, b_a, w_x, b_x, lam, h0, None if first_reset else flags)
         _check_fused_inputs(x, w_a, h0, flags)
         lib = _lib.load()
         x = x.contiguous()
@@ -282,17 +298,18 @@ class _HipRGLRU(torch.autograd.Function):
                 pre, _, _ = _gate_projections(x, w_a, w_x)
                 _lib.check(lib.rglru_hip_prepare(*(t.data_ptr() for t in operands), float(c), W, nb, code, vec_code,
                                                  image.data_ptr(), _stream_ptr(device)), "rglru_hip_prepare")
-                _lib.check(lib.rglru_hip_fwd_pre(x.data_ptr(), pre.data_ptr(), image.data_ptr(), _ptr(h0c), _ptr(flags),
+                _lib.check(lib.rglru_hip_fwd_pre(x.data_ptr(), pre.data_ptr(), image.data_ptr(), _ptr(h0c), _flags_ptr(flags),
                                                  y.data_ptr(), h_last.data_ptr(), ws.data_ptr(), B, T, W, nb, code,
                                                  _stream_ptr(device)), "rglru_hip_fwd_pre")
                 del pre
             else:
                 # parameter conversion, workspace clearing and the forward kernel: two launches
                 _lib.check(lib.rglru_hip_prepare_fwd(*(t.data_ptr() for t in operands), float(c), vec_code,
-                                                     image.data_ptr(), x.data_ptr(), _ptr(h0c), _ptr(flags),
+                                                     image.data_ptr(), x.data_ptr(), _ptr(h0c), _flags_ptr(flags),
                                                      y.data_ptr(), h_last.data_ptr(), ws.data_ptr(), B, T, W, nb, code,
                                                      _stream_ptr(device)), "rglru_hip_prepare_fwd")
-        ctx.save_for_backward(x, w_a, w_x, h0c, flags, ws, image, y)
+        ctx.save_for_backward(x, w_a, w_x, h0c, None if first_reset else flags, ws, image, y)
+        ctx.first_reset = first_reset
         ctx.param_dtypes = (w_a.dtype, b_a.dtype, w_x.dtype, b_x.dtype, lam.dtype)
         ctx.h0_dtype = None if h0 is None else h0.dtype
         ctx.set_materialize_grads(False)      # an unused output arrives as None, not as a tensor of zeros
@@ -302,6 +319,8 @@ class _HipRGLRU(torch.autograd.Function):
     @once_differentiable
     def backward(ctx, dy, dh_last):
         x, w_a, w_x, h0c, flags, ws, image, y = ctx.saved_tensors
+        if ctx.first_reset:
+            flags = FIRST_TOKEN_RESET
         dx, dw_a, db_a, dw_x, db_x, dlam, dh0 = rglru_backward(
             x, y, w_a, w_x, h0c, flags, ws, image, dy, dh_last, ctx.param_dtypes, ctx.needs_input_grad[6])
         return (dx, dw_a, db_a, dw_x, db_x, dlam, None if dh0 is None else dh0.to(ctx.h0_dtype), None, None)
@@ -336,7 +355,7 @@ def rglru_backward(x, y, w_a, w_x, h0c, flags, ws, image, dy, dh_last, param_dty
             # everything in hand-written kernels, including the two gate GEMMs
             dw_a = torch.empty(nb, bw, bw, dtype=gdt, device=device)
             dw_x = torch.empty(nb, bw, bw, dtype=gdt, device=device)
-            _lib.check(lib.rglru_hip_bwd_full(x.data_ptr(), y.data_ptr(), image.data_ptr(), _ptr(h0c), _ptr(flags),
+            _lib.check(lib.rglru_hip_bwd_full(x.data_ptr(), y.data_ptr(), image.data_ptr(), _ptr(h0c), _flags_ptr(flags),
                                               dy.data_ptr(), _ptr(dhl), ws.data_ptr(), scratch.data_ptr(), dx.data_ptr(), dw_a.data_ptr(),
                                               dw_x.data_ptr(), db_a.data_ptr(), db_x.data_ptr(), dlam.data_ptr(),
                                               _ptr(dh0), B, T, W, nb, code, gcode, _stream_ptr(device)),
@@ -345,7 +364,7 @@ def rglru_backward(x, y, w_a, w_x, h0c, flags, ws, image, dy, dh_last, param_dty
             # blocks of 160 .. 384 channels: scan and gate math, then the two gate GEMMs, all hand-written
             dw_a = torch.empty(nb, bw, bw, dtype=gdt, device=device)
             dw_x = torch.empty(nb, bw, bw, dtype=gdt, device=device)
-            _lib.check(lib.rglru_hip_bwd_wide(x.data_ptr(), image.data_ptr(), _ptr(h0c), _ptr(flags),
+            _lib.check(lib.rglru_hip_bwd_wide(x.data_ptr(), image.data_ptr(), _ptr(h0c), _flags_ptr(flags),
                                               dy.data_ptr(), _ptr(dhl), ws.data_ptr(), scratch.data_ptr(), dx.data_ptr(), dw_a.data_ptr(),
                                               dw_x.data_ptr(), db_a.data_ptr(), db_x.data_ptr(), dlam.data_ptr(),
                                               _ptr(dh0), B, T, W, nb, code, gcode, _stream_ptr(device)),
@@ -355,7 +374,7 @@ def rglru_backward(x, y, w_a, w_x, h0c, flags, ws, image, dy, dh_last, param_dty
             # HIP kernel, then the two GEMMs of the gate gradients on the kernel's du
             pre, stacked, xk = _gate_projections(x, w_a, w_x)
             du = torch.empty_like(pre)
-            _lib.check(lib.rglru_hip_bwd_pre(x.data_ptr(), pre.data_ptr(), image.data_ptr(), _ptr(h0c), _ptr(flags),
+            _lib.check(lib.rglru_hip_bwd_pre(x.data_ptr(), pre.data_ptr(), image.data_ptr(), _ptr(h0c), _flags_ptr(flags),
                                              dy.data_ptr(), _ptr(dhl), ws.data_ptr(), scratch.data_ptr(), dx.data_ptr(),
                                              du.data_ptr(), db_a.data_ptr(), db_x.data_ptr(), dlam.data_ptr(),
                                              _ptr(dh0), B, T, W, nb, code, gcode, _stream_ptr(device)),
@@ -368,7 +387,7 @@ def rglru_backward(x, y, w_a, w_x, h0c, flags, ws, image, dy, dh_last, param_dty
         else:
             du_a = torch.empty_like(x)
             du_x = torch.empty_like(x)
-            _lib.check(lib.rglru_hip_bwd(x.data_ptr(), image.data_ptr(), _ptr(h0c), _ptr(flags),
+            _lib.check(lib.rglru_hip_bwd(x.data_ptr(), image.data_ptr(), _ptr(h0c), _flags_ptr(flags),
                                          dy.data_ptr(), _ptr(dhl), ws.data_ptr(), scratch.data_ptr(), dx.data_ptr(), du_a.data_ptr(),
                                          du_x.data_ptr(), db_a.data_ptr(), db_x.data_ptr(), dlam.data_ptr(),
                                          _ptr(dh0), B, T, W, nb, code, gcode, _stream_ptr(device)), "rglru_hip_bwd")
@@ -389,10 +408,17 @@ def rglru_backward(x, y, w_a, w_x, h0c, flags, ws, image, dy, dh_last, param_dty
 
 def hip_rglru(x: Tensor, w_a: Tensor, b_a: Tensor, w_x: Tensor, b_x: Tensor, lam: Tensor, c: float = 8.0,
               h0: Tensor | None = None, reset_mask: Tensor | None = None,
-              active_mask: Tensor | None = None) -> tuple[Tensor, Tensor]:
+              active_mask: Tensor | None = None, first_token_reset: bool = False) -> tuple[Tensor, Tensor]:
     """Fused RG-LRU on the GPU: returns (y in x.dtype, final state in fp32).  Differentiable in
-    x, the five parameters and h0 (first order)."""
-    flags = pack_flags(reset_mask, active_mask)
+    x, the five parameters and h0 (first order).  ``first_token_reset`` stands for the reset mask that is True
+    at token 0 of every row and nowhere else (rows that each hold one document from its beginning), without
+    building it: the kernels then run without per-token flags."""
+    if first_token_reset:
+        if reset_mask is not None or active_mask is not None:
+            raise ValueError("first_token_reset replaces the masks; pass one or the other")
+        flags = FIRST_TOKEN_RESET
+    else:
+        flags = pack_flags(reset_mask, active_mask)
     return _HipRGLRU.apply(x, w_a, b_a, w_x, b_x, lam, h0, flags, c)
 
 

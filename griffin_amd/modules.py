@@ -167,9 +167,14 @@ class RG_LRU(nn.Module):
                 y = hip_scan.hip_rglru_step(xt[:, 0], prep, state, None if flags is None else flags.reshape(batch))
                 y = y.unsqueeze(1)
                 return (y, state) if return_state else y
+            # the reset mask of the default positions (a document start at token 0 of every row, nothing else)
+            # is known by identity: the kernels then need no per-token flags at all
+            default = _DEFAULT_POSITIONS.get((batch, steps, xt.device))
+            first_only = default is not None and reset_mask is default[1] and active_mask is None
             y, state = hip_scan.hip_rglru(
                 xt, self.recurrence_gate.weight, self.recurrence_gate.bias, self.input_gate.weight,
-                self.input_gate.bias, self.Lambda, self.c, ht_minus_1, reset_mask, active_mask,
+                self.input_gate.bias, self.Lambda, self.c, ht_minus_1, None if first_only else reset_mask, active_mask,
+                first_token_reset=first_only,
             )
             return (y, state) if return_state else y
 
@@ -214,21 +219,6 @@ def _default_positions(batch: int, steps: int, device: torch.device):
             if len(_DEFAULT_POSITIONS) >= 16:
                 _DEFAULT_POSITIONS.clear()
             _DEFAULT_POSITIONS[key] = hit
-    return hit
-
-
-_DEFAULT_BLOCK_FLAGS: dict = {}
-
-
-def _default_block_flags(batch: int, steps: int, device: torch.device) -> Tensor | None:
-    """Flag bytes of the one-launch block forward for the default positions, built once like them (None
-    while a graph is being captured: the operator then derives them inside the capture)."""
-    key = (batch, steps, device)
-    hit = _DEFAULT_BLOCK_FLAGS.get(key)
-    if hit is None and not torch.cuda.is_current_stream_capturing():
-        if len(_DEFAULT_BLOCK_FLAGS) >= 16:
-            _DEFAULT_BLOCK_FLAGS.clear()
-        hit = _DEFAULT_BLOCK_FLAGS[key] = hip_block_ops.hip_block_flags(_default_positions(batch, steps, device)[0])
     return hit
 
 
@@ -504,7 +494,7 @@ class RecurrentBlock(nn.Module):
                           self.temporal_conv.bias, *self.rg_lru._gate_parameters()))
             gated, new_rnn_state, new_conv_state = hip_block_ops.hip_block_forward(
                 projected, gate_input, conv_state, self.temporal_conv.weight, self.temporal_conv.bias, segment_pos,
-                _default_block_flags(batch, steps, x.device) if (default is not None and segment_pos is default[0]) else None,
+                hip_scan.FIRST_TOKEN_RESET if (cache is None and default is not None and segment_pos is default[0]) else None,
                 *self.rg_lru._gate_parameters(), rnn_state, self.rg_lru.c,
                 None if needs_grad else self.rg_lru._prepared(projected.dtype, projected.device))
         else:

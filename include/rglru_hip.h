@@ -63,6 +63,11 @@ enum {
 
 #define RGLRU_FLAG_RESET 1u
 #define RGLRU_FLAG_INACTIVE 2u
+/* In place of a flag array (the forward and backward entry points of whole sequences, not the decode steps):
+ * token 0 of every sequence carries RGLRU_FLAG_RESET and no other token any flag -- what the recurrent block
+ * passes when every row holds one document from its beginning (griffin/griffin.py:309-338 without cache).  The
+ * kernels then need no per-token flags; rglru_hip_block_fwd also takes the rows' convolution history as empty. */
+#define RGLRU_FLAGS_FIRST_RESET ((const uint8_t*)(uintptr_t)1)
 /* Bits 2-3 of a flag byte are read by rglru_hip_block_fwd only (convolution lags that reach in front of the
  * token's document); every other entry point ignores them. */
 #define RGLRU_FLAG_CONV_SHIFT 2

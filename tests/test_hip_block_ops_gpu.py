@@ -496,10 +496,13 @@ def test_block_forward_matches_the_three_kernels(case):
     B, T, W, nb, K, kind, carried, strided = case
     p = _block_case(B, T, W, nb, K, kind, carried, strided, seed=B + T)
     _say("block forward", case)
+    from griffin_amd.hip_scan import FIRST_TOKEN_RESET
+
     with torch.no_grad():
         want_gated, want_h, want_conv = _three_kernels(p)
         got_gated, got_h, got_conv = hip_block_forward(
-            p["u"], p["v"], p["conv_state"], p["weight"], p["bias"], p["pos"], None,
+            p["u"], p["v"], p["conv_state"], p["weight"], p["bias"], p["pos"],
+            FIRST_TOKEN_RESET if (kind == "fresh" and not carried) else None,   # positions 0 .. T-1: no flag tensor
             p["w_a"], p["b_a"], p["w_x"], p["b_x"], p["lam"], p["h0"], 8.0)
     torch.cuda.synchronize()
     if K > 1:
@@ -516,6 +519,7 @@ def test_block_forward_gradients_match_the_three_kernels(case):
     """Autograd through the one-launch forward (its backward runs gate, scan and convolution reverse kernels
     on the x and y the forward kept) against autograd through the three separate operators."""
     from griffin_amd.hip_block_ops import hip_block_flags, hip_block_forward
+    from griffin_amd.hip_scan import FIRST_TOKEN_RESET
 
     B, T, W, nb, K, kind, carried, strided = case
     p = _block_case(B, T, W, nb, K, kind, carried, strided, seed=B + T)
@@ -532,7 +536,7 @@ def test_block_forward_gradients_match_the_three_kernels(case):
         if fused:
             gated, h_last, carried_rows = hip_block_forward(
                 q["u"], q["v"], q["conv_state"], q["weight"], q["bias"], q["pos"],
-                hip_block_flags(q["pos"]) if B % 2 else None,
+                FIRST_TOKEN_RESET if (kind == "fresh" and not carried) else hip_block_flags(q["pos"]) if B % 2 else None,
                 q["w_a"], q["b_a"], q["w_x"], q["b_x"], q["lam"], q["h0"], 8.0)
         else:
             gated, h_last, carried_rows = _three_kernels(q)

@@ -275,6 +275,59 @@ def test_reproducible_mode_repeats_bit_for_bit(dtype, shape, everything):
         assert rel_err(g.float().cpu(), rgrads[k]) < tol, k
 
 
+@pytest.mark.parametrize("dtype,shape", [
+    (torch.bfloat16, (8, 2048, 1024, 8)),     # plain kernels of the blocks up to 128 channels
+    (torch.bfloat16, (3, 200, 256, 4)),       # their masked variants (ragged last tile), packed 64-wide blocks
+    (torch.bfloat16, (2, 1024, 640, 2)),      # 320-wide blocks
+    (torch.bfloat16, (2, 300, 896, 2)),       # 448-wide blocks: projections by the library
+    (torch.float32, (2, 70, 48, 3)),          # portable kernels
+])
+def test_first_token_reset_equals_the_explicit_mask(dtype, shape):
+    """RGLRU_FLAGS_FIRST_RESET in place of a flag array (`first_token_reset=True`) against the reset mask it
+    stands for, True at token 0 of every row (griffin/griffin.py:248-251 with segment_pos = 0 .. T-1): output,
+    final state and every gradient, with an initial state that the reset has to cut off."""
+    from griffin_amd import hip_rglru
+
+    B, T, W, nb = shape
+    _say("first-token reset", dtype, shape)
+    case = orc.make_case(B, T, W, nb, seed=31, bias_std=0.3)
+    h0 = torch.randn(B, W, generator=torch.Generator().manual_seed(6))
+    dy = case["dy"].to(dtype).cuda()
+    dh = torch.randn(B, W, generator=torch.Generator().manual_seed(7)).cuda()
+    mask = torch.zeros(B, T, dtype=torch.bool)
+    mask[:, 0] = True
+
+    def run(first):
+        leaves = [case[k].to(dtype).cuda().requires_grad_(True) for k in PARAMS]
+        h = h0.cuda().requires_grad_(True)
+        if first:
+            y, h_last = hip_rglru(*leaves, 8.0, h, first_token_reset=True)
+        else:
+            y, h_last = hip_rglru(*leaves, 8.0, h, mask.cuda())
+        grads = torch.autograd.grad([y, h_last], leaves + [h], [dy, dh])
+        torch.cuda.synchronize()
+        return [y.detach(), h_last.detach()] + list(grads)
+
+    want, got = run(False), run(True)
+    tol = 1e-5 if dtype == torch.float32 else 1e-2        # bf16: the two kernel variants may round an output differently
+    for name, a, b in zip(["y", "h_last"] + ["d" + k for k in PARAMS] + ["dh0"], got, want):
+        assert rel_err(a.float(), b.float()) < tol, name
+    assert float(got[-1].abs().max()) < 1e-30             # nothing reaches the state in front of a document start
+    ry, rh, _ = oracle_run(case, dtype, mask, None, None)
+    assert rel_err(got[0].float().cpu(), ry) < (FP32_TOL if dtype == torch.float32 else BF16_TOL)
+
+
+def test_first_token_reset_is_rejected_by_the_decode_steps():
+    from griffin_amd import _lib
+
+    lib = _lib.load()
+    buf = torch.zeros(1 << 14, device="cuda")
+    p = buf.data_ptr()
+    assert lib.rglru_hip_step(p, p, p, 1, p, 4, 64, 2, 0, None) != 0
+    assert b"FIRST_RESET" in lib.rglru_hip_last_error()
+    assert lib.rglru_hip_steps(p, p, p, 1, p, 3, 4, 64, 2, 0, None) != 0
+
+
 def test_reproducible_mode_of_the_scan_only_operator():
     """The scan-only operator (contract of triton_scan.py:274) in reproducible mode: forward and both gradients
     repeat bit for bit and equal the default mode to rounding."""
