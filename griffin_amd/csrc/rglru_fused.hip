@@ -1883,7 +1883,7 @@ __global__ __launch_bounds__(kGradThreads, 1) void gate_grad_wide_kernel(FusedAr
   __shared__ __attribute__((aligned(16))) IO lds_dut[K2 * ROW_T];          // du2 transposed: [kappa][token]
   __shared__ __attribute__((aligned(16))) IO lds_x[TR * ROW_X];
   __shared__ __attribute__((aligned(16))) IO lds_dx[TR * ROW_X];
-  __shared__ __attribute__((aligned(16))) float lds_red[2][3][16][64];     // partial dx tiles of quarters 1..3
+  __shared__ __attribute__((aligned(16))) f32x4 lds_red[2][3][4][64];      // partial dx tiles of quarters 1..3, four registers a vector
   __shared__ __attribute__((aligned(16))) unsigned char stage_all[2 * WaveStage<TR>::kBytes];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, hf = lane >> 5;
@@ -2024,7 +2024,10 @@ __global__ __launch_bounds__(kGradThreads, 1) void gate_grad_wide_kernel(FusedAr
       }
       if (q != 0) {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) lds_red[sl][q - 1][v][lane] = acc[v];
+        for (int v4 = 0; v4 < 4; ++v4) {
+          const f32x4 part = {acc[4 * v4], acc[4 * v4 + 1], acc[4 * v4 + 2], acc[4 * v4 + 3]};
+          lds_red[sl][q - 1][v4][lane] = part;
+        }
       }
     }
     __syncthreads();
@@ -2042,9 +2045,13 @@ __global__ __launch_bounds__(kGradThreads, 1) void gate_grad_wide_kernel(FusedAr
       if (q == 0) {
         unsigned char* my = stage + WaveStage<TR>::row_offset(hf * 16) + r * 2;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const float sum = acc[v] + (lds_red[sl][0][v][lane] + (lds_red[sl][1][v][lane] + lds_red[sl][2][v][lane]));
-          *reinterpret_cast<IO*>(my + v * WaveStage<TR>::kRowBytes) = (IO)sum;
+        for (int v4 = 0; v4 < 4; ++v4) {
+          const f32x4 p0 = lds_red[sl][0][v4][lane], p1 = lds_red[sl][1][v4][lane], p2 = lds_red[sl][2][v4][lane];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const float sum = acc[4 * v4 + e] + (p0[e] + (p1[e] + p2[e]));
+            *reinterpret_cast<IO*>(my + (4 * v4 + e) * WaveStage<TR>::kRowBytes) = (IO)sum;
+          }
         }
         wave_lds_fence();
         const int rows = (int)((rows_total - row0) < TR ? (rows_total - row0) : TR);
