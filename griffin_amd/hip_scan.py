@@ -596,6 +596,46 @@ def _validate_hip_scan(device: torch.device) -> None:
         torch.testing.assert_close(got, want, atol=3e-5 * scale, rtol=3e-5)
 
 
+    # 16-bit storage: the kernels with register-held weights, the convolution, the RG-LRU and the output gate
+    # in one forward launch and their backward, against the same computation in fp32 on the rounded operands
+    from .hip_block_ops import hip_block_forward, hip_block_forward_covers
+
+    if hip_block_forward_covers(W * 2, nb, 4, torch.bfloat16):
+        bf = torch.bfloat16
+        W2, bw2 = W * 2, 2 * bw                                    # 96 channels in 3 blocks of 32
+        k2 = torch.arange(B * T * W2, device=device, dtype=torch.float32)
+        u16 = torch.sin(k2 / 37.0).reshape(B, T, W2).to(bf)
+        v16 = torch.cos(k2 / 23.0).reshape(B, T, W2).to(bf)
+        kw2 = torch.arange(nb * bw2 * bw2, device=device, dtype=torch.float32)
+        params16 = [(0.2 * torch.cos(kw2 / 11.0)).reshape(nb, bw2, bw2).to(bf), torch.cat((b_a, b_a), 1).to(bf),
+                    (0.2 * torch.sin(kw2 / 13.0)).reshape(nb, bw2, bw2).to(bf), torch.cat((b_x, b_x), 1).to(bf),
+                    torch.cat((lam, lam)).to(bf)]
+        taps16 = torch.cat((taps, taps)).to(bf)
+        cbias16 = torch.cat((conv_bias, conv_bias)).to(bf)
+        up16 = torch.cos(k2 / 29.0).reshape(B, T, W2).to(bf)
+
+        def run_block(use_hip):
+            dtype = bf if use_hip else torch.float32
+            leaves = [t.detach().to(dtype).clone().requires_grad_(True) for t in (u16, v16, taps16, cbias16, *params16)]
+            uu, vv, tt, cb, *prm = leaves
+            if use_hip:
+                out, _, _ = hip_block_forward(uu, vv, None, tt, cb, positions, None, *prm, None, 8.0)
+            else:
+                xc, _ = portable.causal_depthwise_conv(uu, torch.zeros(B, 3, W2, device=device), tt, cb, positions)
+                a, z = portable.decay_and_input(xc, *prm, 8.0, positions == 0,
+                                                torch.ones(B, T, dtype=torch.bool, device=device), torch.float32)
+                out = _loop_scan(a, z, torch.zeros(B, W2, device=device)) * torch.nn.functional.gelu(vv, approximate="tanh")
+            return out, torch.autograd.grad(out, leaves, up16.to(dtype))
+
+        ref_o, ref_g = run_block(False)
+        hip_o, hip_g = run_block(True)
+        torch.cuda.synchronize(device)
+        for got, want in zip((hip_o, *hip_g), (ref_o, *ref_g)):
+            err = float((got.float() - want).norm() / want.norm().clamp_min(1e-30))
+            if not err < 2e-2:
+                raise AssertionError(f"16-bit block forward self-test: relative error {err:.3e}")
+
+
 def hip_scan_is_usable(device: torch.device | str) -> bool:
     """Validate the HIP kernels once per device before ``scan_mode="auto"`` may use them."""
     resolved = torch.device(device)
