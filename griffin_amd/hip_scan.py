@@ -631,7 +631,8 @@ def _validate_hip_scan(device: torch.device) -> None:
         hip_o, hip_g = run_block(True)
         torch.cuda.synchronize(device)
         for got, want in zip((hip_o, *hip_g), (ref_o, *ref_g)):
-            err = float((got.float() - want).norm() / want.norm().clamp_min(1e-30))
+            got, want = got.detach().float(), want.detach()
+            err = float((got - want).norm() / want.norm().clamp_min(1e-30))
             if not err < 2e-2:
                 raise AssertionError(f"16-bit block forward self-test: relative error {err:.3e}")
 
