@@ -83,3 +83,39 @@ def test_oversized_sequences_are_rejected_on_the_host(lib):
 def test_spin_limit_hook_round_trips(lib):
     previous = lib.rglru_hip_set_spin_limit(1234)
     assert lib.rglru_hip_set_spin_limit(previous) == 1234
+
+
+def test_reproducible_switch_round_trips(lib):
+    previous = lib.rglru_hip_set_reproducible(1)
+    assert lib.rglru_hip_set_reproducible(previous) == 1
+    assert lib.rglru_hip_set_reproducible(previous) == previous
+
+
+def test_block_forward_queries_and_errors_without_a_gpu(lib):
+    """Where the one-launch block forward applies, and its host-side argument checks (nothing is launched)."""
+    assert lib.rglru_hip_block_fwd_path(1024, 8, 4, _lib.RGLRU_BF16) == 1      # blocks of 128 channels
+    assert lib.rglru_hip_block_fwd_path(1024, 16, 4, _lib.RGLRU_BF16) == 1     # 64
+    assert lib.rglru_hip_block_fwd_path(1024, 32, 1, _lib.RGLRU_BF16) == 1     # 32, a single tap
+    assert lib.rglru_hip_block_fwd_path(2560, 8, 4, _lib.RGLRU_BF16) == 0      # 320: three launches
+    assert lib.rglru_hip_block_fwd_path(1024, 8, 4, _lib.RGLRU_F32) == 0
+    assert lib.rglru_hip_block_fwd_path(1024, 8, 5, _lib.RGLRU_BF16) == 0
+    fake = ctypes.c_void_p(256)            # never dereferenced: the checks come first
+    # (u, u_stride, v, v_stride, conv_state, taps, conv_bias, K, vec_dtype, prep, h0, flags, x_conv, y, gated,
+    #  new_conv_state, h_last, ws, B, T, W, nb, dtype, stream)
+    base = [fake, 0, fake, 0, None, fake, None, 4, _lib.RGLRU_BF16, fake, None, None, None, None, fake, None, None, fake,
+            2, 16, 128, 2, _lib.RGLRU_BF16, None]
+    wide = list(base); wide[20], wide[21] = 640, 2
+    assert lib.rglru_hip_block_fwd(*wide) == 2
+    assert b"block_fwd" in lib.rglru_hip_last_error()
+    no_gate = list(base); no_gate[2] = None
+    assert lib.rglru_hip_block_fwd(*no_gate) == 1
+    short = list(base); short[1] = 64
+    assert lib.rglru_hip_block_fwd(*short) == 1
+    assert b"stride" in lib.rglru_hip_last_error()
+    odd = list(base); odd[0] = ctypes.c_void_p(258)
+    assert lib.rglru_hip_block_fwd(*odd) == 2
+    assert b"aligned" in lib.rglru_hip_last_error()
+    assert lib.rglru_hip_block_flags(None, None, 4, None) == 1
+    # the sentinel for "every row starts a document" is not a flag array of the decode steps
+    assert lib.rglru_hip_step(fake, fake, fake, ctypes.c_void_p(1), fake, 4, 64, 2, _lib.RGLRU_BF16, None) == 1
+    assert b"FIRST_RESET" in lib.rglru_hip_last_error()
