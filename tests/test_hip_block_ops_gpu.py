@@ -553,6 +553,51 @@ def test_block_forward_gradients_match_the_three_kernels(case):
         assert rel_err(a.float().cpu(), b.float().cpu()) < 5e-3, n
 
 
+def test_block_forward_random_shapes():
+    """Forty seeded draws of batch, length, width, gate blocks, taps, position pattern, carried state and row
+    strides: outputs and, for every second draw, gradients against the three separate operators."""
+    import random
+
+    from griffin_amd.hip_block_ops import hip_block_forward
+    from griffin_amd.hip_scan import FIRST_TOKEN_RESET
+
+    rng = random.Random(20)
+    for trial in range(40):
+        bw, nb = rng.choice([32, 64, 128]), rng.choice([1, 2, 3, 5, 8])
+        B, T = rng.choice([1, 2, 3, 7]), rng.choice([1, 2, 3, 5, 31, 64, 65, 127, 128, 200, 257, 500])
+        K, kind = rng.choice([1, 2, 3, 4]), rng.choice(["fresh", "continued", "packed"])
+        carried, strided, with_grads = rng.random() < 0.5, rng.random() < 0.4, trial % 2 == 1
+        _say("block forward draw", trial, (B, T, bw * nb, nb, K, kind, carried, strided, with_grads))
+        p = _block_case(B, T, bw * nb, nb, K, kind, carried, strided, seed=trial)
+        names = [n for n in ("u", "v", "weight", "bias", "w_a", "b_a", "w_x", "b_x", "lam") if p[n] is not None]
+        marker = FIRST_TOKEN_RESET if (kind == "fresh" and not carried) else None
+
+        def run(fused):
+            q = dict(p)
+            for n in names:
+                q[n] = p[n].detach().clone().requires_grad_(with_grads)
+            if fused:
+                outs = hip_block_forward(q["u"], q["v"], q["conv_state"], q["weight"], q["bias"], q["pos"], marker,
+                                         q["w_a"], q["b_a"], q["w_x"], q["b_x"], q["lam"], q["h0"], 8.0)
+            else:
+                outs = _three_kernels(q)
+            got = [o.detach() for o in outs]
+            if with_grads:
+                ups = [torch.full_like(outs[0], 0.5), torch.ones_like(outs[1])]
+                got += list(torch.autograd.grad(list(outs[:2]), [q[n] for n in names], ups))
+            return got
+
+        with torch.set_grad_enabled(with_grads):
+            want, got = run(False), run(True)
+        torch.cuda.synchronize()
+        if K > 1:
+            assert torch.equal(got[2], want[2]), trial
+        for i, (a, b) in enumerate(zip(got, want)):
+            assert a.shape == b.shape, (trial, i)
+            if a.numel():                                    # one tap carries no rows
+                assert rel_err(a.float().cpu(), b.float().cpu()) < 1e-2, (trial, i)
+
+
 def test_block_forward_argument_errors():
     from griffin_amd import _lib
     from griffin_amd.hip_block_ops import hip_block_forward_covers
