@@ -9,6 +9,7 @@ from .hip_scan import (
     hip_rglru_steps,
     hip_scan_available,
     hip_scan_is_usable,
+    set_chain_forward,
     set_reproducible,
 )
 from .hip_block_ops import (hip_block_forward, hip_causal_conv, hip_causal_conv_padded, hip_gelu_gate, hip_linear,
@@ -41,5 +42,6 @@ __all__ = [
     "hip_rglru_steps",
     "hip_scan_available",
     "hip_scan_is_usable",
+    "set_chain_forward",
     "set_reproducible",
 ]

@@ -14,7 +14,7 @@ RGLRU_BF16 = 1
 FLAG_RESET = 1
 FLAG_INACTIVE = 2
 CHUNK = 32
-ABI_VERSION = 15
+ABI_VERSION = 16
 
 _lock = threading.Lock()
 _lib = None
@@ -73,6 +73,7 @@ _SIGNATURES = {
     "rglru_hip_step_gated": (ctypes.c_int, [_P] * 6 + [_I, _P] + [_I, _I, _I, ctypes.c_int, _P]),
     "rglru_hip_set_spin_limit": (ctypes.c_int64, [_I]),
     "rglru_hip_set_reproducible": (ctypes.c_int, [ctypes.c_int]),
+    "rglru_hip_set_chain_forward": (ctypes.c_int, [ctypes.c_int]),
     "rglru_hip_set_timing": (ctypes.c_int, [ctypes.c_int]),
     "rglru_hip_kernel_ms": (ctypes.c_float, [ctypes.c_int]),
     "rglru_hip_workspace_status": (ctypes.c_int, [_P, _I, _I, _I, _I, ctypes.c_int, _P, ctypes.POINTER(ctypes.c_int)]),

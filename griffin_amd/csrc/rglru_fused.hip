@@ -849,6 +849,176 @@ __global__ __launch_bounds__(kThreads, (BLOCK ? 2 : NKG < 0 ? RGLRU_GIVEN_OCC : 
 }
 
 // ------------------------------------------------------------------------------------------
+// Forward for shapes with many chains (sequences x 32-channel slabs: about one per compute unit or more).
+// A workgroup owns ONE chain for the whole sequence, so nothing is exchanged between workgroups: no tickets,
+// no records in memory, no look-back, and the composition order is fixed (results repeat bit for bit).  Its
+// sixteen waves take the chain's 32-token tiles round robin (wave j: tiles j, j + 16, ...).  Each wave stages
+// its own x tiles (32 rows of the block's K range) in a private LDS area, so the loop has no workgroup
+// barrier; the slab's rows of both gate matrices sit in LDS once for all waves, which keeps a wave at 128
+// registers (four waves a SIMD); the output tile is transposed through the x tile's area once that is
+// consumed.  The state goes from tile to tile through LDS: one 8-byte entry {tile number + 1, state} per
+// channel, written by the tile's wave and polled by the wave of the next tile, which is resident by
+// construction.  The slabs of a gate block run as workgroups of one XCD (block index = XCD + 8 * slot), so
+// the x tile they share is fetched from memory once and served to the others by that XCD's L2.
+// Measured at B8 T2048 W1024 (256 chains on 256 compute units): 33 us against 39 us for the tiled kernel
+// with look-back; the vector unit is busy 77 % of the waves' lifetime (4.8 cycles per instruction: a
+// transcendental takes 8.5, 96 of a tile's 429 are).
+// ------------------------------------------------------------------------------------------
+constexpr int kChainWaves = 16;
+
+template <typename IO, int NKG, bool MASKED>
+__global__ __launch_bounds__(kChainWaves * 64, 1) void fwd_chain_kernel(FusedArgs p) {
+  typedef Io<IO> Tr;
+  typedef typename Tr::Frag Frag;
+  static_assert(sizeof(IO) == 2 && (NKG == 8 || NKG == 4 || NKG == 2), "16-bit storage, gate blocks of 128, 64 or 32 channels");
+  constexpr int TR = 32;
+  constexpr int KC = NKG * Tr::KG;                         // block width = K range of the gate products
+  constexpr int S = KC / 32;                               // slabs (chains) per block
+  constexpr int LDSROW = KC + Tr::HW;
+  constexpr int VPR = KC / Tr::HW;                         // 16-byte vectors per tile row
+  constexpr int NV = TR * VPR / 64;                        // vectors per lane and tile
+  static_assert(TR * LDSROW * (int)sizeof(IO) >= WaveStage<TR>::kBytes, "the staging area lies over the x tile");
+  __shared__ __attribute__((aligned(16))) IO lds_all[kChainWaves][TR * LDSROW];
+  __shared__ __attribute__((aligned(16))) IO lds_w[2 * 32 * LDSROW];                // [gate][output channel][K]
+  __shared__ __attribute__((aligned(8))) unsigned long long carry[kChainWaves][32];
+
+  const int tid = threadIdx.x, lane = tid & 63, r = lane & 31, hf = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);   // known to be wave-uniform: what derives from it stays scalar
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int sl = slot % S, u = (slot / S) * 8 + xcd;       // slab of the block; (sequence, block) pair
+  const bool chain_ok = u < p.B * p.nb;                    // the grid is rounded up to whole rounds of eight pairs
+  const int b = chain_ok ? u / p.nb : 0, k = chain_ok ? u - b * p.nb : 0;
+  for (int i = tid; i < kChainWaves * 32; i += kChainWaves * 64) (&carry[0][0])[i] = 0ull;
+  {
+    const IO* wg = (const IO*)p.wg;
+    for (int i = tid; i < 2 * 32 * VPR; i += kChainWaves * 64) {
+      const int gate = i / (32 * VPR), o = (i / VPR) % 32, cv = i % VPR;
+      *reinterpret_cast<Frag*>(lds_w + (gate * 32 + o) * LDSROW + cv * Tr::HW) =
+          *reinterpret_cast<const Frag*>(wg + ((long long)(gate * p.nb + k) * p.bwp + sl * 32 + o) * p.bwp + cv * Tr::HW);
+    }
+  }
+  __syncthreads();
+  if (!chain_ok) return;
+  const int col0 = k * KC;                                 // first channel of the block
+  const int ch = col0 + sl * 32 + r;                       // the lane's channel
+  const long long W = p.W;
+  IO* lds = lds_all[wave];
+  unsigned char* stage = reinterpret_cast<unsigned char*>(lds);
+  const float nba = -kLog2e * p.bias[ch], nbx = -kLog2e * p.bias[p.Wp + ch];
+  const float sp = p.sp[ch];
+  const int nC = (p.T + TR - 1) / TR;
+  const unsigned row_bytes = (unsigned)p.W * 2u;
+  const long long limit = p.limit < 0 ? -p.limit : p.limit;
+
+  Frag pre[NV];
+  unsigned pre_off[NV];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int idx = lane + 64 * i, row = idx / VPR, cv = idx - row * VPR;
+    pre_off[i] = (unsigned)row * row_bytes + (unsigned)(col0 + cv * Tr::HW) * 2u;
+  }
+  const IO* xb = (const IO*)p.x + (long long)b * p.T * W;
+  auto issue = [&](int c) {                                // a tile past the end: empty extent, nothing is fetched
+    const int rows = c >= nC ? 0 : ((p.T - c * TR) < TR ? (p.T - c * TR) : TR);
+    const rsrc_t rx = make_rsrc(xb + (long long)(c < nC ? c : 0) * TR * W, (unsigned)rows * row_bytes);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) pre[i] = buf_load_frag<Frag>(rx, pre_off[i]);
+  };
+  const rsrc_t rck = make_rsrc(p.ckpt + (long long)b * p.ckpt_nC * W, (unsigned)p.ckpt_nC * (unsigned)W * 4u);
+  const rsrc_t rhl = make_rsrc(p.h_last, p.h_last ? (unsigned)p.B * (unsigned)W * 4u : 0u);
+  const int prev_wave = (wave + kChainWaves - 1) % kChainWaves;
+  bool gave_up = false;
+  // initial state of the chain (used by the wave of tile 0 only): no memory operation inside the loop is conditional
+  const float h_first = p.h0 ? p.h0[(long long)b * W + ch] : 0.f;
+  issue(wave);
+  {
+    // The loop's back edge has four stores in flight behind the prefetched tile (final state, checkpoint, two
+    // output segments).  The same four, dropped through their offsets, in front of its entry: the wait for the
+    // tile at the loop's top can then leave the stores in flight on both paths.
+    BufIo<float>::store(0.f, rhl, kOutOfRange, 0u);
+    BufIo<float>::store(0.f, rck, kOutOfRange, 0u);
+    const i32x4 nothing = {0, 0, 0, 0};
+    buf_store_b128(nothing, rck, kOutOfRange);
+    buf_store_b128(nothing, rhl, kOutOfRange);
+  }
+  for (int c = wave; c < nC; c += kChainWaves) {
+    const int t0 = c * TR;
+    unsigned flbits = 0u;
+    if constexpr (MASKED) flbits = flag_run(p, (long long)b * p.T + t0 + hf * 16, t0 + hf * 16);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int idx = lane + 64 * i, row = idx / VPR, cv = idx - row * VPR;
+      *reinterpret_cast<Frag*>(lds + row * LDSROW + cv * Tr::HW) = pre[i];
+    }
+    wave_lds_fence();
+    issue(c + kChainWaves);
+    f32x16 ua, ux;
+    float xv[16], a[16], z[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) { ua[v] = 0.0f; ux[v] = 0.0f; }     // the biases enter inside the sigmoids
+    {
+      const IO* xrow = lds + tile_row<1>(0, r) * LDSROW + hf * Tr::HW;
+      const IO* wrow = lds_w + r * LDSROW + hf * Tr::HW;
+#pragma unroll
+      for (int kg = 0; kg < NKG; ++kg) {
+        const Frag xa = *reinterpret_cast<const Frag*>(xrow + kg * Tr::KG);
+        Tr::mma(ua, xa, *reinterpret_cast<const Frag*>(wrow + kg * Tr::KG));
+        Tr::mma(ux, xa, *reinterpret_cast<const Frag*>(wrow + 32 * LDSROW + kg * Tr::KG));
+      }
+#pragma unroll
+      for (int e = 0; e < 16; ++e) xv[e] = (float)lds[(hf * 16 + e) * LDSROW + sl * 32 + r];
+    }
+    fwd_gates<IO, MASKED>(flbits, ua, ux, xv, sp, a, z, nba, nbx, p.first_reset && c == 0 && hf == 0);
+    // affine map of the lane's 16 tokens, then of the lower half and of the whole tile
+    float A = 1.f, H = 0.f;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) { H = fmaf(a[e], H, z[e]); A *= a[e]; }
+    const float A_o = xhalf(A, hf), H_o = xhalf(H, hf);
+    const float A_lo = hf ? A_o : A, H_lo = hf ? H_o : H;
+    const float A_hi = hf ? A : A_o, H_hi = hf ? H : H_o;
+    const float A_t = A_hi * A_lo, H_t = fmaf(A_hi, H_lo, H_hi);
+    // the state in front of the tile: h0, or what the wave of the tile before has left in LDS.  A wait that
+    // runs out of polls hands on NaN, so the failure shows in the results; every wave still reaches the end.
+    float h_in = h_first;
+    if (c != 0) {
+      long long polls = 0;
+      bool ok;
+      for (;;) {
+        const unsigned long long e = __hip_atomic_load(&carry[prev_wave][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        ok = (unsigned)e == (unsigned)c;
+        h_in = __uint_as_float((unsigned)(e >> 32));
+        if (__all(ok) || ++polls > limit) break;
+        __builtin_amdgcn_s_sleep(1);
+      }
+      gave_up |= !__all(ok);
+      if (!ok) h_in = __builtin_nanf("");
+    }
+    const float h_end = fmaf(A_t, h_in, H_t);
+    const float h_mid = fmaf(A_lo, h_in, H_lo);
+    if (hf == 0) __hip_atomic_store(&carry[wave][r], ((unsigned long long)__float_as_uint(h_end) << 32) | (unsigned long long)(unsigned)(c + 1),
+                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    BufIo<float>::store(h_end, rhl, (hf == 0 && c == nC - 1) ? ((unsigned)b * (unsigned)W + (unsigned)ch) * 4u : kOutOfRange, 0u);
+
+    float h = hf ? h_mid : h_in;
+    const int rows = (p.T - t0) < TR ? (p.T - t0) : TR;
+    const rsrc_t ry = make_rsrc((IO*)p.y + ((long long)b * p.T + t0) * W, (unsigned)rows * row_bytes);
+    wave_lds_fence();                                      // the x tile has been read: its area becomes the staging area
+    unsigned char* my = stage + WaveStage<TR>::row_offset(hf * 16) + r * 2;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      h = fmaf(a[e], h, z[e]);
+      *reinterpret_cast<IO*>(my + e * WaveStage<TR>::kRowBytes) = (IO)h;
+    }
+    // checkpoint for the backward pass: the state after the lane's 16 tokens (slot = token / 16)
+    BufIo<float>::store(h, rck, ((unsigned)(2 * c + hf) * (unsigned)W + (unsigned)ch) * 4u, 0u);
+    wave_lds_fence();
+    stage_flush<TR>(stage, ry, row_bytes, (unsigned)(col0 + sl * 32) * 2u, lane);
+    wave_lds_fence();
+  }
+  if (gave_up && lane == 0) atomicOr(p.fail, 1u);
+}
+
+// ------------------------------------------------------------------------------------------
 // Backward (gate recomputation + reverse scan).  Chunks of 32 tokens, walked from the last to the
 // first.  Emits the direct input gradient, the gradients at both gate pre-activations and
 // per-workgroup partial sums for the bias and Lambda gradients.
@@ -2727,6 +2897,27 @@ struct BlockFwd {
   void* x_conv; void* gated; void* new_conv_state;
 };
 
+// Whether the forward runs one workgroup per chain (fwd_chain_kernel) instead of tiles with look-back:
+// 0 = by shape, 1 = never, 2 = whenever that kernel covers the shape (tests).
+static std::atomic<int> g_chain_forward{0};
+static bool fwd_chain_pays(int64_t B, int64_t T, int64_t W) {
+  const int mode = g_chain_forward.load(std::memory_order_relaxed);
+  if (mode == 1) return false;
+  if (mode == 2) return true;
+  // Its sixteen waves want at least two rounds of tiles, and a workgroup fills a compute unit: the launch
+  // takes ceil(chains / units) rounds, and the tiled kernel (1.18 times slower at equal filling) wins when the
+  // last round is too empty.
+  if (T < 32 * kChainWaves * 2) return false;
+  static const int units = [] {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 0;
+    return n;
+  }();
+  if (units <= 0) return false;
+  const long long chains = B * (W / 32), rounds = (chains + units - 1) / units;
+  return chains * 100 >= rounds * units * 85;
+}
+
 static int fwd_impl(const void* x, const void* prep, const float* h0, const uint8_t* flags,
                     void* y, float* h_last, void* ws,
                     int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, bool cleared, void* stream,
@@ -2781,6 +2972,20 @@ static int fwd_impl(const void* x, const void* prep, const float* h0, const uint
   if (!cleared) {
     rc = launch_clear(wb, L.f_begin, L.b_end, s);       // carry records and tickets of both passes, failure word
     if (rc) return rc;
+  }
+  if (!blk && !pre && (nkg == 8 || nkg == 4 || nkg == 2) && fwd_chain_pays(B, T, W)) {
+    const int S = (int)(g.bw / 32);
+    const dim3 grid((unsigned)(8 * ((B * nb + 7) / 8) * S));
+    const int masked = (flags != nullptr) || (T % 32 != 0);
+    KernelTimer timer(0, s);
+#define RGLRU_CHAIN_CASE(N)                                                                                            \
+    if (nkg == N) {                                                                                                    \
+      if (masked) hipLaunchKernelGGL((fwd_chain_kernel<__bf16, N, true>), grid, dim3(kChainWaves * 64), 0, s, a);      \
+      else hipLaunchKernelGGL((fwd_chain_kernel<__bf16, N, false>), grid, dim3(kChainWaves * 64), 0, s, a);            \
+    }
+    RGLRU_CHAIN_CASE(8) RGLRU_CHAIN_CASE(4) RGLRU_CHAIN_CASE(2)
+#undef RGLRU_CHAIN_CASE
+    return check_launch("fwd");
   }
   pack_units(a, g, nkg);
   const int tile_tokens = 32 * fwd_mt(nkg);
@@ -3310,6 +3515,7 @@ int rglru_hip_steps(const void* x, const void* prep, float* h, const uint8_t* fl
   return check_launch("steps");
 }
 
+int rglru_hip_set_chain_forward(int mode) { return g_chain_forward.exchange(mode < 0 || mode > 2 ? 0 : mode); }
 int rglru_hip_set_timing(int enable) { return g_timing.exchange(enable ? 1 : 0); }
 
 float rglru_hip_kernel_ms(int which) {

@@ -39,6 +39,13 @@ def set_reproducible(enable: bool) -> bool:
     return bool(_lib.load().rglru_hip_set_reproducible(1 if enable else 0))
 
 
+def set_chain_forward(mode: int) -> int:
+    """Choice of the forward kernel for bf16 storage and gate blocks of 32, 64 or 128 channels
+    (rglru_hip_set_chain_forward): 0 = by shape (default), 1 = always tiles with a look-back between
+    workgroups, 2 = one workgroup per chain whenever that kernel covers the shape.  Returns the previous mode."""
+    return int(_lib.load().rglru_hip_set_chain_forward(int(mode)))
+
+
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 _raw_device = getattr(torch._C, "_cuda_getDevice", None)
 

@@ -50,7 +50,7 @@
 extern "C" {
 #endif
 
-#define RGLRU_ABI_VERSION 15
+#define RGLRU_ABI_VERSION 16
 
 enum { RGLRU_F32 = 0, RGLRU_BF16 = 1 };
 
@@ -364,6 +364,13 @@ int64_t rglru_hip_set_spin_limit(int64_t polls);
  * composition follows the ticket order).  The chain becomes one memory round trip per chunk: slower,
  * mostly for long sequences.  Applies to launches made after the call; returns the previous setting. */
 int rglru_hip_set_reproducible(int enable);
+/* Which forward kernel rglru_hip_fwd uses for bf16 storage and gate blocks of 32, 64 or 128 channels (no
+ * counterpart in the reference).  0 (default): by shape -- when the sequences x 32-channel slabs fill the
+ * compute units evenly and the sequence has at least 1024 tokens, one workgroup walks a whole chain (no exchange
+ * between workgroups, bit-reproducible); otherwise tiles with a look-back between workgroups.  1: always the
+ * tiled kernel.  2: the chain kernel whenever it covers the storage type and block width (tests).  Applies to
+ * launches made after the call; returns the previous setting. */
+int rglru_hip_set_chain_forward(int mode);
 /* Synchronising debug helper: copies the failure word of a workspace to the host (0 = clean). */
 int rglru_hip_workspace_status(const void* ws, int64_t B, int64_t T, int64_t W, int64_t nb,
                                int scan_only, void* stream, int* status);

@@ -91,6 +91,12 @@ def test_reproducible_switch_round_trips(lib):
     assert lib.rglru_hip_set_reproducible(previous) == previous
 
 
+def test_chain_forward_switch_round_trips(lib):
+    previous = lib.rglru_hip_set_chain_forward(2)
+    assert lib.rglru_hip_set_chain_forward(7) == 2          # out of range selects the default
+    assert lib.rglru_hip_set_chain_forward(previous) == 0
+
+
 def test_block_forward_queries_and_errors_without_a_gpu(lib):
     """Where the one-launch block forward applies, and its host-side argument checks (nothing is launched)."""
     assert lib.rglru_hip_block_fwd_path(1024, 8, 4, _lib.RGLRU_BF16) == 1      # blocks of 128 channels

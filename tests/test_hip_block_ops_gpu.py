@@ -507,7 +507,8 @@ def test_block_forward_matches_the_three_kernels(case):
     torch.cuda.synchronize()
     if K > 1:
         assert torch.equal(got_conv, want_conv)
-    assert rel_err(got_gated.float().cpu(), want_gated.float().cpu()) < 2e-3
+    # one bf16 rounding step at the largest value is 2^-8 of it
+    assert rel_err(got_gated.float().cpu(), want_gated.float().cpu()) < 5e-3
     assert rel_err(got_h.cpu(), want_h.cpu()) < 1e-5
     # a changed bit here and there, not a systematic difference
     differing = (got_gated != want_gated).float().mean().item()

@@ -360,6 +360,107 @@ def test_reproducible_mode_of_the_scan_only_operator():
         assert rel_err(a, b) < 1e-5
 
 
+# ------------------------------------------------------------------ one workgroup per chain (fwd_chain_kernel)
+CHAIN_CASES = [
+    # B, T, W, nb, masks, carried state
+    (2, 64, 128, 1, False, False),
+    (3, 1, 256, 2, False, True),
+    (2, 31, 128, 4, True, False),
+    (3, 33, 192, 3, False, True),
+    (2, 200, 256, 8, True, True),
+    (5, 1000, 256, 2, True, True),
+    (2, 1537, 128, 1, False, False),
+    (8, 2048, 1024, 8, False, False),
+    (8, 2048, 1024, 16, True, True),
+]
+
+
+@pytest.mark.parametrize("cfg", CHAIN_CASES)
+def test_chain_forward_matches_tiled_forward_and_oracle(cfg):
+    """bf16 storage, gate blocks of 32/64/128 channels: the forward that walks a whole chain in one workgroup
+    (mode 2) against the tiled forward with look-back (mode 1) and, on sizes the oracle finishes quickly,
+    against the oracle (griffin/griffin.py:237-289); the backward runs on the checkpoints each of them left."""
+    from griffin_amd import set_chain_forward
+
+    B, T, W, nb, masks, carried = cfg
+    _say("chain forward", cfg)
+    case = orc.make_case(B, T, W, nb, seed=B + T, lo=0.9, hi=0.999)
+    gen = torch.Generator().manual_seed(T)
+    if carried:
+        case["h0"] = torch.randn(B, W, generator=gen)
+    reset = active = None
+    if masks:
+        reset = torch.rand(B, T, generator=gen) < 0.05
+        active = torch.ones(B, T, dtype=torch.bool)
+        active[0, T // 2:] = False                       # a right-padded row
+    dh = torch.randn(B, W, generator=gen)
+    was = set_chain_forward(2)
+    try:
+        y, h_last, grads = hip_run(case, torch.bfloat16, reset, active, dh)
+        set_chain_forward(1)
+        ty, th, tgrads = hip_run(case, torch.bfloat16, reset, active, dh)
+    finally:
+        set_chain_forward(was)
+    assert rel_err(y.float(), ty.float()) < 5e-3          # one bf16 rounding step at the largest value is 2^-8 of it
+    assert rel_err(h_last, th) < 1e-5
+    for k in grads:
+        assert rel_err(grads[k].float(), tgrads[k].float()) < 1e-2, k
+    if B * T * W <= 3 * 1024 * 1024:
+        ry, rh, rgrads = oracle_run(case, torch.bfloat16, reset, active, dh)
+        assert rel_err(y.float().cpu(), ry) < BF16_TOL and rel_err(h_last.cpu(), rh) < BF16_TOL
+        for k in grads:
+            assert rel_err(grads[k].float().cpu(), rgrads[k]) < BF16_TOL, k
+
+
+def test_chain_forward_repeats_bit_for_bit_and_is_the_default_at_the_training_shape():
+    """The chain kernel composes carries in a fixed order, so repeated runs agree bit for bit without the
+    reproducible mode; at B8 T2048 W1024 (256 chains) the default mode selects it."""
+    from griffin_amd import hip_rglru, set_chain_forward
+
+    case = orc.make_case(8, 2048, 1024, 8, seed=3, lo=0.9, hi=0.999)
+    leaves = [case[k].bfloat16().cuda() for k in PARAMS]
+
+    def run():
+        with torch.no_grad():
+            y, h_last = hip_rglru(*leaves, 8.0)
+        torch.cuda.synchronize()
+        return y, h_last
+
+    default = run()
+    was = set_chain_forward(2)
+    try:
+        runs = [run() for _ in range(3)]
+    finally:
+        set_chain_forward(was)
+    for y, h_last in runs + [default]:
+        assert torch.equal(y, runs[0][0]) and torch.equal(h_last, runs[0][1])
+
+
+def test_chain_forward_that_gives_up_poisons_its_results():
+    """A wave that runs out of polls while it waits for the tile before hands on NaN and sets the failure word
+    (forced from the host with a one-poll budget; every wave still finishes)."""
+    from griffin_amd import _lib, hip_rglru, set_chain_forward
+
+    lib = _lib.load()
+    case = orc.make_case(4, 4096, 256, 2, seed=1)
+    leaves = [case[k].bfloat16().cuda() for k in PARAMS]
+    was = set_chain_forward(2)
+    previous = lib.rglru_hip_set_spin_limit(1)
+    try:
+        with torch.no_grad():
+            y, h_last = hip_rglru(*leaves, 8.0)
+        torch.cuda.synchronize()
+    finally:
+        lib.rglru_hip_set_spin_limit(previous)
+        set_chain_forward(was)
+    gave_up = not bool(torch.isfinite(h_last).all())
+    if gave_up:                                           # whether a wait runs out is a matter of timing
+        assert not bool(torch.isfinite(y.float()).all())
+    with torch.no_grad():
+        y2, h2 = hip_rglru(*leaves, 8.0)                  # the budget is back: clean results
+    assert bool(torch.isfinite(y2.float()).all()) and bool(torch.isfinite(h2).all())
+
+
 # ------------------------------------------------------------------ golden vectors of the reference
 @pytest.mark.parametrize("name", ["rglru_plain_b2_t16_w32", "rglru_masks_b2_t16_w32", "rglru_odd_b3_t37_w65"])
 def test_fused_matches_reference_golden_vectors(golden_dir, name):
