@@ -1684,6 +1684,183 @@ __global__ __launch_bounds__(kThreads, (MT == 1 ? 4 : RGLRU_DELTA_OCC)) void bwd
   }
 }
 
+// The reverse scan with one workgroup per chain, the counterpart of fwd_chain_kernel: sixteen waves take the
+// chain's 32-token tiles round robin from the last tile to the first, the recurrence gate's rows of the slab
+// sit in LDS, and the carry goes from tile c + 1 to tile c through LDS.  A wave stages its own x tile (the
+// block's K range) and its own 32 channels of dy; delta leaves through the x tile's area.
+template <typename IO, int NKG, bool MASKED>
+__global__ __launch_bounds__(kChainWaves * 64, 1) void bwd_delta_chain_kernel(FusedArgs p) {
+  typedef Io<IO> Tr;
+  typedef typename Tr::Frag Frag;
+  static_assert(sizeof(IO) == 2 && (NKG == 8 || NKG == 4 || NKG == 2), "16-bit storage, gate blocks of 128, 64 or 32 channels");
+  constexpr int TR = 32;
+  constexpr int KC = NKG * Tr::KG;
+  constexpr int S = KC / 32;
+  constexpr int LDSROW = KC + Tr::HW;
+  constexpr int VPR = KC / Tr::HW;
+  constexpr int NV = TR * VPR / 64;
+  constexpr int DYROW = 32 + Tr::HW;                       // the wave's 32 channels of dy, padded
+  static_assert(TR * LDSROW * (int)sizeof(IO) >= WaveStage<TR>::kBytes, "the staging area lies over the x tile");
+  __shared__ __attribute__((aligned(16))) IO lds_all[kChainWaves][TR * LDSROW];
+  __shared__ __attribute__((aligned(16))) IO lds_w[32 * LDSROW];                    // [output channel][K], recurrence gate
+  __shared__ __attribute__((aligned(8))) unsigned long long carry[kChainWaves][32];
+
+  const int tid = threadIdx.x, lane = tid & 63, r = lane & 31, hf = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int sl = slot % S, u = (slot / S) * 8 + xcd;
+  const bool chain_ok = u < p.B * p.nb;
+  const int b = chain_ok ? u / p.nb : 0, k = chain_ok ? u - b * p.nb : 0;
+  for (int i = tid; i < kChainWaves * 32; i += kChainWaves * 64) (&carry[0][0])[i] = 0ull;
+  {
+    const IO* wg = (const IO*)p.wg;
+    for (int i = tid; i < 32 * VPR; i += kChainWaves * 64) {
+      const int o = i / VPR, cv = i % VPR;
+      *reinterpret_cast<Frag*>(lds_w + o * LDSROW + cv * Tr::HW) =
+          *reinterpret_cast<const Frag*>(wg + ((long long)(0 * p.nb + k) * p.bwp + sl * 32 + o) * p.bwp + cv * Tr::HW);
+    }
+  }
+  __syncthreads();
+  if (!chain_ok) return;
+  const int col0 = k * KC;
+  const int ch = col0 + sl * 32 + r;
+  const long long W = p.W;
+  IO* lds = lds_all[wave];
+  IO* lds_dy = lds;                                        // dy takes the x tile's place once the gate products have read it
+  unsigned char* stage = reinterpret_cast<unsigned char*>(lds);
+  const float nba = -kLog2e * p.bias[ch];
+  const float sp = p.sp[ch];
+  const int nC = (p.T + TR - 1) / TR;
+  const unsigned row_bytes = (unsigned)p.W * 2u;
+  const long long limit = p.limit < 0 ? -p.limit : p.limit;
+
+  Frag pre[NV], pre_dy[2];
+  unsigned pre_off[NV], dy_off[2];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int idx = lane + 64 * i, row = idx / VPR, cv = idx - row * VPR;
+    pre_off[i] = (unsigned)row * row_bytes + (unsigned)(col0 + cv * Tr::HW) * 2u;
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {                            // 32 rows x four 16-byte vectors
+    const int idx = lane + 64 * i, row = idx >> 2, cv = idx & 3;
+    dy_off[i] = (unsigned)row * row_bytes + (unsigned)(col0 + sl * 32 + cv * Tr::HW) * 2u;
+  }
+  const IO* xb = (const IO*)p.x + (long long)b * p.T * W;
+  const IO* dyb = (const IO*)p.dy + (long long)b * p.T * W;
+  auto issue = [&](int c) {                                // a tile in front of the first: empty extent, nothing is fetched
+    const int rows = c < 0 ? 0 : ((p.T - c * TR) < TR ? (p.T - c * TR) : TR);
+    const long long first = (long long)(c < 0 ? 0 : c) * TR * W;
+    const rsrc_t rx = make_rsrc(xb + first, (unsigned)rows * row_bytes);
+    const rsrc_t rdy = make_rsrc(dyb + first, (unsigned)rows * row_bytes);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) pre[i] = buf_load_frag<Frag>(rx, pre_off[i]);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) pre_dy[i] = buf_load_frag<Frag>(rdy, dy_off[i]);
+  };
+  const rsrc_t rh0 = make_rsrc(p.dh0, p.dh0 ? (unsigned)p.B * (unsigned)W * 4u : 0u);
+  const int next_wave = (wave + kChainWaves - 1) % kChainWaves;    // the wave of tile c + 1
+  bool gave_up = false;
+  // carry into the chain's last tile (used by its wave only): no memory operation inside the loop is conditional
+  const float d_first = p.dh_last ? p.dh_last[(long long)b * W + ch] : 0.f;
+  issue(nC - 1 - wave);
+  {
+    // the stores the loop's back edge has in flight behind the prefetched tiles (dh0, two delta segments),
+    // dropped through their offsets, in front of its entry (see fwd_chain_kernel)
+    BufIo<float>::store(0.f, rh0, kOutOfRange, 0u);
+    const i32x4 nothing = {0, 0, 0, 0};
+    buf_store_b128(nothing, rh0, kOutOfRange);
+    buf_store_b128(nothing, rh0, kOutOfRange + 16u);
+  }
+  for (int c = nC - 1 - wave; c >= 0; c -= kChainWaves) {
+    const int t0 = c * TR;
+    unsigned flbits = 0u;
+    if constexpr (MASKED) flbits = flag_run(p, (long long)b * p.T + t0 + hf * 16, t0 + hf * 16);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int idx = lane + 64 * i, row = idx / VPR, cv = idx - row * VPR;
+      *reinterpret_cast<Frag*>(lds + row * LDSROW + cv * Tr::HW) = pre[i];
+    }
+    wave_lds_fence();
+    f32x16 ua;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) ua[v] = 0.0f;             // the bias enters inside the sigmoid
+    {
+      const IO* xrow = lds + tile_row<1>(0, r) * LDSROW + hf * Tr::HW;
+      const IO* wrow = lds_w + r * LDSROW + hf * Tr::HW;
+      Frag xa[NKG];
+#pragma unroll
+      for (int kg = 0; kg < NKG; ++kg) xa[kg] = *reinterpret_cast<const Frag*>(xrow + kg * Tr::KG);
+      wave_lds_fence();                                    // the x tile is in registers: dy may take its place
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const int idx = lane + 64 * i, row = idx >> 2, cv = idx & 3;
+        *reinterpret_cast<Frag*>(lds_dy + row * DYROW + cv * Tr::HW) = pre_dy[i];
+      }
+#pragma unroll
+      for (int kg = 0; kg < NKG; ++kg) Tr::mma(ua, xa[kg], *reinterpret_cast<const Frag*>(wrow + kg * Tr::KG));
+    }
+    wave_lds_fence();
+    issue(c - kChainWaves);
+    float a[16], gy[16];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      float l2 = sigmoid_fast(ua[v], nba) * sp;
+      if constexpr (MASKED) l2 = masked_log2_decay_run(l2, flbits, v);
+      else if (v == 0) l2 = (p.first_reset && c == 0 && hf == 0) ? kResetLog2 : l2;
+      a[v] = __builtin_amdgcn_exp2f(l2);
+      gy[v] = (float)lds_dy[(hf * 16 + v) * DYROW + r];
+    }
+    // reverse affine map of this lane's run and of the tile: carry_out = A carry_in + D
+    float A = 1.f, run = 0.f;
+#pragma unroll
+    for (int e = 15; e >= 0; --e) { const float d = gy[e] + run; run = a[e] * d; A *= a[e]; }
+    const float D = run;
+    const float A_o = xhalf(A, hf), D_o = xhalf(D, hf);
+    const float A_lo = hf ? A_o : A, A_hi = hf ? A : A_o;
+    const float D_lo = hf ? D_o : D, D_hi = hf ? D : D_o;
+    const float A_t = A_lo * A_hi, D_t = fmaf(A_lo, D_hi, D_lo);
+    // the carry behind the tile: dh_last, or what the wave of tile c + 1 has left in LDS (entry tag = c + 2)
+    float d_in = d_first;
+    if (c != nC - 1) {
+      long long polls = 0;
+      bool ok;
+      for (;;) {
+        const unsigned long long e = __hip_atomic_load(&carry[next_wave][r], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        ok = (unsigned)e == (unsigned)(c + 2);
+        d_in = __uint_as_float((unsigned)(e >> 32));
+        if (__all(ok) || ++polls > limit) break;
+        __builtin_amdgcn_s_sleep(1);
+      }
+      gave_up |= !__all(ok);
+      if (!ok) d_in = __builtin_nanf("");
+    }
+    const float d_out = fmaf(A_t, d_in, D_t);
+    if (hf == 0) __hip_atomic_store(&carry[wave][r], ((unsigned long long)__float_as_uint(d_out) << 32) | (unsigned long long)(unsigned)(c + 1),
+                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    BufIo<float>::store(d_out, rh0, (hf == 0 && c == 0) ? ((unsigned)b * (unsigned)W + (unsigned)ch) * 4u : kOutOfRange, 0u);
+
+    // delta of every token, through the x tile's area, as 16-byte row segments
+    run = hf ? d_in : fmaf(A_hi, d_in, D_hi);
+    wave_lds_fence();                                      // dy has been read: its area becomes the staging area
+    unsigned char* my = stage + WaveStage<TR>::row_offset(hf * 16) + r * 2;
+#pragma unroll
+    for (int e = 15; e >= 0; --e) {
+      const float d = gy[e] + run;
+      run = a[e] * d;
+      *reinterpret_cast<IO*>(my + e * WaveStage<TR>::kRowBytes) = (IO)d;
+    }
+    wave_lds_fence();
+    {
+      const int rows = (p.T - t0) < TR ? (p.T - t0) : TR;
+      const rsrc_t rd = make_rsrc((const IO*)p.du_a + ((long long)b * p.T + t0) * W, (unsigned)rows * row_bytes);
+      stage_flush<TR>(stage, rd, row_bytes, (unsigned)(col0 + sl * 32) * 2u, lane);
+    }
+    wave_lds_fence();
+  }
+  if (gave_up && lane == 0) atomicOr(p.fail, 1u);
+}
+
 constexpr int kGradWaves = 8;                            // waves per workgroup of the gradient kernel
 constexpr int kGradThreads = 64 * kGradWaves;
 
@@ -3286,7 +3463,17 @@ int rglru_hip_bwd_full(const void* x, const void* y, const void* prep, const flo
   a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
   const bool masked = (flags != nullptr) || (T % (32 * kDeltaMT) != 0);
   dim3 grid((unsigned)(a.wg_per_unit * a.units));
-  {
+  if (fwd_chain_pays(B, T, W)) {
+    // enough chains to give every compute unit one of its own (see fwd_impl)
+    const dim3 cgrid((unsigned)(8 * ((B * nb + 7) / 8) * (g.bw / 32)));
+    const bool cmasked = (flags != nullptr) || (T % 32 != 0);
+    KernelTimer timer(1, s);
+#define RGLRU_LAUNCH_DELTA_CHAIN(N)                                                                                  \
+    if (cmasked) hipLaunchKernelGGL((bwd_delta_chain_kernel<__bf16, N, true>), cgrid, dim3(kChainWaves * 64), 0, s, a); \
+    else hipLaunchKernelGGL((bwd_delta_chain_kernel<__bf16, N, false>), cgrid, dim3(kChainWaves * 64), 0, s, a)
+    if (nkg == 8) { RGLRU_LAUNCH_DELTA_CHAIN(8); } else if (nkg == 4) { RGLRU_LAUNCH_DELTA_CHAIN(4); } else { RGLRU_LAUNCH_DELTA_CHAIN(2); }
+#undef RGLRU_LAUNCH_DELTA_CHAIN
+  } else {
     KernelTimer timer(1, s);
 #define RGLRU_LAUNCH_DELTA(N)                                                                                        \
     if (masked) hipLaunchKernelGGL((bwd_delta_kernel<__bf16, N, true, kDeltaMT>), grid, dim3(kThreads), 0, s, a);      \
