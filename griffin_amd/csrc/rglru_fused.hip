@@ -153,6 +153,9 @@ struct FusedArgs {
   void* x_out; void* conv_new_state; void* gated;
   long long ld_x;                                         // elements between rows of x (>= W)
   int conv_k, conv_vec_dtype;
+  // chain forward that also prepares (rglru_hip_prepare_fwd): the caller's parameters, the image to build from
+  // them and the workspace region to zero, all in the forward launch
+  PrepArgs prep;
   // workspace
   float* ckpt; rec_t* rec_a; unsigned* ticket;
   unsigned* fail; float* partial; float* dw_partial;
@@ -866,7 +869,9 @@ __global__ __launch_bounds__(kThreads, (BLOCK ? 2 : NKG < 0 ? RGLRU_GIVEN_OCC : 
 // ------------------------------------------------------------------------------------------
 constexpr int kChainWaves = 16;
 
-template <typename IO, int NKG, bool MASKED>
+// PREP: the launch also does what prepare_kernel does (the parameter image for the backward kernels, the zeroed
+// workspace region) and takes its own weights, biases and decay constants straight from the caller's parameters.
+template <typename IO, int NKG, bool MASKED, bool PREP = false>
 __global__ __launch_bounds__(kChainWaves * 64, 1) void fwd_chain_kernel(FusedArgs p) {
   typedef Io<IO> Tr;
   typedef typename Tr::Frag Frag;
@@ -889,23 +894,59 @@ __global__ __launch_bounds__(kChainWaves * 64, 1) void fwd_chain_kernel(FusedArg
   const bool chain_ok = u < p.B * p.nb;                    // the grid is rounded up to whole rounds of eight pairs
   const int b = chain_ok ? u / p.nb : 0, k = chain_ok ? u - b * p.nb : 0;
   for (int i = tid; i < kChainWaves * 32; i += kChainWaves * 64) (&carry[0][0])[i] = 0ull;
+  if constexpr (PREP) {
+    // The workspace region that starts out zero, shared among the workgroups of the first round (at most one per
+    // compute unit): a later round would wipe a failure word that a workgroup of an earlier one has set.
+    const int sweepers = gridDim.x < 256 ? (int)gridDim.x : 256;
+    if ((int)blockIdx.x < sweepers)
+      for (long long z = (long long)blockIdx.x * (kChainWaves * 64) + tid; z < p.prep.clear_n; z += (long long)sweepers * (kChainWaves * 64))
+        p.prep.clear[z] = make_uint4(0u, 0u, 0u, 0u);
+  }
   {
-    const IO* wg = (const IO*)p.wg;
     for (int i = tid; i < 2 * 32 * VPR; i += kChainWaves * 64) {
       const int gate = i / (32 * VPR), o = (i / VPR) % 32, cv = i % VPR;
-      *reinterpret_cast<Frag*>(lds_w + (gate * 32 + o) * LDSROW + cv * Tr::HW) =
-          *reinterpret_cast<const Frag*>(wg + ((long long)(gate * p.nb + k) * p.bwp + sl * 32 + o) * p.bwp + cv * Tr::HW);
+      const IO* wg = PREP ? (const IO*)(gate ? p.prep.w_x : p.prep.w_a) + ((long long)k * p.bwp + sl * 32 + o) * p.bwp
+                          : (const IO*)p.wg + ((long long)(gate * p.nb + k) * p.bwp + sl * 32 + o) * p.bwp;
+      *reinterpret_cast<Frag*>(lds_w + (gate * 32 + o) * LDSROW + cv * Tr::HW) = *reinterpret_cast<const Frag*>(wg + cv * Tr::HW);
     }
   }
   __syncthreads();
   if (!chain_ok) return;
+  if constexpr (PREP) {
+    if (b == 0) {
+      // The first sequence's workgroups write the image of their slab: the rows of both matrices as they are,
+      // the transposed and gate-interleaved copy w2t[k][j][2 o + gate] (one 32-bit pair per (j, o)), and the
+      // per-channel constants.
+      IO* wg_out = (IO*)p.prep.wg;
+      for (int i = tid; i < 2 * 32 * VPR; i += kChainWaves * 64) {
+        const int gate = i / (32 * VPR), o = (i / VPR) % 32, cv = i % VPR;
+        *reinterpret_cast<Frag*>(wg_out + ((long long)(gate * p.nb + k) * p.bwp + sl * 32 + o) * p.bwp + cv * Tr::HW) =
+            *reinterpret_cast<const Frag*>(lds_w + (gate * 32 + o) * LDSROW + cv * Tr::HW);
+      }
+      unsigned* w2t = (unsigned*)p.prep.w2t;
+      const unsigned short* lw = (const unsigned short*)lds_w;
+      for (int i = tid; i < KC * 32; i += kChainWaves * 64) {
+        const int j = i >> 5, o = i & 31;
+        const unsigned pair = (unsigned)lw[o * LDSROW + j] | ((unsigned)lw[(32 + o) * LDSROW + j] << 16);
+        w2t[((long long)k * p.bwp + j) * p.bwp + sl * 32 + o] = pair;
+      }
+      if (tid < 32) prepare_channel(p.prep, k * p.bwp + sl * 32 + tid);
+    }
+  }
   const int col0 = k * KC;                                 // first channel of the block
   const int ch = col0 + sl * 32 + r;                       // the lane's channel
   const long long W = p.W;
   IO* lds = lds_all[wave];
   unsigned char* stage = reinterpret_cast<unsigned char*>(lds);
-  const float nba = -kLog2e * p.bias[ch], nbx = -kLog2e * p.bias[p.Wp + ch];
-  const float sp = p.sp[ch];
+  float nba, nbx, sp;
+  if constexpr (PREP) {                                    // the constants prepare_channel derives, for this lane's channel
+    nba = -kLog2e * load_vec(p.prep.b_a, ch, p.prep.vec_dtype);
+    nbx = -kLog2e * load_vec(p.prep.b_x, ch, p.prep.vec_dtype);
+    sp = p.prep.c * log_sigmoid(load_vec(p.prep.lambda, ch, p.prep.vec_dtype)) * kLog2e;
+  } else {
+    nba = -kLog2e * p.bias[ch]; nbx = -kLog2e * p.bias[p.Wp + ch];
+    sp = p.sp[ch];
+  }
   const int nC = (p.T + TR - 1) / TR;
   const unsigned row_bytes = (unsigned)p.W * 2u;
   const long long limit = p.limit < 0 ? -p.limit : p.limit;
@@ -3014,9 +3055,10 @@ size_t rglru_hip_prep_bytes(int64_t W, int64_t nb, int dtype) {
   return make_prep_layout(make_geometry(W, nb), elem_size(dtype)).total;
 }
 
-static int prepare_impl(const void* w_a, const void* b_a, const void* w_x, const void* b_x,
-                        const void* lambda, float c, int64_t W, int64_t nb, int dtype, int vec_dtype,
-                        void* prep, void* clear, size_t clear_bytes, void* stream) {
+// The arguments of a parameter conversion (validated), and its launch.
+static int build_prep_args(const void* w_a, const void* b_a, const void* w_x, const void* b_x,
+                           const void* lambda, float c, int64_t W, int64_t nb, int dtype, int vec_dtype,
+                           void* prep, void* clear, size_t clear_bytes, PrepArgs& a) {
   int rc = check_geometry("prepare", W, nb, dtype);
   if (rc) return rc;
   if (vec_dtype != RGLRU_F32 && vec_dtype != RGLRU_BF16) return fail(RGLRU_E_ARG, "prepare: unknown vector dtype %d", vec_dtype);
@@ -3024,7 +3066,6 @@ static int prepare_impl(const void* w_a, const void* b_a, const void* w_x, const
   Geometry g = make_geometry(W, nb);
   PrepLayout pl = make_prep_layout(g, elem_size(dtype));
   char* pb = (char*)prep;
-  PrepArgs a;
   a.w_a = w_a; a.w_x = w_x; a.b_a = b_a; a.b_x = b_x; a.lambda = lambda;
   a.wg = pb + pl.wg; a.bias = (float*)(pb + pl.bias); a.sp = (float*)(pb + pl.sp); a.cs = (float*)(pb + pl.cs);
   a.dsp = (float*)(pb + pl.dsp); a.vec_dtype = vec_dtype;
@@ -3033,13 +3074,27 @@ static int prepare_impl(const void* w_a, const void* b_a, const void* w_x, const
   a.clear = (uint4*)clear; a.clear_n = (long long)(clear_bytes / 16);
   a.vec_ok = dtype == RGLRU_BF16 && g.bw == g.bwp && g.bw % 8 == 0 && (uintptr_t)w_a % 16 == 0 && (uintptr_t)w_x % 16 == 0 &&
              (uintptr_t)a.wg % 16 == 0 && (uintptr_t)a.w2t % 16 == 0;
-  long long total = a.vec_ok ? 4 * g.nb * g.bwp * g.bwp / 8 + g.Wp : 4 * g.nb * g.bwp * g.bwp + g.Wp;
+  return RGLRU_OK;
+}
+
+static int launch_prepare(const PrepArgs& a, int dtype, void* stream) {
+  const long long cells = (long long)a.nb * a.bwp * a.bwp;
+  long long total = a.vec_ok ? 4 * cells / 8 + a.Wp : 4 * cells + a.Wp;
   if (a.clear_n > total) total = a.clear_n;
   int blocks = (int)((total + 255) / 256); if (blocks > 2048) blocks = 2048;
   hipStream_t s = (hipStream_t)stream;
   if (dtype == RGLRU_BF16) hipLaunchKernelGGL(prepare_kernel<__bf16>, dim3(blocks), dim3(256), 0, s, a);
   else hipLaunchKernelGGL(prepare_kernel<float>, dim3(blocks), dim3(256), 0, s, a);
   return check_launch("prepare");
+}
+
+static int prepare_impl(const void* w_a, const void* b_a, const void* w_x, const void* b_x,
+                        const void* lambda, float c, int64_t W, int64_t nb, int dtype, int vec_dtype,
+                        void* prep, void* clear, size_t clear_bytes, void* stream) {
+  PrepArgs a;
+  const int rc = build_prep_args(w_a, b_a, w_x, b_x, lambda, c, W, nb, dtype, vec_dtype, prep, clear, clear_bytes, a);
+  if (rc) return rc;
+  return launch_prepare(a, dtype, stream);
 }
 
 int rglru_hip_prepare(const void* w_a, const void* b_a, const void* w_x, const void* b_x,
@@ -3098,7 +3153,7 @@ static bool fwd_chain_pays(int64_t B, int64_t T, int64_t W) {
 static int fwd_impl(const void* x, const void* prep, const float* h0, const uint8_t* flags,
                     void* y, float* h_last, void* ws,
                     int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, bool cleared, void* stream,
-                    const void* pre = nullptr, const BlockFwd* blk = nullptr) {
+                    const void* pre = nullptr, const BlockFwd* blk = nullptr, const PrepArgs* fuse = nullptr) {
   int rc = check_geometry("fwd", W, nb, dtype);
   if (rc) return rc;
   if (B <= 0 || T <= 0) return fail(RGLRU_E_ARG, "fwd: B and T must be positive (got %lld, %lld)", (long long)B, (long long)T);
@@ -3150,18 +3205,29 @@ static int fwd_impl(const void* x, const void* prep, const float* h0, const uint
     rc = launch_clear(wb, L.f_begin, L.b_end, s);       // carry records and tickets of both passes, failure word
     if (rc) return rc;
   }
-  if (!blk && !pre && (nkg == 8 || nkg == 4 || nkg == 2) && fwd_chain_pays(B, T, W)) {
+  // fuse: the parameter conversion (and the clearing of the workspace region it names) still has to happen.  The
+  // chain kernel does both itself when the caller's weights can be read as 16-byte vectors; else one launch first.
+  const bool chain = !blk && !pre && (nkg == 8 || nkg == 4 || nkg == 2) && fwd_chain_pays(B, T, W);
+  const bool fused_prepare = fuse && chain && fuse->vec_ok;
+  if (fuse && !fused_prepare) {
+    rc = launch_prepare(*fuse, dtype, stream);
+    if (rc) return rc;
+  }
+  if (chain) {
     const int S = (int)(g.bw / 32);
     const dim3 grid((unsigned)(8 * ((B * nb + 7) / 8) * S));
     const int masked = (flags != nullptr) || (T % 32 != 0);
+    if (fused_prepare) a.prep = *fuse;
     KernelTimer timer(0, s);
+#define RGLRU_CHAIN_LAUNCH(N, M, P) hipLaunchKernelGGL((fwd_chain_kernel<__bf16, N, M, P>), grid, dim3(kChainWaves * 64), 0, s, a)
 #define RGLRU_CHAIN_CASE(N)                                                                                            \
     if (nkg == N) {                                                                                                    \
-      if (masked) hipLaunchKernelGGL((fwd_chain_kernel<__bf16, N, true>), grid, dim3(kChainWaves * 64), 0, s, a);      \
-      else hipLaunchKernelGGL((fwd_chain_kernel<__bf16, N, false>), grid, dim3(kChainWaves * 64), 0, s, a);            \
+      if (fused_prepare) { if (masked) RGLRU_CHAIN_LAUNCH(N, true, true); else RGLRU_CHAIN_LAUNCH(N, false, true); }   \
+      else { if (masked) RGLRU_CHAIN_LAUNCH(N, true, false); else RGLRU_CHAIN_LAUNCH(N, false, false); }               \
     }
     RGLRU_CHAIN_CASE(8) RGLRU_CHAIN_CASE(4) RGLRU_CHAIN_CASE(2)
 #undef RGLRU_CHAIN_CASE
+#undef RGLRU_CHAIN_LAUNCH
     return check_launch("fwd");
   }
   pack_units(a, g, nkg);
@@ -3313,11 +3379,13 @@ int rglru_hip_prepare_fwd(const void* w_a, const void* b_a, const void* w_x, con
   if (rc) return rc;
   if (B <= 0 || T <= 0) return fail(RGLRU_E_ARG, "prepare_fwd: B and T must be positive (got %lld, %lld)", (long long)B, (long long)T);
   if (!ws) return fail(RGLRU_E_ARG, "prepare_fwd: null pointer");
-  // one launch converts the parameters and zeroes the records, tickets and failure word of `ws`
+  // The parameter conversion also zeroes the records, tickets and failure word of `ws`.  It is a launch of its
+  // own in front of the forward kernel, or part of the forward launch where that kernel can do it (fwd_impl).
   const WorkLayout L = make_work_layout(B, T, make_geometry(W, nb));
-  rc = prepare_impl(w_a, b_a, w_x, b_x, lambda, c, W, nb, dtype, vec_dtype, prep, (char*)ws + L.f_begin, L.b_end - L.f_begin, stream);
+  PrepArgs pa;
+  rc = build_prep_args(w_a, b_a, w_x, b_x, lambda, c, W, nb, dtype, vec_dtype, prep, (char*)ws + L.f_begin, L.b_end - L.f_begin, pa);
   if (rc) return rc;
-  return fwd_impl(x, prep, h0, flags, y, h_last, ws, B, T, W, nb, dtype, true, stream);
+  return fwd_impl(x, prep, h0, flags, y, h_last, ws, B, T, W, nb, dtype, true, stream, nullptr, nullptr, &pa);
 }
 
 int rglru_hip_block_fwd(const void* u, int64_t u_stride, const void* v, int64_t v_stride,
