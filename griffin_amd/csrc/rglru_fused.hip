@@ -3531,7 +3531,8 @@ int rglru_hip_bwd_full(const void* x, const void* y, const void* prep, const flo
   a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
   const bool masked = (flags != nullptr) || (T % (32 * kDeltaMT) != 0);
   dim3 grid((unsigned)(a.wg_per_unit * a.units));
-  if (fwd_chain_pays(B, T, W)) {
+  const bool chain_scan = fwd_chain_pays(B, T, W);
+  if (chain_scan) {
     // enough chains to give every compute unit one of its own (see fwd_impl)
     const dim3 cgrid((unsigned)(8 * ((B * nb + 7) / 8) * (g.bw / 32)));
     const bool cmasked = (flags != nullptr) || (T % 32 != 0);
@@ -3573,7 +3574,8 @@ int rglru_hip_bwd_full(const void* x, const void* y, const void* prep, const flo
   r.dw_partial = a.dw_partial; r.dw_a = dw_a; r.dw_x = dw_x;
   r.W = (int)W; r.nb = (int)nb; r.bw = (int)g.bw; r.bwp = (int)g.bwp; r.Wp = (int)g.Wp; r.wg_per_unit = n_wg;
   r.n_wg = n_wg; r.vec_blocks = (int)((W + 15) / 16); r.grad_dtype = grad_dtype; r.dw_bf16 = a.dw_bf16;
-  r.clean = (uint4*)(wb + L.b_begin); r.clean_n = (long long)((L.b_end - L.b_begin) / 16);
+  // the chain scan writes no records and takes no tickets: the region is as clean as it was on entry
+  r.clean = (uint4*)(wb + L.b_begin); r.clean_n = chain_scan ? 0 : (long long)((L.b_end - L.b_begin) / 16);
   const long long total = nb * g.bw * 2 * g.bw;
   hipLaunchKernelGGL(finish_kernel, dim3((unsigned)(r.vec_blocks + (total / 4 + 255) / 256)), dim3(256), 0, s, r);
   return check_launch("bwd_full finish");
