@@ -310,7 +310,8 @@ class _HipRGLRU(torch.autograd.Function):
                                                  _stream_ptr(device)), "rglru_hip_fwd_pre")
                 del pre
             else:
-                # parameter conversion, workspace clearing and the forward kernel: two launches
+                # parameter conversion, workspace clearing and the forward kernel: two launches, or one where the
+                # forward kernel does all three (batch-rich shapes)
                 _lib.check(lib.rglru_hip_prepare_fwd(*(t.data_ptr() for t in operands), float(c), vec_code,
                                                      image.data_ptr(), x.data_ptr(), _ptr(h0c), _flags_ptr(flags),
                                                      y.data_ptr(), h_last.data_ptr(), ws.data_ptr(), B, T, W, nb, code,

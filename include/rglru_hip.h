@@ -138,10 +138,11 @@ int rglru_hip_fwd_static(const void* x, const void* prep, const float* h0, const
                          void* y, float* h_last,
                          int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, void* stream);
 
-/* rglru_hip_prepare followed by rglru_hip_fwd on the same stream with one launch fewer: the
- * parameter conversion and the clearing of the workspace share a kernel.  For training, where
- * every forward (griffin/griffin.py:237-289) sees freshly updated parameters; `prep` is written
- * and stays valid for the matching backward call. */
+/* rglru_hip_prepare followed by rglru_hip_fwd on the same stream with fewer launches: the
+ * parameter conversion and the clearing of the workspace share a kernel, and where the forward runs
+ * one workgroup per chain (see rglru_hip_set_chain_forward) that kernel is the forward kernel itself,
+ * one launch in all.  For training, where every forward (griffin/griffin.py:237-289) sees freshly
+ * updated parameters; `prep` is written and stays valid for the matching backward call. */
 int rglru_hip_prepare_fwd(const void* w_a, const void* b_a, const void* w_x, const void* b_x,
                           const void* lambda, float c, int vec_dtype, void* prep,
                           const void* x, const float* h0, const uint8_t* flags,
