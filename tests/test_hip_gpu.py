@@ -436,6 +436,51 @@ def test_chain_forward_repeats_bit_for_bit_and_is_the_default_at_the_training_sh
         assert torch.equal(y, runs[0][0]) and torch.equal(h_last, runs[0][1])
 
 
+@pytest.mark.parametrize("shape", [(2, 96, 256, 2), (3, 40, 192, 6), (2, 64, 128, 1)])
+@pytest.mark.parametrize("vec_dtype", [torch.float32, torch.bfloat16])
+def test_chain_forward_builds_the_same_parameter_image_as_prepare(shape, vec_dtype):
+    """rglru_hip_prepare_fwd on the chain path converts the parameters inside the forward launch: the image it
+    leaves for the backward kernels is byte for byte the one rglru_hip_prepare writes, and the workspace region
+    it has to zero is zero."""
+    from griffin_amd import _lib, set_chain_forward
+
+    lib = _lib.load()
+    B, T, W, nb = shape
+    case = orc.make_case(B, T, W, nb, seed=4, bias_std=0.3)
+    x, w_a, w_x = (case[k].bfloat16().cuda() for k in ("x", "w_a", "w_x"))
+    b_a, b_x, lam = (case[k].to(vec_dtype).cuda() for k in ("b_a", "b_x", "lam"))
+    code = _lib.RGLRU_BF16
+    vec_code = _lib.RGLRU_BF16 if vec_dtype == torch.bfloat16 else _lib.RGLRU_F32
+    n_img = lib.rglru_hip_prep_bytes(W, nb, code)
+    n_ws = lib.rglru_hip_workspace_bytes(B, T, W, nb)
+    stream = torch.cuda.current_stream().cuda_stream
+    want = torch.full((n_img,), 0x5A, dtype=torch.uint8, device="cuda")
+    got = torch.full((n_img,), 0xA5, dtype=torch.uint8, device="cuda")
+    _lib.check(lib.rglru_hip_prepare(w_a.data_ptr(), b_a.data_ptr(), w_x.data_ptr(), b_x.data_ptr(), lam.data_ptr(), 8.0,
+                                     W, nb, code, vec_code, want.data_ptr(), stream), "rglru_hip_prepare")
+    ws = torch.full((n_ws,), 0x77, dtype=torch.uint8, device="cuda")
+    y = torch.empty_like(x)
+    h_last = torch.empty(B, W, device="cuda")
+    was = set_chain_forward(2)
+    try:
+        _lib.check(lib.rglru_hip_prepare_fwd(w_a.data_ptr(), b_a.data_ptr(), w_x.data_ptr(), b_x.data_ptr(), lam.data_ptr(), 8.0,
+                                             vec_code, got.data_ptr(), x.data_ptr(), None, None, y.data_ptr(), h_last.data_ptr(),
+                                             ws.data_ptr(), B, T, W, nb, code, stream), "rglru_hip_prepare_fwd")
+    finally:
+        set_chain_forward(was)
+    torch.cuda.synchronize()
+    # the image has padding between its parts that neither call writes: compare what rglru_hip_prepare wrote
+    written = want != 0x5A
+    assert bool(written.any())
+    assert torch.equal(got[written], want[written])
+    # checkpoints come first in the workspace; everything behind them is the region that starts out zero
+    ckpt_bytes = B * 2 * (2 * ((T + 63) // 64)) * W * 4
+    assert int(ws[ckpt_bytes + 256:].count_nonzero()) == 0
+    ry, rh = orc.rglru_forward(*[case[k].bfloat16().float() for k in ("x", "w_a")], case["b_a"].to(vec_dtype).float(),
+                               case["w_x"].bfloat16().float(), case["b_x"].to(vec_dtype).float(), case["lam"].to(vec_dtype).float())
+    assert rel_err(y.float().cpu(), ry) < BF16_TOL and rel_err(h_last.cpu(), rh) < BF16_TOL
+
+
 def test_chain_forward_that_gives_up_poisons_its_results():
     """A wave that runs out of polls while it waits for the tile before hands on NaN and sets the failure word
     (forced from the host with a one-poll budget; every wave still finishes)."""
