@@ -3136,10 +3136,10 @@ static bool fwd_chain_pays(int64_t B, int64_t T, int64_t W) {
   const int mode = g_chain_forward.load(std::memory_order_relaxed);
   if (mode == 1) return false;
   if (mode == 2) return true;
-  // Its sixteen waves want at least two rounds of tiles, and a workgroup fills a compute unit: the launch
-  // takes ceil(chains / units) rounds, and the tiled kernel (1.18 times slower at equal filling) wins when the
-  // last round is too empty.
-  if (T < 32 * kChainWaves * 2) return false;
+  // A workgroup fills a compute unit, so the launch takes ceil(chains / units) rounds, and the tiled kernel (1.18
+  // times slower at equal filling) wins when the last round is too empty.  Measured at W1024: with one or two
+  // rounds the chain kernels are ahead from 256 tokens on (8 tiles for 16 waves), with more rounds from 1024 on.
+  if (T < 256) return false;
   static const int units = [] {
     int dev = 0, n = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 0;
@@ -3147,6 +3147,7 @@ static bool fwd_chain_pays(int64_t B, int64_t T, int64_t W) {
   }();
   if (units <= 0) return false;
   const long long chains = B * (W / 32), rounds = (chains + units - 1) / units;
+  if (T < 1024 && rounds > 2) return false;
   return chains * 100 >= rounds * units * 85;
 }
 
