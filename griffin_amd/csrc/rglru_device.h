@@ -353,6 +353,21 @@ RGLRU_DEVICE float one_minus_exp(float y, float a) {
   }
 }
 
+// g^2 = 1 - a^2 for a = 2^l2, l2 <= 0.  PRECISE: the series above in y = 2 ln2 l2, clamped at zero.  Otherwise the
+// two-term series written as a polynomial in l2 itself, -y (1 + y / 2) = l2 (k1 + k2 l2), so that no product
+// with 2 ln2 is spent on an argument; neither branch can turn negative for l2 <= 0 (a <= 1), so there is no clamp
+// (a NaN then stays a NaN instead of turning into g = 0).
+template <bool PRECISE>
+RGLRU_DEVICE float one_minus_a2(float l2, float a) {
+  if constexpr (PRECISE) {
+    return fmaxf(one_minus_exp<true>(l2 * (2.0f * kLn2), a), 0.0f);
+  } else {
+    constexpr float k1 = -2.0f * kLn2, k2 = -2.0f * kLn2 * kLn2;
+    const float series = l2 * fmaf(l2, k2, k1);
+    return l2 > -0.0078125f / (2.0f * kLn2) ? series : fmaf(-a, a, 1.0f);
+  }
+}
+
 // log2 of the decay under the token's flags.  Both masks of the reference act through it alone:
 //   padding (a <- 1, z <- 0): log2 a = 0 gives a = 1 and, through the series branch of
 //     one_minus_exp, g = 0 exactly, hence z = 0;
@@ -382,7 +397,7 @@ RGLRU_DEVICE GateOut gate_outputs(float r, float i, float x, float l2) {
   GateOut o;
   o.r = r; o.i = i;
   const float a = __builtin_amdgcn_exp2f(l2);
-  const float g2 = fmaxf(one_minus_exp<PRECISE>(l2 * (2.0f * kLn2), a), 0.0f);
+  const float g2 = one_minus_a2<PRECISE>(l2, a);
   const float g = __builtin_amdgcn_sqrtf(g2);
   o.g2 = g2;
   o.a = a; o.g = g; o.z = g * i * x;

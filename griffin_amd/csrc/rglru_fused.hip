@@ -894,14 +894,10 @@ __global__ __launch_bounds__(kChainWaves * 64, 1) void fwd_chain_kernel(FusedArg
   const bool chain_ok = u < p.B * p.nb;                    // the grid is rounded up to whole rounds of eight pairs
   const int b = chain_ok ? u / p.nb : 0, k = chain_ok ? u - b * p.nb : 0;
   for (int i = tid; i < kChainWaves * 32; i += kChainWaves * 64) (&carry[0][0])[i] = 0ull;
-  if constexpr (PREP) {
-    // The workspace region that starts out zero, shared among the workgroups of the first round (at most one per
-    // compute unit): a later round would wipe a failure word that a workgroup of an earlier one has set.
-    const int sweepers = gridDim.x < 256 ? (int)gridDim.x : 256;
-    if ((int)blockIdx.x < sweepers)
-      for (long long z = (long long)blockIdx.x * (kChainWaves * 64) + tid; z < p.prep.clear_n; z += (long long)sweepers * (kChainWaves * 64))
-        p.prep.clear[z] = make_uint4(0u, 0u, 0u, 0u);
-  }
+  // The chain kernels use no carry records and no tickets: all this pass needs from the workspace is a failure word
+  // that starts out zero.  Workgroup 0 clears it in its first instructions; a workgroup sets it only after it
+  // has walked its whole chain, by which time that store has long landed.
+  if (blockIdx.x == 0 && tid == 0) __hip_atomic_store(p.fail, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   {
     for (int i = tid; i < 2 * 32 * VPR; i += kChainWaves * 64) {
       const int gate = i / (32 * VPR), o = (i / VPR) % 32, cv = i % VPR;
@@ -1461,7 +1457,7 @@ __global__ __launch_bounds__(kThreads, (NKG > 8 ? 1 : 2)) void bwd_scan_kernel(F
       const float ie = sigmoid_fast(ux[e], nbx);
       float l2 = r[e] * sp;
       if constexpr (MASKED) l2 = masked_log2_decay_run(l2, flbits, e);     // gives g = 1 / g = 0
-      const float ge = __builtin_amdgcn_sqrtf(fmaxf(one_minus_exp<false>(l2 * (2.0f * kLn2), a[e]), 0.0f));
+      const float ge = __builtin_amdgcn_sqrtf(one_minus_a2<false>(l2, a[e]));
       gi[e] = ie; g[e] = ge;
     }
     issue(tk_next);
@@ -2075,8 +2071,7 @@ __global__ __launch_bounds__(kGradThreads, 1) void bwd_grad_kernel(FusedArgs p) 
           if constexpr (MASKED) l2 = masked_log2_decay_run(l2, flbits, v);
           else if (v == 0) l2 = (p.first_reset && c == 0 && hf == 0) ? kResetLog2 : l2;
           const float ae = __builtin_amdgcn_exp2f(l2);
-          // l2 <= 0 and a <= 1, so neither branch of one_minus_exp can turn negative: no clamp needed
-          const float g2 = one_minus_exp<false>(l2 * (2.0f * kLn2), ae);
+          const float g2 = one_minus_a2<false>(l2, ae);
           const float ge = __builtin_amdgcn_sqrtf(g2);
           // With z = g i x, a = exp(l), g = sqrt(1 - a^2) (bounded derivative 1 / sqrt(max(4 g^2, 1e-6))):
           //   dx_direct = delta g i,  di = delta g x,  dl = delta a (h_{t-1} - a i x / sqrt(max(g^2, 2.5e-7)))
@@ -2126,7 +2121,7 @@ __global__ __launch_bounds__(kGradThreads, 1) void bwd_grad_kernel(FusedArgs p) 
 #pragma unroll
       for (int kg = 0; kg < NKG2; ++kg) w2[kg] = *reinterpret_cast<const Frag*>(row + kg * Tr::KG);
     }
-    f32x16 dw[2][S];                                     // [gate][input slab of the block] x own output slab
+    f32x16 dw[2][S];                                     // [gate][input slab js of the block]: rows = own output channels, columns = j
 #pragma unroll
     for (int g = 0; g < 2; ++g)
 #pragma unroll
@@ -2186,8 +2181,8 @@ __global__ __launch_bounds__(kGradThreads, 1) void bwd_grad_kernel(FusedArgs p) 
           for (int js = 0; js < S; ++js) xt[js] = lds_xt[prev][blk * S + js][q][lane];
 #pragma unroll
           for (int js = 0; js < S; ++js) {
-            Tr::mma(dw[0][js], xt[js], ba);
-            Tr::mma(dw[1][js], xt[js], bx);
+            Tr::mma(dw[0][js], ba, xt[js]);
+            Tr::mma(dw[1][js], bx, xt[js]);
           }
         }
         // input gradient of this slab's channels: direct part + du . w2t^T.  The A fragments are
@@ -2220,20 +2215,35 @@ __global__ __launch_bounds__(kGradThreads, 1) void bwd_grad_kernel(FusedArgs p) 
       __syncthreads();
     }
     if (slab_ok) {
-      // per-workgroup partial of the weight gradients: [wg][k][gate][j][o]
+      // per-workgroup partial of the weight gradients, laid out like the gradients themselves: [wg][k][gate][o][j].
+      // Register v of an accumulator is row o = 8 (v / 4) + 4 hf + v % 4 of the wave's slab, the lane's r its column j.
+      // 16-bit partials cross the wave's staging area and leave as 16-byte row segments.
 #pragma unroll
       for (int g = 0; g < 2; ++g) {
-        const long long first = ((((long long)wg_in_unit * p.nb + k) * 2 + g) * p.bwp) * p.bwp;
-        float* part = p.dw_partial + first;
-        __bf16* part16 = (__bf16*)p.dw_partial + first;
+        const long long first = ((((long long)wg_in_unit * p.nb + k) * 2 + g) * p.bwp + sl * 32) * p.bwp;
+        if (p.dw_bf16) {
+          const rsrc_t rp = make_rsrc((__bf16*)p.dw_partial + first, 32u * (unsigned)p.bwp * 2u);
 #pragma unroll
-        for (int js = 0; js < S; ++js)
+          for (int js = 0; js < S; ++js) {
 #pragma unroll
-          for (int v = 0; v < 16; ++v) {
-            const int j = js * 32 + 8 * (v >> 2) + 4 * hf + (v & 3);
-            if (p.dw_bf16) part16[(long long)j * p.bwp + sl * 32 + r] = (__bf16)dw[g][js][v];
-            else part[(long long)j * p.bwp + sl * 32 + r] = dw[g][js][v];
+            for (int v = 0; v < 16; ++v) {
+              const int o = 8 * (v >> 2) + 4 * hf + (v & 3);
+              *reinterpret_cast<IO*>(stage + WaveStage<TR>::row_offset(o) + r * 2) = (IO)dw[g][js][v];
+            }
+            wave_lds_fence();
+            stage_flush<TR>(stage, rp, (unsigned)p.bwp * 2u, (unsigned)(js * 32) * 2u, lane);
+            wave_lds_fence();
           }
+        } else {
+          float* part = p.dw_partial + first;
+#pragma unroll
+          for (int js = 0; js < S; ++js)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+              const int o = 8 * (v >> 2) + 4 * hf + (v & 3);
+              part[(long long)o * p.bwp + js * 32 + r] = dw[g][js][v];
+            }
+        }
       }
     }
   }
@@ -2449,7 +2459,8 @@ __global__ __launch_bounds__(kGradThreads, 1) void gate_grad_wide_kernel(FusedAr
       }
     }
   }
-  // per-workgroup partial of the weight gradients: [wg][k][gate][j][o]
+  // per-workgroup partial of the weight gradients, laid out like the gradients themselves: [wg][k][gate][o][j];
+  // a lane's registers 4 v4 .. 4 v4 + 3 are four consecutive input channels j of its (gate, o)
   if (slab_ok) {
     float* part = p.dw_partial + ((long long)wg_in_unit * p.nb + k) * 2 * p.bwp * p.bwp;
 #pragma unroll
@@ -2458,9 +2469,10 @@ __global__ __launch_bounds__(kGradThreads, 1) void gate_grad_wide_kernel(FusedAr
       if (kt < NKT) {
         const int kappa = kt * 32 + r, o = kappa >> 1, gate = kappa & 1;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int j = j0 + 8 * (v >> 2) + 4 * hf + (v & 3);
-          part[((long long)gate * p.bwp + j) * p.bwp + o] = dw[i][v];
+        for (int v4 = 0; v4 < 4; ++v4) {
+          const int j = j0 + 8 * v4 + 4 * hf;
+          const f32x4 four = {dw[i][4 * v4], dw[i][4 * v4 + 1], dw[i][4 * v4 + 2], dw[i][4 * v4 + 3]};
+          *reinterpret_cast<f32x4*>(part + ((long long)gate * p.bwp + o) * p.bwp + j) = four;
         }
       }
     }
@@ -2469,75 +2481,80 @@ __global__ __launch_bounds__(kGradThreads, 1) void gate_grad_wide_kernel(FusedAr
 
 // Last launch of a backward pass: sums the per-workgroup partial results and writes the parameter
 // gradients in the caller's type.  Workgroups [0, vec_blocks) own 16 channels each of db_a, db_x and
-// dLambda; the rest (fast backward only) own 1024 elements each of the two weight gradients,
-// dW_gate[k][o][j] = sum over workgroups of the partials [wg][k][gate][j][o].
+// dLambda; the rest (backward paths with their own weight-gradient GEMM) own 2048 elements each of the two weight
+// gradients, dW_gate[k][o][j] = sum over workgroups of the partials [wg][k][gate][o][j].
 struct FinishArgs {
   const float* partial; const float* dsp; void* db_a; void* db_x; void* dlambda;
   const float* dw_partial; void* dw_a; void* dw_x;
   int W, nb, bw, bwp, Wp, wg_per_unit, n_wg, vec_blocks, grad_dtype, dw_bf16;
-  uint4* clean; long long clean_n;                         // backward records and tickets, zeroed for the next pass
 };
 
 __global__ __launch_bounds__(256) void finish_kernel(FinishArgs p) {
   __shared__ float part_sum[3][16][16];
-  // the scan kernels of this pass are done: leave their records and tickets zeroed, so that another
-  // backward pass over the same forward needs no clearing launch of its own
-  for (long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x; i < p.clean_n; i += (long long)gridDim.x * blockDim.x)
-    p.clean[i] = make_uint4(0u, 0u, 0u, 0u);
   if ((int)blockIdx.x >= p.vec_blocks) {
-    // four consecutive output channels o of one (block, gate, input channel j) per thread, 16-byte
-    // loads; bw is a multiple of 32 on this path, so a group of four never crosses a row
-    const long long total4 = (long long)p.nb * 2 * p.bw * p.bw / 4;
-    const long long i4 = (long long)(blockIdx.x - p.vec_blocks) * blockDim.x + threadIdx.x;
-    if (i4 >= total4) return;
-    const long long i = i4 * 4;
-    const int o = (int)(i % p.bw);
-    const int j = (int)((i / p.bw) % p.bw);
-    const int gate = (int)((i / ((long long)p.bw * p.bw)) % 2);
-    const int k = (int)(i / ((long long)2 * p.bw * p.bw));
-    const long long stride = (long long)p.nb * 2 * p.bwp * p.bwp;
-    const float* src = p.dw_partial + i;
-    // fixed summation order; eight loads in flight per thread
-    float4 s0 = make_float4(0.f, 0.f, 0.f, 0.f), s1 = s0;
-    int g = 0;
+    // eight consecutive input channels j of one (block, gate, output channel o) per thread: the partials are laid
+    // out like the gradients, so this is a streaming sum in a fixed order with 16-byte accesses (bw is a multiple
+    // of 32 on these paths and equals the padded width)
+    const long long per_gate = (long long)p.bw * p.bw;
+    const long long total8 = (long long)p.nb * 2 * per_gate / 8;
+    const long long i8 = (long long)(blockIdx.x - p.vec_blocks) * blockDim.x + threadIdx.x;
+    if (i8 >= total8) return;
+    const long long i = i8 * 8;
+    const int gate = (int)((i / per_gate) % 2);
+    const long long k = i / (2 * per_gate);
+    const long long stride = (long long)p.nb * 2 * per_gate;
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
     if (p.dw_bf16) {
-      typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
       const __bf16* src16 = (const __bf16*)p.dw_partial + i;
-      for (; g + 7 < p.n_wg; g += 8) {
-        bf16x4 v[8];
+      int g = 0;
+      for (; g + 7 < p.n_wg; g += 8) {                       // eight loads in flight per thread
+        bf16x8 v[8];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const bf16x4*>(src16 + (long long)(g + u) * stride);
+        for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const bf16x8*>(src16 + (long long)(g + u) * stride);
 #pragma unroll
-        for (int u = 0; u < 8; u += 2) {
-          s0.x += (float)v[u][0]; s0.y += (float)v[u][1]; s0.z += (float)v[u][2]; s0.w += (float)v[u][3];
-          s1.x += (float)v[u + 1][0]; s1.y += (float)v[u + 1][1]; s1.z += (float)v[u + 1][2]; s1.w += (float)v[u + 1][3];
-        }
+        for (int u = 0; u < 8; ++u)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[e] += (float)v[u][e];
       }
       for (; g < p.n_wg; ++g) {
-        const bf16x4 v = *reinterpret_cast<const bf16x4*>(src16 + (long long)g * stride);
-        s0.x += (float)v[0]; s0.y += (float)v[1]; s0.z += (float)v[2]; s0.w += (float)v[3];
-      }
-    }
-    for (; g + 7 < p.n_wg; g += 8) {
-      float4 v[8];
+        const bf16x8 v = *reinterpret_cast<const bf16x8*>(src16 + (long long)g * stride);
 #pragma unroll
-      for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const float4*>(src + (long long)(g + u) * stride);
-#pragma unroll
-      for (int u = 0; u < 8; u += 2) {
-        s0.x += v[u].x; s0.y += v[u].y; s0.z += v[u].z; s0.w += v[u].w;
-        s1.x += v[u + 1].x; s1.y += v[u + 1].y; s1.z += v[u + 1].z; s1.w += v[u + 1].w;
+        for (int e = 0; e < 8; ++e) acc[e] += (float)v[e];
       }
-    }
-    for (; g < p.n_wg; ++g) {
-      const float4 v = *reinterpret_cast<const float4*>(src + (long long)g * stride);
-      s0.x += v.x; s0.y += v.y; s0.z += v.z; s0.w += v.w;
+    } else {
+      const float* src = p.dw_partial + i;
+      int g = 0;
+      for (; g + 3 < p.n_wg; g += 4) {
+        f32x4 v[4][2];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          v[u][0] = *reinterpret_cast<const f32x4*>(src + (long long)(g + u) * stride);
+          v[u][1] = *reinterpret_cast<const f32x4*>(src + (long long)(g + u) * stride + 4);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) acc[e] += v[u][e >> 2][e & 3];
+      }
+      for (; g < p.n_wg; ++g) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] += src[(long long)g * stride + e];
+      }
     }
     void* dst = gate ? p.dw_x : p.dw_a;
-    const long long o0 = ((long long)k * p.bw + o) * p.bw + j;               // element (k, o, j); o + 1 is bw further
-    store_vec(dst, o0, s0.x + s1.x, p.grad_dtype);
-    store_vec(dst, o0 + p.bw, s0.y + s1.y, p.grad_dtype);
-    store_vec(dst, o0 + 2 * p.bw, s0.z + s1.z, p.grad_dtype);
-    store_vec(dst, o0 + 3 * p.bw, s0.w + s1.w, p.grad_dtype);
+    const long long at = k * per_gate + (i % per_gate);      // element (k, o, j) of one gate's gradient
+    if (p.grad_dtype == RGLRU_BF16) {
+      bf16x8 out;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) out[e] = (__bf16)acc[e];
+      *reinterpret_cast<bf16x8*>((__bf16*)dst + at) = out;
+    } else {
+      const f32x4 lo = {acc[0], acc[1], acc[2], acc[3]}, hi = {acc[4], acc[5], acc[6], acc[7]};
+      *reinterpret_cast<f32x4*>((float*)dst + at) = lo;
+      *reinterpret_cast<f32x4*>((float*)dst + at + 4) = hi;
+    }
     return;
   }
   // 16 channels per workgroup; sixteen threads per channel each sum a share of the per-workgroup
@@ -3202,16 +3219,21 @@ static int fwd_impl(const void* x, const void* prep, const float* h0, const uint
     a.conv_k = (int)blk->K; a.conv_vec_dtype = blk->vec_dtype;
     a.x_out = blk->x_conv; a.gated = blk->gated; a.conv_new_state = blk->K > 1 ? blk->new_conv_state : nullptr;
   }
-  if (!cleared) {
-    rc = launch_clear(wb, L.f_begin, L.b_end, s);       // carry records and tickets of both passes, failure word
+  // The tiled kernels need the forward records, tickets and failure word zeroed; the chain kernel needs the
+  // failure word only and clears it itself.  (Every backward entry point that uses records clears its own.)
+  const bool chain = !blk && !pre && (nkg == 8 || nkg == 4 || nkg == 2) && fwd_chain_pays(B, T, W);
+  if (!cleared && !chain) {
+    rc = launch_clear(wb, L.f_begin, L.f_end, s);
     if (rc) return rc;
   }
-  // fuse: the parameter conversion (and the clearing of the workspace region it names) still has to happen.  The
-  // chain kernel does both itself when the caller's weights can be read as 16-byte vectors; else one launch first.
-  const bool chain = !blk && !pre && (nkg == 8 || nkg == 4 || nkg == 2) && fwd_chain_pays(B, T, W);
+  // fuse: the parameter conversion (and, for the tiled kernels, the clearing of the workspace region it names)
+  // still has to happen.  The chain kernel converts by itself when the caller's weights can be read as 16-byte
+  // vectors; else one launch first.
   const bool fused_prepare = fuse && chain && fuse->vec_ok;
   if (fuse && !fused_prepare) {
-    rc = launch_prepare(*fuse, dtype, stream);
+    PrepArgs pa = *fuse;
+    if (chain) { pa.clear = nullptr; pa.clear_n = 0; }
+    rc = launch_prepare(pa, dtype, stream);
     if (rc) return rc;
   }
   if (chain) {
@@ -3354,6 +3376,8 @@ int rglru_hip_bwd_pre(const void* x, const void* pre, const void* prep, const fl
   a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
   const bool masked = (flags != nullptr) || a.first_reset || (T % kChunk != 0);
   dim3 grid((unsigned)(a.wg_per_unit * a.units));
+  rc = launch_clear(wb, L.b_begin, L.b_end, s);          // records and tickets of this pass
+  if (rc) return rc;
   {
     KernelTimer timer(1, s);
     if (masked) hipLaunchKernelGGL((bwd_scan_kernel<__bf16, -1, true>), grid, dim3(kThreads), 0, s, a);
@@ -3366,7 +3390,6 @@ int rglru_hip_bwd_pre(const void* x, const void* pre, const void* prep, const fl
   r.partial = a.partial; r.dsp = finish_dsp(g, prep, dtype); r.db_a = db_a; r.db_x = db_x; r.dlambda = dlambda;
   r.W = (int)W; r.nb = (int)nb; r.bw = (int)g.bw; r.bwp = (int)g.bwp; r.Wp = (int)g.Wp; r.wg_per_unit = a.wg_per_unit;
   r.vec_blocks = (int)((W + 15) / 16); r.grad_dtype = grad_dtype;
-  r.clean = (uint4*)(wb + L.b_begin); r.clean_n = (long long)((L.b_end - L.b_begin) / 16);
   hipLaunchKernelGGL(finish_kernel, dim3((unsigned)r.vec_blocks), dim3(256), 0, s, r);
   return check_launch("bwd_pre finish");
 }
@@ -3380,11 +3403,11 @@ int rglru_hip_prepare_fwd(const void* w_a, const void* b_a, const void* w_x, con
   if (rc) return rc;
   if (B <= 0 || T <= 0) return fail(RGLRU_E_ARG, "prepare_fwd: B and T must be positive (got %lld, %lld)", (long long)B, (long long)T);
   if (!ws) return fail(RGLRU_E_ARG, "prepare_fwd: null pointer");
-  // The parameter conversion also zeroes the records, tickets and failure word of `ws`.  It is a launch of its
-  // own in front of the forward kernel, or part of the forward launch where that kernel can do it (fwd_impl).
+  // The parameter conversion also zeroes the forward records, tickets and failure word of `ws`.  It is a launch
+  // of its own in front of the forward kernel, or part of the forward launch where that kernel can do it (fwd_impl).
   const WorkLayout L = make_work_layout(B, T, make_geometry(W, nb));
   PrepArgs pa;
-  rc = build_prep_args(w_a, b_a, w_x, b_x, lambda, c, W, nb, dtype, vec_dtype, prep, (char*)ws + L.f_begin, L.b_end - L.f_begin, pa);
+  rc = build_prep_args(w_a, b_a, w_x, b_x, lambda, c, W, nb, dtype, vec_dtype, prep, (char*)ws + L.f_begin, L.f_end - L.f_begin, pa);
   if (rc) return rc;
   return fwd_impl(x, prep, h0, flags, y, h_last, ws, B, T, W, nb, dtype, true, stream, nullptr, nullptr, &pa);
 }
@@ -3410,7 +3433,7 @@ int rglru_hip_prepare_block_fwd(const void* w_a, const void* b_a, const void* w_
   if (B <= 0 || T <= 0) return fail(RGLRU_E_ARG, "prepare_block_fwd: B and T must be positive (got %lld, %lld)", (long long)B, (long long)T);
   if (!ws) return fail(RGLRU_E_ARG, "prepare_block_fwd: null pointer");
   const WorkLayout L = make_work_layout(B, T, make_geometry(W, nb));
-  rc = prepare_impl(w_a, b_a, w_x, b_x, lambda, c, W, nb, dtype, vec_dtype, prep, (char*)ws + L.f_begin, L.b_end - L.f_begin, stream);
+  rc = prepare_impl(w_a, b_a, w_x, b_x, lambda, c, W, nb, dtype, vec_dtype, prep, (char*)ws + L.f_begin, L.f_end - L.f_begin, stream);
   if (rc) return rc;
   const BlockFwd blk = {v, u_stride, v_stride, conv_state, taps, conv_bias, K, vec_dtype, x_conv, gated, new_conv_state};
   return fwd_impl(u, prep, h0, flags, y, h_last, ws, B, T, W, nb, dtype, true, stream, nullptr, &blk);
@@ -3454,6 +3477,8 @@ int rglru_hip_bwd(const void* x, const void* prep, const float* h0,
   a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nC, 2, L.max_wg);
   a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
   dim3 grid((unsigned)(a.wg_per_unit * a.units));
+  rc = launch_clear(wb, L.b_begin, L.b_end, s);          // records and tickets of this pass
+  if (rc) return rc;
   {
     KernelTimer timer(1, s);
     RGLRU_DISPATCH(bwd_kernel, grid, s, a, dtype, held_groups(g, dtype, a.aligned));
@@ -3465,7 +3490,6 @@ int rglru_hip_bwd(const void* x, const void* prep, const float* h0,
   r.partial = a.partial; r.dsp = finish_dsp(g, prep, dtype); r.db_a = db_a; r.db_x = db_x; r.dlambda = dlambda;
   r.W = (int)W; r.nb = (int)nb; r.bw = (int)g.bw; r.bwp = (int)g.bwp; r.Wp = (int)g.Wp; r.wg_per_unit = a.wg_per_unit;
   r.vec_blocks = (int)((W + 15) / 16); r.grad_dtype = grad_dtype;
-  r.clean = (uint4*)(wb + L.b_begin); r.clean_n = (long long)((L.b_end - L.b_begin) / 16);
   hipLaunchKernelGGL(finish_kernel, dim3((unsigned)r.vec_blocks), dim3(256), 0, s, r);
   return check_launch("bwd finish");
 }
@@ -3501,6 +3525,8 @@ int rglru_hip_bwd_full(const void* x, const void* y, const void* prep, const flo
   Geometry g = make_geometry(W, nb);
   if (!is_aligned(x, W, g.bw, 2) || !is_aligned(y, W, g.bw, 2) || !is_aligned(dy, W, g.bw, 2) || !is_aligned(dx, W, g.bw, 2))
     return fail(RGLRU_E_UNSUPPORTED, "bwd_full: x, y, dy and dx must be 16-byte aligned");
+  if ((uintptr_t)dw_a % 16 || (uintptr_t)dw_x % 16 || (uintptr_t)scratch % 16)
+    return fail(RGLRU_E_UNSUPPORTED, "bwd_full: dw_a, dw_x and scratch must be 16-byte aligned");
   WorkLayout L = make_work_layout(B, T, g);
   hipStream_t s = (hipStream_t)stream;
   char* wb = (char*)ws;
@@ -3544,6 +3570,8 @@ int rglru_hip_bwd_full(const void* x, const void* y, const void* prep, const flo
     if (nkg == 8) { RGLRU_LAUNCH_DELTA_CHAIN(8); } else if (nkg == 4) { RGLRU_LAUNCH_DELTA_CHAIN(4); } else { RGLRU_LAUNCH_DELTA_CHAIN(2); }
 #undef RGLRU_LAUNCH_DELTA_CHAIN
   } else {
+    rc = launch_clear(wb, L.b_begin, L.b_end, s);        // records and tickets of this pass
+    if (rc) return rc;
     KernelTimer timer(1, s);
 #define RGLRU_LAUNCH_DELTA(N)                                                                                        \
     if (masked) hipLaunchKernelGGL((bwd_delta_kernel<__bf16, N, true, kDeltaMT>), grid, dim3(kThreads), 0, s, a);      \
@@ -3575,10 +3603,8 @@ int rglru_hip_bwd_full(const void* x, const void* y, const void* prep, const flo
   r.dw_partial = a.dw_partial; r.dw_a = dw_a; r.dw_x = dw_x;
   r.W = (int)W; r.nb = (int)nb; r.bw = (int)g.bw; r.bwp = (int)g.bwp; r.Wp = (int)g.Wp; r.wg_per_unit = n_wg;
   r.n_wg = n_wg; r.vec_blocks = (int)((W + 15) / 16); r.grad_dtype = grad_dtype; r.dw_bf16 = a.dw_bf16;
-  // the chain scan writes no records and takes no tickets: the region is as clean as it was on entry
-  r.clean = (uint4*)(wb + L.b_begin); r.clean_n = chain_scan ? 0 : (long long)((L.b_end - L.b_begin) / 16);
   const long long total = nb * g.bw * 2 * g.bw;
-  hipLaunchKernelGGL(finish_kernel, dim3((unsigned)(r.vec_blocks + (total / 4 + 255) / 256)), dim3(256), 0, s, r);
+  hipLaunchKernelGGL(finish_kernel, dim3((unsigned)(r.vec_blocks + (total / 8 + 255) / 256)), dim3(256), 0, s, r);
   return check_launch("bwd_full finish");
 }
 
@@ -3606,6 +3632,8 @@ int rglru_hip_bwd_wide(const void* x, const void* prep, const float* h0,
   Geometry g = make_geometry(W, nb);
   if (!is_aligned(x, W, g.bw, 2) || !is_aligned(dy, W, g.bw, 2) || !is_aligned(dx, W, g.bw, 2))
     return fail(RGLRU_E_UNSUPPORTED, "bwd_wide: x, dy and dx must be 16-byte aligned");
+  if ((uintptr_t)dw_a % 16 || (uintptr_t)dw_x % 16 || (uintptr_t)scratch % 16)
+    return fail(RGLRU_E_UNSUPPORTED, "bwd_wide: dw_a, dw_x and scratch must be 16-byte aligned");
   WorkLayout L = make_work_layout(B, T, g);
   hipStream_t s = (hipStream_t)stream;
   char* wb = (char*)ws;
@@ -3630,6 +3658,8 @@ int rglru_hip_bwd_wide(const void* x, const void* prep, const float* h0,
   const bool masked = (flags != nullptr) || a.first_reset || (T % kChunk != 0);
   a.xcd_map = 1;
   dim3 grid((unsigned)(8 * (((long long)nb * a.wg_per_unit + 7) / 8) * a.groups));
+  rc = launch_clear(wb, L.b_begin, L.b_end, s);          // records and tickets of this pass
+  if (rc) return rc;
   {
     KernelTimer timer(1, s);
 #define RGLRU_LAUNCH_WIDE_SCAN(N)                                                                                    \
@@ -3676,9 +3706,8 @@ int rglru_hip_bwd_wide(const void* x, const void* prep, const float* h0,
   r.dw_partial = a.dw_partial; r.dw_a = dw_a; r.dw_x = dw_x;
   r.W = (int)W; r.nb = (int)nb; r.bw = (int)g.bw; r.bwp = (int)g.bwp; r.Wp = (int)g.Wp; r.wg_per_unit = scan_wg_per_unit;
   r.n_wg = n_wg; r.vec_blocks = (int)((W + 15) / 16); r.grad_dtype = grad_dtype;
-  r.clean = (uint4*)(wb + L.b_begin); r.clean_n = (long long)((L.b_end - L.b_begin) / 16);
   const long long total = nb * g.bw * 2 * g.bw;
-  hipLaunchKernelGGL(finish_kernel, dim3((unsigned)(r.vec_blocks + (total / 4 + 255) / 256)), dim3(256), 0, s, r);
+  hipLaunchKernelGGL(finish_kernel, dim3((unsigned)(r.vec_blocks + (total / 8 + 255) / 256)), dim3(256), 0, s, r);
   return check_launch("bwd_wide finish");
 }
 

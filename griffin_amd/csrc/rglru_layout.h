@@ -56,11 +56,12 @@ inline PrepLayout make_prep_layout(const Geometry& g, size_t elem) {
 // of 64 tokens.
 //   ckpt        [B][2 nC][W]    fp32 state after every 16 tokens (kept for backward: each lane of the
 //                               backward scan owns 16 consecutive tokens and starts from one of these)
-//   --- [f_begin, b_end) is cleared at the start of the forward pass ---
+//   --- [f_begin, f_end) is cleared at the start of a forward pass that uses records (the kernels with one
+//       workgroup per chain use none and clear the failure word only) ---
 //   f_rec_a     [B][<=nC][W]    64-bit carry records of the forward chain
 //   f_ticket    [units][kMaxQueues]
 //   fail        [1]             failure word (either pass sets it; only forward clears it)
-//   --- [b_begin, b_end): clean on entry to a backward pass, which cleans it again when it is done ---
+//   --- [b_begin, b_end): cleared at the start of every backward pass that uses records ---
 //   b_rec_a     [B][nC][W]      64-bit carry records of the backward chain
 //   b_ticket    [units][kMaxQueues]
 constexpr int kMaxQueues = 64;          // ticket queues per unit (sequences are dealt round-robin to them)

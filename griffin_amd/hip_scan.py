@@ -194,7 +194,10 @@ def pack_flags(reset_mask: Tensor | None, active_mask: Tensor | None) -> Tensor 
         hit = _PACKED_FLAGS.get(id(reset_mask))
         if hit is not None and hit[0]() is reset_mask and hit[1] == reset_mask._version:
             return hit[2]
-        flags = reset_mask.to(torch.uint8).contiguous()
+        # outside inference mode whatever the caller's mode: the bytes outlive this call, and an inference tensor
+        # cannot be saved for the backward pass of a later training step that finds them here
+        with torch.inference_mode(False):
+            flags = reset_mask.to(torch.uint8).contiguous()
         if not (reset_mask.is_cuda and torch.cuda.is_current_stream_capturing()):   # made under capture: valid inside that graph only
             if len(_PACKED_FLAGS) >= 64:
                 _PACKED_FLAGS.clear()

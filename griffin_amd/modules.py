@@ -111,9 +111,32 @@ class RG_LRU(nn.Module):
         params = self._gate_parameters()
         key = (dtype, device, float(self.c)) + tuple((q.data_ptr(), q._version) for q in params)
         if getattr(self, "_prep_key", None) != key:
-            self._prep = hip_scan.PreparedParams(*params, self.c, dtype)
+            prep = hip_scan.PreparedParams(*params, self.c, dtype)
+            if device.type == "cuda" and torch.cuda.is_current_stream_capturing():
+                return prep                                  # allocated by the graph being captured: this call only
+            self._prep = prep
             self._prep_key = key
         return self._prep
+
+    def invalidate_caches(self) -> None:
+        """Forget the kernel-side parameter image.  It is rebuilt by itself when a parameter is replaced or
+        updated in place through PyTorch operators; writes that bypass the version counter (``p.data.copy_()``,
+        ``p.data.mul_()``) need this call.  ``module.to()``/``.cuda()``, ``train()``/``eval()`` and
+        ``load_state_dict`` call it."""
+        self._prep = None
+        self._prep_key = None
+
+    def _apply(self, fn, *args, **kwargs):
+        self.invalidate_caches()
+        return super()._apply(fn, *args, **kwargs)
+
+    def train(self, mode: bool = True):
+        self.invalidate_caches()
+        return super().train(mode)
+
+    def _load_from_state_dict(self, *args, **kwargs):
+        self.invalidate_caches()
+        return super()._load_from_state_dict(*args, **kwargs)
 
     def forward(
         self,
@@ -211,8 +234,11 @@ def _default_positions(batch: int, steps: int, device: torch.device):
     key = (batch, steps, device)
     hit = _DEFAULT_POSITIONS.get(key)
     if hit is None:
-        pos = torch.arange(steps, device=device, dtype=torch.long).expand(batch, steps).contiguous()
-        hit = (pos, pos == 0)
+        # Built outside inference mode whatever the caller's mode: an inference tensor cannot be saved for a
+        # backward pass, and an evaluation pass followed by a training step at the same shape is the normal loop.
+        with torch.inference_mode(False):
+            pos = torch.arange(steps, device=device, dtype=torch.long).expand(batch, steps).contiguous()
+            hit = (pos, pos == 0)
         # tensors made while a graph is being captured live in that graph's memory and hold nothing until
         # it is replayed: they are used for this call only
         if not (device.type == "cuda" and torch.cuda.is_current_stream_capturing()):
@@ -313,6 +339,26 @@ class RecurrentBlock(nn.Module):
         nn.init.normal_(self.temporal_conv.weight, std=math.sqrt(0.01 / self.conv_kernel_size))
         for layer in (self.linear_x, self.linear_y, self.linear_out, self.temporal_conv):
             nn.init.zeros_(layer.bias)
+
+    def invalidate_caches(self) -> None:
+        """Forget the stacked decode projection (and the RG-LRU's parameter image).  Both are rebuilt by
+        themselves when a parameter is replaced or updated in place through PyTorch operators; writes that
+        bypass the version counter (``p.data.copy_()``) need this call.  ``module.to()``, ``train()``/``eval()``
+        and ``load_state_dict`` call it."""
+        self._stacked_projection = None
+        self.rg_lru.invalidate_caches()
+
+    def _apply(self, fn, *args, **kwargs):
+        self._stacked_projection = None
+        return super()._apply(fn, *args, **kwargs)
+
+    def train(self, mode: bool = True):
+        self._stacked_projection = None
+        return super().train(mode)
+
+    def _load_from_state_dict(self, *args, **kwargs):
+        self._stacked_projection = None
+        return super()._load_from_state_dict(*args, **kwargs)
 
     def _empty_conv_state(self, x: Tensor) -> Tensor:
         return x.new_zeros(x.size(0), self.conv_kernel_size - 1, self.rnn_width)

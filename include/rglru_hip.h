@@ -107,9 +107,10 @@ int rglru_hip_prepare(const void* w_a, const void* b_a, const void* w_x, const v
                       void* prep, void* stream);
 
 /* Workspace shared by one forward call and its backward call(s).  Forward initialises it (chunk
- * checkpoints of the fp32 state, cleared carry records for both passes), so its contents on entry
- * to forward do not matter; a backward call must be given the workspace of its forward call, reads
- * the checkpoints, uses the rest as scratch and leaves it ready for another backward call. */
+ * checkpoints of the fp32 state, the failure word, its own carry records where the kernel uses any),
+ * so its contents on entry to forward do not matter; a backward call must be given the workspace of its
+ * forward call, reads the checkpoints, clears and uses its own part as scratch, and any number of backward
+ * calls may follow one forward call. */
 size_t rglru_hip_workspace_bytes(int64_t B, int64_t T, int64_t W, int64_t nb);
 
 /* Scratch of one backward call (per-workgroup partial sums; for the fast configurations also the

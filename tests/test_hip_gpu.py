@@ -440,8 +440,8 @@ def test_chain_forward_repeats_bit_for_bit_and_is_the_default_at_the_training_sh
 @pytest.mark.parametrize("vec_dtype", [torch.float32, torch.bfloat16])
 def test_chain_forward_builds_the_same_parameter_image_as_prepare(shape, vec_dtype):
     """rglru_hip_prepare_fwd on the chain path converts the parameters inside the forward launch: the image it
-    leaves for the backward kernels is byte for byte the one rglru_hip_prepare writes, and the workspace region
-    it has to zero is zero."""
+    leaves for the backward kernels is byte for byte the one rglru_hip_prepare writes, and the failure word of the
+    workspace is cleared."""
     from griffin_amd import _lib, set_chain_forward
 
     lib = _lib.load()
@@ -473,37 +473,97 @@ def test_chain_forward_builds_the_same_parameter_image_as_prepare(shape, vec_dty
     written = want != 0x5A
     assert bool(written.any())
     assert torch.equal(got[written], want[written])
-    # checkpoints come first in the workspace; everything behind them is the region that starts out zero
+    # the chain kernels use no records and no tickets: of the workspace behind the checkpoints the launch clears
+    # the failure word and nothing else
+    import ctypes
+    status = ctypes.c_int(-1)
+    assert lib.rglru_hip_workspace_status(ws.data_ptr(), B, T, W, nb, 0, stream, ctypes.byref(status)) == 0
+    assert status.value == 0
     ckpt_bytes = B * 2 * (2 * ((T + 63) // 64)) * W * 4
-    assert int(ws[ckpt_bytes + 256:].count_nonzero()) == 0
+    behind = ws[ckpt_bytes + 256:]
+    assert int((behind != 0x77).sum()) == 4
     ry, rh = orc.rglru_forward(*[case[k].bfloat16().float() for k in ("x", "w_a")], case["b_a"].to(vec_dtype).float(),
                                case["w_x"].bfloat16().float(), case["b_x"].to(vec_dtype).float(), case["lam"].to(vec_dtype).float())
     assert rel_err(y.float().cpu(), ry) < BF16_TOL and rel_err(h_last.cpu(), rh) < BF16_TOL
 
 
-def test_chain_forward_that_gives_up_poisons_its_results():
-    """A wave that runs out of polls while it waits for the tile before hands on NaN and sets the failure word
-    (forced from the host with a one-poll budget; every wave still finishes)."""
-    from griffin_amd import _lib, hip_rglru, set_chain_forward
+def test_chain_kernels_that_give_up_poison_their_results_and_set_the_failure_word():
+    """A wave that runs out of polls while it waits for the tile next to it hands on NaN and sets the failure word
+    of the workspace (forced from the host with a one-poll budget; every wave still finishes).  Both chain kernels,
+    called through the C ABI on a workspace of the test's own: the word is set exactly when the outputs are not
+    finite.  T = 4096: 128 tiles for 16 waves, so every wave waits many times."""
+    import ctypes
+
+    from griffin_amd import _lib, set_chain_forward
 
     lib = _lib.load()
-    case = orc.make_case(4, 4096, 256, 2, seed=1)
-    leaves = [case[k].bfloat16().cuda() for k in PARAMS]
-    was = set_chain_forward(2)
-    previous = lib.rglru_hip_set_spin_limit(1)
-    try:
-        with torch.no_grad():
-            y, h_last = hip_rglru(*leaves, 8.0)
+    B, T, W, nb = 4, 4096, 256, 2
+    case = orc.make_case(B, T, W, nb, seed=1)
+    x, w_a, b_a, w_x, b_x, lam = (case[k].bfloat16().cuda() for k in PARAMS)
+    dy = case["dy"].bfloat16().cuda()
+    code = _lib.RGLRU_BF16
+    stream = torch.cuda.current_stream().cuda_stream
+    image = torch.empty(lib.rglru_hip_prep_bytes(W, nb, code), dtype=torch.uint8, device="cuda")
+    scratch = torch.empty(lib.rglru_hip_bwd_scratch_bytes(B, T, W, nb, code), dtype=torch.uint8, device="cuda")
+
+    def status_of(ws):
+        word = ctypes.c_int(-1)
+        assert lib.rglru_hip_workspace_status(ws.data_ptr(), B, T, W, nb, 0, stream, ctypes.byref(word)) == 0
+        return word.value
+
+    def forward(ws):
+        y = torch.empty_like(x)
+        h_last = torch.empty(B, W, device="cuda")
+        _lib.check(lib.rglru_hip_prepare_fwd(w_a.data_ptr(), b_a.data_ptr(), w_x.data_ptr(), b_x.data_ptr(), lam.data_ptr(), 8.0,
+                                             code, image.data_ptr(), x.data_ptr(), None, None, y.data_ptr(), h_last.data_ptr(),
+                                             ws.data_ptr(), B, T, W, nb, code, stream), "rglru_hip_prepare_fwd")
         torch.cuda.synchronize()
+        return y, h_last
+
+    def backward(ws, y):
+        dx = torch.empty_like(x)
+        dw_a, dw_x = torch.empty_like(w_a), torch.empty_like(w_x)
+        db_a, db_x, dlam = torch.empty_like(b_a), torch.empty_like(b_x), torch.empty_like(lam)
+        dh0 = torch.empty(B, W, device="cuda")
+        _lib.check(lib.rglru_hip_bwd_full(x.data_ptr(), y.data_ptr(), image.data_ptr(), None, None, dy.data_ptr(), None,
+                                          ws.data_ptr(), scratch.data_ptr(), dx.data_ptr(), dw_a.data_ptr(), dw_x.data_ptr(),
+                                          db_a.data_ptr(), db_x.data_ptr(), dlam.data_ptr(), dh0.data_ptr(), B, T, W, nb,
+                                          code, code, stream), "rglru_hip_bwd_full")
+        torch.cuda.synchronize()
+        return dx, dh0
+
+    def finite(*tensors):
+        return all(bool(torch.isfinite(t.float()).all()) for t in tensors)
+
+    n_ws = lib.rglru_hip_workspace_bytes(B, T, W, nb)
+    was = set_chain_forward(2)
+    try:
+        # forward with a one-poll budget
+        ws = torch.full((n_ws,), 0x77, dtype=torch.uint8, device="cuda")
+        previous = lib.rglru_hip_set_spin_limit(1)
+        try:
+            y, h_last = forward(ws)
+        finally:
+            lib.rglru_hip_set_spin_limit(previous)
+        assert (status_of(ws) != 0) == (not finite(y, h_last))
+        assert finite(y) == finite(h_last)                    # NaN travels down the chain to the final state
+        # the budget is back: clean results, and the word is cleared by the launch itself
+        y, h_last = forward(ws)
+        assert finite(y, h_last) and status_of(ws) == 0
+        # reverse scan with a one-poll budget on the clean forward
+        previous = lib.rglru_hip_set_spin_limit(1)
+        try:
+            dx, dh0 = backward(ws, y)
+        finally:
+            lib.rglru_hip_set_spin_limit(previous)
+        assert (status_of(ws) != 0) == (not finite(dx, dh0))
+        assert finite(dx) == finite(dh0)
+        # a forward pass clears the word again; the backward after it is clean
+        y, h_last = forward(ws)
+        dx, dh0 = backward(ws, y)
+        assert finite(dx, dh0) and status_of(ws) == 0
     finally:
-        lib.rglru_hip_set_spin_limit(previous)
         set_chain_forward(was)
-    gave_up = not bool(torch.isfinite(h_last).all())
-    if gave_up:                                           # whether a wait runs out is a matter of timing
-        assert not bool(torch.isfinite(y.float()).all())
-    with torch.no_grad():
-        y2, h2 = hip_rglru(*leaves, 8.0)                  # the budget is back: clean results
-    assert bool(torch.isfinite(y2.float()).all()) and bool(torch.isfinite(h2).all())
 
 
 # ------------------------------------------------------------------ golden vectors of the reference

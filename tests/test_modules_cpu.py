@@ -293,3 +293,64 @@ def test_stacked_decode_projection_follows_the_two_linear_layers():
         assert torch.allclose(px, block.linear_x(token), atol=1e-6)
         assert torch.allclose(py, block.linear_y(token), atol=1e-6)
     assert "_stacked_projection" not in block.state_dict()
+
+
+def test_inference_mode_pass_then_training_step_at_the_same_shape():
+    """An evaluation pass under inference_mode followed by a training step at the same (batch, length): the
+    default positions and the packed flags remembered from the first must be usable by the second (an
+    inference tensor cannot be saved for backward).  The reference builds them on every call."""
+    from griffin_amd import modules
+    from griffin_amd.hip_scan import _PACKED_FLAGS, pack_flags
+
+    modules._DEFAULT_POSITIONS.clear()
+    _PACKED_FLAGS.clear()
+    torch.manual_seed(0)
+    block = RecurrentBlock(12, 16, gate_blocks=2, scan_mode="sequential")
+    x = torch.randn(2, 9, 12)
+    with torch.inference_mode():
+        block(x)
+        pos, first = modules._default_positions(2, 9, x.device)
+        packed = pack_flags(first, None)
+    assert not pos.is_inference() and not first.is_inference() and not packed.is_inference()
+    assert pack_flags(first, None) is packed
+    leaf = x.clone().requires_grad_(True)
+    block(leaf).sum().backward()
+    assert torch.isfinite(leaf.grad).all() and leaf.grad.abs().max() > 0
+
+    class Keep(torch.autograd.Function):                      # what the HIP operators do with the flag bytes
+        @staticmethod
+        def forward(ctx, t, flags):
+            ctx.save_for_backward(flags)
+            return t * 2.0
+
+        @staticmethod
+        def backward(ctx, g):
+            return g * 2.0, None
+
+    Keep.apply(leaf, packed).sum().backward()
+
+
+def test_caches_are_dropped_by_invalidate_and_module_state_changes():
+    """Writes through ``.data`` bump no version counter; ``invalidate_caches`` (and ``to``, ``train``/``eval``,
+    ``load_state_dict``) drop the stacked decode projection and the RG-LRU's parameter image."""
+    torch.manual_seed(0)
+    block = RecurrentBlock(12, 16, gate_blocks=2, scan_mode="sequential")
+    token = torch.randn(5, 12)
+    with torch.no_grad():
+        block._decode_projections(token)
+        block.rg_lru._prep, block.rg_lru._prep_key = object(), ("stale",)
+        held = block._stacked_projection
+        block.linear_x.weight.data.mul_(3.0)                   # invisible to the (data_ptr, version) key
+        block._decode_projections(token)
+        assert block._stacked_projection is held
+        block.invalidate_caches()
+        assert block._stacked_projection is None and block.rg_lru._prep is None and block.rg_lru._prep_key is None
+        px, _ = block._decode_projections(token)
+        assert torch.allclose(px, block.linear_x(token), atol=1e-6)
+        for change in (lambda: block.eval(), lambda: block.train(), lambda: block.double(),
+                       lambda: block.load_state_dict(copy.deepcopy(block.state_dict()))):
+            block._decode_projections(token.to(block.linear_x.weight.dtype))
+            block.rg_lru._prep, block.rg_lru._prep_key = object(), ("stale",)
+            assert block._stacked_projection is not None
+            change()
+            assert block._stacked_projection is None and block.rg_lru._prep is None
