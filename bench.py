@@ -50,6 +50,8 @@ def parse_args():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="time eager launches instead of a HIP graph replay")
+    ap.add_argument("--no-masked-graph", action="store_true",
+                    help="skip the captured step of the masked kernel variants (T=2000, flags, h0) compared with eager")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also run a plain 64 MiB device copy a few times (known traffic, for scaling profiler counters)")
     ap.add_argument("--repeats", type=int, default=5, help="timed regions of K steps each; the median is reported")
@@ -377,6 +379,58 @@ def measured_traffic():
 KERNEL_SLOTS = {"fwd_kernel": 0, "bwd_delta_kernel": 1, "bwd_grad_kernel": 3}
 
 
+def masked_graph_check(hip_rglru, x_full, dy_full, params, tokens=2000, replays=3):
+    """One captured step of the MASKED kernel variants against eager launches: a length that is no multiple of
+    the tile (2000 tokens), document starts inside the rows, a right-padded row, a carried initial state, and
+    the final state among the captured outputs with a gradient of its own.  The graph is replayed several
+    times with eager work (the outputs zeroed) and synchronisations in between; every replay must give the
+    eager results (the chain kernels compose in a fixed order, so equal to rounding of nothing: 1e-6)."""
+    B, T, W = x_full.shape
+    tokens = min(tokens, T)
+    dev = x_full.device
+    gen = torch.Generator(device=dev).manual_seed(7)
+    x = x_full.detach()[:, :tokens].contiguous().requires_grad_(True)
+    dy = dy_full[:, :tokens].contiguous()
+    h0 = (0.5 * torch.randn(B, W, device=dev, generator=gen)).requires_grad_(True)
+    dh = torch.randn(B, W, device=dev, generator=gen)
+    reset = torch.zeros(B, tokens, dtype=torch.bool, device=dev)
+    reset[:, 0] = True
+    reset[0, tokens // 3] = True
+    reset[B - 1, (2 * tokens) // 3 + 5] = True
+    active = torch.ones(B, tokens, dtype=torch.bool, device=dev)
+    active[B - 1, tokens - 37:] = False
+
+    def step():
+        y, h_last = hip_rglru(x, *params, 8.0, h0, reset, active)
+        return (y, h_last) + torch.autograd.grad([y, h_last], [x, h0] + params, [dy, dh])
+
+    for _ in range(3):
+        eager = [t.detach().clone() for t in step()]
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = step()
+    worst = 0.0
+    for _ in range(replays):
+        for t in captured:
+            t.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, want in zip(captured, eager):
+            scale = want.float().abs().max().item() or 1.0
+            err = (got.float() - want.float()).abs().max().item() / scale
+            worst = max(worst, err if err == err else float("inf"))
+    return {"masked_graph_matches_eager": bool(worst < 1e-2), "masked_graph_vs_eager_max_rel_err": worst,
+            "masked_graph_case": f"T={tokens}, resets inside the rows, one right-padded row, h0, dh_last; {replays} replays"}
+
+
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -477,6 +531,8 @@ def main():
             scale = want.float().abs().max().item() or 1.0
             worst = max(worst, (got.float() - want.float()).abs().max().item() / scale)
         graph_check = {"graph_matches_eager": bool(worst < 1e-2), "graph_vs_eager_max_rel_err": worst}
+        if not args.no_masked_graph:
+            graph_check.update(masked_graph_check(hip_rglru, xs[0], dys[0], params))
         launch = f"hip graph replay, {per_graph} steps per graph, {n_sets} input sets in rotation"
     else:
         per_graph = 1
@@ -555,7 +611,7 @@ def main():
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(case)
     print(json.dumps(out))
-    if graph_check is not None and not graph_check["graph_matches_eager"]:
+    if graph_check is not None and not (graph_check["graph_matches_eager"] and graph_check.get("masked_graph_matches_eager", True)):
         print("bench.py: results of the captured step differ from an eager step", file=sys.stderr)
         sys.exit(1)
 
