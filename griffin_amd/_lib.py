@@ -14,7 +14,9 @@ RGLRU_BF16 = 1
 FLAG_RESET = 1
 FLAG_INACTIVE = 2
 CHUNK = 32
-ABI_VERSION = 16
+ABI_VERSION = 17
+PATH_PORTABLE, PATH_FAST_TILED, PATH_FAST_CHAIN, PATH_WIDE, PATH_PRE = range(5)
+PATH_NAMES = ("portable", "fast_tiled", "fast_chain", "wide", "pre")
 
 _lock = threading.Lock()
 _lib = None
@@ -37,14 +39,15 @@ _SIGNATURES = {
     "rglru_hip_static_workspace_bytes": (ctypes.c_size_t, []),
     "rglru_hip_fwd_static": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, ctypes.c_int, _P]),
     "rglru_hip_prepare_fwd": (ctypes.c_int, [_P, _P, _P, _P, _P, ctypes.c_float, ctypes.c_int, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, ctypes.c_int, _P]),
-    "rglru_hip_bwd": (ctypes.c_int, [_P] * 15 + [_I, _I, _I, _I, ctypes.c_int, ctypes.c_int, _P]),
+    "rglru_hip_bwd": (ctypes.c_int, [_P] * 17 + [_I, _I, _I, _I, ctypes.c_int, ctypes.c_int, _P]),
     "rglru_hip_fast_path": (ctypes.c_int, [_I, _I, ctypes.c_int]),
     "rglru_hip_wide_path": (ctypes.c_int, [_I, _I, ctypes.c_int]),
     "rglru_hip_bwd_full": (ctypes.c_int, [_P] * 16 + [_I, _I, _I, _I, ctypes.c_int, ctypes.c_int, _P]),
     "rglru_hip_bwd_wide": (ctypes.c_int, [_P] * 15 + [_I, _I, _I, _I, ctypes.c_int, ctypes.c_int, _P]),
     "rglru_hip_pre_path": (ctypes.c_int, [_I, _I, ctypes.c_int]),
+    "rglru_hip_backward_path": (ctypes.c_int, [_I, _I, _I, _I, ctypes.c_int, ctypes.c_int]),
     "rglru_hip_fwd_pre": (ctypes.c_int, [_P] * 8 + [_I, _I, _I, _I, ctypes.c_int, _P]),
-    "rglru_hip_bwd_pre": (ctypes.c_int, [_P] * 15 + [_I, _I, _I, _I, ctypes.c_int, ctypes.c_int, _P]),
+    "rglru_hip_bwd_pre": (ctypes.c_int, [_P] * 17 + [_I, _I, _I, _I, ctypes.c_int, ctypes.c_int, _P]),
     "rglru_hip_step": (ctypes.c_int, [_P, _P, _P, _P, _P, _I, _I, _I, ctypes.c_int, _P]),
     "rglru_hip_steps": (ctypes.c_int, [_P, _P, _P, _P, _P, _I, _I, _I, _I, ctypes.c_int, _P]),
     "rglru_hip_conv_max_kernel_size": (ctypes.c_int, []),

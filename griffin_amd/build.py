@@ -16,7 +16,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_NAME = "librglru_hip.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
-SOURCES = ["rglru_scan.hip", "rglru_fused.hip", "rglru_block_ops.hip"]
+SOURCES = ["rglru_scan.hip", "rglru_fused.hip", "rglru_gate_gemm.hip", "rglru_block_ops.hip"]
 ARCH = "gfx950"
 
 

@@ -2487,15 +2487,32 @@ struct FinishArgs {
   const float* partial; const float* dsp; void* db_a; void* db_x; void* dlambda;
   const float* dw_partial; void* dw_a; void* dw_x;
   int W, nb, bw, bwp, Wp, wg_per_unit, n_wg, vec_blocks, grad_dtype, dw_bf16;
+  int dw_vec;                                              // unpadded blocks of a multiple of 8 channels, 16-byte aligned gradients
 };
 
 __global__ __launch_bounds__(256) void finish_kernel(FinishArgs p) {
   __shared__ float part_sum[3][16][16];
   if ((int)blockIdx.x >= p.vec_blocks) {
     // eight consecutive input channels j of one (block, gate, output channel o) per thread: the partials are laid
-    // out like the gradients, so this is a streaming sum in a fixed order with 16-byte accesses (bw is a multiple
-    // of 32 on these paths and equals the padded width)
+    // out like the gradients, so this is a streaming sum in a fixed order with 16-byte accesses (dw_vec: the
+    // block width equals the padded width)
     const long long per_gate = (long long)p.bw * p.bw;
+    if (!p.dw_vec) {
+      // any width, any alignment: eight elements of the unpadded gradients per thread, one at a time
+      const long long total = (long long)p.nb * 2 * per_gate;
+      const long long first = ((long long)(blockIdx.x - p.vec_blocks) * blockDim.x + threadIdx.x) * 8;
+      const long long stride = (long long)p.nb * 2 * p.bwp * p.bwp;
+      for (long long i = first; i < first + 8 && i < total; ++i) {
+        const int j = (int)(i % p.bw), o = (int)((i / p.bw) % p.bw);
+        const int gate = (int)((i / per_gate) % 2);
+        const long long k = i / (2 * per_gate);
+        const float* src = p.dw_partial + (((k * 2 + gate) * p.bwp + o) * p.bwp + j);
+        float sum = 0.f;
+        for (int g = 0; g < p.n_wg; ++g) sum += src[(long long)g * stride];
+        store_vec(gate ? p.dw_x : p.dw_a, (k * p.bw + o) * p.bw + j, sum, p.grad_dtype);
+      }
+      return;
+    }
     const long long total8 = (long long)p.nb * 2 * per_gate / 8;
     const long long i8 = (long long)(blockIdx.x - p.vec_blocks) * blockDim.x + threadIdx.x;
     if (i8 >= total8) return;
@@ -3201,6 +3218,8 @@ static int fwd_impl(const void* x, const void* prep, const float* h0, const uint
     if (!a.aligned || (uintptr_t)pre % 16) return fail(RGLRU_E_UNSUPPORTED, "fwd_pre: x, pre and y must be 16-byte aligned");
     a.pre = pre; a.rows_total = B * T;
     nkg = -1;
+    rc = launch_gate_pre_gemm(x, a.wg, const_cast<void*>(pre), B * T, g, s);
+    if (rc) return rc;
   }
   if (blk) {
     const int64_t xs = blk->x_stride ? blk->x_stride : W, vs = blk->v_stride ? blk->v_stride : W;
@@ -3326,22 +3345,45 @@ int rglru_hip_fwd_static(const void* x, const void* prep, const float* h0, const
 
 static int check_grad_dtype(const char* who, int grad_dtype);
 
+// Tail of the backward entry points whose scan kernel leaves the gradients at the gate pre-activations in
+// memory: the two gate-gradient GEMMs (dx += du W; weight-gradient partials), then the fixed-order sums.
+static int gate_gemms_and_finish(const FusedArgs& a, const Geometry& g, const void* prep, int dtype, int grad_dtype,
+                                 const void* x, const void* du_a, const void* du_x, long long du_ld, long long du_blk,
+                                 void* dx, char* scratch, int64_t B, int64_t T,
+                                 void* dw_a, void* dw_x, void* db_a, void* db_x, void* dlambda, hipStream_t s) {
+  const ScratchLayout SL = make_scratch_layout(B, T, g, kScratchPlain);
+  const int splits = gate_dw_splits(B * T, g);
+  float* dw_partial = (float*)(scratch + SL.dw_partial);
+  int rc = launch_gate_gemms(x, du_a, du_x, du_ld, du_blk, a.w2t, dx, dw_partial, B * T, g, dtype, splits, s);
+  if (rc) return rc;
+  FinishArgs r;
+  memset(&r, 0, sizeof(r));
+  r.partial = a.partial; r.dsp = finish_dsp(g, prep, dtype); r.db_a = db_a; r.db_x = db_x; r.dlambda = dlambda;
+  r.dw_partial = dw_partial; r.dw_a = dw_a; r.dw_x = dw_x;
+  r.W = (int)g.W; r.nb = (int)g.nb; r.bw = (int)g.bw; r.bwp = (int)g.bwp; r.Wp = (int)g.Wp; r.wg_per_unit = a.wg_per_unit;
+  r.n_wg = splits; r.vec_blocks = (int)((g.W + 15) / 16); r.grad_dtype = grad_dtype;
+  r.dw_vec = (g.bw == g.bwp && (uintptr_t)dw_a % 16 == 0 && (uintptr_t)dw_x % 16 == 0) ? 1 : 0;
+  const long long total = g.nb * g.bw * 2 * g.bw;
+  hipLaunchKernelGGL(finish_kernel, dim3((unsigned)(r.vec_blocks + (total / 8 + 255) / 256)), dim3(256), 0, s, r);
+  return check_launch("bwd finish");
+}
+
 int rglru_hip_pre_path(int64_t W, int64_t nb, int dtype) {
   if (dtype != RGLRU_BF16 || W <= 0 || nb <= 0 || W % nb) return 0;
   const int64_t bw = W / nb;
   return (bw % 32 == 0 && bw <= 512) ? 1 : 0;
 }
 
-int rglru_hip_fwd_pre(const void* x, const void* pre, const void* prep, const float* h0, const uint8_t* flags,
+int rglru_hip_fwd_pre(const void* x, void* pre, const void* prep, const float* h0, const uint8_t* flags,
                       void* y, float* h_last, void* ws,
                       int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, void* stream) {
   if (!pre) return fail(RGLRU_E_ARG, "fwd_pre: null pointer");
   return fwd_impl(x, prep, h0, flags, y, h_last, ws, B, T, W, nb, dtype, false, stream, pre);
 }
 
-int rglru_hip_bwd_pre(const void* x, const void* pre, const void* prep, const float* h0,
+int rglru_hip_bwd_pre(const void* x, void* pre, const void* prep, const float* h0,
                       const uint8_t* flags, const void* dy, const float* dh_last, void* ws, void* scratch,
-                      void* dx, void* du, void* db_a, void* db_x, void* dlambda, float* dh0,
+                      void* dx, void* du, void* dw_a, void* dw_x, void* db_a, void* db_x, void* dlambda, float* dh0,
                       int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, int grad_dtype, void* stream) {
   int rc = check_geometry("bwd_pre", W, nb, dtype);
   if (rc) return rc;
@@ -3349,7 +3391,7 @@ int rglru_hip_bwd_pre(const void* x, const void* pre, const void* prep, const fl
   if (rc) return rc;
   if (!rglru_hip_pre_path(W, nb, dtype)) return fail(RGLRU_E_UNSUPPORTED, "bwd_pre: needs bf16 storage and gate blocks of a multiple of 32 channels");
   if (B <= 0 || T <= 0) return fail(RGLRU_E_ARG, "bwd_pre: B and T must be positive (got %lld, %lld)", (long long)B, (long long)T);
-  if (!x || !pre || !prep || !dy || !ws || !scratch || !dx || !du || !db_a || !db_x || !dlambda)
+  if (!x || !pre || !prep || !dy || !ws || !scratch || !dx || !du || !dw_a || !dw_x || !db_a || !db_x || !dlambda)
     return fail(RGLRU_E_ARG, "bwd_pre: null pointer");
   rc = check_extents("bwd_pre", B, T, W);
   if (rc) return rc;
@@ -3378,6 +3420,8 @@ int rglru_hip_bwd_pre(const void* x, const void* pre, const void* prep, const fl
   dim3 grid((unsigned)(a.wg_per_unit * a.units));
   rc = launch_clear(wb, L.b_begin, L.b_end, s);          // records and tickets of this pass
   if (rc) return rc;
+  rc = launch_gate_pre_gemm(x, a.wg, pre, B * T, g, s);  // the gate projections again
+  if (rc) return rc;
   {
     KernelTimer timer(1, s);
     if (masked) hipLaunchKernelGGL((bwd_scan_kernel<__bf16, -1, true>), grid, dim3(kThreads), 0, s, a);
@@ -3385,13 +3429,9 @@ int rglru_hip_bwd_pre(const void* x, const void* pre, const void* prep, const fl
   }
   rc = check_launch("bwd_pre scan");
   if (rc) return rc;
-  FinishArgs r;
-  memset(&r, 0, sizeof(r));
-  r.partial = a.partial; r.dsp = finish_dsp(g, prep, dtype); r.db_a = db_a; r.db_x = db_x; r.dlambda = dlambda;
-  r.W = (int)W; r.nb = (int)nb; r.bw = (int)g.bw; r.bwp = (int)g.bwp; r.Wp = (int)g.Wp; r.wg_per_unit = a.wg_per_unit;
-  r.vec_blocks = (int)((W + 15) / 16); r.grad_dtype = grad_dtype;
-  hipLaunchKernelGGL(finish_kernel, dim3((unsigned)r.vec_blocks), dim3(256), 0, s, r);
-  return check_launch("bwd_pre finish");
+  // du is [nb][B T][du_a (bw) | du_x (bw)]
+  return gate_gemms_and_finish(a, g, prep, dtype, grad_dtype, x, du, (const __bf16*)du + g.bw, 2 * g.bw, B * T * 2 * g.bw,
+                               dx, (char*)scratch, B, T, dw_a, dw_x, db_a, db_x, dlambda, s);
 }
 
 int rglru_hip_prepare_fwd(const void* w_a, const void* b_a, const void* w_x, const void* b_x,
@@ -3446,7 +3486,7 @@ static int check_grad_dtype(const char* who, int grad_dtype) {
 
 int rglru_hip_bwd(const void* x, const void* prep, const float* h0,
                   const uint8_t* flags, const void* dy, const float* dh_last, void* ws, void* scratch,
-                  void* dx, void* du_a, void* du_x, void* db_a, void* db_x, void* dlambda,
+                  void* dx, void* du_a, void* du_x, void* dw_a, void* dw_x, void* db_a, void* db_x, void* dlambda,
                   float* dh0, int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, int grad_dtype,
                   void* stream) {
   int rc = check_geometry("bwd", W, nb, dtype);
@@ -3454,7 +3494,7 @@ int rglru_hip_bwd(const void* x, const void* prep, const float* h0,
   rc = check_grad_dtype("bwd", grad_dtype);
   if (rc) return rc;
   if (B <= 0 || T <= 0) return fail(RGLRU_E_ARG, "bwd: B and T must be positive (got %lld, %lld)", (long long)B, (long long)T);
-  if (!x || !prep || !dy || !ws || !scratch || !dx || !du_a || !du_x || !db_a || !db_x || !dlambda)
+  if (!x || !prep || !dy || !ws || !scratch || !dx || !du_a || !du_x || !dw_a || !dw_x || !db_a || !db_x || !dlambda)
     return fail(RGLRU_E_ARG, "bwd: null pointer");
   rc = check_extents("bwd", B, T, W);
   if (rc) return rc;
@@ -3485,13 +3525,8 @@ int rglru_hip_bwd(const void* x, const void* prep, const float* h0,
   }
   rc = check_launch("bwd");
   if (rc) return rc;
-  FinishArgs r;
-  memset(&r, 0, sizeof(r));
-  r.partial = a.partial; r.dsp = finish_dsp(g, prep, dtype); r.db_a = db_a; r.db_x = db_x; r.dlambda = dlambda;
-  r.W = (int)W; r.nb = (int)nb; r.bw = (int)g.bw; r.bwp = (int)g.bwp; r.Wp = (int)g.Wp; r.wg_per_unit = a.wg_per_unit;
-  r.vec_blocks = (int)((W + 15) / 16); r.grad_dtype = grad_dtype;
-  hipLaunchKernelGGL(finish_kernel, dim3((unsigned)r.vec_blocks), dim3(256), 0, s, r);
-  return check_launch("bwd finish");
+  return gate_gemms_and_finish(a, g, prep, dtype, grad_dtype, x, du_a, du_x, W, g.bw, dx, (char*)scratch, B, T,
+                               dw_a, dw_x, db_a, db_x, dlambda, s);
 }
 
 int rglru_hip_fast_path(int64_t W, int64_t nb, int dtype) {
@@ -3602,7 +3637,7 @@ int rglru_hip_bwd_full(const void* x, const void* y, const void* prep, const flo
   r.partial = a.partial; r.dsp = finish_dsp(g, prep, dtype); r.db_a = db_a; r.db_x = db_x; r.dlambda = dlambda;
   r.dw_partial = a.dw_partial; r.dw_a = dw_a; r.dw_x = dw_x;
   r.W = (int)W; r.nb = (int)nb; r.bw = (int)g.bw; r.bwp = (int)g.bwp; r.Wp = (int)g.Wp; r.wg_per_unit = n_wg;
-  r.n_wg = n_wg; r.vec_blocks = (int)((W + 15) / 16); r.grad_dtype = grad_dtype; r.dw_bf16 = a.dw_bf16;
+  r.n_wg = n_wg; r.vec_blocks = (int)((W + 15) / 16); r.grad_dtype = grad_dtype; r.dw_bf16 = a.dw_bf16; r.dw_vec = 1;
   const long long total = nb * g.bw * 2 * g.bw;
   hipLaunchKernelGGL(finish_kernel, dim3((unsigned)(r.vec_blocks + (total / 8 + 255) / 256)), dim3(256), 0, s, r);
   return check_launch("bwd_full finish");
@@ -3611,6 +3646,14 @@ int rglru_hip_bwd_full(const void* x, const void* y, const void* prep, const flo
 int rglru_hip_wide_path(int64_t W, int64_t nb, int dtype) {
   if (W <= 0 || nb <= 0 || W % nb) return 0;
   return wide_groups(make_geometry(W, nb), dtype, 1) != 0 ? 1 : 0;
+}
+
+int rglru_hip_backward_path(int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, int aligned) {
+  if (B <= 0 || T <= 0 || W <= 0 || nb <= 0 || W % nb || (dtype != RGLRU_F32 && dtype != RGLRU_BF16)) return -1;
+  if (aligned && rglru_hip_fast_path(W, nb, dtype)) return fwd_chain_pays(B, T, W) ? RGLRU_PATH_FAST_CHAIN : RGLRU_PATH_FAST_TILED;
+  if (aligned && rglru_hip_wide_path(W, nb, dtype)) return RGLRU_PATH_WIDE;
+  if (aligned && rglru_hip_pre_path(W, nb, dtype)) return RGLRU_PATH_PRE;
+  return RGLRU_PATH_PORTABLE;
 }
 
 int rglru_hip_bwd_wide(const void* x, const void* prep, const float* h0,
@@ -3705,7 +3748,7 @@ int rglru_hip_bwd_wide(const void* x, const void* prep, const float* h0,
   r.partial = a.partial; r.dsp = finish_dsp(g, prep, dtype); r.db_a = db_a; r.db_x = db_x; r.dlambda = dlambda;
   r.dw_partial = a.dw_partial; r.dw_a = dw_a; r.dw_x = dw_x;
   r.W = (int)W; r.nb = (int)nb; r.bw = (int)g.bw; r.bwp = (int)g.bwp; r.Wp = (int)g.Wp; r.wg_per_unit = scan_wg_per_unit;
-  r.n_wg = n_wg; r.vec_blocks = (int)((W + 15) / 16); r.grad_dtype = grad_dtype;
+  r.n_wg = n_wg; r.vec_blocks = (int)((W + 15) / 16); r.grad_dtype = grad_dtype; r.dw_vec = 1;
   const long long total = nb * g.bw * 2 * g.bw;
   hipLaunchKernelGGL(finish_kernel, dim3((unsigned)(r.vec_blocks + (total / 8 + 255) / 256)), dim3(256), 0, s, r);
   return check_launch("bwd_wide finish");

@@ -26,6 +26,14 @@ static __global__ void clear_words_kernel(unsigned* p, long long n) {
   for (; i < n4; i += stride) q[i] = make_uint4(0u, 0u, 0u, 0u);
 }
 
+struct Geometry;
+// The block-diagonal GEMMs of the gate projections and their gradients (rglru_gate_gemm.hip).
+int gate_dw_splits(long long N, const Geometry& g);
+int launch_gate_pre_gemm(const void* x, const void* wg, void* pre, long long N, const Geometry& g, hipStream_t s);
+int launch_gate_gemms(const void* x, const void* du_a, const void* du_x, long long du_ld, long long du_blk,
+                      const void* w2t, void* dx, float* dw_partial, long long N, const Geometry& g, int dtype,
+                      int n_split, hipStream_t s);
+
 inline int check_launch(const char* what) {
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(RGLRU_E_LAUNCH, "%s: %s", what, hipGetErrorString(e));

@@ -96,14 +96,18 @@ inline WorkLayout make_work_layout(int64_t B, int64_t T, const Geometry& g) {
   return w;
 }
 
+// Splits of the token axis (= partial sets) of the weight-gradient GEMM of the paths without a fused one
+// (rglru_gate_gemm.hip).
+int gate_dw_splits(long long N, const Geometry& g);
+
 // Scratch of one backward call; nothing in it outlives the call, its contents on entry do not matter.
 //   partial     [maxWg][3][Wp]  per-workgroup sums for db_a, db_x, dLambda
 //   delta       fast backward (blocks of 32, 64, 128 channels): [B][T][W] 16-bit, dL/dh_t after the
 //               reverse scan; wide backward (blocks of 160 .. 384 channels): [B][T][nb][2 bw] 16-bit,
 //               the gradients at the gate pre-activations as pairs (element 2 o + gate)
-//   dw_partial  [sets][nb][2][bwp][bwp] per-workgroup weight-gradient sums, sets = kGemmWgPerUnit (fast)
-//               or kWideWgPerUnit (wide); fp32, or bf16 in the fast backward when 16-bit gradients are
-//               asked for (sized for fp32 either way)
+//   dw_partial  [sets][nb][2][bwp][bwp] per-workgroup weight-gradient sums, sets = kGemmWgPerUnit (fast),
+//               kWideWgPerUnit (wide) or gate_dw_splits (the other paths); fp32, or bf16 in the fast backward
+//               when 16-bit gradients are asked for (sized for fp32 either way)
 enum ScratchKind { kScratchPlain = 0, kScratchFast = 1, kScratchWide = 2 };
 struct ScratchLayout {
   size_t partial, delta, dw_partial, total;
@@ -115,7 +119,7 @@ inline ScratchLayout make_scratch_layout(int64_t B, int64_t T, const Geometry& g
   auto take = [&](int64_t bytes) { size_t at = off; off += (size_t)round_up(bytes, 256); return at; };
   s.partial = take((int64_t)256 * 3 * g.Wp * 4);
   s.delta = take(kind == kScratchFast ? B * T * g.W * 2 : kind == kScratchWide ? B * T * g.W * 4 : 0);
-  const int64_t sets = kind == kScratchFast ? kGemmWgPerUnit : kind == kScratchWide ? kWideWgPerUnit : 0;
+  const int64_t sets = kind == kScratchFast ? kGemmWgPerUnit : kind == kScratchWide ? kWideWgPerUnit : gate_dw_splits(B * T, g);
   s.dw_partial = take(sets * g.nb * g.bwp * 2 * g.bwp * 4);
   s.total = off;
   return s;

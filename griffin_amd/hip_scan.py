@@ -266,21 +266,15 @@ def _check_fused_inputs(x: Tensor, w_a: Tensor, h0: Tensor | None, flags: Tensor
     _dtype_code(x.dtype)
 
 
-def _uses_pre_path(lib, x: Tensor, W: int, nb: int, code: int) -> bool:
-    """Block widths that are a multiple of 32 but have no kernel with register-held weights (416, 448,
-    480, 512): the gate projections run as one library GEMM, everything else in the HIP kernels."""
-    return bool(not lib.rglru_hip_fast_path(W, nb, code) and not lib.rglru_hip_wide_path(W, nb, code)
-                and lib.rglru_hip_pre_path(W, nb, code) and x.data_ptr() % 16 == 0)
-
-
-def _gate_projections(x: Tensor, w_a: Tensor, w_x: Tensor) -> tuple[Tensor, Tensor, Tensor]:
-    """pre[k][n] = [W_a[k] x[n, k] | W_x[k] x[n, k]] as one batched GEMM (griffin/griffin.py:149-154
-    without the bias).  Returns (pre [nb, n, 2 bw], the stacked weights [nb, 2 bw, bw], x as [nb, n, bw])."""
-    nb, bw, _ = w_a.shape
-    n = x.shape[0] * x.shape[1]
-    stacked = torch.cat((w_a.detach().to(x.dtype), w_x.detach().to(x.dtype)), dim=1)
-    xk = x.view(n, nb, bw).transpose(0, 1)
-    return torch.bmm(xk, stacked.transpose(1, 2)), stacked, xk
+def kernel_path(B: int, T: int, W: int, nb: int, dtype: torch.dtype, *tensors: Tensor) -> int:
+    """Which kernel family of the library serves this configuration (rglru_hip_backward_path): one of
+    ``_lib.PATH_*``.  ``tensors``: the activation tensors of the call; one that is not 16-byte aligned
+    sends the call to the portable kernels."""
+    aligned = all(t is None or t.data_ptr() % 16 == 0 for t in tensors)
+    path = _lib.load().rglru_hip_backward_path(B, T, W, nb, _dtype_code(dtype), 1 if aligned else 0)
+    if path < 0:
+        _lib.check(2, "rglru_hip_backward_path")
+    return path
 
 
 class _HipRGLRU(torch.autograd.Function):
@@ -304,8 +298,8 @@ class _HipRGLRU(torch.autograd.Function):
             h_last = torch.empty(B, W, dtype=torch.float32, device=device)
             image = torch.empty(_prep_bytes(W, nb, code), dtype=torch.uint8, device=device)
             ws = torch.empty(lib.rglru_hip_workspace_bytes(B, T, W, nb), dtype=torch.uint8, device=device)
-            if _uses_pre_path(lib, x, W, nb, code):
-                pre, _, _ = _gate_projections(x, w_a, w_x)
+            if kernel_path(B, T, W, nb, x.dtype, x) == _lib.PATH_PRE:
+                pre = torch.empty(nb, B * T, 2 * (W // nb), dtype=x.dtype, device=device)   # scratch of the call
                 _lib.check(lib.rglru_hip_prepare(*(t.data_ptr() for t in operands), float(c), W, nb, code, vec_code,
                                                  image.data_ptr(), _stream_ptr(device)), "rglru_hip_prepare")
                 _lib.check(lib.rglru_hip_fwd_pre(x.data_ptr(), pre.data_ptr(), image.data_ptr(), _ptr(h0c), _flags_ptr(flags),
@@ -361,8 +355,8 @@ def rglru_backward(x, y, w_a, w_x, h0c, flags, ws, image, dy, dh_last, param_dty
         dh0 = torch.empty(B, W, dtype=torch.float32, device=device) if need_dh0 else None
         # scratch of this call only (the workspace kept since forward holds just checkpoints and records)
         scratch = torch.empty(lib.rglru_hip_bwd_scratch_bytes(B, T, W, nb, code), dtype=torch.uint8, device=device)
-        if (lib.rglru_hip_fast_path(W, nb, code) and dy.data_ptr() % 16 == 0 and x.data_ptr() % 16 == 0
-                and y.data_ptr() % 16 == 0):
+        path = kernel_path(B, T, W, nb, x.dtype, x, y, dy, dx)
+        if path in (_lib.PATH_FAST_CHAIN, _lib.PATH_FAST_TILED):
             # everything in hand-written kernels, including the two gate GEMMs
             dw_a = torch.empty(nb, bw, bw, dtype=gdt, device=device)
             dw_x = torch.empty(nb, bw, bw, dtype=gdt, device=device)
@@ -371,7 +365,7 @@ def rglru_backward(x, y, w_a, w_x, h0c, flags, ws, image, dy, dh_last, param_dty
                                               dw_x.data_ptr(), db_a.data_ptr(), db_x.data_ptr(), dlam.data_ptr(),
                                               _ptr(dh0), B, T, W, nb, code, gcode, _stream_ptr(device)),
                        "rglru_hip_bwd_full")
-        elif lib.rglru_hip_wide_path(W, nb, code) and dy.data_ptr() % 16 == 0 and x.data_ptr() % 16 == 0:
+        elif path == _lib.PATH_WIDE:
             # blocks of 160 .. 384 channels: scan and gate math, then the two gate GEMMs, all hand-written
             dw_a = torch.empty(nb, bw, bw, dtype=gdt, device=device)
             dw_x = torch.empty(nb, bw, bw, dtype=gdt, device=device)
@@ -380,40 +374,29 @@ def rglru_backward(x, y, w_a, w_x, h0c, flags, ws, image, dy, dh_last, param_dty
                                               dw_x.data_ptr(), db_a.data_ptr(), db_x.data_ptr(), dlam.data_ptr(),
                                               _ptr(dh0), B, T, W, nb, code, gcode, _stream_ptr(device)),
                        "rglru_hip_bwd_wide")
-        elif _uses_pre_path(lib, x, W, nb, code) and dy.data_ptr() % 16 == 0:
-            # gate projections recomputed by the library GEMM, the scan and all gate math in the
-            # HIP kernel, then the two GEMMs of the gate gradients on the kernel's du
-            pre, stacked, xk = _gate_projections(x, w_a, w_x)
+        elif path == _lib.PATH_PRE:
+            # bf16 blocks of 416 .. 512 channels: a GEMM kernel for the gate projections, the scan and all gate math
+            # in the scan kernel, then the two GEMM kernels of the gate gradients
+            dw_a = torch.empty(nb, bw, bw, dtype=gdt, device=device)
+            dw_x = torch.empty(nb, bw, bw, dtype=gdt, device=device)
+            pre = torch.empty(nb, B * T, 2 * bw, dtype=x.dtype, device=device)
             du = torch.empty_like(pre)
             _lib.check(lib.rglru_hip_bwd_pre(x.data_ptr(), pre.data_ptr(), image.data_ptr(), _ptr(h0c), _flags_ptr(flags),
                                              dy.data_ptr(), _ptr(dhl), ws.data_ptr(), scratch.data_ptr(), dx.data_ptr(),
-                                             du.data_ptr(), db_a.data_ptr(), db_x.data_ptr(), dlam.data_ptr(),
-                                             _ptr(dh0), B, T, W, nb, code, gcode, _stream_ptr(device)),
+                                             du.data_ptr(), dw_a.data_ptr(), dw_x.data_ptr(), db_a.data_ptr(), db_x.data_ptr(),
+                                             dlam.data_ptr(), _ptr(dh0), B, T, W, nb, code, gcode, _stream_ptr(device)),
                        "rglru_hip_bwd_pre")
-            del pre
-            dw = torch.bmm(du.transpose(1, 2), xk)                 # [nb, 2 bw, bw] = [dW_a ; dW_x]
-            dw_a, dw_x = dw[:, :bw], dw[:, bw:]
-            dx_blocks = dx.view(B * T, nb, bw).transpose(0, 1)     # [nb, n, bw], row stride W: written in place
-            torch.baddbmm(dx_blocks, du, stacked, out=dx_blocks)
         else:
+            # any storage type, width and alignment: the scan kernel leaves the gradients at the gate
+            # pre-activations in du_a, du_x; two GEMM kernels of the library finish dW and dx
+            dw_a = torch.empty(nb, bw, bw, dtype=gdt, device=device)
+            dw_x = torch.empty(nb, bw, bw, dtype=gdt, device=device)
             du_a = torch.empty_like(x)
             du_x = torch.empty_like(x)
             _lib.check(lib.rglru_hip_bwd(x.data_ptr(), image.data_ptr(), _ptr(h0c), _flags_ptr(flags),
                                          dy.data_ptr(), _ptr(dhl), ws.data_ptr(), scratch.data_ptr(), dx.data_ptr(), du_a.data_ptr(),
-                                         du_x.data_ptr(), db_a.data_ptr(), db_x.data_ptr(), dlam.data_ptr(),
-                                         _ptr(dh0), B, T, W, nb, code, gcode, _stream_ptr(device)), "rglru_hip_bwd")
-            # block-diagonal library GEMMs: dW[k] = du[:, k]^T x[:, k];  dx[:, k] += du[:, k] W[k]
-            n = B * T
-            xk = x.view(n, nb, bw).transpose(0, 1)               # [nb, n, bw] (strided view)
-            ua = du_a.view(n, nb, bw).transpose(0, 1)
-            ux = du_x.view(n, nb, bw).transpose(0, 1)
-            wa = w_a.detach().to(x.dtype)
-            wx = w_x.detach().to(x.dtype)
-            dw_a = torch.bmm(ua.transpose(1, 2), xk)
-            dw_x = torch.bmm(ux.transpose(1, 2), xk)
-            dx_blocks = dx.view(n, nb, bw).transpose(0, 1)       # [nb, n, bw], row stride W: written in place
-            torch.baddbmm(dx_blocks, ua, wa, out=dx_blocks)
-            torch.baddbmm(dx_blocks, ux, wx, out=dx_blocks)
+                                         du_x.data_ptr(), dw_a.data_ptr(), dw_x.data_ptr(), db_a.data_ptr(), db_x.data_ptr(),
+                                         dlam.data_ptr(), _ptr(dh0), B, T, W, nb, code, gcode, _stream_ptr(device)), "rglru_hip_bwd")
     return dx, dw_a.to(pd[0]), db_a.to(pd[1]), dw_x.to(pd[2]), db_x.to(pd[3]), dlam.to(pd[4]), dh0
 
 

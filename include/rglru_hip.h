@@ -11,7 +11,7 @@
  *   griffin/griffin.py:237-289      RG_LRU.forward (gates + scan, T > 1)   rglru_hip_prepare + rglru_hip_fwd
  *   autograd of griffin/griffin.py:237-289                                   rglru_hip_bwd_full (blocks of 32/64/128 channels),
  *                                                                            rglru_hip_bwd_wide (160 .. 384), rglru_hip_bwd (any)
- *   the same with the gate projections (griffin/griffin.py:149-154) left to a BLAS GEMM   rglru_hip_fwd_pre, rglru_hip_bwd_pre
+ *   the same for bf16 blocks of 416 .. 512 channels (gate projections of griffin/griffin.py:149-154 as a GEMM kernel of their own)   rglru_hip_fwd_pre, rglru_hip_bwd_pre
  *   griffin/griffin.py:279-284 with T == 1 (decode step, carried state)     rglru_hip_step, rglru_hip_steps (K steps a launch)
  *   (no counterpart: forward for callers that cannot allocate)              rglru_hip_fwd_static
  *   griffin/griffin.py:474-487      causal depthwise convolution of the caller   rglru_hip_conv_fwd
@@ -50,7 +50,7 @@
 extern "C" {
 #endif
 
-#define RGLRU_ABI_VERSION 16
+#define RGLRU_ABI_VERSION 17
 
 enum { RGLRU_F32 = 0, RGLRU_BF16 = 1 };
 
@@ -150,15 +150,16 @@ int rglru_hip_prepare_fwd(const void* w_a, const void* b_a, const void* w_x, con
                           void* y, float* h_last, void* ws,
                           int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, void* stream);
 
-/* Backward of rglru_hip_fwd.  Recomputes the gates and the decay from x (nothing but the chunk
- * checkpoints in `ws` is kept from forward).  dy[B,T,W] (dtype); dh_last[B,W] fp32 or NULL.
- * Outputs: dx[B,T,W] (dtype) receives only the direct path dL/dz * g * i; du_a, du_x [B,T,W]
- * (dtype) receive the gradients at the two gate pre-activations, from which the caller forms
- * dW = du^T x, and dx += du W with two library GEMMs; db_a, db_x [nb*bw] and dlambda [W]
- * (grad_dtype) and dh0 [B,W] (fp32, may be NULL) are complete. */
+/* Backward of rglru_hip_fwd for any configuration (fp32 storage, block widths that are no multiple of 32,
+ * unaligned tensors).  Recomputes the gates and the decay from x (nothing but the chunk checkpoints in `ws`
+ * is kept from forward).  dy[B,T,W] (dtype); dh_last[B,W] fp32 or NULL.  Outputs, all complete: dx[B,T,W]
+ * (dtype), dw_a, dw_x [nb,bw,bw], db_a, db_x [nb*bw] and dlambda [W] (grad_dtype), dh0 [B,W] (fp32, may be
+ * NULL).  du_a, du_x [B,T,W] (dtype) are scratch of the call: the scan kernel leaves the gradients at the two
+ * gate pre-activations there, and two GEMM kernels of this library (matrix unit; griffin/griffin.py:149-154
+ * under autograd) form dW = du^T x and dx += du W from them. */
 int rglru_hip_bwd(const void* x, const void* prep, const float* h0,
                   const uint8_t* flags, const void* dy, const float* dh_last, void* ws, void* scratch,
-                  void* dx, void* du_a, void* du_x, void* db_a, void* db_x, void* dlambda,
+                  void* dx, void* du_a, void* du_x, void* dw_a, void* dw_x, void* db_a, void* db_x, void* dlambda,
                   float* dh0, int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, int grad_dtype,
                   void* stream);
 
@@ -195,26 +196,37 @@ int rglru_hip_bwd_wide(const void* x, const void* prep, const float* h0,
 
 /* Variant for the block widths that neither rglru_hip_fast_path nor rglru_hip_wide_path covers (any
  * multiple of 32 channels up to 512, i.e. 416, 448, 480 or 512; bf16 storage, 16-byte aligned tensors;
- * rglru_hip_pre_path() says whether a configuration qualifies).  The caller runs the two block-diagonal
- * projections of griffin/griffin.py:149-154 as ONE batched GEMM of its BLAS library and hands the
- * result in:
- *   pre[nb][B*T][2*bw] (dtype):  pre[k][n][o] = sum_j W_a[k][o][j] x[n][k*bw+j],
- *                                pre[k][n][bw+o] = the same with W_x        (biases NOT added)
- * rglru_hip_fwd_pre is rglru_hip_fwd with that operand.  rglru_hip_bwd_pre takes the same `pre`
- * (recomputed by the caller), writes the direct part of the input gradient into dx[B,T,W] and the
- * gradients at the pre-activations into du[nb][B*T][2*bw] (dtype; same two halves), plus db_a, db_x,
- * dlambda (grad_dtype) and dh0; the caller finishes with two batched GEMMs:
+ * rglru_hip_pre_path() says whether a configuration qualifies).  The two block-diagonal projections of
+ * griffin/griffin.py:149-154 run as a GEMM kernel of their own in front of the scan kernel, which takes
+ * their result as an operand.  `pre` and `du` are scratch of the call, [nb][B*T][2*bw] (dtype) each:
+ *   pre[k][n][o] = sum_j W_a[k][o][j] x[n][k*bw+j],  pre[k][n][bw+o] = the same with W_x  (biases not added)
+ *   du: the gradients at the pre-activations in the same two halves.
+ * rglru_hip_fwd_pre is rglru_hip_fwd with that scratch operand.  rglru_hip_bwd_pre recomputes `pre`, runs
+ * the reverse scan and the gate math, and finishes with the two gate-gradient GEMM kernels:
  *   dx[n][k*bw+j] += sum_o du[k][n][o] W_a[k][o][j] + du[k][n][bw+o] W_x[k][o][j]
  *   dW_a[k][o][j] = sum_n du[k][n][o] x[n][k*bw+j],  dW_x likewise from the second half.
- * `prep`, `ws` and `scratch` (rglru_hip_bwd_scratch_bytes) are those of rglru_hip_fwd / rglru_hip_bwd. */
+ * Outputs as rglru_hip_bwd_full.  `prep`, `ws` and `scratch` (rglru_hip_bwd_scratch_bytes) are those of
+ * rglru_hip_fwd / rglru_hip_bwd. */
 int rglru_hip_pre_path(int64_t W, int64_t nb, int dtype);
-int rglru_hip_fwd_pre(const void* x, const void* pre, const void* prep, const float* h0, const uint8_t* flags,
+int rglru_hip_fwd_pre(const void* x, void* pre, const void* prep, const float* h0, const uint8_t* flags,
                       void* y, float* h_last, void* ws,
                       int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, void* stream);
-int rglru_hip_bwd_pre(const void* x, const void* pre, const void* prep, const float* h0,
+int rglru_hip_bwd_pre(const void* x, void* pre, const void* prep, const float* h0,
                       const uint8_t* flags, const void* dy, const float* dh_last, void* ws, void* scratch,
-                      void* dx, void* du, void* db_a, void* db_x, void* dlambda, float* dh0,
+                      void* dx, void* du, void* dw_a, void* dw_x, void* db_a, void* db_x, void* dlambda, float* dh0,
                       int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, int grad_dtype, void* stream);
+
+/* Which backward entry point (and kernel family) covers a configuration: what a host wrapper dispatches on,
+ * and what a test asserts.  `aligned`: every activation tensor of the call (x, y, dy, dx) is 16-byte aligned.
+ * Returns one of RGLRU_PATH_*, or -1 for a geometry the library rejects.
+ *   RGLRU_PATH_FAST_CHAIN  rglru_hip_bwd_full, reverse scan with one workgroup per chain (and the forward likewise)
+ *   RGLRU_PATH_FAST_TILED  rglru_hip_bwd_full, reverse scan in tiles with a look-back between workgroups
+ *   RGLRU_PATH_WIDE        rglru_hip_bwd_wide
+ *   RGLRU_PATH_PRE         rglru_hip_fwd_pre / rglru_hip_bwd_pre
+ *   RGLRU_PATH_PORTABLE    rglru_hip_bwd
+ * (the choice between chain and tiles also follows rglru_hip_set_chain_forward). */
+enum { RGLRU_PATH_PORTABLE = 0, RGLRU_PATH_FAST_TILED = 1, RGLRU_PATH_FAST_CHAIN = 2, RGLRU_PATH_WIDE = 3, RGLRU_PATH_PRE = 4 };
+int rglru_hip_backward_path(int64_t B, int64_t T, int64_t W, int64_t nb, int dtype, int aligned);
 
 /* One decode step (T == 1): h[B,W] fp32 is updated in place, y[B,W] (dtype) = h as stored. */
 int rglru_hip_step(const void* x, const void* prep, float* h, const uint8_t* flags, void* y,

@@ -127,7 +127,7 @@ BF16_CASES = [
     (2, 128, 640, 2, False, False),  # 320-wide blocks, whole tiles, no flags, no state: the unmasked wide kernels
     (1, 300, 768, 2, True, True),    # 384-wide blocks, the widest the kernels hold in registers
     (5, 70, 320, 1, True, False),    # one 320-wide block, more sequences than tiles per sequence
-    (1, 90, 448, 1, True, True),     # 448-wide block: not held in registers, projections by the library GEMM
+    (1, 90, 448, 1, True, True),     # 448-wide block: not held in registers, projections by a GEMM kernel of their own
     (2, 70, 448, 2, True, True),     # 224-wide blocks: seven slabs, K tiles not a multiple of four
     (1, 100, 288, 1, False, True),   # one 288-wide block
     (1, 64, 704, 2, True, False),    # 352-wide blocks
@@ -279,7 +279,7 @@ def test_reproducible_mode_repeats_bit_for_bit(dtype, shape, everything):
     (torch.bfloat16, (8, 2048, 1024, 8)),     # plain kernels of the blocks up to 128 channels
     (torch.bfloat16, (3, 200, 256, 4)),       # their masked variants (ragged last tile), packed 64-wide blocks
     (torch.bfloat16, (2, 1024, 640, 2)),      # 320-wide blocks
-    (torch.bfloat16, (2, 300, 896, 2)),       # 448-wide blocks: projections by the library
+    (torch.bfloat16, (2, 300, 896, 2)),       # 448-wide blocks: projections by a GEMM kernel of their own
     (torch.float32, (2, 70, 48, 3)),          # portable kernels
 ])
 def test_first_token_reset_equals_the_explicit_mask(dtype, shape):
@@ -564,6 +564,57 @@ def test_chain_kernels_that_give_up_poison_their_results_and_set_the_failure_wor
         assert finite(dx, dh0) and status_of(ws) == 0
     finally:
         set_chain_forward(was)
+
+
+def test_kernel_family_selected_for_each_baseline_configuration():
+    """Which kernel family serves a shape is a fact of the library (rglru_hip_backward_path), not of pointer luck in
+    the wrapper: the five BASELINE configurations, the widths in between, and what a misaligned tensor does."""
+    from griffin_amd import _lib
+    from griffin_amd.hip_scan import kernel_path
+
+    bf, f32 = torch.bfloat16, torch.float32
+    assert kernel_path(2, 256, 256, 8, f32) == _lib.PATH_PORTABLE           # config 1: fp32 storage
+    assert kernel_path(8, 2048, 1024, 8, bf) == _lib.PATH_FAST_CHAIN        # configs 2 and 5: 256 chains on 256 units
+    assert kernel_path(1, 32768, 2560, 8, bf) == _lib.PATH_WIDE             # config 3: 320-wide blocks
+    assert kernel_path(256, 2048, 1024, 8, bf) == _lib.PATH_FAST_CHAIN      # config 4's prefill
+    assert kernel_path(1, 32768, 1024, 8, bf) == _lib.PATH_FAST_TILED       # too few chains for the compute units
+    assert kernel_path(8, 2048, 1024, 16, bf) == _lib.PATH_FAST_CHAIN       # the reference's default of 16 blocks
+    assert kernel_path(2, 300, 896, 2, bf) == _lib.PATH_PRE                 # 448-wide blocks
+    assert kernel_path(2, 300, 260, 2, bf) == _lib.PATH_PORTABLE            # 130-wide blocks
+    # a tensor that is not 16-byte aligned sends the call to the portable kernels, whose GEMMs are kernels of
+    # this library as well
+    x = torch.empty(8 * 2048 * 1024 + 8, dtype=bf, device="cuda")[1:-7].view(8, 2048, 1024)
+    assert x.data_ptr() % 16 == 2
+    assert kernel_path(8, 2048, 1024, 8, bf, x) == _lib.PATH_PORTABLE
+
+
+def test_misaligned_upstream_gradient_takes_the_portable_kernels_and_agrees():
+    """bf16 at a fast-path shape with a dy that is not 16-byte aligned: forward on the fast kernels, backward on
+    the portable scan kernel and the library's own gate-gradient GEMM kernels; same gradients to rounding."""
+    from griffin_amd import hip_rglru
+
+    B, T, W, nb = 2, 300, 256, 2
+    case = orc.make_case(B, T, W, nb, seed=12)
+    leaves = [case[k].bfloat16().cuda().requires_grad_(True) for k in PARAMS]
+    dy = case["dy"].bfloat16().cuda()
+    odd = torch.empty(B * T * W + 8, dtype=torch.bfloat16, device="cuda")[1:1 + B * T * W].view(B, T, W)
+    odd.copy_(dy)
+
+    class Misalign(torch.autograd.Function):                  # hands the operator's backward the misaligned copy
+        @staticmethod
+        def forward(ctx, y):
+            return y.clone()
+
+        @staticmethod
+        def backward(ctx, g):
+            return odd
+
+    y, _ = hip_rglru(*leaves, 8.0)
+    want = torch.autograd.grad(y, leaves, dy, retain_graph=True)
+    got = torch.autograd.grad(Misalign.apply(y), leaves, dy)
+    torch.cuda.synchronize()
+    for name, g, w in zip(PARAMS, got, want):
+        assert rel_err(g.float(), w.float()) < 1e-2, name
 
 
 # ------------------------------------------------------------------ golden vectors of the reference
