@@ -30,7 +30,7 @@ _SIGNATURES = {
     "rglru_hip_max_block_width": (ctypes.c_int, []),
     "rglru_hip_scan_workspace_bytes": (ctypes.c_size_t, [_I, _I, _I]),
     "rglru_hip_scan_fwd": (ctypes.c_int, [_P, _P, _P, _P, _P, _I, _I, _I, _P]),
-    "rglru_hip_scan_bwd": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _P]),
+    "rglru_hip_scan_bwd": (ctypes.c_int, [_P, _P, _P, _P, _P, _P, _P, _P, ctypes.c_int, _I, _I, _I, _P]),
     "rglru_hip_prep_bytes": (ctypes.c_size_t, [_I, _I, ctypes.c_int]),
     "rglru_hip_prepare": (ctypes.c_int, [_P, _P, _P, _P, _P, ctypes.c_float, _I, _I, ctypes.c_int, ctypes.c_int, _P, _P]),
     "rglru_hip_workspace_bytes": (ctypes.c_size_t, [_I, _I, _I, _I]),

@@ -34,6 +34,17 @@ int launch_gate_gemms(const void* x, const void* du_a, const void* du_x, long lo
                       const void* w2t, void* dx, float* dw_partial, long long N, const Geometry& g, int dtype,
                       int n_split, hipStream_t s);
 
+// The same for two ranges in one launch.
+static __global__ void clear_two_kernel(unsigned* p0, long long n0, unsigned* p1, long long n1) {
+  long long i = blockIdx.x * (long long)blockDim.x + threadIdx.x;
+  const long long stride = (long long)gridDim.x * blockDim.x;
+  const long long a = n0 >> 2, b = n1 >> 2;
+  for (; i < a + b; i += stride) {
+    if (i < a) reinterpret_cast<uint4*>(p0)[i] = make_uint4(0u, 0u, 0u, 0u);
+    else reinterpret_cast<uint4*>(p1)[i - a] = make_uint4(0u, 0u, 0u, 0u);
+  }
+}
+
 inline int check_launch(const char* what) {
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) return fail(RGLRU_E_LAUNCH, "%s: %s", what, hipGetErrorString(e));

@@ -125,13 +125,16 @@ inline ScratchLayout make_scratch_layout(int64_t B, int64_t T, const Geometry& g
   return s;
 }
 
-// Scan-only workspace; what a pass uses is cleared at its start.  Tickets and the failure word come
-// first, so that the clearing launch covers them and only as many records as the kernel variant needs
-// (one per sequence, channel and 32-token chunk, or one per 128-token run of the vector kernels).
+// Scan-only workspace of one forward / backward pair: two regions of the same layout, the forward pass uses
+// the first and the backward pass the second.  Tickets and the failure word come first in a region, so that a
+// clearing launch covers them and only as many records as the kernel variant needs (one per sequence, channel
+// and 32-token chunk, or one per 128-token run of the vector kernels).  The forward call clears the used part
+// of BOTH regions in its one clearing launch; a backward call clears its region itself unless told that the
+// workspace is fresh from its forward call.  The failure word of the pair is the first region's.
 //   ticket [B][groups]; fail; rec_a [B][nC][W] 64-bit carry records.
 struct ScanLayout {
   int64_t nC, groups;
-  size_t ticket, fail, rec_a, total;
+  size_t ticket, fail, rec_a, region, total;
 };
 
 inline ScanLayout make_scan_layout(int64_t B, int64_t T, int64_t W) {
@@ -143,7 +146,8 @@ inline ScanLayout make_scan_layout(int64_t B, int64_t T, int64_t W) {
   s.ticket = take(B * s.groups * 4);
   s.fail = take(4);
   s.rec_a = take(B * s.nC * W * 8);
-  s.total = off;
+  s.region = off;
+  s.total = 2 * off;
   return s;
 }
 

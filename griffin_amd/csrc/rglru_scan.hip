@@ -364,24 +364,31 @@ static bool pointers_aligned16(const void* const* ptrs, int n) {
   return true;
 }
 
-// Fills the workspace part of the arguments and clears what the pass will use.  `vec`: the vector
-// kernels run (rows of 128-token runs instead of 32-token chunks in the record array).
-static int scan_common(ScanArgs& p, void* ws, int64_t B, int64_t T, int64_t W, bool vec, hipStream_t s) {
+// Fills the workspace part of the arguments and clears what is asked for.  `vec`: the vector kernels run (rows
+// of 128-token runs instead of 32-token chunks in the record array).  `region`: 0 = forward, 1 = backward.
+// `clear`: 0 = nothing (the region is known to be clear), 1 = this pass's region, 2 = both regions (forward).
+static int scan_common(ScanArgs& p, void* ws, int64_t B, int64_t T, int64_t W, bool vec, int region, int clear, hipStream_t s) {
   if (B <= 0 || T <= 0 || W <= 0) return fail(RGLRU_E_ARG, "scan: B, T, W must be positive (got %lld, %lld, %lld)", (long long)B, (long long)T, (long long)W);
   if (!ws) return fail(RGLRU_E_ARG, "scan: workspace pointer is null");
   if (B * T * W >= (1ll << 40)) return fail(RGLRU_E_UNSUPPORTED, "scan: tensor too large");
   ScanLayout L = make_scan_layout(B, T, W);
   if (B * L.nC * L.groups >= (1ll << 31)) return fail(RGLRU_E_UNSUPPORTED, "scan: too many tiles");
-  char* base = (char*)ws;
+  char* base = (char*)ws + (size_t)region * L.region;
   p.rec_a = (rec_t*)(base + L.rec_a);
-  p.ticket = (unsigned*)(base + L.ticket); p.fail = (unsigned*)(base + L.fail);
+  p.ticket = (unsigned*)(base + L.ticket); p.fail = (unsigned*)((char*)ws + L.fail);
   p.B = (int)B; p.T = (int)T; p.W = (int)W; p.groups = (int)L.groups;
   p.nC = vec ? (int)((T + kVecRun - 1) / kVecRun) : (int)L.nC;       // rows per sequence of the record array
   p.tiles = B * L.nC * L.groups;
   p.limit = spin_limit();
-  long long words = ((long long)L.rec_a + round_up(B * (long long)p.nC * W * 8, 16)) / 4;
+  if (clear == 0) return RGLRU_OK;
+  // tickets, failure word and the records in use; the other pass of a pair may run the other kernel variant
+  // (its tensors decide), so a forward call clears the second region for the variant with more records
+  const long long own = ((long long)L.rec_a + round_up(B * (long long)p.nC * W * 8, 16)) / 4;
+  const long long full = ((long long)L.rec_a + round_up(B * L.nC * W * 8, 16)) / 4;
+  const long long words = clear == 2 ? own + full : own;
   int cb = (int)((words + 1023) / 1024); if (cb > 2048) cb = 2048;
-  hipLaunchKernelGGL(clear_words_kernel, dim3(cb), dim3(256), 0, s, (unsigned*)base, words);
+  if (clear == 2) hipLaunchKernelGGL(clear_two_kernel, dim3(cb), dim3(256), 0, s, (unsigned*)base, own, (unsigned*)(base + L.region), full);
+  else hipLaunchKernelGGL(clear_words_kernel, dim3(cb), dim3(256), 0, s, (unsigned*)base, own);
   return check_launch("scan workspace clear");
 }
 
@@ -414,7 +421,7 @@ int rglru_hip_scan_fwd(const float* a, const float* z, const float* h0, float* h
   hipStream_t s = (hipStream_t)stream;
   const void* ptrs[] = {a, z, h0, h};
   const bool vec = W % 4 == 0 && pointers_aligned16(ptrs, 4);
-  int rc = scan_common(p, ws, B, T, W, vec, s);
+  int rc = scan_common(p, ws, B, T, W, vec, 0, 2, s);
   if (rc) return rc;
   p.a = a; p.z = z; p.h0 = h0; p.h = h;
   if (vec) {
@@ -428,7 +435,7 @@ int rglru_hip_scan_fwd(const float* a, const float* z, const float* h0, float* h
 }
 
 int rglru_hip_scan_bwd(const float* a, const float* h0, const float* h, const float* dh,
-                       float* da, float* dz, float* dh0, void* ws,
+                       float* da, float* dz, float* dh0, void* ws, int ws_fresh,
                        int64_t B, int64_t T, int64_t W, void* stream) {
   if (!a || !h0 || !h || !dh || !da || !dz || !dh0) return fail(RGLRU_E_ARG, "scan_bwd: null tensor pointer");
   ScanArgs p;
@@ -436,7 +443,7 @@ int rglru_hip_scan_bwd(const float* a, const float* h0, const float* h, const fl
   hipStream_t s = (hipStream_t)stream;
   const void* ptrs[] = {a, h0, h, dh, da, dz, dh0};
   const bool vec = W % 4 == 0 && pointers_aligned16(ptrs, 7);
-  int rc = scan_common(p, ws, B, T, W, vec, s);
+  int rc = scan_common(p, ws, B, T, W, vec, 1, ws_fresh ? 0 : 1, s);
   if (rc) return rc;
   p.a = a; p.h0 = h0; p.h_saved = h; p.dh = dh; p.da = da; p.dz = dz; p.dh0 = dh0;
   if (vec) {

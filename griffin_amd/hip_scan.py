@@ -141,6 +141,9 @@ class _HipScan(torch.autograd.Function):
                                               out.data_ptr(), ws.data_ptr(), B, T, W, _stream_ptr(decay.device)),
                        "rglru_hip_scan_fwd")
         ctx.save_for_backward(decay, initial_state, out)
+        # the forward call has cleared the backward part of the workspace too: the first backward call over this
+        # forward finds it clear (a repeated one clears its part itself)
+        ctx.workspace = [ws]
         return out
 
     @staticmethod
@@ -156,10 +159,14 @@ class _HipScan(torch.autograd.Function):
         if decay.numel() == 0:
             return d_decay, d_input, d_state.zero_()
         with _on_device(decay.device):
-            ws = torch.empty(lib.rglru_hip_scan_workspace_bytes(B, T, W), dtype=torch.uint8, device=decay.device)
+            held = getattr(ctx, "workspace", None)
+            fresh = bool(held)
+            ws = held.pop() if fresh else torch.empty(lib.rglru_hip_scan_workspace_bytes(B, T, W), dtype=torch.uint8,
+                                                      device=decay.device)
             _lib.check(lib.rglru_hip_scan_bwd(decay.data_ptr(), initial_state.data_ptr(), out.data_ptr(),
                                               grad_out.data_ptr(), d_decay.data_ptr(), d_input.data_ptr(),
-                                              d_state.data_ptr(), ws.data_ptr(), B, T, W, _stream_ptr(decay.device)),
+                                              d_state.data_ptr(), ws.data_ptr(), 1 if fresh else 0, B, T, W,
+                                              _stream_ptr(decay.device)),
                        "rglru_hip_scan_bwd")
         return d_decay, d_input, d_state
 

@@ -85,14 +85,17 @@ int rglru_hip_max_block_width(void);
 
 /* ---- scan-only contract: h_t = a_t * h_{t-1} + z_t, all fp32 ------------------------------
  * Replaces griffin/triton_scan.py:31-60 and :63-122.  a, z, h, dh, da, dz are [B, T, W];
- * h0, dh0 are [B, W].  `ws` is scratch of rglru_hip_scan_workspace_bytes(B, T, W) bytes; its
- * contents on entry do not matter and a forward and a backward call may not share it
- * concurrently. */
+ * h0, dh0 are [B, W].  `ws` is scratch of rglru_hip_scan_workspace_bytes(B, T, W) bytes with a part for each
+ * pass; its contents on entry to a forward call do not matter, and a forward and a backward call may not
+ * use it concurrently.  The forward call clears both parts in its one clearing launch, so a training step pays
+ * for one such launch: pass ws_fresh != 0 to the FIRST backward call that is given the workspace of its forward
+ * call; ws_fresh == 0 (any other workspace, or a repeated backward call) makes the backward call clear its part
+ * itself.  Nothing but that is carried from forward to backward in `ws`. */
 size_t rglru_hip_scan_workspace_bytes(int64_t B, int64_t T, int64_t W);
 int rglru_hip_scan_fwd(const float* a, const float* z, const float* h0, float* h, void* ws,
                        int64_t B, int64_t T, int64_t W, void* stream);
 int rglru_hip_scan_bwd(const float* a, const float* h0, const float* h, const float* dh,
-                       float* da, float* dz, float* dh0, void* ws,
+                       float* da, float* dz, float* dh0, void* ws, int ws_fresh,
                        int64_t B, int64_t T, int64_t W, void* stream);
 
 /* ---- fused RG-LRU ---------------------------------------------------------------------------

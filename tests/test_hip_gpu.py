@@ -45,6 +45,28 @@ def test_scan_op_matches_loop(shape):
     assert max(errs) < FP32_TOL
 
 
+def test_scan_op_backward_twice_over_one_forward():
+    """The forward call clears the backward part of the workspace as well; a second backward pass over the same
+    forward (retain_graph) finds that part used and has to clear it itself: same gradients both times."""
+    from griffin_amd import hip_rglru_scan
+
+    B, T, W = 3, 700, 260
+    gen = torch.Generator().manual_seed(5)
+    a = torch.sigmoid(torch.randn(B, T, W, generator=gen) + 2.0)
+    z = torch.randn(B, T, W, generator=gen)
+    h0 = torch.randn(B, W, generator=gen)
+    dh = torch.randn(B, T, W, generator=gen)
+    want = orc.scan_autograd(a, z, h0, dh)
+    leaves = [t.cuda().requires_grad_(True) for t in (a, z, h0)]
+    h = hip_rglru_scan(*leaves)
+    first = torch.autograd.grad(h, leaves, dh.cuda(), retain_graph=True)
+    second = torch.autograd.grad(h, leaves, dh.cuda())
+    torch.cuda.synchronize()
+    for g1, g2, w in zip(first, second, want[1:]):
+        torch.testing.assert_close(g1.cpu(), w, atol=3e-5, rtol=3e-5)
+        torch.testing.assert_close(g2.cpu(), w, atol=3e-5, rtol=3e-5)
+
+
 def test_scan_op_selftest_inputs():
     from griffin_amd import hip_rglru_scan
 

@@ -418,6 +418,56 @@ def test_config5_recurrent_block_bf16_matches_fp32_oracle():
         assert err < BF16_TOL, (name, err)
 
 
+@pytest.mark.parametrize("cfg", [(2, 300, 96, 128, 4, 4), (3, 200, 64, 192, 3, 3), (2, 129, 48, 64, 2, 2),
+                                 (2, 260, 96, 256, 2, 4)])
+def test_one_launch_block_forward_against_the_oracle_directly(cfg):
+    """The block's one-launch forward (convolution prologue, RG-LRU, output gate; bf16) against the oracle's
+    block in fp32 on the same rounded parameters, forward and every gradient, at gate blocks of 32 (four to a
+    unit), 64 (two to a unit) and 128 channels and with fewer than four taps: cfg = (B, T, D, W, blocks, taps)."""
+    from griffin_amd import RecurrentBlock, hip_block_ops
+
+    B, T, D, W, nb, K = cfg
+    torch.manual_seed(21 + W)
+    block = RecurrentBlock(D, W, conv_kernel_size=K, gate_blocks=nb, scan_mode="hip").to(torch.bfloat16)
+    assert hip_block_ops.hip_block_forward_covers(W, nb, K, torch.bfloat16)
+    with torch.no_grad():
+        block.rg_lru.recurrence_gate.bias.copy_(0.3 * torch.randn(nb, W // nb))
+        block.rg_lru.input_gate.bias.copy_(0.3 * torch.randn(nb, W // nb))
+        block.temporal_conv.bias.copy_(0.1 * torch.randn(W))
+    x = torch.randn(B, T, D).to(torch.bfloat16)
+    up = torch.randn(B, T, D).to(torch.bfloat16)
+    p = {k: v.clone().requires_grad_(True) for k, v in _block_params(block).items()}
+    xr = x.float().requires_grad_(True)
+    want, _ = orc.recurrent_block_forward(xr, p)
+    names = list(p)
+    want_grads = torch.autograd.grad(want, [xr] + [p[k] for k in names], up.float())
+
+    hip_block = block.cuda()
+    calls = []
+    real = hip_block_ops.hip_block_forward
+
+    def spy(*args, **kwargs):
+        calls.append(1)
+        return real(*args, **kwargs)
+
+    hip_block_ops.hip_block_forward = spy
+    try:
+        xh = x.cuda().requires_grad_(True)
+        got = hip_block(xh)
+        got.backward(up.cuda())
+        torch.cuda.synchronize()
+    finally:
+        hip_block_ops.hip_block_forward = real
+    assert calls, "the one-launch forward did not run"
+    mine = _block_params_grads(hip_block)
+    errs = {"out": rel_err(got.float(), want), "x": rel_err(xh.grad.float(), want_grads[0])}
+    for name, ref in zip(names, want_grads[1:]):
+        errs[name] = rel_err(mine[name], ref)
+    _say("one-launch block forward", cfg, {k: "%.2e" % v for k, v in errs.items()})
+    for name, err in errs.items():
+        assert err < BF16_TOL, (name, err)
+
+
 # ------------------------------------------------------------------ failure handling
 def test_bounded_wait_gives_up_instead_of_hanging():
     """With the poll budget forced to one, waves that do not find their carry at once record the
