@@ -273,6 +273,13 @@ def _check_fused_inputs(x: Tensor, w_a: Tensor, h0: Tensor | None, flags: Tensor
     _dtype_code(x.dtype)
 
 
+def _aligned(t: Tensor) -> Tensor:
+    """``t`` itself when its storage starts on a 16-byte boundary (what every fresh allocation does), else a
+    copy that does: a view at an odd offset costs one copy instead of sending the whole call to the portable
+    kernels, which are several times slower."""
+    return t if t.data_ptr() % 16 == 0 else t.clone(memory_format=torch.contiguous_format)
+
+
 def kernel_path(B: int, T: int, W: int, nb: int, dtype: torch.dtype, *tensors: Tensor) -> int:
     """Which kernel family of the library serves this configuration (rglru_hip_backward_path): one of
     ``_lib.PATH_*``.  ``tensors``: the activation tensors of the call; one that is not 16-byte aligned
@@ -293,7 +300,7 @@ class _HipRGLRU(torch.autograd.Function):
         _require_gpu("hip RG-LRU", x, w_a, b_a, w_x, b_x, lam, h0, None if first_reset else flags)
         _check_fused_inputs(x, w_a, h0, flags)
         lib = _lib.load()
-        x = x.contiguous()
+        x = _aligned(x.contiguous())
         B, T, W = x.shape
         nb = w_a.shape[0]
         code = _dtype_code(x.dtype)
@@ -347,7 +354,7 @@ def rglru_backward(x, y, w_a, w_x, h0c, flags, ws, image, dy, dh_last, param_dty
     nb, bw, _ = w_a.shape
     code = _dtype_code(x.dtype)
     device = x.device
-    dy = torch.zeros_like(x) if dy is None else dy.to(x.dtype).contiguous()
+    dy = torch.zeros_like(x) if dy is None else _aligned(dy.to(x.dtype).contiguous())
     dhl = None if dh_last is None else dh_last.to(torch.float32).contiguous()
     # parameter gradients come back in the parameters' own type when all five share one the
     # library writes (fp32 or bf16); otherwise in fp32, converted below

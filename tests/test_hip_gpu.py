@@ -610,31 +610,41 @@ def test_kernel_family_selected_for_each_baseline_configuration():
     assert kernel_path(8, 2048, 1024, 8, bf, x) == _lib.PATH_PORTABLE
 
 
-def test_misaligned_upstream_gradient_takes_the_portable_kernels_and_agrees():
-    """bf16 at a fast-path shape with a dy that is not 16-byte aligned: forward on the fast kernels, backward on
-    the portable scan kernel and the library's own gate-gradient GEMM kernels; same gradients to rounding."""
-    from griffin_amd import hip_rglru
+def test_misaligned_tensors_stay_on_the_fast_kernels_and_agree():
+    """bf16 at a fast-path shape with an x and a dy that are views at an odd storage offset: the wrapper realigns
+    them with one copy each instead of dropping the call onto the portable kernels; same results to rounding."""
+    from griffin_amd import _lib, hip_rglru, hip_scan
 
     B, T, W, nb = 2, 300, 256, 2
     case = orc.make_case(B, T, W, nb, seed=12)
     leaves = [case[k].bfloat16().cuda().requires_grad_(True) for k in PARAMS]
     dy = case["dy"].bfloat16().cuda()
-    odd = torch.empty(B * T * W + 8, dtype=torch.bfloat16, device="cuda")[1:1 + B * T * W].view(B, T, W)
-    odd.copy_(dy)
 
-    class Misalign(torch.autograd.Function):                  # hands the operator's backward the misaligned copy
-        @staticmethod
-        def forward(ctx, y):
-            return y.clone()
+    def odd_view(t):
+        out = torch.empty(t.numel() + 8, dtype=t.dtype, device="cuda")[1:1 + t.numel()].view(t.shape)
+        out.copy_(t)
+        assert out.data_ptr() % 16 == 2
+        return out
 
-        @staticmethod
-        def backward(ctx, g):
-            return odd
+    seen = []
+    real = hip_scan.kernel_path
+
+    def spy(*args):
+        seen.append(real(*args))
+        return seen[-1]
 
     y, _ = hip_rglru(*leaves, 8.0)
-    want = torch.autograd.grad(y, leaves, dy, retain_graph=True)
-    got = torch.autograd.grad(Misalign.apply(y), leaves, dy)
+    want = torch.autograd.grad(y, leaves, dy)
+    x_odd = odd_view(leaves[0].detach()).requires_grad_(True)
+    hip_scan.kernel_path = spy
+    try:
+        y2, _ = hip_rglru(x_odd, *leaves[1:], 8.0)
+        got = torch.autograd.grad(y2, [x_odd] + leaves[1:], odd_view(dy))
+    finally:
+        hip_scan.kernel_path = real
     torch.cuda.synchronize()
+    assert seen and all(path in (_lib.PATH_FAST_TILED, _lib.PATH_FAST_CHAIN) for path in seen), seen
+    assert rel_err(y2.float(), y.float()) < 1e-2
     for name, g, w in zip(PARAMS, got, want):
         assert rel_err(g.float(), w.float()) < 1e-2, name
 
