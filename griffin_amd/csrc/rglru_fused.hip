@@ -15,6 +15,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+#include <cmath>
 #include <cstring>
 #include <type_traits>
 
@@ -3075,6 +3077,26 @@ static int pick_wg_per_unit(int units, long long tiles_per_unit, int per_cu, lon
   return (int)n;
 }
 
+// How many ticket queues a unit's workgroups share.  Queue j owns the sequences j, j + q, ... and is served by
+// the workgroups j, j + q, ...; the launch ends with the queue that has the most sequences per workgroup, so
+// take the q that makes that ratio smallest (9 sequences on 16 workgroups: one queue, not nine of which seven
+// have two workgroups and two have one).  Among equals the largest q, which spreads the ticket atomics.
+static int pick_queues(long long B, int wg) {
+  long long qmax = B < wg ? B : wg;
+  if (qmax > kMaxQueues) qmax = kMaxQueues;
+  int best = 1;
+  long long best_num = B, best_den = wg;                  // one queue: B sequences on wg workgroups
+  for (int q = 2; q <= qmax; ++q) {
+    long long num = 0, den = 1;
+    for (int j = 0; j < q; ++j) {
+      const long long n = (B - j + q - 1) / q, w = (wg - j + q - 1) / q;
+      if (n * den > num * w) { num = n; den = w; }
+    }
+    if (num * best_den <= best_num * den) { best = q; best_num = num; best_den = den; }
+  }
+  return best;
+}
+
 }  // namespace rglru
 
 using namespace rglru;
@@ -3170,19 +3192,26 @@ static bool fwd_chain_pays(int64_t B, int64_t T, int64_t W) {
   const int mode = g_chain_forward.load(std::memory_order_relaxed);
   if (mode == 1) return false;
   if (mode == 2) return true;
-  // A workgroup fills a compute unit, so the launch takes ceil(chains / units) rounds, and the tiled kernel (1.18
-  // times slower at equal filling) wins when the last round is too empty.  Measured at W1024: with one or two
-  // rounds the chain kernels are ahead from 256 tokens on (8 tiles for 16 waves), with more rounds from 1024 on.
-  if (T < 256) return false;
+  // Two time models, in microseconds for the forward and the reverse scan together, fitted to both kernel
+  // pairs timed on 358 shapes (widths 512 to 4096, blocks of 32 to 128 channels, 16 to 8192 chains, 128 to 8192
+  // tokens); the faster model wins.  A chain workgroup fills a compute unit, so the chains run in
+  // ceil(chains / units) rounds, each as long as its sequence (a start-up cost, then a time per token that
+  // grows with the share of the units that are busy, since they share the memory system); the tiled kernels
+  // spread any shape over the whole chip, pay two longer launches plus one for the parameters, and their time
+  // per token is 1.1 to 1.2 times the chain kernels' when those fill their rounds.
   static const int units = [] {
     int dev = 0, n = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 0;
     return n;
   }();
   if (units <= 0) return false;
-  const long long chains = B * (W / 32), rounds = (chains + units - 1) / units;
-  if (T < 1024 && rounds > 2) return false;
-  return chains * 100 >= rounds * units * 85;
+  const double chains = (double)B * (double)(W / 32), tokens = (double)T;
+  const double rounds = std::ceil(chains / units), last = (chains - (rounds - 1) * units) / units;
+  const double full_round = 4.7 + tokens * (0.01465 + 0.01208), last_round = 4.7 + tokens * (0.01465 + 0.01208 * last);
+  const double t_chain = 6.6 + (rounds - 1) * full_round + last_round;
+  const double work = chains * tokens * (256.0 / units);
+  const double t_tiled = std::max(31.4, 24.2 + 1.025e-4 * work + 0.0030 * tokens);
+  return t_chain < t_tiled;
 }
 
 static int fwd_impl(const void* x, const void* prep, const float* h0, const uint8_t* flags,
@@ -3277,7 +3306,7 @@ static int fwd_impl(const void* x, const void* prep, const float* h0, const uint
   a.nCf = (int)((T + tile_tokens - 1) / tile_tokens);
   // without weights in registers three workgroups fit a compute unit
   a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nCf, blk ? 2 : nkg < 0 ? RGLRU_GIVEN_OCC : ((nkg == 4 || nkg == 2) ? RGLRU_NARROW_OCC : nkg > 8 ? fwd_wide_occ(nkg) : 2), 1 << 20);
-  a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
+  a.queues = pick_queues(B, a.wg_per_unit);
   dim3 grid((unsigned)(a.wg_per_unit * a.units));
   if (nkg > 8) {
     a.xcd_map = 1;
@@ -3415,7 +3444,7 @@ int rglru_hip_bwd_pre(const void* x, void* pre, const void* prep, const float* h
   a.B = (int)B; a.T = (int)T; a.nC = (int)((T + kChunk - 1) / kChunk); a.ckpt_nC = 2 * (int)L.nC;
   a.aligned = 1;
   a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nC, 2, L.max_wg);
-  a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
+  a.queues = pick_queues(B, a.wg_per_unit);
   const bool masked = (flags != nullptr) || a.first_reset || (T % kChunk != 0);
   dim3 grid((unsigned)(a.wg_per_unit * a.units));
   rc = launch_clear(wb, L.b_begin, L.b_end, s);          // records and tickets of this pass
@@ -3515,7 +3544,7 @@ int rglru_hip_bwd(const void* x, const void* prep, const float* h0,
   a.B = (int)B; a.T = (int)T; a.nC = (int)((T + kChunk - 1) / kChunk); a.ckpt_nC = 2 * (int)L.nC; a.nCf = (int)L.nCf;
   a.aligned = is_aligned(x, W, g.bw, elem_size(dtype));
   a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nC, 2, L.max_wg);
-  a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
+  a.queues = pick_queues(B, a.wg_per_unit);
   dim3 grid((unsigned)(a.wg_per_unit * a.units));
   rc = launch_clear(wb, L.b_begin, L.b_end, s);          // records and tickets of this pass
   if (rc) return rc;
@@ -3590,7 +3619,7 @@ int rglru_hip_bwd_full(const void* x, const void* y, const void* prep, const flo
   // reverse scan: delta[B, T, W] (and dh0)
   const long long chunks = (T + 32 * kDeltaMT - 1) / (32 * kDeltaMT);
   a.wg_per_unit = pick_wg_per_unit(a.units, B * chunks, kDeltaMT == 1 ? 4 : RGLRU_DELTA_OCC, L.max_wg);
-  a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
+  a.queues = pick_queues(B, a.wg_per_unit);
   const bool masked = (flags != nullptr) || (T % (32 * kDeltaMT) != 0);
   dim3 grid((unsigned)(a.wg_per_unit * a.units));
   const bool chain_scan = fwd_chain_pays(B, T, W);
@@ -3697,7 +3726,7 @@ int rglru_hip_bwd_wide(const void* x, const void* prep, const float* h0,
   const int nkg = wide_groups(g, dtype, 1);
   // reverse scan and gate math: direct part of dx, du2, per-workgroup bias and Lambda sums
   a.wg_per_unit = pick_wg_per_unit(a.units, B * (long long)a.nC, 1, L.max_wg);
-  a.queues = (int)(B < a.wg_per_unit ? B : a.wg_per_unit); if (a.queues > kMaxQueues) a.queues = kMaxQueues;
+  a.queues = pick_queues(B, a.wg_per_unit);
   const bool masked = (flags != nullptr) || a.first_reset || (T % kChunk != 0);
   a.xcd_map = 1;
   dim3 grid((unsigned)(8 * (((long long)nb * a.wg_per_unit + 7) / 8) * a.groups));
