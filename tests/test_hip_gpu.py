@@ -158,10 +158,21 @@ BF16_CASES = [
 ]
 
 
+@pytest.fixture(params=["by shape", "tiled"])
+def kernel_choice(request):
+    """Small shapes go to the one-workgroup-per-chain kernels by default (they start faster); the tiled kernels
+    with look-back, which long sequences and large batches use, are run on the same cases by forcing them."""
+    from griffin_amd import set_chain_forward
+
+    was = set_chain_forward(1 if request.param == "tiled" else 0)
+    yield request.param
+    set_chain_forward(was)
+
+
 @pytest.mark.parametrize("cfg", BF16_CASES)
-def test_fused_bf16_matches_fp32_oracle(cfg):
+def test_fused_bf16_matches_fp32_oracle(cfg, kernel_choice):
     B, T, W, nb, masks, with_h0 = cfg
-    _say("fused bf16 case", cfg)
+    _say("fused bf16 case", cfg, kernel_choice)
     # per-channel biases: the reference initialises them to zero, training does not keep them there
     case = orc.make_case(B, T, W, nb, seed=2, h0_std=0.5 if with_h0 else 0.0, bias_std=0.5)
     reset, active = _masks(B, T, masks)
@@ -204,7 +215,7 @@ def _random_case(rng, index, seed):
     return dtype, (B, T, W, nb), case, reset, active, dh_last
 
 
-def test_random_shapes_match_oracle():
+def test_random_shapes_match_oracle(kernel_choice):
     """Sixty random configurations (fixed seed) across every kernel family: portable, register-held
     weights, packed narrow blocks, library-GEMM wide blocks; ragged lengths, random resets and
     padding, initial state and a gradient at the final state."""
