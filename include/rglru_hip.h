@@ -382,10 +382,11 @@ int64_t rglru_hip_set_spin_limit(int64_t polls);
  * mostly for long sequences.  Applies to launches made after the call; returns the previous setting. */
 int rglru_hip_set_reproducible(int enable);
 /* Which forward kernel rglru_hip_fwd uses for bf16 storage and gate blocks of 32, 64 or 128 channels (no
- * counterpart in the reference).  0 (default): by shape -- when the sequences x 32-channel slabs fill the
- * compute units evenly and the sequence has at least 256 tokens (1024 where the slabs make more than two
- * rounds over the compute units), one workgroup walks a whole chain (no exchange between workgroups,
- * bit-reproducible); otherwise tiles with a look-back between workgroups.  1: always the
+ * counterpart in the reference).  0 (default): by shape -- the library estimates the time of both kernel pairs
+ * from the number of (sequence, 32-channel slab) chains, the compute units and the sequence length and takes
+ * the faster: one workgroup walks a whole chain (no exchange between workgroups, bit-reproducible) for small
+ * and short problems and where the chains fill one to a few rounds over the compute units; tiles with a
+ * look-back between workgroups for few long sequences and for very large batches.  1: always the
  * tiled kernel.  2: the chain kernel whenever it covers the storage type and block width (tests).  Applies to
  * launches made after the call; returns the previous setting. */
 int rglru_hip_set_chain_forward(int mode);
