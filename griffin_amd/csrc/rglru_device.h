@@ -135,6 +135,22 @@ RGLRU_DEVICE void stage_flush(const unsigned char* stage, rsrc_t r, unsigned row
   }
 }
 
+// Matrix operand from a row-major bf16 tile in LDS whose ROWS are the contraction index (ds_read_b64_tr_b16, a
+// gfx950 instruction).  Within a group of 16 lanes, lane s names four consecutive elements and lane i receives
+// element i % 4 of the lanes i / 4, i / 4 + 4, i / 4 + 8, i / 4 + 12.  With lane s pointing at row s / 4,
+// columns 4 (s % 4) .. + 3 of a 4 x 16 patch, lane i ends up with the patch's column i, rows 0 .. 3.  Two
+// such reads give the fragment of a 32 x 32 x 16 product: lane (n = lane % 32, hf = lane / 32) holds rows
+// k0 + 8 hf .. + 7 of column col0 + n.  (The 16-byte row-wise read needs the tile transposed first.)
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4_lds;
+RGLRU_DEVICE bf16x8 lds_transposed_frag(const __bf16* tile, int row_stride, int k0, int col0, int lane) {
+  typedef __attribute__((address_space(3))) bf16x4_lds* lds_ptr_t;
+  const int i = lane & 15, g = lane >> 4;
+  const __bf16* src = tile + (k0 + 8 * (g >> 1) + (i >> 2)) * row_stride + col0 + 16 * (g & 1) + 4 * (i & 3);
+  const bf16x4_lds lo = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_ptr_t)(src));
+  const bf16x4_lds hi = __builtin_amdgcn_ds_read_tr16_b64_v4bf16((lds_ptr_t)(src + 4 * row_stride));
+  return __builtin_bit_cast(bf16x8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+}
+
 // Row m (0..31) of accumulator tile mt holds local time step tile_row(mt, m).  With this map,
 // register v of tile mt in lane half hf is local time hf * 16 * MT + 16 * mt + v: each lane
 // owns 16 * MT consecutive steps, the lower half-wave the first half of the tile.

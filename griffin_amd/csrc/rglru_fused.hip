@@ -1339,25 +1339,27 @@ __global__ __launch_bounds__(kThreads, (NKG > 8 ? 1 : 2)) void bwd_scan_kernel(F
     }
   };
 
+  // A pass of the loop ends with six 16-byte stores behind the loads of the next tile.  The wait for those loads at
+  // the top of the loop counts operations in issue order and must hold on every path into the loop, so the paths
+  // that store nothing (the first pass, a wave without a slab) issue six stores that their offset drops: the wait
+  // then leaves six operations in flight instead of draining the stores of the tile just finished.
+  auto six_dropped_stores = [&]() {
+    const rsrc_t nowhere = make_rsrc(p.dx, 0u);
+    const i32x4 nothing = {0, 0, 0, 0};
+#pragma unroll
+    for (int i = 0; i < 6; ++i) buf_store_b128(nothing, nowhere, kOutOfRange - 16u * (unsigned)i);   // distinct, or they are merged
+  };
   if (tid == 0) s_ticket[0] = atomicAdd(q.counter, 1u);
   __syncthreads();
   unsigned tk = s_ticket[0];
   int par = 0;
   issue(tk);
+  six_dropped_stores();
   while ((long long)tk < q.tiles) {
     int c, b;
     decode(tk, c, b);
     const int t0 = c * TR;
     const long long trow = (long long)b * p.T + t0 + hf * EL;
-    unsigned next_raw = 0;
-    if (tid == 0) next_raw = atomicAdd(q.counter, 1u);
-    // token flags (two bits per local step) and the state at the start of the chunk (forward
-    // checkpoint), requested early
-    unsigned flbits = 0u;
-    if constexpr (MASKED) flbits = flag_run(p, trow, t0 + hf * EL);
-    float h_start = 0.f;                                 // state in front of this lane's 16 tokens
-    if (c == 0 && hf == 0) { if (p.h0) h_start = p.h0[(long long)b * W + w.ch]; }
-    else h_start = p.ckpt[((long long)b * p.ckpt_nC + (2 * c - 1 + hf)) * W + w.ch];
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int idx = tid + i * kThreads;
@@ -1376,6 +1378,16 @@ __global__ __launch_bounds__(kThreads, (NKG > 8 ? 1 : 2)) void bwd_scan_kernel(F
       const int row = idx / VPR_DY, cv = idx - row * VPR_DY;
       if (idx < TR * VPR_DY) *reinterpret_cast<Frag*>(lds_dy + row * DYROW + cv * Tr::HW) = pre_dy[i];
     }
+    // the next ticket, the token flags (two bits per local step) and the state at the start of the chunk (forward
+    // checkpoint) are requested once the tile is in LDS: in front of it their latency would sit in the wait above
+    // (one atomic instruction for the workgroup, live in its first lane only: atomicAdd would combine the lanes'
+    // operations first and wait for the result on the spot)
+    const unsigned next_raw = (unsigned)__builtin_amdgcn_raw_ptr_buffer_atomic_add_i32(1, make_rsrc(q.counter, 4u), tid == 0 ? 0u : kOutOfRange, 0, 0);
+    unsigned flbits = 0u;
+    if constexpr (MASKED) flbits = flag_run(p, trow, t0 + hf * EL);
+    float h_start = 0.f;                                 // state in front of this lane's 16 tokens
+    if (c == 0 && hf == 0) { if (p.h0) h_start = p.h0[(long long)b * W + w.ch]; }
+    else h_start = p.ckpt[((long long)b * p.ckpt_nC + (2 * c - 1 + hf)) * W + w.ch];
     __syncthreads();
     f32x16 ua, ux;
     float xv[EL], gy[EL];
@@ -1418,6 +1430,7 @@ __global__ __launch_bounds__(kThreads, (NKG > 8 ? 1 : 2)) void bwd_scan_kernel(F
     const unsigned tk_next = s_ticket[par];
     if (!w.slab_ok) {                                    // a wave without a slab only helps with the loads
       issue(tk_next);
+      six_dropped_stores();
       tk = tk_next;
       continue;
     }
@@ -1462,9 +1475,11 @@ __global__ __launch_bounds__(kThreads, (NKG > 8 ? 1 : 2)) void bwd_scan_kernel(F
       const float ge = __builtin_amdgcn_sqrtf(one_minus_a2<false>(l2, a[e]));
       gi[e] = ie; g[e] = ge;
     }
-    issue(tk_next);
     float d_in = (last_chunk && p.dh_last) ? p.dh_last[(long long)b * W + w.ch] : 0.f;
     if (!last_chunk) d_in = carry_lookback(chain, c, +1, p.nC, 0.f, true, p.limit, p.fail);
+    // the next tile's loads go out behind the look-back: loads return in issue order, so requested in front of it
+    // they would put their latency into every round trip of the walk
+    issue(tk_next);
     const float d_out = fmaf(A_t, d_in, D_t);
     if (hf == 0) carry_publish(chain, c, 0.f, d_out, true);
     if (hf == 0 && c == 0 && p.dh0) p.dh0[(long long)b * W + w.ch] = d_out;
@@ -2261,32 +2276,46 @@ __global__ __launch_bounds__(kGradThreads, 1) void bwd_grad_kernel(FusedArgs p) 
 // 32-wide kappa tile, and for those it keeps its slab's w2t fragments (B operand of the first GEMM,
 // which it contracts over its own kappa only: the four quarters' partial tiles are added through LDS)
 // and its slab's 32 x 32 accumulators of the second GEMM in registers for the whole launch.  The
-// second GEMM contracts over tokens; both operands reach the layout it needs through the matrix
-// unit (a tile times the identity comes back in accumulator layout, where a lane holds 16 consecutive
-// tokens of one column), du2 once per tile for all waves (lds_dut).
+// second GEMM contracts over tokens, i.e. over the ROWS of the du2 and x tiles as they lie in LDS:
+// both operands come from transposing LDS reads (lds_transposed_frag), nothing is transposed by hand.
+// Where LDS has room for two tiles (blocks of up to 320 channels) the next tile is written while this
+// one is multiplied and a tile costs one barrier; the wider blocks keep one tile and two barriers.
 // ------------------------------------------------------------------------------------------
+template <int NKG> struct GateGradWideLds {
+  static constexpr int TR = 32, K2 = 2 * NKG * 16, JW = 64;
+  // du2 rows: K2 * 2 bytes is a multiple of 128, + 64 bytes makes the stride 64 or 192 modulo the 256 bytes of the
+  // banks, so the four rows a transposing read touches (64 bytes of each) fall on different banks
+  static constexpr int ROW_DU = K2 + 32, ROW_X = JW + 8;
+  static constexpr int kDuBytes = TR * ROW_DU * 2, kXBytes = TR * ROW_X * 2, kRedBytes = 2 * 3 * 4 * 64 * 16;
+  static constexpr int kStageBytes = 2 * WaveStage<TR>::kBytes;
+  static constexpr bool kDouble = 2 * (kDuBytes + 2 * kXBytes + kRedBytes) + kStageBytes <= 160 * 1024;
+  static constexpr int kBuffers = kDouble ? 2 : 1;
+};
+
 template <typename IO, int NKG>
 __global__ __launch_bounds__(kGradThreads, 1) void gate_grad_wide_kernel(FusedArgs p) {
   typedef Io<IO> Tr;
   typedef typename Tr::Frag Frag;
+  typedef GateGradWideLds<NKG> Lds;
   static_assert(sizeof(IO) == 2 && NKG > 8, "16-bit storage, blocks wider than 128 channels");
-  constexpr int TR = 32;
+  constexpr int TR = Lds::TR;
   constexpr int KC = NKG * Tr::KG;                       // block width
-  constexpr int K2 = 2 * KC;                             // kappa per block
+  constexpr int K2 = Lds::K2;                            // kappa per block
   constexpr int S = KC / 32;                             // slabs in the block
   constexpr int JG = (S + 1) / 2;                        // units per block (two slabs each)
   constexpr int NKT = K2 / 32;                           // kappa tiles
   constexpr int NI = (NKT + 3) / 4;                      // ... per wave
-  constexpr int JW = 64;                                 // columns of the unit's x / dx tiles
-  constexpr int ROW_DU = K2 + Tr::HW, ROW_X = JW + Tr::HW, ROW_T = TR + Tr::HW;
-  __shared__ __attribute__((aligned(16))) IO lds_du[TR * ROW_DU];
-  __shared__ __attribute__((aligned(16))) IO lds_dut[K2 * ROW_T];          // du2 transposed: [kappa][token]
-  __shared__ __attribute__((aligned(16))) IO lds_x[TR * ROW_X];
-  __shared__ __attribute__((aligned(16))) IO lds_dx[TR * ROW_X];
-  __shared__ __attribute__((aligned(16))) f32x4 lds_red[2][3][4][64];      // partial dx tiles of quarters 1..3, four registers a vector
-  __shared__ __attribute__((aligned(16))) unsigned char stage_all[2 * WaveStage<TR>::kBytes];
+  constexpr int JW = Lds::JW;                            // columns of the unit's x / dx tiles
+  constexpr int ROW_DU = Lds::ROW_DU, ROW_X = Lds::ROW_X;
+  constexpr bool DB = Lds::kDouble;
+  constexpr int NB = Lds::kBuffers;
+  __shared__ __attribute__((aligned(16))) IO lds_du[NB][TR * ROW_DU];
+  __shared__ __attribute__((aligned(16))) IO lds_x[NB][TR * ROW_X];
+  __shared__ __attribute__((aligned(16))) IO lds_dx[NB][TR * ROW_X];
+  __shared__ __attribute__((aligned(16))) f32x4 lds_red[NB][2][4][3][64];  // [slab][receiving quarter][sender][lane]: four accumulator registers a vector
+  __shared__ __attribute__((aligned(16))) unsigned char stage_all[Lds::kStageBytes];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, r = lane & 31, hf = lane >> 5;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6), r = lane & 31, hf = lane >> 5;
   const int sl = wave & 1, q = wave >> 1;
   // The JG units of a block that walk the same tiles read the same du2 rows.  Workgroups go to the eight XCDs
   // round-robin by index, each XCD has its own L2: index = xcd + 8 * slot puts the JG members of a
@@ -2316,13 +2345,6 @@ __global__ __launch_bounds__(kGradThreads, 1) void gate_grad_wide_kernel(FusedAr
         w2[i][g] = (slab_ok && kt < NKT) ? *reinterpret_cast<const Frag*>(row + kt * 32 + g * Tr::KG) : Tr::zero();
       }
   }
-  // identity fragments: element i of ident[g] is 1 where 16 g + 8 hf + i == r
-  Frag ident[2];
-#pragma unroll
-  for (int g = 0; g < 2; ++g)
-#pragma unroll
-    for (int i = 0; i < Tr::HW; ++i) ident[g][i] = (IO)((16 * g + 8 * hf + i == r) ? 1.0f : 0.0f);
-
   f32x16 dw[NI];
 #pragma unroll
   for (int i = 0; i < NI; ++i)
@@ -2359,107 +2381,108 @@ __global__ __launch_bounds__(kGradThreads, 1) void gate_grad_wide_kernel(FusedAr
     pre_x = buf_load_frag<Frag>(rx, x_off);
     pre_dx = buf_load_frag<Frag>(rdx, x_off);
   };
-
-  long long tile = wg_in_unit;
-  issue(tile);
-  for (; tile < n_tiles; tile += n_wg) {
+  // the tile in the registers above goes to LDS buffer b
+  auto deposit = [&](int b) {
 #pragma unroll
     for (int i = 0; i < NV_DU; ++i) {
       const int idx = tid + i * kGradThreads;
       const int row = idx / VPR_DU, cv = idx - row * VPR_DU;
-      if (idx < TR * VPR_DU) *reinterpret_cast<Frag*>(lds_du + row * ROW_DU + cv * Tr::HW) = pre_du[i];
+      if (idx < TR * VPR_DU) *reinterpret_cast<Frag*>(lds_du[b] + row * ROW_DU + cv * Tr::HW) = pre_du[i];
     }
     if (tid < TR * VPR_X) {
       const int row = tid / VPR_X, cv = tid - row * VPR_X;
-      *reinterpret_cast<Frag*>(lds_x + row * ROW_X + cv * Tr::HW) = pre_x;
-      *reinterpret_cast<Frag*>(lds_dx + row * ROW_X + cv * Tr::HW) = pre_dx;
+      *reinterpret_cast<Frag*>(lds_x[b] + row * ROW_X + cv * Tr::HW) = pre_x;
+      *reinterpret_cast<Frag*>(lds_dx[b] + row * ROW_X + cv * Tr::HW) = pre_dx;
     }
-    __syncthreads();
-    issue(tile + n_wg);
+  };
 
-    const long long row0 = tile * TR;
-    const IO* a_row_du = lds_du + tile_row<1>(0, r) * ROW_DU + hf * Tr::HW;
-    const IO* a_row_x = lds_x + tile_row<1>(0, r) * ROW_X + hf * Tr::HW;
-    // x of this wave's slab with tokens along the lane vector (A operand of the second GEMM)
-    Frag xt_lo = Tr::zero(), xt_hi = Tr::zero();
-    if (slab_ok) {
-      f32x16 xc;
-#pragma unroll
-      for (int v = 0; v < 16; ++v) xc[v] = 0.f;
-      Tr::mma(xc, *reinterpret_cast<const Frag*>(a_row_x + (2 * sl) * Tr::KG), ident[0]);
-      Tr::mma(xc, *reinterpret_cast<const Frag*>(a_row_x + (2 * sl + 1) * Tr::KG), ident[1]);
-#pragma unroll
-      for (int i = 0; i < 8; ++i) { xt_lo[i] = (IO)xc[i]; xt_hi[i] = (IO)xc[8 + i]; }
+  long long tile = wg_in_unit;
+  issue(tile);
+  if (DB) {
+    deposit(0);
+    issue(tile + n_wg);
+    __syncthreads();
+  }
+  // Every pass of the loop ends with one store behind the loads of the tile after next.  A store that its offset
+  // drops puts the first pass into the same state, so the wait for those loads can leave one operation in flight
+  // on every path into the loop (the counter is in issue order; without this the compiler must wait for everything,
+  // the store of the tile just finished included).
+  {
+    const i32x4 nothing = {0, 0, 0, 0};
+    buf_store_b128(nothing, make_rsrc(p.dx, 0u), kOutOfRange);
+  }
+  int buf = 0;
+  for (; tile < n_tiles; tile += n_wg) {
+    if (DB) {
+      // the buffer of the tile before this one: every wave has passed the barrier that ended its reads
+      deposit(buf ^ 1);
+      issue(tile + 2 * n_wg);
+    } else {
+      deposit(0);
+      issue(tile + n_wg);
+      __syncthreads();
     }
-    // transposes of du2: the eight waves share the kappa tiles
+    const long long row0 = tile * TR;
+    const IO* du_tile = lds_du[buf];
+    const IO* a_row_du = du_tile + tile_row<1>(0, r) * ROW_DU + hf * Tr::HW;
+    // first GEMM over this wave's share of kappa.  The four quarters' partial tiles are added through LDS, each
+    // quarter finishing four of a lane's sixteen tokens: registers 4 v4 .. 4 v4 + 3 go to quarter v4.  (A slab past
+    // the block's end multiplies zeros; its stores are dropped through their offset, so that every wave issues the
+    // same memory operations and the wait for the next tile's loads does not have to cover the stores.)
+    float direct[4];
 #pragma unroll
-    for (int h = 0; h < (NKT + kGradWaves - 1) / kGradWaves; ++h) {
-      const int kt = kGradWaves * h + wave;
+    for (int e = 0; e < 4; ++e) direct[e] = (float)lds_dx[buf][(hf * 16 + 4 * q + e) * ROW_X + sl * 32 + r];
+    f32x16 acc;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc[v] = 0.f;
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const int kt = q + 4 * i;
       if (kt < NKT) {
-        f32x16 dc;
-#pragma unroll
-        for (int v = 0; v < 16; ++v) dc[v] = 0.f;
-        Tr::mma(dc, *reinterpret_cast<const Frag*>(a_row_du + (2 * kt) * Tr::KG), ident[0]);
-        Tr::mma(dc, *reinterpret_cast<const Frag*>(a_row_du + (2 * kt + 1) * Tr::KG), ident[1]);
-        Frag lo, hi;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) { lo[i] = (IO)dc[i]; hi[i] = (IO)dc[8 + i]; }
-        IO* dst = lds_dut + (kt * 32 + r) * ROW_T + hf * 16;
-        *reinterpret_cast<Frag*>(dst) = lo;
-        *reinterpret_cast<Frag*>(dst + 8) = hi;
+        Tr::mma(acc, *reinterpret_cast<const Frag*>(a_row_du + (2 * kt) * Tr::KG), w2[i][0]);
+        Tr::mma(acc, *reinterpret_cast<const Frag*>(a_row_du + (2 * kt + 1) * Tr::KG), w2[i][1]);
       }
     }
-    // first GEMM, this wave's share of kappa; quarter 0 starts from the direct part and adds the others' tiles
-    f32x16 acc;
-    if (slab_ok) {
+    f32x4 mine = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int v = 0; v < 16; ++v) acc[v] = (q == 0) ? (float)lds_dx[(hf * 16 + v) * ROW_X + sl * 32 + r] : 0.f;
+    for (int v4 = 0; v4 < 4; ++v4) {
+      const f32x4 part = {acc[4 * v4], acc[4 * v4 + 1], acc[4 * v4 + 2], acc[4 * v4 + 3]};
+      if (v4 == q) mine = part;
+      else lds_red[buf][sl][v4][q < v4 ? q : q - 1][lane] = part;
+    }
+    // second GEMM: dW2T[j, kappa] += sum over the tile's tokens, this wave's kappa tiles; tokens 0..15, then 16..31
+    {
+      const Frag xt0 = lds_transposed_frag(lds_x[buf], ROW_X, 0, sl * 32, lane);
+      const Frag xt1 = lds_transposed_frag(lds_x[buf], ROW_X, 16, sl * 32, lane);
 #pragma unroll
       for (int i = 0; i < NI; ++i) {
         const int kt = q + 4 * i;
         if (kt < NKT) {
-          Tr::mma(acc, *reinterpret_cast<const Frag*>(a_row_du + (2 * kt) * Tr::KG), w2[i][0]);
-          Tr::mma(acc, *reinterpret_cast<const Frag*>(a_row_du + (2 * kt + 1) * Tr::KG), w2[i][1]);
-        }
-      }
-      if (q != 0) {
-#pragma unroll
-        for (int v4 = 0; v4 < 4; ++v4) {
-          const f32x4 part = {acc[4 * v4], acc[4 * v4 + 1], acc[4 * v4 + 2], acc[4 * v4 + 3]};
-          lds_red[sl][q - 1][v4][lane] = part;
+          Tr::mma(dw[i], xt0, lds_transposed_frag(du_tile, ROW_DU, 0, kt * 32, lane));
+          Tr::mma(dw[i], xt1, lds_transposed_frag(du_tile, ROW_DU, 16, kt * 32, lane));
         }
       }
     }
     __syncthreads();
-    if (slab_ok) {
-      // second GEMM: dW2T[j, kappa] += sum over the tile's tokens, this wave's kappa tiles
+    {
+      const f32x4 p0 = lds_red[buf][sl][q][0][lane], p1 = lds_red[buf][sl][q][1][lane], p2 = lds_red[buf][sl][q][2][lane];
+      unsigned char* my = stage + WaveStage<TR>::row_offset(hf * 16 + 4 * q) + r * 2;
 #pragma unroll
-      for (int i = 0; i < NI; ++i) {
-        const int kt = q + 4 * i;
-        if (kt < NKT) {
-          const IO* b_row = lds_dut + (kt * 32 + r) * ROW_T + hf * 16;
-          Tr::mma(dw[i], xt_lo, *reinterpret_cast<const Frag*>(b_row));
-          Tr::mma(dw[i], xt_hi, *reinterpret_cast<const Frag*>(b_row + 8));
-        }
+      for (int e = 0; e < 4; ++e) {
+        const float sum = (direct[e] + mine[e]) + (p0[e] + (p1[e] + p2[e]));
+        *reinterpret_cast<IO*>(my + e * WaveStage<TR>::kRowBytes) = (IO)sum;
       }
-      if (q == 0) {
-        unsigned char* my = stage + WaveStage<TR>::row_offset(hf * 16) + r * 2;
-#pragma unroll
-        for (int v4 = 0; v4 < 4; ++v4) {
-          const f32x4 p0 = lds_red[sl][0][v4][lane], p1 = lds_red[sl][1][v4][lane], p2 = lds_red[sl][2][v4][lane];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const float sum = acc[4 * v4 + e] + (p0[e] + (p1[e] + p2[e]));
-            *reinterpret_cast<IO*>(my + (4 * v4 + e) * WaveStage<TR>::kRowBytes) = (IO)sum;
-          }
-        }
-        wave_lds_fence();
-        const int rows = (int)((rows_total - row0) < TR ? (rows_total - row0) : TR);
-        const rsrc_t rdx = make_rsrc((const IO*)p.dx + row0 * p.W, (unsigned)rows * row_bytes);
-        stage_flush<TR>(stage, rdx, row_bytes, (unsigned)(k * p.bw + j0) * 2u, lane);
-        wave_lds_fence();
-      }
+      wave_lds_fence();
+      // the wave's eight rows (tokens 4 q .. + 3 and 16 + 4 q .. + 3) as 16-byte segments, one per lane of the lower half
+      const int rows = (int)((rows_total - row0) < TR ? (rows_total - row0) : TR);
+      const rsrc_t rdx = make_rsrc((const IO*)p.dx + row0 * p.W, (unsigned)rows * row_bytes);
+      const int frow = ((lane >> 4) & 1) * 16 + 4 * q + ((lane >> 2) & 3);
+      const unsigned seg = (unsigned)(lane & 3) * 16u;
+      const i32x4 v = *reinterpret_cast<const i32x4*>(stage + WaveStage<TR>::row_offset(frow) + seg);
+      buf_store_b128(v, rdx, (lane < 32 && slab_ok) ? (unsigned)frow * row_bytes + (unsigned)(k * p.bw + j0) * 2u + seg : kOutOfRange);
+      wave_lds_fence();
     }
+    if (DB) buf ^= 1;
   }
   // per-workgroup partial of the weight gradients, laid out like the gradients themselves: [wg][k][gate][o][j];
   // a lane's registers 4 v4 .. 4 v4 + 3 are four consecutive input channels j of its (gate, o)
