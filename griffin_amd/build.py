@@ -50,6 +50,14 @@ def build(verbose: bool = False) -> str:
         raise RuntimeError("hipcc failed:\n" + log)
     if verbose and log.strip():
         print(log)
+    # A kernel template whose body the host pass cannot instantiate (seen with a target builtin called directly in a
+    # __global__ template) loses its launch stub without any diagnostic; the library then links but does not load.
+    missing = [line.split()[-1] for line in
+               subprocess.run(["nm", "-D", "--undefined-only", tmp], capture_output=True, text=True).stdout.splitlines()
+               if "__device_stub__" in line]
+    if missing:
+        os.remove(tmp)
+        raise RuntimeError("hipcc produced a library with undefined kernel stubs (would not load): " + ", ".join(missing[:4]))
     os.replace(tmp, LIB_PATH)
     return LIB_PATH
 
