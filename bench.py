@@ -7,7 +7,8 @@ One step = one forward + one backward of the RG-LRU (gates + scan, recomputing b
 batch of synthetic input, B=8, T=2048, W=1024, 8 gate blocks, bf16 storage with fp32 state: the
 configuration the headline metric is quoted on.  Inputs are resident in HBM before the timed region.
 The steps are replayed as HIP graphs of ten steps that rotate through S distinct input sets (cache-cold);
-the figure is the median of R timed regions of exactly K steps.  Prints ONE JSON line: metric, the
+the figure is the median of R timed regions of exactly K steps, taken after the W warm-up steps and 0.2 s
+more of untimed steps (an idle GPU runs its first 50 ms of load about 10 % slower).  Prints ONE JSON line: metric, the
 whole-step HBM roofline (5 s N algorithmic bytes over the step time; measured traffic from the committed
 profile summary if it was taken on the current kernel sources), per-kernel HIP-event durations, a check
 of the captured step against an eager one (exit status 1 if they differ) and the CPU baseline (the oracle
@@ -41,6 +42,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0
 
 BENCH_SHAPE = (8, 2048, 1024, 8)
+SETTLE_S = 0.2      # untimed steps in front of the timed regions, see time_region
 
 
 def parse_args():
@@ -502,9 +504,19 @@ def main():
             graphs = {}
 
     def time_region(run, calls):
-        """Median over `repeats` timed regions of exactly K steps each (ms per step)."""
+        """Median over `repeats` timed regions of exactly K steps each (ms per step).  In front of them, untimed:
+        the W warm-up steps, then the same launches for SETTLE_S seconds.  A GPU that has been idle runs its first
+        50 ms of load about 10 % slower (five regions of 20 steps read 0.128, 0.124, 0.123, 0.121, 0.121 ms straight
+        after five warm-up steps and 0.1134 +- 0.0003 after sixty milliseconds of them), and a training run is not
+        in that state."""
         for _ in range(max((args.warmup + per_graph - 1) // per_graph, 1)):
             run()
+        torch.cuda.synchronize()
+        settle_until = time.perf_counter() + SETTLE_S
+        while time.perf_counter() < settle_until:
+            for _ in range(calls):
+                run()
+            torch.cuda.synchronize()
         samples = []
         for _ in range(args.repeats):
             torch.cuda.synchronize()
@@ -588,7 +600,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"RG-LRU fwd+bwd B{B} T{T} W{W} nb{nb} bf16", "batch": B, "seq_len": T,
                    "width": W, "gate_blocks": nb, "state_dtype": "f32", "launch": launch,
-                   "timed_regions": args.repeats, "ms_per_step_samples": samples},
+                   "timed_regions": args.repeats, "ms_per_step_samples": samples,
+                   "settle": f"{SETTLE_S} s of untimed steps after the warm-up steps (clock ramp of an idle GPU)"},
         "roofline": {"bound": "hbm", "scope": "whole fwd+bwd step (5 s N algorithmic bytes over ms_per_step)",
                      "achieved": step_gbps, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": step_gbps / HBM_PEAK_GBS,
                      "traffic": None if traffic_rec is None else traffic_rec["whole_step_bytes"],
