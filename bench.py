@@ -68,10 +68,15 @@ def parse_args():
 
 
 def _timed(run, steps, warmup):
-    """Milliseconds per call of run(), eager launches, synchronised on both sides."""
+    """Milliseconds per call of run(), synchronised on both sides; after the warm-up calls the same call is
+    repeated, untimed, for SETTLE_S seconds (clock ramp of an idle GPU, see time_region)."""
     for _ in range(max(warmup, 1)):
         run()
     torch.cuda.synchronize()
+    settle_until = time.perf_counter() + SETTLE_S
+    while time.perf_counter() < settle_until:
+        run()
+        torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
         run()
@@ -160,6 +165,10 @@ def secondary_workload(args):
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph):
             kept = [one() for _ in range(per_graph)]
+        settle_until = time.perf_counter() + SETTLE_S
+        while time.perf_counter() < settle_until:
+            graph.replay()
+            torch.cuda.synchronize()
         samples = []
         for _ in range(6):
             torch.cuda.synchronize()
