@@ -2356,7 +2356,8 @@ __global__ __launch_bounds__(kGradThreads, 1) void gate_grad_wide_kernel(FusedAr
   constexpr int NV_DU = (TR * VPR_DU + kGradThreads - 1) / kGradThreads;
   static_assert(TR * VPR_X <= kGradThreads, "one x vector per thread");
   const int unit_col = k * p.bw + jg * JW;                 // first channel of the unit
-  Frag pre_du[NV_DU], pre_x, pre_dx;
+  struct Pre { Frag du[NV_DU]; Frag x, dx; };
+  Pre preA, preB;                                          // register sets of the tiles one and two passes ahead
   unsigned du_off[NV_DU], x_off;
 #pragma unroll
   for (int i = 0; i < NV_DU; ++i) {
@@ -2368,7 +2369,7 @@ __global__ __launch_bounds__(kGradThreads, 1) void gate_grad_wide_kernel(FusedAr
     const int row = tid / VPR_X, cv = tid - row * VPR_X;
     x_off = (tid < TR * VPR_X && jg * JW + cv * Tr::HW < KC) ? (unsigned)row * row_bytes + (unsigned)(unit_col + cv * Tr::HW) * 2u : kOutOfRange;
   }
-  auto issue = [&](long long tile) {
+  auto issue = [&](Pre& s, long long tile) {
     // a tile past the end keeps valid addresses but an empty extent: nothing is fetched
     const bool live = tile < n_tiles;
     const long long row0 = live ? tile * TR : 0;
@@ -2377,49 +2378,56 @@ __global__ __launch_bounds__(kGradThreads, 1) void gate_grad_wide_kernel(FusedAr
     const rsrc_t rx = make_rsrc((const IO*)p.x + row0 * p.W, (unsigned)rows * row_bytes);
     const rsrc_t rdx = make_rsrc((const IO*)p.dx + row0 * p.W, (unsigned)rows * row_bytes);
 #pragma unroll
-    for (int i = 0; i < NV_DU; ++i) pre_du[i] = buf_load_frag<Frag>(rdu, du_off[i]);
-    pre_x = buf_load_frag<Frag>(rx, x_off);
-    pre_dx = buf_load_frag<Frag>(rdx, x_off);
+    for (int i = 0; i < NV_DU; ++i) s.du[i] = buf_load_frag<Frag>(rdu, du_off[i]);
+    s.x = buf_load_frag<Frag>(rx, x_off);
+    s.dx = buf_load_frag<Frag>(rdx, x_off);
   };
   // the tile in the registers above goes to LDS buffer b
-  auto deposit = [&](int b) {
+  auto deposit = [&](const Pre& s, int b) {
 #pragma unroll
     for (int i = 0; i < NV_DU; ++i) {
       const int idx = tid + i * kGradThreads;
       const int row = idx / VPR_DU, cv = idx - row * VPR_DU;
-      if (idx < TR * VPR_DU) *reinterpret_cast<Frag*>(lds_du[b] + row * ROW_DU + cv * Tr::HW) = pre_du[i];
+      if (idx < TR * VPR_DU) *reinterpret_cast<Frag*>(lds_du[b] + row * ROW_DU + cv * Tr::HW) = s.du[i];
     }
     if (tid < TR * VPR_X) {
       const int row = tid / VPR_X, cv = tid - row * VPR_X;
-      *reinterpret_cast<Frag*>(lds_x[b] + row * ROW_X + cv * Tr::HW) = pre_x;
-      *reinterpret_cast<Frag*>(lds_dx[b] + row * ROW_X + cv * Tr::HW) = pre_dx;
+      *reinterpret_cast<Frag*>(lds_x[b] + row * ROW_X + cv * Tr::HW) = s.x;
+      *reinterpret_cast<Frag*>(lds_dx[b] + row * ROW_X + cv * Tr::HW) = s.dx;
     }
   };
 
+  // The tiles are requested two passes ahead, into two register sets that alternate (one pass of 2 us does not
+  // cover a load that misses L2: 378 -> 345 us at B1 T32768 W2560).  Every pass ends with one store behind the loads
+  // it issued; stores that their offset drops put the passes in front of the loop into the same state, so the wait
+  // for a set's loads leaves the younger set's loads and the stores in flight on every path into the loop (the
+  // counter is in issue order; without this the compiler must wait for everything, the store of the tile just
+  // finished included).
   long long tile = wg_in_unit;
-  issue(tile);
+  const i32x4 nothing = {0, 0, 0, 0};
+  const rsrc_t nowhere = make_rsrc(p.dx, 0u);
+  issue(preA, tile);
   if (DB) {
-    deposit(0);
-    issue(tile + n_wg);
+    deposit(preA, 0);
+    issue(preB, tile + n_wg);
+    buf_store_b128(nothing, nowhere, kOutOfRange);
+    issue(preA, tile + 2 * n_wg);
+    buf_store_b128(nothing, nowhere, kOutOfRange - 16u);
     __syncthreads();
-  }
-  // Every pass of the loop ends with one store behind the loads of the tile after next.  A store that its offset
-  // drops puts the first pass into the same state, so the wait for those loads can leave one operation in flight
-  // on every path into the loop (the counter is in issue order; without this the compiler must wait for everything,
-  // the store of the tile just finished included).
-  {
-    const i32x4 nothing = {0, 0, 0, 0};
-    buf_store_b128(nothing, make_rsrc(p.dx, 0u), kOutOfRange);
+  } else {
+    buf_store_b128(nothing, nowhere, kOutOfRange);
+    issue(preB, tile + n_wg);
+    buf_store_b128(nothing, nowhere, kOutOfRange - 16u);
   }
   int buf = 0;
-  for (; tile < n_tiles; tile += n_wg) {
+  auto pass = [&](Pre& s) {
     if (DB) {
       // the buffer of the tile before this one: every wave has passed the barrier that ended its reads
-      deposit(buf ^ 1);
-      issue(tile + 2 * n_wg);
+      deposit(s, buf ^ 1);
+      issue(s, tile + 3 * n_wg);
     } else {
-      deposit(0);
-      issue(tile + n_wg);
+      deposit(s, 0);
+      issue(s, tile + 2 * n_wg);
       __syncthreads();
     }
     const long long row0 = tile * TR;
@@ -2483,6 +2491,13 @@ __global__ __launch_bounds__(kGradThreads, 1) void gate_grad_wide_kernel(FusedAr
       wave_lds_fence();
     }
     if (DB) buf ^= 1;
+    tile += n_wg;
+  };
+  for (;;) {
+    if (tile >= n_tiles) break;
+    pass(DB ? preB : preA);
+    if (tile >= n_tiles) break;
+    pass(DB ? preA : preB);
   }
   // per-workgroup partial of the weight gradients, laid out like the gradients themselves: [wg][k][gate][o][j];
   // a lane's registers 4 v4 .. 4 v4 + 3 are four consecutive input channels j of its (gate, o)
