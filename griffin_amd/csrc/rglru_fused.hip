@@ -895,7 +895,16 @@ __global__ __launch_bounds__(kChainWaves * 64, 1) void fwd_chain_kernel(FusedArg
   const int sl = slot % S, u = (slot / S) * 8 + xcd;       // slab of the block; (sequence, block) pair
   const bool chain_ok = u < p.B * p.nb;                    // the grid is rounded up to whole rounds of eight pairs
   const int b = chain_ok ? u / p.nb : 0, k = chain_ok ? u - b * p.nb : 0;
-  for (int i = tid; i < kChainWaves * 32; i += kChainWaves * 64) (&carry[0][0])[i] = 0ull;
+  // Hand-off entries {tile number + 1, state}, all "nothing yet" -- except the last wave's, which tile 0 reads: it
+  // starts out as {0, h0}, what a tile in front of the sequence would have left.  Tile 0 then takes its state like
+  // every other tile (the initial state kept in a register for it was spilled, and the reload on that path put a
+  // wait for all memory operations into every hand-off).
+  for (int i = tid; i < kChainWaves * 32; i += kChainWaves * 64) {
+    unsigned long long entry = 0ull;
+    if (i >= (kChainWaves - 1) * 32 && chain_ok && p.h0)
+      entry = (unsigned long long)__float_as_uint(p.h0[(long long)b * p.W + k * KC + sl * 32 + (i - (kChainWaves - 1) * 32)]) << 32;
+    (&carry[0][0])[i] = entry;
+  }
   // The chain kernels use no carry records and no tickets: all this pass needs from the workspace is a failure word
   // that starts out zero.  Workgroup 0 clears it in its first instructions; a workgroup sets it only after it
   // has walked its whole chain, by which time that store has long landed.
@@ -967,8 +976,6 @@ __global__ __launch_bounds__(kChainWaves * 64, 1) void fwd_chain_kernel(FusedArg
   const rsrc_t rhl = make_rsrc(p.h_last, p.h_last ? (unsigned)p.B * (unsigned)W * 4u : 0u);
   const int prev_wave = (wave + kChainWaves - 1) % kChainWaves;
   bool gave_up = false;
-  // initial state of the chain (used by the wave of tile 0 only): no memory operation inside the loop is conditional
-  const float h_first = p.h0 ? p.h0[(long long)b * W + ch] : 0.f;
   issue(wave);
   {
     // The loop's back edge has four stores in flight behind the prefetched tile (final state, checkpoint, two
@@ -1016,10 +1023,10 @@ __global__ __launch_bounds__(kChainWaves * 64, 1) void fwd_chain_kernel(FusedArg
     const float A_lo = hf ? A_o : A, H_lo = hf ? H_o : H;
     const float A_hi = hf ? A : A_o, H_hi = hf ? H : H_o;
     const float A_t = A_hi * A_lo, H_t = fmaf(A_hi, H_lo, H_hi);
-    // the state in front of the tile: h0, or what the wave of the tile before has left in LDS.  A wait that
-    // runs out of polls hands on NaN, so the failure shows in the results; every wave still reaches the end.
-    float h_in = h_first;
-    if (c != 0) {
+    // the state in front of the tile: what the wave of the tile before has left in LDS (h0 for tile 0).  A wait
+    // that runs out of polls hands on NaN, so the failure shows in the results; every wave still reaches the end.
+    float h_in;
+    {
       long long polls = 0;
       bool ok;
       for (;;) {
