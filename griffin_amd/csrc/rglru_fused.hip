@@ -2413,28 +2413,37 @@ __global__ __launch_bounds__(kGradThreads, 1) void gate_grad_wide_kernel(FusedAr
   long long tile = wg_in_unit;
   const i32x4 nothing = {0, 0, 0, 0};
   const rsrc_t nowhere = make_rsrc(p.dx, 0u);
+  // (352 and 384 channels: six accumulator tiles a wave, no room for the second set -- one pass ahead.)
+  constexpr bool TWO = NI <= 5;
+  constexpr int AHEAD = (DB ? 2 : 1) + (TWO ? 1 : 0);      // passes between a tile's request and its multiplication
   issue(preA, tile);
   if (DB) {
     deposit(preA, 0);
-    issue(preB, tile + n_wg);
-    buf_store_b128(nothing, nowhere, kOutOfRange);
-    issue(preA, tile + 2 * n_wg);
+    if (TWO) {
+      issue(preB, tile + n_wg);
+      buf_store_b128(nothing, nowhere, kOutOfRange);
+      issue(preA, tile + 2 * n_wg);
+    } else {
+      issue(preA, tile + n_wg);
+    }
     buf_store_b128(nothing, nowhere, kOutOfRange - 16u);
     __syncthreads();
   } else {
     buf_store_b128(nothing, nowhere, kOutOfRange);
-    issue(preB, tile + n_wg);
-    buf_store_b128(nothing, nowhere, kOutOfRange - 16u);
+    if (TWO) {
+      issue(preB, tile + n_wg);
+      buf_store_b128(nothing, nowhere, kOutOfRange - 16u);
+    }
   }
   int buf = 0;
   auto pass = [&](Pre& s) {
     if (DB) {
       // the buffer of the tile before this one: every wave has passed the barrier that ended its reads
       deposit(s, buf ^ 1);
-      issue(s, tile + 3 * n_wg);
+      issue(s, tile + AHEAD * n_wg);
     } else {
       deposit(s, 0);
-      issue(s, tile + 2 * n_wg);
+      issue(s, tile + AHEAD * n_wg);
       __syncthreads();
     }
     const long long row0 = tile * TR;
@@ -2502,9 +2511,9 @@ __global__ __launch_bounds__(kGradThreads, 1) void gate_grad_wide_kernel(FusedAr
   };
   for (;;) {
     if (tile >= n_tiles) break;
-    pass(DB ? preB : preA);
+    pass(TWO && DB ? preB : preA);
     if (tile >= n_tiles) break;
-    pass(DB ? preA : preB);
+    pass(TWO && !DB ? preB : preA);
   }
   // per-workgroup partial of the weight gradients, laid out like the gradients themselves: [wg][k][gate][o][j];
   // a lane's registers 4 v4 .. 4 v4 + 3 are four consecutive input channels j of its (gate, o)
