@@ -169,6 +169,7 @@ struct FusedArgs {
   int dw_bf16;                                            // fast backward: per-workgroup weight-gradient sums stored as bf16
   int xcd_map;                                            // wide blocks: the workgroups that share a block's x tiles sit on one XCD
   int first_reset;                                        // token 0 of every sequence carries RGLRU_FLAG_RESET (and flags is null)
+  unsigned bw_magic;                                      // decode step: ceil(2^32 / bw), channel / bw as a multiply-high (channel < 2^16)
   long long limit;
 };
 
@@ -2752,14 +2753,14 @@ __global__ __launch_bounds__(kThreads) void step16_kernel(FusedArgs p) {
   typedef bf16x8 Frag;
   typedef float f32x4v __attribute__((ext_vector_type(4)));
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, n = lane & 15, q = lane >> 4;
-  const int ctiles = p.W / 16;
-  const long long wv = (long long)blockIdx.x * kWaves + wave;
-  const int ct = (int)(wv % ctiles);
-  const long long row0 = (wv / ctiles) * 16;
-  if (row0 >= p.B) return;
+  // Grid: x = groups of four channel tiles (one per wave), y = tiles of 16 sequences.  No division on the way to the
+  // first load: what this kernel takes is latency, and a 64-bit division by the tile count alone was 150 instructions.
+  const int ct = (int)blockIdx.x * kWaves + wave;
+  if (ct * 16 >= p.W) return;
+  const long long row0 = (long long)blockIdx.y * 16;
   const long long W = p.W;
   const int ch = ct * 16 + n;                              // the lane's channel; a tile lies inside one gate block
-  const int k = ch / p.bw, o = ch - k * p.bw;
+  const int k = (int)__umulhi((unsigned)(ct * 16), p.bw_magic), o = ch - k * p.bw;
   const int kp = k * p.bwp + o;
   // A fragments: row m = lane % 16 is sequence row0 + m, element j of K step ks is input channel 32 ks + 8 q + j
   const long long arow = row0 + n;
@@ -2767,7 +2768,7 @@ __global__ __launch_bounds__(kThreads) void step16_kernel(FusedArgs p) {
   const IO* xr = (const IO*)p.x + (arow_ok ? arow : 0) * W + k * p.bw + 8 * q;
   Frag xa[NKS], fa[NKS], fx[NKS];
 #pragma unroll
-  for (int ks = 0; ks < NKS; ++ks) xa[ks] = arow_ok ? *reinterpret_cast<const Frag*>(xr + 32 * ks) : Io<IO>::zero();
+  for (int ks = 0; ks < NKS; ++ks) xa[ks] = *reinterpret_cast<const Frag*>(xr + 32 * ks);   // a row past the end reads row 0: its products are not used
   // B fragments: column n is output channel o, same K elements: rows of the two weight matrices
   const IO* wa = (const IO*)p.wg + ((long long)(0 * p.nb + k) * p.bwp + o) * p.bwp + 8 * q;
   const IO* wx = (const IO*)p.wg + ((long long)(1 * p.nb + k) * p.bwp + o) * p.bwp + 8 * q;
@@ -2779,17 +2780,32 @@ __global__ __launch_bounds__(kThreads) void step16_kernel(FusedArgs p) {
   // accumulator register v of the lane is sequence row0 + 4 q + v
   float h_old[4], gate[4], xv[4];
   unsigned fls[4];
+  // Every load below is made on every path, from row 0 where the lane's row does not exist (its value is never used)
+  // and from x where there is no gate or flag tensor: loads under a condition end up in blocks of their own, each
+  // waiting for its data before the next block issues its loads -- eight memory round trips in a row in a kernel that
+  // is nothing but latency.  Unconditional, all of them are in flight together behind the fragment loads.
+  const IO* gate_src = p.gate_v ? (const IO*)p.gate_v : (const IO*)p.x;
+  const long long gate_ld = p.gate_v ? p.ld_gate : W;
+  const unsigned char* flag_src = p.flags ? p.flags : (const unsigned char*)p.x;
+  IO x_raw[4], gate_raw[4];
+  unsigned char fl_raw[4];
 #pragma unroll
   for (int v = 0; v < 4; ++v) {
     const long long row = row0 + 4 * q + v;
-    const bool ok = row < p.B;
-    const long long at = ok ? row * W + ch : 0;
-    h_old[v] = ok ? p.h_prev[at] : 0.f;
-    xv[v] = ok ? (float)((const IO*)p.x)[at] : 0.f;
-    gate[v] = (ok && p.gate_v) ? (float)((const IO*)p.gate_v)[row * p.ld_gate + ch] : 0.f;
-    fls[v] = (ok && p.flags) ? (unsigned)p.flags[row] : 0u;
+    const long long rr = row < p.B ? row : 0;
+    h_old[v] = p.h_prev[rr * W + ch];
+    x_raw[v] = ((const IO*)p.x)[rr * W + ch];
+    gate_raw[v] = gate_src[rr * gate_ld + ch];
+    fl_raw[v] = flag_src[rr];
   }
   const float bias_a = p.bias[kp], bias_x = p.bias[p.Wp + kp], sp = p.sp[kp];
+  __builtin_amdgcn_sched_barrier(0);                       // or the compiler issues some of them behind the matrix products
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    xv[v] = (float)x_raw[v];
+    gate[v] = (float)gate_raw[v];
+    fls[v] = p.flags ? (unsigned)fl_raw[v] : 0u;
+  }
   f32x4v ua = {bias_a, bias_a, bias_a, bias_a}, ux = {bias_x, bias_x, bias_x, bias_x};
 #pragma unroll
   for (int ks = 0; ks < NKS; ++ks) {
@@ -2797,16 +2813,22 @@ __global__ __launch_bounds__(kThreads) void step16_kernel(FusedArgs p) {
     ux = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[ks], fx[ks], ux, 0, 0, 0);
   }
   IO* y = (IO*)p.y;
+  // the four elements side by side (their transcendental chains overlap), then the stores of the rows that exist
+  float h_new[4], out[4];
+#pragma unroll
+  for (int v = 0; v < 4; ++v) {
+    const GateOut go = gate_forward<Precise<IO>::value, true>(ua[v], ux[v], xv[v], sp, fls[v]);
+    h_new[v] = fmaf(go.a, h_old[v], go.z);
+    out[v] = p.gate_v ? h_new[v] * gelu_tanh_parts(gate[v]).gelu : h_new[v];
+  }
 #pragma unroll
   for (int v = 0; v < 4; ++v) {
     const long long row = row0 + 4 * q + v;
-    if (row >= p.B) break;
-    const GateOut go = gate_forward<Precise<IO>::value, true>(ua[v], ux[v], xv[v], sp, fls[v]);
-    const long long at = row * W + ch;
-    float h = fmaf(go.a, h_old[v], go.z);
-    p.h_state[at] = h;
-    if (p.gate_v) h *= gelu_tanh_parts(gate[v]).gelu;
-    y[at] = (IO)h;
+    if (row < p.B) {
+      const long long at = row * W + ch;
+      p.h_state[at] = h_new[v];
+      y[at] = (IO)out[v];
+    }
   }
 }
 
@@ -2841,51 +2863,70 @@ __global__ __launch_bounds__(kThreads) void steps16_kernel(FusedArgs p) {
     fa[ks] = *reinterpret_cast<const Frag*>(wa + 32 * ks);
     fx[ks] = *reinterpret_cast<const Frag*>(wx + 32 * ks);
   }
-  long long at[4];
+  long long at[4], rowc[4];
   bool ok[4];
   float h[4];
 #pragma unroll
   for (int v = 0; v < 4; ++v) {
     const long long row = row0 + 4 * q + v;
     ok[v] = row < p.B;
-    at[v] = ok[v] ? row * W + ch : 0;
-    h[v] = ok[v] ? p.h_prev[at[v]] : 0.f;
+    rowc[v] = ok[v] ? row : 0;                             // a row past the end reads row 0; nothing of it is stored
+    at[v] = rowc[v] * W + ch;
+    h[v] = p.h_prev[at[v]];
   }
   const float bias_a = p.bias[kp], bias_x = p.bias[p.Wp + kp], sp = p.sp[kp];
-  Frag xa[NKS];
-  IO xv[4];
-  unsigned fls[4];
-  auto issue = [&](int t) {
-    const bool live = t < steps;
-    const long long base = live ? (long long)t * step_elems : 0;
+  // Operands of a step: requested kAhead steps ahead, into as many register sets that take turns -- a step takes
+  // under a microsecond, less than a load that comes from memory.  Per token at B256 W1024 (gate blocks of 128
+  // channels): 1.13 us one step ahead, 0.84 / 0.77 / 0.71 / 0.67 / 0.71 us at 2 / 3 / 4 / 6 / 8; wider blocks have
+  // larger sets and take fewer.
+  constexpr int kAhead = NKS <= 4 ? 6 : NKS <= 8 ? 4 : 2;
+  struct In { Frag xa[NKS]; IO xv[4]; unsigned char fl[4]; };
+  In in[kAhead];
+  // Loads and stores of the loop are made on every path (clamped addresses, stores dropped through their offset):
+  // the wait for a step's operands can then leave the younger loads and stores in flight; with conditional ones
+  // the compiler had to wait for everything, the stores just issued included, every step.
+  const unsigned char* flag_src = p.flags ? p.flags : (const unsigned char*)p.x;   // no flags: some readable byte
+  const long long flag_step = p.flags ? p.B : 0;
+  long long flag_row[4];
 #pragma unroll
-    for (int ks = 0; ks < NKS; ++ks) xa[ks] = (arow_ok && live) ? *reinterpret_cast<const Frag*>(xr + base + 32 * ks) : Io<IO>::zero();
+  for (int v = 0; v < 4; ++v) flag_row[v] = p.flags ? rowc[v] : 0;
+  auto issue = [&](In& s, int t) {
+    const long long tt = t < steps ? t : 0;                // a step past the end re-reads step 0
+    const long long base = tt * step_elems;
+#pragma unroll
+    for (int ks = 0; ks < NKS; ++ks) s.xa[ks] = *reinterpret_cast<const Frag*>(xr + base + 32 * ks);
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
-      xv[v] = (ok[v] && live) ? ((const IO*)p.x)[base + at[v]] : (IO)0.0f;
-      fls[v] = (p.flags && ok[v] && live) ? (unsigned)p.flags[(long long)t * p.B + row0 + 4 * q + v] : 0u;
+      s.xv[v] = ((const IO*)p.x)[base + at[v]];
+      s.fl[v] = flag_src[tt * flag_step + flag_row[v]];
     }
   };
-  issue(0);
-  for (int t = 0; t < steps; ++t) {
+  auto step = [&](In& s, int t) {
     f32x4v ua = {bias_a, bias_a, bias_a, bias_a}, ux = {bias_x, bias_x, bias_x, bias_x};
 #pragma unroll
     for (int ks = 0; ks < NKS; ++ks) {
-      ua = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[ks], fa[ks], ua, 0, 0, 0);
-      ux = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xa[ks], fx[ks], ux, 0, 0, 0);
+      ua = __builtin_amdgcn_mfma_f32_16x16x32_bf16(s.xa[ks], fa[ks], ua, 0, 0, 0);
+      ux = __builtin_amdgcn_mfma_f32_16x16x32_bf16(s.xa[ks], fx[ks], ux, 0, 0, 0);
     }
     float xcur[4];
     unsigned fcur[4];
 #pragma unroll
-    for (int v = 0; v < 4; ++v) { xcur[v] = (float)xv[v]; fcur[v] = fls[v]; }
-    issue(t + 1);
-    IO* y = (IO*)p.y + (long long)t * step_elems;
+    for (int v = 0; v < 4; ++v) { xcur[v] = (float)s.xv[v]; fcur[v] = p.flags ? (unsigned)s.fl[v] : 0u; }
+    issue(s, t + kAhead);
+    const rsrc_t ry = make_rsrc((IO*)p.y + (long long)t * step_elems, (unsigned)step_elems * 2u);
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
       const GateOut go = gate_forward<Precise<IO>::value, true>(ua[v], ux[v], xcur[v], sp, fcur[v]);
       h[v] = fmaf(go.a, h[v], go.z);
-      if (ok[v]) y[at[v]] = (IO)h[v];
+      BufIo<IO>::store((IO)h[v], ry, ok[v] ? (unsigned)at[v] * 2u : kOutOfRange, 0u);
     }
+  };
+#pragma unroll
+  for (int j = 0; j < kAhead; ++j) issue(in[j], j);
+  for (int t = 0; t < steps; t += kAhead) {
+#pragma unroll
+    for (int j = 0; j < kAhead; ++j)
+      if (t + j < steps) step(in[j], t + j);
   }
 #pragma unroll
   for (int v = 0; v < 4; ++v) if (ok[v]) p.h_state[at[v]] = h[v];
@@ -3863,8 +3904,9 @@ static int step_impl(const void* x, const void* prep, const float* h_in, float* 
     KernelTimer timer(2, s);
     if (nks > 0) {
       // 16 sequences x 16 channels per wave, four waves per workgroup
-      const long long waves = ((B + 15) / 16) * (W / 16);
-      dim3 grid16((unsigned)((waves + kWaves - 1) / kWaves));
+      if (B > 16ll * 65535 || W >= 65536) return fail(RGLRU_E_UNSUPPORTED, "step: more than 1048560 rows or 65535 channels");
+      a.bw_magic = (unsigned)(((1ull << 32) + (unsigned long long)g.bw - 1) / (unsigned long long)g.bw);
+      dim3 grid16((unsigned)((W / 16 + kWaves - 1) / kWaves), (unsigned)((B + 15) / 16));
       switch (nks) {
 #define RGLRU_STEP16_CASE(N) case N: hipLaunchKernelGGL((step16_kernel<N>), grid16, dim3(kThreads), 0, s, a); break
         RGLRU_STEP16_CASE(1); RGLRU_STEP16_CASE(2); RGLRU_STEP16_CASE(3); RGLRU_STEP16_CASE(4); RGLRU_STEP16_CASE(5);
@@ -3897,7 +3939,7 @@ int rglru_hip_steps(const void* x, const void* prep, float* h, const uint8_t* fl
   if (B <= 0 || K <= 0) return fail(RGLRU_E_ARG, "steps: K and B must be positive (got %lld, %lld)", (long long)K, (long long)B);
   if (!x || !prep || !h || !y) return fail(RGLRU_E_ARG, "steps: null pointer");
   if (flags == RGLRU_FLAGS_FIRST_RESET) return fail(RGLRU_E_ARG, "steps: RGLRU_FLAGS_FIRST_RESET is for whole sequences; pass one flag byte per step and row");
-  if (K * B * W >= (1ll << 40) || K >= (1ll << 31)) return fail(RGLRU_E_UNSUPPORTED, "steps: tensor too large");
+  if (K * B * W >= (1ll << 40) || K >= (1ll << 31) || B * W >= (1ll << 31)) return fail(RGLRU_E_UNSUPPORTED, "steps: tensor too large");
   Geometry g = make_geometry(W, nb);
   FusedArgs a;
   memset(&a, 0, sizeof(a));
