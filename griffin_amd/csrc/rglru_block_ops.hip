@@ -112,9 +112,15 @@ RGLRU_DEVICE void conv_params(const void* base, long long first, int vec_dtype, 
           if (4 * q + i < N) out[4 * q + i] = __uint_as_float(w[i]);
       }
     }
+  } else if (vec_dtype == RGLRU_BF16) {                    // one branch on the type, then all loads in flight together
+    __bf16 raw[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) raw[i] = ((const __bf16*)base)[first + i];
+#pragma unroll
+    for (int i = 0; i < N; ++i) out[i] = (float)raw[i];
   } else {
 #pragma unroll
-    for (int i = 0; i < N; ++i) out[i] = conv_param(base, first + i, vec_dtype);
+    for (int i = 0; i < N; ++i) out[i] = ((const float*)base)[first + i];
   }
 }
 
@@ -708,22 +714,38 @@ __global__ __launch_bounds__(kConvThreads) void decode_prepare_kernel(DecodeArgs
   const int vec = (int)(item % p.nvec), b = (int)(item / p.nvec);
   const int c0 = vec * V;
   const unsigned es = (unsigned)sizeof(IO), uW = (unsigned)p.W;
-  const bool live = p.active ? p.active[b] != 0 : true;
-  const long long before = p.prev_pos ? p.prev_pos[b] : -1;
-  const long long pos = p.seg_pos ? p.seg_pos[b] : before + (live ? 1 : 0);
+  // The step is a chain of latencies, so everything it reads is requested before anything is used: the row's
+  // activity byte and positions (from a readable dummy where the caller passes none; a load under a condition sits
+  // in a block of its own and waits there), then the input row and the carried rows.  The descriptors span the
+  // whole tensors with the row in the lane offset: a descriptor per row differs from lane to lane, and every access
+  // through one becomes a loop over the wave's distinct rows that ends in a wait for all memory operations.
+  const unsigned char* active_src = p.active ? p.active + b : p.flags + b;
+  const long long* before_src = p.prev_pos ? p.prev_pos + b : p.new_pos + b;
+  const long long* pos_src = p.seg_pos ? p.seg_pos + b : p.new_pos + b;
+  const unsigned char active_raw = *active_src;
+  const long long before_raw = *before_src, pos_raw = *pos_src;
+  const rsrc_t ru = make_rsrc(p.u, (unsigned)(((long long)(p.B - 1) * p.ldu + p.W) * es));
+  const rsrc_t rx = make_rsrc(p.x, (unsigned)p.B * uW * es);
+  const unsigned off = (unsigned)c0 * es;
+  const unsigned row_x = (unsigned)b * uW * es, row_s = (unsigned)b * (unsigned)(K - 1) * uW * es;
+  float cur[V], acc[V], hist[K > 1 ? K - 1 : 1][V];          // hist[j] = state row j (oldest first)
+  const rsrc_t rs = make_rsrc(p.state ? p.state : p.u, p.state ? (unsigned)p.B * (unsigned)(K - 1) * uW * es : 0u);
+  const typename Row::Raw cur_raw = Row::request(ru, (unsigned)((long long)b * p.ldu * es) + off);
+  typename Row::Raw hist_raw[K > 1 ? K - 1 : 1];
+#pragma unroll
+  for (int j = 0; j < K - 1; ++j) hist_raw[j] = Row::request(rs, row_s + ((unsigned)j * uW + (unsigned)c0) * es);
+  float tap[K][V], bias[V];
+  conv_load_taps<V, K>(p.taps, p.bias, c0, p.vec_dtype, tap, bias);
+  const bool live = p.active ? active_raw != 0 : true;
+  const long long before = p.prev_pos ? before_raw : -1;
+  const long long pos = p.seg_pos ? pos_raw : before + (live ? 1 : 0);
   if (vec == 0) {
     p.new_pos[b] = live ? pos : before;
     p.flags[b] = (unsigned char)((live && pos == 0 ? RGLRU_FLAG_RESET : 0u) | (live ? 0u : RGLRU_FLAG_INACTIVE));
   }
-  const rsrc_t ru = make_rsrc((const IO*)p.u + (long long)b * p.ldu, uW * es);
-  const rsrc_t rx = make_rsrc((IO*)p.x + (long long)b * p.W, uW * es);
-  const unsigned off = (unsigned)c0 * es;
-  float cur[V], acc[V], hist[K > 1 ? K - 1 : 1][V];          // hist[j] = state row j (oldest first)
-  Row::load(cur, ru, off);
-  const rsrc_t rs = make_rsrc(p.state ? (const IO*)p.state + (long long)b * (K - 1) * p.W : (const IO*)p.u,
-                              p.state ? (unsigned)((K - 1) * p.W) * es : 0u);
+  Row::unpack(cur, cur_raw);
 #pragma unroll
-  for (int j = 0; j < K - 1; ++j) Row::load(hist[j], rs, ((unsigned)j * uW + (unsigned)c0) * es);
+  for (int j = 0; j < K - 1; ++j) Row::unpack(hist[j], hist_raw[j]);
   const bool padded = p.active != nullptr;
   if (padded && live && pos == 0) {                         // griffin/griffin.py:491-492
 #pragma unroll
@@ -731,8 +753,6 @@ __global__ __launch_bounds__(kConvThreads) void decode_prepare_kernel(DecodeArgs
 #pragma unroll
       for (int v = 0; v < V; ++v) hist[j][v] = 0.f;
   }
-  float tap[K][V], bias[V];
-  conv_load_taps<V, K>(p.taps, p.bias, c0, p.vec_dtype, tap, bias);
 #pragma unroll
   for (int v = 0; v < V; ++v) {
     float a = bias[v];
@@ -742,9 +762,9 @@ __global__ __launch_bounds__(kConvThreads) void decode_prepare_kernel(DecodeArgs
       if (padded || pos >= lag) a = fmaf(hist[K - 1 - lag][v], tap[K - 1 - lag][v], a);
     acc[v] = live ? a : 0.f;
   }
-  Row::store(acc, rx, off);
+  Row::store(acc, rx, row_x + off);
   if (K > 1) {
-    const rsrc_t rn = make_rsrc((IO*)p.new_state + (long long)b * (K - 1) * p.W, (unsigned)((K - 1) * p.W) * es);
+    const rsrc_t rn = make_rsrc(p.new_state, (unsigned)p.B * (unsigned)(K - 1) * uW * es);
 #pragma unroll
     for (int j = 0; j < K - 1; ++j) {
       float row[V];
@@ -753,7 +773,7 @@ __global__ __launch_bounds__(kConvThreads) void decode_prepare_kernel(DecodeArgs
         const float shifted = (j + 1 < K - 1) ? hist[j + 1 < K - 1 ? j + 1 : 0][v] : cur[v];
         row[v] = live ? shifted : hist[j][v];
       }
-      Row::store(row, rn, ((unsigned)j * uW + (unsigned)c0) * es);
+      Row::store(row, rn, row_s + ((unsigned)j * uW + (unsigned)c0) * es);
     }
   }
 }
@@ -1230,6 +1250,9 @@ int rglru_hip_decode_prepare(const void* u, int64_t u_stride, const void* conv_s
     return fail(RGLRU_E_ARG, "decode_prepare: null pointer");
   if (u_stride == 0) u_stride = W;
   if (u_stride < W) return fail(RGLRU_E_ARG, "decode_prepare: row stride %lld of u is smaller than the width %lld", (long long)u_stride, (long long)W);
+  // the kernel addresses whole tensors through one descriptor each, with 32-bit offsets
+  if (B * u_stride * 4 >= (1ll << 32) || B * (K > 1 ? K - 1 : 1) * W * 4 >= (1ll << 32))
+    return fail(RGLRU_E_UNSUPPORTED, "decode_prepare: tensors of 4 GiB or more");
   DecodeArgs a;
   memset(&a, 0, sizeof(a));
   a.u = u; a.state = conv_state; a.taps = taps; a.bias = bias;
