@@ -24,7 +24,7 @@ namespace rglru {
 
 constexpr int kConvMaxTaps = 4;        // kernel sizes 1..4 (the reference uses 4)
 constexpr int kConvRunFwd = 16;        // tokens per thread, forward
-constexpr int kConvRunBwd = 32;        // tokens per thread, backward (one partial sum per run)
+constexpr int kConvRunBwd = 16;        // tokens per thread, backward (one partial sum per run; 32 left half the chip's load slots idle)
 constexpr int kConvThreads = 256;
 constexpr int kConvBatch = 8;          // rows requested together, forward
 constexpr int kConvBatchBwd = 4;       // backward (two streams, more live state)
@@ -142,33 +142,50 @@ RGLRU_DEVICE void conv_load_taps(const void* taps, const void* bias_ptr, int c0,
   }
 }
 
-// Which (sequence, run, channel vector) a thread owns; vectors vary fastest, so the lanes of a wave
-// read consecutive addresses of one row.
+// Which (sequence, run, channel vector) a thread owns.  A workgroup stays inside one sequence
+// (blocks_per_seq workgroups each), so that the sequence, and with it every buffer descriptor built
+// from it, is the same in all lanes; vectors vary fastest, so the lanes of a wave read consecutive
+// addresses of one row.
 struct ConvItem { int b, run, c0; bool ok; };
+__host__ __device__ inline long long conv_blocks_per_seq(int runs, int nvec) {
+  return ((long long)runs * nvec + kConvThreads - 1) / kConvThreads;
+}
 RGLRU_DEVICE ConvItem conv_item(const ConvArgs& p) {
   ConvItem it;
-  const long long item = (long long)blockIdx.x * kConvThreads + threadIdx.x;
-  it.ok = item < (long long)p.B * p.runs * p.nvec;
+  const unsigned per_seq = (unsigned)conv_blocks_per_seq(p.runs, p.nvec);
+  it.b = (int)(blockIdx.x / per_seq);
+  const long long item = (long long)(blockIdx.x - (unsigned)it.b * per_seq) * kConvThreads + threadIdx.x;
+  it.ok = item < (long long)p.runs * p.nvec;
   const long long safe = it.ok ? item : 0;
-  const int vec = (int)(safe % p.nvec);
-  const long long rest = safe / p.nvec;
-  it.run = (int)(rest % p.runs); it.b = (int)(rest / p.runs);
-  it.c0 = vec * (p.W / p.nvec);
+  it.run = (int)(safe / p.nvec);
+  it.c0 = (int)(safe - (long long)it.run * p.nvec) * (p.W / p.nvec);
   return it;
 }
 
-// Row `t` of the padded input of sequence b (t < 0: carried state, zeros when there is none).
+// Row `t` of the padded input of one sequence (t < 0: carried state, zeros when there is none).  Both
+// sources are asked, the one that does not hold the row past its end, so that neither the descriptor
+// nor the control flow depends on the lane; `ok` false gives zeros.  `rs` is conv_state_rsrc().
 template <typename IO, int V, int K>
-RGLRU_DEVICE void padded_row(const ConvArgs& p, rsrc_t ru, int b, int t, int c0, float (&v)[V]) {
-  if (t >= 0) {
-    ConvRow<IO, V>::load(v, ru, ((unsigned)t * (unsigned)p.W + (unsigned)c0) * (unsigned)sizeof(IO));
-  } else if (p.state && K - 1 + t >= 0) {
-    const rsrc_t rs = make_rsrc((const IO*)p.state + (long long)b * (K - 1) * p.W, (unsigned)((K - 1) * p.W) * (unsigned)sizeof(IO));
-    ConvRow<IO, V>::load(v, rs, ((unsigned)(K - 1 + t) * (unsigned)p.W + (unsigned)c0) * (unsigned)sizeof(IO));
-  } else {
+RGLRU_DEVICE void padded_row(const ConvArgs& p, rsrc_t ru, rsrc_t rs, bool ok, int t, int c0, float (&v)[V]) {
+  const unsigned es = (unsigned)sizeof(IO);
+  const bool from_state = t < 0;
+  const unsigned off_u = ok && t >= 0 ? ((unsigned)t * (unsigned)p.W + (unsigned)c0) * es : kOutOfRange;
+  const unsigned off_s = ok && from_state && K - 1 + t >= 0 ? ((unsigned)(K - 1 + t) * (unsigned)p.W + (unsigned)c0) * es
+                                                            : kOutOfRange;
+  const typename ConvRow<IO, V>::Raw raw_u = ConvRow<IO, V>::request(ru, off_u);
+  const typename ConvRow<IO, V>::Raw raw_s = ConvRow<IO, V>::request(rs, off_s);
+  float from_u[V], from_s[V];
+  ConvRow<IO, V>::unpack(from_u, raw_u);
+  ConvRow<IO, V>::unpack(from_s, raw_s);
 #pragma unroll
-    for (int i = 0; i < V; ++i) v[i] = 0.f;
-  }
+  for (int i = 0; i < V; ++i) v[i] = from_state ? from_s[i] : from_u[i];
+}
+
+// The carried state of sequence b as a buffer (empty without one, so that its loads return zero).
+template <typename IO, int K>
+RGLRU_DEVICE rsrc_t conv_state_rsrc(const ConvArgs& p, int b) {
+  return make_rsrc(p.state ? (const IO*)p.state + (long long)b * (K - 1) * p.W : (const IO*)p.u,
+                   p.state ? (unsigned)((K - 1) * p.W) * (unsigned)sizeof(IO) : 0u);
 }
 
 template <typename IO, int V, int K>
@@ -182,11 +199,12 @@ __global__ __launch_bounds__(kConvThreads) void conv_fwd_kernel(ConvArgs p) {
   const unsigned seq_bytes = (unsigned)p.T * uW * es;
   const rsrc_t ru = make_rsrc((const IO*)p.u + (long long)b * p.T * p.W, seq_bytes);
   const rsrc_t ro = make_rsrc((const IO*)p.out + (long long)b * p.T * p.W, seq_bytes);
+  const rsrc_t rs = conv_state_rsrc<IO, K>(p, b);
   const long long* sp_row = p.segpos + (long long)b * p.T;
 
   float win[K > 1 ? K - 1 : 1][V];                         // win[j] = padded row t - 1 - j
 #pragma unroll
-  for (int j = 0; j < K - 1; ++j) padded_row<IO, V, K>(p, ru, b, t0 - 1 - j, c0, win[j]);
+  for (int j = 0; j < K - 1; ++j) padded_row<IO, V, K>(p, ru, rs, true, t0 - 1 - j, c0, win[j]);
   for (int t1 = 0; t1 < kConvRunFwd; t1 += kConvBatch) {
    typename ConvRow<IO, V>::Raw raw[kConvBatch];
    long long spb[kConvBatch];
@@ -229,7 +247,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_fwd_kernel(ConvArgs p) {
 #pragma unroll
     for (int j = 0; j < K - 1; ++j) {
       float row[V];
-      padded_row<IO, V, K>(p, ru, b, p.T - (K - 1) + j, c0, row);
+      padded_row<IO, V, K>(p, ru, rs, true, p.T - (K - 1) + j, c0, row);
       ConvRow<IO, V>::store(row, rn, ((unsigned)j * uW + (unsigned)c0) * es);
     }
   }
@@ -254,13 +272,16 @@ __global__ __launch_bounds__(kConvThreads) void conv_bwd_kernel(ConvArgs p) {
   const unsigned es = (unsigned)sizeof(IO), uW = (unsigned)p.W;
   float tap[K][V], bias_unused[V];
   conv_load_taps<V, K>(p.taps, nullptr, c0, p.vec_dtype, tap, bias_unused);
-  // a thread without work sees empty tensors: its loads return zero and its stores are dropped
-  const unsigned seq_bytes = ok ? (unsigned)p.T * uW * es : 0u;
+  // The descriptors are the same in all lanes.  A thread without work addresses past their end:
+  // its loads return zero and its stores are dropped.
+  const unsigned seq_bytes = (unsigned)p.T * uW * es;
   const rsrc_t ru = make_rsrc((const IO*)p.u + (long long)b * p.T * p.W, seq_bytes);
   const rsrc_t rd = make_rsrc((const IO*)p.dout + (long long)b * p.T * p.W, seq_bytes);
   const rsrc_t rg = make_rsrc((const IO*)p.du + (long long)b * p.T * p.W, seq_bytes);
+  const rsrc_t rs_in = conv_state_rsrc<IO, K>(p, b);
   const long long* sp_row = p.segpos + (long long)b * p.T;
   auto position = [&](int t) { return sp_row[t < p.T ? t : p.T - 1]; };
+  auto at = [&](int t) { return ok ? ((unsigned)t * uW + (unsigned)c0) * es : kOutOfRange; };
 
   float dwin[K][V];                                        // dwin[j] = dout row t + j
   long long spw[K];
@@ -274,14 +295,9 @@ __global__ __launch_bounds__(kConvThreads) void conv_bwd_kernel(ConvArgs p) {
   }
 #pragma unroll
   for (int j = 0; j < K - 1; ++j) {
-    ConvRow<IO, V>::load(dwin[j], rd, ((unsigned)(t0 + j) * uW + (unsigned)c0) * es);
+    ConvRow<IO, V>::load(dwin[j], rd, at(t0 + j));
     spw[j] = position(t0 + j);
-    if (ok) {
-      padded_row<IO, V, K>(p, ru, b, t0 - 1 - j, c0, uwin[j]);
-    } else {
-#pragma unroll
-      for (int v = 0; v < V; ++v) uwin[j][v] = 0.f;
-    }
+    padded_row<IO, V, K>(p, ru, rs_in, ok, t0 - 1 - j, c0, uwin[j]);
   }
   for (int t1 = 0; t1 < kConvRunBwd; t1 += kConvBatchBwd) {
     typename ConvRow<IO, V>::Raw raw_u[kConvBatchBwd], raw_d[kConvBatchBwd];
@@ -289,14 +305,14 @@ __global__ __launch_bounds__(kConvThreads) void conv_bwd_kernel(ConvArgs p) {
 #pragma unroll
     for (int i = 0; i < kConvBatchBwd; ++i) {
       const int t = t0 + t1 + i;
-      raw_u[i] = ConvRow<IO, V>::request(ru, ((unsigned)t * uW + (unsigned)c0) * es);
-      raw_d[i] = ConvRow<IO, V>::request(rd, ((unsigned)(t + K - 1) * uW + (unsigned)c0) * es);
+      raw_u[i] = ConvRow<IO, V>::request(ru, at(t));
+      raw_d[i] = ConvRow<IO, V>::request(rd, at(t + K - 1));
       spb[i] = position(t + K - 1);
     }
 #pragma unroll
     for (int i = 0; i < kConvBatchBwd; ++i) {
       const int t = t0 + t1 + i;
-      const unsigned off = ((unsigned)t * uW + (unsigned)c0) * es;
+      const unsigned off = at(t);
       ConvRow<IO, V>::unpack(dwin[K - 1], raw_d[i]);
       spw[K - 1] = spb[i];
       float cur[V], g[V];
@@ -1113,8 +1129,9 @@ int rglru_hip_conv_fwd(const void* u, const void* state, const void* taps, const
   const bool vec = conv_vector_ok(W, dtype, {u, state, out, new_state});
   a.nvec = (int)(vec ? W / (dtype == RGLRU_BF16 ? 8 : 4) : W);
   a.runs = (int)((T + kConvRunFwd - 1) / kConvRunFwd);
-  const long long items = (long long)B * a.runs * a.nvec;
-  dim3 grid((unsigned)((items + kConvThreads - 1) / kConvThreads));
+  const long long blocks = B * conv_blocks_per_seq(a.runs, a.nvec);
+  if (blocks >= (1ll << 31)) return fail(RGLRU_E_UNSUPPORTED, "conv_fwd: tensor too large");
+  dim3 grid((unsigned)blocks);
   hipStream_t s = (hipStream_t)stream;
   RGLRU_CONV_DISPATCH(conv_fwd_kernel, dtype, vec, grid, s, a);
   return check_launch("conv_fwd");
