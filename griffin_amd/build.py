@@ -11,12 +11,15 @@ import os
 import shutil
 import subprocess
 import sys
+import tempfile
+from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB_NAME = "librglru_hip.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
-SOURCES = ["rglru_scan.hip", "rglru_fused.hip", "rglru_gate_gemm.hip", "rglru_block_ops.hip"]
+SOURCES = ["rglru_scan.hip", "rglru_fused.hip", "rglru_fused_bwd.hip", "rglru_decode.hip", "rglru_gate_gemm.hip",
+           "rglru_block_ops.hip"]
 ARCH = "gfx950"
 
 
@@ -32,24 +35,35 @@ def hipcc_path() -> str:
 
 def build(verbose: bool = False) -> str:
     """Compile every kernel for gfx950 and link the shared library; returns its path."""
-    cmd = [
-        hipcc_path(), "-O3", "-std=c++17", "-fPIC", "-shared", f"--offload-arch={ARCH}",
+    flags = [
+        "-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}",
         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
         "-Wno-unused-command-line-argument", "-ffp-contract=off", "-fno-strict-aliasing",
         "-I", os.path.join(os.path.dirname(HERE), "include"),
     ]
-    cmd += [os.path.join(CSRC, s) for s in SOURCES]
-    tmp = LIB_PATH + ".tmp"
-    cmd += ["-o", tmp]
-    if verbose:
-        print(" ".join(cmd))
-    proc = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
-    log = "\n".join(line for line in (proc.stdout + proc.stderr).splitlines() if noise not in line)
-    if proc.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + log)
-    if verbose and log.strip():
-        print(log)
+    logs: list[str] = []
+
+    def run(cmd: list[str]) -> None:
+        if verbose:
+            print(" ".join(cmd))
+        proc = subprocess.run(cmd, capture_output=True, text=True)
+        log = "\n".join(line for line in (proc.stdout + proc.stderr).splitlines() if noise not in line)
+        if proc.returncode != 0:
+            raise RuntimeError("hipcc failed:\n" + log)
+        if log.strip():
+            logs.append(log)
+
+    # one object per source, compiled side by side, then one link
+    tmp = LIB_PATH + ".tmp"
+    with tempfile.TemporaryDirectory(prefix="rglru_build_") as objdir:
+        objects = [os.path.join(objdir, os.path.splitext(s)[0] + ".o") for s in SOURCES]
+        jobs = [[hipcc_path(), *flags, "-c", os.path.join(CSRC, s), "-o", o] for s, o in zip(SOURCES, objects)]
+        with ThreadPoolExecutor(max_workers=min(len(jobs), os.cpu_count() or 1)) as pool:
+            list(pool.map(run, jobs))
+        run([hipcc_path(), "-shared", "-fPIC", f"--offload-arch={ARCH}", *objects, "-o", tmp])
+    if verbose and logs:
+        print("\n".join(logs))
     # A kernel template whose body the host pass cannot instantiate (seen with a target builtin called directly in a
     # __global__ template) loses its launch stub without any diagnostic; the library then links but does not load.
     missing = [line.split()[-1] for line in

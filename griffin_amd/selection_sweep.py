@@ -1,6 +1,6 @@
 """Times both kernel pairs of the bf16 fast path -- tiles with a look-back between workgroups, and one workgroup per
 (sequence, 32-channel slab) chain -- over a grid of shapes and compares the faster one with what the library picks
-(rglru_hip_backward_path, i.e. the time models in fwd_chain_pays, rglru_fused.hip).
+(rglru_hip_backward_path, i.e. the time models in fwd_chain_pays, rglru_fused.h).
 
     python -m griffin_amd.selection_sweep [--quick]
 
