@@ -35,6 +35,7 @@ struct ConvArgs {
   const void* u; const void* state; const void* taps; const void* bias; const long long* segpos;
   void* out; void* new_state;                               // forward
   const void* dout; void* du; void* dstate; float* partial;  // backward
+  long long ld_du;                                          // elements between rows of du (>= W)
   int B, T, W, K, nvec, runs, vec_dtype;
 };
 
@@ -277,11 +278,13 @@ __global__ __launch_bounds__(kConvThreads) void conv_bwd_kernel(ConvArgs p) {
   const unsigned seq_bytes = (unsigned)p.T * uW * es;
   const rsrc_t ru = make_rsrc((const IO*)p.u + (long long)b * p.T * p.W, seq_bytes);
   const rsrc_t rd = make_rsrc((const IO*)p.dout + (long long)b * p.T * p.W, seq_bytes);
-  const rsrc_t rg = make_rsrc((const IO*)p.du + (long long)b * p.T * p.W, seq_bytes);
+  const unsigned ld_du = (unsigned)p.ld_du;
+  const rsrc_t rg = make_rsrc((const IO*)p.du + (long long)b * p.T * p.ld_du, ((unsigned)(p.T - 1) * ld_du + uW) * es);
   const rsrc_t rs_in = conv_state_rsrc<IO, K>(p, b);
   const long long* sp_row = p.segpos + (long long)b * p.T;
   auto position = [&](int t) { return sp_row[t < p.T ? t : p.T - 1]; };
   auto at = [&](int t) { return ok ? ((unsigned)t * uW + (unsigned)c0) * es : kOutOfRange; };
+  auto at_du = [&](int t) { return ok ? ((unsigned)t * ld_du + (unsigned)c0) * es : kOutOfRange; };
 
   float dwin[K][V];                                        // dwin[j] = dout row t + j
   long long spw[K];
@@ -312,7 +315,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_bwd_kernel(ConvArgs p) {
 #pragma unroll
     for (int i = 0; i < kConvBatchBwd; ++i) {
       const int t = t0 + t1 + i;
-      const unsigned off = at(t);
+      const unsigned off = at_du(t);
       ConvRow<IO, V>::unpack(dwin[K - 1], raw_d[i]);
       spw[K - 1] = spb[i];
       float cur[V], g[V];
@@ -802,7 +805,11 @@ __global__ __launch_bounds__(kConvThreads) void decode_prepare_kernel(DecodeArgs
 constexpr int kGateThreads = 256;
 constexpr int kGateBatch = 4;
 
-struct GateArgs { const void* h; const void* v; const void* dout; void* out; void* dh; void* dv; long long n; };
+struct GateArgs {
+  const void* h; const void* v; const void* dout; void* out; void* dh; void* dv; long long n;
+  long long ld_dv; int row_vecs; unsigned dv_bytes;         // backward with dv rows ld_dv elements apart (row_vecs vectors per row); 0: flat
+  unsigned row_magic;                                       // ceil(2^32 / row_vecs) where (vectors + row_vecs) * row_vecs < 2^32 (the multiply-high is then exact), else 0
+};
 
 template <typename IO, int V, bool BACKWARD>
 __global__ __launch_bounds__(kGateThreads) void gelu_gate_kernel(GateArgs p) {
@@ -818,7 +825,9 @@ __global__ __launch_bounds__(kGateThreads) void gelu_gate_kernel(GateArgs p) {
     const rsrc_t rv = make_rsrc((const IO*)p.v + w0, bytes);
     const rsrc_t rd = make_rsrc(BACKWARD ? (const IO*)p.dout + w0 : (const IO*)p.h, BACKWARD ? bytes : 0u);
     const rsrc_t ro = make_rsrc(BACKWARD ? (IO*)p.dh + w0 : (IO*)p.out + w0, bytes);
-    const rsrc_t rw = make_rsrc(BACKWARD ? (IO*)p.dv + w0 : (IO*)p.out, BACKWARD ? bytes : 0u);
+    // dv is flat like the rest, or has rows of its own stride (then the tensor is one window)
+    const bool dv_rows = BACKWARD && p.row_vecs > 0;
+    const rsrc_t rw = make_rsrc(BACKWARD ? (dv_rows ? (IO*)p.dv : (IO*)p.dv + w0) : (IO*)p.out, BACKWARD ? (dv_rows ? p.dv_bytes : bytes) : 0u);
     const long long wvec = (wn + V - 1) / V;
     (void)nvec;
     for (long long i0 = (long long)blockIdx.x * kGateThreads + threadIdx.x; i0 < wvec; i0 += stride * kGateBatch) {
@@ -848,7 +857,13 @@ __global__ __launch_bounds__(kGateThreads) void gelu_gate_kernel(GateArgs p) {
             b[e] = (d[e] * h[e]) * g.dgelu;
           }
           Row::store(a, ro, off);
-          Row::store(b, rw, off);
+          unsigned off_dv = off;
+          if (dv_rows && i < wvec) {
+            const unsigned row = p.row_magic ? __umulhi((unsigned)i, p.row_magic) : (unsigned)i / (unsigned)p.row_vecs;
+            const unsigned cv = (unsigned)i - row * (unsigned)p.row_vecs;
+            off_dv = (row * (unsigned)p.ld_dv + cv * V) * (unsigned)sizeof(IO);
+          }
+          Row::store(b, rw, off_dv);
         } else {
 #pragma unroll
           for (int e = 0; e < V; ++e) a[e] = h[e] * gelu_tanh_parts(v[e]).gelu;
@@ -1145,19 +1160,23 @@ size_t rglru_hip_conv_scratch_bytes(int64_t B, int64_t T, int64_t W, int64_t K) 
 }
 
 int rglru_hip_conv_bwd(const void* u, const void* state, const void* taps, const int64_t* segment_pos,
-                       const void* dout, void* scratch, void* du, void* dstate, void* dtaps, void* dbias,
+                       const void* dout, void* scratch, void* du, int64_t du_stride, void* dstate, void* dtaps, void* dbias,
                        int64_t B, int64_t T, int64_t W, int64_t K, int dtype, int vec_dtype, int grad_dtype,
                        void* stream) {
   int rc = conv_check("conv_bwd", B, T, W, K, dtype, vec_dtype);
+  if (rc) return rc;
+  if (du_stride == 0) du_stride = W;
+  if (du_stride < W) return fail(RGLRU_E_ARG, "conv_bwd: du_stride %lld is smaller than the width %lld", (long long)du_stride, (long long)W);
+  rc = conv_check("conv_bwd", B, T, du_stride, K, dtype, vec_dtype);      // the strided rows obey the same per-sequence limit
   if (rc) return rc;
   if (grad_dtype != RGLRU_F32 && grad_dtype != RGLRU_BF16) return fail(RGLRU_E_ARG, "conv_bwd: unknown gradient dtype %d", grad_dtype);
   if (!u || !taps || !segment_pos || !dout || !scratch || !du) return fail(RGLRU_E_ARG, "conv_bwd: null pointer");
   ConvArgs a;
   memset(&a, 0, sizeof(a));
   a.u = u; a.state = state; a.taps = taps; a.segpos = (const long long*)segment_pos;
-  a.dout = dout; a.du = du; a.dstate = dstate; a.partial = (float*)scratch;
+  a.dout = dout; a.du = du; a.dstate = dstate; a.partial = (float*)scratch; a.ld_du = du_stride;
   a.B = (int)B; a.T = (int)T; a.W = (int)W; a.K = (int)K; a.vec_dtype = vec_dtype;
-  const bool vec = conv_vector_ok(W, dtype, {u, state, dout, du, dstate});
+  const bool vec = conv_vector_ok(W, dtype, {u, state, dout, du, dstate}) && (du_stride * (dtype == RGLRU_BF16 ? 2 : 4)) % 16 == 0;
   a.nvec = (int)(vec ? W / (dtype == RGLRU_BF16 ? 8 : 4) : W);
   a.runs = (int)((T + kConvRunBwd - 1) / kConvRunBwd);
   const long long run_groups = (a.runs + kConvBwdRuns - 1) / kConvBwdRuns;
@@ -1249,11 +1268,25 @@ int rglru_hip_gelu_gate_fwd(const void* h, const void* v, void* out, int64_t n, 
 }
 
 int rglru_hip_gelu_gate_bwd(const void* dout, const void* h, const void* v, void* dh, void* dv,
-                            int64_t n, int dtype, void* stream) {
+                            int64_t n, int64_t W, int64_t dv_stride, int dtype, void* stream) {
   if (!dout || !h || !v || !dh || !dv) return fail(RGLRU_E_ARG, "gelu_gate_bwd: null pointer");
   GateArgs a;
   memset(&a, 0, sizeof(a));
   a.h = h; a.v = v; a.dout = dout; a.dh = dh; a.dv = dv; a.n = n;
+  if (dv_stride != 0 && dv_stride != W) {
+    if (dtype != RGLRU_F32 && dtype != RGLRU_BF16) return fail(RGLRU_E_ARG, "gelu_gate_bwd: dtype must be RGLRU_F32 or RGLRU_BF16, got %d", dtype);
+    if (W <= 0 || n <= 0 || n % W || dv_stride < W) return fail(RGLRU_E_ARG, "gelu_gate_bwd: n = %lld is not rows of W = %lld elements, or dv_stride %lld < W", (long long)n, (long long)W, (long long)dv_stride);
+    const int64_t es = dtype == RGLRU_BF16 ? 2 : 4, rows = n / W;
+    if (rows * dv_stride * es >= (1ll << 31) || n * es > (1ll << 30)) return fail(RGLRU_E_UNSUPPORTED, "gelu_gate_bwd: a strided dv must stay below 2 GiB");
+    const int vlen = dtype == RGLRU_BF16 ? 8 : 4;
+    const bool vec = conv_vector_ok(n, dtype, {h, v, dout, dh, dv}) && W % vlen == 0 && (dv_stride * es) % 16 == 0;
+    // rows of 16-byte vectors, or single elements: the launch below takes the vector kernel exactly when `vec` holds
+    if (!vec && conv_vector_ok(n, dtype, {h, v, dout, dh, dv})) return fail(RGLRU_E_UNSUPPORTED, "gelu_gate_bwd: a strided dv needs W and dv_stride in whole 16-byte vectors");
+    a.ld_dv = dv_stride; a.row_vecs = (int)(vec ? W / vlen : W);
+    a.dv_bytes = (unsigned)(((rows - 1) * dv_stride + W) * es);
+    const long long vectors = rows * a.row_vecs;
+    if (a.row_vecs > 1 && (vectors + a.row_vecs) * a.row_vecs < (1ll << 32)) a.row_magic = (unsigned)(((1ull << 32) + a.row_vecs - 1) / a.row_vecs);
+  }
   return gate_launch("gelu_gate_bwd", true, a, dtype, stream);
 }
 

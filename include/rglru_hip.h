@@ -50,7 +50,7 @@
 extern "C" {
 #endif
 
-#define RGLRU_ABI_VERSION 17
+#define RGLRU_ABI_VERSION 18
 
 enum { RGLRU_F32 = 0, RGLRU_BF16 = 1 };
 
@@ -258,11 +258,14 @@ int rglru_hip_conv_fwd(const void* u, const void* state, const void* taps, const
 
 /* Reverse mode of rglru_hip_conv_fwd.  dout[B,T,W] (dtype) is the gradient at `out`.  Writes
  * du[B,T,W] and, when not NULL, dstate[B,K-1,W] (dtype), dtaps[W,K] and dbias[W] (grad_dtype).
+ * du_stride is the distance between rows of du in elements (0 or W: contiguous; larger: du is a
+ * column range of a wider [B*T, du_stride] matrix, e.g. the left half of the stacked gradient of
+ * two projections that one GEMM then consumes).
  * `scratch` holds rglru_hip_conv_scratch_bytes(B, T, W, K) bytes of per-run partial sums; its
  * contents on entry do not matter. */
 size_t rglru_hip_conv_scratch_bytes(int64_t B, int64_t T, int64_t W, int64_t K);
 int rglru_hip_conv_bwd(const void* u, const void* state, const void* taps, const int64_t* segment_pos,
-                       const void* dout, void* scratch, void* du, void* dstate, void* dtaps, void* dbias,
+                       const void* dout, void* scratch, void* du, int64_t du_stride, void* dstate, void* dtaps, void* dbias,
                        int64_t B, int64_t T, int64_t W, int64_t K, int dtype, int vec_dtype, int grad_dtype,
                        void* stream);
 
@@ -290,10 +293,12 @@ int rglru_hip_conv_padded_bwd(const void* u, const void* state, const void* taps
 /* Output gate of the recurrent block, out = h * gelu_tanh(v) (griffin/griffin.py:464 and :520: the
  * GeLU of the second branch and the product with the RG-LRU output in one pass), flat over n
  * elements of `dtype`; and its reverse mode: dh = dout * gelu_tanh(v), dv = dout * h * gelu_tanh'(v).
- * Arithmetic in fp32. */
+ * The reverse mode can write dv as rows of W elements that lie dv_stride elements apart (n a multiple
+ * of W; a column range of a wider matrix, as for du of rglru_hip_conv_bwd); dv_stride 0 or W: flat like
+ * the other tensors, W is then not used.  Arithmetic in fp32. */
 int rglru_hip_gelu_gate_fwd(const void* h, const void* v, void* out, int64_t n, int dtype, void* stream);
 int rglru_hip_gelu_gate_bwd(const void* dout, const void* h, const void* v, void* dh, void* dv,
-                            int64_t n, int dtype, void* stream);
+                            int64_t n, int64_t W, int64_t dv_stride, int dtype, void* stream);
 
 /* RMSNorm in front of the block (griffin/griffin.py:68-80), over the last axis of x[rows, D]:
  *   y = x * rsqrt(mean(x^2) + eps) * (1 + g),   g[D] read in vec_dtype;

@@ -433,6 +433,92 @@ def test_hip_linear_pair_matches_two_linear_layers(shape, dtype, used):
         assert err < tol, name
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(2, 50, 64, 3), (3, 37, 13, 4), (1, 1, 8, 2), (8, 2048, 1024, 4)])
+def test_strided_gradient_outputs_equal_the_contiguous_ones(shape, dtype):
+    """rglru_hip_conv_bwd with du_stride and rglru_hip_gelu_gate_bwd with dv_stride (C ABI): du and dv written as the
+    column halves of one [B, T, 2 W + pad] matrix are bit for bit what the contiguous calls write, nothing else of
+    that matrix is touched, and the other outputs do not change."""
+    from griffin_amd import _lib
+    from griffin_amd.hip_block_ops import _DTYPE_CODES, _dtype_code, _ptr, _stream_ptr
+
+    B, T, W, K = shape
+    _say("strided gradient outputs case", shape, dtype)
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(35)
+    rnd = lambda *s: torch.randn(*s, generator=g).to(dtype).cuda()
+    u, dout, h, v, dgate = rnd(B, T, W), rnd(B, T, W), rnd(B, T, W), rnd(B, T, W) * 2, rnd(B, T, W)
+    taps = (torch.randn(W, K, generator=g) * 0.4).to(dtype).cuda()
+    pos = torch.arange(T).repeat(B, 1).cuda()
+    pos[:, T // 2:] -= T // 2                                 # a document start in the middle of every row
+    code, stream = _dtype_code(dtype), _stream_ptr(u.device)
+    pad = 8 if W % 8 == 0 else 3                              # rows of whole 16-byte vectors where W allows the vector kernels
+    ld = 2 * W + pad
+
+    def conv_bwd(du):
+        scratch = torch.empty(lib.rglru_hip_conv_scratch_bytes(B, T, W, K), dtype=torch.uint8, device="cuda")
+        dtaps = torch.empty(W, K, dtype=dtype, device="cuda")
+        dbias = torch.empty(W, dtype=dtype, device="cuda")
+        _lib.check(lib.rglru_hip_conv_bwd(_ptr(u), None, _ptr(taps), _ptr(pos), _ptr(dout), _ptr(scratch), _ptr(du), du.stride(1),
+                                          None, _ptr(dtaps), _ptr(dbias), B, T, W, K, code, _DTYPE_CODES[dtype], _DTYPE_CODES[dtype],
+                                          stream), "rglru_hip_conv_bwd")
+        return dtaps, dbias
+
+    def gate_bwd(dv):
+        dh = torch.empty_like(h)
+        _lib.check(lib.rglru_hip_gelu_gate_bwd(_ptr(dgate), _ptr(h), _ptr(v), _ptr(dh), _ptr(dv), h.numel(), W, dv.stride(1),
+                                               code, stream), "rglru_hip_gelu_gate_bwd")
+        return dh
+
+    du_c, dv_c = torch.empty_like(u), torch.empty_like(v)
+    want_conv, want_dh = conv_bwd(du_c), gate_bwd(dv_c)
+    both = torch.full((B, T, ld), 7.0, dtype=dtype, device="cuda")
+    got_conv, got_dh = conv_bwd(both[..., :W]), gate_bwd(both[..., W:2 * W])
+    torch.cuda.synchronize()
+    assert torch.equal(both[..., :W], du_c)
+    assert torch.equal(both[..., W:2 * W], dv_c)
+    assert torch.all(both[..., 2 * W:] == 7.0)
+    assert torch.equal(got_dh, want_dh)
+    for a, b in zip(got_conv, want_conv):
+        assert torch.equal(a, b)
+    # a stride below the width is an error, not a memory fault
+    with pytest.raises(ValueError):
+        _lib.check(lib.rglru_hip_gelu_gate_bwd(_ptr(dgate), _ptr(h), _ptr(v), _ptr(torch.empty_like(h)), _ptr(dv_c), h.numel(), W, W - 1,
+                                               code, stream), "rglru_hip_gelu_gate_bwd")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(2, 50, 64, 96), (3, 7, 13, 5), (8, 2048, 768, 1024)])
+def test_hip_linear_pair_with_stacked_gradients(shape, dtype):
+    """The pair's backward when its two incoming gradients are the column halves of one matrix (what the
+    one-launch block forward's backward hands it): one GEMM for dx, one for both weight gradients, one column
+    sum -- against two torch.nn.functional.linear calls in fp64."""
+    from griffin_amd.hip_block_ops import _stacked_halves, hip_linear_pair
+
+    B, T, D, W = shape
+    _say("linear pair, stacked gradients, case", shape, dtype)
+    gen = torch.Generator().manual_seed(36)
+    x = torch.randn(B, T, D, generator=gen).to(dtype)
+    ws = [(torch.randn(W, D, generator=gen) / D ** 0.5).to(dtype) for _ in range(2)]
+    bs = [(torch.randn(W, generator=gen) * 0.1).to(dtype) for _ in range(2)]
+    both = torch.randn(B, T, 2 * W, generator=gen).to(dtype)
+    ref = [t.double().requires_grad_(True) for t in (x, ws[0], bs[0], ws[1], bs[1])]
+    outs = (torch.nn.functional.linear(ref[0], ref[1], ref[2]), torch.nn.functional.linear(ref[0], ref[3], ref[4]))
+    torch.autograd.backward(outs, [both[..., :W].double(), both[..., W:].double()])
+    dev = [t.cuda().requires_grad_(True) for t in (x, ws[0], bs[0], ws[1], bs[1])]
+    got = hip_linear_pair(*dev)
+    both_d = both.cuda()
+    halves = [both_d[..., :W], both_d[..., W:]]
+    assert _stacked_halves(*halves) is not None
+    torch.autograd.backward(got, halves)
+    torch.cuda.synchronize()
+    tol = 2e-5 if dtype == torch.float32 else BF16_TOL
+    for name, r, d in zip(("x", "w1", "b1", "w2", "b2"), ref, dev):
+        err = rel_err(d.grad.double().cpu(), r.grad)
+        _say("  d%s rel error: %.2e" % (name, err))
+        assert err < tol, name
+
+
 # ----------------------------------------------------------------------------------------------
 # convolution + RG-LRU + output gate in one forward launch (rglru_hip_block_fwd), griffin/griffin.py:464-520
 # ----------------------------------------------------------------------------------------------

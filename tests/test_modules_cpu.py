@@ -354,3 +354,27 @@ def test_caches_are_dropped_by_invalidate_and_module_state_changes():
             assert block._stacked_projection is not None
             change()
             assert block._stacked_projection is None and block.rg_lru._prep is None
+
+
+def test_stacked_halves_are_recognised_only_when_they_are_one_matrix():
+    """hip_block_ops._stacked_halves: the two gradients the block's backward writes side by side are found again
+    as one [rows, 2 W] matrix; anything else (separate tensors, swapped halves, a gap, other strides) is not."""
+    from griffin_amd.hip_block_ops import _stacked_halves
+
+    both = torch.arange(2 * 3 * 8, dtype=torch.float32).view(2, 3, 8)
+    left, right = both[..., :4], both[..., 4:]
+    got = _stacked_halves(left, right)
+    assert got is not None and got.shape == (6, 8) and torch.equal(got, both.view(6, 8))
+    assert got.data_ptr() == both.data_ptr()
+    assert _stacked_halves(right, left) is None
+    assert _stacked_halves(left, None) is None
+    assert _stacked_halves(left.contiguous(), right.contiguous()) is None
+    assert _stacked_halves(left, right.clone()) is None
+    wide = torch.zeros(2, 3, 10)
+    assert _stacked_halves(wide[..., :4], wide[..., 4:8]) is None          # rows are 10 apart, not 8
+    assert _stacked_halves(both[:, ::2, :4], both[:, ::2, 4:]) is None    # every other row
+    one_row = torch.zeros(1, 1, 8)
+    assert _stacked_halves(one_row[..., :4], one_row[..., 4:]).shape == (1, 8)
+    offset = torch.zeros(5 + 2 * 3 * 8)[5:].view(2, 3, 8)                 # a storage offset carries over
+    got = _stacked_halves(offset[..., :4], offset[..., 4:])
+    assert got is not None and got.storage_offset() == 5
