@@ -301,16 +301,25 @@ RGLRU_DEVICE void gate_tile_generic(const FusedArgs& p, const IO* xmat, long lon
   }
 }
 
-// Register-resident weights: the wave's 32 rows of both gate matrices, NKG K groups each.
-template <typename IO, int NKG>
+// Register-resident weights: the wave's 32 rows of both gate matrices, NKG K groups each.  The last LDSG K
+// groups can live in LDS instead (`spill`: [group][gate][lane] fragments private to the wave): where the registers
+// run out, the compiler's own spill goes to scratch memory, whose reloads count as vector memory operations and
+// make the wave wait for every load it has in flight.
+template <typename IO, int NKG, int LDSG = 0>
 struct HeldWeights {
-  typename Io<IO>::Frag a[NKG > 0 ? NKG : 1], x[NKG > 0 ? NKG : 1];
-  RGLRU_DEVICE void load(const IO* w_a_row, const IO* w_x_row) {
+  static constexpr int kRegs = NKG > 0 ? NKG - LDSG : 1;
+  typename Io<IO>::Frag a[kRegs], x[kRegs];
+  RGLRU_DEVICE void load(const IO* w_a_row, const IO* w_x_row, typename Io<IO>::Frag* spill = nullptr, int lane = 0) {
     if constexpr (NKG > 0) {
 #pragma unroll
-      for (int kg = 0; kg < NKG; ++kg) {
+      for (int kg = 0; kg < NKG - LDSG; ++kg) {
         a[kg] = *reinterpret_cast<const typename Io<IO>::Frag*>(w_a_row + kg * Io<IO>::KG);
         x[kg] = *reinterpret_cast<const typename Io<IO>::Frag*>(w_x_row + kg * Io<IO>::KG);
+      }
+#pragma unroll
+      for (int g = 0; g < LDSG; ++g) {
+        spill[(2 * g) * 64 + lane] = *reinterpret_cast<const typename Io<IO>::Frag*>(w_a_row + (NKG - LDSG + g) * Io<IO>::KG);
+        spill[(2 * g + 1) * 64 + lane] = *reinterpret_cast<const typename Io<IO>::Frag*>(w_x_row + (NKG - LDSG + g) * Io<IO>::KG);
       }
     }
   }
@@ -319,9 +328,10 @@ struct HeldWeights {
 // MFMA phase for register-held weights, one accumulator tile: the whole block width (NKG * KG
 // columns) is in LDS with row stride NKG * KG + HW.  Also returns the 16 x values of the tile in
 // accumulator layout.
-template <typename IO, int MT, int NKG, int TW = NKG * Io<IO>::KG>
-RGLRU_DEVICE void gate_mfma_held(const IO* lds, const HeldWeights<IO, NKG>& hw, int mt, int slab, int r, int hf,
-                                 float bias_a, float bias_x, f32x16& ua, f32x16& ux, float (&xv)[16], int kb = 0) {
+template <typename IO, int MT, int NKG, int TW = NKG * Io<IO>::KG, int LDSG = 0>
+RGLRU_DEVICE void gate_mfma_held(const IO* lds, const HeldWeights<IO, NKG, LDSG>& hw, int mt, int slab, int r, int hf,
+                                 float bias_a, float bias_x, f32x16& ua, f32x16& ux, float (&xv)[16], int kb = 0,
+                                 const typename Io<IO>::Frag* spill = nullptr, int lane = 0) {
   typedef Io<IO> Tr;
   typedef typename Tr::Frag Frag;
   constexpr int KG = Tr::KG, HW = Tr::HW;
@@ -330,10 +340,16 @@ RGLRU_DEVICE void gate_mfma_held(const IO* lds, const HeldWeights<IO, NKG>& hw, 
   for (int v = 0; v < 16; ++v) { ua[v] = bias_a; ux[v] = bias_x; }
   const IO* row = lds + tile_row<MT>(mt, r) * LDSROW + kb + hf * HW;
 #pragma unroll
-  for (int kg = 0; kg < NKG; ++kg) {
+  for (int kg = 0; kg < NKG - LDSG; ++kg) {
     Frag xa = *reinterpret_cast<const Frag*>(row + kg * KG);
     Tr::mma(ua, xa, hw.a[kg]);
     Tr::mma(ux, xa, hw.x[kg]);
+  }
+#pragma unroll
+  for (int g = 0; g < LDSG; ++g) {
+    Frag xa = *reinterpret_cast<const Frag*>(row + (NKG - LDSG + g) * KG);
+    Tr::mma(ua, xa, spill[(2 * g) * 64 + lane]);
+    Tr::mma(ux, xa, spill[(2 * g + 1) * 64 + lane]);
   }
 #pragma unroll
   for (int e = 0; e < 16; ++e) xv[e] = (float)lds[(hf * 16 * MT + 16 * mt + e) * LDSROW + kb + slab * 32 + r];

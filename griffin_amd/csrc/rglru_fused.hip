@@ -176,6 +176,14 @@ constexpr int kFwdMT = 2;
 //   workgroups (320: 14 spilled registers); 256, 352, 384 are fastest as they were.
 constexpr int fwd_mt(int nkg) { return (nkg == 18 || nkg == 20) ? 1 : kFwdMT; }
 constexpr int fwd_wide_occ(int nkg) { return (nkg == 16 || nkg > 20) ? 1 : 2; }
+// K groups of the weights that a wave keeps in LDS instead of registers (HeldWeights) where two workgroups a
+// compute unit leave too few registers.  The compiler's own spill goes to scratch memory: its reloads sit at the top of
+// the gate products and wait for every vector memory operation in flight, the record prefetch of the look-back
+// included.  Chosen so that nothing spills (224-wide masked: 4 registers still do) and two workgroups still fit the
+// LDS (8 KB per group and workgroup).  Forward at B1 T32768, us: 224-wide 163 -> 158, 320-wide 314 -> 292.
+constexpr int fwd_lds_groups(int nkg, bool masked) {
+  return nkg == 14 ? (masked ? 4 : 3) : nkg == 18 ? (masked ? 5 : 0) : nkg == 20 ? (masked ? 6 : 4) : 0;
+}
 
 // workgroups per compute unit of the forward kernel without weights in registers (NKG < 0); 4 spills
 #define RGLRU_GIVEN_OCC 3
@@ -241,8 +249,14 @@ __global__ __launch_bounds__(kThreads, (BLOCK ? 2 : NKG < 0 ? RGLRU_GIVEN_OCC : 
   if constexpr (NKG != 0) {
     // software-pipelined loop: the next ticket is taken while the current tile's MFMAs run and the
     // next x tile is requested right before the wave starts waiting for its carry
-    HeldWeights<IO, NKG> hw;
-    hw.load(w_a_row, w_x_row);
+    constexpr int LDSG = NKG > 0 ? fwd_lds_groups(NKG, MASKED) : 0;
+    Frag* spill = nullptr;
+    if constexpr (LDSG > 0) {
+      __shared__ __attribute__((aligned(16))) Frag lds_hw[kWaves * 2 * LDSG * 64];
+      spill = lds_hw + w.wave * (2 * LDSG * 64);
+    }
+    HeldWeights<IO, NKG, LDSG> hw;
+    hw.load(w_a_row, w_x_row, spill, w.lane);
     constexpr int VPR = KC / Tr::HW;                     // 16-byte vectors per tile row
     constexpr int NV = (TR * VPR + kThreads - 1) / kThreads;
     Frag pre[NV], pre_a[GIVEN ? NV : 1], pre_x[GIVEN ? NV : 1];
@@ -442,7 +456,7 @@ __global__ __launch_bounds__(kThreads, (BLOCK ? 2 : NKG < 0 ? RGLRU_GIVEN_OCC : 
               ux[e] = (float)lds_pre[TR * LDSROW + at];
             }
           } else
-          gate_mfma_held<IO, MT, NKG, KC>(lds, hw, mt, w.slab, w.r, hf, 0.0f, 0.0f, ua, ux, xv, NKG >= 8 ? 0 : w.kb);
+          gate_mfma_held<IO, MT, NKG, KC, LDSG>(lds, hw, mt, w.slab, w.r, hf, 0.0f, 0.0f, ua, ux, xv, NKG >= 8 ? 0 : w.kb, spill, w.lane);
           fwd_gates<IO, MASKED>(flbits[mt], ua, ux, xv, sp, cur.a + 16 * mt, cur.z + 16 * mt, nba, nbx,
                                 p.first_reset && mt == 0 && cur.c == 0 && hf == 0);
         }
