@@ -194,9 +194,12 @@ constexpr int kPackedWidth = 128;
 // Waves of a chain kernel's workgroup (fwd_chain_kernel, bwd_delta_chain_kernel: one workgroup per chain).
 constexpr int kChainWaves = 16;
 
-RGLRU_DEVICE WaveId wave_identity(const FusedArgs& p, int block) {
+RGLRU_DEVICE WaveId wave_identity(const FusedArgs& p, int block, bool scalar_wave = false) {
   WaveId w;
-  w.lane = threadIdx.x & 63; w.r = w.lane & 31; w.hf = w.lane >> 5; w.wave = threadIdx.x >> 6;
+  w.lane = threadIdx.x & 63; w.r = w.lane & 31; w.hf = w.lane >> 5;
+  // scalar_wave: the wave index is made known to be wave-uniform, so what derives from it (slab, block, buffer
+  // descriptors) stays in scalar registers; where registers are short that costs more than it saves
+  w.wave = scalar_wave ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : (int)(threadIdx.x >> 6);
   w.unit = block % p.units; w.wg_in_unit = block / p.units;
   if (p.xcd_map) {
     // Workgroups go to the eight XCDs round-robin by index and each XCD has its own L2.  The `groups` units

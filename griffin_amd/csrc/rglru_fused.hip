@@ -217,7 +217,7 @@ __global__ __launch_bounds__(kThreads, (BLOCK ? 2 : NKG < 0 ? RGLRU_GIVEN_OCC : 
   __shared__ unsigned s_ticket[2];
   __shared__ __attribute__((aligned(16))) float conv_w[BLOCK ? 5 * KC : 4];    // taps of lag 0..3, then the bias
 
-  const WaveId w = wave_identity(p, blockIdx.x);
+  const WaveId w = wave_identity(p, blockIdx.x, NKG > 8);
   if (w.wg_in_unit >= p.wg_per_unit) return;             // only with xcd_map: the grid's last round is not full
   const int hf = w.hf, tid = threadIdx.x;
   unsigned char* stage = stage_all + w.wave * WaveStage<TR>::kBytes;
