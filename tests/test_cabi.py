@@ -32,6 +32,15 @@ def test_header_and_binding_agree():
     assert _declared_symbols() == sorted(_lib.EXPORTED_SYMBOLS)
 
 
+def test_build_compiles_every_kernel_source():
+    """Every .hip file under griffin_amd/csrc is part of the library (a new translation unit that the build
+    list misses would compile nowhere and its entry points would be undefined at load time)."""
+    from griffin_amd import build
+
+    present = sorted(f for f in os.listdir(build.CSRC) if f.endswith(".hip"))
+    assert sorted(build.SOURCES) == present
+
+
 def test_library_exports_every_declared_symbol(lib):
     raw = ctypes.CDLL(_lib.LIB_PATH)
     for name in _declared_symbols():
