@@ -670,3 +670,141 @@ def test_decode_row_stride_below_width_is_rejected():
     p = buf.data_ptr()
     rc = lib.rglru_hip_decode_prepare(p, 16, None, p, None, None, None, None, p, p, p, p, 2, 32, 4, 0, 0, None)
     assert rc != 0 and b"stride" in lib.rglru_hip_last_error()
+
+
+# ----------------------------------------------------------------------------------------------
+# random sweeps of the block: the HIP kernels against the same block on the CPU, driven the same way
+# ----------------------------------------------------------------------------------------------
+def _random_block_pair(rng, dtype, widths, dims):
+    """A RecurrentBlock with random geometry on the CPU (fp32 values rounded to `dtype`) and its copy on the HIP path."""
+    from griffin_amd import RecurrentBlock
+
+    bw = rng.choice(widths)
+    nb = rng.choice([1, 2, 4, 8])
+    if bw * nb > 1280:
+        nb = max(1, 1280 // bw)
+    W, D, K = bw * nb, rng.choice(dims), rng.choice([4, 4, 4, 2, 3])
+    ref = RecurrentBlock(D, W, gate_blocks=nb, conv_kernel_size=K, scan_mode="sequential")
+    with torch.no_grad():
+        ref.rg_lru.recurrence_gate.bias.copy_(0.3 * torch.randn_like(ref.rg_lru.recurrence_gate.bias))
+        ref.rg_lru.input_gate.bias.copy_(0.3 * torch.randn_like(ref.rg_lru.input_gate.bias))
+    ref = ref.to(dtype).float()
+    hip = copy.deepcopy(ref).to(dtype).cuda()
+    hip.scan_mode = None
+    hip.rg_lru.scan_mode = "hip"
+    return ref, hip, (D, W, nb, K)
+
+
+def test_random_blocks_train_like_the_cpu_block():
+    """Forty random blocks (fixed seed): storage type, gate block width and count, model width, convolution size,
+    batch, length; plain, packed documents, right padding, both, or two calls chained through the cache.  Output,
+    cache and every gradient against the block on the CPU with the sequential scan."""
+    import random
+
+    rng = random.Random(11)
+    failures = []
+    for index in range(40):
+        torch.manual_seed(1100 + index)
+        dtype = rng.choice([torch.float32, torch.bfloat16, torch.bfloat16])
+        ref, hip, (D, W, nb, K) = _random_block_pair(rng, dtype, [8, 16, 24, 32, 64, 96, 128, 160, 320], [32, 48, 96, 256, 768])
+        B = rng.choice([1, 2, 3, 8])
+        T = rng.choice([1, 2, 3, 4, 5, 17, 32, 33, 64, 100, 255, 256, 600, 1024])
+        if B * T * W > 1500000:
+            T = max(1, 1500000 // (B * W))
+        kind = rng.choice(["plain", "packed", "padded", "both", "chunked"])
+        _say("random block", index, str(dtype), (B, T, D, W, nb, K), kind)
+        x = torch.randn(B, T, D).to(dtype).float()
+        up = torch.randn(B, T, D).to(dtype).float()
+        kw = {}
+        if kind in ("packed", "both"):
+            pos = torch.arange(T).repeat(B, 1)
+            for b in range(B):
+                if T > 2 and rng.random() < 0.7:
+                    cut = rng.randrange(1, T)
+                    pos[b, cut:] -= cut
+            kw["segment_pos"] = pos
+        if kind in ("padded", "both"):
+            lens = torch.tensor([rng.choice([T, T, max(0, T - 1), T // 2, 0]) for _ in range(B)])
+            kw["active_mask"] = torch.arange(T)[None, :] < lens[:, None]
+        xc = x.clone().requires_grad_(True)
+        xh = x.to(dtype).cuda().requires_grad_(True)
+        if kind == "chunked" and T >= 2:
+            cut = rng.randrange(1, T)
+            y1, cache_c = ref(xc[:, :cut], return_cache=True)
+            y2, cache_c = ref(xc[:, cut:], cache_c, return_cache=True)
+            yc = torch.cat([y1, y2], 1)
+            z1, cache_h = hip(xh[:, :cut], return_cache=True)
+            z2, cache_h = hip(xh[:, cut:], cache_h, return_cache=True)
+            yh = torch.cat([z1, z2], 1)
+        else:
+            yc, cache_c = ref(xc, return_cache=True, **kw)
+            yh, cache_h = hip(xh, return_cache=True, **{k: v.cuda() for k, v in kw.items()})
+        yc.backward(up)
+        yh.backward(up.to(dtype).cuda())
+        torch.cuda.synchronize()
+        errs = {"y": rel_err(yh.float(), yc), "dx": rel_err(xh.grad.float(), xc.grad),
+                "rnn_state": rel_err(cache_h.rnn_state.float(), cache_c.rnn_state),
+                "conv_state": rel_err(cache_h.conv_state.float(), cache_c.conv_state),
+                "position": 0.0 if torch.equal(cache_h.segment_position.cpu(), cache_c.segment_position) else 1.0}
+        for (name, ph), (_, pc) in zip(hip.named_parameters(), ref.named_parameters()):
+            errs[name] = rel_err(ph.grad.float(), pc.grad)
+        tol = 2e-4 if dtype == torch.float32 else BF16_TOL
+        if not max(errs.values()) < tol:
+            failures.append((index, kind, {k: "%.2e" % v for k, v in errs.items() if not v < tol}))
+    assert not failures, failures
+
+
+def test_random_prefill_and_decode_like_the_cpu_block():
+    """Forty random prefill + single-token decode runs (fixed seed) with document restarts and rows that stop,
+    against the CPU block called with the same slices.  The same call pattern matters: the reference's all-active
+    convolution keeps a finished document's rows in the cache (griffin/griffin.py:487) and its padded one uses the
+    whole window (:496-500), so step-by-step calls and one pass over the sequence differ there by design."""
+    import random
+
+    rng = random.Random(12)
+    failures = []
+    for index in range(40):
+        torch.manual_seed(1200 + index)
+        dtype = rng.choice([torch.float32, torch.bfloat16, torch.bfloat16])
+        ref, hip, (D, W, nb, K) = _random_block_pair(rng, dtype, [8, 16, 24, 32, 40, 64, 96, 128, 160, 320, 384], [32, 48, 96, 256])
+        ref, hip = ref.eval(), hip.eval()
+        B = rng.choice([1, 2, 3, 16, 17, 64, 100, 256])
+        T0, S = rng.choice([0, 1, 2, 3, 5, 40]), rng.choice([1, 2, 5, 12])
+        T = T0 + S
+        kind = rng.choice(["plain", "restart", "padded", "both"])
+        _say("random decode", index, str(dtype), (B, T0, S, D, W, nb, K), kind)
+        x = torch.randn(B, T, D).to(dtype).float()
+        kw = {}
+        active = torch.ones(B, T, dtype=torch.bool)
+        if kind in ("restart", "both"):
+            pos = torch.arange(T).repeat(B, 1)
+            for b in range(B):
+                if T > 1 and rng.random() < 0.5:
+                    cut = rng.randrange(max(T0, 1) if T0 < T else T - 1, T)
+                    pos[b, cut:] -= cut
+            kw["segment_pos"] = pos
+        if kind in ("padded", "both"):
+            for b in range(B):
+                if rng.random() < 0.4:
+                    active[b, rng.randrange(T0, T + 1):] = False
+            kw["active_mask"] = active
+        cuts = ([(0, T0)] if T0 else []) + [(t, t + 1) for t in range(T0, T)]
+        with torch.no_grad():
+            cache_c = cache_h = None
+            outs_c, outs_h = [], []
+            xh = x.to(dtype).cuda()
+            for lo, hi in cuts:
+                yc, cache_c = ref(x[:, lo:hi], cache_c, return_cache=True, **{k: v[:, lo:hi] for k, v in kw.items()})
+                yh, cache_h = hip(xh[:, lo:hi], cache_h, return_cache=True, **{k: v[:, lo:hi].cuda() for k, v in kw.items()})
+                outs_c.append(yc)
+                outs_h.append(yh)
+        torch.cuda.synchronize()
+        live = active[..., None]
+        errs = {"y": rel_err(torch.cat(outs_h, 1).float().cpu() * live, torch.cat(outs_c, 1) * live),
+                "rnn_state": rel_err(cache_h.rnn_state.float(), cache_c.rnn_state),
+                "conv_state": rel_err(cache_h.conv_state.float(), cache_c.conv_state),
+                "position": 0.0 if torch.equal(cache_h.segment_position.cpu(), cache_c.segment_position) else 1.0}
+        tol = 2e-4 if dtype == torch.float32 else BF16_TOL
+        if not max(errs.values()) < tol:
+            failures.append((index, kind, {k: "%.2e" % v for k, v in errs.items() if not v < tol}))
+    assert not failures, failures
