@@ -36,8 +36,18 @@ struct ConvArgs {
   void* out; void* new_state;                               // forward
   const void* dout; void* du; void* dstate; float* partial;  // backward
   long long ld_du;                                          // elements between rows of du (>= W)
+  // Right-padded batches whose active tokens are a prefix of the row run on these kernels too: rows[b] = number of
+  // active tokens, rows[2 * B + b] != 0 where the row is such a prefix (the others are left to the kernels for
+  // arbitrary masks).  Null: every row has T tokens.
+  const int* rows;
   int B, T, W, K, nvec, runs, vec_dtype;
 };
+
+// Tokens of row b these kernels work on (inputs past them read as zero), or -1 where the row is not theirs.
+RGLRU_DEVICE int conv_row_tokens(const ConvArgs& p, int b) {
+  if (!p.rows) return p.T;
+  return p.rows[2 * p.B + b] ? p.rows[b] : -1;
+}
 
 // V values of one row.  `Raw` is the row as loaded (requests are issued in batches before any of
 // them is used); unpack turns it into floats.
@@ -194,11 +204,13 @@ __global__ __launch_bounds__(kConvThreads) void conv_fwd_kernel(ConvArgs p) {
   const ConvItem it = conv_item(p);
   if (!it.ok) return;
   const int b = it.b, c0 = it.c0, t0 = it.run * kConvRunFwd;
+  const int n = conv_row_tokens(p, b);
+  if (n < 0) return;
   const unsigned es = (unsigned)sizeof(IO), uW = (unsigned)p.W;
   float tap[K][V], bias[V];
   conv_load_taps<V, K>(p.taps, p.bias, c0, p.vec_dtype, tap, bias);
   const unsigned seq_bytes = (unsigned)p.T * uW * es;
-  const rsrc_t ru = make_rsrc((const IO*)p.u + (long long)b * p.T * p.W, seq_bytes);
+  const rsrc_t ru = make_rsrc((const IO*)p.u + (long long)b * p.T * p.W, (unsigned)n * uW * es);
   const rsrc_t ro = make_rsrc((const IO*)p.out + (long long)b * p.T * p.W, seq_bytes);
   const rsrc_t rs = conv_state_rsrc<IO, K>(p, b);
   const long long* sp_row = p.segpos + (long long)b * p.T;
@@ -229,7 +241,7 @@ __global__ __launch_bounds__(kConvThreads) void conv_fwd_kernel(ConvArgs p) {
 #pragma unroll
       for (int lag = 1; lag < K; ++lag)
         if (sp >= lag) a = fmaf(win[lag - 1][v], tap[K - 1 - lag][v], a);
-      acc[v] = a;
+      acc[v] = t < n ? a : 0.f;                            // padding behind the row's tokens
     }
     ConvRow<IO, V>::store(acc, ro, off);
 #pragma unroll
@@ -275,7 +287,9 @@ __global__ __launch_bounds__(kConvThreads) void conv_bwd_kernel(ConvArgs p) {
   conv_load_taps<V, K>(p.taps, nullptr, c0, p.vec_dtype, tap, bias_unused);
   // The descriptors are the same in all lanes.  A thread without work addresses past their end:
   // its loads return zero and its stores are dropped.
-  const unsigned seq_bytes = (unsigned)p.T * uW * es;
+  const int n = conv_row_tokens(p, b);
+  if (n < 0) return;                                       // the whole workgroup: it lies inside one sequence
+  const unsigned seq_bytes = (unsigned)n * uW * es;        // the gradient of a padded output is not read: it counts as zero
   const rsrc_t ru = make_rsrc((const IO*)p.u + (long long)b * p.T * p.W, seq_bytes);
   const rsrc_t rd = make_rsrc((const IO*)p.dout + (long long)b * p.T * p.W, seq_bytes);
   const unsigned ld_du = (unsigned)p.ld_du;
@@ -468,7 +482,13 @@ static bool conv_vector_ok(int64_t W, int dtype, std::initializer_list<const voi
 //       list ordinal -> token, by ballots and population counts over 64 tokens at a time;
 //   conv_padded_fwd_kernel    per token and channel vector, like the dense kernel, gathering the
 //       rows of the K-1 previous active tokens (or carried state rows, or zeros) through that list.
-// Scratch (32-bit words): ord[B][T], start[B][T], list[B][T], count[B], final_start[B].
+// A row whose active tokens are a prefix of it (a right-padded batch: every row of one) needs none of
+// that: there the ordinal is the token, and the convolution is the dense one over the first `count` tokens
+// with the position `ordinal - document start` (unbounded where no document starts inside the call).  The
+// index kernel writes those positions as well and marks such rows; conv_fwd_kernel / conv_bwd_kernel take
+// them (ConvArgs::rows) and the two kernels here leave them alone.
+// Scratch: position[B][T] (64-bit), then 32-bit words ord[B][T], start[B][T], list[B][T], count[B],
+// final_start[B], prefix[B].
 // ------------------------------------------------------------------------------------------
 struct PaddedArgs {
   const void* u; const void* state; const void* taps; const void* bias;
@@ -478,18 +498,50 @@ struct PaddedArgs {
   int B, T, W, K, nvec, runs, vec_dtype;
 };
 
+// The parts of the index of sequence b.
+struct PaddedIndex { long long* position; int* ord; int* start; int* list; int* tail; };
+RGLRU_DEVICE PaddedIndex padded_index(const PaddedArgs& p, int b) {
+  PaddedIndex x;
+  const long long cells = (long long)p.B * p.T;
+  x.position = reinterpret_cast<long long*>(p.scratch) + (long long)b * p.T;
+  int* words = p.scratch + 2 * cells;
+  x.ord = words + (long long)b * p.T;
+  x.start = words + cells + (long long)b * p.T;
+  x.list = words + 2 * cells + (long long)b * p.T;
+  x.tail = words + 3 * cells;
+  return x;
+}
+constexpr long long kUnboundedPosition = 1ll << 30;        // no document start in front of the token inside this call
+
 __global__ __launch_bounds__(64) void conv_padded_index_kernel(PaddedArgs p) {
   const int b = blockIdx.x, lane = threadIdx.x;
-  int* ord = p.scratch + (long long)b * p.T;
-  int* start = p.scratch + ((long long)p.B + b) * p.T;
-  int* list = p.scratch + (2ll * p.B + b) * p.T;
-  int* tail = p.scratch + 3ll * p.B * p.T;
-  int count = 0, doc_start = -1;                           // wave-uniform running values
-  for (int t0 = 0; t0 < p.T; t0 += 64) {
+  const PaddedIndex x = padded_index(p, b);
+  int* ord = x.ord; int* start = x.start; int* list = x.list; int* tail = x.tail;
+  int count = 0, doc_start = -1, last_active = -1;         // wave-uniform running values
+  // The walk is a chain of wave-uniform values, so a chunk's loads must not wait behind the chunk in front of
+  // it: the flags and positions of kAhead chunks are requested together (clamped index, so every load is
+  // unconditional), then the chunks are walked from registers.
+  constexpr int kAhead = 8;
+  const unsigned char* act_row = p.active + (long long)b * p.T;
+  const long long* pos_row = p.segpos + (long long)b * p.T;
+  for (int base = 0; base < p.T; base += 64 * kAhead) {
+    unsigned char act_v[kAhead];
+    long long pos_v[kAhead];
+#pragma unroll
+    for (int q = 0; q < kAhead; ++q) {
+      const int tq = base + 64 * q + lane;
+      const int tc = tq < p.T ? tq : p.T - 1;
+      act_v[q] = act_row[tc];
+      pos_v[q] = pos_row[tc];
+    }
+#pragma unroll
+    for (int q = 0; q < kAhead; ++q) {
+    const int t0 = base + 64 * q;
+    if (t0 >= p.T) break;
     const int t = t0 + lane;
     const bool in = t < p.T;
-    const bool act = in && p.active[(long long)b * p.T + t] != 0;
-    const bool rst = act && p.segpos[(long long)b * p.T + t] == 0;
+    const bool act = in && act_v[q] != 0;
+    const bool rst = act && pos_v[q] == 0;
     const unsigned long long am = __ballot(act), rm = __ballot(rst);
     const unsigned long long below = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
     const int my_ord = count + __popcll(am & below);
@@ -500,15 +552,24 @@ __global__ __launch_bounds__(64) void conv_padded_index_kernel(PaddedArgs p) {
       const int at = 63 - __clzll(upto);
       my_start = count + __popcll(am & ((at == 0) ? 0ull : (~0ull >> (64 - at))));
     }
-    if (in) { ord[t] = act ? my_ord : -1; start[t] = my_start; }
+    if (in) {
+      ord[t] = act ? my_ord : -1; start[t] = my_start;
+      x.position[t] = my_start < 0 ? kUnboundedPosition : (long long)(my_ord - my_start);   // read for prefix rows only
+    }
     if (act) list[my_ord] = t;
+    if (am) last_active = t0 + 63 - __clzll(am);
     if (rm) {
       const int at = 63 - __clzll(rm);
       doc_start = count + __popcll(am & ((at == 0) ? 0ull : (~0ull >> (64 - at))));
     }
     count += __popcll(am);
+    }
   }
-  if (lane == 0) { tail[b] = count; tail[p.B + b] = doc_start; }
+  if (lane == 0) { tail[b] = count; tail[p.B + b] = doc_start; tail[2 * p.B + b] = count == last_active + 1 ? 1 : 0; }
+}
+
+__host__ __device__ inline long long padded_blocks_per_seq(int T, int nvec) {
+  return ((long long)(T + 1) * nvec + kConvThreads - 1) / kConvThreads;
 }
 
 // Row that stands `lag` active tokens before ordinal i of sequence b, as floats.
@@ -517,26 +578,32 @@ RGLRU_DEVICE void padded_source(const PaddedArgs& p, rsrc_t ru, rsrc_t rs, const
                                 int c0, float (&v)[V]) {
   const int j = i - lag;
   const unsigned es = (unsigned)sizeof(IO), uW = (unsigned)p.W;
-  unsigned off = kOutOfRange;
+  // both sources are asked (the one that does not apply at an offset that reads as zero) and the row is selected
+  // afterwards: a descriptor chosen per lane would turn the load into a loop over the lanes' choices
+  unsigned off_u = kOutOfRange, off_s = kOutOfRange;
   bool from_state = false;
-  if (j >= 0 && j >= doc_start) off = ((unsigned)list[j] * uW + (unsigned)c0) * es;
-  else if (doc_start < 0 && j < 0 && K - 1 + j >= 0) { off = ((unsigned)(K - 1 + j) * uW + (unsigned)c0) * es; from_state = true; }
-  ConvRow<IO, V>::load(v, from_state ? rs : ru, off);
+  if (j >= 0 && j >= doc_start) off_u = ((unsigned)list[j] * uW + (unsigned)c0) * es;
+  else if (doc_start < 0 && j < 0 && K - 1 + j >= 0) { off_s = ((unsigned)(K - 1 + j) * uW + (unsigned)c0) * es; from_state = true; }
+  float s[V];
+  ConvRow<IO, V>::load(v, ru, off_u);
+  ConvRow<IO, V>::load(s, rs, off_s);
+#pragma unroll
+  for (int e = 0; e < V; ++e) v[e] = from_state ? s[e] : v[e];
 }
 
 template <typename IO, int V, int K>
 __global__ __launch_bounds__(kConvThreads) void conv_padded_fwd_kernel(PaddedArgs p) {
-  const long long item = (long long)blockIdx.x * kConvThreads + threadIdx.x;
+  // a workgroup stays inside one sequence, so the descriptors below are the same in all its lanes
   const long long per_seq = (long long)(p.T + 1) * p.nvec;    // one extra "token" per row writes the new state
-  if (item >= (long long)p.B * per_seq) return;
-  const int b = (int)(item / per_seq);
-  const long long rest = item - (long long)b * per_seq;
+  const unsigned wg_per_seq = (unsigned)padded_blocks_per_seq(p.T, p.nvec);
+  const int b = __builtin_amdgcn_readfirstlane((int)(blockIdx.x / wg_per_seq));   // the quotient comes out of the vector unit
+  const long long rest = (long long)(blockIdx.x - (unsigned)b * wg_per_seq) * kConvThreads + threadIdx.x;
+  if (rest >= per_seq) return;
   const int t = (int)(rest / p.nvec), c0 = (int)(rest - (long long)t * p.nvec) * V;
   const unsigned es = (unsigned)sizeof(IO), uW = (unsigned)p.W;
-  const int* ord = p.scratch + (long long)b * p.T;
-  const int* start = p.scratch + ((long long)p.B + b) * p.T;
-  const int* list = p.scratch + (2ll * p.B + b) * p.T;
-  const int* tail = p.scratch + 3ll * p.B * p.T;
+  const PaddedIndex x = padded_index(p, b);
+  const int* ord = x.ord; const int* start = x.start; const int* list = x.list; const int* tail = x.tail;
+  if (t < p.T && tail[2 * p.B + b]) return;                // a prefix row: the dense kernel writes its outputs
   const rsrc_t ru = make_rsrc((const IO*)p.u + (long long)b * p.T * p.W, (unsigned)p.T * uW * es);
   const rsrc_t rs = make_rsrc(p.state ? (const IO*)p.state + (long long)b * (K - 1) * p.W : (const IO*)p.u,
                               p.state ? (unsigned)((K - 1) * p.W) * es : 0u);
@@ -591,27 +658,30 @@ __global__ __launch_bounds__(kConvThreads) void conv_padded_bwd_kernel(PaddedArg
   __shared__ float red[kConvBwdRuns][(K + 1) * V][kConvBwdVecs + 1];
   const int vec_groups = (p.nvec + kConvBwdVecs - 1) / kConvBwdVecs;
   const int run_groups = (p.runs + kConvBwdRuns - 1) / kConvBwdRuns;
-  const int vg = blockIdx.x % vec_groups;
-  const int rest = blockIdx.x / vec_groups;
-  const int rgp = rest % run_groups, b = rest / run_groups;
+  // quotients of workgroup-uniform values come out of the vector unit (integer division runs there): said to be
+  // uniform here, so that the sequence's descriptors live in scalar registers
+  const int vg = __builtin_amdgcn_readfirstlane((int)(blockIdx.x % vec_groups));
+  const int rest = __builtin_amdgcn_readfirstlane((int)(blockIdx.x / vec_groups));
+  const int rgp = __builtin_amdgcn_readfirstlane(rest % run_groups), b = __builtin_amdgcn_readfirstlane(rest / run_groups);
   const int lane_vec = threadIdx.x % kConvBwdVecs, lane_run = threadIdx.x / kConvBwdVecs;
   const int vec = vg * kConvBwdVecs + lane_vec, run = rgp * kConvBwdRuns + lane_run;
   const bool ok = vec < p.nvec && run < p.runs;
   const int c0 = (vec < p.nvec ? vec : 0) * V, t0 = run * kConvRunBwd;
   const unsigned es = (unsigned)sizeof(IO), uW = (unsigned)p.W;
-  const int* ord = p.scratch + (long long)b * p.T;
-  const int* start = p.scratch + ((long long)p.B + b) * p.T;
-  const int* list = p.scratch + (2ll * p.B + b) * p.T;
-  const int* tail = p.scratch + 3ll * p.B * p.T;
+  const PaddedIndex x = padded_index(p, b);
+  const int* ord = x.ord; const int* start = x.start; const int* list = x.list; const int* tail = x.tail;
+  if (tail[2 * p.B + b]) return;                           // a prefix row: the dense kernel does it, partial sums included
   const int n = tail[b];                                   // active tokens of the row
   float tap[K][V], bias_unused[V];
   conv_load_taps<V, K>(p.taps, nullptr, c0, p.vec_dtype, tap, bias_unused);
-  const unsigned seq_bytes = ok ? (unsigned)p.T * uW * es : 0u;
+  // the descriptors are the same in every lane (a thread without work leaves the token loop at once and takes no
+  // part in the state gradient), so no access through them becomes a loop over the lanes' values
+  const unsigned seq_bytes = (unsigned)p.T * uW * es;
   const rsrc_t ru = make_rsrc((const IO*)p.u + (long long)b * p.T * p.W, seq_bytes);
   const rsrc_t rd = make_rsrc((const IO*)p.dout + (long long)b * p.T * p.W, seq_bytes);
   const rsrc_t rg = make_rsrc((const IO*)p.du + (long long)b * p.T * p.W, seq_bytes);
   const rsrc_t rs = make_rsrc(p.state ? (const IO*)p.state + (long long)b * (K - 1) * p.W : (const IO*)p.u,
-                              (p.state && ok) ? (unsigned)((K - 1) * p.W) * es : 0u);
+                              p.state ? (unsigned)((K - 1) * p.W) * es : 0u);
   float acc_tap[K][V], acc_bias[V];
 #pragma unroll
   for (int v = 0; v < V; ++v) {
@@ -1198,6 +1268,10 @@ int rglru_hip_conv_bwd(const void* u, const void* state, const void* taps, const
   return rc;
 }
 
+// Host-side view of the index (see padded_index): the positions of prefix rows and the per-row words.
+static const long long* padded_positions(const void* scratch) { return (const long long*)scratch; }
+static const int* padded_rows(const void* scratch, int64_t B, int64_t T) { return (const int*)scratch + 5 * B * T; }
+
 int rglru_hip_conv_padded_bwd(const void* u, const void* state, const void* taps,
                               const int64_t* segment_pos, const uint8_t* active, const void* dout,
                               void* index_scratch, void* scratch, void* du, void* dstate, void* dtaps, void* dbias,
@@ -1208,6 +1282,7 @@ int rglru_hip_conv_padded_bwd(const void* u, const void* state, const void* taps
   if (grad_dtype != RGLRU_F32 && grad_dtype != RGLRU_BF16) return fail(RGLRU_E_ARG, "conv_padded_bwd: unknown gradient dtype %d", grad_dtype);
   if (!u || !taps || !segment_pos || !active || !dout || !index_scratch || !scratch || !du)
     return fail(RGLRU_E_ARG, "conv_padded_bwd: null pointer");
+  if ((uintptr_t)index_scratch % 8) return fail(RGLRU_E_ARG, "conv_padded_bwd: index scratch must be 8-byte aligned");
   if (B * T >= (1ll << 29)) return fail(RGLRU_E_UNSUPPORTED, "conv_padded_bwd: tensor too large");
   PaddedArgs a;
   memset(&a, 0, sizeof(a));
@@ -1228,6 +1303,17 @@ int rglru_hip_conv_padded_bwd(const void* u, const void* state, const void* taps
   RGLRU_CONV_DISPATCH(conv_padded_bwd_kernel, dtype, vec, grid, s, a);
   rc = check_launch("conv_padded_bwd");
   if (rc) return rc;
+  {
+    // rows whose active tokens are a prefix: the dense kernel, same grid and same partial rows
+    ConvArgs d;
+    memset(&d, 0, sizeof(d));
+    d.u = u; d.state = state; d.taps = taps; d.dout = dout; d.du = du; d.dstate = dstate; d.partial = a.partial;
+    d.ld_du = W; d.segpos = padded_positions(index_scratch); d.rows = padded_rows(index_scratch, B, T);
+    d.B = (int)B; d.T = (int)T; d.W = (int)W; d.K = (int)K; d.vec_dtype = vec_dtype; d.nvec = a.nvec; d.runs = a.runs;
+    RGLRU_CONV_DISPATCH(conv_bwd_kernel, dtype, vec, grid, s, d);
+    rc = check_launch("conv_padded_bwd prefix rows");
+    if (rc) return rc;
+  }
   if (dtaps || dbias) {
     ConvFinishArgs f;
     f.partial = a.partial; f.dtaps = dtaps; f.dbias = dbias; f.W = (int)W; f.K = (int)K;
@@ -1321,7 +1407,7 @@ int rglru_hip_decode_prepare(const void* u, int64_t u_stride, const void* conv_s
 
 size_t rglru_hip_conv_padded_scratch_bytes(int64_t B, int64_t T) {
   if (B <= 0 || T <= 0) return 0;
-  return (size_t)((3 * B * T + 2 * B) * 4);
+  return (size_t)(B * T * 8 + (3 * B * T + 3 * B) * 4);
 }
 
 int rglru_hip_conv_padded_fwd(const void* u, const void* state, const void* taps, const void* bias,
@@ -1331,6 +1417,7 @@ int rglru_hip_conv_padded_fwd(const void* u, const void* state, const void* taps
   int rc = conv_check("conv_padded_fwd", B, T, W, K, dtype, vec_dtype);
   if (rc) return rc;
   if (!u || !taps || !segment_pos || !active || !scratch || !out) return fail(RGLRU_E_ARG, "conv_padded_fwd: null pointer");
+  if ((uintptr_t)scratch % 8) return fail(RGLRU_E_ARG, "conv_padded_fwd: scratch must be 8-byte aligned");
   if (B * T >= (1ll << 29)) return fail(RGLRU_E_UNSUPPORTED, "conv_padded_fwd: tensor too large");
   PaddedArgs a;
   memset(&a, 0, sizeof(a));
@@ -1343,10 +1430,24 @@ int rglru_hip_conv_padded_fwd(const void* u, const void* state, const void* taps
   hipLaunchKernelGGL(conv_padded_index_kernel, dim3((unsigned)B), dim3(64), 0, s, a);
   rc = check_launch("conv_padded_fwd index");
   if (rc) return rc;
-  const long long items = (long long)B * (T + 1) * a.nvec;
-  dim3 grid((unsigned)((items + kConvThreads - 1) / kConvThreads));
+  const long long blocks = (long long)B * padded_blocks_per_seq((int)T, a.nvec);
+  if (blocks > 0x7fffffffll) return fail(RGLRU_E_UNSUPPORTED, "conv_padded_fwd: problem too large for one launch");
+  dim3 grid((unsigned)blocks);
   RGLRU_CONV_DISPATCH(conv_padded_fwd_kernel, dtype, vec, grid, s, a);
-  return check_launch("conv_padded_fwd");
+  rc = check_launch("conv_padded_fwd");
+  if (rc) return rc;
+  // rows whose active tokens are a prefix: the dense kernel over the positions the index kernel derived
+  ConvArgs d;
+  memset(&d, 0, sizeof(d));
+  d.u = u; d.state = state; d.taps = taps; d.bias = bias; d.out = out;
+  d.segpos = padded_positions(scratch); d.rows = padded_rows(scratch, B, T);
+  d.B = (int)B; d.T = (int)T; d.W = (int)W; d.K = (int)K; d.vec_dtype = vec_dtype; d.nvec = a.nvec;
+  d.runs = (int)((T + kConvRunFwd - 1) / kConvRunFwd);
+  const long long dense_blocks = B * conv_blocks_per_seq(d.runs, d.nvec);
+  if (dense_blocks >= (1ll << 31)) return fail(RGLRU_E_UNSUPPORTED, "conv_padded_fwd: tensor too large");
+  dim3 dense_grid((unsigned)dense_blocks);
+  RGLRU_CONV_DISPATCH(conv_fwd_kernel, dtype, vec, dense_grid, s, d);
+  return check_launch("conv_padded_fwd prefix rows");
 }
 
 int rglru_hip_rmsnorm_max_width(int dtype, int aligned) {

@@ -278,7 +278,9 @@ int rglru_hip_conv_bwd(const void* u, const void* state, const void* taps, const
  * per-token Python loop): dout[B,T,W] in; du[B,T,W] (zero at inactive tokens), dstate[B,K-1,W],
  * dtaps[W,K], dbias[W] out (the last three may be NULL).  `index_scratch` holds
  * rglru_hip_conv_padded_scratch_bytes(B, T) bytes and `scratch` rglru_hip_conv_scratch_bytes(B, T, W, K)
- * bytes; their contents on entry do not matter. */
+ * bytes; their contents on entry do not matter.  Both index buffers must be 8-byte aligned.
+ * Rows whose active tokens are a prefix of the row (all rows of a right-padded batch) run at the speed of
+ * rglru_hip_conv_fwd / _bwd; rows with holes take kernels that gather through an index. */
 size_t rglru_hip_conv_padded_scratch_bytes(int64_t B, int64_t T);
 int rglru_hip_conv_padded_fwd(const void* u, const void* state, const void* taps, const void* bias,
                               const int64_t* segment_pos, const uint8_t* active, void* scratch,

@@ -234,6 +234,10 @@ def _padded_inputs(B, T, W, K, seed, pattern):
         if B > 1:
             lengths[1] = 0                                   # an empty row: state must pass through
         active = torch.arange(T)[None, :] < lengths[:, None]
+    elif pattern == "mixed":                                 # right-padded rows and rows with holes side by side:
+        lengths = torch.randint(0, T + 1, (B,), generator=g)  # the two kinds go to different kernels of one call
+        active = torch.arange(T)[None, :] < lengths[:, None]
+        active[::2] = torch.rand((B + 1) // 2, T, generator=g) > 0.3
     else:                                                    # holes anywhere
         active = torch.rand(B, T, generator=g) > 0.3
     pos = _positions(B, T, "packed", seed + 1)
@@ -242,7 +246,8 @@ def _padded_inputs(B, T, W, K, seed, pattern):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("cfg", [(3, 50, 64, 4, "right"), (4, 200, 24, 4, "holes"), (2, 130, 13, 3, "holes"),
-                                 (3, 65, 128, 2, "right"), (2, 7, 16, 1, "holes")])
+                                 (3, 65, 128, 2, "right"), (2, 7, 16, 1, "holes"), (5, 300, 64, 4, "mixed"),
+                                 (4, 2100, 256, 4, "right")])
 def test_padded_conv_matches_oracle(cfg, dtype):
     from griffin_amd.hip_block_ops import hip_causal_conv_padded
 
@@ -284,7 +289,8 @@ def test_padded_conv_all_active_equals_dense_kernel_at_training_shape():
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("cfg", [(3, 50, 64, 4, "right"), (4, 200, 24, 4, "holes"), (2, 130, 13, 3, "holes"),
-                                 (3, 65, 128, 2, "right"), (2, 7, 16, 1, "holes"), (2, 300, 1024, 4, "holes")])
+                                 (3, 65, 128, 2, "right"), (2, 7, 16, 1, "holes"), (2, 300, 1024, 4, "holes"),
+                                 (5, 300, 64, 4, "mixed"), (4, 700, 256, 3, "right")])
 def test_padded_conv_gradients_match_oracle_autograd(cfg, dtype):
     """Reverse mode of the padded convolution (C ABI: rglru_hip_conv_padded_bwd) against autograd through
     the oracle's token-by-token loop: gradients at the input, the carried state, the taps and the bias."""
