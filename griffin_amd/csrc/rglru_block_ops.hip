@@ -998,17 +998,22 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(NormArgs p) {
   const long long wave = (long long)blockIdx.x * (kNormThreads / 64) + (threadIdx.x >> 6);
   const long long n_waves = (long long)gridDim.x * (kNormThreads / 64);
   const unsigned row_bytes = (unsigned)p.D * (unsigned)sizeof(IO);
-  float w[kNormSlots][V], dg[kNormSlots][V];
-#pragma unroll
-  for (int s = 0; s < kNormSlots; ++s) {
+  // The widest backward variant would hold x, dy, the scale and its gradient sums of 128 elements per lane, more
+  // than the register file: there the scale is fetched again for every row (it stays in the cache).
+  constexpr bool kHoldScale = !(BACKWARD && SLOTS * V > 64);
+  float w[kHoldScale ? kNormSlots : 1][V], dg[kNormSlots][V];
+  auto scale_of = [&](int s, float (&out)[V]) {
     const bool has = lane + 64 * s < p.nvec;
     float g[V];
     conv_params<V>(p.g, has ? (long long)(lane + 64 * s) * V : 0, p.vec_dtype, g);
 #pragma unroll
-    for (int v = 0; v < V; ++v) {
-      w[s][v] = has ? 1.0f + g[v] : 0.f;
-      dg[s][v] = 0.f;
-    }
+    for (int v = 0; v < V; ++v) out[v] = has ? 1.0f + g[v] : 0.f;
+  };
+#pragma unroll
+  for (int s = 0; s < kNormSlots; ++s) {
+    if constexpr (kHoldScale) scale_of(s, w[s]);
+#pragma unroll
+    for (int v = 0; v < V; ++v) dg[s][v] = 0.f;
   }
   const float inv_d = 1.0f / (float)p.D;
   for (long long row = wave; row < p.rows; row += n_waves) {
@@ -1020,13 +1025,27 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(NormArgs p) {
       raw_x[s] = Row::request(rx, off);
       if (BACKWARD) raw_d[s] = Row::request(make_rsrc((const IO*)p.dy + row * p.D, row_bytes), off);
     }
-    float x[kNormSlots][V];
+    // the row as floats, except in the widest backward variant, which keeps the rows as loaded and converts a
+    // slot each time it needs it (x, dy and the gradient sums as floats would not fit the registers)
+    float x[kHoldScale ? kNormSlots : 1][V];
+    auto x_of = [&](int s, float (&out)[V]) {
+      if constexpr (kHoldScale) {
+#pragma unroll
+        for (int v = 0; v < V; ++v) out[v] = x[s][v];
+      } else {
+        Row::unpack(out, raw_x[s]);
+      }
+    };
     float acc = 0.f;
 #pragma unroll
     for (int s = 0; s < kNormSlots; ++s) {
-      Row::unpack(x[s], raw_x[s]);
+      float xs[V];
+      Row::unpack(xs, raw_x[s]);
 #pragma unroll
-      for (int v = 0; v < V; ++v) acc = fmaf(x[s][v], x[s][v], acc);
+      for (int v = 0; v < V; ++v) {
+        if constexpr (kHoldScale) x[s][v] = xs[v];
+        acc = fmaf(xs[v], xs[v], acc);
+      }
     }
     if (!BACKWARD) {
       const float inv = __builtin_amdgcn_rsqf(wave_sum(acc) * inv_d + p.eps);
@@ -1041,25 +1060,46 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_kernel(NormArgs p) {
       }
     } else {
       const float inv = p.inv_in[row];
-      float d[kNormSlots][V];
+      float d[kHoldScale ? kNormSlots : 1][V];
       float dot = 0.f;
 #pragma unroll
       for (int s = 0; s < kNormSlots; ++s) {
-        Row::unpack(d[s], raw_d[s]);
+        float ds[V], xs[V];
+        Row::unpack(ds, raw_d[s]);
+        x_of(s, xs);
+        float ws[V];
+        if constexpr (kHoldScale) {
+#pragma unroll
+          for (int v = 0; v < V; ++v) ws[v] = w[s][v];
+        } else {
+          scale_of(s, ws);
+        }
 #pragma unroll
         for (int v = 0; v < V; ++v) {
-          dg[s][v] = fmaf(d[s][v] * inv, x[s][v], dg[s][v]);
-          d[s][v] *= w[s][v];
-          dot = fmaf(d[s][v], x[s][v], dot);
+          dg[s][v] = fmaf(ds[v] * inv, xs[v], dg[s][v]);
+          ds[v] *= ws[v];
+          if constexpr (kHoldScale) d[s][v] = ds[v];
+          dot = fmaf(ds[v], xs[v], dot);
         }
       }
       const float k = wave_sum(dot) * inv_d * inv * inv;
       const rsrc_t rdx = make_rsrc((IO*)p.dx + row * p.D, row_bytes);
 #pragma unroll
       for (int s = 0; s < kNormSlots; ++s) {
-        float g[V];
+        float g[V], xs[V], ds[V];
+        x_of(s, xs);
+        if constexpr (kHoldScale) {
 #pragma unroll
-        for (int v = 0; v < V; ++v) g[v] = inv * fmaf(-k, x[s][v], d[s][v]);
+          for (int v = 0; v < V; ++v) ds[v] = d[s][v];
+        } else {
+          float ws[V];
+          Row::unpack(ds, raw_d[s]);
+          scale_of(s, ws);
+#pragma unroll
+          for (int v = 0; v < V; ++v) ds[v] *= ws[v];
+        }
+#pragma unroll
+        for (int v = 0; v < V; ++v) g[v] = inv * fmaf(-k, xs[v], ds[v]);
         Row::store(g, rdx, (lane + 64 * s < p.nvec) ? (unsigned)((lane + 64 * s) * V) * (unsigned)sizeof(IO) : kOutOfRange);
       }
     }

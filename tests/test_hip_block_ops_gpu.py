@@ -326,11 +326,16 @@ def test_padded_conv_gradients_match_oracle_autograd(cfg, dtype):
 # RMSNorm in front of the block (C ABI: rglru_hip_rmsnorm_fwd / _bwd)
 # ----------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("shape", [(2, 50, 64), (3, 7, 13), (1, 1, 768), (4, 33, 1024), (2, 5, 2560), (300, 24)])
+@pytest.mark.parametrize("shape", [(2, 50, 64), (3, 7, 13), (1, 1, 768), (4, 33, 1024), (2, 5, 2560), (300, 24),
+                                   (70, 4096), (9, 5000), (33, 8192)])
 def test_rmsnorm_matches_oracle(shape, dtype):
     from griffin_amd.hip_block_ops import hip_rmsnorm
 
+    from griffin_amd.hip_block_ops import rmsnorm_max_width
+
     _say("rmsnorm case", shape, dtype)
+    if shape[-1] > rmsnorm_max_width(dtype):
+        pytest.skip("wider than one wave holds in this storage type: the module uses the portable operators there")
     gen = torch.Generator().manual_seed(21)
     x = torch.randn(*shape, generator=gen) * 1.7 + 0.3
     scale = torch.randn(shape[-1], generator=gen) * 0.2
