@@ -17,7 +17,8 @@ on a bounded sample of the same workload, all threads and one thread).
 --workload selects one of the other measured configurations instead (one JSON line without the CPU
 leg; their per-kernel figures come from rocprofv3 runs of the same command, summarised under profiles/):
     scan_only     the scan-only operator (fp32 a, z -> h) forward + backward at B8 T2048 W1024, HIP graph
-    block         RMSNorm + RecurrentBlock(768, 1024) forward + backward at B8 T2048, bf16, eager
+    block         RMSNorm + RecurrentBlock(768, 1024) forward + backward at B8 T2048, bf16, eager and as a HIP graph
+    block_padded  the same block on a right-padded batch (rows of 77 to 2048 tokens), eager
     long_context  RG-LRU forward + backward at B1 T32768 W2560, 8 blocks of 320 channels, slow decay, eager
     decode        512 single-token RG-LRU steps at B256 W1024 after a T2048 prefill: eager, a HIP graph of
                   64 single-step launches, and one launch for all steps
@@ -63,7 +64,7 @@ def parse_args():
     ap.add_argument("--seq", type=int, default=2048)
     ap.add_argument("--width", type=int, default=1024)
     ap.add_argument("--blocks", type=int, default=8)
-    ap.add_argument("--workload", default="rglru", choices=["rglru", "block", "long_context", "decode", "block_decode", "scan_only"])
+    ap.add_argument("--workload", default="rglru", choices=["rglru", "block", "block_padded", "long_context", "decode", "block_decode", "scan_only"])
     return ap.parse_args()
 
 
@@ -137,6 +138,27 @@ def secondary_workload(args):
                        "graph_vs_eager_max_rel_err": worst, "ms_forward_no_grad_graph": ms_prefill}
         metric, tokens = "RMSNorm + RecurrentBlock fwd+bwd tokens/s", B * T
         workload = f"RMSNorm + RecurrentBlock({D}, {W}) fwd+bwd B{B} T{T} bf16 (HIP graph of {per_graph} steps)"
+    elif name == "block_padded":
+        # the same block on a right-padded batch (griffin/griffin.py:488-510: rows of different lengths, padding
+        # excluded from the convolution's history and from the state).  The module asks the host whether every token is
+        # active, as the reference does, so the step cannot be captured: eager launches, host time included; the kernel
+        # times are in the rocprofv3 summary of this command.
+        B, T, D, W = 8, 2048, 768, 1024
+        block = RecurrentBlock(D, W, scan_mode="hip").to(dev).to(dt)
+        norm = RMSNorm(D).to(dev).to(dt)
+        x = torch.randn(B, T, D, device=dev, dtype=dt, requires_grad=True)
+        dy = torch.randn(B, T, D, device=dev, dtype=dt)
+        lengths = torch.tensor([2048, 2000, 1500, 1024, 2048, 77, 1900, 2047], device=dev)
+        active = torch.arange(T, device=dev)[None, :] < lengths[:, None]
+        leaves = [x] + list(block.parameters()) + list(norm.parameters())
+        one = lambda: torch.autograd.grad(block(norm(x), active_mask=active), leaves, dy)
+        ms = _timed(one, args.steps, args.warmup)
+        grads = one()
+        torch.cuda.synchronize()
+        padding_gets_no_gradient = bool(torch.count_nonzero(grads[0][~active]).item() == 0)
+        block_extra = {"active_tokens": int(lengths.sum().item()), "padding_gets_no_gradient": padding_gets_no_gradient}
+        metric, tokens = "RMSNorm + RecurrentBlock fwd+bwd active tokens/s (right-padded batch)", int(lengths.sum().item())
+        workload = f"RMSNorm + RecurrentBlock({D}, {W}) fwd+bwd B{B} T{T} bf16, rows of {lengths.tolist()} tokens (eager)"
     elif name == "scan_only":
         # the scan-only operator (contract of the reference's fused_rglru_scan: fp32 a, z, h0 -> h) at the
         # benchmark shape: forward reads a, z and writes h (12 N bytes), backward reads a, dh, h and writes
@@ -315,7 +337,7 @@ def secondary_workload(args):
         "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic", "config": {"workload": workload, "launch": "hip graph" if name in ("decode", "block_decode", "block") else "eager"},
         **({"decode": extra} if name in ("decode", "block_decode") else {}),
-        **({"block": block_extra} if name == "block" else {}),
+        **({"block": block_extra} if name in ("block", "block_padded") else {}),
     }))
 
 
