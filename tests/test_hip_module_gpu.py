@@ -672,6 +672,46 @@ def test_decode_row_stride_below_width_is_rejected():
     assert rc != 0 and b"stride" in lib.rglru_hip_last_error()
 
 
+def test_block_under_autocast_with_fp32_master_parameters():
+    """Mixed-precision training as a trainer sets it up: fp32 parameters, `torch.autocast(bfloat16)` around the
+    forward.  The block on the HIP kernels returns bf16, every parameter gets an fp32 gradient, and all of it agrees
+    with the fp32 block on the CPU to bf16 accuracy; a forward on a side stream and one on a non-contiguous input
+    agree with it too."""
+    from griffin_amd import RecurrentBlock
+
+    torch.manual_seed(0)
+    B, T, D, W = 2, 300, 96, 256
+    ref = RecurrentBlock(D, W, gate_blocks=4, scan_mode="sequential")
+    hip = copy.deepcopy(ref).cuda()
+    hip.scan_mode = None
+    hip.rg_lru.scan_mode = "hip"
+    x = torch.randn(B, T, D)
+    up = torch.randn(B, T, D)
+    xc = x.clone().requires_grad_(True)
+    xh = x.clone().cuda().requires_grad_(True)
+    yc = ref(xc)
+    yc.backward(up)
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        yh = hip(xh)
+    assert yh.dtype == torch.bfloat16
+    yh.float().backward(up.cuda())
+    torch.cuda.synchronize()
+    assert rel_err(yh.float(), yc) < BF16_TOL and rel_err(xh.grad, xc.grad) < BF16_TOL
+    for (name, ph), (_, pc) in zip(hip.named_parameters(), ref.named_parameters()):
+        assert ph.grad.dtype == torch.float32, name
+        assert rel_err(ph.grad, pc.grad) < BF16_TOL, name
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            y_side = hip(xh.detach())
+        side.synchronize()
+        assert rel_err(y_side, yc) < 1e-5
+        strided = x.transpose(0, 1).contiguous().transpose(0, 1).cuda()
+        assert not strided.is_contiguous()
+        assert rel_err(hip(strided), yc) < 1e-5
+
+
 # ----------------------------------------------------------------------------------------------
 # random sweeps of the block: the HIP kernels against the same block on the CPU, driven the same way
 # ----------------------------------------------------------------------------------------------
