@@ -14,7 +14,7 @@ RGLRU_BF16 = 1
 FLAG_RESET = 1
 FLAG_INACTIVE = 2
 CHUNK = 32
-ABI_VERSION = 18
+ABI_VERSION = 19
 PATH_PORTABLE, PATH_FAST_TILED, PATH_FAST_CHAIN, PATH_WIDE, PATH_PRE = range(5)
 PATH_NAMES = ("portable", "fast_tiled", "fast_chain", "wide", "pre")
 
@@ -59,6 +59,7 @@ _SIGNATURES = {
     "rglru_hip_conv_padded_bwd": (ctypes.c_int, [_P] * 12 + [_I, _I, _I, _I, ctypes.c_int, ctypes.c_int, ctypes.c_int, _P]),
     "rglru_hip_colsum_scratch_bytes": (ctypes.c_size_t, [_I, _I]),
     "rglru_hip_colsum": (ctypes.c_int, [_P, _P, _P, _I, _I, ctypes.c_int, ctypes.c_int, _P]),
+    "rglru_hip_sum_sets": (ctypes.c_int, [_P, _P, _I, _I, ctypes.c_int, _P]),
     "rglru_hip_gelu_gate_fwd": (ctypes.c_int, [_P, _P, _P, _I, ctypes.c_int, _P]),
     "rglru_hip_gelu_gate_bwd": (ctypes.c_int, [_P, _P, _P, _P, _P, _I, _I, _I, ctypes.c_int, _P]),
     "rglru_hip_rmsnorm_max_width": (ctypes.c_int, [ctypes.c_int, ctypes.c_int]),

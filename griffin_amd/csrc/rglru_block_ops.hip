@@ -1202,6 +1202,49 @@ __global__ __launch_bounds__(256) void colsum_kernel(ColsumArgs p) {
   }
 }
 
+// Sum of `sets` arrays of n elements each, x[s * n + i] -> out[i]: what is left of a weight gradient whose
+// contraction over the tokens was split into a batch of shorter GEMMs.  A thread owns V consecutive elements and
+// asks for up to eight sets at once; fp32 accumulation in the order of the sets.
+struct SumSetsArgs { const void* x; void* out; long long n; int sets; };
+template <typename IO, int V>
+__global__ __launch_bounds__(256) void sum_sets_kernel(SumSetsArgs p) {
+  typedef typename ConvRow<IO, V>::Raw Raw;
+  const long long i = ((long long)blockIdx.x * 256 + threadIdx.x) * V;
+  if (i >= p.n) return;
+  const IO* src = (const IO*)p.x + i;
+  float acc[V];
+#pragma unroll
+  for (int v = 0; v < V; ++v) acc[v] = 0.f;
+  for (int s0 = 0; s0 < p.sets; s0 += 8) {
+    Raw raw[8];
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      const int s = s0 + q < p.sets ? s0 + q : p.sets - 1;   // a set past the last is asked again and not added
+      if constexpr (V == 1) raw[q] = (float)src[(long long)s * p.n];
+      else raw[q] = *reinterpret_cast<const Raw*>(src + (long long)s * p.n);
+    }
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {
+      float v[V];
+      ConvRow<IO, V>::unpack(v, raw[q]);
+      if (s0 + q < p.sets) {
+#pragma unroll
+        for (int e = 0; e < V; ++e) acc[e] += v[e];
+      }
+    }
+  }
+  IO* dst = (IO*)p.out + i;
+  if constexpr (V == 1) {
+    dst[0] = (IO)acc[0];
+  } else {
+    typedef IO Vec __attribute__((ext_vector_type(V)));
+    Vec o;
+#pragma unroll
+    for (int e = 0; e < V; ++e) o[e] = (IO)acc[e];
+    *reinterpret_cast<Vec*>(dst) = o;
+  }
+}
+
 template <typename IO, int V, bool BACKWARD>
 static void norm_launch(int nvec, dim3 grid, hipStream_t s, const NormArgs& a) {
   const int slots = (nvec + 63) / 64;
@@ -1549,6 +1592,29 @@ int rglru_hip_rmsnorm_bwd(const void* x, const void* g, const float* inv, const 
 
 static long long colsum_slots(int64_t rows) {
   return (rows + kColsumLanes * kColsumRowsPerLane - 1) / (kColsumLanes * kColsumRowsPerLane);
+}
+
+int rglru_hip_sum_sets(const void* x, void* out, int64_t sets, int64_t n, int dtype, void* stream) {
+  if (!x || !out) return fail(RGLRU_E_ARG, "sum_sets: null pointer");
+  if (dtype != RGLRU_F32 && dtype != RGLRU_BF16) return fail(RGLRU_E_ARG, "sum_sets: dtype must be RGLRU_F32 or RGLRU_BF16, got %d", dtype);
+  if (sets <= 0 || n <= 0) return fail(RGLRU_E_ARG, "sum_sets: sets and n must be positive (got %lld, %lld)", (long long)sets, (long long)n);
+  if (sets >= (1 << 20) || n >= (1ll << 38)) return fail(RGLRU_E_UNSUPPORTED, "sum_sets: problem too large");
+  const bool vec = conv_vector_ok(n, dtype, {x, out});
+  const int V = vec ? (dtype == RGLRU_BF16 ? 8 : 4) : 1;
+  SumSetsArgs a;
+  a.x = x; a.out = out; a.n = n; a.sets = (int)sets;
+  const long long blocks = ((n + V - 1) / V + 255) / 256;
+  if (blocks >= (1ll << 31)) return fail(RGLRU_E_UNSUPPORTED, "sum_sets: problem too large");
+  dim3 grid((unsigned)blocks);
+  hipStream_t s = (hipStream_t)stream;
+  if (dtype == RGLRU_BF16) {
+    if (vec) hipLaunchKernelGGL((sum_sets_kernel<__bf16, 8>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((sum_sets_kernel<__bf16, 1>), grid, dim3(256), 0, s, a);
+  } else {
+    if (vec) hipLaunchKernelGGL((sum_sets_kernel<float, 4>), grid, dim3(256), 0, s, a);
+    else hipLaunchKernelGGL((sum_sets_kernel<float, 1>), grid, dim3(256), 0, s, a);
+  }
+  return check_launch("sum_sets");
 }
 
 size_t rglru_hip_colsum_scratch_bytes(int64_t rows, int64_t D) {

@@ -479,6 +479,20 @@ class _HipLinear(torch.autograd.Function):
         return dx, dw, db
 
 
+def _sum_sets(sets: Tensor) -> Tensor:
+    """``sets.sum(0)`` for a contiguous [sets, ...] tensor on the GPU by a kernel of the library (one pass over the
+    sets, 16-byte accesses; the generic reduction takes about three times as long for eight sets of a weight
+    gradient); anything else goes to ``sum``."""
+    if not sets.is_cuda or sets.dtype not in _DTYPE_CODES or not sets.is_contiguous() or sets.numel() == 0:
+        return sets.sum(0)
+    lib = _lib.load()
+    with _on_device(sets.device):
+        out = torch.empty(sets.shape[1:], dtype=sets.dtype, device=sets.device)
+        _lib.check(lib.rglru_hip_sum_sets(_ptr(sets), _ptr(out), sets.size(0), out.numel(), _dtype_code(sets.dtype),
+                                          _stream_ptr(sets.device)), "rglru_hip_sum_sets")
+    return out
+
+
 def _linear_parameter_grads(x: Tensor, weight: Tensor, dy: Tensor, need_w: bool, bias_dtype):
     """(dW, db) of ``y = x W^T + b`` for the incoming ``dy``; ``bias_dtype`` None skips db."""
     dy2 = dy.reshape(-1, dy.size(-1))
@@ -494,7 +508,7 @@ def _linear_parameter_grads(x: Tensor, weight: Tensor, dy: Tensor, need_w: bool,
             chunks //= 2
         if chunks > 1:
             per = rows // chunks
-            dw = torch.bmm(dy2.view(chunks, per, -1).transpose(1, 2), x2.view(chunks, per, -1)).sum(0)
+            dw = _sum_sets(torch.bmm(dy2.view(chunks, per, -1).transpose(1, 2), x2.view(chunks, per, -1)))
         else:
             dw = torch.mm(dy2.t(), x2)
         dw = dw.to(weight.dtype)

@@ -22,6 +22,7 @@
  *   griffin/griffin.py:68-80        RMSNorm in front of the block and its autograd   rglru_hip_rmsnorm_fwd, _bwd
  *   griffin/griffin.py:459-528 with T == 1 (block decode: positions, conv, step, gate)   rglru_hip_decode_prepare + rglru_hip_step_gated
  *   autograd of the bias of griffin/griffin.py:379-389 (the block's Linear layers)      rglru_hip_colsum
+ *   the sum that ends their weight gradient when its contraction is split             rglru_hip_sum_sets
  *
  * Conventions
  *   - every pointer is a DEVICE pointer owned by the caller; tensors are row-major with the
@@ -50,7 +51,7 @@
 extern "C" {
 #endif
 
-#define RGLRU_ABI_VERSION 18
+#define RGLRU_ABI_VERSION 19
 
 enum { RGLRU_F32 = 0, RGLRU_BF16 = 1 };
 
@@ -323,6 +324,12 @@ int rglru_hip_rmsnorm_bwd(const void* x, const void* g, const float* inv, const 
 size_t rglru_hip_colsum_scratch_bytes(int64_t rows, int64_t D);
 int rglru_hip_colsum(const void* x, void* scratch, void* out, int64_t rows, int64_t D, int dtype, int out_dtype,
                      void* stream);
+
+/* out[i] = sum over s < sets of x[s * n + i] (both `dtype`, fp32 accumulation in the order of the sets): the last
+ * step of the weight gradient of the block's Linear layers (griffin/griffin.py:379-389; autograd of `nn.Linear`:
+ * dW = dy^T x) where the caller splits the contraction over all tokens into a batch of shorter GEMMs of its BLAS
+ * library and has their results added. */
+int rglru_hip_sum_sets(const void* x, void* out, int64_t sets, int64_t n, int dtype, void* stream);
 
 /* Single-token step of the recurrent block (griffin/griffin.py:459-528 with one token per row) in
  * two launches around the caller's three Linear layers:

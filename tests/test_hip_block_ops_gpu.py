@@ -377,6 +377,39 @@ def test_rmsnorm_module_and_properties_at_training_shape():
 
 
 # ----------------------------------------------------------------------------------------------
+# sum of the partial weight gradients of a split contraction (C ABI: rglru_hip_sum_sets)
+# ----------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(8, 2048, 768), (16, 768, 1024), (3, 7, 13), (1, 64, 64), (9, 1, 5), (2, 1000001)])
+def test_sum_sets_matches_a_float64_sum(shape, dtype):
+    from griffin_amd.hip_block_ops import _sum_sets
+
+    _say("sum of sets", shape, dtype)
+    x = torch.randn(*shape, generator=torch.Generator().manual_seed(41)).to(dtype)
+    want = x.double().sum(0)
+    got = _sum_sets(x.cuda())
+    torch.cuda.synchronize()
+    assert got.dtype == dtype and got.shape == want.shape
+    # fp32 accumulation, one rounding to the storage type
+    tol = 1e-6 if dtype == torch.float32 else 4e-3
+    assert rel_err(got.double(), want) < tol
+    # a view that is not contiguous takes the generic reduction and still agrees
+    strided = x.cuda().transpose(0, 1) if x.dim() == 3 else None
+    if strided is not None:
+        assert rel_err(_sum_sets(strided).double(), x.double().transpose(0, 1).sum(0)) < tol
+
+
+def test_sum_sets_rejects_bad_arguments():
+    from griffin_amd import _lib
+
+    lib = _lib.load()
+    buf = torch.zeros(64, device="cuda")
+    assert lib.rglru_hip_sum_sets(buf.data_ptr(), buf.data_ptr(), 0, 8, 0, None) != 0
+    assert lib.rglru_hip_sum_sets(None, buf.data_ptr(), 2, 8, 0, None) != 0
+    assert lib.rglru_hip_sum_sets(buf.data_ptr(), buf.data_ptr(), 2, 8, 7, None) != 0
+
+
+# ----------------------------------------------------------------------------------------------
 # bias gradient of the block's Linear layers (C ABI: rglru_hip_colsum)
 # ----------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
