@@ -605,7 +605,7 @@ def test_chain_kernels_that_give_up_poison_their_results_and_set_the_failure_wor
 
 def test_kernel_family_selected_for_each_baseline_configuration():
     """Which kernel family serves a shape is a fact of the library (rglru_hip_backward_path), not of pointer luck in
-    the wrapper: the five BASELINE configurations, the widths in between, and what a misaligned tensor does."""
+    the wrapper: the five benchmark configurations of the reference, the widths in between, and what a misaligned tensor does."""
     from griffin_amd import _lib
     from griffin_amd.hip_scan import kernel_path
 
